@@ -1,0 +1,88 @@
+"""ctypes binding of libd2conv.so, the C-ABI HIP library (include/d2conv.h).
+
+There is no fallback: if the library has not been built, or a call fails, an
+exception is raised.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libd2conv.so")
+
+D2C_F32, D2C_F64, D2C_BF16 = 0, 1, 2
+ALGO_AUTO, ALGO_GENERIC, ALGO_MFMA, ALGO_DEPTHWISE = 0, 1, 2, 3
+ALGO_NAMES = {ALGO_GENERIC: "generic", ALGO_MFMA: "mfma", ALGO_DEPTHWISE: "depthwise"}
+
+# every symbol that include/d2conv.h declares
+EXPORTS = (
+    "d2c_output_size", "d2c_conv3d_check", "d2c_conv3d_algo",
+    "d2c_conv3d_forward_workspace_bytes", "d2c_conv3d_backward_workspace_bytes",
+    "d2c_conv3d_forward", "d2c_conv3d_backward",
+    "d2c_conv1d_check", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
+    "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
+    "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
+    "d2c_set_algo_override", "d2c_last_error", "d2c_version",
+)
+
+
+class Conv3dDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "N", "Cin", "Cout", "D", "H", "W", "kd", "kh", "kw", "sd", "sh", "sw",
+        "pd", "ph", "pw", "dd", "dh", "dw", "groups", "offset_groups", "Do", "Ho", "Wo",
+        "dtype", "aux_dtype")]
+
+
+class Conv1dDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "N", "Cin", "Cout", "L", "k", "s", "p", "d", "groups", "offset_groups", "Lo",
+        "dtype", "aux_dtype", "reference_quirks")]
+
+
+_lib = None
+
+
+def load():
+    """Returns the loaded library; raises if it was never built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the HIP library has not been built "
+            "(run `python -m d2conv3d_amd.build`); there is no fallback path")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, sz, i32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32
+    p3, p1 = ctypes.POINTER(Conv3dDesc), ctypes.POINTER(Conv1dDesc)
+    lib.d2c_output_size.restype = i32
+    lib.d2c_output_size.argtypes = [i32] * 5
+    lib.d2c_last_error.restype = ctypes.c_char_p
+    lib.d2c_version.restype = ctypes.c_int
+    lib.d2c_get_max_intermediate_elements.restype = ctypes.c_uint64
+    lib.d2c_set_max_intermediate_elements.argtypes = [ctypes.c_uint64]
+    lib.d2c_set_max_intermediate_elements.restype = None
+    lib.d2c_set_algo_override.argtypes = [ctypes.c_int]
+    lib.d2c_set_algo_override.restype = None
+    for name, p in (("conv3d", p3), ("conv1d", p1)):
+        getattr(lib, f"d2c_{name}_check").argtypes = [p]
+        getattr(lib, f"d2c_{name}_check").restype = ctypes.c_int
+        for d in ("forward", "backward"):
+            f = getattr(lib, f"d2c_{name}_{d}_workspace_bytes")
+            f.argtypes, f.restype = [p], sz
+        f = getattr(lib, f"d2c_{name}_forward")
+        f.argtypes, f.restype = [p] + [vp] * 7 + [sz, vp], ctypes.c_int
+        f = getattr(lib, f"d2c_{name}_backward")
+        f.argtypes, f.restype = [p] + [vp] * 11 + [sz, vp], ctypes.c_int
+    lib.d2c_conv3d_algo.argtypes, lib.d2c_conv3d_algo.restype = [p3], ctypes.c_int
+    lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
+    lib.d2c_conv3d_corner_index.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+def last_error():
+    return load().d2c_last_error().decode("utf-8", "replace")
+
+
+def check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what}: {last_error()} (code {rc})")

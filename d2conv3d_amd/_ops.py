@@ -1,0 +1,278 @@
+"""Counterpart of the reference's native module `dconv_native._ops`
+(ops/dconv-native/csrc/ops/dconv.cpp:6-12): `deform_conv1d`, `deform_conv3d`
+with the flat argument lists of dconv1d.h:161-172 / dconv3d.h:188-205, and the
+`config` sub-namespace.  Autograd lives here (torch.autograd.Function) and the
+arithmetic in the C-ABI HIP library.
+"""
+import ctypes
+import types
+
+import torch
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+
+_DT = {torch.float32: _lib.D2C_F32, torch.float64: _lib.D2C_F64, torch.bfloat16: _lib.D2C_BF16}
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream(dev):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _workspace(nbytes, dev):
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+
+def _check_common(nd, input, offset, alpha, weight, bias, groups, offset_groups):
+    """SANITY_CHECK_DCONV_INPUTS / _GROUPS of dconv_gpu_common.h:17-43."""
+    def req(cond, msg):
+        if not cond:
+            raise RuntimeError(f"deform_conv{nd}d: {msg}")
+    for name, t in (("input", input), ("offset", offset), ("weight", weight)):
+        req(isinstance(t, torch.Tensor), f"{name} must be a Tensor")
+        req(t.dim() == nd + 2, f"{name}.ndimension() == {nd + 2} failed (got {t.dim()})")
+    if alpha is not None:
+        req(alpha.dim() == nd + 2, f"alpha.ndimension() == {nd + 2} failed (got {alpha.dim()})")
+    if bias is not None:
+        req(bias.dim() == 1, "bias.ndimension() == 1 failed")
+    for name, t in (("input", input), ("offset", offset), ("alpha", alpha), ("weight", weight), ("bias", bias)):
+        if t is not None:
+            req(t.is_cuda, f"{name}.device().is_cuda() failed: this operator has GPU kernels only")
+            req(t.device == input.device, f"{name} is on {t.device}, input on {input.device}")
+    req(offset.size(0) == input.size(0), "offset.size(0) == input.size(0) failed")
+    if alpha is not None:
+        req(alpha.size(0) == input.size(0), "alpha.size(0) == input.size(0) failed")
+    req(groups > 0 and offset_groups > 0, "group counts must be positive")
+    K = 1
+    for k in weight.shape[2:]:
+        K *= k
+    req(weight.size(1) * groups == input.size(1), "weight.size(1) * n_weight_groups == input.size(1) failed")
+    req(weight.size(0) % groups == 0, "weight.size(0) % n_weight_groups == 0 failed")
+    req(weight.size(0) % offset_groups == 0, "weight.size(0) % n_offset_groups == 0 failed")
+    req(input.size(1) % offset_groups == 0, "input.size(1) % n_offset_groups == 0 failed")
+    req(offset.size(1) == offset_groups * nd * K,
+        f"offset.size(1) == n_offset_groups * {nd} * num_kernel_points failed "
+        f"(got {offset.size(1)}, expected {offset_groups * nd * K})")
+    if alpha is not None:
+        req(alpha.size(1) == offset_groups * K,
+            f"alpha.size(1) == n_offset_groups * num_kernel_points failed "
+            f"(got {alpha.size(1)}, expected {offset_groups * K})")
+        req(tuple(alpha.shape[2:]) == tuple(offset.shape[2:]),
+            f"mask output dims do not match computed dims. Got: {tuple(alpha.shape[2:])} "
+            f"but expected: {tuple(offset.shape[2:])}")
+    if bias is not None:
+        req(bias.size(0) == weight.size(0), "bias.size(0) == weight.size(0) failed")
+
+
+def _unify(input, offset, alpha, weight, bias):
+    """Element types handed to the library: x/weight/bias share `dtype`;
+    offset/mask share `aux_dtype` (= dtype, or float32 next to bfloat16 data)."""
+    dt = input.dtype
+    if dt not in _DT:
+        raise RuntimeError(f"deform_conv: unsupported input dtype {dt}")
+    weight = weight.to(dt)
+    bias = bias.to(dt) if bias is not None else None
+    if dt == torch.bfloat16:
+        adt = torch.bfloat16 if (offset.dtype == torch.bfloat16 and
+                                 (alpha is None or alpha.dtype == torch.bfloat16)) else torch.float32
+    else:
+        adt = dt
+    offset = offset.to(adt)
+    alpha = alpha.to(adt) if alpha is not None else None
+    return input, offset, alpha, weight, bias
+
+
+class _DeformConv3dFunction(torch.autograd.Function):
+    """DeformConv3dFunction of dconv3d.h:70-186."""
+
+    @staticmethod
+    def forward(ctx, input, offset, alpha, weight, bias, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, offset_groups):
+        lib = _lib.load()
+        input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
+        alpha = alpha.contiguous() if alpha is not None else None
+        bias = bias.contiguous() if bias is not None else None
+        N, Cin, D, H, W = input.shape
+        Cout, _, kd, kh, kw = weight.shape
+        Do, Ho, Wo = offset.shape[2:]
+        desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, sd, sh, sw, pd, ph, pw, dd, dh, dw,
+                               groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype])
+        _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d")
+        dev = input.device
+        out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
+        with torch.cuda.device(dev):
+            nb = lib.d2c_conv3d_forward_workspace_bytes(ctypes.byref(desc))
+            ws = _workspace(nb, dev)
+            rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha), _ptr(weight),
+                                        _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
+        _lib.check(rc, "deform_conv3d forward")
+        ctx.save_for_backward(input, offset, alpha, weight, bias)
+        ctx.desc = desc
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        lib = _lib.load()
+        input, offset, alpha, weight, bias = ctx.saved_tensors
+        desc = ctx.desc
+        dev = input.device
+        grad_out = grad_out.contiguous().to(input.dtype)
+        need = ctx.needs_input_grad
+        gx = torch.empty_like(input) if need[0] else None
+        goff = torch.empty_like(offset) if need[1] else None
+        galpha = torch.empty_like(alpha) if (alpha is not None and need[2]) else None
+        gw = torch.empty_like(weight) if need[3] else None
+        gb = torch.empty_like(bias) if (bias is not None and need[4]) else None
+        with torch.cuda.device(dev):
+            nb = lib.d2c_conv3d_backward_workspace_bytes(ctypes.byref(desc))
+            ws = _workspace(nb, dev)
+            rc = lib.d2c_conv3d_backward(ctypes.byref(desc), _ptr(grad_out), _ptr(input), _ptr(offset), _ptr(alpha),
+                                         _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
+                                         _ptr(ws), nb, _stream(dev))
+        _lib.check(rc, "deform_conv3d backward")
+        return (gx, goff, galpha, gw, gb) + (None,) * 11
+
+
+def deform_conv3d(input, offset, alpha, weight, bias, stride_d, stride_h, stride_w, pad_d, pad_h, pad_w,
+                  dilation_d, dilation_h, dilation_w, groups, offset_groups):
+    """deform_conv3d of dconv3d.h:188-226; `alpha` and `bias` may be None."""
+    _check_common(3, input, offset, alpha, weight, bias, groups, offset_groups)
+    input, offset, alpha, weight, bias = _unify(input, offset, alpha, weight, bias)
+    return _DeformConv3dFunction.apply(
+        input, offset, alpha, weight, bias, int(stride_d), int(stride_h), int(stride_w),
+        int(pad_d), int(pad_h), int(pad_w), int(dilation_d), int(dilation_h), int(dilation_w),
+        int(groups), int(offset_groups))
+
+
+class _DeformConv1dFunction(torch.autograd.Function):
+    """DeformConv1dFunction of dconv1d.h:69-159."""
+
+    @staticmethod
+    def forward(ctx, input, offset, alpha, weight, bias, stride, pad, dilation, groups, offset_groups, quirks):
+        lib = _lib.load()
+        input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
+        alpha = alpha.contiguous() if alpha is not None else None
+        bias = bias.contiguous() if bias is not None else None
+        N, Cin, L = input.shape
+        Cout, _, k = weight.shape
+        Lo = offset.shape[2]
+        desc = _lib.Conv1dDesc(N, Cin, Cout, L, k, stride, pad, dilation, groups, offset_groups, Lo,
+                               _DT[input.dtype], _DT[offset.dtype], 1 if quirks else 0)
+        _lib.check(lib.d2c_conv1d_check(ctypes.byref(desc)), "deform_conv1d")
+        dev = input.device
+        out = torch.empty((N, Cout, Lo), dtype=input.dtype, device=dev)
+        with torch.cuda.device(dev):
+            nb = lib.d2c_conv1d_forward_workspace_bytes(ctypes.byref(desc))
+            ws = _workspace(nb, dev)
+            rc = lib.d2c_conv1d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha), _ptr(weight),
+                                        _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
+        _lib.check(rc, "deform_conv1d forward")
+        ctx.save_for_backward(input, offset, alpha, weight, bias)
+        ctx.desc = desc
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        lib = _lib.load()
+        input, offset, alpha, weight, bias = ctx.saved_tensors
+        desc = ctx.desc
+        dev = input.device
+        grad_out = grad_out.contiguous().to(input.dtype)
+        need = ctx.needs_input_grad
+        gx = torch.empty_like(input) if need[0] else None
+        goff = torch.empty_like(offset) if need[1] else None
+        galpha = torch.empty_like(alpha) if (alpha is not None and need[2]) else None
+        gw = torch.empty_like(weight) if need[3] else None
+        gb = torch.empty_like(bias) if (bias is not None and need[4]) else None
+        with torch.cuda.device(dev):
+            nb = lib.d2c_conv1d_backward_workspace_bytes(ctypes.byref(desc))
+            ws = _workspace(nb, dev)
+            rc = lib.d2c_conv1d_backward(ctypes.byref(desc), _ptr(grad_out), _ptr(input), _ptr(offset), _ptr(alpha),
+                                         _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
+                                         _ptr(ws), nb, _stream(dev))
+        _lib.check(rc, "deform_conv1d backward")
+        return (gx, goff, galpha, gw, gb) + (None,) * 6
+
+
+def _one(v):
+    return int(v[0]) if isinstance(v, (tuple, list)) else int(v)
+
+
+def deform_conv1d(input, offset, alpha, weight, bias, stride, pad, dilation, groups, offset_groups,
+                  reference_quirks=True):
+    """deform_conv1d of dconv1d.h:161-187.  Unlike the reference binding, which
+    takes plain ints and defined tensors only, 1-tuples for stride / pad /
+    dilation and None for `alpha` / `bias` are accepted (DeformConv1d.forward,
+    deform_conv.py:168-172, passes exactly those)."""
+    _check_common(1, input, offset, alpha, weight, bias, groups, offset_groups)
+    input, offset, alpha, weight, bias = _unify(input, offset, alpha, weight, bias)
+    return _DeformConv1dFunction.apply(
+        input, offset, alpha, weight, bias, _one(stride), _one(pad), _one(dilation),
+        int(groups), int(offset_groups), bool(reference_quirks))
+
+
+def _get_max_intermediate_elements():
+    return int(_lib.load().d2c_get_max_intermediate_elements())
+
+
+def _set_max_intermediate_elements(m):
+    _lib.load().d2c_set_max_intermediate_elements(int(m))
+
+
+# dconv.cpp:9-11.  Kept for interface parity: no column buffer is ever
+# materialised here, so the limit changes nothing.
+config = types.SimpleNamespace(
+    get_max_intermediate_elements=_get_max_intermediate_elements,
+    set_max_intermediate_elements=_set_max_intermediate_elements,
+)
+
+
+def conv3d_corner_index(input_shape, offset, kernel_size, stride=(1, 1, 1), padding=(0, 0, 0),
+                        dilation=(1, 1, 1), offset_groups=1):
+    """Debug output of the sampler: per (n, g*K+k, p) the int32 floor of the
+    sampling position and the uint8 set of corners the forward pass reads."""
+    lib = _lib.load()
+    offset = offset.contiguous()
+    if offset.dtype == torch.bfloat16:
+        offset = offset.float()
+    N, Cin, D, H, W = input_shape
+    kd, kh, kw = kernel_size
+    Do, Ho, Wo = offset.shape[2:]
+    dt = _DT[offset.dtype]
+    desc = _lib.Conv3dDesc(N, Cin, Cin, D, H, W, kd, kh, kw, *stride, *padding, *dilation,
+                           1, offset_groups, Do, Ho, Wo, dt, dt)
+    K = kd * kh * kw
+    base = torch.empty((N, offset_groups * K, Do * Ho * Wo, 3), dtype=torch.int32, device=offset.device)
+    flags = torch.empty((N, offset_groups * K, Do * Ho * Wo), dtype=torch.uint8, device=offset.device)
+    with torch.cuda.device(offset.device):
+        rc = lib.d2c_conv3d_corner_index(ctypes.byref(desc), _ptr(offset), _ptr(base), _ptr(flags),
+                                         _stream(offset.device))
+    _lib.check(rc, "conv3d_corner_index")
+    return base, flags
+
+
+def conv3d_algo(input, offset, alpha, weight, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
+                groups=1, offset_groups=1):
+    """Name of the kernel family ("generic", "mfma", "depthwise") these arguments are served by."""
+    lib = _lib.load()
+    input, offset, alpha, weight, _ = _unify(input, offset, alpha, weight, None)
+    N, Cin, D, H, W = input.shape
+    Cout, _, kd, kh, kw = weight.shape
+    Do, Ho, Wo = offset.shape[2:]
+    desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, *stride, *padding, *dilation,
+                           groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype])
+    return _lib.ALGO_NAMES.get(lib.d2c_conv3d_algo(ctypes.byref(desc)), "invalid")
+
+
+def set_algo_override(name):
+    """Test hook: force "generic" / "mfma" / "depthwise", or None for the default choice."""
+    code = {None: _lib.ALGO_AUTO, "auto": _lib.ALGO_AUTO, "generic": _lib.ALGO_GENERIC,
+            "mfma": _lib.ALGO_MFMA, "depthwise": _lib.ALGO_DEPTHWISE}[name]
+    _lib.load().d2c_set_algo_override(code)

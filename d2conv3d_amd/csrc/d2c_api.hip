@@ -1,0 +1,253 @@
+// C ABI of the library: argument checks of the reference, kernel-family
+// choice, workspace carving.  Declarations and contracts: include/d2conv.h.
+#include "d2c_common.hpp"
+#include "d2c_tiled.hpp"
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+
+namespace {
+thread_local char g_err[512] = "";
+std::atomic<uint64_t> g_max_intermediate{1ull << 32};  // dconv3d_gpu.cu:12
+std::atomic<int> g_algo_override{D2C_ALGO_AUTO};
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        p[i] = 0u;
+}
+}  // namespace
+
+void d2c_set_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int d2c_check_launch(const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return D2C_OK;
+    d2c_set_error("%s: %s", what, hipGetErrorString(e));
+    return D2C_ERR_LAUNCH;
+}
+
+void d2c_fill_zero(void *p, size_t bytes, hipStream_t st)
+{
+    const size_t n = bytes / 4;
+    if (n == 0) return;
+    size_t g = (n + 255) / 256;
+    if (g > 256 * 32) g = 256 * 32;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)g), dim3(256), 0, st, (uint32_t *)p, n);
+}
+
+#define D2C_REQUIRE(cond, ...)              \
+    do {                                    \
+        if (!(cond)) {                      \
+            d2c_set_error(__VA_ARGS__);     \
+            return D2C_ERR_SHAPE;           \
+        }                                   \
+    } while (0)
+
+extern "C" {
+
+int32_t d2c_output_size(int32_t in, int32_t k, int32_t stride, int32_t pad, int32_t dil)
+{
+    return (in + 2 * pad - (dil * (k - 1) + 1)) / stride + 1;
+}
+
+const char *d2c_last_error(void) { return g_err; }
+int d2c_version(void) { return 1; }
+uint64_t d2c_get_max_intermediate_elements(void) { return g_max_intermediate.load(); }
+void d2c_set_max_intermediate_elements(uint64_t m) { g_max_intermediate.store(m); }
+void d2c_set_algo_override(int algo) { g_algo_override.store(algo); }
+
+static int check_dtypes(int dtype, int aux)
+{
+    if (dtype != D2C_F32 && dtype != D2C_F64 && dtype != D2C_BF16) {
+        d2c_set_error("unsupported dtype code %d", dtype);
+        return D2C_ERR_DTYPE;
+    }
+    if (!(aux == dtype || (dtype == D2C_BF16 && aux == D2C_F32))) {
+        d2c_set_error("aux_dtype %d does not go with dtype %d (offset/mask are of the input's type, or float32 for bfloat16 inputs)", aux, dtype);
+        return D2C_ERR_DTYPE;
+    }
+    return D2C_OK;
+}
+
+// Checks of dconv_gpu_common.h:17-24 (groups) and dconv3d_gpu.cu:504-527
+// (sizes).  Channel counts of offset / mask are implied by the descriptor; the
+// host wrapper compares them with the tensors it holds.
+int d2c_conv3d_check(const d2c_conv3d_desc *q)
+{
+    if (!q) { d2c_set_error("null descriptor"); return D2C_ERR_SHAPE; }
+    if (int rc = check_dtypes(q->dtype, q->aux_dtype)) return rc;
+    D2C_REQUIRE(q->N > 0 && q->Cin > 0 && q->Cout > 0 && q->D > 0 && q->H > 0 && q->W > 0, "empty input");
+    D2C_REQUIRE(q->groups > 0 && q->offset_groups > 0, "group counts must be positive");
+    D2C_REQUIRE(q->Cin % q->groups == 0, "weight.size(1) * n_weight_groups == input.size(1) failed");
+    D2C_REQUIRE(q->Cout % q->groups == 0, "weight.size(0) %% n_weight_groups == 0 failed");
+    D2C_REQUIRE(q->Cout % q->offset_groups == 0, "weight.size(0) %% n_offset_groups == 0 failed");
+    D2C_REQUIRE(q->Cin % q->offset_groups == 0, "input.size(1) %% n_offset_groups == 0 failed");
+    D2C_REQUIRE(q->kd > 0 && q->kh > 0 && q->kw > 0, "kernel size must be positive");
+    D2C_REQUIRE(q->sd > 0 && q->sh > 0 && q->sw > 0, "stride must be positive");
+    D2C_REQUIRE(q->pd >= 0 && q->ph >= 0 && q->pw >= 0, "padding must be non-negative");
+    D2C_REQUIRE(q->dd > 0 && q->dh > 0 && q->dw > 0, "dilation must be positive");
+    const int od = d2c_output_size(q->D, q->kd, q->sd, q->pd, q->dd);
+    const int oh = d2c_output_size(q->H, q->kh, q->sh, q->ph, q->dh);
+    const int ow = d2c_output_size(q->W, q->kw, q->sw, q->pw, q->dw);
+    D2C_REQUIRE(od > 0 && oh > 0 && ow > 0, "computed output size (%d, %d, %d) must be positive", od, oh, ow);
+    D2C_REQUIRE(q->Do == od && q->Ho == oh && q->Wo == ow,
+                "offset output dims do not match computed dims. Got: (%d, %d, %d) but expected: (%d, %d, %d)",
+                q->Do, q->Ho, q->Wo, od, oh, ow);
+    const long K = (long)q->kd * q->kh * q->kw, P = (long)od * oh * ow;
+    D2C_REQUIRE((long)q->N * q->Cin * q->D * q->H * q->W < (1L << 31) && (long)q->N * q->Cout * P < (1L << 31)
+                    && (long)q->N * q->offset_groups * 3 * K * P < (1L << 31)
+                    && (long)q->Cout * (q->Cin / q->groups) * K < (1L << 31),
+                "tensor with 2^31 or more elements is not supported");
+    return D2C_OK;
+}
+
+int d2c_conv1d_check(const d2c_conv1d_desc *q)
+{
+    if (!q) { d2c_set_error("null descriptor"); return D2C_ERR_SHAPE; }
+    if (int rc = check_dtypes(q->dtype, q->aux_dtype)) return rc;
+    D2C_REQUIRE(q->N > 0 && q->Cin > 0 && q->Cout > 0 && q->L > 0, "empty input");
+    D2C_REQUIRE(q->groups > 0 && q->offset_groups > 0, "group counts must be positive");
+    D2C_REQUIRE(q->Cin % q->groups == 0, "weight.size(1) * n_weight_groups == input.size(1) failed");
+    D2C_REQUIRE(q->Cout % q->groups == 0, "weight.size(0) %% n_weight_groups == 0 failed");
+    D2C_REQUIRE(q->Cout % q->offset_groups == 0, "weight.size(0) %% n_offset_groups == 0 failed");
+    D2C_REQUIRE(q->Cin % q->offset_groups == 0, "input.size(1) %% n_offset_groups == 0 failed");
+    D2C_REQUIRE(q->k > 0, "kernel size must be positive");
+    D2C_REQUIRE(q->s > 0, "stride must be positive");
+    D2C_REQUIRE(q->p >= 0, "padding must be non-negative");
+    D2C_REQUIRE(q->d > 0, "dilation must be positive");
+    const int lo = d2c_output_size(q->L, q->k, q->s, q->p, q->d);
+    D2C_REQUIRE(lo > 0, "computed output size %d must be positive", lo);
+    D2C_REQUIRE(q->Lo == lo, "offset output dims do not match computed dims. Got: %d but expected: %d", q->Lo, lo);
+    D2C_REQUIRE((long)q->N * q->Cin * q->L < (1L << 31) && (long)q->N * q->Cout * lo < (1L << 31)
+                    && (long)q->Cout * (q->Cin / q->groups) * q->k < (1L << 31),
+                "tensor with 2^31 or more elements is not supported");
+    return D2C_OK;
+}
+
+static int choose_algo(const d2c_conv3d_desc &q, bool quiet)
+{
+    const int forced = g_algo_override.load();
+    const bool tiled_ok = d2c_tiled_supported(q);
+    if (forced == D2C_ALGO_GENERIC) return D2C_ALGO_GENERIC;
+    if (forced == D2C_ALGO_MFMA || forced == D2C_ALGO_DEPTHWISE) {
+        const int a = tiled_ok ? d2c_tiled_algo(q) : D2C_ALGO_GENERIC;
+        if (a != forced) {
+            if (!quiet) d2c_set_error("forced kernel family %d cannot serve this description", forced);
+            return -1;
+        }
+        return a;
+    }
+    return tiled_ok ? d2c_tiled_algo(q) : D2C_ALGO_GENERIC;
+}
+
+int d2c_conv3d_algo(const d2c_conv3d_desc *q)
+{
+    if (d2c_conv3d_check(q) != D2C_OK) return -1;
+    return choose_algo(*q, true);
+}
+
+size_t d2c_conv3d_forward_workspace_bytes(const d2c_conv3d_desc *q)
+{
+    if (d2c_conv3d_check(q) != D2C_OK) return 0;
+    const int a = choose_algo(*q, true);
+    if (a == D2C_ALGO_MFMA || a == D2C_ALGO_DEPTHWISE) return d2c_tiled_forward_ws(*q);
+    return 0;
+}
+
+size_t d2c_conv3d_backward_workspace_bytes(const d2c_conv3d_desc *q)
+{
+    if (d2c_conv3d_check(q) != D2C_OK) return 0;
+    const int a = choose_algo(*q, true);
+    if (a == D2C_ALGO_MFMA || a == D2C_ALGO_DEPTHWISE) return d2c_tiled_backward_ws(*q);
+    return d2c_generic_conv3d_backward_ws(*q);
+}
+
+static int check_ws(size_t need, void *ws, size_t have)
+{
+    if (need == 0) return D2C_OK;
+    if (!ws || have < need || ((uintptr_t)ws & 255u)) {
+        d2c_set_error("workspace of %zu bytes (256-byte aligned) required, got %zu at %p", need, have, ws);
+        return D2C_ERR_WORKSPACE;
+    }
+    return D2C_OK;
+}
+
+int d2c_conv3d_forward(const d2c_conv3d_desc *q, const void *x, const void *offset, const void *mask,
+                       const void *weight, const void *bias, void *out, void *ws, size_t ws_bytes, void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!x || !offset || !weight || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    const int a = choose_algo(*q, false);
+    if (a < 0) return D2C_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (a == D2C_ALGO_GENERIC) return d2c_generic_conv3d_forward(*q, x, offset, mask, weight, bias, out, st);
+    if (int rc = check_ws(d2c_tiled_forward_ws(*q), ws, ws_bytes)) return rc;
+    return d2c_tiled_forward(*q, x, offset, mask, weight, bias, out, ws, st);
+}
+
+int d2c_conv3d_backward(const d2c_conv3d_desc *q, const void *gout, const void *x, const void *offset,
+                        const void *mask, const void *weight, void *gx, void *goff, void *gmask, void *gw,
+                        void *gb, void *ws, size_t ws_bytes, void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!gout || !x || !offset || !weight) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    const int a = choose_algo(*q, false);
+    if (a < 0) return D2C_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (a == D2C_ALGO_GENERIC) {
+        if (int rc = check_ws(d2c_generic_conv3d_backward_ws(*q), ws, ws_bytes)) return rc;
+        return d2c_generic_conv3d_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws, st);
+    }
+    if (int rc = check_ws(d2c_tiled_backward_ws(*q), ws, ws_bytes)) return rc;
+    return d2c_tiled_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws, st);
+}
+
+int d2c_conv3d_corner_index(const d2c_conv3d_desc *q, const void *offset, int32_t *base, uint8_t *flags,
+                            void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!offset || !base || !flags) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    return d2c_generic_conv3d_corners(*q, offset, base, flags, (hipStream_t)stream);
+}
+
+size_t d2c_conv1d_forward_workspace_bytes(const d2c_conv1d_desc *q)
+{
+    if (d2c_conv1d_check(q) != D2C_OK) return 0;
+    return 0;
+}
+
+size_t d2c_conv1d_backward_workspace_bytes(const d2c_conv1d_desc *q)
+{
+    if (d2c_conv1d_check(q) != D2C_OK) return 0;
+    return d2c_generic_conv1d_backward_ws(*q);
+}
+
+int d2c_conv1d_forward(const d2c_conv1d_desc *q, const void *x, const void *offset, const void *mask,
+                       const void *weight, const void *bias, void *out, void *ws, size_t ws_bytes, void *stream)
+{
+    (void)ws; (void)ws_bytes;
+    if (int rc = d2c_conv1d_check(q)) return rc;
+    if (!x || !offset || !weight || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    return d2c_generic_conv1d_forward(*q, x, offset, mask, weight, bias, out, (hipStream_t)stream);
+}
+
+int d2c_conv1d_backward(const d2c_conv1d_desc *q, const void *gout, const void *x, const void *offset,
+                        const void *mask, const void *weight, void *gx, void *goff, void *gmask, void *gw,
+                        void *gb, void *ws, size_t ws_bytes, void *stream)
+{
+    if (int rc = d2c_conv1d_check(q)) return rc;
+    if (!gout || !x || !offset || !weight) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (int rc = check_ws(d2c_generic_conv1d_backward_ws(*q), ws, ws_bytes)) return rc;
+    return d2c_generic_conv1d_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws,
+                                       (hipStream_t)stream);
+}
+
+}  // extern "C"

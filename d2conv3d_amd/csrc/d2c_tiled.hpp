@@ -1,0 +1,14 @@
+// Host interface of the tiled kernel families (matrix-core implicit GEMM and
+// the depthwise bandwidth kernels).
+#pragma once
+#include "d2c_common.hpp"
+
+bool d2c_tiled_supported(const d2c_conv3d_desc &q);
+int d2c_tiled_algo(const d2c_conv3d_desc &q);  // D2C_ALGO_MFMA or D2C_ALGO_DEPTHWISE
+size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q);
+size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q);
+int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
+                      const void *bias, void *out, void *ws, hipStream_t st);
+int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
+                       const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
+                       void *ws, hipStream_t st);

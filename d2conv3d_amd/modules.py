@@ -1,0 +1,241 @@
+"""Self-deforming layers: a zero-initialised Conv3d predicts offsets (and
+modulation) for a DeformConv3d with the same geometry.  Mirrors
+ops/dconv-native/src/dconv_native/modules.py and the application's superset of
+it in network/layers.py:18-313 (norm on the deformation input, `init`,
+`size_activation`, the XXZ variant, activation checkpointing).
+
+Constructor arguments follow network/layers.py:27-30; the operator package's
+shorter list (modules.py:17-19) is its prefix, and a `deform_param_op` given in
+the position of `init` is recognised as such.
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.nn.modules.utils import _triple
+from torch.utils.checkpoint import checkpoint
+
+from .deform_conv import DeformConv3d
+from .grid import offsets_from_size_map
+
+
+def _apply_size_activation(activation_mode, size_map):
+    # network/layers.py:171-181
+    if activation_mode == "elu":
+        return F.elu(size_map) + 1
+    if activation_mode == "relu":
+        return F.relu(size_map + 1)
+    if activation_mode == "relu_plus_one":
+        return F.relu(size_map + 1e-3) + 1
+    if activation_mode == "linear":
+        return size_map
+    raise ValueError(f"Unexpected size activation mode '{activation_mode}'")
+
+
+class _DConvBase(nn.Module):
+    _activations = {
+        "sigmoid": torch.sigmoid,
+        "relu": torch.relu,
+        "tanh": torch.tanh,
+        "linear": lambda x: x,
+        "none": lambda x: x,
+    }
+    # network/layers.py:99 wraps the deformation branch in torch.utils.checkpoint;
+    # the operator package (modules.py:62-64) does not.  Same numbers either way.
+    checkpoint_deformation = False
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, offset_groups=1, bias=True, activation="sigmoid", init="zero",
+                 norm_type="none", norm_groups=1, size_activation="elu", deform_param_op=nn.Conv3d):
+        super().__init__()
+        if not isinstance(init, str):  # modules.py:17-19: 11th positional is deform_param_op
+            deform_param_op, init = init, "zero"
+        kernel_size = _triple(kernel_size)
+        self.num_kernel_points = kernel_size[0] * kernel_size[1] * kernel_size[2]
+        self.offset_groups = offset_groups
+        self.groups = groups
+        self.size_activation = size_activation
+
+        if norm_type not in ("BatchNorm", "GroupNorm", "none"):
+            raise ValueError(f"Unexpected norm_type: '{norm_type}'")
+        if norm_type == "GroupNorm":
+            self.norm = nn.GroupNorm(norm_groups, in_channels)
+        elif norm_type == "BatchNorm":
+            self.norm = nn.BatchNorm3d(in_channels)
+        else:
+            self.norm = None
+
+        # construction order deform_params -> deform_conv keeps the RNG stream of the reference
+        if isinstance(deform_param_op, nn.Module):
+            self.deform_params = deform_param_op
+        else:
+            self.deform_params = deform_param_op(in_channels, self._deform_channels(), kernel_size,
+                                                 stride, padding, dilation, 1, bias)
+        self.deform_conv = DeformConv3d(in_channels, out_channels, kernel_size, stride, padding,
+                                        dilation, groups, offset_groups, bias)
+        self.activation = self._activations[activation] if isinstance(activation, str) else activation
+        if not isinstance(deform_param_op, nn.Module):
+            self._init_deform_params(activation, init)
+
+    def _init_deform_params(self, activation, init):
+        # network/layers.py:79-86
+        if init == "zero":
+            nn.init.zeros_(self.deform_params.weight)
+            if self.deform_params.bias is not None:
+                nn.init.zeros_(self.deform_params.bias)
+        else:
+            raise ValueError(f"init scheme {init} not supported")
+
+    def _deform_channels(self):
+        return 3 * self.offset_groups * self.num_kernel_points
+
+    def _get_deformation(self, input):
+        return self.deform_params(input), None
+
+    def forward(self, input):
+        deform_input = input if self.norm is None else self.norm(input)
+        if self.checkpoint_deformation and torch.is_grad_enabled():
+            deformation = checkpoint(self._get_deformation, deform_input, use_reentrant=False)
+        else:
+            deformation = self._get_deformation(deform_input)
+        return self.deform_conv(input, *deformation)
+
+
+class DConv3d(_DConvBase):
+    pass
+
+
+class MDConv3d(_DConvBase):
+    def _deform_channels(self):
+        self.offset_channels = 3 * self.offset_groups * self.num_kernel_points
+        self.alpha_channels = self.offset_groups * self.num_kernel_points
+        return self.offset_channels + self.alpha_channels
+
+    def _get_deformation(self, input):
+        deformation = self.deform_params(input)
+        offset, alpha = torch.split(deformation, [self.offset_channels, self.alpha_channels], dim=1)
+        return offset, self.activation(alpha)
+
+    def _init_deform_params(self, activation, init):
+        # network/layers.py:122-132
+        if init == "zero":
+            nn.init.zeros_(self.deform_params.weight)
+        elif init == "random":
+            with torch.no_grad():
+                if activation == "sigmoid" or activation == "tanh":
+                    nn.init.xavier_normal_(self.deform_params.weight[self.offset_channels:])
+                else:
+                    nn.init.kaiming_normal_(self.deform_params.weight[self.offset_channels:])
+        if self.deform_params.bias is not None:
+            nn.init.zeros_(self.deform_params.bias)
+
+
+class _SpatialMixin:
+    def _get_deformation(self, input):
+        # modules.py:87-101: no displacement along the temporal axis
+        offsets, alpha = super()._get_deformation(input)
+        offsets = offsets.clone()
+        offsets[:, ::3] = 0
+        return offsets, alpha
+
+
+class _TemporalMixin:
+    def _get_deformation(self, input):
+        # modules.py:104-120: displacement along the temporal axis only
+        offsets, alpha = super()._get_deformation(input)
+        offsets = offsets.clone()
+        offsets[:, 1::3] = 0
+        offsets[:, 2::3] = 0
+        return offsets, alpha
+
+
+class SpatialDConv3d(_SpatialMixin, DConv3d):
+    pass
+
+
+class SpatialMDConv3d(_SpatialMixin, MDConv3d):
+    pass
+
+
+class TemporalDConv3d(_TemporalMixin, DConv3d):
+    pass
+
+
+class TemporalMDConv3d(_TemporalMixin, MDConv3d):
+    pass
+
+
+class _SizeConditionedD(DConv3d):
+    """modules.py:123-159 / network/layers.py:184-230: the deformation branch
+    predicts a dilation ("size") per location and axis subset; offsets follow
+    from offsets_from_size_map.  Emits 3*K offset channels, i.e. offset_groups=1."""
+    _size_channels = 1
+    _mode = "x"
+
+    def _deform_channels(self):
+        self.offset_channels = self._size_channels
+        return self.offset_channels
+
+    def _get_deformation(self, input):
+        size_map = _apply_size_activation(self.size_activation, self.deform_params(input))
+        offsets = offsets_from_size_map(size_map, self._mode, self.deform_conv.kernel_size,
+                                        self.deform_conv.dilation)
+        return offsets, None
+
+
+class _SizeConditionedMD(MDConv3d):
+    """modules.py:162-219 / network/layers.py:233-313."""
+    _size_channels = 1
+    _mode = "x"
+
+    def _deform_channels(self):
+        self.alpha_channels = self.offset_groups * self.num_kernel_points
+        self.offset_channels = self._size_channels
+        return self.offset_channels + self.alpha_channels
+
+    def _get_deformation(self, input):
+        deformation = self.deform_params(input)
+        size_map, alpha = torch.split(deformation, [self._size_channels, self.alpha_channels], dim=1)
+        size_map = _apply_size_activation(self.size_activation, size_map)
+        offsets = offsets_from_size_map(size_map, self._mode, self.deform_conv.kernel_size,
+                                        self.deform_conv.dilation)
+        return offsets, self.activation(alpha)
+
+
+class SizeConditionedDConv3d(_SizeConditionedD):
+    _size_channels, _mode = 1, "x"
+
+
+class XYSizeConditionedDConv3d(_SizeConditionedD):
+    _size_channels, _mode = 2, "xy"
+
+
+class XXZSizeConditionedDConv3d(_SizeConditionedD):
+    _size_channels, _mode = 2, "xxz"
+
+
+class XYZSizeConditionedDConv3d(_SizeConditionedD):
+    _size_channels, _mode = 3, "xyz"
+
+
+class SizeConditionedMDConv3d(_SizeConditionedMD):
+    _size_channels, _mode = 1, "x"
+
+
+class XYSizeConditionedMDConv3d(_SizeConditionedMD):
+    _size_channels, _mode = 2, "xy"
+
+
+class XXZSizeConditionedMDConv3d(_SizeConditionedMD):
+    _size_channels, _mode = 2, "xxz"
+
+
+class XYZSizeConditionedMDConv3d(_SizeConditionedMD):
+    _size_channels, _mode = 3, "xyz"
+
+
+__all__ = [
+    "DConv3d", "MDConv3d", "SpatialDConv3d", "SpatialMDConv3d", "TemporalDConv3d", "TemporalMDConv3d",
+    "SizeConditionedDConv3d", "XYSizeConditionedDConv3d", "XXZSizeConditionedDConv3d",
+    "XYZSizeConditionedDConv3d", "SizeConditionedMDConv3d", "XYSizeConditionedMDConv3d",
+    "XXZSizeConditionedMDConv3d", "XYZSizeConditionedMDConv3d",
+]

@@ -1,0 +1,71 @@
+"""nn.Conv3d -> deformable layer replacement, mirroring
+ops/dconv-native/src/dconv_native/util.py and utils/replace.py:11-82.
+"""
+import torch.nn as nn
+
+from .modules import *  # noqa: F401,F403  (the reference's util.py re-exports the layer classes)
+from . import modules as _m
+
+
+def replace_module(replacement_func, replaced_cls, module, **kwargs):
+    """util.py:4-21: depth-first replacement; returns (module, number of replacements)."""
+    n_conversions = 0
+    module_output = module
+    if isinstance(module, replaced_cls):
+        module_output = replacement_func(module, **kwargs)
+        n_conversions += 1 if module_output is not module else 0
+    for name, child in module.named_children():
+        converted, conversions = replace_module(replacement_func, replaced_cls, child, **kwargs)
+        module_output.add_module(name, converted)
+        n_conversions += conversions
+    return module_output, n_conversions
+
+
+# util.py:24-37 and utils/replace.py:30-47 (union of both name tables)
+_dconv_versions = {
+    "DCNv1": _m.DConv3d,
+    "DCNv2": _m.MDConv3d,
+    "SpatialDCNv1": _m.SpatialDConv3d,
+    "SpatialDCNv2": _m.SpatialMDConv3d,
+    "TemporalDCNv1": _m.TemporalDConv3d,
+    "TemporalDCNv2": _m.TemporalMDConv3d,
+    "ConditionedDCNv1": _m.SizeConditionedDConv3d,
+    "SizeConditionedDCNv1": _m.SizeConditionedDConv3d,
+    "XYConditionedDCNv1": _m.XYSizeConditionedDConv3d,
+    "XYSizeConditionedDCNv1": _m.XYSizeConditionedDConv3d,
+    "XXZConditionedDCNv1": _m.XXZSizeConditionedDConv3d,
+    "XYZConditionedDCNv1": _m.XYZSizeConditionedDConv3d,
+    "XYZSizeConditionedDCNv1": _m.XYZSizeConditionedDConv3d,
+    "ConditionedDCNv2": _m.SizeConditionedMDConv3d,
+    "SizeConditionedDCNv2": _m.SizeConditionedMDConv3d,
+    "XYConditionedDCNv2": _m.XYSizeConditionedMDConv3d,
+    "XYSizeConditionedDCNv2": _m.XYSizeConditionedMDConv3d,
+    "XXZConditionedDCNv2": _m.XXZSizeConditionedMDConv3d,
+    "XYZConditionedDCNv2": _m.XYZSizeConditionedMDConv3d,
+    "XYZSizeConditionedDCNv2": _m.XYZSizeConditionedMDConv3d,
+}
+
+
+def dconv_replace_layer(conv_module, **kwargs):
+    """utils/replace.py:48-78: 1x1x1 kernels are kept unless `replace_1x1_kernels`;
+    weight and bias of the convolution are carried over."""
+    if not kwargs.get("replace_1x1_kernels") and conv_module.kernel_size == (1, 1, 1):
+        return conv_module
+    DC = _dconv_versions[kwargs["version"]]
+    dconv = DC(
+        conv_module.in_channels, conv_module.out_channels, conv_module.kernel_size,
+        conv_module.stride, conv_module.padding, conv_module.dilation, conv_module.groups,
+        kwargs.get("offset_groups", 1), conv_module.bias is not None,
+        kwargs.get("activation", "sigmoid"), kwargs.get("init", "zero"),
+        kwargs.get("norm_type", "none"), kwargs.get("norm_groups", 1),
+        kwargs.get("size_activation", "elu"),
+    )
+    dconv.deform_conv.weight.data = conv_module.weight.data.detach()
+    if conv_module.bias is not None:
+        dconv.deform_conv.bias.data = conv_module.bias.data.detach()
+    return dconv
+
+
+def add_deformable_conv(module, **kwargs):
+    """util.py:62-63."""
+    return replace_module(dconv_replace_layer, nn.Conv3d, module, **kwargs)

@@ -1,0 +1,142 @@
+/*
+ * d2conv.h -- C ABI of the MI355X (gfx950) D2Conv3D operator library.
+ *
+ * One entry point per native function that the reference's Python extension
+ * binds (ops/dconv-native/csrc/ops/dconv.cpp:6-12):
+ *
+ *   d2c_conv3d_forward    <- deform_conv3d_forward_cuda   (dconv3d_gpu.h:5-16,  dconv3d_gpu.cu:460-560)
+ *   d2c_conv3d_backward   <- deform_conv3d_backward_cuda  (dconv3d_gpu.h:18-30, dconv3d_gpu.cu:1261-1332)
+ *   d2c_conv1d_forward    <- deform_conv1d_forward_cuda   (dconv1d_gpu.h:6-18,  dconv1d_gpu.cu:102-204)
+ *   d2c_conv1d_backward   <- deform_conv1d_backward_cuda  (dconv1d_gpu.h:20-32, dconv1d_gpu.cu:403-542)
+ *   d2c_get/set_max_intermediate_elements
+ *                         <- get/set_max_intermediate_elements (dconv3d_gpu.cu:12-14, dconv.cpp:9-11)
+ *   d2c_conv3d_check / d2c_conv1d_check
+ *                         <- SANITY_CHECK_DCONV_GROUPS and the size checks
+ *                            (dconv_gpu_common.h:17-24, dconv3d_gpu.cu:504-512)
+ *
+ * Conventions
+ *   - All pointers are device pointers to contiguous tensors in the reference's
+ *     layouts:  x [N,Cin,D,H,W], offset [N,G*3*K,Do,Ho,Wo] with channel order
+ *     (g, kd, kh, kw, (dz,dy,dx)), mask [N,G*K,Do,Ho,Wo] (may be NULL),
+ *     weight [Cout,Cin/groups,kd,kh,kw], bias [Cout] (may be NULL),
+ *     out [N,Cout,Do,Ho,Wo]; 1-D: x [N,Cin,L], offset/mask [N,G*K,Lo].
+ *   - `dtype` is the element type of x, weight, bias, out and of their
+ *     gradients; `aux_dtype` is the element type of offset, mask and their
+ *     gradients (equal to dtype, or D2C_F32 when dtype is D2C_BF16).
+ *   - The library allocates nothing.  Scratch memory comes from the caller:
+ *     ask d2c_*_workspace_bytes() and pass a device buffer of at least that
+ *     size, 256-byte aligned.  Its contents are undefined afterwards.
+ *   - Every output is fully overwritten; the caller need not clear it.
+ *     In the backward calls a NULL gradient pointer skips that gradient.
+ *   - `stream` is a hipStream_t (NULL = the default stream).  Calls only
+ *     enqueue work; they do not synchronise.
+ *   - Return value 0 = success; otherwise a D2C_ERR_* code, with a text for
+ *     the calling thread in d2c_last_error().  Nothing throws across the ABI.
+ */
+#ifndef D2CONV_H
+#define D2CONV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { D2C_F32 = 0, D2C_F64 = 1, D2C_BF16 = 2 };
+
+enum {
+    D2C_OK = 0,
+    D2C_ERR_SHAPE = 1,      /* a check of the reference failed (message names it) */
+    D2C_ERR_DTYPE = 2,
+    D2C_ERR_WORKSPACE = 3,  /* workspace NULL, misaligned or too small */
+    D2C_ERR_LAUNCH = 4,     /* HIP reported an error at launch */
+    D2C_ERR_UNSUPPORTED = 5
+};
+
+/* Which kernel family a description is served by (d2c_conv3d_algo). */
+enum {
+    D2C_ALGO_AUTO = 0,
+    D2C_ALGO_GENERIC = 1,   /* direct kernels, any shape, f32/f64/bf16 */
+    D2C_ALGO_MFMA = 2,      /* implicit GEMM on matrix cores, f32/bf16 */
+    D2C_ALGO_DEPTHWISE = 3  /* groups == Cin == Cout, bandwidth kernels */
+};
+
+typedef struct d2c_conv3d_desc {
+    int32_t N, Cin, Cout;
+    int32_t D, H, W;
+    int32_t kd, kh, kw;
+    int32_t sd, sh, sw;
+    int32_t pd, ph, pw;
+    int32_t dd, dh, dw;
+    int32_t groups, offset_groups;
+    int32_t Do, Ho, Wo;   /* spatial size of offset / mask / out as passed by the caller */
+    int32_t dtype, aux_dtype;
+} d2c_conv3d_desc;
+
+typedef struct d2c_conv1d_desc {
+    int32_t N, Cin, Cout;
+    int32_t L, k, s, p, d;
+    int32_t groups, offset_groups;
+    int32_t Lo;
+    int32_t dtype, aux_dtype;
+    int32_t reference_quirks; /* !=0: integer-position rule of dconv1d_gpu.cu:332-336 in grad_offset/grad_mask */
+} d2c_conv1d_desc;
+
+/* get_output_size, dconv_gpu_common.h:13-15 */
+int32_t d2c_output_size(int32_t in, int32_t k, int32_t stride, int32_t pad, int32_t dil);
+
+int d2c_conv3d_check(const d2c_conv3d_desc *desc);
+int d2c_conv3d_algo(const d2c_conv3d_desc *desc);
+size_t d2c_conv3d_forward_workspace_bytes(const d2c_conv3d_desc *desc);
+size_t d2c_conv3d_backward_workspace_bytes(const d2c_conv3d_desc *desc);
+
+int d2c_conv3d_forward(const d2c_conv3d_desc *desc, const void *x, const void *offset,
+                       const void *mask, const void *weight, const void *bias, void *out,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+int d2c_conv3d_backward(const d2c_conv3d_desc *desc, const void *grad_out, const void *x,
+                        const void *offset, const void *mask, const void *weight,
+                        void *grad_x, void *grad_offset, void *grad_mask, void *grad_weight,
+                        void *grad_bias, void *workspace, size_t workspace_bytes, void *stream);
+
+int d2c_conv1d_check(const d2c_conv1d_desc *desc);
+size_t d2c_conv1d_forward_workspace_bytes(const d2c_conv1d_desc *desc);
+size_t d2c_conv1d_backward_workspace_bytes(const d2c_conv1d_desc *desc);
+
+int d2c_conv1d_forward(const d2c_conv1d_desc *desc, const void *x, const void *offset,
+                       const void *mask, const void *weight, const void *bias, void *out,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+int d2c_conv1d_backward(const d2c_conv1d_desc *desc, const void *grad_out, const void *x,
+                        const void *offset, const void *mask, const void *weight,
+                        void *grad_x, void *grad_offset, void *grad_mask, void *grad_weight,
+                        void *grad_bias, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Sampling bookkeeping of the forward pass, for index-exactness checks
+ * (trilinear_interpolate, dconv3d_gpu.cu:59-86): per (n, g*K+k, p)
+ *   base[.][3] = floor(z), floor(y), floor(x) as int32 (positions beyond 4
+ *                voxels outside the volume are clamped there first),
+ *   flags[.]   = bit c set (c = 4*dz + 2*dy + dx) when corner c is read.
+ */
+int d2c_conv3d_corner_index(const d2c_conv3d_desc *desc, const void *offset, int32_t *base,
+                            uint8_t *flags, void *stream);
+
+/* Accepted for interface parity; the library never materialises the column
+ * buffer that this limit governs in the reference (dconv3d_gpu.cu:536-553). */
+uint64_t d2c_get_max_intermediate_elements(void);
+void d2c_set_max_intermediate_elements(uint64_t m);
+
+/* Test hook: force a kernel family (D2C_ALGO_*; D2C_ALGO_AUTO restores the
+ * default choice).  A forced family that cannot serve a description makes the
+ * call fail with D2C_ERR_UNSUPPORTED. */
+void d2c_set_algo_override(int algo);
+
+const char *d2c_last_error(void);
+int d2c_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* D2CONV_H */
