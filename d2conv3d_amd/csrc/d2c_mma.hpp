@@ -1,0 +1,127 @@
+// Matrix-core building blocks shared by the tiled kernels (gfx950, wave64).
+//
+// All operands move in 16-byte vectors: VEC = 8 bfloat16 or 4 float channels.
+// A "k-group" is two such vectors (lane half h = lane / 32 takes vector
+// 2*kg + h): 16 bf16 channels = one v_mfma_f32_32x32x16_bf16, or 8 float
+// channels = four v_mfma_f32_32x32x2_f32 (element i of both operands' vectors
+// feeds MFMA i, so the channel permutation is the same on both sides and the
+// sum is unchanged).
+//
+// Fragment layout of the 32x32 MFMAs (A is M x K, B is K x N, D is M x N):
+//   A: lane l holds row  m = l % 32, its k-slice chosen by l / 32
+//   B: lane l holds col  n = l % 32, same k-slice
+//   D: lane l holds col  n = l % 32, rows m = 8*(r/4) + 4*(l/32) + r%4 for r = 0..15
+#pragma once
+#include "d2c_common.hpp"
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> struct Elem;
+template <> struct Elem<bf16_t> {
+    static constexpr int VEC = 8;          // channels per 16-byte vector
+    static constexpr int DT = D2C_BF16;
+};
+template <> struct Elem<float> {
+    static constexpr int VEC = 4;
+    static constexpr int DT = D2C_F32;
+};
+
+template <typename T> D2C_DEV void mma_kgroup(f32x16 &acc, const uint4 &a, const uint4 &b);
+template <> D2C_DEV void mma_kgroup<bf16_t>(f32x16 &acc, const uint4 &a, const uint4 &b)
+{
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                  acc, 0, 0, 0);
+}
+template <> D2C_DEV void mma_kgroup<float>(f32x16 &acc, const uint4 &a, const uint4 &b)
+{
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
+}
+
+// Two floats -> packed bfloat16 pair (round to nearest even), low half first.
+D2C_DEV uint32_t pack_bf16x2(float lo, float hi)
+{
+    f32x2 v = {lo, hi};
+    bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// acc[i] += w * v[i] over one 16-byte vector of channels (fp32 accumulation).
+template <typename T> struct VecAcc;
+template <> struct VecAcc<bf16_t> {
+    float a[8];
+    D2C_DEV void zero() {
+#pragma unroll
+        for (int i = 0; i < 8; i++) a[i] = 0.f;
+    }
+    D2C_DEV void fma(float w, const uint4 &v)
+    {
+        a[0] = fmaf(w, __uint_as_float(v.x << 16), a[0]);
+        a[1] = fmaf(w, __uint_as_float(v.x & 0xffff0000u), a[1]);
+        a[2] = fmaf(w, __uint_as_float(v.y << 16), a[2]);
+        a[3] = fmaf(w, __uint_as_float(v.y & 0xffff0000u), a[3]);
+        a[4] = fmaf(w, __uint_as_float(v.z << 16), a[4]);
+        a[5] = fmaf(w, __uint_as_float(v.z & 0xffff0000u), a[5]);
+        a[6] = fmaf(w, __uint_as_float(v.w << 16), a[6]);
+        a[7] = fmaf(w, __uint_as_float(v.w & 0xffff0000u), a[7]);
+    }
+    D2C_DEV uint4 pack() const
+    {
+        return make_uint4(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(a[4], a[5]),
+                          pack_bf16x2(a[6], a[7]));
+    }
+};
+template <> struct VecAcc<float> {
+    float a[4];
+    D2C_DEV void zero() { a[0] = a[1] = a[2] = a[3] = 0.f; }
+    D2C_DEV void fma(float w, const uint4 &v)
+    {
+        a[0] = fmaf(w, __uint_as_float(v.x), a[0]);
+        a[1] = fmaf(w, __uint_as_float(v.y), a[1]);
+        a[2] = fmaf(w, __uint_as_float(v.z), a[2]);
+        a[3] = fmaf(w, __uint_as_float(v.w), a[3]);
+    }
+    D2C_DEV uint4 pack() const
+    {
+        return make_uint4(__float_as_uint(a[0]), __float_as_uint(a[1]), __float_as_uint(a[2]), __float_as_uint(a[3]));
+    }
+};
+
+template <typename T> D2C_DEV float elem_to_f32(T v);
+template <> D2C_DEV float elem_to_f32<bf16_t>(bf16_t v) { return bf16_to_f32(v); }
+template <> D2C_DEV float elem_to_f32<float>(float v) { return v; }
+template <typename T> D2C_DEV T f32_to_elem(float v);
+template <> D2C_DEV bf16_t f32_to_elem<bf16_t>(float v) { return f32_to_bf16(v); }
+template <> D2C_DEV float f32_to_elem<float>(float v) { return v; }
+
+// offset / mask element (float32 or bfloat16 storage) as float
+D2C_DEV float ld_aux(const void *p, long i, int adt)
+{
+    return adt == D2C_F32 ? reinterpret_cast<const float *>(p)[i]
+                          : bf16_to_f32(reinterpret_cast<const bf16_t *>(p)[i]);
+}
+D2C_DEV void st_aux(void *p, long i, int adt, float v)
+{
+    if (adt == D2C_F32) reinterpret_cast<float *>(p)[i] = v;
+    else reinterpret_cast<bf16_t *>(p)[i] = f32_to_bf16(v);
+}
+
+// Geometry of the tiled kernels.  Channels are walked in chunks of BKC = 8*VEC
+// (64 bf16 / 32 float): one chunk never straddles an offset group or a weight
+// group, so all of its channels share the 8 corner positions of a tap.
+struct TiledShape {
+    int N, Cin, Cout, D, H, W, K, G, groups, Do, Ho, Wo;
+    int cg, og, cpg;      // channels per weight group (in / out), per offset group
+    int nchunk;           // chunks per weight group = cg / BKC
+    int ogp;              // og rounded up to the output tile width
+    int adt;
+    int P, vol;           // output positions / input voxels per sample
+    int M;                // N * P
+    TapGeom geo;
+};

@@ -1,19 +1,147 @@
-// Tiled kernel families: dispatch.  (Kernels are added family by family.)
+// Tiled kernel families: eligibility, workspace carving, operand packing and
+// dispatch.  Forward / backward kernels live in d2c_tiled_fwd.hip and
+// d2c_tiled_bwd.hip.
 #include "d2c_tiled.hpp"
+#include "d2c_mma.hpp"
 
-bool d2c_tiled_supported(const d2c_conv3d_desc &) { return false; }
-int d2c_tiled_algo(const d2c_conv3d_desc &) { return D2C_ALGO_GENERIC; }
-size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &) { return 0; }
-size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &) { return 0; }
-int d2c_tiled_forward(const d2c_conv3d_desc &, const void *, const void *, const void *, const void *,
-                      const void *, void *, void *, hipStream_t)
+int d2c_fwd_out_tile(int og);
+template <typename T>
+int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
+                         const void *bias, void *out, hipStream_t st);
+
+namespace {
+
+inline int vec_of(int dtype) { return dtype == D2C_BF16 ? 8 : 4; }
+inline int bkc_of(int dtype) { return 8 * vec_of(dtype); }
+
+TiledShape tiled_shape(const d2c_conv3d_desc &q)
 {
-    d2c_set_error("tiled kernels not available");
-    return D2C_ERR_UNSUPPORTED;
+    TiledShape s;
+    s.N = q.N; s.Cin = q.Cin; s.Cout = q.Cout; s.D = q.D; s.H = q.H; s.W = q.W;
+    s.K = q.kd * q.kh * q.kw; s.G = q.offset_groups; s.groups = q.groups;
+    s.Do = q.Do; s.Ho = q.Ho; s.Wo = q.Wo;
+    s.cg = q.Cin / q.groups; s.og = q.Cout / q.groups; s.cpg = q.Cin / q.offset_groups;
+    s.nchunk = s.cg / bkc_of(q.dtype);
+    const int nt = d2c_fwd_out_tile(s.og);
+    s.ogp = (s.og + nt - 1) / nt * nt;
+    s.adt = q.aux_dtype;
+    s.P = q.Do * q.Ho * q.Wo; s.vol = q.D * q.H * q.W; s.M = q.N * s.P;
+    s.geo = make_geom(q);
+    return s;
 }
-int d2c_tiled_backward(const d2c_conv3d_desc &, const void *, const void *, const void *, const void *,
-                       const void *, void *, void *, void *, void *, void *, void *, hipStream_t)
+
+// x [N][C][vol] -> xcl [N][vol][C]  (32 x 32 element tiles through LDS)
+template <typename T>
+__global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int C, int vol)
 {
-    d2c_set_error("tiled kernels not available");
-    return D2C_ERR_UNSUPPORTED;
+    __shared__ T tile[32][33];
+    const int b = blockIdx.z, v0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const T *xb = x + (long)b * C * vol;
+    T *ob = xcl + (long)b * C * vol;
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int c = c0 + ty + i, v = v0 + tx;
+        if (c < C && v < vol) tile[ty + i][tx] = xb[(long)c * vol + v];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int v = v0 + ty + i, c = c0 + tx;
+        if (c < C && v < vol) ob[(long)v * C + c] = tile[tx][ty + i];
+    }
+}
+
+// Forward weight operand in MFMA fragment order:
+//   wp[wg][step = chunk*K + k][o-block of 32][k-group][lane] = 16 bytes =
+//   W[wg*og + ob*32 + lane%32][chunk*BKC + (2*kg + lane/32)*VEC + 0..VEC-1][k]
+// (rows past og are zero), so a wavefront's fragment load is 1 KiB contiguous.
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_fwd_kernel(const T *w, T *wp, TiledShape s, long total)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
+    const int OBT = s.ogp / 32, S = s.nchunk * s.K;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int lane = (int)(i & 63);
+        const int kg = (int)((i >> 6) & 3);
+        long r = i >> 8;
+        const int obg = (int)(r % OBT); r /= OBT;
+        const int st = (int)(r % S);
+        const int wg = (int)(r / S);
+        const int j = st / s.K, k = st - j * s.K;
+        const int ol = obg * 32 + (lane & 31);
+        const int ch = j * BKC + (2 * kg + (lane >> 5)) * VEC;
+        T *dst = wp + i * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            dst[e] = ol < s.og ? w[((long)(wg * s.og + ol) * s.cg + ch + e) * s.K + k] : (T)0;
+    }
+}
+
+struct FwdWs {
+    size_t xcl, wp, total;
+};
+FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    const size_t es = d2c_elem_size(q.dtype);
+    FwdWs w;
+    w.xcl = 0;
+    w.wp = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
+    w.total = w.wp + d2c_align_up((size_t)s.groups * s.nchunk * s.K * s.ogp * bkc_of(q.dtype) * es);
+    return w;
+}
+
+template <typename T>
+int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st)
+{
+    dim3 grid((s.vol + 31) / 32, (s.Cin + 31) / 32, s.N);
+    hipLaunchKernelGGL(pack_input_kernel<T>, grid, dim3(256), 0, st, (const T *)x, (T *)xcl, s.Cin, s.vol);
+    return d2c_check_launch("pack_input_kernel");
+}
+
+template <typename T>
+int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
+              const void *bias, void *out, void *ws, hipStream_t st)
+{
+    const TiledShape s = tiled_shape(q);
+    const FwdWs l = fwd_ws(q, s);
+    char *base = (char *)ws;
+    if (int rc = pack_input<T>(s, x, base + l.xcl, st)) return rc;
+    const long total = (long)s.groups * s.nchunk * s.K * (s.ogp / 32) * 4 * 64;
+    long g = (total + 255) / 256;
+    if (g > 8192) g = 8192;
+    hipLaunchKernelGGL(pack_weight_fwd_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, (const T *)w,
+                       (T *)(base + l.wp), s, total);
+    if (int rc = d2c_check_launch("pack_weight_fwd_kernel")) return rc;
+    return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, st);
+}
+
+}  // namespace
+
+bool d2c_tiled_supported(const d2c_conv3d_desc &q)
+{
+    if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
+    const int bkc = bkc_of(q.dtype);
+    const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
+    return cg % bkc == 0 && cpg % bkc == 0;
+}
+
+int d2c_tiled_algo(const d2c_conv3d_desc &) { return D2C_ALGO_MFMA; }
+
+size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q) { return fwd_ws(q, tiled_shape(q)).total; }
+
+size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q) { return d2c_generic_conv3d_backward_ws(q); }
+
+int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
+                      const void *bias, void *out, void *ws, hipStream_t st)
+{
+    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st);
+    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st);
+}
+
+int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
+                       const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
+                       void *ws, hipStream_t st)
+{
+    return d2c_generic_conv3d_backward(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st);
 }

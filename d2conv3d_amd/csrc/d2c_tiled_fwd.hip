@@ -1,0 +1,249 @@
+// Forward pass as an implicit GEMM on the matrix cores.
+//
+//   out[b, o, p] = bias[o] + sum_{c, k} W[o, c, k] * alpha[b,g,k,p] * trilinear(x[b, c], pos(b,g,k,p))
+//
+// GEMM view: rows = output channels, columns = output positions (N*P of
+// them), reduction = (channel chunk, tap).  The sampled operand is produced on
+// the fly: for one (chunk, tap) step every thread gathers the 8 corners of its
+// position as 16-byte channel vectors from the channels-last copy of the
+// input, interpolates in fp32 with the modulation folded into the corner
+// weights, and drops the result into an LDS tile in MFMA operand order.  The
+// im2col column buffer of the reference (dconv3d_gpu.cu:297) never exists.
+//
+// One workgroup = 512 threads = 128 positions x NT output channels.  Steps are
+// software-pipelined: while the matrix cores work on step s, the corner loads
+// of step s+1 are in flight and the corner weights of step s+2 are computed.
+#include "d2c_mma.hpp"
+#include "d2c_tiled.hpp"
+
+namespace {
+
+constexpr int kMT = 128;       // positions per workgroup
+constexpr int kNV = 8;         // 16-byte vectors per sampled row (one chunk)
+constexpr int kRS = kNV * 16 + 16;  // LDS row stride in bytes (padded: conflict-free 16-byte reads)
+constexpr int kThreads = 512;
+
+struct FwdArgs {
+    TiledShape s;
+    const void *xcl;   // [N][vol][Cin]
+    const void *off, *mask;
+    const void *wp;    // packed weights, see pack_weight_fwd
+    const void *bias;
+    void *out;
+};
+
+// Tiles that are neighbours in space go to the same XCD (workgroups are dealt
+// round-robin over the 8 XCDs), so that its L2 sees a compact part of the input.
+D2C_DEV int xcd_swizzle(int bid, int n)
+{
+    const int x = bid & 7, idx = bid >> 3;
+    const int q = n >> 3, r = n & 7;
+    return x * q + (x < r ? x : r) + idx;
+}
+
+template <typename T, int WAVES_O, int WAVES_P>
+__global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int BKC = kNV * VEC;
+    constexpr int WPOS = kMT / WAVES_P;   // positions per MMA wave
+    constexpr int PB = WPOS / 32;         // 32-position blocks per MMA wave
+    constexpr int OB = 2;                 // 32-channel blocks per MMA wave
+    constexpr int NT = 64 * WAVES_O;      // output channels per workgroup
+    constexpr int ITEMS = kMT * kNV / kThreads;  // (position, vector) items per thread
+    static_assert(ITEMS == 2, "two gather items per thread");
+    static_assert(WAVES_O * WAVES_P <= kThreads / 64, "too many MMA waves");
+
+    __shared__ __align__(16) unsigned char s_tile[2][kMT * kRS];
+    __shared__ float s_w[2][8][kMT];
+    __shared__ int s_idx[2][kMT];
+    __shared__ int s_flag[2][kMT];
+
+    const TiledShape &s = a.s;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
+    const int otile = blockIdx.y, wg = blockIdx.z;
+    const int m0 = tile * kMT;
+    const int S = s.nchunk * s.K;
+    const int HW = s.H * s.W;
+
+    // --- per-position constants of the coordinate threads
+    int cb = 0, cp = 0, coz = 0, coy = 0, cox = 0;
+    bool cvalid = false;
+    if (tid < kMT) {
+        const int m = m0 + tid;
+        cvalid = m < s.M;
+        if (cvalid) {
+            cb = m / s.P; cp = m - cb * s.P;
+            cox = cp % s.Wo; coy = (cp / s.Wo) % s.Ho; coz = cp / (s.Wo * s.Ho);
+        }
+    }
+
+    // corner weights (modulation folded in, dead corners zero), base voxel, live mask of step st
+    auto coords = [&](int st, int buf) {
+        if (tid < kMT) {
+            float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            int idx = 0;
+            unsigned live = 0;
+            if (cvalid) {
+                const int j = st / s.K, k = st - j * s.K;
+                const int g = (wg * s.cg + j * BKC) / s.cpg;
+                const long ob = (((long)cb * s.G + g) * s.K + k) * 3 * s.P + cp;
+                const float o0 = ld_aux(a.off, ob, s.adt);
+                const float o1 = ld_aux(a.off, ob + s.P, s.adt);
+                const float o2 = ld_aux(a.off, ob + 2 * (long)s.P, s.adt);
+                const float al = a.mask ? ld_aux(a.mask, (((long)cb * s.G + g) * s.K + k) * s.P + cp, s.adt) : 1.f;
+                int bz, by, bx;
+                tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
+                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+                live = t.live;
+                idx = cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0;
+#pragma unroll
+                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
+            }
+#pragma unroll
+            for (int c = 0; c < 8; c++) s_w[buf][c][tid] = w[c];
+            s_idx[buf][tid] = idx;
+            s_flag[buf][tid] = (int)live;
+        }
+    };
+
+    // --- gather: item i of this thread = (position ipos[i], vector ivec[i])
+    uint4 gv[ITEMS][8];
+    auto gather_issue = [&](int st, int buf) {
+        const int j = st / s.K;
+        const int c0 = wg * s.cg + j * BKC;
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) {
+            const int item = tid + i * kThreads;
+            const int pos = item / kNV, vec = item % kNV;
+            const int idx = s_idx[buf][pos];
+            const unsigned live = (unsigned)s_flag[buf][pos];
+            const T *base = reinterpret_cast<const T *>(a.xcl) + c0 + vec * VEC;
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
+                gv[i][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint4 *>(base + (long)v * s.Cin)
+                                              : make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    auto interp_store = [&](int cbuf, int tbuf) {
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) {
+            const int item = tid + i * kThreads;
+            const int pos = item / kNV, vec = item % kNV;
+            VecAcc<T> acc;
+            acc.zero();
+#pragma unroll
+            for (int c = 0; c < 8; c++) acc.fma(s_w[cbuf][c][pos], gv[i][c]);
+            *reinterpret_cast<uint4 *>(&s_tile[tbuf][pos * kRS + vec * 16]) = acc.pack();
+        }
+    };
+
+    // --- MMA role
+    const bool mma_wave = wave < WAVES_O * WAVES_P;
+    const int wave_o = wave % WAVES_O, wave_p = wave / WAVES_O;
+    const int OBT = s.ogp / 32;  // 32-channel blocks per weight group in the packed weights
+    f32x16 acc[OB][PB];
+#pragma unroll
+    for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[ob][pb][r] = 0.f;
+
+    const uint4 *wp4 = reinterpret_cast<const uint4 *>(a.wp);
+    auto mma_step = [&](int st, int tbuf) {
+        if (!mma_wave) return;
+        const long wbase = (((long)wg * S + st) * OBT + (otile * (NT / 32) + wave_o * OB)) * (kNV / 2) * 64 + lane;
+        const unsigned char *tb = &s_tile[tbuf][(wave_p * WPOS + (lane & 31)) * kRS + (lane >> 5) * 16];
+#pragma unroll
+        for (int kg = 0; kg < kNV / 2; kg++) {
+            uint4 af[OB], bf[PB];
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++) af[ob] = wp4[wbase + ((long)ob * (kNV / 2) + kg) * 64];
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++)
+                bf[pb] = *reinterpret_cast<const uint4 *>(tb + pb * 32 * kRS + kg * 32);
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[ob], bf[pb]);
+        }
+    };
+
+    // --- pipeline
+    coords(0, 0);
+    __syncthreads();
+    gather_issue(0, 0);
+    if (S > 1) coords(1, 1);
+    interp_store(0, 0);
+    __syncthreads();
+    for (int st = 0; st < S; st++) {
+        if (st + 1 < S) gather_issue(st + 1, (st + 1) & 1);
+        if (st + 2 < S) coords(st + 2, st & 1);
+        mma_step(st, st & 1);
+        if (st + 1 < S) interp_store((st + 1) & 1, (st + 1) & 1);
+        __syncthreads();
+    }
+
+    // --- epilogue: bias, convert, store (32 consecutive positions per row of a block)
+    if (mma_wave) {
+        T *out = reinterpret_cast<T *>(a.out);
+        const T *bias = reinterpret_cast<const T *>(a.bias);
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) {
+            const int m = m0 + wave_p * WPOS + pb * 32 + (lane & 31);
+            if (m >= s.M) continue;
+            const int b = m / s.P, p = m - b * s.P;
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int ol = otile * NT + wave_o * 64 + ob * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (ol < s.og) {
+                        const int o = wg * s.og + ol;
+                        float v = acc[ob][pb][r];
+                        if (bias) v += elem_to_f32<T>(bias[o]);
+                        out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(v);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int WO, int WP>
+int launch_fwd(const FwdArgs &a, hipStream_t st)
+{
+    const int ntile = (a.s.M + kMT - 1) / kMT;
+    const int NT = 64 * WO;
+    dim3 grid(ntile, a.s.ogp / NT, a.s.groups);
+    hipLaunchKernelGGL((tiled_fwd_kernel<T, WO, WP>), grid, dim3(kThreads), 0, st, a);
+    return d2c_check_launch("tiled_fwd_kernel");
+}
+
+}  // namespace
+
+int d2c_fwd_out_tile(int og)
+{
+    return og > 256 ? 512 : (og > 128 ? 256 : (og > 64 ? 128 : 64));
+}
+
+template <typename T>
+int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
+                         const void *bias, void *out, hipStream_t st)
+{
+    FwdArgs a{s, xcl, off, mask, wp, bias, out};
+    switch (d2c_fwd_out_tile(s.og)) {
+    case 512: return launch_fwd<T, 8, 1>(a, st);
+    case 256: return launch_fwd<T, 4, 2>(a, st);
+    case 128: return launch_fwd<T, 2, 4>(a, st);
+    default: return launch_fwd<T, 1, 4>(a, st);
+    }
+}
+template int d2c_tiled_fwd_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
+                                          const void *, void *, hipStream_t);
+template int d2c_tiled_fwd_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
+                                         const void *, void *, hipStream_t);

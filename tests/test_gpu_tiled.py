@@ -1,0 +1,105 @@
+"""GPU parity of the tiled kernel families (matrix-core implicit GEMM,
+depthwise) against the CPU oracle, at sizes the oracle finishes in seconds.
+
+float32: 1e-4 relative / 1e-5 absolute (scaled by the tensor's magnitude for
+the gradients, which are long sums).  bfloat16: the oracle consumes the
+bfloat16-rounded tensors up-cast to float32; results must agree within 2e-2
+relative (L2 over the tensor, and element-wise against the tensor's scale).
+"""
+import pytest
+import torch
+
+import d2conv3d_amd as d2c
+from d2conv3d_amd import _ops
+from oracle import cpu
+from _util import assert_close, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+# name: (N, Cin, Cout, (D,H,W), k, stride, pad, dil, groups, G, bias, mask, offset_sigma)
+SHAPES = {
+    "c64_g1": (2, 64, 64, (4, 6, 7), 3, 1, 1, 1, 1, 1, True, True, 1.0),
+    "c128_G2_o96": (1, 128, 96, (3, 6, 9), 3, 1, 1, 1, 1, 2, True, True, 2.0),
+    "c128_groups2": (2, 128, 192, (3, 5, 6), 3, 1, 1, 1, 2, 2, False, True, 1.5),
+    "c64_o320_nomask": (1, 64, 320, (3, 5, 5), 3, 1, 1, 1, 1, 1, True, False, 1.0),
+    "c64_o600": (1, 64, 600, (2, 5, 5), (1, 3, 3), 1, (0, 1, 1), 1, 1, 1, True, True, 1.0),
+    "c64_stride_dil": (2, 64, 64, (5, 9, 8), 3, (1, 2, 1), (1, 2, 2), (1, 2, 1), 1, 1, True, True, 1.0),
+    "c64_tail": (3, 64, 32, (3, 7, 7), 3, 1, 1, 1, 1, 1, True, True, 1.0),   # N*P = 441: ragged last tile
+}
+
+
+def make(name, dtype, seed=0):
+    N, Cin, Cout, dims, k, s, p, d, groups, G, bias, mask, sig = SHAPES[name]
+    t3 = lambda v: (v,) * 3 if isinstance(v, int) else tuple(v)
+    k, s, p, d = t3(k), t3(s), t3(p), t3(d)
+    od = tuple((n + 2 * pp - (dd * (kk - 1) + 1)) // ss + 1 for n, kk, ss, pp, dd in zip(dims, k, s, p, d))
+    K = k[0] * k[1] * k[2]
+    g = torch.Generator().manual_seed(1000 + seed)
+    rn = lambda *sh: torch.randn(*sh, generator=g)
+    x = rn(N, Cin, *dims)
+    fan_in = Cin // groups * K
+    w = (torch.rand(Cout, Cin // groups, *k, generator=g) * 2 - 1) / fan_in ** 0.5
+    b = (torch.rand(Cout, generator=g) * 2 - 1) / fan_in ** 0.5 if bias else None
+    off = rn(N, G * 3 * K, *od) * sig
+    m = torch.sigmoid(rn(N, G * K, *od)) if mask else None
+    gout = rn(N, Cout, *od)
+    if dtype == torch.bfloat16:
+        x, w, gout = x.bfloat16(), w.bfloat16(), gout.bfloat16()
+        b = b.bfloat16() if b is not None else None
+    return (x, off, m, w, b), gout, (s, p, d, groups, G)
+
+
+def f32(t):
+    return t.float() if t is not None else None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("name", list(SHAPES))
+def test_tiled_forward_backward(name, dtype, dev):
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, dtype)
+    ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+    assert _ops.conv3d_algo(ts[0], ts[1], ts[2], ts[3], s, p, d, groups, G) == "mfma"
+    out = d2c.deform_conv3d(*ts, s, p, d, groups, G)
+    exp = cpu.conv3d_forward(f32(x), off, m, f32(w), f32(b), s, p, d, groups, G)
+    eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+    out.backward(gout.to(dev))
+    names = ("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias")
+    if dtype == torch.float32:
+        assert_close(out, exp, 1e-4, 1e-5, "forward")
+        for n, t, e in zip(names, ts, eg):
+            if t is not None:
+                assert_close(t.grad, e, 1e-4, 1e-5 * max(1.0, e.abs().max().item()), n)
+    else:
+        assert out.dtype == torch.bfloat16
+        assert rel_l2(out, exp) < 2e-2, rel_l2(out, exp)
+        assert_close(out, exp, 2e-2, 2e-2 * exp.abs().max().item(), "forward")
+        for n, t, e in zip(names, ts, eg):
+            if t is not None:
+                assert t.grad.dtype == t.dtype
+                assert rel_l2(t.grad, e) < 2e-2, (n, rel_l2(t.grad, e))
+                assert_close(t.grad, e, 2e-2, 2e-2 * e.abs().max().item(), n)
+
+
+def test_tiled_matches_generic_family(dev):
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make("c128_G2_o96", torch.float32, seed=3)
+    ts = [t.to(dev) if t is not None else None for t in (x, off, m, w, b)]
+    out = d2c.deform_conv3d(*ts, s, p, d, groups, G)
+    _ops.set_algo_override("generic")
+    try:
+        ref = d2c.deform_conv3d(*ts, s, p, d, groups, G)
+    finally:
+        _ops.set_algo_override(None)
+    assert_close(out, ref, 1e-4, 1e-5, "tiled vs generic")
+
+
+def test_bfloat16_offsets_and_masks_in_bfloat16(dev):
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make("c64_g1", torch.bfloat16, seed=4)
+    off, m = off.bfloat16(), m.bfloat16()
+    ts = [t.to(dev).requires_grad_(True) for t in (x, off, m, w, b)]
+    out = d2c.deform_conv3d(*ts, s, p, d, groups, G)
+    exp = cpu.conv3d_forward(f32(x), f32(off), f32(m), f32(w), f32(b), s, p, d, groups, G)
+    assert rel_l2(out, exp) < 2e-2
+    out.backward(gout.to(dev))
+    eg = cpu.conv3d_backward(f32(gout), f32(x), f32(off), f32(m), f32(w), True, s, p, d, groups, G)
+    for t, e in zip(ts, eg):
+        assert t.grad.dtype == torch.bfloat16 and rel_l2(t.grad, e) < 2e-2
