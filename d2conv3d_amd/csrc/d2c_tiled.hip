@@ -9,6 +9,19 @@ template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
                          const void *bias, void *out, hipStream_t st);
 
+bool d2c_tiled_bwd_data_supported(const TiledShape &s, int dtype);
+bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype);
+int d2c_bwd_ogk(int og, int dtype);
+template <typename T>
+int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
+                              const void *mask, const void *w, void *wt, float *gxcl, void *goff, void *gmask,
+                              hipStream_t st);
+template <typename T>
+int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
+                                const void *mask, float *gwacc, void *gw, hipStream_t st);
+template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
+template <typename T> int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st);
+
 namespace {
 
 inline int vec_of(int dtype) { return dtype == D2C_BF16 ? 8 : 4; }
@@ -116,6 +129,60 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
     return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, st);
 }
 
+struct BwdWs {
+    size_t xcl, wt, gxcl, gwacc, total;
+};
+BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    const size_t es = d2c_elem_size(q.dtype);
+    BwdWs w;
+    w.xcl = 0;
+    w.wt = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
+    w.gxcl = w.wt + d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * d2c_bwd_ogk(s.og, q.dtype) * es);
+    w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
+    w.total = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
+    return w;
+}
+
+template <typename T>
+int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off, const void *mask,
+               const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws, hipStream_t st)
+{
+    const TiledShape s = tiled_shape(q);
+    const BwdWs l = bwd_ws(q, s);
+    char *base = (char *)ws;
+    if (!mask) gmask = nullptr;
+    if (int rc = pack_input<T>(s, x, base + l.xcl, st)) return rc;
+    if (gx || goff || gmask) {
+        if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
+            float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
+            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt, gxcl, goff,
+                                                     gmask, st))
+                return rc;
+            if (gx)
+                if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
+        } else {
+            // shapes the fused kernel does not hold on chip: direct kernels (f32 staging in the same region)
+            if (int rc = d2c_generic_conv3d_backward(q, gout, x, off, mask, w, gx, goff, gmask, nullptr, nullptr,
+                                                     base + l.gxcl, st))
+                return rc;
+        }
+    }
+    if (gw) {
+        if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
+            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, (float *)(base + l.gwacc),
+                                                       gw, st))
+                return rc;
+        } else {
+            if (int rc = d2c_generic_conv3d_backward(q, gout, x, off, mask, w, nullptr, nullptr, nullptr, gw, nullptr,
+                                                     nullptr, st))
+                return rc;
+        }
+    }
+    if (gb) return d2c_tiled_bias_grad<T>(s, gout, gb, st);
+    return D2C_OK;
+}
+
 }  // namespace
 
 bool d2c_tiled_supported(const d2c_conv3d_desc &q)
@@ -130,7 +197,7 @@ int d2c_tiled_algo(const d2c_conv3d_desc &) { return D2C_ALGO_MFMA; }
 
 size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q) { return fwd_ws(q, tiled_shape(q)).total; }
 
-size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q) { return d2c_generic_conv3d_backward_ws(q); }
+size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q) { return bwd_ws(q, tiled_shape(q)).total; }
 
 int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
                       const void *bias, void *out, void *ws, hipStream_t st)
@@ -143,5 +210,6 @@ int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x
                        const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
                        void *ws, hipStream_t st)
 {
-    return d2c_generic_conv3d_backward(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st);
+    if (q.dtype == D2C_BF16) return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st);
+    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st);
 }

@@ -1,0 +1,621 @@
+// Backward pass on the matrix cores, without a column buffer.
+//
+// Kernel 1 (tiled_bwd_data_kernel), per workgroup a tile of output positions,
+// per step one (tap, channel chunk):
+//     gcol[pos, c]  = sum_o gout[pos, o] * W[o, c, k]                (MFMA; dconv3d_gpu.cu:976-1000)
+//     gx[corner, c] += a_corner * alpha * gcol[pos, c]               (atomics; :593-642)
+//     dot[corner]    = sum_c gcol[pos, c] * x[corner, c]
+//     gmask          = sum_corner a_corner * dot[corner]             (:837-839)
+//     goff_axis      = alpha * sum_corner (d a_corner / d axis) * dot[corner]   (:708-754, :848-858)
+//   The gout operand of a wavefront (its 32 positions x all output channels of
+//   the weight group) stays in registers for the whole kernel; the weight
+//   operand of the step is staged in LDS; gcol never leaves the chip.
+//
+// Kernel 2 (tiled_bwd_weight_kernel), per workgroup one (tap, channel chunk)
+// and all output channels, looping over position tiles:
+//     gW[o, c, k] += sum_pos gout[o, pos] * alpha * trilinear(x[c], pos)       (:1037-1088)
+//   The sampler writes its tile position-contiguous so that it is an MFMA
+//   operand as it lies.
+#include "d2c_mma.hpp"
+#include "d2c_tiled.hpp"
+
+namespace {
+
+constexpr int kThreads = 512;
+
+D2C_DEV int xcd_swizzle(int bid, int n)
+{
+    const int x = bid & 7, idx = bid >> 3;
+    const int q = n >> 3, r = n & 7;
+    return x * q + (x < r ? x : r) + idx;
+}
+
+// ============================================================ kernel 1
+struct BwdDataArgs {
+    TiledShape s;
+    const void *gout;   // [N][Cout][P]
+    const void *xcl;    // [N][vol][Cin]
+    const void *off, *mask;
+    const void *wt;     // [groups][K*nchunk][BKC][ogk]   (W transposed per step, zero padded to ogk)
+    float *gxcl;        // [N][vol][Cin] fp32 accumulator (zeroed) or NULL
+    void *goff, *gmask; // or NULL
+    int ogk;            // og rounded up to a whole k-group
+};
+
+// NKG = k-groups of the reduction over output channels held in registers.
+template <typename T, int NKG>
+__global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int NV = 8, BKC = NV * VEC;
+    constexpr int CB = BKC / 32;           // 32-channel blocks per step (2 for bf16, 1 for float)
+    constexpr int PBW = 8 / CB;            // 32-position blocks per workgroup
+    constexpr int MT = 32 * PBW;           // positions per workgroup (128 / 256)
+    constexpr int GRS = BKC * 4 + 16;      // gcol tile row stride (bytes)
+    constexpr int ITEMS = MT * NV / kThreads;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    const TiledShape &s = a.s;
+    const int wrs = a.ogk * (int)sizeof(T) + 16;        // weight tile row stride (bytes)
+    unsigned char *s_wt = smem;                          // [BKC][wrs]
+    unsigned char *s_gcol = s_wt + BKC * wrs;            // [MT][GRS]
+    float *s_w = reinterpret_cast<float *>(s_gcol + MT * GRS);   // [8][MT]  live corner weights * alpha
+    float *s_frac = s_w + 8 * MT;                        // [6][MT]  lz ly lx hz hy hx
+    float *s_alpha = s_frac + 6 * MT;                    // [MT]
+    int *s_idx = reinterpret_cast<int *>(s_alpha + MT);  // [MT]
+    int *s_flag = s_idx + MT;                            // [MT]     live | inrange << 8
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
+    const int wg = blockIdx.y;
+    const int m0 = tile * MT;
+    const int S = s.nchunk * s.K;
+    const int HW = s.H * s.W;
+    const int cb = wave % CB, pb = wave / CB;
+    const int nkg = a.ogk / (2 * VEC);
+
+    // ---- stationary operand: gout[pos, o] of this wavefront's 32 positions
+    uint4 ga[NKG];
+    {
+        const int m = m0 + pb * 32 + (lane & 31);
+        const bool ok = m < s.M;
+        const int b = ok ? m / s.P : 0, p = ok ? m - b * s.P : 0;
+        const T *gp = reinterpret_cast<const T *>(a.gout) + ((long)b * s.Cout + wg * s.og) * s.P + p;
+#pragma unroll
+        for (int kg = 0; kg < NKG; kg++) {
+            T e[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const int o = (kg * 2 + (lane >> 5)) * VEC + i;
+                e[i] = (ok && kg < nkg && o < s.og) ? gp[(long)o * s.P] : (T)0;
+            }
+            ga[kg] = *reinterpret_cast<uint4 *>(e);
+        }
+    }
+
+    // ---- per-position constants of the coordinate threads
+    int cbatch = 0, cp = 0, coz = 0, coy = 0, cox = 0;
+    bool cvalid = false;
+    if (tid < MT) {
+        const int m = m0 + tid;
+        cvalid = m < s.M;
+        if (cvalid) {
+            cbatch = m / s.P; cp = m - cbatch * s.P;
+            cox = cp % s.Wo; coy = (cp / s.Wo) % s.Ho; coz = cp / (s.Wo * s.Ho);
+        }
+    }
+
+    // offset / mask gradient accumulators of the positions this thread finalises
+    float g_acc[ITEMS][4];
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) g_acc[i][0] = g_acc[i][1] = g_acc[i][2] = g_acc[i][3] = 0.f;
+
+    const bool want_aux = a.goff != nullptr || a.gmask != nullptr;
+
+    for (int st = 0; st < S; st++) {
+        const int k = st / s.nchunk, j = st - k * s.nchunk;
+        const int c0 = wg * s.cg + j * BKC;
+        const int g = c0 / s.cpg;
+        // last chunk of this offset group inside this weight group -> flush goff / gmask
+        const bool group_end = (j + 1 == s.nchunk) || ((c0 + BKC) / s.cpg != g);
+
+        // (a) coordinates of the step and the weight tile
+        if (tid < MT) {
+            float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            float fr[6] = {0, 0, 0, 0, 0, 0};
+            float al = 0.f;
+            int idx = 0, flag = 0;
+            if (cvalid) {
+                const long ob = (((long)cbatch * s.G + g) * s.K + k) * 3 * s.P + cp;
+                const float o0 = ld_aux(a.off, ob, s.adt);
+                const float o1 = ld_aux(a.off, ob + s.P, s.adt);
+                const float o2 = ld_aux(a.off, ob + 2 * (long)s.P, s.adt);
+                al = a.mask ? ld_aux(a.mask, (((long)cbatch * s.G + g) * s.K + k) * s.P + cp, s.adt) : 1.f;
+                int bz, by, bx;
+                tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
+                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+                idx = cbatch * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0;
+                flag = (int)(t.live | (t.inrange << 8));
+#pragma unroll
+                for (int c = 0; c < 8; c++) w[c] = ((t.live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
+                fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
+            }
+#pragma unroll
+            for (int c = 0; c < 8; c++) s_w[c * MT + tid] = w[c];
+#pragma unroll
+            for (int c = 0; c < 6; c++) s_frac[c * MT + tid] = fr[c];
+            s_alpha[tid] = al;
+            s_idx[tid] = idx;
+            s_flag[tid] = flag;
+        }
+        {
+            const int row16 = a.ogk * (int)sizeof(T) / 16;   // 16-byte pieces per weight row
+            const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * row16;
+            for (int q = tid; q < BKC * row16; q += kThreads) {
+                const int row = q / row16, col = q - row * row16;
+                *reinterpret_cast<uint4 *>(s_wt + row * wrs + col * 16) = src[q];
+            }
+        }
+        __syncthreads();
+
+        // (b) gcol block of this wavefront: rows = positions, columns = channels
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.f;
+        {
+            const unsigned char *wb = s_wt + (cb * 32 + (lane & 31)) * wrs + (lane >> 5) * 16;
+#pragma unroll
+            for (int kg = 0; kg < NKG; kg++) {
+                if (kg < nkg) {
+                    const uint4 bf = *reinterpret_cast<const uint4 *>(wb + kg * 32);
+                    mma_kgroup<T>(acc, ga[kg], bf);
+                }
+            }
+        }
+
+        // (c) gcol -> LDS (for the dot products), and scatter into grad_input straight from
+        //     the accumulators: lanes 0..31 / 32..63 each cover 32 consecutive channels.
+        const int ch = cb * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int pl = pb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            *reinterpret_cast<float *>(s_gcol + pl * GRS + ch * 4) = acc[r];
+        }
+        if (a.gxcl) {
+            float *gbase = a.gxcl + c0 + ch;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int pl = pb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const unsigned live = (unsigned)s_flag[pl] & 0xffu;
+                if (live) {
+                    const int idx = s_idx[pl];
+                    const float gv = acc[r];
+#pragma unroll
+                    for (int c = 0; c < 8; c++) {
+                        if ((live >> c) & 1u) {
+                            const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
+                            atomicAdd(gbase + (long)v * s.Cin, s_w[c * MT + pl] * gv);
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+
+        // (d) dot products with the corner vectors, offset / mask gradient
+        if (want_aux) {
+#pragma unroll
+            for (int i = 0; i < ITEMS; i++) {
+                const int item = tid + i * kThreads;
+                const int pos = item / NV, vec = item % NV;
+                const int idx = s_idx[pos];
+                const unsigned flag = (unsigned)s_flag[pos];
+                const unsigned inr = flag >> 8, live = flag & 0xffu;
+                float gc[VEC];
+                {
+                    const float4 *gp4 = reinterpret_cast<const float4 *>(s_gcol + pos * GRS + vec * VEC * 4);
+#pragma unroll
+                    for (int e = 0; e < VEC / 4; e++) {
+                        const float4 t4 = gp4[e];
+                        gc[4 * e] = t4.x; gc[4 * e + 1] = t4.y; gc[4 * e + 2] = t4.z; gc[4 * e + 3] = t4.w;
+                    }
+                }
+                const T *xb = reinterpret_cast<const T *>(a.xcl) + c0 + vec * VEC;
+                float dot[8];
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    float d = 0.f;
+                    if ((inr >> c) & 1u) {
+                        const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
+                        const uint4 xv = *reinterpret_cast<const uint4 *>(xb + (long)v * s.Cin);
+                        const T *xe = reinterpret_cast<const T *>(&xv);
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) d = fmaf(gc[e], elem_to_f32<T>(xe[e]), d);
+                    }
+                    dot[c] = d;
+                }
+                // sum over the 8 lanes that share the position
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    dot[c] += __shfl_xor(dot[c], 1, 64);
+                    dot[c] += __shfl_xor(dot[c], 2, 64);
+                    dot[c] += __shfl_xor(dot[c], 4, 64);
+                }
+                if (vec == 0) {
+                    const float lz = s_frac[0 * MT + pos], ly = s_frac[1 * MT + pos], lx = s_frac[2 * MT + pos];
+                    const float hz = s_frac[3 * MT + pos], hy = s_frac[4 * MT + pos], hx = s_frac[5 * MT + pos];
+                    float gz = 0.f, gy = 0.f, gxx = 0.f, gm = 0.f;
+#pragma unroll
+                    for (int c = 0; c < 8; c++) {
+                        const float wz = (c & 4) ? hz : lz, wy = (c & 2) ? hy : ly, wx = (c & 1) ? hx : lx;
+                        const float d = dot[c];
+                        gz += ((c & 4) ? d : -d) * (wy * wx);
+                        gy += ((c & 2) ? d : -d) * (wz * wx);
+                        gxx += ((c & 1) ? d : -d) * (wz * wy);
+                        if ((live >> c) & 1u) gm += (wz * wy * wx) * d;
+                    }
+                    const float al = s_alpha[pos];
+                    g_acc[i][0] += al * gz; g_acc[i][1] += al * gy; g_acc[i][2] += al * gxx; g_acc[i][3] += gm;
+                    if (group_end) {
+                        const int m = m0 + pos;
+                        if (m < s.M) {
+                            const int b = m / s.P, p = m - b * s.P;
+                            if (a.goff) {
+                                const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
+                                st_aux(a.goff, ob, s.adt, g_acc[i][0]);
+                                st_aux(a.goff, ob + s.P, s.adt, g_acc[i][1]);
+                                st_aux(a.goff, ob + 2 * (long)s.P, s.adt, g_acc[i][2]);
+                            }
+                            if (a.gmask) st_aux(a.gmask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt, g_acc[i][3]);
+                        }
+                        g_acc[i][0] = g_acc[i][1] = g_acc[i][2] = g_acc[i][3] = 0.f;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T> size_t bwd_data_lds(int ogk)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
+    return (size_t)BKC * (ogk * sizeof(T) + 16) + (size_t)MT * (BKC * 4 + 16) + (size_t)MT * (8 + 6 + 1 + 1 + 1) * 4;
+}
+
+template <typename T, int NKG>
+int launch_bwd_data(const BwdDataArgs &a, hipStream_t st)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
+    const size_t lds = bwd_data_lds<T>(a.ogk);
+    if (hipFuncSetAttribute((const void *)tiled_bwd_data_kernel<T, NKG>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024) != hipSuccess)
+        return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_data_kernel)");
+    dim3 grid((a.s.M + MT - 1) / MT, a.s.groups);
+    hipLaunchKernelGGL((tiled_bwd_data_kernel<T, NKG>), grid, dim3(kThreads), lds, st, a);
+    return d2c_check_launch("tiled_bwd_data_kernel");
+}
+
+// ============================================================ kernel 2
+struct BwdWeightArgs {
+    TiledShape s;
+    const void *gout, *xcl, *off, *mask;
+    float *gwacc;   // [Cout][cg][K] fp32 accumulator (zeroed)
+    int split;      // position tiles are dealt round-robin to `split` workgroups per step
+};
+
+constexpr int kWMT = 128;  // positions per iteration
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArgs a)
+{
+    constexpr int VEC = Elem<T>::VEC;          // positions per 16-byte operand vector
+    constexpr int BKC = 8 * VEC;               // channels per step (64 / 32)
+    constexpr int CB = BKC / 32;
+    constexpr int OB = 2;                      // 32-row blocks of output channels per wavefront
+    constexpr int NT = 64 * 8;                 // output channels per workgroup
+    constexpr int CPI = sizeof(T) == 2 ? 2 : 1;  // channels per gather item (one 4-byte load)
+    constexpr int TRS = kWMT * (int)sizeof(T) + 16;   // tile row stride: [channel][position]
+    constexpr int NOCT = kWMT / VEC;           // position groups per tile
+    constexpr int NITEM = NOCT * (BKC / CPI);  // gather items per tile
+    constexpr int ITEMS = NITEM / kThreads;
+    static_assert(ITEMS * kThreads == NITEM, "gather items divide evenly");
+
+    __shared__ __align__(16) unsigned char s_tile[BKC * TRS];
+    __shared__ float s_w[8][kWMT];
+    __shared__ int s_idx[kWMT];
+    __shared__ int s_flag[kWMT];
+
+    const TiledShape &s = a.s;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int st = blockIdx.x;                 // step = chunk * K + tap
+    const int otile = blockIdx.y;
+    const int wg = blockIdx.z / a.split, sp = blockIdx.z % a.split;
+    const int j = st / s.K, k = st - j * s.K;
+    const int c0 = wg * s.cg + j * BKC;
+    const int g = c0 / s.cpg;
+    const int HW = s.H * s.W;
+    const int ntile = (s.M + kWMT - 1) / kWMT;
+    const int o_base = otile * NT + wave * 64;   // first output channel (in the weight group) of this wavefront
+    const bool mma_wave = o_base < s.og;
+
+    f32x16 acc[OB][CB];
+#pragma unroll
+    for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[ob][cb][r] = 0.f;
+
+    for (int tile = sp; tile < ntile; tile += a.split) {
+        const int m0 = tile * kWMT;
+        // corner weights of the tile's positions for this tap
+        if (tid < kWMT) {
+            float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            int idx = 0;
+            unsigned live = 0;
+            const int m = m0 + tid;
+            if (m < s.M) {
+                const int b = m / s.P, p = m - b * s.P;
+                const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
+                const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
+                const float o0 = ld_aux(a.off, ob, s.adt);
+                const float o1 = ld_aux(a.off, ob + s.P, s.adt);
+                const float o2 = ld_aux(a.off, ob + 2 * (long)s.P, s.adt);
+                const float al = a.mask ? ld_aux(a.mask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt) : 1.f;
+                int bz, by, bx;
+                tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
+                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+                live = t.live;
+                idx = b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0;
+#pragma unroll
+                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
+            }
+#pragma unroll
+            for (int c = 0; c < 8; c++) s_w[c][tid] = w[c];
+            s_idx[tid] = idx;
+            s_flag[tid] = (int)live;
+        }
+        __syncthreads();
+
+        // sample: one item = CPI channels x VEC consecutive positions; 32 lanes read one 128-byte row
+#pragma unroll
+        for (int it = 0; it < ITEMS; it++) {
+            const int item = tid + it * kThreads;
+            const int cpi = item % (BKC / CPI), oct = item / (BKC / CPI);
+            const T *xb = reinterpret_cast<const T *>(a.xcl) + c0 + cpi * CPI;
+            float r0[VEC], r1[VEC];
+#pragma unroll
+            for (int q = 0; q < VEC; q++) {
+                const int pos = oct * VEC + q;
+                const int idx = s_idx[pos];
+                const unsigned live = (unsigned)s_flag[pos];
+                float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    if ((live >> c) & 1u) {
+                        const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
+                        const float wc = s_w[c][pos];
+                        if constexpr (sizeof(T) == 2) {
+                            const uint32_t u = *reinterpret_cast<const uint32_t *>(xb + (long)v * s.Cin);
+                            v0 = fmaf(wc, __uint_as_float(u << 16), v0);
+                            v1 = fmaf(wc, __uint_as_float(u & 0xffff0000u), v1);
+                        } else {
+                            v0 = fmaf(wc, *reinterpret_cast<const float *>(xb + (long)v * s.Cin), v0);
+                        }
+                    }
+                }
+                r0[q] = v0; r1[q] = v1;
+            }
+            if constexpr (sizeof(T) == 2) {
+                uint4 p0 = make_uint4(pack_bf16x2(r0[0], r0[1]), pack_bf16x2(r0[2], r0[3]),
+                                      pack_bf16x2(r0[4], r0[5]), pack_bf16x2(r0[6], r0[7]));
+                uint4 p1 = make_uint4(pack_bf16x2(r1[0], r1[1]), pack_bf16x2(r1[2], r1[3]),
+                                      pack_bf16x2(r1[4], r1[5]), pack_bf16x2(r1[6], r1[7]));
+                *reinterpret_cast<uint4 *>(&s_tile[(cpi * 2) * TRS + oct * 16]) = p0;
+                *reinterpret_cast<uint4 *>(&s_tile[(cpi * 2 + 1) * TRS + oct * 16]) = p1;
+            } else {
+                *reinterpret_cast<uint4 *>(&s_tile[cpi * TRS + oct * 16]) =
+                    make_uint4(__float_as_uint(r0[0]), __float_as_uint(r0[1]), __float_as_uint(r0[2]),
+                               __float_as_uint(r0[3]));
+            }
+        }
+        __syncthreads();
+
+        // gW block += gout[o, pos] * tile[pos, c]
+        if (mma_wave) {
+            const T *gp = reinterpret_cast<const T *>(a.gout);
+#pragma unroll 2
+            for (int kg = 0; kg < kWMT / (2 * VEC); kg++) {
+                const int mv = m0 + (kg * 2 + (lane >> 5)) * VEC;   // first of VEC consecutive positions
+                uint4 af[OB], bf[CB];
+                const bool ok = mv < s.M;
+                const int b = ok ? mv / s.P : 0, p = ok ? mv - b * s.P : 0;
+#pragma unroll
+                for (int ob = 0; ob < OB; ob++) {
+                    const int ol = o_base + ob * 32 + (lane & 31);
+                    af[ob] = (ok && ol < s.og)
+                                 ? *reinterpret_cast<const uint4 *>(gp + ((long)b * s.Cout + wg * s.og + ol) * s.P + p)
+                                 : make_uint4(0, 0, 0, 0);
+                }
+#pragma unroll
+                for (int cb = 0; cb < CB; cb++)
+                    bf[cb] = *reinterpret_cast<const uint4 *>(&s_tile[(cb * 32 + (lane & 31)) * TRS + (kg * 2 + (lane >> 5)) * 16]);
+#pragma unroll
+                for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+                    for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], af[ob], bf[cb]);
+            }
+        }
+        __syncthreads();
+    }
+
+    if (mma_wave) {
+#pragma unroll
+        for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int ol = o_base + ob * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    const int cl = j * BKC + cb * 32 + (lane & 31);
+                    if (ol < s.og)
+                        atomicAdd(a.gwacc + ((long)(wg * s.og + ol) * s.cg + cl) * s.K + k, acc[ob][cb][r]);
+                }
+    }
+}
+
+// ============================================================ small kernels
+// W[o][c][k] -> wt[wg][step = k*nchunk + j][cc][oo]  (oo padded with zeros to ogk)
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt, TiledShape s, int ogk, long total)
+{
+    constexpr int BKC = 8 * Elem<T>::VEC;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int oo = (int)(i % ogk);
+        long r = i / ogk;
+        const int cc = (int)(r % BKC); r /= BKC;
+        const int st = (int)(r % (s.K * s.nchunk));
+        const int wg = (int)(r / (s.K * s.nchunk));
+        const int k = st / s.nchunk, j = st - k * s.nchunk;
+        wt[i] = oo < s.og ? w[((long)(wg * s.og + oo) * s.cg + j * BKC + cc) * s.K + k] : (T)0;
+    }
+}
+
+// fp32 channels-last accumulator [N][vol][C] -> grad_input [N][C][vol] of type T
+template <typename T>
+__global__ void __launch_bounds__(256) unpack_grad_input_kernel(const float *gxcl, T *gx, int C, int vol)
+{
+    __shared__ float tile[32][33];
+    const int b = blockIdx.z, v0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const float *ib = gxcl + (long)b * C * vol;
+    T *ob = gx + (long)b * C * vol;
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int v = v0 + ty + i, c = c0 + tx;
+        if (c < C && v < vol) tile[ty + i][tx] = ib[(long)v * C + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int c = c0 + ty + i, v = v0 + tx;
+        if (c < C && v < vol) ob[(long)c * vol + v] = f32_to_elem<T>(tile[tx][ty + i]);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) cvt_grad_weight_kernel(const float *src, T *dst, long n)
+{
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        dst[i] = f32_to_elem<T>(src[i]);
+}
+
+// gb[o] = sum_{b,p} gout[b,o,p]   (dconv3d_gpu.cu:1329)
+template <typename T>
+__global__ void __launch_bounds__(256) bias_grad_kernel(const T *gout, T *gb, int N, int Cout, int P)
+{
+    __shared__ float part[4];
+    const int o = blockIdx.x;
+    float acc = 0.f;
+    for (int b = 0; b < N; b++) {
+        const T *row = gout + ((long)b * Cout + o) * P;
+        for (int p = threadIdx.x; p < P; p += 256) acc += elem_to_f32<T>(row[p]);
+    }
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) gb[o] = f32_to_elem<T>(part[0] + part[1] + part[2] + part[3]);
+}
+
+inline unsigned grid1d(long n, int cap = 8192)
+{
+    long g = (n + 255) / 256;
+    return (unsigned)(g < 1 ? 1 : (g > cap ? cap : g));
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ host
+int d2c_bwd_ogk(int og, int dtype) { const int kgw = dtype == D2C_BF16 ? 16 : 8; return (og + kgw - 1) / kgw * kgw; }
+
+bool d2c_tiled_bwd_data_supported(const TiledShape &s, int dtype)
+{
+    const int ogk = d2c_bwd_ogk(s.og, dtype);
+    const int nkg = ogk / (dtype == D2C_BF16 ? 16 : 8);
+    if (nkg > 32) return false;
+    if (s.cg % s.cpg != 0) return false;  // an offset group must lie inside one weight group
+    const size_t lds = dtype == D2C_BF16 ? bwd_data_lds<bf16_t>(ogk) : bwd_data_lds<float>(ogk);
+    return lds <= 160 * 1024;
+}
+
+bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype)
+{
+    return s.P % (dtype == D2C_BF16 ? 8 : 4) == 0;
+}
+
+template <typename T>
+int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
+                              const void *mask, const void *w, void *wt, float *gxcl, void *goff, void *gmask,
+                              hipStream_t st)
+{
+    constexpr int BKC = 8 * Elem<T>::VEC;
+    const int ogk = d2c_bwd_ogk(s.og, Elem<T>::DT);
+    const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
+    hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w, (T *)wt, s, ogk,
+                       total);
+    if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
+    if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
+    BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, goff, gmask, ogk};
+    const int nkg = ogk / (2 * Elem<T>::VEC);
+    if (nkg <= 4) return launch_bwd_data<T, 4>(a, st);
+    if (nkg <= 8) return launch_bwd_data<T, 8>(a, st);
+    if (nkg <= 16) return launch_bwd_data<T, 16>(a, st);
+    return launch_bwd_data<T, 32>(a, st);
+}
+
+template <typename T>
+int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
+                                const void *mask, float *gwacc, void *gw, hipStream_t st)
+{
+    const long nw = (long)s.Cout * s.cg * s.K;
+    d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
+    const int steps = s.nchunk * s.K;
+    const int otiles = (s.og + 511) / 512;
+    const int ntile = (s.M + kWMT - 1) / kWMT;
+    int split = (512 + steps * otiles * s.groups - 1) / (steps * otiles * s.groups);
+    if (split > ntile) split = ntile;
+    if (split < 1) split = 1;
+    BwdWeightArgs a{s, gout, xcl, off, mask, gwacc, split};
+    hipLaunchKernelGGL(tiled_bwd_weight_kernel<T>, dim3(steps, otiles, s.groups * split), dim3(kThreads), 0, st, a);
+    if (int rc = d2c_check_launch("tiled_bwd_weight_kernel")) return rc;
+    hipLaunchKernelGGL(cvt_grad_weight_kernel<T>, dim3(grid1d(nw)), dim3(256), 0, st, gwacc, (T *)gw, nw);
+    return d2c_check_launch("cvt_grad_weight_kernel");
+}
+
+template <typename T>
+int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st)
+{
+    dim3 grid((s.vol + 31) / 32, (s.Cin + 31) / 32, s.N);
+    hipLaunchKernelGGL(unpack_grad_input_kernel<T>, grid, dim3(256), 0, st, gxcl, (T *)gx, s.Cin, s.vol);
+    return d2c_check_launch("unpack_grad_input_kernel");
+}
+
+template <typename T>
+int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st)
+{
+    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(s.Cout), dim3(256), 0, st, (const T *)gout, (T *)gb, s.N, s.Cout, s.P);
+    return d2c_check_launch("bias_grad_kernel");
+}
+
+#define INST(T)                                                                                                    \
+    template int d2c_tiled_bwd_data_launch<T>(const TiledShape &, const void *, const void *, const void *,        \
+                                              const void *, const void *, void *, float *, void *, void *,        \
+                                              hipStream_t);                                                        \
+    template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
+                                                const void *, float *, void *, hipStream_t);                      \
+    template int d2c_tiled_unpack_gx<T>(const TiledShape &, const float *, void *, hipStream_t);                   \
+    template int d2c_tiled_bias_grad<T>(const TiledShape &, const void *, void *, hipStream_t);
+INST(bf16_t)
+INST(float)
