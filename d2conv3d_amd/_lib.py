@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libd2conv.so")
 
 D2C_F32, D2C_F64, D2C_BF16 = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_MFMA, ALGO_DEPTHWISE = 0, 1, 2, 3
+PROF_FWD, PROF_BWD_DATA, PROF_BWD_WEIGHT, PROF_PACK = 0, 1, 2, 3
 ALGO_NAMES = {ALGO_GENERIC: "generic", ALGO_MFMA: "mfma", ALGO_DEPTHWISE: "depthwise"}
 
 # every symbol that include/d2conv.h declares
@@ -22,6 +23,7 @@ EXPORTS = (
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
     "d2c_set_algo_override", "d2c_last_error", "d2c_version",
+    "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read",
 )
 
 
@@ -75,6 +77,10 @@ def load():
     lib.d2c_conv3d_algo.argtypes, lib.d2c_conv3d_algo.restype = [p3], ctypes.c_int
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int
+    lib.d2c_profile_enable.argtypes, lib.d2c_profile_enable.restype = [ctypes.c_int], None
+    lib.d2c_profile_reset.argtypes, lib.d2c_profile_reset.restype = [], None
+    lib.d2c_profile_read.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]
+    lib.d2c_profile_read.restype = ctypes.c_int
     _lib = lib
     return lib
 

@@ -5,11 +5,22 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
+#include <vector>
 
 namespace {
 thread_local char g_err[512] = "";
 std::atomic<uint64_t> g_max_intermediate{1ull << 32};  // dconv3d_gpu.cu:12
 std::atomic<int> g_algo_override{D2C_ALGO_AUTO};
+
+struct ProfState {
+    std::mutex mu;
+    bool on = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> pending[D2C_PROF_COUNT];
+    hipEvent_t open_start[D2C_PROF_COUNT] = {};
+    double total_ms[D2C_PROF_COUNT] = {};
+    int launches[D2C_PROF_COUNT] = {};
+} g_prof;
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n)
 {
@@ -32,6 +43,28 @@ int d2c_check_launch(const char *what)
     if (e == hipSuccess) return D2C_OK;
     d2c_set_error("%s: %s", what, hipGetErrorString(e));
     return D2C_ERR_LAUNCH;
+}
+
+void d2c_prof_begin(int id, hipStream_t st)
+{
+    if (!g_prof.on) return;
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    (void)hipEventRecord(e, st);
+    g_prof.open_start[id] = e;
+}
+
+void d2c_prof_end(int id, hipStream_t st)
+{
+    if (!g_prof.on) return;
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    if (!g_prof.open_start[id]) return;
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    (void)hipEventRecord(e, st);
+    g_prof.pending[id].emplace_back(g_prof.open_start[id], e);
+    g_prof.open_start[id] = nullptr;
 }
 
 void d2c_fill_zero(void *p, size_t bytes, hipStream_t st)
@@ -63,6 +96,46 @@ int d2c_version(void) { return 1; }
 uint64_t d2c_get_max_intermediate_elements(void) { return g_max_intermediate.load(); }
 void d2c_set_max_intermediate_elements(uint64_t m) { g_max_intermediate.store(m); }
 void d2c_set_algo_override(int algo) { g_algo_override.store(algo); }
+
+void d2c_profile_enable(int on)
+{
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    g_prof.on = on != 0;
+}
+
+static void prof_drain(int id)
+{
+    for (auto &pr : g_prof.pending[id]) {
+        float ms = 0.f;
+        if (hipEventSynchronize(pr.second) == hipSuccess && hipEventElapsedTime(&ms, pr.first, pr.second) == hipSuccess) {
+            g_prof.total_ms[id] += ms;
+            g_prof.launches[id] += 1;
+        }
+        (void)hipEventDestroy(pr.first);
+        (void)hipEventDestroy(pr.second);
+    }
+    g_prof.pending[id].clear();
+}
+
+void d2c_profile_reset(void)
+{
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    for (int i = 0; i < D2C_PROF_COUNT; i++) {
+        prof_drain(i);
+        g_prof.total_ms[i] = 0.0;
+        g_prof.launches[i] = 0;
+    }
+}
+
+int d2c_profile_read(int id, double *total_ms, int *launches)
+{
+    if (id < 0 || id >= D2C_PROF_COUNT) return D2C_ERR_SHAPE;
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    prof_drain(id);
+    if (total_ms) *total_ms = g_prof.total_ms[id];
+    if (launches) *launches = g_prof.launches[id];
+    return D2C_OK;
+}
 
 static int check_dtypes(int dtype, int aux)
 {

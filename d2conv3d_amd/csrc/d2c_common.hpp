@@ -125,6 +125,15 @@ int d2c_check_launch(const char *what);
 // Clears `bytes` (a multiple of 4) with a fill kernel; safe to record into a HIP graph.
 void d2c_fill_zero(void *p, size_t bytes, hipStream_t st);
 
+// Event bracket around a kernel launch when instrumentation is on (see d2c_profile_enable).
+void d2c_prof_begin(int id, hipStream_t st);
+void d2c_prof_end(int id, hipStream_t st);
+struct D2cProfScope {
+    int id; hipStream_t st;
+    D2cProfScope(int i, hipStream_t s) : id(i), st(s) { d2c_prof_begin(id, st); }
+    ~D2cProfScope() { d2c_prof_end(id, st); }
+};
+
 static inline size_t d2c_align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
 // Kernel families (defined in their own translation units).

@@ -108,6 +108,7 @@ template <typename T>
 int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st)
 {
     dim3 grid((s.vol + 31) / 32, (s.Cin + 31) / 32, s.N);
+    D2cProfScope prof(D2C_PROF_PACK, st);
     hipLaunchKernelGGL(pack_input_kernel<T>, grid, dim3(256), 0, st, (const T *)x, (T *)xcl, s.Cin, s.vol);
     return d2c_check_launch("pack_input_kernel");
 }
@@ -123,8 +124,11 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
     const long total = (long)s.groups * s.nchunk * s.K * (s.ogp / 32) * 4 * 64;
     long g = (total + 255) / 256;
     if (g > 8192) g = 8192;
-    hipLaunchKernelGGL(pack_weight_fwd_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, (const T *)w,
-                       (T *)(base + l.wp), s, total);
+    {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        hipLaunchKernelGGL(pack_weight_fwd_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, (const T *)w,
+                           (T *)(base + l.wp), s, total);
+    }
     if (int rc = d2c_check_launch("pack_weight_fwd_kernel")) return rc;
     return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, st);
 }

@@ -292,6 +292,7 @@ int launch_bwd_data(const BwdDataArgs &a, hipStream_t st)
                             160 * 1024) != hipSuccess)
         return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_data_kernel)");
     dim3 grid((a.s.M + MT - 1) / MT, a.s.groups);
+    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
     hipLaunchKernelGGL((tiled_bwd_data_kernel<T, NKG>), grid, dim3(kThreads), lds, st, a);
     return d2c_check_launch("tiled_bwd_data_kernel");
 }
@@ -563,10 +564,13 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
     constexpr int BKC = 8 * Elem<T>::VEC;
     const int ogk = d2c_bwd_ogk(s.og, Elem<T>::DT);
     const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
-    hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w, (T *)wt, s, ogk,
-                       total);
+    {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w, (T *)wt, s,
+                           ogk, total);
+        if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
+    }
     if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
-    if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
     BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, goff, gmask, ogk};
     const int nkg = ogk / (2 * Elem<T>::VEC);
     if (nkg <= 4) return launch_bwd_data<T, 4>(a, st);
@@ -580,7 +584,10 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
                                 const void *mask, float *gwacc, void *gw, hipStream_t st)
 {
     const long nw = (long)s.Cout * s.cg * s.K;
-    d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
+    {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
+    }
     const int steps = s.nchunk * s.K;
     const int otiles = (s.og + 511) / 512;
     const int ntile = (s.M + kWMT - 1) / kWMT;
@@ -588,8 +595,12 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     if (split > ntile) split = ntile;
     if (split < 1) split = 1;
     BwdWeightArgs a{s, gout, xcl, off, mask, gwacc, split};
-    hipLaunchKernelGGL(tiled_bwd_weight_kernel<T>, dim3(steps, otiles, s.groups * split), dim3(kThreads), 0, st, a);
+    {
+        D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
+        hipLaunchKernelGGL(tiled_bwd_weight_kernel<T>, dim3(steps, otiles, s.groups * split), dim3(kThreads), 0, st, a);
+    }
     if (int rc = d2c_check_launch("tiled_bwd_weight_kernel")) return rc;
+    D2cProfScope prof(D2C_PROF_PACK, st);
     hipLaunchKernelGGL(cvt_grad_weight_kernel<T>, dim3(grid1d(nw)), dim3(256), 0, st, gwacc, (T *)gw, nw);
     return d2c_check_launch("cvt_grad_weight_kernel");
 }
@@ -598,6 +609,7 @@ template <typename T>
 int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st)
 {
     dim3 grid((s.vol + 31) / 32, (s.Cin + 31) / 32, s.N);
+    D2cProfScope prof(D2C_PROF_PACK, st);
     hipLaunchKernelGGL(unpack_grad_input_kernel<T>, grid, dim3(256), 0, st, gxcl, (T *)gx, s.Cin, s.vol);
     return d2c_check_launch("unpack_grad_input_kernel");
 }
@@ -605,6 +617,7 @@ int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStr
 template <typename T>
 int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st)
 {
+    D2cProfScope prof(D2C_PROF_PACK, st);
     hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(s.Cout), dim3(256), 0, st, (const T *)gout, (T *)gb, s.N, s.Cout, s.P);
     return d2c_check_launch("bias_grad_kernel");
 }

@@ -220,6 +220,7 @@ int launch_fwd(const FwdArgs &a, hipStream_t st)
     const int ntile = (a.s.M + kMT - 1) / kMT;
     const int NT = 64 * WO;
     dim3 grid(ntile, a.s.ogp / NT, a.s.groups);
+    D2cProfScope prof(D2C_PROF_FWD, st);
     hipLaunchKernelGGL((tiled_fwd_kernel<T, WO, WP>), grid, dim3(kThreads), 0, st, a);
     return d2c_check_launch("tiled_fwd_kernel");
 }

@@ -133,6 +133,25 @@ void d2c_set_max_intermediate_elements(uint64_t m);
  * call fail with D2C_ERR_UNSUPPORTED. */
 void d2c_set_algo_override(int algo);
 
+/*
+ * Instrumentation (no counterpart in the reference): when enabled, the main
+ * kernels are bracketed by HIP events on the stream they are launched on.
+ * d2c_profile_read() waits for the recorded events, adds their elapsed times
+ * to the totals of kernel `id` (D2C_PROF_*) and returns them; d2c_profile_reset
+ * clears the totals.  Enabling it creates events, i.e. it is not for hot loops
+ * that must not allocate.
+ */
+enum {
+    D2C_PROF_FWD = 0,         /* forward implicit-GEMM / depthwise kernel */
+    D2C_PROF_BWD_DATA = 1,    /* grad_input + grad_offset + grad_mask kernel */
+    D2C_PROF_BWD_WEIGHT = 2,  /* grad_weight kernel */
+    D2C_PROF_PACK = 3,        /* layout changes, clears, conversions (sum) */
+    D2C_PROF_COUNT = 4
+};
+void d2c_profile_enable(int on);
+void d2c_profile_reset(void);
+int d2c_profile_read(int id, double *total_ms, int *launches);
+
 const char *d2c_last_error(void);
 int d2c_version(void);
 
