@@ -22,6 +22,15 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
 template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
 template <typename T> int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st);
 
+bool d2c_depthwise_supported(const TiledShape &s);
+template <typename T>
+int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *w,
+                          void *wt, const void *bias, void *out, hipStream_t st);
+template <typename T>
+int d2c_depthwise_backward(const TiledShape &s, const void *gout, const void *xcl, const void *off, const void *mask,
+                           const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *gwacc, void *gw,
+                           hipStream_t st);
+
 namespace {
 
 inline int vec_of(int dtype) { return dtype == D2C_BF16 ? 8 : 4; }
@@ -113,13 +122,41 @@ int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st)
     return d2c_check_launch("pack_input_kernel");
 }
 
+bool is_depthwise(const d2c_conv3d_desc &q)
+{
+    if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
+    return q.groups == q.Cin && q.Cout == q.Cin && q.Cin > 1 && d2c_depthwise_supported(tiled_shape(q));
+}
+
+// depthwise workspace: channels-last input | weights [K][C] | grad_input accumulator | grad_weight accumulator
+struct DwWs {
+    size_t xcl, wt, gxcl, gwacc, total_fwd, total_bwd;
+};
+DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    const size_t es = d2c_elem_size(q.dtype);
+    DwWs w;
+    w.xcl = 0;
+    w.wt = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
+    w.total_fwd = w.wt + d2c_align_up((size_t)s.K * s.Cin * es);
+    w.gxcl = w.total_fwd;
+    w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
+    w.total_bwd = w.gwacc + d2c_align_up((size_t)s.K * s.Cin * sizeof(float));
+    return w;
+}
+
 template <typename T>
 int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
               const void *bias, void *out, void *ws, hipStream_t st)
 {
     const TiledShape s = tiled_shape(q);
-    const FwdWs l = fwd_ws(q, s);
     char *base = (char *)ws;
+    if (is_depthwise(q)) {
+        const DwWs d = dw_ws(q, s);
+        if (int rc = pack_input<T>(s, x, base + d.xcl, st)) return rc;
+        return d2c_depthwise_forward<T>(s, base + d.xcl, off, mask, w, base + d.wt, bias, out, st);
+    }
+    const FwdWs l = fwd_ws(q, s);
     if (int rc = pack_input<T>(s, x, base + l.xcl, st)) return rc;
     const long total = (long)s.groups * s.nchunk * s.K * (s.ogp / 32) * 4 * 64;
     long g = (total + 255) / 256;
@@ -153,9 +190,24 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws, hipStream_t st)
 {
     const TiledShape s = tiled_shape(q);
-    const BwdWs l = bwd_ws(q, s);
     char *base = (char *)ws;
     if (!mask) gmask = nullptr;
+    if (is_depthwise(q)) {
+        const DwWs d = dw_ws(q, s);
+        if (int rc = pack_input<T>(s, x, base + d.xcl, st)) return rc;
+        float *gxcl = gx ? (float *)(base + d.gxcl) : nullptr;
+        float *gwacc = gw ? (float *)(base + d.gwacc) : nullptr;
+        if (gx || goff || gmask || gw) {
+            if (int rc = d2c_depthwise_backward<T>(s, gout, base + d.xcl, off, mask, w, base + d.wt, gxcl, goff, gmask,
+                                                  gwacc, gw, st))
+                return rc;
+            if (gx)
+                if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
+        }
+        if (gb) return d2c_tiled_bias_grad<T>(s, gout, gb, st);
+        return D2C_OK;
+    }
+    const BwdWs l = bwd_ws(q, s);
     if (int rc = pack_input<T>(s, x, base + l.xcl, st)) return rc;
     if (gx || goff || gmask) {
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
@@ -192,16 +244,25 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
 bool d2c_tiled_supported(const d2c_conv3d_desc &q)
 {
     if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
+    if (is_depthwise(q)) return true;
     const int bkc = bkc_of(q.dtype);
     const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
     return cg % bkc == 0 && cpg % bkc == 0;
 }
 
-int d2c_tiled_algo(const d2c_conv3d_desc &) { return D2C_ALGO_MFMA; }
+int d2c_tiled_algo(const d2c_conv3d_desc &q) { return is_depthwise(q) ? D2C_ALGO_DEPTHWISE : D2C_ALGO_MFMA; }
 
-size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q) { return fwd_ws(q, tiled_shape(q)).total; }
+size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q)
+{
+    const TiledShape s = tiled_shape(q);
+    return is_depthwise(q) ? dw_ws(q, s).total_fwd : fwd_ws(q, s).total;
+}
 
-size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q) { return bwd_ws(q, tiled_shape(q)).total; }
+size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q)
+{
+    const TiledShape s = tiled_shape(q);
+    return is_depthwise(q) ? dw_ws(q, s).total_bwd : bwd_ws(q, s).total;
+}
 
 int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
                       const void *bias, void *out, void *ws, hipStream_t st)

@@ -25,7 +25,13 @@ SHAPES = {
     "c64_o600": (1, 64, 600, (2, 5, 5), (1, 3, 3), 1, (0, 1, 1), 1, 1, 1, True, True, 1.0),
     "c64_stride_dil": (2, 64, 64, (5, 9, 8), 3, (1, 2, 1), (1, 2, 2), (1, 2, 1), 1, 1, True, True, 1.0),
     "c64_tail": (3, 64, 32, (3, 7, 7), 3, 1, 1, 1, 1, 1, True, True, 1.0),   # N*P = 441: ragged last tile
+    # channel-separated (groups == Cin == Cout)
+    "dw64": (2, 64, 64, (4, 6, 7), 3, 1, 1, 1, 64, 1, True, True, 1.5),
+    "dw96_G3_nomask": (1, 96, 96, (3, 5, 9), 3, 1, 1, 1, 96, 3, False, False, 1.0),
+    "dw1100_stride": (1, 1100, 1100, (3, 6, 6), (1, 3, 3), (1, 2, 1), (0, 1, 1), 1, 1100, 1, True, True, 1.0),
+    "dw32_45taps": (2, 32, 32, (3, 7, 5), (3, 5, 3), 1, (1, 2, 1), 1, 32, 2, True, True, 1.5),
 }
+ALGO = {k: ("depthwise" if k.startswith("dw") else "mfma") for k in SHAPES}
 
 
 def make(name, dtype, seed=0):
@@ -58,7 +64,7 @@ def f32(t):
 def test_tiled_forward_backward(name, dtype, dev):
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, dtype)
     ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
-    assert _ops.conv3d_algo(ts[0], ts[1], ts[2], ts[3], s, p, d, groups, G) == "mfma"
+    assert _ops.conv3d_algo(ts[0], ts[1], ts[2], ts[3], s, p, d, groups, G) == ALGO[name]
     out = d2c.deform_conv3d(*ts, s, p, d, groups, G)
     exp = cpu.conv3d_forward(f32(x), off, m, f32(w), f32(b), s, p, d, groups, G)
     eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
