@@ -19,7 +19,7 @@ EXPORTS = (
     "d2c_output_size", "d2c_conv3d_check", "d2c_conv3d_algo",
     "d2c_conv3d_forward_workspace_bytes", "d2c_conv3d_backward_workspace_bytes",
     "d2c_conv3d_forward", "d2c_conv3d_backward",
-    "d2c_conv1d_check", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
+    "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
     "d2c_set_algo_override", "d2c_last_error", "d2c_version",
@@ -75,6 +75,7 @@ def load():
         f = getattr(lib, f"d2c_{name}_backward")
         f.argtypes, f.restype = [p] + [vp] * 11 + [sz, vp], ctypes.c_int
     lib.d2c_conv3d_algo.argtypes, lib.d2c_conv3d_algo.restype = [p3], ctypes.c_int
+    lib.d2c_conv1d_algo.argtypes, lib.d2c_conv1d_algo.restype = [p1], ctypes.c_int
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int
     lib.d2c_profile_enable.argtypes, lib.d2c_profile_enable.restype = [ctypes.c_int], None

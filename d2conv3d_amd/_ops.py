@@ -271,6 +271,17 @@ def conv3d_algo(input, offset, alpha, weight, stride=(1, 1, 1), padding=(0, 0, 0
     return _lib.ALGO_NAMES.get(lib.d2c_conv3d_algo(ctypes.byref(desc)), "invalid")
 
 
+def conv1d_algo(input, offset, alpha, weight, stride=1, padding=0, dilation=1, groups=1, offset_groups=1):
+    """Name of the kernel family ("generic" or "mfma") that serves these 1-D arguments."""
+    lib = _lib.load()
+    input, offset, alpha, weight, _ = _unify(input, offset, alpha, weight, None)
+    N, Cin, L = input.shape
+    Cout, _, k = weight.shape
+    desc = _lib.Conv1dDesc(N, Cin, Cout, L, k, _one(stride), _one(padding), _one(dilation), groups, offset_groups,
+                           offset.shape[2], _DT[input.dtype], _DT[offset.dtype], 1)
+    return _lib.ALGO_NAMES.get(lib.d2c_conv1d_algo(ctypes.byref(desc)), "invalid")
+
+
 def set_algo_override(name):
     """Test hook: force "generic" / "mfma" / "depthwise", or None for the default choice."""
     code = {None: _lib.ALGO_AUTO, "auto": _lib.ALGO_AUTO, "generic": _lib.ALGO_GENERIC,

@@ -291,24 +291,38 @@ int d2c_conv3d_corner_index(const d2c_conv3d_desc *q, const void *offset, int32_
     return d2c_generic_conv3d_corners(*q, offset, base, flags, (hipStream_t)stream);
 }
 
+static bool use_tiled1d(const d2c_conv1d_desc &q)
+{
+    return g_algo_override.load() != D2C_ALGO_GENERIC && d2c_tiled1d_supported(q);
+}
+
+int d2c_conv1d_algo(const d2c_conv1d_desc *q)
+{
+    if (d2c_conv1d_check(q) != D2C_OK) return -1;
+    return use_tiled1d(*q) ? D2C_ALGO_MFMA : D2C_ALGO_GENERIC;
+}
+
 size_t d2c_conv1d_forward_workspace_bytes(const d2c_conv1d_desc *q)
 {
     if (d2c_conv1d_check(q) != D2C_OK) return 0;
-    return 0;
+    return use_tiled1d(*q) ? d2c_tiled1d_forward_ws(*q) : 0;
 }
 
 size_t d2c_conv1d_backward_workspace_bytes(const d2c_conv1d_desc *q)
 {
     if (d2c_conv1d_check(q) != D2C_OK) return 0;
-    return d2c_generic_conv1d_backward_ws(*q);
+    return use_tiled1d(*q) ? d2c_tiled1d_backward_ws(*q) : d2c_generic_conv1d_backward_ws(*q);
 }
 
 int d2c_conv1d_forward(const d2c_conv1d_desc *q, const void *x, const void *offset, const void *mask,
                        const void *weight, const void *bias, void *out, void *ws, size_t ws_bytes, void *stream)
 {
-    (void)ws; (void)ws_bytes;
     if (int rc = d2c_conv1d_check(q)) return rc;
     if (!x || !offset || !weight || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (use_tiled1d(*q)) {
+        if (int rc = check_ws(d2c_tiled1d_forward_ws(*q), ws, ws_bytes)) return rc;
+        return d2c_tiled1d_forward(*q, x, offset, mask, weight, bias, out, ws, (hipStream_t)stream);
+    }
     return d2c_generic_conv1d_forward(*q, x, offset, mask, weight, bias, out, (hipStream_t)stream);
 }
 
@@ -318,6 +332,10 @@ int d2c_conv1d_backward(const d2c_conv1d_desc *q, const void *gout, const void *
 {
     if (int rc = d2c_conv1d_check(q)) return rc;
     if (!gout || !x || !offset || !weight) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (use_tiled1d(*q)) {
+        if (int rc = check_ws(d2c_tiled1d_backward_ws(*q), ws, ws_bytes)) return rc;
+        return d2c_tiled1d_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws, (hipStream_t)stream);
+    }
     if (int rc = check_ws(d2c_generic_conv1d_backward_ws(*q), ws, ws_bytes)) return rc;
     return d2c_generic_conv1d_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws,
                                        (hipStream_t)stream);

@@ -123,5 +123,23 @@ struct TiledShape {
     int adt;
     int P, vol;           // output positions / input voxels per sample
     int M;                // N * P
+    int nd;               // 3, or 1 for the 1-D operator mapped onto a 1 x 1 x L volume
+    int quirks;           // 1-D only: integer-position rule of dconv1d_gpu.cu:332-336 in grad_offset / grad_mask
     TapGeom geo;
 };
+
+// The three offsets (dz, dy, dx) of (b, g, k, p).  The 1-D operator stores one
+// offset per tap ([N, G*K, Lo], dconv1d_gpu.cu:40); it displaces along x only.
+D2C_DEV void load_offsets(const TiledShape &s, const void *off, int b, int g, int k, int p, float &o0, float &o1,
+                          float &o2)
+{
+    if (s.nd == 3) {
+        const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
+        o0 = ld_aux(off, ob, s.adt);
+        o1 = ld_aux(off, ob + s.P, s.adt);
+        o2 = ld_aux(off, ob + 2 * (long)s.P, s.adt);
+    } else {
+        o0 = 0.f; o1 = 0.f;
+        o2 = ld_aux(off, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt);
+    }
+}

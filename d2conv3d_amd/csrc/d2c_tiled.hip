@@ -4,7 +4,7 @@
 #include "d2c_tiled.hpp"
 #include "d2c_mma.hpp"
 
-int d2c_fwd_out_tile(int og);
+int d2c_fwd_out_tile(int og, int M);
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
                          const void *bias, void *out, hipStream_t st);
@@ -12,6 +12,7 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
 bool d2c_tiled_bwd_data_supported(const TiledShape &s, int dtype);
 bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype);
 int d2c_bwd_ogk(int og, int dtype);
+int d2c_bwd_pass_channels(int dtype);
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *goff, void *gmask,
@@ -36,18 +37,30 @@ namespace {
 inline int vec_of(int dtype) { return dtype == D2C_BF16 ? 8 : 4; }
 inline int bkc_of(int dtype) { return 8 * vec_of(dtype); }
 
-TiledShape tiled_shape(const d2c_conv3d_desc &q)
+// The 1-D operator as a 3-D problem on a 1 x 1 x L volume with a 1 x 1 x k kernel.
+d2c_conv3d_desc as_3d(const d2c_conv1d_desc &q)
+{
+    d2c_conv3d_desc r;
+    r.N = q.N; r.Cin = q.Cin; r.Cout = q.Cout; r.D = 1; r.H = 1; r.W = q.L;
+    r.kd = 1; r.kh = 1; r.kw = q.k; r.sd = 1; r.sh = 1; r.sw = q.s; r.pd = 0; r.ph = 0; r.pw = q.p;
+    r.dd = 1; r.dh = 1; r.dw = q.d; r.groups = q.groups; r.offset_groups = q.offset_groups;
+    r.Do = 1; r.Ho = 1; r.Wo = q.Lo; r.dtype = q.dtype; r.aux_dtype = q.aux_dtype;
+    return r;
+}
+
+TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0)
 {
     TiledShape s;
+    s.nd = nd; s.quirks = quirks;
     s.N = q.N; s.Cin = q.Cin; s.Cout = q.Cout; s.D = q.D; s.H = q.H; s.W = q.W;
     s.K = q.kd * q.kh * q.kw; s.G = q.offset_groups; s.groups = q.groups;
     s.Do = q.Do; s.Ho = q.Ho; s.Wo = q.Wo;
     s.cg = q.Cin / q.groups; s.og = q.Cout / q.groups; s.cpg = q.Cin / q.offset_groups;
     s.nchunk = s.cg / bkc_of(q.dtype);
-    const int nt = d2c_fwd_out_tile(s.og);
-    s.ogp = (s.og + nt - 1) / nt * nt;
     s.adt = q.aux_dtype;
     s.P = q.Do * q.Ho * q.Wo; s.vol = q.D * q.H * q.W; s.M = q.N * s.P;
+    const int nt = d2c_fwd_out_tile(s.og, s.M);
+    s.ogp = (s.og + nt - 1) / nt * nt;
     s.geo = make_geom(q);
     return s;
 }
@@ -147,11 +160,11 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 
 template <typename T>
 int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
-              const void *bias, void *out, void *ws, hipStream_t st)
+              const void *bias, void *out, void *ws, hipStream_t st, int nd = 3)
 {
-    const TiledShape s = tiled_shape(q);
+    const TiledShape s = tiled_shape(q, nd, 0);
     char *base = (char *)ws;
-    if (is_depthwise(q)) {
+    if (nd == 3 && is_depthwise(q)) {
         const DwWs d = dw_ws(q, s);
         if (int rc = pack_input<T>(s, x, base + d.xcl, st)) return rc;
         return d2c_depthwise_forward<T>(s, base + d.xcl, off, mask, w, base + d.wt, bias, out, st);
@@ -179,7 +192,9 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     BwdWs w;
     w.xcl = 0;
     w.wt = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
-    w.gxcl = w.wt + d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * d2c_bwd_ogk(s.og, q.dtype) * es);
+    const int omax = d2c_bwd_pass_channels(q.dtype);
+    const int ogk = d2c_bwd_ogk(s.og < omax ? s.og : omax, q.dtype);
+    w.gxcl = w.wt + d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * ogk * es);
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
     w.total = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
     return w;
@@ -187,12 +202,13 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 
 template <typename T>
 int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off, const void *mask,
-               const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws, hipStream_t st)
+               const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws, hipStream_t st,
+               int nd = 3, int quirks = 0)
 {
-    const TiledShape s = tiled_shape(q);
+    const TiledShape s = tiled_shape(q, nd, quirks);
     char *base = (char *)ws;
     if (!mask) gmask = nullptr;
-    if (is_depthwise(q)) {
+    if (nd == 3 && is_depthwise(q)) {
         const DwWs d = dw_ws(q, s);
         if (int rc = pack_input<T>(s, x, base + d.xcl, st)) return rc;
         float *gxcl = gx ? (float *)(base + d.gxcl) : nullptr;
@@ -240,6 +256,51 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
 }
 
 }  // namespace
+
+static bool mfma_channels_ok(const d2c_conv3d_desc &q)
+{
+    if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
+    const int bkc = bkc_of(q.dtype);
+    const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
+    return cg % bkc == 0 && cpg % bkc == 0;
+}
+
+// ---- 1-D operator on the matrix-core kernels -----------------------------
+// Served when the channel counts fit the chunking and both backward kernels
+// can take the shape; otherwise the direct 1-D kernels run.
+bool d2c_tiled1d_supported(const d2c_conv1d_desc &q1)
+{
+    const d2c_conv3d_desc q = as_3d(q1);
+    if (!mfma_channels_ok(q)) return false;
+    const TiledShape s = tiled_shape(q, 1, q1.reference_quirks);
+    return d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_weight_supported(s, q.dtype);
+}
+size_t d2c_tiled1d_forward_ws(const d2c_conv1d_desc &q1)
+{
+    const d2c_conv3d_desc q = as_3d(q1);
+    return fwd_ws(q, tiled_shape(q, 1, 0)).total;
+}
+size_t d2c_tiled1d_backward_ws(const d2c_conv1d_desc &q1)
+{
+    const d2c_conv3d_desc q = as_3d(q1);
+    return bwd_ws(q, tiled_shape(q, 1, 0)).total;
+}
+int d2c_tiled1d_forward(const d2c_conv1d_desc &q1, const void *x, const void *off, const void *mask, const void *w,
+                        const void *bias, void *out, void *ws, hipStream_t st)
+{
+    const d2c_conv3d_desc q = as_3d(q1);
+    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 1);
+    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 1);
+}
+int d2c_tiled1d_backward(const d2c_conv1d_desc &q1, const void *gout, const void *x, const void *off,
+                         const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
+                         void *ws, hipStream_t st)
+{
+    const d2c_conv3d_desc q = as_3d(q1);
+    if (q.dtype == D2C_BF16)
+        return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 1, q1.reference_quirks);
+    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 1, q1.reference_quirks);
+}
 
 bool d2c_tiled_supported(const d2c_conv3d_desc &q)
 {

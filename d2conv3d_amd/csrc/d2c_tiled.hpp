@@ -12,3 +12,13 @@ int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, 
 int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
                        const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
                        void *ws, hipStream_t st);
+
+// 1-D operator served by the same matrix-core kernels (1 x 1 x L volume).
+bool d2c_tiled1d_supported(const d2c_conv1d_desc &q);
+size_t d2c_tiled1d_forward_ws(const d2c_conv1d_desc &q);
+size_t d2c_tiled1d_backward_ws(const d2c_conv1d_desc &q);
+int d2c_tiled1d_forward(const d2c_conv1d_desc &q, const void *x, const void *off, const void *mask, const void *w,
+                        const void *bias, void *out, void *ws, hipStream_t st);
+int d2c_tiled1d_backward(const d2c_conv1d_desc &q, const void *gout, const void *x, const void *off,
+                         const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
+                         void *ws, hipStream_t st);

@@ -39,7 +39,9 @@ struct BwdDataArgs {
     const void *wt;     // [groups][K*nchunk][BKC][ogk]   (W transposed per step, zero padded to ogk)
     float *gxcl;        // [N][vol][Cin] fp32 accumulator (zeroed) or NULL
     void *goff, *gmask; // or NULL
-    int ogk;            // og rounded up to a whole k-group
+    int ogk;            // output channels of this pass rounded up to a whole k-group
+    int o0, ogn;        // this pass reduces over output channels [o0, o0 + ogn) of each weight group
+    int add_aux;        // later passes add to the offset / mask gradient of earlier ones
 };
 
 // NKG = k-groups of the reduction over output channels held in registers.
@@ -63,7 +65,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
     float *s_frac = s_w + 8 * MT;                        // [6][MT]  lz ly lx hz hy hx
     float *s_alpha = s_frac + 6 * MT;                    // [MT]
     int *s_idx = reinterpret_cast<int *>(s_alpha + MT);  // [MT]
-    int *s_flag = s_idx + MT;                            // [MT]     live | inrange << 8
+    int *s_flag = s_idx + MT;                            // [MT]     live | inrange << 8 | 1-D low-corner shift << 16 | mask-gradient corners << 24
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
@@ -80,14 +82,14 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
         const int m = m0 + pb * 32 + (lane & 31);
         const bool ok = m < s.M;
         const int b = ok ? m / s.P : 0, p = ok ? m - b * s.P : 0;
-        const T *gp = reinterpret_cast<const T *>(a.gout) + ((long)b * s.Cout + wg * s.og) * s.P + p;
+        const T *gp = reinterpret_cast<const T *>(a.gout) + ((long)b * s.Cout + wg * s.og + a.o0) * s.P + p;
 #pragma unroll
         for (int kg = 0; kg < NKG; kg++) {
             T e[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; i++) {
                 const int o = (kg * 2 + (lane >> 5)) * VEC + i;
-                e[i] = (ok && kg < nkg && o < s.og) ? gp[(long)o * s.P] : (T)0;
+                e[i] = (ok && kg < nkg && o < a.ogn) ? gp[(long)o * s.P] : (T)0;
             }
             ga[kg] = *reinterpret_cast<uint4 *>(e);
         }
@@ -126,19 +128,35 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
             float al = 0.f;
             int idx = 0, flag = 0;
             if (cvalid) {
-                const long ob = (((long)cbatch * s.G + g) * s.K + k) * 3 * s.P + cp;
-                const float o0 = ld_aux(a.off, ob, s.adt);
-                const float o1 = ld_aux(a.off, ob + s.P, s.adt);
-                const float o2 = ld_aux(a.off, ob + 2 * (long)s.P, s.adt);
+                float o0, o1, o2;
+                load_offsets(s, a.off, cbatch, g, k, cp, o0, o1, o2);
                 al = a.mask ? ld_aux(a.mask, (((long)cbatch * s.G + g) * s.K + k) * s.P + cp, s.adt) : 1.f;
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
                 idx = cbatch * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0;
-                flag = (int)(t.live | (t.inrange << 8));
+                unsigned inr = t.inrange, auxlive = t.live;
+                fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
+                if (s.nd == 1) {
+                    // 1-D: both corners are gated by range only (dconv1d_gpu.cu:338-339), and at
+                    // integer positions the low corner steps down by one while the high corner stays
+                    // (:332-336); grad_offset / grad_mask then interpolate with t' = x - (x0 - 1).
+                    int x0q = t.x0;
+                    if (s.quirks && (double)t.hx < 1e-8) {
+                        x0q -= 1;
+                        flag |= 1 << 16;
+                        const float x = (float)bx + o2;
+                        const float tq = x - (float)x0q;
+                        fr[2] = 1.f - tq; fr[5] = tq;
+                    }
+                    const unsigned lo = (x0q >= 0 && x0q < s.W) ? 1u : 0u;
+                    const unsigned hi = (t.x0 + 1 >= 0 && t.x0 + 1 < s.W) ? 2u : 0u;
+                    inr = lo | hi;
+                    auxlive = inr;
+                }
+                flag |= (int)(t.live | (inr << 8) | (auxlive << 24));
 #pragma unroll
                 for (int c = 0; c < 8; c++) w[c] = ((t.live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
-                fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
             }
 #pragma unroll
             for (int c = 0; c < 8; c++) s_w[c * MT + tid] = w[c];
@@ -210,7 +228,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                 const int pos = item / NV, vec = item % NV;
                 const int idx = s_idx[pos];
                 const unsigned flag = (unsigned)s_flag[pos];
-                const unsigned inr = flag >> 8, live = flag & 0xffu;
+                const unsigned inr = (flag >> 8) & 0xffu, live = flag >> 24;
+                const int qshift = (flag >> 16) & 1;
                 float gc[VEC];
                 {
                     const float4 *gp4 = reinterpret_cast<const float4 *>(s_gcol + pos * GRS + vec * VEC * 4);
@@ -226,7 +245,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                 for (int c = 0; c < 8; c++) {
                     float d = 0.f;
                     if ((inr >> c) & 1u) {
-                        const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
+                        const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + ((c & 1) ? 1 : -qshift);
                         const uint4 xv = *reinterpret_cast<const uint4 *>(xb + (long)v * s.Cin);
                         const T *xe = reinterpret_cast<const T *>(&xv);
 #pragma unroll
@@ -260,13 +279,19 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                         const int m = m0 + pos;
                         if (m < s.M) {
                             const int b = m / s.P, p = m - b * s.P;
-                            if (a.goff) {
-                                const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
-                                st_aux(a.goff, ob, s.adt, g_acc[i][0]);
-                                st_aux(a.goff, ob + s.P, s.adt, g_acc[i][1]);
-                                st_aux(a.goff, ob + 2 * (long)s.P, s.adt, g_acc[i][2]);
+                            const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
+                            if (a.goff && s.nd == 3) {
+                                const long ob = 3 * ab - 2 * (long)p;   // ((b*G+g)*K+k)*3*P + p
+#pragma unroll
+                                for (int ax = 0; ax < 3; ax++) {
+                                    const long oi = ob + ax * (long)s.P;
+                                    st_aux(a.goff, oi, s.adt, g_acc[i][ax] + (a.add_aux ? ld_aux(a.goff, oi, s.adt) : 0.f));
+                                }
+                            } else if (a.goff) {
+                                st_aux(a.goff, ab, s.adt, g_acc[i][2] + (a.add_aux ? ld_aux(a.goff, ab, s.adt) : 0.f));
                             }
-                            if (a.gmask) st_aux(a.gmask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt, g_acc[i][3]);
+                            if (a.gmask)
+                                st_aux(a.gmask, ab, s.adt, g_acc[i][3] + (a.add_aux ? ld_aux(a.gmask, ab, s.adt) : 0.f));
                         }
                         g_acc[i][0] = g_acc[i][1] = g_acc[i][2] = g_acc[i][3] = 0.f;
                     }
@@ -359,10 +384,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
             if (m < s.M) {
                 const int b = m / s.P, p = m - b * s.P;
                 const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
-                const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
-                const float o0 = ld_aux(a.off, ob, s.adt);
-                const float o1 = ld_aux(a.off, ob + s.P, s.adt);
-                const float o2 = ld_aux(a.off, ob + 2 * (long)s.P, s.adt);
+                float o0, o1, o2;
+                load_offsets(s, a.off, b, g, k, p, o0, o1, o2);
                 const float al = a.mask ? ld_aux(a.mask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt) : 1.f;
                 int bz, by, bx;
                 tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
@@ -467,9 +490,10 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
 }
 
 // ============================================================ small kernels
-// W[o][c][k] -> wt[wg][step = k*nchunk + j][cc][oo]  (oo padded with zeros to ogk)
+// W[o][c][k] -> wt[wg][step = k*nchunk + j][cc][oo] for oo in [o0, o0 + ogn), padded with zeros to ogk
 template <typename T>
-__global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt, TiledShape s, int ogk, long total)
+__global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt, TiledShape s, int ogk, int o0,
+                                                              int ogn, long total)
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
@@ -479,7 +503,7 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
         const int st = (int)(r % (s.K * s.nchunk));
         const int wg = (int)(r / (s.K * s.nchunk));
         const int k = st / s.nchunk, j = st - k * s.nchunk;
-        wt[i] = oo < s.og ? w[((long)(wg * s.og + oo) * s.cg + j * BKC + cc) * s.K + k] : (T)0;
+        wt[i] = oo < ogn ? w[((long)(wg * s.og + o0 + oo) * s.cg + j * BKC + cc) * s.K + k] : (T)0;
     }
 }
 
@@ -541,14 +565,13 @@ inline unsigned grid1d(long n, int cap = 8192)
 // ------------------------------------------------------------------ host
 int d2c_bwd_ogk(int og, int dtype) { const int kgw = dtype == D2C_BF16 ? 16 : 8; return (og + kgw - 1) / kgw * kgw; }
 
-bool d2c_tiled_bwd_data_supported(const TiledShape &s, int dtype)
+// Output channels one pass of the data kernel reduces over: 32 k-groups of the
+// stationary operand fit the register file (512 bf16 / 256 float channels).
+int d2c_bwd_pass_channels(int dtype) { return 32 * (dtype == D2C_BF16 ? 16 : 8); }
+
+bool d2c_tiled_bwd_data_supported(const TiledShape &s, int)
 {
-    const int ogk = d2c_bwd_ogk(s.og, dtype);
-    const int nkg = ogk / (dtype == D2C_BF16 ? 16 : 8);
-    if (nkg > 32) return false;
-    if (s.cg % s.cpg != 0) return false;  // an offset group must lie inside one weight group
-    const size_t lds = dtype == D2C_BF16 ? bwd_data_lds<bf16_t>(ogk) : bwd_data_lds<float>(ogk);
-    return lds <= 160 * 1024;
+    return s.cg % s.cpg == 0;  // an offset group must lie inside one weight group
 }
 
 bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype)
@@ -562,21 +585,33 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                               hipStream_t st)
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
-    const int ogk = d2c_bwd_ogk(s.og, Elem<T>::DT);
-    const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
-    {
+    const int omax = d2c_bwd_pass_channels(Elem<T>::DT);
+    if (gxcl) {
         D2cProfScope prof(D2C_PROF_PACK, st);
-        hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w, (T *)wt, s,
-                           ogk, total);
-        if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
+        d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
     }
-    if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
-    BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, goff, gmask, ogk};
-    const int nkg = ogk / (2 * Elem<T>::VEC);
-    if (nkg <= 4) return launch_bwd_data<T, 4>(a, st);
-    if (nkg <= 8) return launch_bwd_data<T, 8>(a, st);
-    if (nkg <= 16) return launch_bwd_data<T, 16>(a, st);
-    return launch_bwd_data<T, 32>(a, st);
+    // Weight groups wider than one pass can hold are reduced in several passes; every
+    // quantity downstream of the grad-column product is linear in it, so the passes add up.
+    for (int o0 = 0; o0 < s.og; o0 += omax) {
+        const int ogn = s.og - o0 < omax ? s.og - o0 : omax;
+        const int ogk = d2c_bwd_ogk(ogn, Elem<T>::DT);
+        const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
+        {
+            D2cProfScope prof(D2C_PROF_PACK, st);
+            hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w, (T *)wt,
+                               s, ogk, o0, ogn, total);
+        }
+        if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
+        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0};
+        const int nkg = ogk / (2 * Elem<T>::VEC);
+        int rc;
+        if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, st);
+        else if (nkg <= 8) rc = launch_bwd_data<T, 8>(a, st);
+        else if (nkg <= 16) rc = launch_bwd_data<T, 16>(a, st);
+        else rc = launch_bwd_data<T, 32>(a, st);
+        if (rc) return rc;
+    }
+    return D2C_OK;
 }
 
 template <typename T>

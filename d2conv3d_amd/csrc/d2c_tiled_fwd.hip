@@ -88,10 +88,8 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
             if (cvalid) {
                 const int j = st / s.K, k = st - j * s.K;
                 const int g = (wg * s.cg + j * BKC) / s.cpg;
-                const long ob = (((long)cb * s.G + g) * s.K + k) * 3 * s.P + cp;
-                const float o0 = ld_aux(a.off, ob, s.adt);
-                const float o1 = ld_aux(a.off, ob + s.P, s.adt);
-                const float o2 = ld_aux(a.off, ob + 2 * (long)s.P, s.adt);
+                float o0, o1, o2;
+                load_offsets(s, a.off, cb, g, k, cp, o0, o1, o2);
                 const float al = a.mask ? ld_aux(a.mask, (((long)cb * s.G + g) * s.K + k) * s.P + cp, s.adt) : 1.f;
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
@@ -227,9 +225,15 @@ int launch_fwd(const FwdArgs &a, hipStream_t st)
 
 }  // namespace
 
-int d2c_fwd_out_tile(int og)
+// Output channels per workgroup: as wide as the weight group needs (the sampled
+// tile is then produced once), but narrower when there are too few position
+// tiles to occupy the chip.
+int d2c_fwd_out_tile(int og, int M)
 {
-    return og > 256 ? 512 : (og > 128 ? 256 : (og > 64 ? 128 : 64));
+    int nt = og > 256 ? 512 : (og > 128 ? 256 : (og > 64 ? 128 : 64));
+    const int ntile = (M + kMT - 1) / kMT;
+    while (nt > 64 && ntile * ((og + nt - 1) / nt) < 128) nt >>= 1;
+    return nt;
 }
 
 template <typename T>
@@ -237,7 +241,7 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
                          const void *bias, void *out, hipStream_t st)
 {
     FwdArgs a{s, xcl, off, mask, wp, bias, out};
-    switch (d2c_fwd_out_tile(s.og)) {
+    switch (d2c_fwd_out_tile(s.og, s.M)) {
     case 512: return launch_fwd<T, 8, 1>(a, st);
     case 256: return launch_fwd<T, 4, 2>(a, st);
     case 128: return launch_fwd<T, 2, 4>(a, st);

@@ -101,6 +101,7 @@ int d2c_conv3d_backward(const d2c_conv3d_desc *desc, const void *grad_out, const
                         void *grad_bias, void *workspace, size_t workspace_bytes, void *stream);
 
 int d2c_conv1d_check(const d2c_conv1d_desc *desc);
+int d2c_conv1d_algo(const d2c_conv1d_desc *desc);   /* D2C_ALGO_GENERIC or D2C_ALGO_MFMA */
 size_t d2c_conv1d_forward_workspace_bytes(const d2c_conv1d_desc *desc);
 size_t d2c_conv1d_backward_workspace_bytes(const d2c_conv1d_desc *desc);
 

@@ -109,3 +109,73 @@ def test_bfloat16_offsets_and_masks_in_bfloat16(dev):
     eg = cpu.conv3d_backward(f32(gout), f32(x), f32(off), f32(m), f32(w), True, s, p, d, groups, G)
     for t, e in zip(ts, eg):
         assert t.grad.dtype == torch.bfloat16 and rel_l2(t.grad, e) < 2e-2
+
+
+# ------------------------------------------------------------------ 1-D operator on the tiled kernels
+SHAPES_1D = {
+    # name: (N, Cin, Cout, L, k, stride, pad, dil, groups, G, bias, mask, sigma)
+    "l64_c64": (4, 64, 64, 64, 3, 1, 1, 1, 1, 1, True, True, 1.5),
+    "l40_c128_G2_o96": (2, 128, 96, 40, 5, 1, 2, 1, 1, 2, True, True, 2.0),
+    "l50_groups2_stride": (2, 128, 128, 50, 3, 2, 1, 2, 2, 2, False, False, 1.0),
+}
+
+
+def make1d(name, dtype, seed=0):
+    N, Cin, Cout, L, k, s, p, d, groups, G, bias, mask, sig = SHAPES_1D[name]
+    Lo = (L + 2 * p - (d * (k - 1) + 1)) // s + 1
+    g = torch.Generator().manual_seed(2000 + seed)
+    x = torch.randn(N, Cin, L, generator=g)
+    w = (torch.rand(Cout, Cin // groups, k, generator=g) * 2 - 1) / (Cin // groups * k) ** 0.5
+    b = (torch.rand(Cout, generator=g) * 2 - 1) / (Cin // groups * k) ** 0.5 if bias else None
+    off = torch.randn(N, G * k, Lo, generator=g) * sig
+    m = torch.sigmoid(torch.randn(N, G * k, Lo, generator=g)) if mask else None
+    gout = torch.randn(N, Cout, Lo, generator=g)
+    if dtype == torch.bfloat16:
+        x, w, gout = x.bfloat16(), w.bfloat16(), gout.bfloat16()
+        b = b.bfloat16() if b is not None else None
+    return (x, off, m, w, b), gout, (s, p, d, groups, G)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("name", list(SHAPES_1D))
+def test_tiled_conv1d_forward_backward(name, dtype, dev):
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make1d(name, dtype)
+    ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+    assert _ops.conv1d_algo(ts[0], ts[1], ts[2], ts[3], s, p, d, groups, G) == "mfma"
+    out = d2c.deform_conv1d(*ts, s, p, d, groups, G)
+    exp = cpu.conv1d_forward(f32(x), off, m, f32(w), f32(b), s, p, d, groups, G)
+    eg = cpu.conv1d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+    out.backward(gout.to(dev))
+    names = ("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias")
+    if dtype == torch.float32:
+        assert_close(out, exp, 1e-4, 1e-5, "forward")
+        for n, t, e in zip(names, ts, eg):
+            if t is not None:
+                assert_close(t.grad, e, 1e-4, 1e-5 * max(1.0, e.abs().max().item()), n)
+    else:
+        assert rel_l2(out, exp) < 2e-2
+        for n, t, e in zip(names, ts, eg):
+            if t is not None:
+                assert rel_l2(t.grad, e) < 2e-2, (n, rel_l2(t.grad, e))
+
+
+@pytest.mark.parametrize("quirks", [True, False])
+def test_tiled_conv1d_integer_positions(quirks, dev):
+    # integer sampling positions (the state at zero-initialised offsets): dconv1d_gpu.cu:332-351
+    g = torch.Generator().manual_seed(5)
+    N, C, L = 2, 32, 16
+    x = torch.randn(N, C, L, generator=g)
+    w = torch.randn(C, C, 3, generator=g) / 10
+    off = torch.zeros(N, 3, L)
+    off[:, 1, ::2] = 2.0          # a mix of integer offsets; some land outside the signal
+    off[:, 2, 1::3] = -3.0
+    off[1, 0, :] = torch.randn(L, generator=g)   # and non-integer ones
+    m = torch.sigmoid(torch.randn(N, 3, L, generator=g))
+    gout = torch.randn(N, C, L, generator=g)
+    eg = cpu.conv1d_backward(gout, x, off, m, w, False, 1, 1, 1, 1, 1, quirks=quirks)
+    ts = [t.to(dev).requires_grad_(True) for t in (x, off, m, w)]
+    assert _ops.conv1d_algo(ts[0], ts[1], ts[2], ts[3], 1, 1, 1, 1, 1) == "mfma"
+    out = _ops.deform_conv1d(ts[0], ts[1], ts[2], ts[3], None, 1, 1, 1, 1, 1, reference_quirks=quirks)
+    out.backward(gout.to(dev))
+    for n, t, e in zip(("grad_input", "grad_offset", "grad_mask", "grad_weight"), ts, eg):
+        assert_close(t.grad, e, 1e-4, 1e-5 * max(1.0, e.abs().max().item()), f"{n} quirks={quirks}")
