@@ -241,16 +241,20 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                 }
                 const T *xb = reinterpret_cast<const T *>(a.xcl) + c0 + vec * VEC;
                 float dot[8];
+                uint4 xv[8];
+                // all eight (predicated) loads are issued before any of them is used
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
-                    float d = 0.f;
-                    if ((inr >> c) & 1u) {
-                        const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + ((c & 1) ? 1 : -qshift);
-                        const uint4 xv = *reinterpret_cast<const uint4 *>(xb + (long)v * s.Cin);
-                        const T *xe = reinterpret_cast<const T *>(&xv);
+                    const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + ((c & 1) ? 1 : -qshift);
+                    xv[c] = ((inr >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + (long)v * s.Cin)
+                                              : make_uint4(0, 0, 0, 0);
+                }
 #pragma unroll
-                        for (int e = 0; e < VEC; e++) d = fmaf(gc[e], elem_to_f32<T>(xe[e]), d);
-                    }
+                for (int c = 0; c < 8; c++) {
+                    const T *xe = reinterpret_cast<const T *>(&xv[c]);
+                    float d = 0.f;
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) d = fmaf(gc[e], elem_to_f32<T>(xe[e]), d);
                     dot[c] = d;
                 }
                 // sum over the 8 lanes that share the position
@@ -415,18 +419,22 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
                 const int idx = s_idx[pos];
                 const unsigned live = (unsigned)s_flag[pos];
                 float v0 = 0.f, v1 = 0.f;
+                uint32_t u[8];
+                // all eight (predicated) loads are issued before any of them is used
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
-                    if ((live >> c) & 1u) {
-                        const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
-                        const float wc = s_w[c][pos];
-                        if constexpr (sizeof(T) == 2) {
-                            const uint32_t u = *reinterpret_cast<const uint32_t *>(xb + (long)v * s.Cin);
-                            v0 = fmaf(wc, __uint_as_float(u << 16), v0);
-                            v1 = fmaf(wc, __uint_as_float(u & 0xffff0000u), v1);
-                        } else {
-                            v0 = fmaf(wc, *reinterpret_cast<const float *>(xb + (long)v * s.Cin), v0);
-                        }
+                    const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
+                    u[c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint32_t *>(xb + (long)v * s.Cin) : 0u;
+                }
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    const float wc = s_w[c][pos];
+                    const uint32_t uc = u[c];
+                    if constexpr (sizeof(T) == 2) {
+                        v0 = fmaf(wc, __uint_as_float(uc << 16), v0);
+                        v1 = fmaf(wc, __uint_as_float(uc & 0xffff0000u), v1);
+                    } else {
+                        v0 = fmaf(wc, __uint_as_float(uc), v0);
                     }
                 }
                 r0[q] = v0; r1[q] = v1;
