@@ -150,7 +150,8 @@ def main():
     lib.d2c_profile_enable(0)
     kern = {}
     for kid, kname in ((_lib.PROF_FWD, "tiled_fwd_kernel"), (_lib.PROF_BWD_DATA, "tiled_bwd_data_kernel"),
-                       (_lib.PROF_BWD_WEIGHT, "tiled_bwd_weight_kernel"), (_lib.PROF_PACK, "pack/clear/convert")):
+                       (_lib.PROF_BWD_WEIGHT, "tiled_bwd_weight_kernel"), (_lib.PROF_GX_OWNER, "gx_owner_kernel"),
+                       (_lib.PROF_PACK, "pack/clear/convert/lists")):
         tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
         lib.d2c_profile_read(kid, ctypes.byref(tot), ctypes.byref(cnt))
         if cnt.value:

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libd2conv.so")
 
 D2C_F32, D2C_F64, D2C_BF16 = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_MFMA, ALGO_DEPTHWISE = 0, 1, 2, 3
-PROF_FWD, PROF_BWD_DATA, PROF_BWD_WEIGHT, PROF_PACK = 0, 1, 2, 3
+PROF_FWD, PROF_BWD_DATA, PROF_BWD_WEIGHT, PROF_PACK, PROF_GX_OWNER = 0, 1, 2, 3, 4
 ALGO_NAMES = {ALGO_GENERIC: "generic", ALGO_MFMA: "mfma", ALGO_DEPTHWISE: "depthwise"}
 
 # every symbol that include/d2conv.h declares
@@ -22,7 +22,7 @@ EXPORTS = (
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
-    "d2c_set_algo_override", "d2c_last_error", "d2c_version",
+    "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_last_error", "d2c_version",
     "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read",
 )
 
@@ -78,6 +78,7 @@ def load():
     lib.d2c_conv1d_algo.argtypes, lib.d2c_conv1d_algo.restype = [p1], ctypes.c_int
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int
+    lib.d2c_set_grad_input_mode.argtypes, lib.d2c_set_grad_input_mode.restype = [ctypes.c_int], None
     lib.d2c_profile_enable.argtypes, lib.d2c_profile_enable.restype = [ctypes.c_int], None
     lib.d2c_profile_reset.argtypes, lib.d2c_profile_reset.restype = [], None
     lib.d2c_profile_read.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]

@@ -12,6 +12,7 @@ namespace {
 thread_local char g_err[512] = "";
 std::atomic<uint64_t> g_max_intermediate{1ull << 32};  // dconv3d_gpu.cu:12
 std::atomic<int> g_algo_override{D2C_ALGO_AUTO};
+std::atomic<int> g_gx_mode{1};
 
 struct ProfState {
     std::mutex mu;
@@ -28,6 +29,8 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n)
         p[i] = 0u;
 }
 }  // namespace
+
+int d2c_gx_mode() { return g_gx_mode.load(); }
 
 void d2c_set_error(const char *fmt, ...)
 {
@@ -96,6 +99,7 @@ int d2c_version(void) { return 1; }
 uint64_t d2c_get_max_intermediate_elements(void) { return g_max_intermediate.load(); }
 void d2c_set_max_intermediate_elements(uint64_t m) { g_max_intermediate.store(m); }
 void d2c_set_algo_override(int algo) { g_algo_override.store(algo); }
+void d2c_set_grad_input_mode(int mode) { g_gx_mode.store(mode ? 1 : 0); }
 
 void d2c_profile_enable(int on)
 {

@@ -1,0 +1,231 @@
+// grad_input without atomics: inverse sample lists + owner-computes gather.
+//
+// The reference scatters every sampled value into grad_input with atomicAdd
+// (deformable_col2im_gpu_kernel, dconv3d_gpu.cu:562-643).  On this part fp32
+// atomics retire at about one element per clock and L2 channel, which makes
+// that scatter the slowest piece of the backward pass.  Here the scatter is
+// turned around:
+//
+//   1. every live sample (b, g, k, p) is filed under its base voxel
+//      floor(z, y, x) (counting sort: count, scan, fill), with its tap, its
+//      three fractions and its modulation;
+//   2. the grad-column values gcol[p, (k, chunk), c] are written once by the
+//      data kernel (in the element type of the call);
+//   3. one 8-lane group per (voxel, channel chunk) walks the lists of the 8 base
+//      voxels that can reach it, recomputes the corner weight, reads the gcol
+//      row segment and accumulates in registers; every grad_input element is
+//      written exactly once.
+#include "d2c_mma.hpp"
+#include "d2c_tiled.hpp"
+
+namespace {
+
+struct alignas(16) InvEntry {
+    int p, k;              // output position inside the sample, tap
+    float hz, hy, hx;      // fractions z - floor(z), ...
+    float alpha;           // modulation
+    int pad0, pad1;
+};
+static_assert(sizeof(InvEntry) == 32, "two 16-byte loads per entry");
+
+D2C_DEV int bin_of(const TiledShape &s, int b, int g, int z0, int y0, int x0)
+{
+    return (((b * s.G + g) * (s.D + 1) + (z0 + 1)) * (s.H + 1) + (y0 + 1)) * (s.W + 1) + (x0 + 1);
+}
+
+template <bool FILL>
+__global__ void __launch_bounds__(256)
+invlist_pass_kernel(TiledShape s, const void *off, const void *mask, int *counts, const int *starts, InvEntry *entries)
+{
+    const long total = (long)s.N * s.G * s.K * s.P;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int p = (int)(i % s.P);
+        const int k = (int)((i / s.P) % s.K);
+        const int g = (int)((i / ((long)s.P * s.K)) % s.G);
+        const int b = (int)(i / ((long)s.P * s.K * s.G));
+        const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
+        float o0, o1, o2;
+        load_offsets(s, off, b, g, k, p, o0, o1, o2);
+        int bz, by, bx;
+        tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
+        const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+        if (!t.live) continue;
+        const int bin = bin_of(s, b, g, t.z0, t.y0, t.x0);
+        const int n = atomicAdd(&counts[bin], 1);
+        if (FILL) {
+            InvEntry e;
+            e.p = p; e.k = k; e.hz = t.hz; e.hy = t.hy; e.hx = t.hx;
+            e.alpha = mask ? ld_aux(mask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt) : 1.f;
+            e.pad0 = 0; e.pad1 = 0;
+            entries[starts[bin] + n] = e;
+        }
+    }
+}
+
+// exclusive prefix sum of `n` ints in three launches (1024 elements per block)
+constexpr int kScanBlock = 1024;
+__global__ void __launch_bounds__(256) scan_block_sums(const int *in, int *bsum, int n)
+{
+    __shared__ int part[4];
+    const int base = blockIdx.x * kScanBlock;
+    int acc = 0;
+    for (int i = threadIdx.x; i < kScanBlock; i += 256) acc += (base + i < n) ? in[base + i] : 0;
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) bsum[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
+}
+__global__ void __launch_bounds__(256) scan_of_sums(int *bsum, int nb)
+{
+    // one workgroup, sequential over chunks of 256 block sums
+    __shared__ int buf[256];
+    __shared__ int carry;
+    if (threadIdx.x == 0) carry = 0;
+    __syncthreads();
+    for (int base = 0; base < nb; base += 256) {
+        const int i = base + threadIdx.x;
+        const int v = i < nb ? bsum[i] : 0;
+        buf[threadIdx.x] = v;
+        __syncthreads();
+        for (int d = 1; d < 256; d <<= 1) {   // Hillis-Steele inclusive scan
+            const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+            __syncthreads();
+            buf[threadIdx.x] += t;
+            __syncthreads();
+        }
+        if (i < nb) bsum[i] = carry + buf[threadIdx.x] - v;
+        __syncthreads();
+        if (threadIdx.x == 255) carry += buf[255];
+        __syncthreads();
+    }
+}
+__global__ void __launch_bounds__(256) scan_apply(const int *in, const int *bsum, int *out, int n)
+{
+    // sequential-per-thread scan of 4 elements, then a block scan of the 256 partial sums
+    __shared__ int buf[256];
+    const int base = blockIdx.x * kScanBlock + threadIdx.x * 4;
+    int v[4], s = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) { v[j] = (base + j < n) ? in[base + j] : 0; s += v[j]; }
+    buf[threadIdx.x] = s;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+        const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+        __syncthreads();
+        buf[threadIdx.x] += t;
+        __syncthreads();
+    }
+    int run = bsum[blockIdx.x] + buf[threadIdx.x] - s;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if (base + j < n) out[base + j] = run;
+        run += v[j];
+    }
+}
+__global__ void set_total(const int *counts, int *starts, int n)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) starts[n] = n > 0 ? starts[n - 1] + counts[n - 1] : 0;
+}
+
+// ---- owner-computes accumulation ------------------------------------------
+// gcol layout: [chunk][tap][m = b*P + p][BKC] of T.  One 8-lane group per (voxel, chunk).
+template <typename T>
+__global__ void __launch_bounds__(256)
+gx_owner_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *entries, float *gxcl)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
+    const int sub = threadIdx.x & 7;
+    const long vg = (long)blockIdx.x * 32 + (threadIdx.x >> 3);   // voxel index over the batch
+    const int cidx = blockIdx.y;                                  // channel chunk
+    if (vg >= (long)s.N * s.vol) return;
+    const int b = (int)(vg / s.vol), v = (int)(vg - (long)b * s.vol);
+    const int x = v % s.W, y = (v / s.W) % s.H, z = v / (s.W * s.H);
+    const int g = (cidx * BKC) / s.cpg;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++) acc[i] = 0.f;
+    const T *gbase = gcol + ((long)cidx * s.K * s.M + (long)b * s.P) * BKC + sub * VEC;
+#pragma unroll 1
+    for (int d = 0; d < 8; d++) {
+        const int dz = (d >> 2) & 1, dy = (d >> 1) & 1, dx = d & 1;
+        const int bin = bin_of(s, b, g, z - dz, y - dy, x - dx);
+        const int e0 = starts[bin], e1 = starts[bin + 1];
+        for (int e = e0; e < e1; e++) {
+            const uint4 q0 = reinterpret_cast<const uint4 *>(entries + e)[0];
+            const uint4 q1 = reinterpret_cast<const uint4 *>(entries + e)[1];
+            const int p = (int)q0.x, k = (int)q0.y;
+            const float hz = __uint_as_float(q0.z), hy = __uint_as_float(q0.w), hx = __uint_as_float(q1.x);
+            const float al = __uint_as_float(q1.y);
+            const float w = (dz ? hz : 1.f - hz) * (dy ? hy : 1.f - hy) * (dx ? hx : 1.f - hx) * al;
+            const uint4 row = *reinterpret_cast<const uint4 *>(gbase + ((long)k * s.M + p) * BKC);
+            const T *re = reinterpret_cast<const T *>(&row);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) acc[i] = fmaf(w, elem_to_f32<T>(re[i]), acc[i]);
+        }
+    }
+    float *o = gxcl + vg * s.Cin + cidx * BKC + sub * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; i += 4) *reinterpret_cast<float4 *>(o + i) = make_float4(acc[i], acc[i + 1], acc[i + 2], acc[i + 3]);
+}
+
+inline unsigned g1d(long n, int cap = 16384)
+{
+    long g = (n + 255) / 256;
+    return (unsigned)(g < 1 ? 1 : (g > cap ? cap : g));
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ host
+long d2c_invlist_bins(const TiledShape &s) { return (long)s.N * s.G * (s.D + 1) * (s.H + 1) * (s.W + 1); }
+
+// workspace pieces (bytes), in this order: counts | starts | block sums | entries
+void d2c_invlist_ws(const TiledShape &s, size_t *counts, size_t *starts, size_t *bsums, size_t *entries)
+{
+    const long nb = d2c_invlist_bins(s);
+    *counts = d2c_align_up((size_t)(nb + 1) * 4);
+    *starts = d2c_align_up((size_t)(nb + 1) * 4);
+    *bsums = d2c_align_up((size_t)((nb + kScanBlock - 1) / kScanBlock + 1) * 4);
+    *entries = d2c_align_up((size_t)s.N * s.G * s.K * s.P * sizeof(InvEntry));
+}
+
+int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, int *counts, int *starts, int *bsums,
+                      void *entries, hipStream_t st)
+{
+    D2cProfScope prof(D2C_PROF_PACK, st);
+    const long nbl = d2c_invlist_bins(s);
+    if (nbl >= (1L << 31) - kScanBlock) {
+        d2c_set_error("too many sample bins");
+        return D2C_ERR_UNSUPPORTED;
+    }
+    const int nb = (int)nbl;
+    const long total = (long)s.N * s.G * s.K * s.P;
+    d2c_fill_zero(counts, (size_t)(nb + 1) * 4, st);
+    hipLaunchKernelGGL(invlist_pass_kernel<false>, dim3(g1d(total)), dim3(256), 0, st, s, off, mask, counts,
+                       (const int *)nullptr, (InvEntry *)nullptr);
+    const int nblk = (nb + kScanBlock - 1) / kScanBlock;
+    hipLaunchKernelGGL(scan_block_sums, dim3(nblk), dim3(256), 0, st, counts, bsums, nb);
+    hipLaunchKernelGGL(scan_of_sums, dim3(1), dim3(256), 0, st, bsums, nblk);
+    hipLaunchKernelGGL(scan_apply, dim3(nblk), dim3(256), 0, st, counts, bsums, starts, nb);
+    hipLaunchKernelGGL(set_total, dim3(1), dim3(64), 0, st, counts, starts, nb);
+    d2c_fill_zero(counts, (size_t)(nb + 1) * 4, st);   // reused as the per-bin cursor of the fill pass
+    hipLaunchKernelGGL(invlist_pass_kernel<true>, dim3(g1d(total)), dim3(256), 0, st, s, off, mask, counts, starts,
+                       (InvEntry *)entries);
+    return d2c_check_launch("invlist_build");
+}
+
+template <typename T>
+int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts, const void *entries, float *gxcl,
+                        hipStream_t st)
+{
+    constexpr int BKC = 8 * Elem<T>::VEC;
+    D2cProfScope prof(D2C_PROF_GX_OWNER, st);
+    const long nv = (long)s.N * s.vol;
+    dim3 grid((unsigned)((nv + 31) / 32), s.Cin / BKC);
+    hipLaunchKernelGGL(gx_owner_kernel<T>, grid, dim3(256), 0, st, s, (const T *)gcol, starts,
+                       (const InvEntry *)entries, gxcl);
+    return d2c_check_launch("gx_owner_kernel");
+}
+template int d2c_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const int *, const void *, float *, hipStream_t);
+template int d2c_gx_owner_launch<float>(const TiledShape &, const void *, const int *, const void *, float *, hipStream_t);

@@ -13,10 +13,18 @@ bool d2c_tiled_bwd_data_supported(const TiledShape &s, int dtype);
 bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype);
 int d2c_bwd_ogk(int og, int dtype);
 int d2c_bwd_pass_channels(int dtype);
+bool d2c_tiled_bwd_single_pass(const TiledShape &s, int dtype);
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                              const void *mask, const void *w, void *wt, float *gxcl, void *goff, void *gmask,
-                              hipStream_t st);
+                              const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
+                              void *gmask, hipStream_t st);
+void d2c_invlist_ws(const TiledShape &s, size_t *counts, size_t *starts, size_t *bsums, size_t *entries);
+int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, int *counts, int *starts, int *bsums,
+                      void *entries, hipStream_t st);
+template <typename T>
+int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts, const void *entries, float *gxcl,
+                        hipStream_t st);
+int d2c_gx_mode();
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                                 const void *mask, float *gwacc, void *gw, hipStream_t st);
@@ -183,8 +191,15 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
     return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, st);
 }
 
+// grad_input by sample lists (see d2c_invlist.hip) needs the whole reduction over output
+// channels in one pass of the data kernel.
+bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    return d2c_gx_mode() == 1 && d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
+}
+
 struct BwdWs {
-    size_t xcl, wt, gxcl, gwacc, total;
+    size_t xcl, wt, gxcl, gwacc, gcol, counts, starts, bsums, entries, total;
 };
 BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -197,6 +212,17 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.gxcl = w.wt + d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * ogk * es);
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
     w.total = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
+    w.gcol = w.counts = w.starts = w.bsums = w.entries = 0;
+    if (use_lists(q, s)) {
+        size_t c, st, bs, en;
+        d2c_invlist_ws(s, &c, &st, &bs, &en);
+        w.gcol = w.total;
+        w.counts = w.gcol + d2c_align_up((size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M * bkc_of(q.dtype) * es);
+        w.starts = w.counts + c;
+        w.bsums = w.starts + st;
+        w.entries = w.bsums + bs;
+        w.total = w.entries + en;
+    }
     return w;
 }
 
@@ -228,9 +254,19 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
     if (gx || goff || gmask) {
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
-            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt, gxcl, goff,
+            const bool lists = gx && use_lists(q, s);
+            if (lists)
+                if (int rc = d2c_invlist_build(s, off, mask, (int *)(base + l.counts), (int *)(base + l.starts),
+                                               (int *)(base + l.bsums), base + l.entries, st))
+                    return rc;
+            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt,
+                                                     lists ? nullptr : gxcl, lists ? base + l.gcol : nullptr, goff,
                                                      gmask, st))
                 return rc;
+            if (lists)
+                if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, (const int *)(base + l.starts), base + l.entries,
+                                                    gxcl, st))
+                    return rc;
             if (gx)
                 if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
         } else {

@@ -37,7 +37,8 @@ struct BwdDataArgs {
     const void *xcl;    // [N][vol][Cin]
     const void *off, *mask;
     const void *wt;     // [groups][K*nchunk][BKC][ogk]   (W transposed per step, zero padded to ogk)
-    float *gxcl;        // [N][vol][Cin] fp32 accumulator (zeroed) or NULL
+    float *gxcl;        // [N][vol][Cin] fp32 accumulator (zeroed) for the atomic scatter, or NULL
+    void *gcolbuf;      // [chunk][tap][N*P][BKC] grad-column values for the list-based grad_input, or NULL
     void *goff, *gmask; // or NULL
     int ogk;            // output channels of this pass rounded up to a whole k-group
     int o0, ogn;        // this pass reduces over output channels [o0, o0 + ogn) of each weight group
@@ -220,7 +221,28 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
         }
         __syncthreads();
 
-        // (d) dot products with the corner vectors, offset / mask gradient
+        // (d) grad-column rows out to memory (list-based grad_input)
+        if (a.gcolbuf) {
+            T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
+#pragma unroll
+            for (int i = 0; i < ITEMS; i++) {
+                const int item = tid + i * kThreads;
+                const int pos = item / NV, vec = item % NV;
+                const int m = m0 + pos;
+                if (m < s.M) {
+                    const float *gp = reinterpret_cast<const float *>(s_gcol + pos * GRS + vec * VEC * 4);
+                    uint4 o;
+                    if constexpr (sizeof(T) == 2) {
+                        o = make_uint4(pack_bf16x2(gp[0], gp[1]), pack_bf16x2(gp[2], gp[3]), pack_bf16x2(gp[4], gp[5]),
+                                       pack_bf16x2(gp[6], gp[7]));
+                    } else {
+                        o = *reinterpret_cast<const uint4 *>(gp);
+                    }
+                    *reinterpret_cast<uint4 *>(gb + (long)m * BKC + vec * VEC) = o;
+                }
+            }
+        }
+        // (e) dot products with the corner vectors, offset / mask gradient
         if (want_aux) {
 #pragma unroll
             for (int i = 0; i < ITEMS; i++) {
@@ -587,10 +609,13 @@ bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype)
     return s.P % (dtype == D2C_BF16 ? 8 : 4) == 0;
 }
 
+// One pass reduces over all output channels of a weight group (the list-based grad_input needs that).
+bool d2c_tiled_bwd_single_pass(const TiledShape &s, int dtype) { return s.og <= d2c_bwd_pass_channels(dtype); }
+
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                              const void *mask, const void *w, void *wt, float *gxcl, void *goff, void *gmask,
-                              hipStream_t st)
+                              const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
+                              void *gmask, hipStream_t st)
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
     const int omax = d2c_bwd_pass_channels(Elem<T>::DT);
@@ -610,7 +635,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                                s, ogk, o0, ogn, total);
         }
         if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
-        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0};
+        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
         if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, st);
@@ -667,7 +692,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
 
 #define INST(T)                                                                                                    \
     template int d2c_tiled_bwd_data_launch<T>(const TiledShape &, const void *, const void *, const void *,        \
-                                              const void *, const void *, void *, float *, void *, void *,        \
+                                              const void *, const void *, void *, float *, void *, void *, void *, \
                                               hipStream_t);                                                        \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
                                                 const void *, float *, void *, hipStream_t);                      \

@@ -146,12 +146,18 @@ enum {
     D2C_PROF_FWD = 0,         /* forward implicit-GEMM / depthwise kernel */
     D2C_PROF_BWD_DATA = 1,    /* grad_input + grad_offset + grad_mask kernel */
     D2C_PROF_BWD_WEIGHT = 2,  /* grad_weight kernel */
-    D2C_PROF_PACK = 3,        /* layout changes, clears, conversions (sum) */
-    D2C_PROF_COUNT = 4
+    D2C_PROF_PACK = 3,        /* layout changes, clears, conversions, sample lists (sum) */
+    D2C_PROF_GX_OWNER = 4,    /* grad_input accumulation from the sample lists */
+    D2C_PROF_COUNT = 5
 };
 void d2c_profile_enable(int on);
 void d2c_profile_reset(void);
 int d2c_profile_read(int id, double *total_ms, int *launches);
+
+/* Test hook for the matrix-core backward pass: 1 (default) builds grad_input from
+ * per-voxel sample lists, every element written once; 0 scatters with fp32 atomics
+ * like the reference (dconv3d_gpu.cu:637).  Workspace sizes depend on the mode. */
+void d2c_set_grad_input_mode(int mode);
 
 const char *d2c_last_error(void);
 int d2c_version(void);
