@@ -352,7 +352,8 @@ int launch_bwd_data(const BwdDataArgs &a, hipStream_t st)
 struct BwdWeightArgs {
     TiledShape s;
     const void *gout, *xcl, *off, *mask;
-    float *gwacc;   // [Cout][cg][K] fp32 accumulator (zeroed)
+    float *gwacc;   // [group][chunk*K + tap][og][BKC] fp32 accumulator (zeroed): channel-contiguous rows, so that
+                    // the atomics of a wavefront fill whole cache lines
     int split;      // position tiles are dealt round-robin to `split` workgroups per step
 };
 
@@ -373,10 +374,11 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
     constexpr int ITEMS = NITEM / kThreads;
     static_assert(ITEMS * kThreads == NITEM, "gather items divide evenly");
 
-    __shared__ __align__(16) unsigned char s_tile[BKC * TRS];
-    __shared__ float s_w[8][kWMT];
-    __shared__ int s_idx[kWMT];
-    __shared__ int s_flag[kWMT];
+    __shared__ __align__(16) unsigned char s_tile[2][BKC * TRS];
+    __shared__ __align__(16) unsigned char s_stage[8 * 64 * (128 + 16)];   // per-wavefront patch of the gout operand
+    __shared__ float s_w[2][8][kWMT];
+    __shared__ int s_idx[2][kWMT];
+    __shared__ int s_flag[2][kWMT];
 
     const TiledShape &s = a.s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -388,6 +390,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
     const int g = c0 / s.cpg;
     const int HW = s.H * s.W;
     const int ntile = (s.M + kWMT - 1) / kWMT;
+    const int nmy = ntile > sp ? (ntile - sp + a.split - 1) / a.split : 0;   // tiles of this workgroup
     const int o_base = otile * NT + wave * 64;   // first output channel (in the weight group) of this wavefront
     const bool mma_wave = o_base < s.og;
 
@@ -399,14 +402,13 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[ob][cb][r] = 0.f;
 
-    for (int tile = sp; tile < ntile; tile += a.split) {
-        const int m0 = tile * kWMT;
-        // corner weights of the tile's positions for this tap
+    // corner weights of tile i's positions for this tap
+    auto coords = [&](int i, int buf) {
         if (tid < kWMT) {
             float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             int idx = 0;
             unsigned live = 0;
-            const int m = m0 + tid;
+            const int m = (sp + i * a.split) * kWMT + tid;
             if (m < s.M) {
                 const int b = m / s.P, p = m - b * s.P;
                 const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
@@ -422,36 +424,47 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
                 for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
             }
 #pragma unroll
-            for (int c = 0; c < 8; c++) s_w[c][tid] = w[c];
-            s_idx[tid] = idx;
-            s_flag[tid] = (int)live;
+            for (int c = 0; c < 8; c++) s_w[buf][c][tid] = w[c];
+            s_idx[buf][tid] = idx;
+            s_flag[buf][tid] = (int)live;
         }
-        __syncthreads();
+    };
 
-        // sample: one item = CPI channels x VEC consecutive positions; 32 lanes read one 128-byte row
+    // sample: one item = CPI channels x VEC consecutive positions; 32 lanes read one 128-byte row
+    uint32_t u[ITEMS][VEC][8];
+    auto gather_issue = [&](int buf) {
 #pragma unroll
         for (int it = 0; it < ITEMS; it++) {
             const int item = tid + it * kThreads;
             const int cpi = item % (BKC / CPI), oct = item / (BKC / CPI);
             const T *xb = reinterpret_cast<const T *>(a.xcl) + c0 + cpi * CPI;
+#pragma unroll
+            for (int q = 0; q < VEC; q++) {
+                const int pos = oct * VEC + q;
+                const int idx = s_idx[buf][pos];
+                const unsigned live = (unsigned)s_flag[buf][pos];
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
+                    u[it][q][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint32_t *>(xb + (long)v * s.Cin) : 0u;
+                }
+            }
+        }
+    };
+    auto interp_store = [&](int cbuf, int tbuf) {
+#pragma unroll
+        for (int it = 0; it < ITEMS; it++) {
+            const int item = tid + it * kThreads;
+            const int cpi = item % (BKC / CPI), oct = item / (BKC / CPI);
             float r0[VEC], r1[VEC];
 #pragma unroll
             for (int q = 0; q < VEC; q++) {
                 const int pos = oct * VEC + q;
-                const int idx = s_idx[pos];
-                const unsigned live = (unsigned)s_flag[pos];
                 float v0 = 0.f, v1 = 0.f;
-                uint32_t u[8];
-                // all eight (predicated) loads are issued before any of them is used
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
-                    const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
-                    u[c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint32_t *>(xb + (long)v * s.Cin) : 0u;
-                }
-#pragma unroll
-                for (int c = 0; c < 8; c++) {
-                    const float wc = s_w[c][pos];
-                    const uint32_t uc = u[c];
+                    const float wc = s_w[cbuf][c][pos];
+                    const uint32_t uc = u[it][q][c];
                     if constexpr (sizeof(T) == 2) {
                         v0 = fmaf(wc, __uint_as_float(uc << 16), v0);
                         v1 = fmaf(wc, __uint_as_float(uc & 0xffff0000u), v1);
@@ -466,42 +479,89 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
                                       pack_bf16x2(r0[4], r0[5]), pack_bf16x2(r0[6], r0[7]));
                 uint4 p1 = make_uint4(pack_bf16x2(r1[0], r1[1]), pack_bf16x2(r1[2], r1[3]),
                                       pack_bf16x2(r1[4], r1[5]), pack_bf16x2(r1[6], r1[7]));
-                *reinterpret_cast<uint4 *>(&s_tile[(cpi * 2) * TRS + oct * 16]) = p0;
-                *reinterpret_cast<uint4 *>(&s_tile[(cpi * 2 + 1) * TRS + oct * 16]) = p1;
+                *reinterpret_cast<uint4 *>(&s_tile[tbuf][(cpi * 2) * TRS + oct * 16]) = p0;
+                *reinterpret_cast<uint4 *>(&s_tile[tbuf][(cpi * 2 + 1) * TRS + oct * 16]) = p1;
             } else {
-                *reinterpret_cast<uint4 *>(&s_tile[cpi * TRS + oct * 16]) =
+                *reinterpret_cast<uint4 *>(&s_tile[tbuf][cpi * TRS + oct * 16]) =
                     make_uint4(__float_as_uint(r0[0]), __float_as_uint(r0[1]), __float_as_uint(r0[2]),
                                __float_as_uint(r0[3]));
             }
         }
-        __syncthreads();
+    };
 
-        // gW block += gout[o, pos] * tile[pos, c]
-        if (mma_wave) {
-            const T *gp = reinterpret_cast<const T *>(a.gout);
-#pragma unroll 2
-            for (int kg = 0; kg < kWMT / (2 * VEC); kg++) {
-                const int mv = m0 + (kg * 2 + (lane >> 5)) * VEC;   // first of VEC consecutive positions
-                uint4 af[OB], bf[CB];
-                const bool ok = mv < s.M;
-                const int b = ok ? mv / s.P : 0, p = ok ? mv - b * s.P : 0;
+    // gW block += gout[o, pos] * tile[pos, c].  The gout operand wants 8 (4) consecutive positions of one
+    // output channel per lane; read that way from memory every lane would touch its own cache line.  Each
+    // wavefront therefore pulls its 64 rows in 128-byte segments with coalesced loads (8 lanes per row),
+    // parks them in a private LDS patch and reads the operand vectors from there.
+    constexpr int SP = 128 / (int)sizeof(T);     // positions per stage = one 128-byte row segment
+    constexpr int NSTG = kWMT / SP;
+    constexpr int SRS = 128 + 16;                // patch row stride (bytes)
+    const T *gp = reinterpret_cast<const T *>(a.gout);
+    unsigned char *stg = s_stage + wave * (64 * SRS);
+    auto mma_tile = [&](int i, int tbuf) {
+        if (!mma_wave) return;
+        const int m0 = (sp + i * a.split) * kWMT;
+        const int b0 = m0 / s.P;
+        uint4 ld[8];
+        auto issue = [&](int sg) {
 #pragma unroll
-                for (int ob = 0; ob < OB; ob++) {
-                    const int ol = o_base + ob * 32 + (lane & 31);
-                    af[ob] = (ok && ol < s.og)
-                                 ? *reinterpret_cast<const uint4 *>(gp + ((long)b * s.Cout + wg * s.og + ol) * s.P + p)
-                                 : make_uint4(0, 0, 0, 0);
-                }
+            for (int q = 0; q < 8; q++) {
+                const int piece = q * 64 + lane, row = piece >> 3, c16 = piece & 7;
+                const int ol = o_base + row;
+                const int mv = m0 + sg * SP + c16 * VEC;
+                int b = b0, pp = mv - b0 * s.P;
+                if (pp >= s.P) { pp -= s.P; b += 1; }
+                ld[q] = (mv < s.M && ol < s.og)
+                            ? *reinterpret_cast<const uint4 *>(gp + ((long)b * s.Cout + wg * s.og + ol) * s.P + pp)
+                            : make_uint4(0, 0, 0, 0);
+            }
+        };
+        issue(0);
+#pragma unroll
+        for (int sg = 0; sg < NSTG; sg++) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // operand reads of the previous stage are done
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const int piece = q * 64 + lane, row = piece >> 3, c16 = piece & 7;
+                *reinterpret_cast<uint4 *>(stg + row * SRS + c16 * 16) = ld[q];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            if (sg + 1 < NSTG) issue(sg + 1);
+#pragma unroll
+            for (int kq = 0; kq < 4; kq++) {
+                const int kg = sg * 4 + kq;
+                uint4 af[OB], bf[CB];
+#pragma unroll
+                for (int ob = 0; ob < OB; ob++)
+                    af[ob] = *reinterpret_cast<const uint4 *>(stg + (ob * 32 + (lane & 31)) * SRS + (kq * 2 + (lane >> 5)) * 16);
 #pragma unroll
                 for (int cb = 0; cb < CB; cb++)
-                    bf[cb] = *reinterpret_cast<const uint4 *>(&s_tile[(cb * 32 + (lane & 31)) * TRS + (kg * 2 + (lane >> 5)) * 16]);
+                    bf[cb] = *reinterpret_cast<const uint4 *>(&s_tile[tbuf][(cb * 32 + (lane & 31)) * TRS + (kg * 2 + (lane >> 5)) * 16]);
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++)
 #pragma unroll
                     for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], af[ob], bf[cb]);
             }
         }
+    };
+
+    // software pipeline over this workgroup's tiles: while the matrix cores take tile i, the corner
+    // rows of tile i+1 are in flight and the corner weights of tile i+2 are computed
+    if (nmy > 0) {
+        coords(0, 0);
         __syncthreads();
+        gather_issue(0);
+        if (nmy > 1) coords(1, 1);
+        interp_store(0, 0);
+        __syncthreads();
+        for (int i = 0; i < nmy; i++) {
+            if (i + 1 < nmy) gather_issue((i + 1) & 1);
+            if (i + 2 < nmy) coords(i + 2, i & 1);
+            mma_tile(i, i & 1);
+            if (i + 1 < nmy) interp_store((i + 1) & 1, (i + 1) & 1);
+            __syncthreads();
+        }
     }
 
     if (mma_wave) {
@@ -512,9 +572,9 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int ol = o_base + ob * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    const int cl = j * BKC + cb * 32 + (lane & 31);
                     if (ol < s.og)
-                        atomicAdd(a.gwacc + ((long)(wg * s.og + ol) * s.cg + cl) * s.K + k, acc[ob][cb][r]);
+                        atomicAdd(a.gwacc + (((long)wg * s.nchunk * s.K + st) * s.og + ol) * BKC + cb * 32 + (lane & 31),
+                                  acc[ob][cb][r]);
                 }
     }
 }
@@ -559,11 +619,18 @@ __global__ void __launch_bounds__(256) unpack_grad_input_kernel(const float *gxc
     }
 }
 
+// fp32 accumulator [group][chunk*K + tap][og][BKC] -> grad_weight [Cout][cg][K] of type T
 template <typename T>
-__global__ void __launch_bounds__(256) cvt_grad_weight_kernel(const float *src, T *dst, long n)
+__global__ void __launch_bounds__(256) cvt_grad_weight_kernel(const float *src, T *dst, TiledShape s, long n)
 {
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
-        dst[i] = f32_to_elem<T>(src[i]);
+    constexpr int BKC = 8 * Elem<T>::VEC;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const int k = (int)(i % s.K);
+        const int cl = (int)((i / s.K) % s.cg);
+        const int o = (int)(i / ((long)s.K * s.cg));
+        const int wg = o / s.og, ol = o - wg * s.og, j = cl / BKC, cc = cl - j * BKC;
+        dst[i] = f32_to_elem<T>(src[(((long)wg * s.nchunk * s.K + j * s.K + k) * s.og + ol) * BKC + cc]);
+    }
 }
 
 // gb[o] = sum_{b,p} gout[b,o,p]   (dconv3d_gpu.cu:1329)
@@ -669,7 +736,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     }
     if (int rc = d2c_check_launch("tiled_bwd_weight_kernel")) return rc;
     D2cProfScope prof(D2C_PROF_PACK, st);
-    hipLaunchKernelGGL(cvt_grad_weight_kernel<T>, dim3(grid1d(nw)), dim3(256), 0, st, gwacc, (T *)gw, nw);
+    hipLaunchKernelGGL(cvt_grad_weight_kernel<T>, dim3(grid1d(nw)), dim3(256), 0, st, gwacc, (T *)gw, s, nw);
     return d2c_check_launch("cvt_grad_weight_kernel");
 }
 
