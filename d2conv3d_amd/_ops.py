@@ -287,3 +287,9 @@ def set_algo_override(name):
     code = {None: _lib.ALGO_AUTO, "auto": _lib.ALGO_AUTO, "generic": _lib.ALGO_GENERIC,
             "mfma": _lib.ALGO_MFMA, "depthwise": _lib.ALGO_DEPTHWISE}[name]
     _lib.load().d2c_set_algo_override(code)
+
+
+def set_grad_input_mode(mode):
+    """Test hook: "lists" (default; grad_input gathered from per-voxel sample lists, every element
+    written once) or "atomics" (scatter with fp32 atomics like the reference)."""
+    _lib.load().d2c_set_grad_input_mode({"lists": 1, "atomics": 0}[mode])

@@ -296,6 +296,8 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
 static bool mfma_channels_ok(const d2c_conv3d_desc &q)
 {
     if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
+    // the tiled kernels address the channels-last input with 32-bit byte offsets
+    if ((size_t)q.N * q.Cin * q.D * q.H * q.W * d2c_elem_size(q.dtype) >= (1ull << 32)) return false;
     const int bkc = bkc_of(q.dtype);
     const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
     return cg % bkc == 0 && cpg % bkc == 0;
@@ -342,9 +344,7 @@ bool d2c_tiled_supported(const d2c_conv3d_desc &q)
 {
     if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
     if (is_depthwise(q)) return true;
-    const int bkc = bkc_of(q.dtype);
-    const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
-    return cg % bkc == 0 && cpg % bkc == 0;
+    return mfma_channels_ok(q);
 }
 
 int d2c_tiled_algo(const d2c_conv3d_desc &q) { return is_depthwise(q) ? D2C_ALGO_DEPTHWISE : D2C_ALGO_MFMA; }

@@ -73,7 +73,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
     const int wg = blockIdx.y;
     const int m0 = tile * MT;
     const int S = s.nchunk * s.K;
-    const int HW = s.H * s.W;
+    const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;   // element strides of a step in z / y
     const int cb = wave % CB, pb = wave / CB;
     const int nkg = a.ogk / (2 * VEC);
 
@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
-                idx = cbatch * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0;
+                idx = (cbatch * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
                 unsigned inr = t.inrange, auxlive = t.live;
                 fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
                 if (s.nd == 1) {
@@ -212,8 +212,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 #pragma unroll
                     for (int c = 0; c < 8; c++) {
                         if ((live >> c) & 1u) {
-                            const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
-                            atomicAdd(gbase + (long)v * s.Cin, s_w[c * MT + pl] * gv);
+                            const unsigned o = (unsigned)(idx + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc + (c & 1) * s.Cin);
+                            atomicAdd(gbase + o, s_w[c * MT + pl] * gv);
                         }
                     }
                 }
@@ -261,15 +261,16 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                         gc[4 * e] = t4.x; gc[4 * e + 1] = t4.y; gc[4 * e + 2] = t4.z; gc[4 * e + 3] = t4.w;
                     }
                 }
-                const T *xb = reinterpret_cast<const T *>(a.xcl) + c0 + vec * VEC;
+                const char *xb = reinterpret_cast<const char *>(a.xcl);
+                const int ib = idx + c0 + vec * VEC;
                 float dot[8];
                 uint4 xv[8];
-                // all eight (predicated) loads are issued before any of them is used
+                // all eight (predicated) loads are issued before any of them is used; 32-bit byte offsets
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
-                    const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + ((c & 1) ? 1 : -qshift);
-                    xv[c] = ((inr >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + (long)v * s.Cin)
-                                              : make_uint4(0, 0, 0, 0);
+                    const unsigned o = (unsigned)(ib + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc
+                                                  + ((c & 1) ? s.Cin : -qshift * s.Cin)) * (unsigned)sizeof(T);
+                    xv[c] = ((inr >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + o) : make_uint4(0, 0, 0, 0);
                 }
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
@@ -388,7 +389,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
     const int j = st / s.K, k = st - j * s.K;
     const int c0 = wg * s.cg + j * BKC;
     const int g = c0 / s.cpg;
-    const int HW = s.H * s.W;
+    const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;   // element strides of a step in z / y
     const int ntile = (s.M + kWMT - 1) / kWMT;
     const int nmy = ntile > sp ? (ntile - sp + a.split - 1) / a.split : 0;   // tiles of this workgroup
     const int o_base = otile * NT + wave * 64;   // first output channel (in the weight group) of this wavefront
@@ -419,7 +420,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
                 tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
                 live = t.live;
-                idx = b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0;
+                idx = (b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
 #pragma unroll
                 for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
             }
@@ -437,16 +438,17 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
         for (int it = 0; it < ITEMS; it++) {
             const int item = tid + it * kThreads;
             const int cpi = item % (BKC / CPI), oct = item / (BKC / CPI);
-            const T *xb = reinterpret_cast<const T *>(a.xcl) + c0 + cpi * CPI;
+            const char *xb = reinterpret_cast<const char *>(a.xcl);
 #pragma unroll
             for (int q = 0; q < VEC; q++) {
                 const int pos = oct * VEC + q;
-                const int idx = s_idx[buf][pos];
+                const int idx = s_idx[buf][pos] + c0 + cpi * CPI;
                 const unsigned live = (unsigned)s_flag[buf][pos];
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
-                    const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
-                    u[it][q][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint32_t *>(xb + (long)v * s.Cin) : 0u;
+                    const unsigned o = (unsigned)(idx + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc + (c & 1) * s.Cin)
+                                       * (unsigned)sizeof(T);
+                    u[it][q][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint32_t *>(xb + o) : 0u;
                 }
             }
         }

@@ -65,7 +65,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
     const int otile = blockIdx.y, wg = blockIdx.z;
     const int m0 = tile * kMT;
     const int S = s.nchunk * s.K;
-    const int HW = s.H * s.W;
+    const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;   // element strides of a step in z / y
 
     // --- per-position constants of the coordinate threads
     int cb = 0, cp = 0, coz = 0, coy = 0, cox = 0;
@@ -95,7 +95,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
                 live = t.live;
-                idx = cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0;
+                idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
 #pragma unroll
                 for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
             }
@@ -115,14 +115,15 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
         for (int i = 0; i < ITEMS; i++) {
             const int item = tid + i * kThreads;
             const int pos = item / kNV, vec = item % kNV;
-            const int idx = s_idx[buf][pos];
+            const int idx = s_idx[buf][pos] + c0 + vec * VEC;
             const unsigned live = (unsigned)s_flag[buf][pos];
-            const T *base = reinterpret_cast<const T *>(a.xcl) + c0 + vec * VEC;
+            // 32-bit byte offsets from a uniform base: the whole input is below 4 GiB (checked on the host)
+            const char *base = reinterpret_cast<const char *>(a.xcl);
 #pragma unroll
             for (int c = 0; c < 8; c++) {
-                const int v = idx + ((c >> 2) & 1) * HW + ((c >> 1) & 1) * s.W + (c & 1);
-                gv[i][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint4 *>(base + (long)v * s.Cin)
-                                              : make_uint4(0, 0, 0, 0);
+                const unsigned o = (unsigned)(idx + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc + (c & 1) * s.Cin)
+                                   * (unsigned)sizeof(T);
+                gv[i][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint4 *>(base + o) : make_uint4(0, 0, 0, 0);
             }
         }
     };

@@ -86,6 +86,27 @@ def test_tiled_forward_backward(name, dtype, dev):
                 assert_close(t.grad, e, 2e-2, 2e-2 * e.abs().max().item(), n)
 
 
+@pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_grad_input_by_atomics_matches_lists(name, dtype, dev):
+    # the matrix-core backward has two ways to build grad_input; both must agree with the oracle
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, dtype, seed=7)
+    eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+    grads = {}
+    for mode in ("atomics", "lists"):
+        _ops.set_grad_input_mode(mode)
+        try:
+            ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+            d2c.deform_conv3d(*ts, s, p, d, groups, G).backward(gout.to(dev))
+            grads[mode] = ts[0].grad
+        finally:
+            _ops.set_grad_input_mode("lists")
+        if dtype == torch.float32:
+            assert_close(grads[mode], eg[0], 1e-4, 1e-5 * max(1.0, eg[0].abs().max().item()), f"grad_input ({mode})")
+        else:
+            assert rel_l2(grads[mode], eg[0]) < 2e-2, mode
+
+
 def test_tiled_matches_generic_family(dev):
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make("c128_G2_o96", torch.float32, seed=3)
     ts = [t.to(dev) if t is not None else None for t in (x, off, m, w, b)]
