@@ -100,6 +100,13 @@ template <typename T> D2C_DEV T f32_to_elem(float v);
 template <> D2C_DEV bf16_t f32_to_elem<bf16_t>(float v) { return f32_to_bf16(v); }
 template <> D2C_DEV float f32_to_elem<float>(float v) { return v; }
 
+// offset / mask element with the storage type fixed at compile time (no branch in hot loops)
+template <bool AUX16> D2C_DEV float ld_auxT(const void *p, long i)
+{
+    if constexpr (AUX16) return bf16_to_f32(reinterpret_cast<const bf16_t *>(p)[i]);
+    else return reinterpret_cast<const float *>(p)[i];
+}
+
 // offset / mask element (float32 or bfloat16 storage) as float
 D2C_DEV float ld_aux(const void *p, long i, int adt)
 {

@@ -10,18 +10,20 @@
 // weights, and drops the result into an LDS tile in MFMA operand order.  The
 // im2col column buffer of the reference (dconv3d_gpu.cu:297) never exists.
 //
-// One workgroup = 512 threads = 128 positions x NT output channels.  Steps are
-// software-pipelined: while the matrix cores work on step s, the corner loads
-// of step s+1 are in flight and the corner weights of step s+2 are computed.
+// One workgroup = 512 threads = MT positions x NT output channels.  Steps are
+// software-pipelined over three stages: while the matrix cores work on step s,
+// the corner rows of step s+1 and the weight fragments of step s+1 are in
+// flight and the offsets of step s+2 are being fetched; nothing waits on
+// memory inside a step except at its one barrier.
 #include "d2c_mma.hpp"
 #include "d2c_tiled.hpp"
 
 namespace {
 
-constexpr int kMT = 128;       // positions per workgroup
 constexpr int kNV = 8;         // 16-byte vectors per sampled row (one chunk)
 constexpr int kRS = kNV * 16 + 16;  // LDS row stride in bytes (padded: conflict-free 16-byte reads)
 constexpr int kThreads = 512;
+constexpr int kMT = 128;       // positions per workgroup
 
 struct FwdArgs {
     TiledShape s;
@@ -41,36 +43,37 @@ D2C_DEV int xcd_swizzle(int bid, int n)
     return x * q + (x < r ? x : r) + idx;
 }
 
-template <typename T, int WAVES_O, int WAVES_P>
+template <typename T, bool AUX16, int MT, int WAVES_O, int WAVES_P>
 __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
 {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int BKC = kNV * VEC;
-    constexpr int WPOS = kMT / WAVES_P;   // positions per MMA wave
+    constexpr int WPOS = MT / WAVES_P;    // positions per MMA wave
     constexpr int PB = WPOS / 32;         // 32-position blocks per MMA wave
     constexpr int OB = 2;                 // 32-channel blocks per MMA wave
     constexpr int NT = 64 * WAVES_O;      // output channels per workgroup
-    constexpr int ITEMS = kMT * kNV / kThreads;  // (position, vector) items per thread
-    static_assert(ITEMS == 2, "two gather items per thread");
-    static_assert(WAVES_O * WAVES_P <= kThreads / 64, "too many MMA waves");
+    constexpr int NKG = kNV / 2;          // k-groups per step
+    constexpr int ITEMS = MT * kNV / kThreads;   // (position, vector) items per thread
+    static_assert(ITEMS >= 1 && ITEMS * kThreads == MT * kNV, "gather items divide evenly");
+    static_assert(WAVES_O * WAVES_P <= kThreads / 64 && PB >= 1, "MMA wave layout");
 
-    __shared__ __align__(16) unsigned char s_tile[2][kMT * kRS];
-    __shared__ float s_w[2][8][kMT];
-    __shared__ int s_idx[2][kMT];
-    __shared__ int s_flag[2][kMT];
+    __shared__ __align__(16) unsigned char s_tile[2][MT * kRS];
+    __shared__ float s_w[2][8][MT];
+    __shared__ int s_idx[2][MT];
+    __shared__ int s_flag[2][MT];
 
     const TiledShape &s = a.s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
     const int otile = blockIdx.y, wg = blockIdx.z;
-    const int m0 = tile * kMT;
+    const int m0 = tile * MT;
     const int S = s.nchunk * s.K;
     const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;   // element strides of a step in z / y
 
     // --- per-position constants of the coordinate threads
     int cb = 0, cp = 0, coz = 0, coy = 0, cox = 0;
     bool cvalid = false;
-    if (tid < kMT) {
+    if (tid < MT) {
         const int m = m0 + tid;
         cvalid = m < s.M;
         if (cvalid) {
@@ -79,25 +82,39 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
         }
     }
 
-    // corner weights (modulation folded in, dead corners zero), base voxel, live mask of step st
-    auto coords = [&](int st, int buf) {
-        if (tid < kMT) {
+    // offsets and modulation of step st: fetched early (coords_issue), turned into corner weights
+    // (modulation folded in, dead corners zero), base offset and live mask late (coords_finish)
+    float craw[4];
+    auto coords_issue = [&](int st) {
+        if (tid < MT && cvalid) {
+            const int j = st / s.K, k = st - j * s.K;
+            const int g = (wg * s.cg + j * BKC) / s.cpg;
+            if (s.nd == 3) {
+                const long ob = (((long)cb * s.G + g) * s.K + k) * 3 * s.P + cp;
+                craw[0] = ld_auxT<AUX16>(a.off, ob);
+                craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
+                craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
+            } else {
+                craw[0] = 0.f; craw[1] = 0.f;
+                craw[2] = ld_auxT<AUX16>(a.off, (((long)cb * s.G + g) * s.K + k) * s.P + cp);
+            }
+            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, (((long)cb * s.G + g) * s.K + k) * s.P + cp) : 1.f;
+        }
+    };
+    auto coords_finish = [&](int st, int buf) {
+        if (tid < MT) {
             float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             int idx = 0;
             unsigned live = 0;
             if (cvalid) {
-                const int j = st / s.K, k = st - j * s.K;
-                const int g = (wg * s.cg + j * BKC) / s.cpg;
-                float o0, o1, o2;
-                load_offsets(s, a.off, cb, g, k, cp, o0, o1, o2);
-                const float al = a.mask ? ld_aux(a.mask, (((long)cb * s.G + g) * s.K + k) * s.P + cp, s.adt) : 1.f;
+                const int k = st % s.K;
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
-                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+                const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
                 live = t.live;
                 idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
 #pragma unroll
-                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
+                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * craw[3] : 0.f;
             }
 #pragma unroll
             for (int c = 0; c < 8; c++) s_w[buf][c][tid] = w[c];
@@ -106,19 +123,19 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
         }
     };
 
-    // --- gather: item i of this thread = (position ipos[i], vector ivec[i])
+    // --- gather: item i of this thread = (position, 16-byte channel vector)
     uint4 gv[ITEMS][8];
     auto gather_issue = [&](int st, int buf) {
         const int j = st / s.K;
         const int c0 = wg * s.cg + j * BKC;
+        // 32-bit byte offsets from a uniform base: the whole input is below 4 GiB (checked on the host)
+        const char *base = reinterpret_cast<const char *>(a.xcl);
 #pragma unroll
         for (int i = 0; i < ITEMS; i++) {
             const int item = tid + i * kThreads;
             const int pos = item / kNV, vec = item % kNV;
             const int idx = s_idx[buf][pos] + c0 + vec * VEC;
             const unsigned live = (unsigned)s_flag[buf][pos];
-            // 32-bit byte offsets from a uniform base: the whole input is below 4 GiB (checked on the host)
-            const char *base = reinterpret_cast<const char *>(a.xcl);
 #pragma unroll
             for (int c = 0; c < 8; c++) {
                 const unsigned o = (unsigned)(idx + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc + (c & 1) * s.Cin)
@@ -152,37 +169,55 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[ob][pb][r] = 0.f;
 
+    // weight fragments of one whole step live in registers; those of the next step are requested
+    // as soon as the matrix cores have taken the current ones
     const uint4 *wp4 = reinterpret_cast<const uint4 *>(a.wp);
+    uint4 af[NKG][OB];
+    auto wfrag = [&](int st, int kg, int ob) {
+        const long wbase = (((long)wg * S + st) * OBT + (otile * (NT / 32) + wave_o * OB)) * NKG * 64 + lane;
+        return wp4[wbase + ((long)ob * NKG + kg) * 64];
+    };
     auto mma_step = [&](int st, int tbuf) {
         if (!mma_wave) return;
-        const long wbase = (((long)wg * S + st) * OBT + (otile * (NT / 32) + wave_o * OB)) * (kNV / 2) * 64 + lane;
         const unsigned char *tb = &s_tile[tbuf][(wave_p * WPOS + (lane & 31)) * kRS + (lane >> 5) * 16];
 #pragma unroll
-        for (int kg = 0; kg < kNV / 2; kg++) {
-            uint4 af[OB], bf[PB];
-#pragma unroll
-            for (int ob = 0; ob < OB; ob++) af[ob] = wp4[wbase + ((long)ob * (kNV / 2) + kg) * 64];
+        for (int kg = 0; kg < NKG; kg++) {
+            uint4 bf[PB];
 #pragma unroll
             for (int pb = 0; pb < PB; pb++)
                 bf[pb] = *reinterpret_cast<const uint4 *>(tb + pb * 32 * kRS + kg * 32);
 #pragma unroll
             for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[ob], bf[pb]);
+                for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[kg][ob], bf[pb]);
+            if (st + 1 < S) {
+#pragma unroll
+                for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(st + 1, kg, ob);
+            }
         }
     };
 
     // --- pipeline
-    coords(0, 0);
+    coords_issue(0);
+    if (mma_wave) {
+#pragma unroll
+        for (int kg = 0; kg < NKG; kg++)
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(0, kg, ob);
+    }
+    coords_finish(0, 0);
+    if (S > 1) coords_issue(1);
     __syncthreads();
     gather_issue(0, 0);
-    if (S > 1) coords(1, 1);
+    if (S > 1) coords_finish(1, 1);
+    if (S > 2) coords_issue(2);
     interp_store(0, 0);
     __syncthreads();
     for (int st = 0; st < S; st++) {
         if (st + 1 < S) gather_issue(st + 1, (st + 1) & 1);
-        if (st + 2 < S) coords(st + 2, st & 1);
         mma_step(st, st & 1);
+        if (st + 2 < S) coords_finish(st + 2, st & 1);
+        if (st + 3 < S) coords_issue(st + 3);
         if (st + 1 < S) interp_store((st + 1) & 1, (st + 1) & 1);
         __syncthreads();
     }
@@ -213,18 +248,31 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
     }
 }
 
-template <typename T, int WO, int WP>
+template <typename T, bool AUX16, int MT, int WO, int WP>
 int launch_fwd(const FwdArgs &a, hipStream_t st)
 {
-    const int ntile = (a.s.M + kMT - 1) / kMT;
+    const int ntile = (a.s.M + MT - 1) / MT;
     const int NT = 64 * WO;
     dim3 grid(ntile, a.s.ogp / NT, a.s.groups);
     D2cProfScope prof(D2C_PROF_FWD, st);
-    hipLaunchKernelGGL((tiled_fwd_kernel<T, WO, WP>), grid, dim3(kThreads), 0, st, a);
+    hipLaunchKernelGGL((tiled_fwd_kernel<T, AUX16, MT, WO, WP>), grid, dim3(kThreads), 0, st, a);
     return d2c_check_launch("tiled_fwd_kernel");
 }
 
+template <typename T, bool AUX16>
+int launch_fwd_cfg(const FwdArgs &a, int nt, hipStream_t st)
+{
+    switch (nt) {
+    case 512: return launch_fwd<T, AUX16, kMT, 8, 1>(a, st);
+    case 256: return launch_fwd<T, AUX16, kMT, 4, 2>(a, st);
+    case 128: return launch_fwd<T, AUX16, kMT, 2, 4>(a, st);
+    default: return launch_fwd<T, AUX16, kMT, 1, 4>(a, st);
+    }
+}
+
 }  // namespace
+
+int d2c_fwd_pos_tile() { return kMT; }
 
 // Output channels per workgroup: as wide as the weight group needs (the sampled
 // tile is then produced once), but narrower when there are too few position
@@ -232,7 +280,8 @@ int launch_fwd(const FwdArgs &a, hipStream_t st)
 int d2c_fwd_out_tile(int og, int M)
 {
     int nt = og > 256 ? 512 : (og > 128 ? 256 : (og > 64 ? 128 : 64));
-    const int ntile = (M + kMT - 1) / kMT;
+    const int mt = d2c_fwd_pos_tile();
+    const int ntile = (M + mt - 1) / mt;
     while (nt > 64 && ntile * ((og + nt - 1) / nt) < 128) nt >>= 1;
     return nt;
 }
@@ -242,12 +291,11 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
                          const void *bias, void *out, hipStream_t st)
 {
     FwdArgs a{s, xcl, off, mask, wp, bias, out};
-    switch (d2c_fwd_out_tile(s.og, s.M)) {
-    case 512: return launch_fwd<T, 8, 1>(a, st);
-    case 256: return launch_fwd<T, 4, 2>(a, st);
-    case 128: return launch_fwd<T, 2, 4>(a, st);
-    default: return launch_fwd<T, 1, 4>(a, st);
+    const int nt = d2c_fwd_out_tile(s.og, s.M);
+    if constexpr (sizeof(T) == 2) {
+        if (s.adt == D2C_BF16) return launch_fwd_cfg<T, true>(a, nt, st);
     }
+    return launch_fwd_cfg<T, false>(a, nt, st);
 }
 template int d2c_tiled_fwd_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
                                           const void *, void *, hipStream_t);
