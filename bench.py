@@ -60,6 +60,20 @@ def make_inputs(name, torch, crop=None):
     return x, off, m, w, b, gout, G
 
 
+def hbm_traffic_bytes(kernel):
+    """HBM bytes per launch of `kernel` on the headline workload, from the committed rocprofv3 --pmc
+    summary (FETCH_SIZE + WRITE_SIZE, calibrated on a plain copy kernel); None if not recorded."""
+    path = os.path.join(ROOT, "profiles", "c3_hbm_traffic.md")
+    try:
+        for row in open(path):
+            cells = [c.strip().strip("`") for c in row.split("|")]
+            if len(cells) > 4 and cells[1].startswith(kernel):
+                return int(float(cells[4]) * 1e6)
+    except (OSError, ValueError):
+        pass
+    return None
+
+
 def cpu_baseline(name, torch):
     """The oracle (reference algorithm restated in C, OpenMP) on a cropped sample."""
     from oracle import cpu
@@ -156,14 +170,26 @@ def main():
         lib.d2c_profile_read(kid, ctypes.byref(tot), ctypes.byref(cnt))
         if cnt.value:
             kern[kname] = tot.value / nprof  # ms per step spent in this kernel (all launches of it)
-    main_k = {k: v for k, v in kern.items() if k.startswith("tiled_")}
+    # the kernel that takes the most time, against the roofline that bounds it
+    main_k = {k: v for k, v in kern.items() if not k.startswith("pack")}
     dom = max(main_k, key=main_k.get) if main_k else None
     roofline = None
     if dom:
-        ach = f_fwd / (main_k[dom] * 1e-3) / 1e12  # each of the three kernels carries one GEMM of f_fwd flops
-        roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 2), "peak": PEAK_TFLOPS[dt],
-                    "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dt], 4), "traffic": None,
-                    "kernel_ms": {k: round(v, 4) for k, v in kern.items()}}
+        traffic = hbm_traffic_bytes(dom)
+        kms = {k: round(v, 4) for k, v in kern.items()}
+        if dom == "gx_owner_kernel":
+            # memory-bound: every grad-column row (N*P*K*Cin elements), every list entry (32 B per live
+            # sample) and every grad_input element (fp32 accumulator) once
+            es = 2 if dt == "bf16" else 4
+            nbytes = N * P * 27 * C * es + N * P * 27 * G * 32 + N * C * P * 4
+            ach = nbytes / (main_k[dom] * 1e-3) / 1e9
+            roofline = {"bound": "hbm", "kernel": dom, "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s",
+                        "frac": round(ach / 8000.0, 4), "traffic": traffic, "kernel_ms": kms}
+        else:
+            ach = f_fwd / (main_k[dom] * 1e-3) / 1e12  # each of the three tiled kernels carries one GEMM of f_fwd flops
+            roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 2), "peak": PEAK_TFLOPS[dt],
+                        "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dt], 4), "traffic": traffic,
+                        "kernel_ms": kms}
 
     line = {
         "metric": "mdconv3d fwd+bwd effective TFLOP/s (C=512, 8x30x54, k3) on 1 GPU" if name == "c3"

@@ -20,6 +20,13 @@
 
 namespace {
 
+D2C_DEV int xcd_swizzle(int bid, int n)
+{
+    const int x = bid & 7, idx = bid >> 3;
+    const int q = n >> 3, r = n & 7;
+    return x * q + (x < r ? x : r) + idx;
+}
+
 struct alignas(16) InvEntry {
     int p, k;              // output position inside the sample, tap
     float hz, hy, hx;      // fractions z - floor(z), ...
@@ -135,33 +142,57 @@ __global__ void __launch_bounds__(256)
 gx_owner_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *entries, float *gxcl)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
-    const int sub = threadIdx.x & 7;
-    const long vg = (long)blockIdx.x * 32 + (threadIdx.x >> 3);   // voxel index over the batch
+    // a workgroup owns a compact 2 x 4 x 4 block of voxels: the 8 voxels that share a sample are then
+    // mostly served by one workgroup and the grad-column row is fetched once
+    const int sub = threadIdx.x & 7, vi = threadIdx.x >> 3;
     const int cidx = blockIdx.y;                                  // channel chunk
-    if (vg >= (long)s.N * s.vol) return;
-    const int b = (int)(vg / s.vol), v = (int)(vg - (long)b * s.vol);
-    const int x = v % s.W, y = (v / s.W) % s.H, z = v / (s.W * s.H);
+    const int nbx = (s.W + 3) / 4, nby = (s.H + 3) / 4, nbz = (s.D + 1) / 2;
+    int blk = xcd_swizzle(blockIdx.x, gridDim.x);                 // neighbouring blocks on the same XCD (L2)
+    const int bx = blk % nbx; blk /= nbx;
+    const int by = blk % nby; blk /= nby;
+    const int bz = blk % nbz;
+    const int b = blk / nbz;
+    const int x = bx * 4 + (vi & 3), y = by * 4 + ((vi >> 2) & 3), z = bz * 2 + (vi >> 4);
+    if (x >= s.W || y >= s.H || z >= s.D) return;
+    const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;   // voxel index over the batch
     const int g = (cidx * BKC) / s.cpg;
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; i++) acc[i] = 0.f;
     const T *gbase = gcol + ((long)cidx * s.K * s.M + (long)b * s.P) * BKC + sub * VEC;
+    // The base voxels (x-1) and (x) of one (z - dz, y - dy) row are neighbours in the bin order, so
+    // their lists form one contiguous range: 4 ranges per voxel, walked 4 entries at a time with all
+    // loads of a batch issued before their first use (entries past the end repeat the last one with
+    // weight 0).
 #pragma unroll 1
-    for (int d = 0; d < 8; d++) {
-        const int dz = (d >> 2) & 1, dy = (d >> 1) & 1, dx = d & 1;
-        const int bin = bin_of(s, b, g, z - dz, y - dy, x - dx);
-        const int e0 = starts[bin], e1 = starts[bin + 1];
-        for (int e = e0; e < e1; e++) {
-            const uint4 q0 = reinterpret_cast<const uint4 *>(entries + e)[0];
-            const uint4 q1 = reinterpret_cast<const uint4 *>(entries + e)[1];
-            const int p = (int)q0.x, k = (int)q0.y;
-            const float hz = __uint_as_float(q0.z), hy = __uint_as_float(q0.w), hx = __uint_as_float(q1.x);
-            const float al = __uint_as_float(q1.y);
-            const float w = (dz ? hz : 1.f - hz) * (dy ? hy : 1.f - hy) * (dx ? hx : 1.f - hx) * al;
-            const uint4 row = *reinterpret_cast<const uint4 *>(gbase + ((long)k * s.M + p) * BKC);
-            const T *re = reinterpret_cast<const T *>(&row);
+    for (int d = 0; d < 4; d++) {
+        const int dz = (d >> 1) & 1, dy = d & 1;
+        const int bin1 = bin_of(s, b, g, z - dz, y - dy, x - 1);   // dx = 1
+        const int e0 = starts[bin1], em = starts[bin1 + 1], e1 = starts[bin1 + 2];
+        for (int e = e0; e < e1; e += 4) {
+            uint4 q0[4], q1[4], row[4];
 #pragma unroll
-            for (int i = 0; i < VEC; i++) acc[i] = fmaf(w, elem_to_f32<T>(re[i]), acc[i]);
+            for (int i = 0; i < 4; i++) {
+                const int ei = min(e + i, e1 - 1);
+                q0[i] = reinterpret_cast<const uint4 *>(entries + ei)[0];
+                q1[i] = reinterpret_cast<const uint4 *>(entries + ei)[1];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int p = (int)q0[i].x, k = (int)q0[i].y;
+                row[i] = *reinterpret_cast<const uint4 *>(gbase + ((long)k * s.M + p) * BKC);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float hz = __uint_as_float(q0[i].z), hy = __uint_as_float(q0[i].w);
+                const float hx = __uint_as_float(q1[i].x), al = __uint_as_float(q1[i].y);
+                const bool dx = e + i < em;      // entries of base voxel x-1 come first
+                float w = (dz ? hz : 1.f - hz) * (dy ? hy : 1.f - hy) * (dx ? hx : 1.f - hx) * al;
+                w = e + i < e1 ? w : 0.f;
+                const T *re = reinterpret_cast<const T *>(&row[i]);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc[j] = fmaf(w, elem_to_f32<T>(re[j]), acc[j]);
+            }
         }
     }
     float *o = gxcl + vg * s.Cin + cidx * BKC + sub * VEC;
@@ -221,8 +252,8 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
     D2cProfScope prof(D2C_PROF_GX_OWNER, st);
-    const long nv = (long)s.N * s.vol;
-    dim3 grid((unsigned)((nv + 31) / 32), s.Cin / BKC);
+    const long nblk = (long)s.N * ((s.D + 1) / 2) * ((s.H + 3) / 4) * ((s.W + 3) / 4);
+    dim3 grid((unsigned)nblk, s.Cin / BKC);
     hipLaunchKernelGGL(gx_owner_kernel<T>, grid, dim3(256), 0, st, s, (const T *)gcol, starts,
                        (const InvEntry *)entries, gxcl);
     return d2c_check_launch("gx_owner_kernel");

@@ -36,7 +36,7 @@ struct BwdDataArgs {
     const void *gout;   // [N][Cout][P]
     const void *xcl;    // [N][vol][Cin]
     const void *off, *mask;
-    const void *wt;     // [groups][K*nchunk][BKC][ogk]   (W transposed per step, zero padded to ogk)
+    const void *wt;     // [groups][step][BKC][ogk]   (W transposed per step, zero padded to ogk)
     float *gxcl;        // [N][vol][Cin] fp32 accumulator (zeroed) for the atomic scatter, or NULL
     void *gcolbuf;      // [chunk][tap][N*P][BKC] grad-column values for the list-based grad_input, or NULL
     void *goff, *gmask; // or NULL
@@ -116,11 +116,15 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
     const bool want_aux = a.goff != nullptr || a.gmask != nullptr;
 
     for (int st = 0; st < S; st++) {
-        const int k = st / s.nchunk, j = st - k * s.nchunk;
+        // step order: offset group (outer), tap, chunk of the group (inner).  The chunks of a group share
+        // the sampling positions of a tap, so its offset / mask gradient accumulates in registers over the
+        // inner loop; and a group's channel slice of the input stays in L2 across its taps.
+        const int cpc = s.cpg / BKC;                 // chunks per offset group
+        const int jj = st % cpc, k = (st / cpc) % s.K, gi = st / (cpc * s.K);
+        const int j = gi * cpc + jj;                  // chunk inside the weight group
         const int c0 = wg * s.cg + j * BKC;
         const int g = c0 / s.cpg;
-        // last chunk of this offset group inside this weight group -> flush goff / gmask
-        const bool group_end = (j + 1 == s.nchunk) || ((c0 + BKC) / s.cpg != g);
+        const bool group_end = jj + 1 == cpc;         // last chunk of the group for this tap -> flush goff / gmask
 
         // (a) coordinates of the step and the weight tile
         if (tid < MT) {
@@ -582,7 +586,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
 }
 
 // ============================================================ small kernels
-// W[o][c][k] -> wt[wg][step = k*nchunk + j][cc][oo] for oo in [o0, o0 + ogn), padded with zeros to ogk
+// W[o][c][k] -> wt[wg][step][cc][oo] for oo in [o0, o0 + ogn), padded with zeros to ogk; steps in the
+// order of the data kernel (offset group, tap, chunk of the group)
 template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt, TiledShape s, int ogk, int o0,
                                                               int ogn, long total)
@@ -594,7 +599,8 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
         const int cc = (int)(r % BKC); r /= BKC;
         const int st = (int)(r % (s.K * s.nchunk));
         const int wg = (int)(r / (s.K * s.nchunk));
-        const int k = st / s.nchunk, j = st - k * s.nchunk;
+        const int cpc = s.cpg / BKC;   // same step order as tiled_bwd_data_kernel
+        const int k = (st / cpc) % s.K, j = (st / (cpc * s.K)) * cpc + st % cpc;
         wt[i] = oo < ogn ? w[((long)(wg * s.og + o0 + oo) * s.cg + j * BKC + cc) * s.K + k] : (T)0;
     }
 }
