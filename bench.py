@@ -1,21 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the D2Conv3D operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2_bf16|c2_f32|c5b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b]
 
-One step = one forward + one backward (all five gradients) of the modulated
-deformable conv3d through the C ABI of libd2conv.so, inputs resident in HBM,
-outputs and workspace pre-allocated.  Default workload: the headline
-configuration (N=2, Cin=Cout=512, 8x30x54, 3x3x3, pad 1, 8 offset groups,
-offsets ~N(0,2), bfloat16 in / fp32 accumulate).
+One step = one forward (+ one backward with all five gradients, except for
+the forward-only workload c1) of the modulated deformable convolution through
+the C ABI of libd2conv.so, inputs resident in HBM, outputs and workspace
+pre-allocated.  Default workload: the headline configuration c3 (N=2,
+Cin=Cout=512, 8x30x54, 3x3x3, pad 1, 8 offset groups, offsets ~N(0,2),
+bfloat16 in / fp32 accumulate).
 
 Prints ONE JSON line: whole-job effective TFLOP/s (GEMM-equivalent flops
-2*N*P*Cout*Cin*K forward, twice that backward), ms per step, a `roofline`
-object for the kernel that takes the most time (its own flops over its average
-duration, measured with HIP events on the launch stream, against the 2.5
-PFLOP/s dense bf16 MFMA peak) and a `cpu_baseline` object (the CPU oracle,
-i.e. the reference's algorithm restated in C, timed on the host cores on a
-cropped sample of the same workload).
+2*N*P*Cout*(Cin/groups)*K forward, twice that backward), ms per step (and the
+forward / backward split), a `roofline` object for the kernel that takes the
+most time (its algorithmic flops or bytes over its average duration, measured
+with HIP events on the launch stream inside the library) and a `cpu_baseline`
+object (the CPU oracle, i.e. the reference's algorithm restated in C, timed
+on the host cores on a bounded sample of the same workload).
 """
 import argparse
 import ctypes
@@ -27,43 +28,79 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# name: nd, N, Cin, Cout, spatial dims, weight groups, offset groups, dtype, offsets, seed, backward, roofline bound
+#   offsets: ("normal", sigma) or ("dilation", lo, hi) = per-location, per-axis dilation map expanded to tap offsets
 WORKLOADS = {
-    # name: (N, C, (T,H,W), offset groups, dtype, offset sigma, seed)
-    "c3": (2, 512, (8, 30, 54), 8, "bf16", 2.0, 1003),
-    "c2_bf16": (2, 256, (8, 30, 54), 1, "bf16", None, 1002),
-    "c2_f32": (2, 256, (8, 30, 54), 1, "f32", None, 1002),
-    "c5b": (1, 256, (32, 60, 108), 1, "bf16", 1.0, 1005),
+    "c1": dict(nd=3, N=1, C=64, dims=(8, 32, 32), groups=1, G=1, dt="f32", off=("normal", 1.0), seed=1001,
+               backward=False, bound="mfma"),
+    "c2_f32": dict(nd=3, N=2, C=256, dims=(8, 30, 54), groups=1, G=1, dt="f32", off=("dilation", 0.5, 4.0), seed=1002,
+                   backward=True, bound="mfma"),
+    "c2_bf16": dict(nd=3, N=2, C=256, dims=(8, 30, 54), groups=1, G=1, dt="bf16", off=("dilation", 0.5, 4.0),
+                    seed=1002, backward=True, bound="mfma"),
+    "c3": dict(nd=3, N=2, C=512, dims=(8, 30, 54), groups=1, G=8, dt="bf16", off=("normal", 2.0), seed=1003,
+               backward=True, bound="mfma"),
+    "c4": dict(nd=3, N=2, C=1024, dims=(8, 15, 27), groups=1024, G=1, dt="f32", off=("normal", 1.5), seed=1004,
+               backward=True, bound="hbm"),
+    "c5a": dict(nd=1, N=4, C=512, dims=(64,), groups=1, G=1, dt="f32", off=("normal", 1.5), seed=1005,
+                backward=True, bound="hbm"),
+    "c5b": dict(nd=3, N=1, C=256, dims=(32, 60, 108), groups=1, G=1, dt="bf16", off=("normal", 1.0), seed=1005,
+                backward=True, bound="mfma"),
 }
 PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+PEAK_GBS = 8000.0
+# largest sample the CPU leg runs (the oracle does ~0.09 TFLOP/s on 16 cores): N and leading dim cut down to this
+CPU_CROP = {"c5b": (1, (16, 60, 108))}
 
 
 def make_inputs(name, torch, crop=None):
-    """Seeded synthetic tensors of the workload (generated on the CPU).  `crop`
-    replaces (T,H,W) for the CPU sample."""
+    """Seeded synthetic tensors of the workload (generated on the CPU so that the CPU leg and the GPU see the
+    same numbers).  `crop` = (N, dims) replaces the batch and spatial size for the CPU sample."""
     from d2conv3d_amd.grid import offsets_from_size_map
-    N, C, dims, G, dt, sig, seed = WORKLOADS[name]
-    if crop is not None:
-        N, dims = 1, crop
-    g = torch.Generator().manual_seed(seed)
-    K = 27
+    c = WORKLOADS[name]
+    N, dims = (c["N"], c["dims"]) if crop is None else crop
+    C, nd, G, groups = c["C"], c["nd"], c["G"], c["groups"]
+    g = torch.Generator().manual_seed(c["seed"])
+    ks = (3,) * nd
+    K = 3 ** nd
     x = torch.randn(N, C, *dims, generator=g)
-    bound = 1.0 / (C * K) ** 0.5
-    w = (torch.rand(C, C, 3, 3, 3, generator=g) * 2 - 1) * bound
+    bound = 1.0 / (C // groups * K) ** 0.5
+    w = (torch.rand(C, C // groups, *ks, generator=g) * 2 - 1) * bound
     b = (torch.rand(C, generator=g) * 2 - 1) * bound
-    if sig is None:  # dynamic dilation: per-location, per-axis dilation ~U(0.5, 4) expanded to tap offsets
-        size = torch.rand(N, 3, *dims, generator=g) * 3.5 + 0.5
+    if c["off"][0] == "dilation":
+        _, lo, hi = c["off"]
+        size = torch.rand(N, 3, *dims, generator=g) * (hi - lo) + lo
         off = offsets_from_size_map(size, "xyz", (3, 3, 3), (1, 1, 1))
     else:
-        off = torch.randn(N, G * 3 * K, *dims, generator=g) * sig
+        off = torch.randn(N, G * nd * K, *dims, generator=g) * c["off"][1]
     m = torch.sigmoid(torch.randn(N, G * K, *dims, generator=g))
     gout = torch.randn(N, C, *dims, generator=g)
-    return x, off, m, w, b, gout, G
+    return x, off, m, w, b, gout
 
 
-def hbm_traffic_bytes(kernel):
-    """HBM bytes per launch of `kernel` on the headline workload, from the committed rocprofv3 --pmc
-    summary (FETCH_SIZE + WRITE_SIZE, calibrated on a plain copy kernel); None if not recorded."""
-    path = os.path.join(ROOT, "profiles", "c3_hbm_traffic.md")
+def algorithmic(name, N=None, dims=None):
+    """GEMM-equivalent flops (forward) and bytes with every tensor counted once (forward, backward)."""
+    c = WORKLOADS[name]
+    N = c["N"] if N is None else N
+    dims = c["dims"] if dims is None else dims
+    C, nd, G, groups = c["C"], c["nd"], c["G"], c["groups"]
+    K = 3 ** nd
+    P = 1
+    for d in dims:
+        P *= d
+    es = 2 if c["dt"] == "bf16" else 4
+    f_fwd = 2.0 * N * P * C * (C // groups) * K
+    sz_x = N * C * P * es
+    sz_off, sz_m = N * G * nd * K * P * es, N * G * K * P * es
+    sz_w, sz_b = C * (C // groups) * K * es, C * es
+    b_fwd = sz_x + sz_off + sz_m + sz_w + sz_b + sz_x
+    b_bwd = 2 * (sz_x + sz_off + sz_m + sz_w) + sz_x + sz_b
+    return f_fwd, b_fwd, b_bwd
+
+
+def hbm_traffic_bytes(workload, kernel):
+    """HBM bytes per launch of `kernel`, from the committed rocprofv3 --pmc summary of the workload
+    (FETCH_SIZE + WRITE_SIZE, calibrated on a plain copy kernel); None if not recorded."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.md")
     try:
         for row in open(path):
             cells = [c.strip().strip("`") for c in row.split("|")]
@@ -75,23 +112,30 @@ def hbm_traffic_bytes(kernel):
 
 
 def cpu_baseline(name, torch):
-    """The oracle (reference algorithm restated in C, OpenMP) on a cropped sample."""
+    """The oracle (reference algorithm restated in C, OpenMP) on a bounded sample of the workload."""
     from oracle import cpu
-    crop = (8, 15, 27) if WORKLOADS[name][1] >= 512 else (8, 30, 27)
-    x, off, m, w, b, gout, G = make_inputs(name, torch, crop)
-    if WORKLOADS[name][4] == "bf16":
-        x, w, b, gout = (t.bfloat16().float() for t in (x, w, b, gout))
+    c = WORKLOADS[name]
+    crop = CPU_CROP.get(name)
+    x, off, m, w, b, gout = make_inputs(name, torch, crop)
+    if c["dt"] == "bf16":
+        x, w, b, gout, off, m = (t.bfloat16().float() for t in (x, w, b, gout, off, m))
+    fwd, bwd = (cpu.conv3d_forward, cpu.conv3d_backward) if c["nd"] == 3 else (cpu.conv1d_forward, cpu.conv1d_backward)
+    reps = 1
     t0 = time.perf_counter()
-    cpu.conv3d_forward(x, off, m, w, b, 1, 1, 1, 1, G)
-    cpu.conv3d_backward(gout, x, off, m, w, True, 1, 1, 1, 1, G)
-    dt = time.perf_counter() - t0
-    C = x.shape[1]
-    P = crop[0] * crop[1] * crop[2]
-    flops = 3 * 2 * P * C * C * 27
+    while True:
+        fwd(x, off, m, w, b, 1, 1, 1, c["groups"], c["G"])
+        if c["backward"]:
+            bwd(gout, x, off, m, w, True, 1, 1, 1, c["groups"], c["G"])
+        dt = time.perf_counter() - t0
+        if dt > 5.0 or reps >= 200:
+            break
+        reps += 1
+    f_fwd, _, _ = algorithmic(name, x.shape[0], tuple(x.shape[2:]))
+    flops = (3 if c["backward"] else 1) * f_fwd * reps
+    what = "full workload" if crop is None else f"same layer on N={crop[0]}, {'x'.join(map(str, crop[1]))} positions"
     return {
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu.num_threads(), "kind": "port",
-        "sample": f"same layer (C={C}, k3, G={G}) on N=1, {crop[0]}x{crop[1]}x{crop[2]} positions, fp32, "
-                  f"forward+backward once: {dt:.2f} s",
+        "sample": f"{what}, fp32, {'forward+backward' if c['backward'] else 'forward'} x{reps}: {dt:.2f} s",
     }
 
 
@@ -116,30 +160,45 @@ def main():
     torch.cuda.set_device(dev)
 
     name = args.workload
-    N, C, dims, G, dt, sig, seed = WORKLOADS[name]
-    x, off, m, w, b, gout, G = make_inputs(name, torch)
+    c = WORKLOADS[name]
+    N, C, dims, G, groups, dt, nd = c["N"], c["C"], c["dims"], c["G"], c["groups"], c["dt"], c["nd"]
+    x, off, m, w, b, gout = make_inputs(name, torch)
     tdt = torch.bfloat16 if dt == "bf16" else torch.float32
-    x, w, b, gout = (t.to(dev, tdt).contiguous() for t in (x, w, b, gout))
-    off, m = (t.to(dev, tdt).contiguous() for t in (off, m))
+    x, w, b, gout, off, m = (t.to(dev, tdt).contiguous() for t in (x, w, b, gout, off, m))
     code = _lib.D2C_BF16 if dt == "bf16" else _lib.D2C_F32
-    T_, H_, W_ = dims
-    desc = _lib.Conv3dDesc(N, C, C, T_, H_, W_, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, G, T_, H_, W_, code, code)
-    _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "check")
-    algo = _lib.ALGO_NAMES[lib.d2c_conv3d_algo(ctypes.byref(desc))]
+    if nd == 3:
+        T_, H_, W_ = dims
+        desc = _lib.Conv3dDesc(N, C, C, T_, H_, W_, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, groups, G, T_, H_, W_,
+                               code, code)
+        kind = "conv3d"
+        algo = _lib.ALGO_NAMES[lib.d2c_conv3d_algo(ctypes.byref(desc))]
+    else:
+        desc = _lib.Conv1dDesc(N, C, C, dims[0], 3, 1, 1, 1, groups, G, dims[0], code, code, 1)
+        kind = "conv1d"
+        algo = _lib.ALGO_NAMES[lib.d2c_conv1d_algo(ctypes.byref(desc))]
+    f_check = getattr(lib, f"d2c_{kind}_check")
+    f_fwd_ws, f_bwd_ws = (getattr(lib, f"d2c_{kind}_{d}_workspace_bytes") for d in ("forward", "backward"))
+    f_fwd, f_bwd = getattr(lib, f"d2c_{kind}_forward"), getattr(lib, f"d2c_{kind}_backward")
+    _lib.check(f_check(ctypes.byref(desc)), "check")
     out = torch.empty(N, C, *dims, device=dev, dtype=tdt)
     gx, goff, gm, gw, gb = (torch.empty_like(t) for t in (x, off, m, w, b))
-    nf = lib.d2c_conv3d_forward_workspace_bytes(ctypes.byref(desc))
-    nb = lib.d2c_conv3d_backward_workspace_bytes(ctypes.byref(desc))
+    nf = f_fwd_ws(ctypes.byref(desc))
+    nb = f_bwd_ws(ctypes.byref(desc)) if c["backward"] else 0
     ws = torch.empty(max(nf, nb, 256), dtype=torch.uint8, device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     p = lambda t: ctypes.c_void_p(t.data_ptr())
 
+    def forward():
+        _lib.check(f_fwd(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, stream), "forward")
+
+    def backward():
+        _lib.check(f_bwd(ctypes.byref(desc), p(gout), p(x), p(off), p(m), p(w), p(gx), p(goff), p(gm), p(gw), p(gb),
+                         p(ws), nb, stream), "backward")
+
     def step():
-        rc = lib.d2c_conv3d_forward(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, stream)
-        _lib.check(rc, "forward")
-        rc = lib.d2c_conv3d_backward(ctypes.byref(desc), p(gout), p(x), p(off), p(m), p(w), p(gx), p(goff), p(gm),
-                                     p(gw), p(gb), p(ws), nb, stream)
-        _lib.check(rc, "backward")
+        forward()
+        if c["backward"]:
+            backward()
 
     for _ in range(args.warmup):
         step()
@@ -150,56 +209,89 @@ def main():
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    P = T_ * H_ * W_
-    f_fwd = 2.0 * N * P * C * C * 27
-    value = 3 * f_fwd / (ms * 1e-3) / 1e12
+    f_fwd_flops, b_fwd, b_bwd = algorithmic(name)
+    nflops = (3 if c["backward"] else 1) * f_fwd_flops
+    value = nflops / (ms * 1e-3) / 1e12
 
-    # per-kernel durations: HIP events on the launch stream, recorded inside the library
+    # forward and backward separately (events on the launch stream), then per-kernel durations recorded by
+    # the library with HIP events around each launch
+    nprof = max(3, min(args.steps, 10))
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    t_f = t_b = 0.0
+    for _ in range(nprof):
+        ev[0].record()
+        forward()
+        ev[1].record()
+        if c["backward"]:
+            backward()
+        ev[2].record()
+        torch.cuda.synchronize()
+        t_f += ev[0].elapsed_time(ev[1]) / nprof
+        t_b += ev[1].elapsed_time(ev[2]) / nprof
     lib.d2c_profile_reset()
     lib.d2c_profile_enable(1)
-    nprof = max(3, min(args.steps, 10))
     for _ in range(nprof):
         step()
     torch.cuda.synchronize()
     lib.d2c_profile_enable(0)
+    fam = {"mfma": "tiled", "depthwise": "dw", "generic": "generic"}[algo]
+    names = {_lib.PROF_FWD: f"{fam}_fwd_kernel", _lib.PROF_BWD_DATA: f"{fam}_bwd_data_kernel",
+             _lib.PROF_BWD_WEIGHT: f"{fam}_bwd_weight_kernel", _lib.PROF_GX_OWNER: "gx_owner_kernel",
+             _lib.PROF_PACK: "pack/clear/convert/lists"}
+    if fam == "dw":
+        names[_lib.PROF_BWD_DATA] = "dw_bwd_kernel"
     kern = {}
-    for kid, kname in ((_lib.PROF_FWD, "tiled_fwd_kernel"), (_lib.PROF_BWD_DATA, "tiled_bwd_data_kernel"),
-                       (_lib.PROF_BWD_WEIGHT, "tiled_bwd_weight_kernel"), (_lib.PROF_GX_OWNER, "gx_owner_kernel"),
-                       (_lib.PROF_PACK, "pack/clear/convert/lists")):
+    for kid, kname in names.items():
         tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
         lib.d2c_profile_read(kid, ctypes.byref(tot), ctypes.byref(cnt))
         if cnt.value:
             kern[kname] = tot.value / nprof  # ms per step spent in this kernel (all launches of it)
+
     # the kernel that takes the most time, against the roofline that bounds it
     main_k = {k: v for k, v in kern.items() if not k.startswith("pack")}
     dom = max(main_k, key=main_k.get) if main_k else None
     roofline = None
     if dom:
-        traffic = hbm_traffic_bytes(dom)
         kms = {k: round(v, 4) for k, v in kern.items()}
+        traffic = hbm_traffic_bytes(name, dom)
+        t_dom = main_k[dom] * 1e-3
+        es = 2 if dt == "bf16" else 4
+        P = 1
+        for d in dims:
+            P *= d
         if dom == "gx_owner_kernel":
-            # memory-bound: every grad-column row (N*P*K*Cin elements), every list entry (32 B per live
-            # sample) and every grad_input element (fp32 accumulator) once
-            es = 2 if dt == "bf16" else 4
-            nbytes = N * P * 27 * C * es + N * P * 27 * G * 32 + N * C * P * 4
-            ach = nbytes / (main_k[dom] * 1e-3) / 1e9
-            roofline = {"bound": "hbm", "kernel": dom, "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s",
-                        "frac": round(ach / 8000.0, 4), "traffic": traffic, "kernel_ms": kms}
+            # every grad-column row (N*P*K*Cin elements), every list entry (32 B per sample) and every
+            # grad_input element (fp32 accumulator) once
+            K = 3 ** nd
+            nbytes = N * P * K * C * es + N * P * K * G * 32 + N * C * P * 4
+            bound, ach = "hbm", nbytes / t_dom / 1e9
+        elif c["bound"] == "hbm":
+            # every tensor of that direction once
+            nbytes = b_fwd if dom.endswith("fwd_kernel") else b_bwd
+            bound, ach = "hbm", nbytes / t_dom / 1e9
         else:
-            ach = f_fwd / (main_k[dom] * 1e-3) / 1e12  # each of the three tiled kernels carries one GEMM of f_fwd flops
-            roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 2), "peak": PEAK_TFLOPS[dt],
-                        "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dt], 4), "traffic": traffic,
-                        "kernel_ms": kms}
+            # each of the three matrix kernels carries one GEMM of f_fwd flops
+            bound, ach = "mfma", f_fwd_flops / t_dom / 1e12
+        peak, unit = (PEAK_GBS, "GB/s") if bound == "hbm" else (PEAK_TFLOPS[dt], "TFLOP/s")
+        roofline = {"bound": bound, "kernel": dom, "achieved": round(ach, 2), "peak": peak, "unit": unit,
+                    "frac": round(ach / peak, 4), "traffic": traffic, "kernel_ms": kms}
 
+    what = "modulated deformable conv%dd %s" % (nd, "fwd+bwd" if c["backward"] else "fwd")
     line = {
         "metric": "mdconv3d fwd+bwd effective TFLOP/s (C=512, 8x30x54, k3) on 1 GPU" if name == "c3"
-                  else f"mdconv3d fwd+bwd effective TFLOP/s ({name})",
-        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                  else f"{what} effective TFLOP/s ({name}) on 1 GPU",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt, "data": "synthetic",
-        "config": {"workload": f"{name}: modulated deformable conv3d fwd+bwd, N={N}, Cin=Cout={C}, "
-                               f"{T_}x{H_}x{W_}, k3 p1, offset_groups={G}, bias, {dt} in / fp32 accumulate",
-                   "kernel_family": algo, "frac_of_peak_whole_step": round(value / PEAK_TFLOPS[dt], 4)},
+        "config": {"workload": f"{name}: {what}, N={N}, Cin=Cout={C}, {'x'.join(map(str, dims))}, k3 p1, "
+                               f"groups={groups}, offset_groups={G}, bias, "
+                               + ("bf16 in / fp32 accumulate" if dt == "bf16" else "fp32"),
+                   "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
+                   "algorithmic_gflop": round(nflops / 1e9, 2),
+                   "algorithmic_mbytes": round((b_fwd + (b_bwd if c["backward"] else 0)) / 1e6, 1),
+                   "frac_of_mfma_peak_whole_step": round(value / PEAK_TFLOPS[dt], 4),
+                   "frac_of_hbm_peak_whole_step": round((b_fwd + (b_bwd if c["backward"] else 0))
+                                                        / (ms * 1e-3) / 1e9 / PEAK_GBS, 4)},
         "roofline": roofline,
     }
     if not args.no_cpu:
