@@ -7,7 +7,8 @@
 int d2c_fwd_out_tile(int og, int M);
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
-                         const void *bias, void *out, hipStream_t st);
+                         const void *bias, void *out, float *outacc, hipStream_t st);
+int d2c_fwd_split(const TiledShape &s);
 
 bool d2c_tiled_bwd_data_supported(const TiledShape &s, int dtype);
 bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype);
@@ -17,7 +18,8 @@ bool d2c_tiled_bwd_single_pass(const TiledShape &s, int dtype);
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
-                              void *gmask, hipStream_t st);
+                              void *gmask, float *auxacc, hipStream_t st);
+int d2c_bwd_data_split(const TiledShape &s, int dtype);
 void d2c_invlist_ws(const TiledShape &s, size_t *counts, size_t *starts, size_t *bsums, size_t *entries);
 int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, int *counts, int *starts, int *bsums,
                       void *entries, hipStream_t st);
@@ -122,7 +124,7 @@ __global__ void __launch_bounds__(256) pack_weight_fwd_kernel(const T *w, T *wp,
 }
 
 struct FwdWs {
-    size_t xcl, wp, total;
+    size_t xcl, wp, outacc, total;
 };
 FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -130,7 +132,10 @@ FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     FwdWs w;
     w.xcl = 0;
     w.wp = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
-    w.total = w.wp + d2c_align_up((size_t)s.groups * s.nchunk * s.K * s.ogp * bkc_of(q.dtype) * es);
+    w.outacc = w.wp + d2c_align_up((size_t)s.groups * s.nchunk * s.K * s.ogp * bkc_of(q.dtype) * es);
+    // fp32 partial sums of the output, used only when the forward kernel splits its steps
+    w.total = w.outacc;
+    if (d2c_fwd_split(s) > 1) w.total += d2c_align_up((size_t)s.N * s.Cout * s.P * sizeof(float));
     return w;
 }
 
@@ -188,7 +193,7 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
                            (T *)(base + l.wp), s, total);
     }
     if (int rc = d2c_check_launch("pack_weight_fwd_kernel")) return rc;
-    return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, st);
+    return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, (float *)(base + l.outacc), st);
 }
 
 // grad_input by sample lists (see d2c_invlist.hip) needs the whole reduction over output
@@ -199,7 +204,7 @@ bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 struct BwdWs {
-    size_t xcl, wt, gxcl, gwacc, gcol, counts, starts, bsums, entries, total;
+    size_t xcl, wt, gxcl, gwacc, auxacc, gcol, counts, starts, bsums, entries, total;
 };
 BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -211,7 +216,11 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     const int ogk = d2c_bwd_ogk(s.og < omax ? s.og : omax, q.dtype);
     w.gxcl = w.wt + d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * ogk * es);
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
-    w.total = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
+    w.auxacc = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
+    // fp32 scratch of the offset / mask gradient, used only when the data kernel splits its steps
+    w.total = w.auxacc;
+    if (d2c_bwd_data_split(s, q.dtype) > 1)
+        w.total += d2c_align_up((size_t)s.N * s.G * s.K * s.P * (s.nd + 1) * sizeof(float));
     w.gcol = w.counts = w.starts = w.bsums = w.entries = 0;
     if (use_lists(q, s)) {
         size_t c, st, bs, en;
@@ -261,7 +270,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                     return rc;
             if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt,
                                                      lists ? nullptr : gxcl, lists ? base + l.gcol : nullptr, goff,
-                                                     gmask, st))
+                                                     gmask, (float *)(base + l.auxacc), st))
                 return rc;
             if (lists)
                 if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, (const int *)(base + l.starts), base + l.entries,

@@ -43,6 +43,10 @@ struct BwdDataArgs {
     int ogk;            // output channels of this pass rounded up to a whole k-group
     int o0, ogn;        // this pass reduces over output channels [o0, o0 + ogn) of each weight group
     int add_aux;        // later passes add to the offset / mask gradient of earlier ones
+    // Few position tiles (small N*P): the steps are dealt to gridDim.z workgroups per tile, and the offset / mask
+    // gradient (a sum over the channel chunks of a group) is accumulated with atomics in fp32 scratch arrays
+    // laid out like goff / gmask, which a finishing kernel converts.
+    float *auxoff, *auxmask;
 };
 
 // NKG = k-groups of the reduction over output channels held in registers.
@@ -115,7 +119,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 
     const bool want_aux = a.goff != nullptr || a.gmask != nullptr;
 
-    for (int st = 0; st < S; st++) {
+    const int st_lo = (int)((long)S * blockIdx.z / gridDim.z), st_hi = (int)((long)S * (blockIdx.z + 1) / gridDim.z);
+    for (int st = st_lo; st < st_hi; st++) {
         // step order: offset group (outer), tap, chunk of the group (inner).  The chunks of a group share
         // the sampling positions of a tap, so its offset / mask gradient accumulates in registers over the
         // inner loop; and a group's channel slice of the input stays in L2 across its taps.
@@ -124,7 +129,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
         const int j = gi * cpc + jj;                  // chunk inside the weight group
         const int c0 = wg * s.cg + j * BKC;
         const int g = c0 / s.cpg;
-        const bool group_end = jj + 1 == cpc;         // last chunk of the group for this tap -> flush goff / gmask
+        // last chunk of the group for this tap (or of this workgroup's share) -> flush goff / gmask
+        const bool group_end = jj + 1 == cpc || st + 1 == st_hi;
 
         // (a) coordinates of the step and the weight tile
         if (tid < MT) {
@@ -311,7 +317,16 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                         if (m < s.M) {
                             const int b = m / s.P, p = m - b * s.P;
                             const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
-                            if (a.goff && s.nd == 3) {
+                            if (a.auxoff) {
+                                if (a.goff && s.nd == 3) {
+                                    const long ob = 3 * ab - 2 * (long)p;
+#pragma unroll
+                                    for (int ax = 0; ax < 3; ax++) atomicAdd(a.auxoff + ob + ax * (long)s.P, g_acc[i][ax]);
+                                } else if (a.goff) {
+                                    atomicAdd(a.auxoff + ab, g_acc[i][2]);
+                                }
+                                if (a.gmask) atomicAdd(a.auxmask + ab, g_acc[i][3]);
+                            } else if (a.goff && s.nd == 3) {
                                 const long ob = 3 * ab - 2 * (long)p;   // ((b*G+g)*K+k)*3*P + p
 #pragma unroll
                                 for (int ax = 0; ax < 3; ax++) {
@@ -321,7 +336,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                             } else if (a.goff) {
                                 st_aux(a.goff, ab, s.adt, g_acc[i][2] + (a.add_aux ? ld_aux(a.goff, ab, s.adt) : 0.f));
                             }
-                            if (a.gmask)
+                            if (a.gmask && !a.auxoff)
                                 st_aux(a.gmask, ab, s.adt, g_acc[i][3] + (a.add_aux ? ld_aux(a.gmask, ab, s.adt) : 0.f));
                         }
                         g_acc[i][0] = g_acc[i][1] = g_acc[i][2] = g_acc[i][3] = 0.f;
@@ -340,14 +355,14 @@ template <typename T> size_t bwd_data_lds(int ogk)
 }
 
 template <typename T, int NKG>
-int launch_bwd_data(const BwdDataArgs &a, hipStream_t st)
+int launch_bwd_data(const BwdDataArgs &a, int nsplit, hipStream_t st)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
     const size_t lds = bwd_data_lds<T>(a.ogk);
     if (hipFuncSetAttribute((const void *)tiled_bwd_data_kernel<T, NKG>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             160 * 1024) != hipSuccess)
         return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_data_kernel)");
-    dim3 grid((a.s.M + MT - 1) / MT, a.s.groups);
+    dim3 grid((a.s.M + MT - 1) / MT, a.s.groups, nsplit);
     D2cProfScope prof(D2C_PROF_BWD_DATA, st);
     hipLaunchKernelGGL((tiled_bwd_data_kernel<T, NKG>), grid, dim3(kThreads), lds, st, a);
     return d2c_check_launch("tiled_bwd_data_kernel");
@@ -659,6 +674,13 @@ __global__ void __launch_bounds__(256) bias_grad_kernel(const T *gout, T *gb, in
     if (threadIdx.x == 0) gb[o] = f32_to_elem<T>(part[0] + part[1] + part[2] + part[3]);
 }
 
+// fp32 scratch of the split data kernel -> offset / mask gradient in its storage type
+__global__ void __launch_bounds__(256) aux_finish_kernel(const float *src, void *dst, int adt, long n)
+{
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        st_aux(dst, i, adt, src[i]);
+}
+
 inline unsigned grid1d(long n, int cap = 8192)
 {
     long g = (n + 255) / 256;
@@ -687,13 +709,33 @@ bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype)
 // One pass reduces over all output channels of a weight group (the list-based grad_input needs that).
 bool d2c_tiled_bwd_single_pass(const TiledShape &s, int dtype) { return s.og <= d2c_bwd_pass_channels(dtype); }
 
+// Workgroups per position tile of the data kernel: 1 when the tiles alone fill the chip.
+int d2c_bwd_data_split(const TiledShape &s, int dtype)
+{
+    const int mt = dtype == D2C_BF16 ? 128 : 256;
+    const long wgs = (long)((s.M + mt - 1) / mt) * s.groups;
+    if (wgs >= 128) return 1;
+    const int S = s.nchunk * s.K;
+    const long want = (256 + wgs - 1) / wgs;
+    return (int)(want < S ? want : S);
+}
+
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
-                              void *gmask, hipStream_t st)
+                              void *gmask, float *auxacc, hipStream_t st)
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
     const int omax = d2c_bwd_pass_channels(Elem<T>::DT);
+    const int nsplit = auxacc ? d2c_bwd_data_split(s, Elem<T>::DT) : 1;
+    const long n_mask = (long)s.N * s.G * s.K * s.P, n_off = n_mask * s.nd;
+    float *auxoff = nullptr, *auxmask = nullptr;
+    if (nsplit > 1 && (goff || gmask)) {
+        auxoff = auxacc;
+        auxmask = auxacc + n_off;
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(auxacc, (size_t)(n_off + n_mask) * sizeof(float), st);
+    }
     if (gxcl) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
@@ -710,14 +752,22 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                                s, ogk, o0, ogn, total);
         }
         if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
-        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0};
+        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0,
+                      auxoff, auxmask};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
-        if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, st);
-        else if (nkg <= 8) rc = launch_bwd_data<T, 8>(a, st);
-        else if (nkg <= 16) rc = launch_bwd_data<T, 16>(a, st);
-        else rc = launch_bwd_data<T, 32>(a, st);
+        if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, nsplit, st);
+        else if (nkg <= 8) rc = launch_bwd_data<T, 8>(a, nsplit, st);
+        else if (nkg <= 16) rc = launch_bwd_data<T, 16>(a, nsplit, st);
+        else rc = launch_bwd_data<T, 32>(a, nsplit, st);
         if (rc) return rc;
+    }
+    if (auxoff) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        if (goff) hipLaunchKernelGGL(aux_finish_kernel, dim3(grid1d(n_off)), dim3(256), 0, st, auxoff, goff, s.adt, n_off);
+        if (gmask)
+            hipLaunchKernelGGL(aux_finish_kernel, dim3(grid1d(n_mask)), dim3(256), 0, st, auxmask, gmask, s.adt, n_mask);
+        if (int rc = d2c_check_launch("aux_finish_kernel")) return rc;
     }
     return D2C_OK;
 }
@@ -768,7 +818,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
 #define INST(T)                                                                                                    \
     template int d2c_tiled_bwd_data_launch<T>(const TiledShape &, const void *, const void *, const void *,        \
                                               const void *, const void *, void *, float *, void *, void *, void *, \
-                                              hipStream_t);                                                        \
+                                              float *, hipStream_t);                                                        \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
                                                 const void *, float *, void *, hipStream_t);                      \
     template int d2c_tiled_unpack_gx<T>(const TiledShape &, const float *, void *, hipStream_t);                   \

@@ -32,6 +32,10 @@ struct FwdArgs {
     const void *wp;    // packed weights, see pack_weight_fwd
     const void *bias;
     void *out;
+    // Few tiles (small N*P): the steps are dealt to `nsplit` workgroups per tile, which add their partial
+    // sums into a zeroed fp32 array laid out like `out`; a finishing kernel adds the bias and converts.
+    float *outacc;
+    int nsplit;
 };
 
 // Tiles that are neighbours in space go to the same XCD (workgroups are dealt
@@ -65,9 +69,11 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
     const TiledShape &s = a.s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
-    const int otile = blockIdx.y, wg = blockIdx.z;
+    const int otile = blockIdx.y / a.nsplit, split = blockIdx.y - otile * a.nsplit, wg = blockIdx.z;
     const int m0 = tile * MT;
-    const int S = s.nchunk * s.K;
+    const int S = s.nchunk * s.K;                           // steps of the whole reduction
+    const int st_lo = (int)((long)S * split / a.nsplit);    // this workgroup's share of them
+    const int st_hi = (int)((long)S * (split + 1) / a.nsplit);
     const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;   // element strides of a step in z / y
 
     // --- per-position constants of the coordinate threads
@@ -190,35 +196,35 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
             for (int ob = 0; ob < OB; ob++)
 #pragma unroll
                 for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[kg][ob], bf[pb]);
-            if (st + 1 < S) {
+            if (st + 1 < st_hi) {
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(st + 1, kg, ob);
             }
         }
     };
 
-    // --- pipeline
-    coords_issue(0);
+    // --- pipeline (buffers alternate with the parity of the step number)
+    coords_issue(st_lo);
     if (mma_wave) {
 #pragma unroll
         for (int kg = 0; kg < NKG; kg++)
 #pragma unroll
-            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(0, kg, ob);
+            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(st_lo, kg, ob);
     }
-    coords_finish(0, 0);
-    if (S > 1) coords_issue(1);
+    coords_finish(st_lo, st_lo & 1);
+    if (st_lo + 1 < st_hi) coords_issue(st_lo + 1);
     __syncthreads();
-    gather_issue(0, 0);
-    if (S > 1) coords_finish(1, 1);
-    if (S > 2) coords_issue(2);
-    interp_store(0, 0);
+    gather_issue(st_lo, st_lo & 1);
+    if (st_lo + 1 < st_hi) coords_finish(st_lo + 1, (st_lo + 1) & 1);
+    if (st_lo + 2 < st_hi) coords_issue(st_lo + 2);
+    interp_store(st_lo & 1, st_lo & 1);
     __syncthreads();
-    for (int st = 0; st < S; st++) {
-        if (st + 1 < S) gather_issue(st + 1, (st + 1) & 1);
+    for (int st = st_lo; st < st_hi; st++) {
+        if (st + 1 < st_hi) gather_issue(st + 1, (st + 1) & 1);
         mma_step(st, st & 1);
-        if (st + 2 < S) coords_finish(st + 2, st & 1);
-        if (st + 3 < S) coords_issue(st + 3);
-        if (st + 1 < S) interp_store((st + 1) & 1, (st + 1) & 1);
+        if (st + 2 < st_hi) coords_finish(st + 2, st & 1);
+        if (st + 3 < st_hi) coords_issue(st + 3);
+        if (st + 1 < st_hi) interp_store((st + 1) & 1, (st + 1) & 1);
         __syncthreads();
     }
 
@@ -239,12 +245,27 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
                     if (ol < s.og) {
                         const int o = wg * s.og + ol;
                         float v = acc[ob][pb][r];
-                        if (bias) v += elem_to_f32<T>(bias[o]);
-                        out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(v);
+                        if (a.outacc) {
+                            atomicAdd(a.outacc + ((long)b * s.Cout + o) * s.P + p, v);
+                        } else {
+                            if (bias) v += elem_to_f32<T>(bias[o]);
+                            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(v);
+                        }
                     }
                 }
             }
         }
+    }
+}
+
+// out = outacc + bias, in the element type of the output
+template <typename T>
+__global__ void __launch_bounds__(256) fwd_finish_kernel(const float *acc, const T *bias, T *out, int Cout, int P, long n)
+{
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        float v = acc[i];
+        if (bias) v += elem_to_f32<T>(bias[(i / P) % Cout]);
+        out[i] = f32_to_elem<T>(v);
     }
 }
 
@@ -253,7 +274,7 @@ int launch_fwd(const FwdArgs &a, hipStream_t st)
 {
     const int ntile = (a.s.M + MT - 1) / MT;
     const int NT = 64 * WO;
-    dim3 grid(ntile, a.s.ogp / NT, a.s.groups);
+    dim3 grid(ntile, a.s.ogp / NT * a.nsplit, a.s.groups);
     D2cProfScope prof(D2C_PROF_FWD, st);
     hipLaunchKernelGGL((tiled_fwd_kernel<T, AUX16, MT, WO, WP>), grid, dim3(kThreads), 0, st, a);
     return d2c_check_launch("tiled_fwd_kernel");
@@ -286,18 +307,45 @@ int d2c_fwd_out_tile(int og, int M)
     return nt;
 }
 
+// Workgroups per (position tile, output tile): 1 when the tiles alone fill the chip.
+int d2c_fwd_split(const TiledShape &s)
+{
+    const int mt = d2c_fwd_pos_tile(), nt = d2c_fwd_out_tile(s.og, s.M);
+    const long wgs = (long)((s.M + mt - 1) / mt) * (s.ogp / nt) * s.groups;
+    if (wgs >= 128) return 1;
+    const int S = s.nchunk * s.K;
+    const long want = (256 + wgs - 1) / wgs;
+    return (int)(want < S ? want : S);
+}
+
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
-                         const void *bias, void *out, hipStream_t st)
+                         const void *bias, void *out, float *outacc, hipStream_t st)
 {
-    FwdArgs a{s, xcl, off, mask, wp, bias, out};
-    const int nt = d2c_fwd_out_tile(s.og, s.M);
-    if constexpr (sizeof(T) == 2) {
-        if (s.adt == D2C_BF16) return launch_fwd_cfg<T, true>(a, nt, st);
+    const int nsplit = outacc ? d2c_fwd_split(s) : 1;
+    const long n = (long)s.N * s.Cout * s.P;
+    FwdArgs a{s, xcl, off, mask, wp, bias, out, nsplit > 1 ? outacc : nullptr, nsplit};
+    if (nsplit > 1) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(outacc, (size_t)n * sizeof(float), st);
     }
-    return launch_fwd_cfg<T, false>(a, nt, st);
+    const int nt = d2c_fwd_out_tile(s.og, s.M);
+    int rc;
+    bool aux16 = false;
+    if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
+    if constexpr (sizeof(T) == 2) {
+        if (aux16) rc = launch_fwd_cfg<T, true>(a, nt, st);
+    }
+    if (!aux16) rc = launch_fwd_cfg<T, false>(a, nt, st);
+    if (rc || nsplit == 1) return rc;
+    long g = (n + 255) / 256;
+    if (g > 8192) g = 8192;
+    D2cProfScope prof(D2C_PROF_PACK, st);
+    hipLaunchKernelGGL(fwd_finish_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, outacc, (const T *)bias, (T *)out,
+                       s.Cout, s.P, n);
+    return d2c_check_launch("fwd_finish_kernel");
 }
 template int d2c_tiled_fwd_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                          const void *, void *, hipStream_t);
+                                          const void *, void *, float *, hipStream_t);
 template int d2c_tiled_fwd_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                         const void *, void *, hipStream_t);
+                                         const void *, void *, float *, hipStream_t);
