@@ -32,7 +32,7 @@ struct DwArgs {
     const void *bias;
     void *out;
     // backward
-    const void *gout;          // [N][C][P]
+    const void *goutcl;        // [N][P][C]  channels-last copy of grad_out
     float *gxcl;               // [N][vol][C] fp32 accumulator (zeroed) or NULL
     void *goff, *gmask;        // or NULL
     float *gwacc;              // [K][C] fp32 accumulator (zeroed) or NULL
@@ -227,7 +227,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
     const int nslice = (s.cpg + kDwThreads * kCV - 1) / (kDwThreads * kCV);
     const T *xcl = reinterpret_cast<const T *>(a.xcl);
     const T *wt = reinterpret_cast<const T *>(a.wt);
-    const T *gout = reinterpret_cast<const T *>(a.gout);
+    const T *goutcl = reinterpret_cast<const T *>(a.goutcl);
     const bool want_aux = a.goff != nullptr || a.gmask != nullptr;
 
     for (int g = 0; g < s.G; g++) {
@@ -255,11 +255,9 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
                         const unsigned inr = flag >> 8, live = flag & 0xffu;
                         if (!inr) continue;                      // uniform over the workgroup
                         const int m = m0 + p;
-                        const int b = m / s.P, pp = m - b * s.P;  // m < M holds where inr != 0
-                        float go[kCV] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                        for (int j = 0; j < kCV; j++)
-                            if ((okm >> j) & 1u) go[j] = elem_to_f32<T>(gout[((long)b * s.Cout + c + j * kDwThreads) * s.P + pp]);
+                        const int b = m / s.P;                    // m < M holds where inr != 0
+                        float go[kCV];
+                        ld4<T>(goutcl + (long)m * s.Cout + c, go, okm);
                         float gc[kCV];
 #pragma unroll
                         for (int j = 0; j < kCV; j++) gc[j] = wv[j] * go[j];
@@ -378,6 +376,14 @@ bool d2c_depthwise_supported(const TiledShape &s)
     return s.cg == 1 && s.og == 1;
 }
 
+template <typename T> int d2c_depthwise_pack_weight(const TiledShape &s, const void *w, void *wt, hipStream_t st)
+{
+    D2cProfScope prof(D2C_PROF_PACK, st);
+    hipLaunchKernelGGL(dw_pack_weight_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, (const T *)w, (T *)wt,
+                       s.Cin, s.K);
+    return d2c_check_launch("dw_pack_weight_kernel");
+}
+
 template <typename T>
 int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *w,
                           void *wt, const void *bias, void *out, hipStream_t st)
@@ -393,8 +399,10 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
     return d2c_check_launch("dw_fwd_kernel");
 }
 
+// `goutcl` is the channels-last copy of grad_out.  `gxcl` NULL: grad_input is not wanted here (or comes
+// from the sample lists afterwards); otherwise it is accumulated with atomics.
 template <typename T>
-int d2c_depthwise_backward(const TiledShape &s, const void *gout, const void *xcl, const void *off, const void *mask,
+int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
                            const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *gwacc, void *gw,
                            hipStream_t st)
 {
@@ -405,7 +413,7 @@ int d2c_depthwise_backward(const TiledShape &s, const void *gout, const void *xc
         if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
         if (gwacc) d2c_fill_zero(gwacc, (size_t)s.Cin * s.K * sizeof(float), st);
     }
-    DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, gout, gxcl, goff, gmask, gwacc};
+    DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, goutcl, gxcl, goff, gmask, gwacc};
     {
         D2cProfScope prof(D2C_PROF_BWD_DATA, st);
         if (hipFuncSetAttribute((const void *)dw_bwd_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -424,6 +432,7 @@ int d2c_depthwise_backward(const TiledShape &s, const void *gout, const void *xc
 }
 
 #define INST(T)                                                                                                      \
+    template int d2c_depthwise_pack_weight<T>(const TiledShape &, const void *, void *, hipStream_t);                \
     template int d2c_depthwise_forward<T>(const TiledShape &, const void *, const void *, const void *, const void *, \
                                           void *, const void *, void *, hipStream_t);                                \
     template int d2c_depthwise_backward<T>(const TiledShape &, const void *, const void *, const void *,             \

@@ -200,6 +200,100 @@ gx_owner_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *
     for (int i = 0; i < VEC; i += 4) *reinterpret_cast<float4 *>(o + i) = make_float4(acc[i], acc[i + 1], acc[i + 2], acc[i + 3]);
 }
 
+// ---- owner-computes accumulation, channel-separated (depthwise) case ---------
+// gcol[p, k, c] = W[c, k] * gout[p, c] is one multiply, so no grad-column buffer
+// exists: the owner of a voxel reads the channels-last grad_out row of each
+// sample that reaches it and the weight row of its tap (staged in LDS).
+// A workgroup = kOwnVox voxels consecutive in x, 256 lanes each; a lane owns
+// kOwnCV channels 256 apart (whole cache lines per wavefront access).
+constexpr int kOwnVox = 4, kOwnCV = 4, kOwnSlice = 256 * kOwnCV;
+
+template <typename T>
+__global__ void __launch_bounds__(256 * kOwnVox)
+dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts, const InvEntry *entries,
+                   float *gxcl, int w_in_lds)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *s_w = reinterpret_cast<T *>(smem);   // [K][kOwnSlice] weights of the channel slice
+    const int t = threadIdx.x & 255;
+    // wavefront-uniform quantities, kept in scalar registers
+    const int vox = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
+    const int nbx = (s.W + kOwnVox - 1) / kOwnVox;
+    int blk = blockIdx.x;
+    const int xb = blk % nbx; blk /= nbx;
+    const int y = blk % s.H; blk /= s.H;
+    const int z = blk % s.D;
+    const int b = blk / s.D;
+    const int x = xb * kOwnVox + vox;
+    const bool valid = x < s.W;
+    const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;
+    const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
+    const T *grow = goutcl + (long)b * s.P * s.Cout;
+
+    for (int g = 0; g < s.G; g++) {
+        for (int sl = 0; sl < nslice; sl++) {
+            const int cl = sl * kOwnSlice + t;            // first channel of this lane inside the offset group
+            const int c = g * s.cpg + cl;
+            unsigned okm = 0;
+#pragma unroll
+            for (int j = 0; j < kOwnCV; j++) okm |= (cl + j * 256 < s.cpg) ? (1u << j) : 0u;
+            if (w_in_lds) {
+                __syncthreads();
+                for (int i = threadIdx.x; i < s.K * kOwnSlice; i += 256 * kOwnVox) {
+                    const int k = i / kOwnSlice, cc = i - k * kOwnSlice;
+                    const int ch = sl * kOwnSlice + cc;
+                    s_w[i] = ch < s.cpg ? wt[(long)k * s.Cin + g * s.cpg + ch] : (T)0;
+                }
+                __syncthreads();
+            }
+            if (!valid) continue;
+            float acc[kOwnCV];
+#pragma unroll
+            for (int j = 0; j < kOwnCV; j++) acc[j] = 0.f;
+#pragma unroll 1
+            for (int d = 0; d < 4; d++) {
+                const int dz = (d >> 1) & 1, dy = d & 1;
+                const int bin1 = bin_of(s, b, g, z - dz, y - dy, x - 1);   // lists of base voxels x-1 and x are adjacent
+                const int e0 = starts[bin1], em = starts[bin1 + 1], e1 = starts[bin1 + 2];
+                for (int e = e0; e < e1; e += 4) {
+                    float w[4];
+                    int kk[4];
+                    float go[4][kOwnCV];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int ei = min(e + i, e1 - 1);
+                        const InvEntry q = entries[ei];
+                        const bool dx = e + i < em;
+                        const float wv = (dz ? q.hz : 1.f - q.hz) * (dy ? q.hy : 1.f - q.hy) * (dx ? q.hx : 1.f - q.hx)
+                                         * q.alpha;
+                        w[i] = e + i < e1 ? wv : 0.f;
+                        kk[i] = q.k;
+                        const T *gp = grow + (long)q.p * s.Cout + c;
+#pragma unroll
+                        for (int j = 0; j < kOwnCV; j++)
+                            go[i][j] = ((okm >> j) & 1u) ? elem_to_f32<T>(gp[j * 256]) : 0.f;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+#pragma unroll
+                        for (int j = 0; j < kOwnCV; j++) {
+                            float wk = 0.f;
+                            if ((okm >> j) & 1u)
+                                wk = elem_to_f32<T>(w_in_lds ? s_w[kk[i] * kOwnSlice + t + j * 256]
+                                                             : wt[(long)kk[i] * s.Cin + c + j * 256]);
+                            acc[j] = fmaf(w[i] * wk, go[i][j], acc[j]);
+                        }
+                    }
+                }
+            }
+            float *o = gxcl + vg * s.Cin + c;
+#pragma unroll
+            for (int j = 0; j < kOwnCV; j++)
+                if ((okm >> j) & 1u) o[j * 256] = acc[j];
+        }
+    }
+}
+
 inline unsigned g1d(long n, int cap = 16384)
 {
     long g = (n + 255) / 256;
@@ -260,3 +354,25 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts
 }
 template int d2c_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const int *, const void *, float *, hipStream_t);
 template int d2c_gx_owner_launch<float>(const TiledShape &, const void *, const int *, const void *, float *, hipStream_t);
+
+// Depthwise case: grad_input from the sample lists, the channels-last grad_out and the tap-major weights.
+template <typename T>
+int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const int *starts,
+                           const void *entries, float *gxcl, hipStream_t st)
+{
+    D2cProfScope prof(D2C_PROF_GX_OWNER, st);
+    size_t lds = (size_t)s.K * kOwnSlice * sizeof(T);
+    const int w_in_lds = lds <= 144 * 1024;
+    if (!w_in_lds) lds = 0;
+    if (hipFuncSetAttribute((const void *)dw_gx_owner_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024) != hipSuccess)
+        return d2c_check_launch("hipFuncSetAttribute(dw_gx_owner_kernel)");
+    const long nblk = (long)s.N * s.D * s.H * ((s.W + kOwnVox - 1) / kOwnVox);
+    hipLaunchKernelGGL(dw_gx_owner_kernel<T>, dim3((unsigned)nblk), dim3(256 * kOwnVox), lds, st, s, (const T *)goutcl,
+                       (const T *)wt, starts, (const InvEntry *)entries, gxcl, w_in_lds);
+    return d2c_check_launch("dw_gx_owner_kernel");
+}
+template int d2c_dw_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const void *, const int *, const void *,
+                                            float *, hipStream_t);
+template int d2c_dw_gx_owner_launch<float>(const TiledShape &, const void *, const void *, const int *, const void *,
+                                           float *, hipStream_t);

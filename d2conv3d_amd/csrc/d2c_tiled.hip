@@ -37,8 +37,12 @@ bool d2c_depthwise_supported(const TiledShape &s);
 template <typename T>
 int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *w,
                           void *wt, const void *bias, void *out, hipStream_t st);
+template <typename T> int d2c_depthwise_pack_weight(const TiledShape &s, const void *w, void *wt, hipStream_t st);
 template <typename T>
-int d2c_depthwise_backward(const TiledShape &s, const void *gout, const void *xcl, const void *off, const void *mask,
+int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const int *starts,
+                           const void *entries, float *gxcl, hipStream_t st);
+template <typename T>
+int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
                            const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *gwacc, void *gw,
                            hipStream_t st);
 
@@ -154,9 +158,10 @@ bool is_depthwise(const d2c_conv3d_desc &q)
     return q.groups == q.Cin && q.Cout == q.Cin && q.Cin > 1 && d2c_depthwise_supported(tiled_shape(q));
 }
 
-// depthwise workspace: channels-last input | weights [K][C] | grad_input accumulator | grad_weight accumulator
+// depthwise workspace: channels-last input | weights [K][C] | grad_input accumulator | grad_weight accumulator |
+// channels-last grad_out | sample lists (counts, starts, block sums, entries)
 struct DwWs {
-    size_t xcl, wt, gxcl, gwacc, total_fwd, total_bwd;
+    size_t xcl, wt, gxcl, gwacc, goutcl, counts, starts, bsums, entries, total_fwd, total_bwd;
 };
 DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -167,7 +172,14 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.total_fwd = w.wt + d2c_align_up((size_t)s.K * s.Cin * es);
     w.gxcl = w.total_fwd;
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
-    w.total_bwd = w.gwacc + d2c_align_up((size_t)s.K * s.Cin * sizeof(float));
+    w.goutcl = w.gwacc + d2c_align_up((size_t)s.K * s.Cin * sizeof(float));
+    w.counts = w.goutcl + d2c_align_up((size_t)s.N * s.P * s.Cout * es);
+    size_t c, st, bs, en;
+    d2c_invlist_ws(s, &c, &st, &bs, &en);
+    w.starts = w.counts + c;
+    w.bsums = w.starts + st;
+    w.entries = w.bsums + bs;
+    w.total_bwd = w.entries + en;
     return w;
 }
 
@@ -249,9 +261,26 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         float *gxcl = gx ? (float *)(base + d.gxcl) : nullptr;
         float *gwacc = gw ? (float *)(base + d.gwacc) : nullptr;
         if (gx || goff || gmask || gw) {
-            if (int rc = d2c_depthwise_backward<T>(s, gout, base + d.xcl, off, mask, w, base + d.wt, gxcl, goff, gmask,
-                                                  gwacc, gw, st))
-                return rc;
+            // grad_out channels-last: [N][P][C]
+            TiledShape so = s;
+            so.Cin = s.Cout; so.vol = s.P;
+            if (int rc = pack_input<T>(so, gout, base + d.goutcl, st)) return rc;
+            const bool lists = gx && d2c_gx_mode() == 1;
+            if (lists)
+                if (int rc = d2c_invlist_build(s, off, mask, (int *)(base + d.counts), (int *)(base + d.starts),
+                                               (int *)(base + d.bsums), base + d.entries, st))
+                    return rc;
+            if (goff || gmask || gw || !lists)
+                if (int rc = d2c_depthwise_backward<T>(s, base + d.goutcl, base + d.xcl, off, mask, w, base + d.wt,
+                                                      lists ? nullptr : gxcl, goff, gmask, gwacc, gw, st))
+                    return rc;
+            if (lists) {
+                if (!(goff || gmask || gw))
+                    if (int rc = d2c_depthwise_pack_weight<T>(s, w, base + d.wt, st)) return rc;
+                if (int rc = d2c_dw_gx_owner_launch<T>(s, base + d.goutcl, base + d.wt, (const int *)(base + d.starts),
+                                                       base + d.entries, gxcl, st))
+                    return rc;
+            }
             if (gx)
                 if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
         }

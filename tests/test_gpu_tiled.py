@@ -86,10 +86,11 @@ def test_tiled_forward_backward(name, dtype, dev):
                 assert_close(t.grad, e, 2e-2, 2e-2 * e.abs().max().item(), n)
 
 
-@pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail"])
+@pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail", "dw64", "dw96_G3_nomask",
+                                  "dw1100_stride", "dw32_45taps"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_grad_input_by_atomics_matches_lists(name, dtype, dev):
-    # the matrix-core backward has two ways to build grad_input; both must agree with the oracle
+    # the tiled and depthwise backward have two ways to build grad_input; both must agree with the oracle
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, dtype, seed=7)
     eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
     grads = {}
