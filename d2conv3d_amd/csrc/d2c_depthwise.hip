@@ -2,12 +2,12 @@
 // conv3d: no GEMM, one multiply per sampled value.  The reference runs this
 // case as Cin single-row cuBLAS products over a column buffer
 // (dconv3d_gpu.cu:321-353); here one kernel per direction works on the
-// channels-last copy of the input, lanes on consecutive channels, so that every
-// corner read and every atomic of a wavefront covers whole cache lines.
+// channels-last copy of the input; a lane owns 4 consecutive channels, so that
+// every corner read of a wavefront is one contiguous 16-byte-per-lane load.
 //
 //   forward : out[b,c,p]  = bias[c] + sum_k W[c,k] * alpha * trilinear(x[b,c], pos)
 //   backward: gcol        = W[c,k] * gout[b,c,p]
-//             gx[corner] += a_corner * alpha * gcol                     (atomics)
+//             gx[corner] += a_corner * alpha * gcol                     (sample lists, see d2c_invlist.hip; or atomics)
 //             goff, gmask = reductions over the channels of the offset group
 //             gW[c,k]    += gout * alpha * trilinear                    (registers, then atomics)
 //
@@ -20,7 +20,9 @@
 namespace {
 
 constexpr int kDwThreads = 256;
-constexpr int kTP = 16;      // positions per tile
+constexpr int kFwdTP = 4;    // positions per tile, forward (small tiles: many workgroups in flight hide the
+                             // latency of the dependent gather -> multiply chains)
+constexpr int kBwdTP = 16;   // positions per tile, backward (one atomic per tap and channel and tile for grad_weight)
 constexpr int kKB = 32;      // taps per batch held in LDS
 constexpr int kCV = 4;       // channels per lane
 
@@ -38,21 +40,32 @@ struct DwArgs {
     float *gwacc;              // [K][C] fp32 accumulator (zeroed) or NULL
 };
 
-constexpr int kNE = kKB * kTP;   // (tap, position) entries per batch
+template <int TP> constexpr int kNEof = kKB * TP;   // (tap, position) entries per batch
+
+// Workgroups are dealt round-robin to the 8 XCDs; this gives each XCD one contiguous run of tiles, so that
+// its L2 sees a compact part of the input.
+D2C_DEV int xcd_swizzle(int bid, int n)
+{
+    const int x = bid & 7, idx = bid >> 3;
+    const int q = n >> 3, r = n & 7;
+    return x * q + (x < r ? x : r) + idx;
+}
 
 // View over dynamic LDS: per entry the live corner weights * alpha, the base
 // voxel and live | inrange << 8; for the backward pass also the per-axis
 // fractions lz ly lx hz hy hx, alpha, and the 4 offset / mask sums.
-struct DwTaps {
+template <int TP> struct DwTaps {
+    static constexpr int kNE = kNEof<TP>;
     float (*w)[kNE];
     int *idx, *flag;
     float (*frac)[kNE];
     float *alpha;
     float (*aux)[4];
 };
-D2C_DEV DwTaps dw_taps(unsigned char *smem, bool bwd)
+template <int TP> D2C_DEV DwTaps<TP> dw_taps(unsigned char *smem, bool bwd)
 {
-    DwTaps t;
+    constexpr int kNE = kNEof<TP>;
+    DwTaps<TP> t;
     float *f = reinterpret_cast<float *>(smem);
     t.w = reinterpret_cast<float (*)[kNE]>(f); f += 8 * kNE;
     t.idx = reinterpret_cast<int *>(f); f += kNE;
@@ -65,11 +78,11 @@ D2C_DEV DwTaps dw_taps(unsigned char *smem, bool bwd)
     }
     return t;
 }
-constexpr size_t kDwLdsFwd = (size_t)10 * kNE * 4;
-constexpr size_t kDwLdsBwd = (size_t)21 * kNE * 4;
+constexpr size_t kDwLdsFwd = (size_t)10 * kNEof<kFwdTP> * 4;
+constexpr size_t kDwLdsBwd = (size_t)21 * kNEof<kBwdTP> * 4;
 
-template <bool BWD>
-D2C_DEV void dw_coords(const DwArgs &a, const DwTaps &t, int m0, int g, int k0, int kn)
+template <bool BWD, int kTP>
+D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<kTP> &t, int m0, int g, int k0, int kn)
 {
     const TiledShape &s = a.s;
     for (int task = threadIdx.x; task < kn * kTP; task += kDwThreads) {
@@ -109,22 +122,30 @@ D2C_DEV void dw_coords(const DwArgs &a, const DwTaps &t, int m0, int g, int k0, 
     }
 }
 
-// A lane owns kCV channels that are kDwThreads apart, so that one load / atomic
-// instruction of a wavefront covers 64 consecutive channels (whole cache lines).
-template <typename T> D2C_DEV void ld4(const T *p, float *v, unsigned okmask = 0xfu)
+// A lane owns kCV consecutive channels (the channel count of an offset group is a multiple of kCV):
+// one vector load per lane, kCV * 64 consecutive channels per wavefront.
+template <typename T> D2C_DEV void ld4(const T *p, float *v)
 {
-#pragma unroll
-    for (int j = 0; j < kCV; j++) v[j] = ((okmask >> j) & 1u) ? elem_to_f32<T>(p[j * kDwThreads]) : 0.f;
+    if constexpr (sizeof(T) == 4) {
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else {
+        const uint2 t = *reinterpret_cast<const uint2 *>(p);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
 }
+static_assert(kCV == 4, "vector loads of 4 channels");
 
 // ------------------------------------------------------------------ forward
 template <typename T>
 __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
 {
+    constexpr int kTP = kFwdTP;
     extern __shared__ __align__(16) unsigned char smem[];
-    const DwTaps taps = dw_taps(smem, false);
+    const DwTaps<kTP> taps = dw_taps<kTP>(smem, false);
     const TiledShape &s = a.s;
-    const int m0 = blockIdx.x * kTP;
+    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * kTP;
     const int HW = s.H * s.W;
     const int nslice = (s.cpg + kDwThreads * kCV - 1) / (kDwThreads * kCV);
     const T *xcl = reinterpret_cast<const T *>(a.xcl);
@@ -135,45 +156,44 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
         for (int k0 = 0; k0 < s.K; k0 += kKB) {   // one batch unless the kernel has more than kKB taps
             const int kn = min(kKB, s.K - k0);
             __syncthreads();
-            dw_coords<false>(a, taps, m0, g, k0, kn);
+            dw_coords<false, kTP>(a, taps, m0, g, k0, kn);
             __syncthreads();
             for (int sl = 0; sl < nslice; sl++) {
-                const int cl = sl * kDwThreads * kCV + threadIdx.x;   // first channel (inside the offset group)
+                const int cl = (sl * kDwThreads + threadIdx.x) * kCV;   // first channel (inside the offset group)
                 if (cl >= s.cpg) continue;
-                unsigned okm = 0;
-#pragma unroll
-                for (int j = 0; j < kCV; j++) okm |= (cl + j * kDwThreads < s.cpg) ? (1u << j) : 0u;
                 const int c = g * s.cpg + cl;
                 float bv[kCV] = {0.f, 0.f, 0.f, 0.f};
-                if (a.bias && k0 == 0) ld4<T>(reinterpret_cast<const T *>(a.bias) + c, bv, okm);
+                if (a.bias && k0 == 0) ld4<T>(reinterpret_cast<const T *>(a.bias) + c, bv);
                 for (int p = 0; p < kTP; p++) {
                     const int m = m0 + p;
                     if (m >= s.M) break;
                     float acc[kCV] = {bv[0], bv[1], bv[2], bv[3]};
                     for (int kk = 0; kk < kn; kk++) {
                         const int e = kk * kTP + p;
-                        const unsigned live = (unsigned)taps.flag[e] & 0xffu;
+                        // the table entry is the same for the whole workgroup: keep it in scalar registers
+                        const unsigned live = (unsigned)__builtin_amdgcn_readfirstlane(taps.flag[e]) & 0xffu;
                         if (!live) continue;
+                        const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
                         float wv[kCV];
-                        ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv, okm);
-                        const int idx = taps.idx[e];
-                        const int safe = (m / s.P) * s.vol;   // any voxel of the sample: address of dead corners
+                        ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
                         float xv[8][kCV];
-                        // all eight corner rows are requested back to back; dead corners read a
-                        // harmless address and are zeroed afterwards
+                        // all live corner rows are requested back to back
 #pragma unroll
                         for (int cc = 0; cc < 8; cc++) {
-                            const int v = ((live >> cc) & 1u)
-                                              ? idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1) : safe;
-                            ld4<T>(xcl + (long)v * s.Cin + c, xv[cc], okm);
+                            const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
+                            if ((live >> cc) & 1u) {
+                                ld4<T>(xcl + (long)v * s.Cin + c, xv[cc]);
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < kCV; j++) xv[cc][j] = 0.f;
+                            }
                         }
                         float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int cc = 0; cc < 8; cc++) {
                             const float wc = taps.w[cc][e];
 #pragma unroll
-                            for (int j = 0; j < kCV; j++)
-                                sv[j] = fmaf(wc, ((live >> cc) & 1u) ? xv[cc][j] : 0.f, sv[j]);
+                            for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, xv[cc][j], sv[j]);
                         }
 #pragma unroll
                         for (int j = 0; j < kCV; j++) acc[j] = fmaf(wv[j], sv[j], acc[j]);
@@ -181,8 +201,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
                     const int b = m / s.P, pp = m - b * s.P;
 #pragma unroll
                     for (int j = 0; j < kCV; j++) {
-                        if (!((okm >> j) & 1u)) continue;
-                        T *o = out + ((long)b * s.Cout + c + j * kDwThreads) * s.P + pp;
+                        T *o = out + ((long)b * s.Cout + c + j) * s.P + pp;
                         // kernels with more than kKB taps: later batches add to the stored partial sum
                         *o = f32_to_elem<T>(k0 == 0 ? acc[j] : acc[j] + elem_to_f32<T>(*o));
                     }
@@ -217,11 +236,12 @@ D2C_DEV float reduce4_over_wave(float v0, float v1, float v2, float v3, int lane
 template <typename T>
 __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
 {
+    constexpr int kTP = kBwdTP;
     extern __shared__ __align__(16) unsigned char smem[];
-    const DwTaps taps = dw_taps(smem, true);
+    const DwTaps<kTP> taps = dw_taps<kTP>(smem, true);
     float (*s_aux)[4] = taps.aux;   // goff z,y,x and gmask sums over the channels of the group
     const TiledShape &s = a.s;
-    const int m0 = blockIdx.x * kTP;
+    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * kTP;
     const int HW = s.H * s.W;
     const int lane = threadIdx.x & 63;
     const int nslice = (s.cpg + kDwThreads * kCV - 1) / (kDwThreads * kCV);
@@ -234,60 +254,58 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
         for (int k0 = 0; k0 < s.K; k0 += kKB) {
             const int kn = min(kKB, s.K - k0);
             __syncthreads();
-            dw_coords<true>(a, taps, m0, g, k0, kn);
+            dw_coords<true, kTP>(a, taps, m0, g, k0, kn);
             for (int e = threadIdx.x; e < kn * kTP; e += kDwThreads)
                 s_aux[e][0] = s_aux[e][1] = s_aux[e][2] = s_aux[e][3] = 0.f;
             __syncthreads();
             for (int sl = 0; sl < nslice; sl++) {
-                const int cl = sl * kDwThreads * kCV + threadIdx.x;
-                const bool cok = cl < s.cpg;
-                unsigned okm = 0;
-#pragma unroll
-                for (int j = 0; j < kCV; j++) okm |= (cl + j * kDwThreads < s.cpg) ? (1u << j) : 0u;
+                const int cl = (sl * kDwThreads + threadIdx.x) * kCV;
+                const bool cok = cl < s.cpg;       // lanes past the group still take part in the reductions
                 const int c = g * s.cpg + (cok ? cl : 0);
                 for (int kk = 0; kk < kn; kk++) {
                     float wv[kCV] = {0.f, 0.f, 0.f, 0.f};
-                    if (cok) ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv, okm);
+                    if (cok) ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
                     float gwv[kCV] = {0.f, 0.f, 0.f, 0.f};
                     for (int p = 0; p < kTP; p++) {
                         const int e = kk * kTP + p;
-                        const unsigned flag = (unsigned)taps.flag[e];
+                        // the table entry is the same for the whole workgroup: keep it in scalar registers
+                        const unsigned flag = (unsigned)__builtin_amdgcn_readfirstlane(taps.flag[e]);
                         const unsigned inr = flag >> 8, live = flag & 0xffu;
-                        if (!inr) continue;                      // uniform over the workgroup
-                        const int m = m0 + p;
-                        const int b = m / s.P;                    // m < M holds where inr != 0
-                        float go[kCV];
-                        ld4<T>(goutcl + (long)m * s.Cout + c, go, okm);
+                        if (!inr) continue;
+                        const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
+                        const int m = m0 + p;                     // m < M holds where inr != 0
+                        float go[kCV] = {0.f, 0.f, 0.f, 0.f};
+                        if (cok) ld4<T>(goutcl + (long)m * s.Cout + c, go);
                         float gc[kCV];
 #pragma unroll
                         for (int j = 0; j < kCV; j++) gc[j] = wv[j] * go[j];
-                        const int idx = taps.idx[e];
-                        const int safe = b * s.vol;
                         float xv[8][kCV];
 #pragma unroll
                         for (int cc = 0; cc < 8; cc++) {
-                            const int v = ((inr >> cc) & 1u)
-                                              ? idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1) : safe;
-                            ld4<T>(xcl + (long)v * s.Cin + c, xv[cc], okm);
+                            const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
+                            if (((inr >> cc) & 1u) && cok) {
+                                ld4<T>(xcl + (long)v * s.Cin + c, xv[cc]);
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < kCV; j++) xv[cc][j] = 0.f;
+                            }
                         }
                         float dot[8];
                         float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int cc = 0; cc < 8; cc++) {
                             float d = 0.f;
-                            const bool in_c = ((inr >> cc) & 1u) && cok;
 #pragma unroll
-                            for (int j = 0; j < kCV; j++) d = fmaf(gc[j], in_c ? xv[cc][j] : 0.f, d);
-                            if (((live >> cc) & 1u) && cok) {
+                            for (int j = 0; j < kCV; j++) d = fmaf(gc[j], xv[cc][j], d);
+                            if ((live >> cc) & 1u) {
                                 const float wc = taps.w[cc][e];   // a_corner * alpha
 #pragma unroll
                                 for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, xv[cc][j], sv[j]);
-                                if (a.gxcl) {
+                                if (a.gxcl && cok) {
                                     const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
                                     float *gp = a.gxcl + (long)v * s.Cin + c;
 #pragma unroll
-                                    for (int j = 0; j < kCV; j++)
-                                        if ((okm >> j) & 1u) atomicAdd(gp + j * kDwThreads, wc * gc[j]);
+                                    for (int j = 0; j < kCV; j++) atomicAdd(gp + j, wc * gc[j]);
                                 }
                             }
                             dot[cc] = d;
@@ -314,8 +332,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
                     if (a.gwacc && cok) {
                         float *gw = a.gwacc + (long)(k0 + kk) * s.Cin + c;
 #pragma unroll
-                        for (int j = 0; j < kCV; j++)
-                            if ((okm >> j) & 1u) atomicAdd(gw + j * kDwThreads, gwv[j]);
+                        for (int j = 0; j < kCV; j++) atomicAdd(gw + j, gwv[j]);
                     }
                 }
             }
@@ -373,7 +390,8 @@ inline unsigned g1d(long n)
 
 bool d2c_depthwise_supported(const TiledShape &s)
 {
-    return s.cg == 1 && s.og == 1;
+    // a lane's vector of channels must not straddle an offset group
+    return s.cg == 1 && s.og == 1 && s.cpg % kCV == 0;
 }
 
 template <typename T> int d2c_depthwise_pack_weight(const TiledShape &s, const void *w, void *wt, hipStream_t st)
@@ -395,7 +413,7 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
     }
     DwArgs a{s, xcl, off, mask, wt, bias, out, nullptr, nullptr, nullptr, nullptr, nullptr};
     D2cProfScope prof(D2C_PROF_FWD, st);
-    hipLaunchKernelGGL(dw_fwd_kernel<T>, dim3((s.M + kTP - 1) / kTP), dim3(kDwThreads), kDwLdsFwd, st, a);
+    hipLaunchKernelGGL(dw_fwd_kernel<T>, dim3((s.M + kFwdTP - 1) / kFwdTP), dim3(kDwThreads), kDwLdsFwd, st, a);
     return d2c_check_launch("dw_fwd_kernel");
 }
 
@@ -419,7 +437,7 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
         if (hipFuncSetAttribute((const void *)dw_bwd_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)kDwLdsBwd) != hipSuccess)
             return d2c_check_launch("hipFuncSetAttribute(dw_bwd_kernel)");
-        hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3((s.M + kTP - 1) / kTP), dim3(kDwThreads), kDwLdsBwd, st, a);
+        hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3((s.M + kBwdTP - 1) / kBwdTP), dim3(kDwThreads), kDwLdsBwd, st, a);
     }
     if (int rc = d2c_check_launch("dw_bwd_kernel")) return rc;
     if (gwacc && gw) {

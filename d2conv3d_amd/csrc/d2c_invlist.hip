@@ -205,8 +205,20 @@ gx_owner_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *
 // exists: the owner of a voxel reads the channels-last grad_out row of each
 // sample that reaches it and the weight row of its tap (staged in LDS).
 // A workgroup = kOwnVox voxels consecutive in x, 256 lanes each; a lane owns
-// kOwnCV channels 256 apart (whole cache lines per wavefront access).
+// kOwnCV consecutive channels (one vector load per lane and row).
 constexpr int kOwnVox = 4, kOwnCV = 4, kOwnSlice = 256 * kOwnCV;
+
+template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
+{
+    if constexpr (sizeof(T) == 4) {
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else {
+        const uint2 t = *reinterpret_cast<const uint2 *>(p);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+}
 
 template <typename T>
 __global__ void __launch_bounds__(256 * kOwnVox)
@@ -219,7 +231,7 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
     // wavefront-uniform quantities, kept in scalar registers
     const int vox = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
     const int nbx = (s.W + kOwnVox - 1) / kOwnVox;
-    int blk = blockIdx.x;
+    int blk = xcd_swizzle(blockIdx.x, gridDim.x);   // one contiguous part of the volume per XCD (L2)
     const int xb = blk % nbx; blk /= nbx;
     const int y = blk % s.H; blk /= s.H;
     const int z = blk % s.D;
@@ -232,11 +244,9 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
 
     for (int g = 0; g < s.G; g++) {
         for (int sl = 0; sl < nslice; sl++) {
-            const int cl = sl * kOwnSlice + t;            // first channel of this lane inside the offset group
+            const int cl = sl * kOwnSlice + t * kOwnCV;   // first channel of this lane inside the offset group
             const int c = g * s.cpg + cl;
-            unsigned okm = 0;
-#pragma unroll
-            for (int j = 0; j < kOwnCV; j++) okm |= (cl + j * 256 < s.cpg) ? (1u << j) : 0u;
+            const bool cok = cl < s.cpg;                  // cpg is a multiple of kOwnCV
             if (w_in_lds) {
                 __syncthreads();
                 for (int i = threadIdx.x; i < s.K * kOwnSlice; i += 256 * kOwnVox) {
@@ -246,7 +256,7 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
                 }
                 __syncthreads();
             }
-            if (!valid) continue;
+            if (!valid || !cok) continue;
             float acc[kOwnCV];
 #pragma unroll
             for (int j = 0; j < kOwnCV; j++) acc[j] = 0.f;
@@ -268,28 +278,19 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
                                          * q.alpha;
                         w[i] = e + i < e1 ? wv : 0.f;
                         kk[i] = q.k;
-                        const T *gp = grow + (long)q.p * s.Cout + c;
-#pragma unroll
-                        for (int j = 0; j < kOwnCV; j++)
-                            go[i][j] = ((okm >> j) & 1u) ? elem_to_f32<T>(gp[j * 256]) : 0.f;
+                        ld_vec4<T>(grow + (long)q.p * s.Cout + c, go[i]);
                     }
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
+                        float wk[kOwnCV];
+                        if (w_in_lds) ld_vec4<T>(s_w + kk[i] * kOwnSlice + t * kOwnCV, wk);
+                        else ld_vec4<T>(wt + (long)kk[i] * s.Cin + c, wk);
 #pragma unroll
-                        for (int j = 0; j < kOwnCV; j++) {
-                            float wk = 0.f;
-                            if ((okm >> j) & 1u)
-                                wk = elem_to_f32<T>(w_in_lds ? s_w[kk[i] * kOwnSlice + t + j * 256]
-                                                             : wt[(long)kk[i] * s.Cin + c + j * 256]);
-                            acc[j] = fmaf(w[i] * wk, go[i][j], acc[j]);
-                        }
+                        for (int j = 0; j < kOwnCV; j++) acc[j] = fmaf(w[i] * wk[j], go[i][j], acc[j]);
                     }
                 }
             }
-            float *o = gxcl + vg * s.Cin + c;
-#pragma unroll
-            for (int j = 0; j < kOwnCV; j++)
-                if ((okm >> j) & 1u) o[j * 256] = acc[j];
+            *reinterpret_cast<float4 *>(gxcl + vg * s.Cin + c) = make_float4(acc[0], acc[1], acc[2], acc[3]);
         }
     }
 }
