@@ -11,20 +11,23 @@
 //             goff, gmask = reductions over the channels of the offset group
 //             gW[c,k]    += gout * alpha * trilinear                    (registers, then atomics)
 //
-// A workgroup owns a tile of 16 output positions.  The corner weights of the
-// tile (16 positions x up to 32 taps) are computed once into LDS and shared by
-// all channel slices.
+// A workgroup owns a tile of output positions and a slice of 256 channels (one
+// 16-byte vector per lane of a wavefront).  The slice is the slow launch
+// dimension: at any time the whole chip works on one channel slice of the
+// input, which then stays in the L2 caches.  The corner weights of the tile are
+// computed once into LDS and shared by the four wavefronts.
 #include "d2c_mma.hpp"
 #include "d2c_tiled.hpp"
 
 namespace {
 
-constexpr int kDwThreads = 256;
-constexpr int kFwdTP = 4;    // positions per tile, forward (small tiles: many workgroups in flight hide the
-                             // latency of the dependent gather -> multiply chains)
-constexpr int kBwdTP = 16;   // positions per tile, backward (one atomic per tap and channel and tile for grad_weight)
-constexpr int kKB = 32;      // taps per batch held in LDS
-constexpr int kCV = 4;       // channels per lane
+constexpr int kDwThreads = 256;   // 4 wavefronts
+constexpr int kCV = 4;            // consecutive channels per lane
+constexpr int kSlice = 64 * kCV;  // channels per workgroup
+// forward: 8 consecutive positions per wavefront (one 32-byte output segment per channel)
+constexpr int kFwdTP = 32, kFwdKB = 16;
+// backward: the taps of a batch are dealt to the wavefronts, each walks all positions of the tile
+constexpr int kBwdTP = 16, kBwdKB = 32;
 
 struct DwArgs {
     TiledShape s;
@@ -35,12 +38,10 @@ struct DwArgs {
     void *out;
     // backward
     const void *goutcl;        // [N][P][C]  channels-last copy of grad_out
-    float *gxcl;               // [N][vol][C] fp32 accumulator (zeroed) or NULL
-    void *goff, *gmask;        // or NULL
+    float *gxcl;               // [N][vol][C] fp32 accumulator (zeroed) for the atomic scatter, or NULL
+    float *auxoff, *auxmask;   // fp32 accumulators (zeroed) laid out like grad_offset / grad_mask, or NULL
     float *gwacc;              // [K][C] fp32 accumulator (zeroed) or NULL
 };
-
-template <int TP> constexpr int kNEof = kKB * TP;   // (tap, position) entries per batch
 
 // Workgroups are dealt round-robin to the 8 XCDs; this gives each XCD one contiguous run of tiles, so that
 // its L2 sees a compact part of the input.
@@ -51,42 +52,40 @@ D2C_DEV int xcd_swizzle(int bid, int n)
     return x * q + (x < r ? x : r) + idx;
 }
 
-// View over dynamic LDS: per entry the live corner weights * alpha, the base
-// voxel and live | inrange << 8; for the backward pass also the per-axis
-// fractions lz ly lx hz hy hx, alpha, and the 4 offset / mask sums.
-template <int TP> struct DwTaps {
-    static constexpr int kNE = kNEof<TP>;
+// View over dynamic LDS, one entry per (tap of the batch, position of the tile): the live corner
+// weights * alpha, the base voxel and live | inrange << 8; for the backward pass also the per-axis
+// fractions lz ly lx hz hy hx and alpha.
+template <int TP, int KB> struct DwTaps {
+    static constexpr int kNE = KB * TP;
     float (*w)[kNE];
     int *idx, *flag;
     float (*frac)[kNE];
     float *alpha;
-    float (*aux)[4];
 };
-template <int TP> D2C_DEV DwTaps<TP> dw_taps(unsigned char *smem, bool bwd)
+template <int TP, int KB> D2C_DEV DwTaps<TP, KB> dw_taps(unsigned char *smem, bool bwd)
 {
-    constexpr int kNE = kNEof<TP>;
-    DwTaps<TP> t;
+    constexpr int kNE = KB * TP;
+    DwTaps<TP, KB> t;
     float *f = reinterpret_cast<float *>(smem);
     t.w = reinterpret_cast<float (*)[kNE]>(f); f += 8 * kNE;
     t.idx = reinterpret_cast<int *>(f); f += kNE;
     t.flag = reinterpret_cast<int *>(f); f += kNE;
-    t.frac = nullptr; t.alpha = nullptr; t.aux = nullptr;
+    t.frac = nullptr; t.alpha = nullptr;
     if (bwd) {
         t.frac = reinterpret_cast<float (*)[kNE]>(f); f += 6 * kNE;
-        t.alpha = f; f += kNE;
-        t.aux = reinterpret_cast<float (*)[4]>(f);
+        t.alpha = f;
     }
     return t;
 }
-constexpr size_t kDwLdsFwd = (size_t)10 * kNEof<kFwdTP> * 4;
-constexpr size_t kDwLdsBwd = (size_t)21 * kNEof<kBwdTP> * 4;
+constexpr size_t kDwLdsFwd = (size_t)10 * kFwdKB * kFwdTP * 4;
+constexpr size_t kDwLdsBwd = (size_t)17 * kBwdKB * kBwdTP * 4;
 
-template <bool BWD, int kTP>
-D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<kTP> &t, int m0, int g, int k0, int kn)
+template <bool BWD, int TP, int KB>
+D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<TP, KB> &t, int m0, int g, int k0, int kn)
 {
     const TiledShape &s = a.s;
-    for (int task = threadIdx.x; task < kn * kTP; task += kDwThreads) {
-        const int pl = task % kTP, kk = task / kTP;
+    for (int task = threadIdx.x; task < kn * TP; task += kDwThreads) {
+        const int pl = task % TP, kk = task / TP;
         const int k = k0 + kk, m = m0 + pl;
         float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         float fr[6] = {0, 0, 0, 0, 0, 0};
@@ -109,7 +108,7 @@ D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<kTP> &t, int m0, int g, int
             for (int c = 0; c < 8; c++) w[c] = ((tp.live >> c) & 1u) ? tap3_weight(tp, c) * al : 0.f;
             fr[0] = tp.lz; fr[1] = tp.ly; fr[2] = tp.lx; fr[3] = tp.hz; fr[4] = tp.hy; fr[5] = tp.hx;
         }
-        const int e = kk * kTP + pl;
+        const int e = kk * TP + pl;
 #pragma unroll
         for (int c = 0; c < 8; c++) t.w[c][e] = w[c];
         if (BWD) {
@@ -141,71 +140,98 @@ static_assert(kCV == 4, "vector loads of 4 channels");
 template <typename T>
 __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
 {
-    constexpr int kTP = kFwdTP;
+    constexpr int TP = kFwdTP, KB = kFwdKB, PW = TP / 4;   // PW positions per wavefront
     extern __shared__ __align__(16) unsigned char smem[];
-    const DwTaps<kTP> taps = dw_taps<kTP>(smem, false);
+    const DwTaps<TP, KB> taps = dw_taps<TP, KB>(smem, false);
     const TiledShape &s = a.s;
-    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * kTP;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * TP;
     const int HW = s.H * s.W;
-    const int nslice = (s.cpg + kDwThreads * kCV - 1) / (kDwThreads * kCV);
+    const int nsl = (s.cpg + kSlice - 1) / kSlice;
+    const int g = blockIdx.y / nsl, sl = blockIdx.y - g * nsl;
+    const int cl = sl * kSlice + lane * kCV;      // first channel of this lane inside the offset group
+    const bool cok = cl < s.cpg;
+    const int c = g * s.cpg + (cok ? cl : 0);
     const T *xcl = reinterpret_cast<const T *>(a.xcl);
     const T *wt = reinterpret_cast<const T *>(a.wt);
-    T *out = reinterpret_cast<T *>(a.out);
 
-    for (int g = 0; g < s.G; g++) {
-        for (int k0 = 0; k0 < s.K; k0 += kKB) {   // one batch unless the kernel has more than kKB taps
-            const int kn = min(kKB, s.K - k0);
-            __syncthreads();
-            dw_coords<false, kTP>(a, taps, m0, g, k0, kn);
-            __syncthreads();
-            for (int sl = 0; sl < nslice; sl++) {
-                const int cl = (sl * kDwThreads + threadIdx.x) * kCV;   // first channel (inside the offset group)
-                if (cl >= s.cpg) continue;
-                const int c = g * s.cpg + cl;
-                float bv[kCV] = {0.f, 0.f, 0.f, 0.f};
-                if (a.bias && k0 == 0) ld4<T>(reinterpret_cast<const T *>(a.bias) + c, bv);
-                for (int p = 0; p < kTP; p++) {
-                    const int m = m0 + p;
-                    if (m >= s.M) break;
-                    float acc[kCV] = {bv[0], bv[1], bv[2], bv[3]};
-                    for (int kk = 0; kk < kn; kk++) {
-                        const int e = kk * kTP + p;
-                        // the table entry is the same for the whole workgroup: keep it in scalar registers
-                        const unsigned live = (unsigned)__builtin_amdgcn_readfirstlane(taps.flag[e]) & 0xffu;
-                        if (!live) continue;
-                        const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
-                        float wv[kCV];
-                        ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
-                        float xv[8][kCV];
-                        // all live corner rows are requested back to back
+    float acc[PW][kCV];
 #pragma unroll
-                        for (int cc = 0; cc < 8; cc++) {
-                            const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
-                            if ((live >> cc) & 1u) {
-                                ld4<T>(xcl + (long)v * s.Cin + c, xv[cc]);
-                            } else {
+    for (int i = 0; i < PW; i++)
 #pragma unroll
-                                for (int j = 0; j < kCV; j++) xv[cc][j] = 0.f;
-                            }
-                        }
-                        float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < kCV; j++) acc[i][j] = 0.f;
+
+    for (int k0 = 0; k0 < s.K; k0 += KB) {
+        const int kn = min(KB, s.K - k0);
+        __syncthreads();
+        dw_coords<false, TP, KB>(a, taps, m0, g, k0, kn);
+        __syncthreads();
+        if (!cok) continue;
+        for (int kk = 0; kk < kn; kk++) {
+            float wv[kCV];
+            ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
 #pragma unroll
-                        for (int cc = 0; cc < 8; cc++) {
-                            const float wc = taps.w[cc][e];
+            for (int i = 0; i < PW; i++) {
+                const int e = kk * TP + wave * PW + i;
+                // the table entry is the same for the whole wavefront: keep it in scalar registers
+                const unsigned live = (unsigned)__builtin_amdgcn_readfirstlane(taps.flag[e]) & 0xffu;
+                if (!live) continue;
+                const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
+                float xv[8][kCV];
+                // all live corner rows are requested back to back
 #pragma unroll
-                            for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, xv[cc][j], sv[j]);
-                        }
+                for (int cc = 0; cc < 8; cc++) {
+                    const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
+                    if ((live >> cc) & 1u) {
+                        ld4<T>(xcl + (long)v * s.Cin + c, xv[cc]);
+                    } else {
 #pragma unroll
-                        for (int j = 0; j < kCV; j++) acc[j] = fmaf(wv[j], sv[j], acc[j]);
-                    }
-                    const int b = m / s.P, pp = m - b * s.P;
-#pragma unroll
-                    for (int j = 0; j < kCV; j++) {
-                        T *o = out + ((long)b * s.Cout + c + j) * s.P + pp;
-                        // kernels with more than kKB taps: later batches add to the stored partial sum
-                        *o = f32_to_elem<T>(k0 == 0 ? acc[j] : acc[j] + elem_to_f32<T>(*o));
+                        for (int j = 0; j < kCV; j++) xv[cc][j] = 0.f;
                     }
                 }
+                float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int cc = 0; cc < 8; cc++) {
+                    const float wc = taps.w[cc][e];
+#pragma unroll
+                    for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, xv[cc][j], sv[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < kCV; j++) acc[i][j] = fmaf(wv[j], sv[j], acc[i][j]);
+            }
+        }
+    }
+    if (!cok) return;
+
+    // --- bias, convert, store: the PW positions of a wavefront are consecutive in the output row of a channel
+    float bv[kCV] = {0.f, 0.f, 0.f, 0.f};
+    if (a.bias) ld4<T>(reinterpret_cast<const T *>(a.bias) + c, bv);
+    T *out = reinterpret_cast<T *>(a.out);
+    const int mf = m0 + wave * PW;
+    if (mf >= s.M) return;
+    const int bf = mf / s.P, pf = mf - bf * s.P;
+    constexpr int EV = 16 / (int)sizeof(T);       // elements per 16-byte store
+    const bool fast = mf + PW <= s.M && pf + PW <= s.P && pf % EV == 0 && s.P % EV == 0;
+    if (fast) {
+#pragma unroll
+        for (int j = 0; j < kCV; j++) {
+            T *o = out + ((long)bf * s.Cout + c + j) * s.P + pf;
+            alignas(16) T e[PW];
+#pragma unroll
+            for (int i = 0; i < PW; i++) e[i] = f32_to_elem<T>(acc[i][j] + bv[j]);
+#pragma unroll
+            for (int q = 0; q < PW / EV; q++) reinterpret_cast<uint4 *>(o)[q] = reinterpret_cast<const uint4 *>(e)[q];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < PW; i++) {
+            const int m = mf + i;
+            if (m < s.M) {
+                const int b = m / s.P, pp = m - b * s.P;
+#pragma unroll
+                for (int j = 0; j < kCV; j++)
+                    out[((long)b * s.Cout + c + j) * s.P + pp] = f32_to_elem<T>(acc[i][j] + bv[j]);
             }
         }
     }
@@ -236,126 +262,120 @@ D2C_DEV float reduce4_over_wave(float v0, float v1, float v2, float v3, int lane
 template <typename T>
 __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
 {
-    constexpr int kTP = kBwdTP;
+    constexpr int TP = kBwdTP, KB = kBwdKB;
     extern __shared__ __align__(16) unsigned char smem[];
-    const DwTaps<kTP> taps = dw_taps<kTP>(smem, true);
-    float (*s_aux)[4] = taps.aux;   // goff z,y,x and gmask sums over the channels of the group
+    const DwTaps<TP, KB> taps = dw_taps<TP, KB>(smem, true);
     const TiledShape &s = a.s;
-    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * kTP;
-    const int HW = s.H * s.W;
     const int lane = threadIdx.x & 63;
-    const int nslice = (s.cpg + kDwThreads * kCV - 1) / (kDwThreads * kCV);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * TP;
+    const int HW = s.H * s.W;
+    const int nsl = (s.cpg + kSlice - 1) / kSlice;
+    const int g = blockIdx.y / nsl, sl = blockIdx.y - g * nsl;
+    const int cl = sl * kSlice + lane * kCV;
+    const bool cok = cl < s.cpg;       // lanes past the group still take part in the reductions
+    const int c = g * s.cpg + (cok ? cl : 0);
     const T *xcl = reinterpret_cast<const T *>(a.xcl);
     const T *wt = reinterpret_cast<const T *>(a.wt);
     const T *goutcl = reinterpret_cast<const T *>(a.goutcl);
-    const bool want_aux = a.goff != nullptr || a.gmask != nullptr;
+    const bool want_aux = a.auxoff != nullptr || a.auxmask != nullptr;
 
-    for (int g = 0; g < s.G; g++) {
-        for (int k0 = 0; k0 < s.K; k0 += kKB) {
-            const int kn = min(kKB, s.K - k0);
-            __syncthreads();
-            dw_coords<true, kTP>(a, taps, m0, g, k0, kn);
-            for (int e = threadIdx.x; e < kn * kTP; e += kDwThreads)
-                s_aux[e][0] = s_aux[e][1] = s_aux[e][2] = s_aux[e][3] = 0.f;
-            __syncthreads();
-            for (int sl = 0; sl < nslice; sl++) {
-                const int cl = (sl * kDwThreads + threadIdx.x) * kCV;
-                const bool cok = cl < s.cpg;       // lanes past the group still take part in the reductions
-                const int c = g * s.cpg + (cok ? cl : 0);
-                for (int kk = 0; kk < kn; kk++) {
-                    float wv[kCV] = {0.f, 0.f, 0.f, 0.f};
-                    if (cok) ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
-                    float gwv[kCV] = {0.f, 0.f, 0.f, 0.f};
-                    for (int p = 0; p < kTP; p++) {
-                        const int e = kk * kTP + p;
-                        // the table entry is the same for the whole workgroup: keep it in scalar registers
-                        const unsigned flag = (unsigned)__builtin_amdgcn_readfirstlane(taps.flag[e]);
-                        const unsigned inr = flag >> 8, live = flag & 0xffu;
-                        if (!inr) continue;
-                        const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
-                        const int m = m0 + p;                     // m < M holds where inr != 0
-                        float go[kCV] = {0.f, 0.f, 0.f, 0.f};
-                        if (cok) ld4<T>(goutcl + (long)m * s.Cout + c, go);
-                        float gc[kCV];
+    for (int k0 = 0; k0 < s.K; k0 += KB) {
+        const int kn = min(KB, s.K - k0);
+        __syncthreads();
+        dw_coords<true, TP, KB>(a, taps, m0, g, k0, kn);
+        __syncthreads();
+        for (int kk = wave; kk < kn; kk += kDwThreads / 64) {
+            float wv[kCV] = {0.f, 0.f, 0.f, 0.f};
+            if (cok) ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
+            float gwv[kCV] = {0.f, 0.f, 0.f, 0.f};
+            for (int p = 0; p < TP; p++) {
+                const int e = kk * TP + p;
+                // the table entry is the same for the whole wavefront: keep it in scalar registers
+                const unsigned flag = (unsigned)__builtin_amdgcn_readfirstlane(taps.flag[e]);
+                const unsigned inr = flag >> 8, live = flag & 0xffu;
+                if (!inr) continue;
+                const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
+                const int m = m0 + p;                     // m < M holds where inr != 0
+                float go[kCV] = {0.f, 0.f, 0.f, 0.f};
+                if (cok) ld4<T>(goutcl + (long)m * s.Cout + c, go);
+                float gc[kCV];
 #pragma unroll
-                        for (int j = 0; j < kCV; j++) gc[j] = wv[j] * go[j];
-                        float xv[8][kCV];
+                for (int j = 0; j < kCV; j++) gc[j] = wv[j] * go[j];
+                float xv[8][kCV];
 #pragma unroll
-                        for (int cc = 0; cc < 8; cc++) {
+                for (int cc = 0; cc < 8; cc++) {
+                    const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
+                    if (((inr >> cc) & 1u) && cok) {
+                        ld4<T>(xcl + (long)v * s.Cin + c, xv[cc]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < kCV; j++) xv[cc][j] = 0.f;
+                    }
+                }
+                float dot[8];
+                float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int cc = 0; cc < 8; cc++) {
+                    float d = 0.f;
+#pragma unroll
+                    for (int j = 0; j < kCV; j++) d = fmaf(gc[j], xv[cc][j], d);
+                    if ((live >> cc) & 1u) {
+                        const float wc = taps.w[cc][e];   // a_corner * alpha
+#pragma unroll
+                        for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, xv[cc][j], sv[j]);
+                        if (a.gxcl && cok) {
                             const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
-                            if (((inr >> cc) & 1u) && cok) {
-                                ld4<T>(xcl + (long)v * s.Cin + c, xv[cc]);
-                            } else {
+                            float *gp = a.gxcl + (long)v * s.Cin + c;
 #pragma unroll
-                                for (int j = 0; j < kCV; j++) xv[cc][j] = 0.f;
-                            }
-                        }
-                        float dot[8];
-                        float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                        for (int cc = 0; cc < 8; cc++) {
-                            float d = 0.f;
-#pragma unroll
-                            for (int j = 0; j < kCV; j++) d = fmaf(gc[j], xv[cc][j], d);
-                            if ((live >> cc) & 1u) {
-                                const float wc = taps.w[cc][e];   // a_corner * alpha
-#pragma unroll
-                                for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, xv[cc][j], sv[j]);
-                                if (a.gxcl && cok) {
-                                    const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
-                                    float *gp = a.gxcl + (long)v * s.Cin + c;
-#pragma unroll
-                                    for (int j = 0; j < kCV; j++) atomicAdd(gp + j, wc * gc[j]);
-                                }
-                            }
-                            dot[cc] = d;
-                        }
-#pragma unroll
-                        for (int j = 0; j < kCV; j++) gwv[j] = fmaf(go[j], sv[j], gwv[j]);   // sv already holds alpha
-                        if (want_aux) {
-                            const float lz = taps.frac[0][e], ly = taps.frac[1][e], lx = taps.frac[2][e];
-                            const float hz = taps.frac[3][e], hy = taps.frac[4][e], hx = taps.frac[5][e];
-                            float gz = 0.f, gy = 0.f, gxx = 0.f, gm = 0.f;
-#pragma unroll
-                            for (int cc = 0; cc < 8; cc++) {
-                                const float wz = (cc & 4) ? hz : lz, wy = (cc & 2) ? hy : ly, wx = (cc & 1) ? hx : lx;
-                                const float d = dot[cc];
-                                gz += ((cc & 4) ? d : -d) * (wy * wx);
-                                gy += ((cc & 2) ? d : -d) * (wz * wx);
-                                gxx += ((cc & 1) ? d : -d) * (wz * wy);
-                                if ((live >> cc) & 1u) gm += (wz * wy * wx) * d;
-                            }
-                            const float r = reduce4_over_wave(gz, gy, gxx, gm, lane);
-                            if ((lane & 15) == 0) atomicAdd(&s_aux[e][(lane >> 5) * 2 + ((lane >> 4) & 1)], r);
+                            for (int j = 0; j < kCV; j++) atomicAdd(gp + j, wc * gc[j]);
                         }
                     }
-                    if (a.gwacc && cok) {
-                        float *gw = a.gwacc + (long)(k0 + kk) * s.Cin + c;
+                    dot[cc] = d;
+                }
 #pragma unroll
-                        for (int j = 0; j < kCV; j++) atomicAdd(gw + j, gwv[j]);
+                for (int j = 0; j < kCV; j++) gwv[j] = fmaf(go[j], sv[j], gwv[j]);   // sv already holds alpha
+                if (want_aux) {
+                    const float lz = taps.frac[0][e], ly = taps.frac[1][e], lx = taps.frac[2][e];
+                    const float hz = taps.frac[3][e], hy = taps.frac[4][e], hx = taps.frac[5][e];
+                    float gz = 0.f, gy = 0.f, gxx = 0.f, gm = 0.f;
+#pragma unroll
+                    for (int cc = 0; cc < 8; cc++) {
+                        const float wz = (cc & 4) ? hz : lz, wy = (cc & 2) ? hy : ly, wx = (cc & 1) ? hx : lx;
+                        const float d = dot[cc];
+                        gz += ((cc & 4) ? d : -d) * (wy * wx);
+                        gy += ((cc & 2) ? d : -d) * (wz * wx);
+                        gxx += ((cc & 1) ? d : -d) * (wz * wy);
+                        if ((live >> cc) & 1u) gm += (wz * wy * wx) * d;
+                    }
+                    // sums over the 256 channels of the slice; the other slices of the group add theirs
+                    const float r = reduce4_over_wave(gz, gy, gxx, gm, lane);
+                    if ((lane & 15) == 0) {
+                        const int which = (lane >> 5) * 2 + ((lane >> 4) & 1);
+                        const int b = m / s.P, pp = m - b * s.P;
+                        const long ab = (((long)b * s.G + g) * s.K + (k0 + kk)) * s.P + pp;
+                        if (which < 3) {
+                            if (a.auxoff) atomicAdd(a.auxoff + 3 * ab - 2 * (long)pp + which * (long)s.P, taps.alpha[e] * r);
+                        } else if (a.auxmask) {
+                            atomicAdd(a.auxmask + ab, r);
+                        }
                     }
                 }
             }
-            __syncthreads();
-            if (want_aux) {
-                for (int e = threadIdx.x; e < kn * kTP; e += kDwThreads) {
-                    const int p = e % kTP, kk = e / kTP;
-                    const int m = m0 + p;
-                    if (m >= s.M) continue;
-                    const int b = m / s.P, pp = m - b * s.P;
-                    const int k = k0 + kk;
-                    const float al = taps.alpha[e];
-                    if (a.goff) {
-                        const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + pp;
-                        st_aux(a.goff, ob, s.adt, al * s_aux[e][0]);
-                        st_aux(a.goff, ob + s.P, s.adt, al * s_aux[e][1]);
-                        st_aux(a.goff, ob + 2 * (long)s.P, s.adt, al * s_aux[e][2]);
-                    }
-                    if (a.gmask) st_aux(a.gmask, (((long)b * s.G + g) * s.K + k) * s.P + pp, s.adt, s_aux[e][3]);
-                }
+            if (a.gwacc && cok) {
+                float *gw = a.gwacc + (long)(k0 + kk) * s.Cin + c;
+#pragma unroll
+                for (int j = 0; j < kCV; j++) atomicAdd(gw + j, gwv[j]);
             }
         }
     }
+}
+
+// fp32 accumulator -> offset / mask gradient in its storage type
+__global__ void __launch_bounds__(256) dw_aux_finish_kernel(const float *src, void *dst, int adt, long n)
+{
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        st_aux(dst, i, adt, src[i]);
 }
 
 // W[c][0][k] -> wt[k][c]
@@ -412,8 +432,9 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
                            (T *)wt, s.Cin, s.K);
     }
     DwArgs a{s, xcl, off, mask, wt, bias, out, nullptr, nullptr, nullptr, nullptr, nullptr};
+    const int nsl = (s.cpg + kSlice - 1) / kSlice;
     D2cProfScope prof(D2C_PROF_FWD, st);
-    hipLaunchKernelGGL(dw_fwd_kernel<T>, dim3((s.M + kFwdTP - 1) / kFwdTP), dim3(kDwThreads), kDwLdsFwd, st, a);
+    hipLaunchKernelGGL(dw_fwd_kernel<T>, dim3((s.M + kFwdTP - 1) / kFwdTP, s.G * nsl), dim3(kDwThreads), kDwLdsFwd, st, a);
     return d2c_check_launch("dw_fwd_kernel");
 }
 
@@ -421,25 +442,37 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
 // from the sample lists afterwards); otherwise it is accumulated with atomics.
 template <typename T>
 int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
-                           const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *gwacc, void *gw,
-                           hipStream_t st)
+                           const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc,
+                           void *gw, hipStream_t st)
 {
+    const long n_mask = (long)s.N * s.G * s.K * s.P, n_off = 3 * n_mask;
+    float *auxoff = goff ? auxacc : nullptr, *auxmask = gmask ? auxacc + n_off : nullptr;
     {
         D2cProfScope prof(D2C_PROF_PACK, st);
         hipLaunchKernelGGL(dw_pack_weight_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, (const T *)w,
                            (T *)wt, s.Cin, s.K);
         if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
         if (gwacc) d2c_fill_zero(gwacc, (size_t)s.Cin * s.K * sizeof(float), st);
+        if (goff || gmask) d2c_fill_zero(auxacc, (size_t)(n_off + n_mask) * sizeof(float), st);
     }
-    DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, goutcl, gxcl, goff, gmask, gwacc};
+    DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, goutcl, gxcl, auxoff, auxmask, gwacc};
+    const int nsl = (s.cpg + kSlice - 1) / kSlice;
     {
         D2cProfScope prof(D2C_PROF_BWD_DATA, st);
         if (hipFuncSetAttribute((const void *)dw_bwd_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)kDwLdsBwd) != hipSuccess)
             return d2c_check_launch("hipFuncSetAttribute(dw_bwd_kernel)");
-        hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3((s.M + kBwdTP - 1) / kBwdTP), dim3(kDwThreads), kDwLdsBwd, st, a);
+        hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3((s.M + kBwdTP - 1) / kBwdTP, s.G * nsl), dim3(kDwThreads), kDwLdsBwd, st,
+                           a);
     }
     if (int rc = d2c_check_launch("dw_bwd_kernel")) return rc;
+    if (goff || gmask) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        if (goff) hipLaunchKernelGGL(dw_aux_finish_kernel, dim3(g1d(n_off)), dim3(256), 0, st, auxoff, goff, s.adt, n_off);
+        if (gmask)
+            hipLaunchKernelGGL(dw_aux_finish_kernel, dim3(g1d(n_mask)), dim3(256), 0, st, auxmask, gmask, s.adt, n_mask);
+        if (int rc = d2c_check_launch("dw_aux_finish_kernel")) return rc;
+    }
     if (gwacc && gw) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         hipLaunchKernelGGL(dw_unpack_gw_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, gwacc, (T *)gw,
@@ -455,6 +488,6 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
                                           void *, const void *, void *, hipStream_t);                                \
     template int d2c_depthwise_backward<T>(const TiledShape &, const void *, const void *, const void *,             \
                                            const void *, const void *, void *, float *, void *, void *, float *,     \
-                                           void *, hipStream_t);
+                                           float *, void *, hipStream_t);
 INST(bf16_t)
 INST(float)

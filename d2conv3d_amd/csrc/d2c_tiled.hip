@@ -43,8 +43,8 @@ int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *
                            const void *entries, float *gxcl, hipStream_t st);
 template <typename T>
 int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
-                           const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *gwacc, void *gw,
-                           hipStream_t st);
+                           const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc,
+                           void *gw, hipStream_t st);
 
 namespace {
 
@@ -161,7 +161,7 @@ bool is_depthwise(const d2c_conv3d_desc &q)
 // depthwise workspace: channels-last input | weights [K][C] | grad_input accumulator | grad_weight accumulator |
 // channels-last grad_out | sample lists (counts, starts, block sums, entries)
 struct DwWs {
-    size_t xcl, wt, gxcl, gwacc, goutcl, counts, starts, bsums, entries, total_fwd, total_bwd;
+    size_t xcl, wt, gxcl, gwacc, auxacc, goutcl, counts, starts, bsums, entries, total_fwd, total_bwd;
 };
 DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -172,7 +172,8 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.total_fwd = w.wt + d2c_align_up((size_t)s.K * s.Cin * es);
     w.gxcl = w.total_fwd;
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
-    w.goutcl = w.gwacc + d2c_align_up((size_t)s.K * s.Cin * sizeof(float));
+    w.auxacc = w.gwacc + d2c_align_up((size_t)s.K * s.Cin * sizeof(float));
+    w.goutcl = w.auxacc + d2c_align_up((size_t)s.N * s.G * s.K * s.P * 4 * sizeof(float));
     w.counts = w.goutcl + d2c_align_up((size_t)s.N * s.P * s.Cout * es);
     size_t c, st, bs, en;
     d2c_invlist_ws(s, &c, &st, &bs, &en);
@@ -272,7 +273,8 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                     return rc;
             if (goff || gmask || gw || !lists)
                 if (int rc = d2c_depthwise_backward<T>(s, base + d.goutcl, base + d.xcl, off, mask, w, base + d.wt,
-                                                      lists ? nullptr : gxcl, goff, gmask, gwacc, gw, st))
+                                                      lists ? nullptr : gxcl, goff, gmask, (float *)(base + d.auxacc),
+                                                      gwacc, gw, st))
                     return rc;
             if (lists) {
                 if (!(goff || gmask || gw))

@@ -63,16 +63,18 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 
     extern __shared__ __align__(16) unsigned char smem[];
     const TiledShape &s = a.s;
-    const int wrs = a.ogk * (int)sizeof(T) + 16;        // weight tile row stride (bytes)
-    unsigned char *s_wt = smem;                          // [BKC][wrs]
-    unsigned char *s_gcol = s_wt + BKC * wrs;            // [MT][GRS]
+    // Weight tile [BKC][ogk], rows unpadded (a multiple of 128 bytes); the 16-byte pieces of row r are stored
+    // at position (piece ^ (r & 7)), which keeps the operand reads of 32 consecutive rows free of bank conflicts.
+    const int rowB = a.ogk * (int)sizeof(T);
+    unsigned char *s_wt = smem;                          // [BKC][rowB]
+    unsigned char *s_gcol = s_wt + BKC * rowB;           // [MT][GRS]
     float *s_w = reinterpret_cast<float *>(s_gcol + MT * GRS);   // [8][MT]  live corner weights * alpha
     float *s_frac = s_w + 8 * MT;                        // [6][MT]  lz ly lx hz hy hx
     float *s_alpha = s_frac + 6 * MT;                    // [MT]
     int *s_idx = reinterpret_cast<int *>(s_alpha + MT);  // [MT]
     int *s_flag = s_idx + MT;                            // [MT]     live | inrange << 8 | 1-D low-corner shift << 16 | mask-gradient corners << 24
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
     const int wg = blockIdx.y;
     const int m0 = tile * MT;
@@ -132,7 +134,22 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
         // last chunk of the group for this tap (or of this workgroup's share) -> flush goff / gmask
         const bool group_end = jj + 1 == cpc || st + 1 == st_hi;
 
-        // (a) coordinates of the step and the weight tile
+        // (a) weight tile of the step (asynchronous), then its coordinates
+        {
+            // global -> LDS without passing through registers: one instruction of a wavefront moves 64
+            // pieces to 1 KiB of consecutive LDS (lane i's piece lands at base + 16 i), so lane i fetches the
+            // piece that the swizzled layout wants there
+            const int rp = rowB / 16;                        // 16-byte pieces per weight row (a multiple of 8)
+            const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * rp;
+            const int ninstr = BKC * rp / 64;
+            for (int i = wave; i < ninstr; i += kThreads / 64) {
+                const int pos = i * 64 + lane;
+                const int row = pos / rp, q = pos - row * rp;
+                const uint4 *g = src + row * rp + (q ^ (row & 7));
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                                 (__attribute__((address_space(3))) void *)(s_wt + i * 1024), 16, 0, 0);
+            }
+        }
         if (tid < MT) {
             float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             float fr[6] = {0, 0, 0, 0, 0, 0};
@@ -177,14 +194,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
             s_idx[tid] = idx;
             s_flag[tid] = flag;
         }
-        {
-            const int row16 = a.ogk * (int)sizeof(T) / 16;   // 16-byte pieces per weight row
-            const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * row16;
-            for (int q = tid; q < BKC * row16; q += kThreads) {
-                const int row = q / row16, col = q - row * row16;
-                *reinterpret_cast<uint4 *>(s_wt + row * wrs + col * 16) = src[q];
-            }
-        }
+        __builtin_amdgcn_s_waitcnt(0);   // the weight-tile transfers of this wavefront have landed
         __syncthreads();
 
         // (b) gcol block of this wavefront: rows = positions, columns = channels
@@ -192,11 +202,13 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = 0.f;
         {
-            const unsigned char *wb = s_wt + (cb * 32 + (lane & 31)) * wrs + (lane >> 5) * 16;
+            const int wrow = cb * 32 + (lane & 31);
+            const unsigned char *wb = s_wt + wrow * rowB;
+            const int wsw = wrow & 7, wh = lane >> 5;
 #pragma unroll
             for (int kg = 0; kg < NKG; kg++) {
                 if (kg < nkg) {
-                    const uint4 bf = *reinterpret_cast<const uint4 *>(wb + kg * 32);
+                    const uint4 bf = *reinterpret_cast<const uint4 *>(wb + (((kg * 2 + wh) ^ wsw) << 4));
                     mma_kgroup<T>(acc, ga[kg], bf);
                 }
             }
@@ -351,7 +363,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 template <typename T> size_t bwd_data_lds(int ogk)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
-    return (size_t)BKC * (ogk * sizeof(T) + 16) + (size_t)MT * (BKC * 4 + 16) + (size_t)MT * (8 + 6 + 1 + 1 + 1) * 4;
+    return (size_t)BKC * ogk * sizeof(T) + (size_t)MT * (BKC * 4 + 16) + (size_t)MT * (8 + 6 + 1 + 1 + 1) * 4;
 }
 
 template <typename T, int NKG>
@@ -690,7 +702,8 @@ inline unsigned grid1d(long n, int cap = 8192)
 }  // namespace
 
 // ------------------------------------------------------------------ host
-int d2c_bwd_ogk(int og, int dtype) { const int kgw = dtype == D2C_BF16 ? 16 : 8; return (og + kgw - 1) / kgw * kgw; }
+// Output channels of a pass rounded up so that a row of the transposed weight tile is a multiple of 128 bytes.
+int d2c_bwd_ogk(int og, int dtype) { const int rw = dtype == D2C_BF16 ? 64 : 32; return (og + rw - 1) / rw * rw; }
 
 // Output channels one pass of the data kernel reduces over: 32 k-groups of the
 // stationary operand fit the register file (512 bf16 / 256 float channels).
