@@ -1,0 +1,104 @@
+"""GPU parity at the full sizes of the measured workloads (the tensors bench.py
+times, same seeds).
+
+Where the CPU oracle finishes in seconds to tens of seconds (C1, C2, C3, C4,
+C5a) the whole forward + backward is compared with it.  For every workload,
+C5b included, size-independent properties are checked as well:
+
+* zero offsets and unit mask reduce the operator to torch's stock convolution;
+* the forward pass is linear in the input, and grad_input / grad_weight are its
+  adjoints:  <op(x), g> = <x, grad_input(g)> = <w, grad_weight(g)> (bias excluded), evaluated at g = op(x);
+* grad_bias = sum of grad_out.
+
+float32: 1e-4 relative / 1e-5 absolute, scaled by the tensor's magnitude for
+the long sums.  bfloat16: 2e-2 relative (L2 over the tensor).
+"""
+import os
+import sys
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+import bench  # noqa: E402  (workload table and seeded input generator)
+import d2conv3d_amd as d2c  # noqa: E402
+from oracle import cpu  # noqa: E402
+from _util import assert_close, rel_l2  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def _tensors(name):
+    c = bench.WORKLOADS[name]
+    x, off, m, w, b, gout = bench.make_inputs(name, torch)
+    if c["dt"] == "bf16":
+        x, w, b, gout, off, m = (t.bfloat16() for t in (x, w, b, gout, off, m))
+    return c, x, off, m, w, b, gout
+
+
+def _run(c, dev, x, off, m, w, b, gout=None):
+    ts = [t.to(dev).requires_grad_(gout is not None) if t is not None else None for t in (x, off, m, w, b)]
+    fn = d2c.deform_conv3d if c["nd"] == 3 else d2c.deform_conv1d
+    out = fn(*ts, 1, 1, 1, c["groups"], c["G"])
+    if gout is None:
+        return out, None
+    out.backward(gout.to(dev))
+    return out.detach(), [t.grad if t is not None else None for t in ts]
+
+
+@pytest.mark.parametrize("name", ["c1", "c5a", "c4", "c2_f32", "c2_bf16", "c3"])
+def test_full_size_against_oracle(name, dev):
+    c, x, off, m, w, b, gout = _tensors(name)
+    f = lambda t: t.float()
+    fwd, bwd = (cpu.conv3d_forward, cpu.conv3d_backward) if c["nd"] == 3 else (cpu.conv1d_forward, cpu.conv1d_backward)
+    e_out = fwd(f(x), f(off), f(m), f(w), f(b), 1, 1, 1, c["groups"], c["G"])
+    out, grads = _run(c, dev, x, off, m, w, b, gout if c["backward"] else None)
+    names = ["grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias"]
+    pairs = [("out", out, e_out)]
+    if c["backward"]:
+        e = bwd(f(gout), f(x), f(off), f(m), f(w), True, 1, 1, 1, c["groups"], c["G"])
+        pairs += [(n, g, ee) for n, g, ee in zip(names, grads, e)]
+    for n, a, ee in pairs:
+        if c["dt"] == "f32":
+            scale = max(1.0, ee.abs().max().item())
+            assert_close(a, ee, 1e-4, 1e-5 * scale, f"{name} {n}")
+        else:
+            assert rel_l2(a, ee) < 2e-2, (name, n, rel_l2(a, ee))
+
+
+@pytest.mark.parametrize("name", ["c2_bf16", "c3", "c4", "c5a", "c5b"])
+def test_full_size_zero_offsets_equal_stock_convolution(name, dev):
+    c, x, off, m, w, b, _ = _tensors(name)
+    out, _ = _run(c, dev, x, torch.zeros_like(off), torch.ones_like(m), w, b)
+    conv = F.conv3d if c["nd"] == 3 else F.conv1d
+    ref = conv(x.to(dev).float(), w.to(dev).float(), b.to(dev).float(), 1, 1, 1, c["groups"])
+    if c["dt"] == "f32":
+        assert_close(out, ref, 1e-4, 1e-5 * max(1.0, ref.abs().max().item()), name)
+    else:
+        assert rel_l2(out, ref) < 1e-2, rel_l2(out, ref)
+
+
+@pytest.mark.parametrize("name", ["c3", "c4", "c5a", "c5b"])
+def test_full_size_linearity_and_adjoints(name, dev):
+    c, x, off, m, w, b, gout = _tensors(name)
+    tol = 2e-2 if c["dt"] == "bf16" else 2e-4
+    g = torch.Generator().manual_seed(7)
+    x2 = torch.randn(x.shape, generator=g).to(x.dtype)
+    o1, _ = _run(c, dev, x, off, m, w, None)
+    o2, _ = _run(c, dev, x2, off, m, w, None)
+    xs = (x.float() * 0.5 + x2.float()).to(x.dtype)        # exact in bfloat16 only up to rounding of the sum
+    o12, _ = _run(c, dev, xs, off, m, w, None)
+    assert rel_l2(o12.float(), 0.5 * o1.float() + o2.float()) < tol
+    # adjoints, with grad_out = op(x) so that the inner products are far from zero
+    go = o1.detach().cpu()
+    _, grads = _run(c, dev, x, off, m, w, b, go)
+    gx, _, _, gw, gb = grads
+    lhs = (o1.double() * o1.double()).sum().item()                      # <op(x), g>, bias excluded
+    via_x = (x.to(dev).double() * gx.double()).sum().item()
+    via_w = (w.to(dev).double() * gw.double()).sum().item()
+    atol = (2e-3 if c["dt"] == "bf16" else 2e-5) * abs(lhs)
+    assert abs(lhs - via_x) < atol, (lhs, via_x)
+    assert abs(lhs - via_w) < atol, (lhs, via_w)
+    e_gb = go.double().sum(dim=[0] + list(range(2, go.dim())))
+    assert rel_l2(gb, e_gb) < (1e-2 if c["dt"] == "bf16" else 1e-5)
