@@ -294,13 +294,29 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                                                   + ((c & 1) ? s.Cin : -qshift * s.Cin)) * (unsigned)sizeof(T);
                     xv[c] = ((inr >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + o) : make_uint4(0, 0, 0, 0);
                 }
+                if constexpr (sizeof(T) == 2) {
+                    // the grad-column values in the precision they are stored with (bfloat16 pairs), two
+                    // products per instruction, fp32 accumulation
+                    bf16x2_t gp[4];
 #pragma unroll
-                for (int c = 0; c < 8; c++) {
-                    const T *xe = reinterpret_cast<const T *>(&xv[c]);
-                    float d = 0.f;
+                    for (int e = 0; e < 4; e++)
+                        gp[e] = __builtin_bit_cast(bf16x2_t, pack_bf16x2(gc[2 * e], gc[2 * e + 1]));
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) d = fmaf(gc[e], elem_to_f32<T>(xe[e]), d);
-                    dot[c] = d;
+                    for (int c = 0; c < 8; c++) {
+                        float d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[c].x), gp[0], 0.f, false);
+                        d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[c].y), gp[1], d, false);
+                        d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[c].z), gp[2], d, false);
+                        dot[c] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[c].w), gp[3], d, false);
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 8; c++) {
+                        const T *xe = reinterpret_cast<const T *>(&xv[c]);
+                        float d = 0.f;
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) d = fmaf(gc[e], elem_to_f32<T>(xe[e]), d);
+                        dot[c] = d;
+                    }
                 }
                 // sum over the 8 lanes that share the position
 #pragma unroll
