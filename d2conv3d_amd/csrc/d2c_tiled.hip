@@ -4,7 +4,7 @@
 #include "d2c_tiled.hpp"
 #include "d2c_mma.hpp"
 
-int d2c_fwd_out_tile(int og, int M);
+int d2c_fwd_out_tile(int og, int M, int groups);
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
                          const void *bias, void *out, float *outacc, hipStream_t st);
@@ -73,7 +73,7 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0)
     s.nchunk = s.cg / bkc_of(q.dtype);
     s.adt = q.aux_dtype;
     s.P = q.Do * q.Ho * q.Wo; s.vol = q.D * q.H * q.W; s.M = q.N * s.P;
-    const int nt = d2c_fwd_out_tile(s.og, s.M);
+    const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
     s.ogp = (s.og + nt - 1) / nt * nt;
     s.geo = make_geom(q);
     return s;
@@ -135,7 +135,7 @@ FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     const size_t es = d2c_elem_size(q.dtype);
     FwdWs w;
     w.xcl = 0;
-    w.wp = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
+    w.wp = d2c_align_up((size_t)s.N * s.vol * s.Cin * es + 256);   // input, then a 256-byte row of zeros
     w.outacc = w.wp + d2c_align_up((size_t)s.groups * s.nchunk * s.K * s.ogp * bkc_of(q.dtype) * es);
     // fp32 partial sums of the output, used only when the forward kernel splits its steps
     w.total = w.outacc;
@@ -197,6 +197,10 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
     }
     const FwdWs l = fwd_ws(q, s);
     if (int rc = pack_input<T>(s, x, base + l.xcl, st)) return rc;
+    {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(base + l.xcl + (size_t)s.N * s.vol * s.Cin * sizeof(T), 256, st);   // what dead corners read
+    }
     const long total = (long)s.groups * s.nchunk * s.K * (s.ogp / 32) * 4 * 64;
     long g = (total + 255) / 256;
     if (g > 8192) g = 8192;
@@ -337,7 +341,7 @@ static bool mfma_channels_ok(const d2c_conv3d_desc &q)
 {
     if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
     // the tiled kernels address the channels-last input with 32-bit byte offsets
-    if ((size_t)q.N * q.Cin * q.D * q.H * q.W * d2c_elem_size(q.dtype) >= (1ull << 32)) return false;
+    if ((size_t)q.N * q.Cin * q.D * q.H * q.W * d2c_elem_size(q.dtype) + 256 >= (1ull << 32)) return false;
     const int bkc = bkc_of(q.dtype);
     const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
     return cg % bkc == 0 && cpg % bkc == 0;

@@ -25,6 +25,9 @@ SHAPES = {
     "c64_o600": (1, 64, 600, (2, 5, 5), (1, 3, 3), 1, (0, 1, 1), 1, 1, 1, True, True, 1.0),
     "c64_stride_dil": (2, 64, 64, (5, 9, 8), 3, (1, 2, 1), (1, 2, 2), (1, 2, 1), 1, 1, True, True, 1.0),
     "c64_tail": (3, 64, 32, (3, 7, 7), 3, 1, 1, 1, 1, 1, True, True, 1.0),   # N*P = 441: ragged last tile
+    # wide weight groups with many position tiles: the forward kernel that moves corner rows by DMA
+    "c64_o320_big": (1, 64, 320, (7, 35, 34), 3, 1, 1, 1, 1, 1, True, True, 1.5),       # N*P = 8330: ragged
+    "c128_groups2_o640_big": (1, 128, 640, (4, 32, 33), 3, 1, 1, 1, 2, 2, True, True, 2.0),
     # channel-separated (groups == Cin == Cout)
     "dw64": (2, 64, 64, (4, 6, 7), 3, 1, 1, 1, 64, 1, True, True, 1.5),
     "dw96_G3_nomask": (1, 96, 96, (3, 5, 9), 3, 1, 1, 1, 96, 3, False, False, 1.0),
