@@ -461,8 +461,8 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
         for (int it = st_lo; it < st_hi; it++) {
             __builtin_amdgcn_s_waitcnt(0);     // the transfers requested in the last iteration have landed
             __syncthreads();
-            if (it + 2 < st_hi) dma_issue(it + 2, it & 1, (it + 2) % 3);
             mma_step(it, it & 1);
+            if (it + 2 < st_hi) dma_issue(it + 2, it & 1, (it + 2) % 3);
             if (it + 1 < st_hi) interp_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
         }
     } else {
