@@ -164,9 +164,12 @@ gx_owner_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *
     // their lists form one contiguous range: 4 ranges per voxel, walked 4 entries at a time with all
     // loads of a batch issued before their first use (entries past the end repeat the last one with
     // weight 0).
+    // Order of the 4 ranges: by the parity of the base voxel's (z, y), so that the voxels that share a list
+    // (4 in z/y, and their x-neighbours) all walk it in the same quarter of the kernel, while its
+    // grad-column rows are still in the caches.
 #pragma unroll 1
-    for (int d = 0; d < 4; d++) {
-        const int dz = (d >> 1) & 1, dy = d & 1;
+    for (int t = 0; t < 4; t++) {
+        const int dz = (z ^ (t >> 1)) & 1, dy = (y ^ t) & 1;
         const int bin1 = bin_of(s, b, g, z - dz, y - dy, x - 1);   // dx = 1
         const int e0 = starts[bin1], em = starts[bin1 + 1], e1 = starts[bin1 + 2];
         for (int e = e0; e < e1; e += 4) {
@@ -261,8 +264,9 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
 #pragma unroll
             for (int j = 0; j < kOwnCV; j++) acc[j] = 0.f;
 #pragma unroll 1
-            for (int d = 0; d < 4; d++) {
-                const int dz = (d >> 1) & 1, dy = d & 1;
+            for (int t4 = 0; t4 < 4; t4++) {
+                // ranges ordered by the parity of the base voxel's (z, y): see gx_owner_kernel
+                const int dz = (z ^ (t4 >> 1)) & 1, dy = (y ^ t4) & 1;
                 const int bin1 = bin_of(s, b, g, z - dz, y - dy, x - 1);   // lists of base voxels x-1 and x are adjacent
                 const int e0 = starts[bin1], em = starts[bin1 + 1], e1 = starts[bin1 + 2];
                 for (int e = e0; e < e1; e += 4) {
