@@ -1,0 +1,272 @@
+// grad_offset / grad_mask from the grad-column rows (dconv3d_gpu.cu:708-864,
+// dconv1d_gpu.cu:318-352), as a kernel of its own.
+//
+//   dot[corner]  = sum_c gcol[p, k, c] * x[corner(p, k), c]          (c over the channels of the offset group)
+//   grad_mask    = sum_corner a_corner * dot[corner]                 (corners of the forward pass)
+//   grad_offset  = alpha * sum_corner (d a_corner / d axis) * dot[corner]   (corners gated by range only)
+//
+// The data kernel writes the grad-column rows [chunk][tap][N*P][BKC] anyway (the
+// list-based grad_input reads them).  Doing the dot products here instead of
+// inside that kernel frees them from its register budget (its stationary
+// operand fills the register file) and from its barriers: here every wavefront
+// works alone (no workgroup synchronisation at all), needs few registers, and
+// twenty of them per CU hide each other's memory latency.
+//
+// One wavefront = 64 output positions of one offset group and a share of the
+// taps.  Per tap: lane = position computes the corner table of the 64 positions
+// into a private LDS patch; then, per channel chunk of the group, 8 rounds of
+// lane = (position, 16-byte vector): 8 corner vectors + 1 grad-column vector ->
+// 8 dot products -> the 4 results (linear in the dots) -> sum over the 8 lanes
+// of the position.
+#include "d2c_mma.hpp"
+#include "d2c_tiled.hpp"
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kMT = 64;                    // positions per wavefront
+constexpr int kTab = 9;                    // table words per position: idx, flag, lz ly lx hz hy hx, alpha
+constexpr int kRounds = 1;                 // rounds whose loads are in flight together
+constexpr int kTapSplit = 9;               // wavefronts per (tile, group), each with its share of the taps (many short
+                                           // tasks balance better than few long ones: 0.49 ms against 0.59 ms at 1)
+
+D2C_DEV int xcd_swizzle(int bid, int n)
+{
+    const int x = bid & 7, idx = bid >> 3;
+    const int q = n >> 3, r = n & 7;
+    return x * q + (x < r ? x : r) + idx;
+}
+
+struct AuxArgs {
+    TiledShape s;
+    const void *xcl;     // [N][vol][Cin]
+    const void *off, *mask;
+    const void *gcol;    // [chunk][tap][N*P][BKC]
+    void *goff, *gmask;  // or NULL
+    int ntile;           // position tiles
+};
+
+template <typename T, bool AUX16>
+__global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a)
+{
+    constexpr int MT = kMT;
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
+    __shared__ float s_tab_all[kWavesPerBlock][kTab][MT];
+
+    const TiledShape &s = a.s;
+    const int lane = threadIdx.x & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float (*s_tab)[MT] = s_tab_all[wib];
+    // wavefront task = (tile, offset group, tap share); tiles that are neighbours in space share an XCD
+    const int tile = xcd_swizzle(blockIdx.x, gridDim.x) * kWavesPerBlock + wib;
+    if (tile >= a.ntile) return;
+    const int g = blockIdx.y;
+    const int k_lo = (int)((long)s.K * blockIdx.z / gridDim.z), k_hi = (int)((long)s.K * (blockIdx.z + 1) / gridDim.z);
+    const int m0 = tile * MT;
+    const int cpc = s.cpg / BKC;                   // chunks per offset group
+    const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;
+
+    // lane = position (coordinate role)
+    int cb = 0, cp = 0, coz = 0, coy = 0, cox = 0;
+    const bool cvalid = m0 + lane < s.M;
+    if (cvalid) {
+        const int m = m0 + lane;
+        cb = m / s.P; cp = m - cb * s.P;
+        cox = cp % s.Wo; coy = (cp / s.Wo) % s.Ho; coz = cp / (s.Wo * s.Ho);
+    }
+    // lane = (position of the round, vector) (dot-product role)
+    const int rpos = lane >> 3, ivec = lane & 7;
+    const char *xb = reinterpret_cast<const char *>(a.xcl);
+    const char *gcb = reinterpret_cast<const char *>(a.gcol);
+
+    // offsets and modulation of a tap are requested while the previous tap is being worked on
+    float craw[4] = {0.f, 0.f, 0.f, 1.f};
+    auto coords_issue = [&](int k) {
+        if (cvalid) {
+            const long ab = (((long)cb * s.G + g) * s.K + k) * s.P + cp;
+            if (s.nd == 3) {
+                const long ob = 3 * ab - 2 * (long)cp;
+                craw[0] = ld_auxT<AUX16>(a.off, ob);
+                craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
+                craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
+            } else {
+                craw[2] = ld_auxT<AUX16>(a.off, ab);
+            }
+            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
+        }
+    };
+    if (k_lo < k_hi) coords_issue(k_lo);
+
+    for (int k = k_lo; k < k_hi; k++) {
+        // ---- corner table of the 64 positions for tap k
+        {
+            float fr[6] = {0, 0, 0, 0, 0, 0};
+            float al = 0.f;
+            int idx = 0, flag = 0;
+            if (cvalid) {
+                const float o0 = craw[0], o1 = craw[1], o2 = craw[2];
+                al = craw[3];
+                int bz, by, bx;
+                tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
+                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+                idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
+                unsigned inr = t.inrange, auxlive = t.live;
+                fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
+                if (s.nd == 1) {
+                    // 1-D: both corners are gated by range only (dconv1d_gpu.cu:338-339), and at integer
+                    // positions the low corner steps down by one while the high corner stays (:332-336);
+                    // grad_offset / grad_mask then interpolate with t' = x - (x0 - 1).
+                    int x0q = t.x0;
+                    if (s.quirks && (double)t.hx < 1e-8) {
+                        x0q -= 1;
+                        flag |= 1 << 16;
+                        const float x = (float)bx + o2;
+                        const float tq = x - (float)x0q;
+                        fr[2] = 1.f - tq; fr[5] = tq;
+                    }
+                    const unsigned lo = (x0q >= 0 && x0q < s.W) ? 1u : 0u;
+                    const unsigned hi = (t.x0 + 1 >= 0 && t.x0 + 1 < s.W) ? 2u : 0u;
+                    inr = lo | hi;
+                    auxlive = inr;
+                }
+                flag |= (int)((inr << 8) | (auxlive << 24));
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the reads of the previous tap are done
+            __builtin_amdgcn_wave_barrier();
+            s_tab[0][lane] = __int_as_float(idx);
+            s_tab[1][lane] = __int_as_float(flag);
+#pragma unroll
+            for (int c = 0; c < 6; c++) s_tab[2 + c][lane] = fr[c];
+            s_tab[8][lane] = al;
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            if (k + 1 < k_hi) coords_issue(k + 1);
+        }
+
+        // ---- dot products: 8 rounds of 8 positions x 8 vectors, kRounds at a time; sums over the chunks of the group
+#pragma unroll 1
+        for (int rp = 0; rp < 8 / kRounds; rp++) {
+            float g_acc[kRounds][4];
+#pragma unroll
+            for (int r = 0; r < kRounds; r++) g_acc[r][0] = g_acc[r][1] = g_acc[r][2] = g_acc[r][3] = 0.f;
+#pragma unroll 1
+            for (int jj = 0; jj < cpc; jj++) {
+                const int c0 = g * s.cpg + jj * BKC;
+                const long grow = ((long)(c0 / BKC) * s.K + k) * s.M;
+                uint4 xv[kRounds][8], gq[kRounds];
+                // all loads of these rounds are requested before any of them is used
+#pragma unroll
+                for (int r = 0; r < kRounds; r++) {
+                    const int pos = (rp * kRounds + r) * 8 + rpos;
+                    const int idx = __float_as_int(s_tab[0][pos]);
+                    const unsigned flag = (unsigned)__float_as_int(s_tab[1][pos]);
+                    const unsigned inr = (flag >> 8) & 0xffu;
+                    const int qshift = (flag >> 16) & 1;
+                    const int ib = idx + c0 + ivec * VEC;
+#pragma unroll
+                    for (int c = 0; c < 8; c++) {
+                        const unsigned o = (unsigned)(ib + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc
+                                                      + ((c & 1) ? s.Cin : -qshift * s.Cin)) * (unsigned)sizeof(T);
+                        xv[r][c] = ((inr >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + o) : make_uint4(0, 0, 0, 0);
+                    }
+                    const int m = m0 + pos;
+                    gq[r] = inr ? *reinterpret_cast<const uint4 *>(gcb + ((grow + m) * BKC + ivec * VEC) * (long)sizeof(T))
+                                : make_uint4(0, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < kRounds; r++) {
+                    const int pos = (rp * kRounds + r) * 8 + rpos;
+                    const unsigned live = (unsigned)__float_as_int(s_tab[1][pos]) >> 24;
+                    float dot[8];
+                    if constexpr (sizeof(T) == 2) {
+                        const bf16x2_t g0 = __builtin_bit_cast(bf16x2_t, gq[r].x), g1 = __builtin_bit_cast(bf16x2_t, gq[r].y);
+                        const bf16x2_t g2 = __builtin_bit_cast(bf16x2_t, gq[r].z), g3 = __builtin_bit_cast(bf16x2_t, gq[r].w);
+#pragma unroll
+                        for (int c = 0; c < 8; c++) {
+                            float d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[r][c].x), g0, 0.f, false);
+                            d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[r][c].y), g1, d, false);
+                            d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[r][c].z), g2, d, false);
+                            dot[c] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, xv[r][c].w), g3, d, false);
+                        }
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < 8; c++) {
+                            float d = __uint_as_float(gq[r].x) * __uint_as_float(xv[r][c].x);
+                            d = fmaf(__uint_as_float(gq[r].y), __uint_as_float(xv[r][c].y), d);
+                            d = fmaf(__uint_as_float(gq[r].z), __uint_as_float(xv[r][c].z), d);
+                            dot[c] = fmaf(__uint_as_float(gq[r].w), __uint_as_float(xv[r][c].w), d);
+                        }
+                    }
+                    // the four results are linear in the 8 dots: combine per lane, then sum over the 8 lanes
+                    const float lz = s_tab[2][pos], ly = s_tab[3][pos], lx = s_tab[4][pos];
+                    const float hz = s_tab[5][pos], hy = s_tab[6][pos], hx = s_tab[7][pos];
+                    float gz = 0.f, gy = 0.f, gxx = 0.f, gm = 0.f;
+#pragma unroll
+                    for (int c = 0; c < 8; c++) {
+                        const float wz = (c & 4) ? hz : lz, wy = (c & 2) ? hy : ly, wx = (c & 1) ? hx : lx;
+                        const float d = dot[c];
+                        gz += ((c & 4) ? d : -d) * (wy * wx);
+                        gy += ((c & 2) ? d : -d) * (wz * wx);
+                        gxx += ((c & 1) ? d : -d) * (wz * wy);
+                        if ((live >> c) & 1u) gm += (wz * wy * wx) * d;
+                    }
+#pragma unroll
+                    for (int sft = 1; sft < 8; sft <<= 1) {
+                        gz += __shfl_xor(gz, sft, 64);
+                        gy += __shfl_xor(gy, sft, 64);
+                        gxx += __shfl_xor(gxx, sft, 64);
+                        gm += __shfl_xor(gm, sft, 64);
+                    }
+                    g_acc[r][0] += gz; g_acc[r][1] += gy; g_acc[r][2] += gxx; g_acc[r][3] += gm;
+                }
+            }
+            // ---- results of tap k for the positions of these rounds
+            if (ivec == 0) {
+#pragma unroll
+                for (int r = 0; r < kRounds; r++) {
+                    const int pos = (rp * kRounds + r) * 8 + rpos;
+                    const int m = m0 + pos;
+                    if (m < s.M) {
+                        const float al = s_tab[8][pos];
+                        const int b = m / s.P, p = m - b * s.P;
+                        const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
+                        if (a.goff && s.nd == 3) {
+                            const long ob = 3 * ab - 2 * (long)p;
+                            st_aux(a.goff, ob, s.adt, al * g_acc[r][0]);
+                            st_aux(a.goff, ob + s.P, s.adt, al * g_acc[r][1]);
+                            st_aux(a.goff, ob + 2 * (long)s.P, s.adt, al * g_acc[r][2]);
+                        } else if (a.goff) {
+                            st_aux(a.goff, ab, s.adt, al * g_acc[r][2]);
+                        }
+                        if (a.gmask) st_aux(a.gmask, ab, s.adt, g_acc[r][3]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace
+
+// grad_offset / grad_mask of the whole problem from the grad-column rows.  Needs offset groups whose
+// channel count is a multiple of the chunk width.
+template <typename T>
+int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
+                        void *goff, void *gmask, hipStream_t st)
+{
+    const int ntile = (s.M + kMT - 1) / kMT;
+    AuxArgs a{s, xcl, off, mask, gcol, goff, gmask, ntile};
+    dim3 grid((ntile + kWavesPerBlock - 1) / kWavesPerBlock, s.G, s.K < kTapSplit ? s.K : kTapSplit);
+    bool aux16 = false;
+    if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
+    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
+    if constexpr (sizeof(T) == 2) {
+        if (aux16) hipLaunchKernelGGL((aux_grad_kernel<T, true>), grid, dim3(64 * kWavesPerBlock), 0, st, a);
+    }
+    if (!aux16) hipLaunchKernelGGL((aux_grad_kernel<T, false>), grid, dim3(64 * kWavesPerBlock), 0, st, a);
+    return d2c_check_launch("aux_grad_kernel");
+}
+template int d2c_aux_grad_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
+                                         void *, void *, hipStream_t);
+template int d2c_aux_grad_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
+                                        void *, void *, hipStream_t);

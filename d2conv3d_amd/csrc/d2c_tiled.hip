@@ -28,6 +28,9 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts
                         hipStream_t st);
 int d2c_gx_mode();
 template <typename T>
+int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
+                        void *goff, void *gmask, hipStream_t st);
+template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                                 const void *mask, float *gwacc, void *gw, hipStream_t st);
 template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
@@ -220,6 +223,14 @@ bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
     return d2c_gx_mode() == 1 && d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
 }
 
+// grad_offset / grad_mask by the kernel of d2c_aux_grad.hip (from the grad-column rows): when the data kernel
+// makes whole rows in one pass and does not split its steps.
+bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    return d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype)
+           && d2c_bwd_data_split(s, q.dtype) == 1;
+}
+
 struct BwdWs {
     size_t xcl, wt, gxcl, gwacc, auxacc, gcol, counts, starts, bsums, entries, total;
 };
@@ -239,11 +250,14 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     if (d2c_bwd_data_split(s, q.dtype) > 1)
         w.total += d2c_align_up((size_t)s.N * s.G * s.K * s.P * (s.nd + 1) * sizeof(float));
     w.gcol = w.counts = w.starts = w.bsums = w.entries = 0;
+    if (use_lists(q, s) || use_aux_kernel(q, s)) {
+        w.gcol = w.total;
+        w.total = w.gcol + d2c_align_up((size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M * bkc_of(q.dtype) * es);
+    }
     if (use_lists(q, s)) {
         size_t c, st, bs, en;
         d2c_invlist_ws(s, &c, &st, &bs, &en);
-        w.gcol = w.total;
-        w.counts = w.gcol + d2c_align_up((size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M * bkc_of(q.dtype) * es);
+        w.counts = w.total;
         w.starts = w.counts + c;
         w.bsums = w.starts + st;
         w.entries = w.bsums + bs;
@@ -299,14 +313,19 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
             const bool lists = gx && use_lists(q, s);
+            const bool auxk = (goff || gmask) && use_aux_kernel(q, s);
             if (lists)
                 if (int rc = d2c_invlist_build(s, off, mask, (int *)(base + l.counts), (int *)(base + l.starts),
                                                (int *)(base + l.bsums), base + l.entries, st))
                     return rc;
             if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt,
-                                                     lists ? nullptr : gxcl, lists ? base + l.gcol : nullptr, goff,
-                                                     gmask, (float *)(base + l.auxacc), st))
+                                                     lists ? nullptr : gxcl, (lists || auxk) ? base + l.gcol : nullptr,
+                                                     auxk ? nullptr : goff, auxk ? nullptr : gmask,
+                                                     (float *)(base + l.auxacc), st))
                 return rc;
+            if (auxk)
+                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff, gmask, st))
+                    return rc;
             if (lists)
                 if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, (const int *)(base + l.starts), base + l.entries,
                                                     gxcl, st))

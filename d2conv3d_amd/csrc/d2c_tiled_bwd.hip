@@ -150,7 +150,9 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                                                  (__attribute__((address_space(3))) void *)(s_wt + i * 1024), 16, 0, 0);
             }
         }
-        if (tid < MT) {
+        // (nobody reads the corner table when grad_input comes from the sample lists and the offset / mask
+        // gradient from the kernel of d2c_aux_grad.hip)
+        if (tid < MT && (a.gxcl != nullptr || want_aux)) {
             float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             float fr[6] = {0, 0, 0, 0, 0, 0};
             float al = 0.f;
