@@ -417,10 +417,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
     constexpr int CB = BKC / 32;
     constexpr int OB = 2;                      // 32-row blocks of output channels per wavefront
     constexpr int NT = 64 * 8;                 // output channels per workgroup
-    constexpr int CPI = sizeof(T) == 2 ? 2 : 1;  // channels per gather item (one 4-byte load)
     constexpr int TRS = kWMT * (int)sizeof(T) + 16;   // tile row stride: [channel][position]
-    constexpr int NOCT = kWMT / VEC;           // position groups per tile
-    constexpr int NITEM = NOCT * (BKC / CPI);  // gather items per tile
+    constexpr int NITEM = kWMT * 8;            // gather items per tile: (position, 16-byte channel vector)
     constexpr int ITEMS = NITEM / kThreads;
     static_assert(ITEMS * kThreads == NITEM, "gather items divide evenly");
 
@@ -480,62 +478,52 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
         }
     };
 
-    // sample: one item = CPI channels x VEC consecutive positions; 32 lanes read one 128-byte row
-    uint32_t u[ITEMS][VEC][8];
+    // sample: one item = one position x one 16-byte vector of channels (8 lanes read one 128-byte corner row)
+    uint4 gv[ITEMS][8];
     auto gather_issue = [&](int buf) {
+        const char *xb = reinterpret_cast<const char *>(a.xcl);
 #pragma unroll
         for (int it = 0; it < ITEMS; it++) {
             const int item = tid + it * kThreads;
-            const int cpi = item % (BKC / CPI), oct = item / (BKC / CPI);
-            const char *xb = reinterpret_cast<const char *>(a.xcl);
+            const int pos = item >> 3, vec = item & 7;
+            const int idx = s_idx[buf][pos] + c0 + vec * VEC;
+            const unsigned live = (unsigned)s_flag[buf][pos];
 #pragma unroll
-            for (int q = 0; q < VEC; q++) {
-                const int pos = oct * VEC + q;
-                const int idx = s_idx[buf][pos] + c0 + cpi * CPI;
-                const unsigned live = (unsigned)s_flag[buf][pos];
-#pragma unroll
-                for (int c = 0; c < 8; c++) {
-                    const unsigned o = (unsigned)(idx + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc + (c & 1) * s.Cin)
-                                       * (unsigned)sizeof(T);
-                    u[it][q][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint32_t *>(xb + o) : 0u;
-                }
+            for (int c = 0; c < 8; c++) {
+                const unsigned o = (unsigned)(idx + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc + (c & 1) * s.Cin)
+                                   * (unsigned)sizeof(T);
+                gv[it][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + o) : make_uint4(0, 0, 0, 0);
             }
         }
     };
+    // interpolate, then store transposed ([channel][position]: the operand order of a reduction over
+    // positions).  bfloat16: the lanes of positions p and p^1 (8 lanes apart) swap values so that each
+    // writes whole 4-byte pairs of positions.
     auto interp_store = [&](int cbuf, int tbuf) {
 #pragma unroll
         for (int it = 0; it < ITEMS; it++) {
             const int item = tid + it * kThreads;
-            const int cpi = item % (BKC / CPI), oct = item / (BKC / CPI);
-            float r0[VEC], r1[VEC];
+            const int pos = item >> 3, vec = item & 7;
+            VecAcc<T> acc;
+            acc.zero();
 #pragma unroll
-            for (int q = 0; q < VEC; q++) {
-                const int pos = oct * VEC + q;
-                float v0 = 0.f, v1 = 0.f;
+            for (int c = 0; c < 8; c++) acc.fma(s_w[cbuf][c][pos], gv[it][c]);
+            unsigned char *tb = &s_tile[tbuf][(vec * VEC) * TRS];
+            if constexpr (sizeof(T) == 2) {
+                const int odd = pos & 1;
 #pragma unroll
-                for (int c = 0; c < 8; c++) {
-                    const float wc = s_w[cbuf][c][pos];
-                    const uint32_t uc = u[it][q][c];
-                    if constexpr (sizeof(T) == 2) {
-                        v0 = fmaf(wc, __uint_as_float(uc << 16), v0);
-                        v1 = fmaf(wc, __uint_as_float(uc & 0xffff0000u), v1);
-                    } else {
-                        v0 = fmaf(wc, __uint_as_float(uc), v0);
+                for (int e = 0; e < VEC; e++) {
+                    const float other = __shfl_xor(acc.a[e], 8, 64);     // same channel, position pos ^ 1
+                    if ((e & 1) == odd) {
+                        const uint32_t pr = odd ? pack_bf16x2(other, acc.a[e]) : pack_bf16x2(acc.a[e], other);
+                        // 16-byte chunks of a row are XOR-swizzled by its 8-channel group: the 8 vectors of a
+                        // position pair would otherwise all hit the same banks (rows 8 apart alias)
+                        *reinterpret_cast<uint32_t *>(tb + e * TRS + ((((pos >> 1) ^ (vec << 2))) << 2)) = pr;
                     }
                 }
-                r0[q] = v0; r1[q] = v1;
-            }
-            if constexpr (sizeof(T) == 2) {
-                uint4 p0 = make_uint4(pack_bf16x2(r0[0], r0[1]), pack_bf16x2(r0[2], r0[3]),
-                                      pack_bf16x2(r0[4], r0[5]), pack_bf16x2(r0[6], r0[7]));
-                uint4 p1 = make_uint4(pack_bf16x2(r1[0], r1[1]), pack_bf16x2(r1[2], r1[3]),
-                                      pack_bf16x2(r1[4], r1[5]), pack_bf16x2(r1[6], r1[7]));
-                *reinterpret_cast<uint4 *>(&s_tile[tbuf][(cpi * 2) * TRS + oct * 16]) = p0;
-                *reinterpret_cast<uint4 *>(&s_tile[tbuf][(cpi * 2 + 1) * TRS + oct * 16]) = p1;
             } else {
-                *reinterpret_cast<uint4 *>(&s_tile[tbuf][cpi * TRS + oct * 16]) =
-                    make_uint4(__float_as_uint(r0[0]), __float_as_uint(r0[1]), __float_as_uint(r0[2]),
-                               __float_as_uint(r0[3]));
+#pragma unroll
+                for (int e = 0; e < VEC; e++) *reinterpret_cast<float *>(tb + e * TRS + pos * 4) = acc.a[e];
             }
         }
     };
@@ -588,7 +576,11 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
                     af[ob] = *reinterpret_cast<const uint4 *>(stg + (ob * 32 + (lane & 31)) * SRS + (kq * 2 + (lane >> 5)) * 16);
 #pragma unroll
                 for (int cb = 0; cb < CB; cb++)
-                    bf[cb] = *reinterpret_cast<const uint4 *>(&s_tile[tbuf][(cb * 32 + (lane & 31)) * TRS + (kg * 2 + (lane >> 5)) * 16]);
+                {
+                    const int row = cb * 32 + (lane & 31);
+                    const int swz = sizeof(T) == 2 ? ((row >> 3) & 7) : 0;   // see interp_store
+                    bf[cb] = *reinterpret_cast<const uint4 *>(&s_tile[tbuf][row * TRS + (((kg * 2 + (lane >> 5)) ^ swz) << 4)]);
+                }
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++)
 #pragma unroll
