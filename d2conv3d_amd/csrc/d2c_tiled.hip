@@ -32,7 +32,8 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
                         void *goff, void *gmask, hipStream_t st);
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                                const void *mask, float *gwacc, void *gw, hipStream_t st);
+                                const void *mask, void *goutp, float *gwacc, void *gw, hipStream_t st);
+size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype);
 template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
 template <typename T> int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st);
 
@@ -232,7 +233,7 @@ bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 struct BwdWs {
-    size_t xcl, wt, gxcl, gwacc, auxacc, gcol, counts, starts, bsums, entries, total;
+    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, starts, bsums, entries, total;
 };
 BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -244,7 +245,8 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     const int ogk = d2c_bwd_ogk(s.og < omax ? s.og : omax, q.dtype);
     w.gxcl = w.wt + d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * ogk * es);
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
-    w.auxacc = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
+    w.goutp = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
+    w.auxacc = w.goutp + d2c_align_up(d2c_bwd_goutp_bytes(s, q.dtype));
     // fp32 scratch of the offset / mask gradient, used only when the data kernel splits its steps
     w.total = w.auxacc;
     if (d2c_bwd_data_split(s, q.dtype) > 1)
@@ -341,7 +343,8 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
     }
     if (gw) {
         if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
-            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, (float *)(base + l.gwacc),
+            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+                                                       (float *)(base + l.gwacc),
                                                        gw, st))
                 return rc;
         } else {

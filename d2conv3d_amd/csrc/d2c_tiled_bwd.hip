@@ -402,6 +402,7 @@ int launch_bwd_data(const BwdDataArgs &a, int nsplit, hipStream_t st)
 struct BwdWeightArgs {
     TiledShape s;
     const void *gout, *xcl, *off, *mask;
+    const void *goutp;   // grad_out in MFMA fragment order, see pack_gout_kernel
     float *gwacc;   // [group][chunk*K + tap][og][BKC] fp32 accumulator (zeroed): channel-contiguous rows, so that
                     // the atomics of a wavefront fill whole cache lines
     int split;      // position tiles are dealt round-robin to `split` workgroups per step
@@ -423,7 +424,6 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
     static_assert(ITEMS * kThreads == NITEM, "gather items divide evenly");
 
     __shared__ __align__(16) unsigned char s_tile[2][BKC * TRS];
-    __shared__ __align__(16) unsigned char s_stage[8 * 64 * (128 + 16)];   // per-wavefront patch of the gout operand
     __shared__ float s_w[2][8][kWMT];
     __shared__ int s_idx[2][kWMT];
     __shared__ int s_flag[2][kWMT];
@@ -528,55 +528,29 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
         }
     };
 
-    // gW block += gout[o, pos] * tile[pos, c].  The gout operand wants 8 (4) consecutive positions of one
-    // output channel per lane; read that way from memory every lane would touch its own cache line.  Each
-    // wavefront therefore pulls its 64 rows in 128-byte segments with coalesced loads (8 lanes per row),
-    // parks them in a private LDS patch and reads the operand vectors from there.
-    constexpr int SP = 128 / (int)sizeof(T);     // positions per stage = one 128-byte row segment
-    constexpr int NSTG = kWMT / SP;
-    constexpr int SRS = 128 + 16;                // patch row stride (bytes)
-    const T *gp = reinterpret_cast<const T *>(a.gout);
-    unsigned char *stg = s_stage + wave * (64 * SRS);
+    // gW block += gout[o, pos] * tile[pos, c].  The gout operand comes from a copy of grad_out in MFMA
+    // fragment order (pack_gout_kernel): one coalesced 1 KiB load per fragment, straight into registers.
+    // Four k-groups (one "stage") are in flight: a slot is refilled with the fragment of the next stage as
+    // soon as the matrix cores have taken it.
+    constexpr int NKGT = kWMT / (2 * VEC);       // k-groups per tile
+    constexpr int NSTG = NKGT / 4;
+    const int OBT = (s.og + 63) / 64 * 2;        // 32-row blocks per weight group in the packed copy
+    const uint4 *gp4 = reinterpret_cast<const uint4 *>(a.goutp);
+    auto gfrag = [&](int i, int kg, int ob) {
+        const long tile = sp + (long)i * a.split;
+        return gp4[((((long)wg * ntile + tile) * OBT + (o_base >> 5) + ob) * NKGT + kg) * 64 + lane];
+    };
+    uint4 ld[8];
     auto mma_tile = [&](int i, int tbuf) {
         if (!mma_wave) return;
-        const int m0 = (sp + i * a.split) * kWMT;
-        const int b0 = m0 / s.P;
-        uint4 ld[8];
-        auto issue = [&](int sg) {
-#pragma unroll
-            for (int q = 0; q < 8; q++) {
-                const int piece = q * 64 + lane, row = piece >> 3, c16 = piece & 7;
-                const int ol = o_base + row;
-                const int mv = m0 + sg * SP + c16 * VEC;
-                int b = b0, pp = mv - b0 * s.P;
-                if (pp >= s.P) { pp -= s.P; b += 1; }
-                ld[q] = (mv < s.M && ol < s.og)
-                            ? *reinterpret_cast<const uint4 *>(gp + ((long)b * s.Cout + wg * s.og + ol) * s.P + pp)
-                            : make_uint4(0, 0, 0, 0);
-            }
-        };
-        issue(0);
 #pragma unroll
         for (int sg = 0; sg < NSTG; sg++) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // operand reads of the previous stage are done
-#pragma unroll
-            for (int q = 0; q < 8; q++) {
-                const int piece = q * 64 + lane, row = piece >> 3, c16 = piece & 7;
-                *reinterpret_cast<uint4 *>(stg + row * SRS + c16 * 16) = ld[q];
-            }
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            if (sg + 1 < NSTG) issue(sg + 1);
 #pragma unroll
             for (int kq = 0; kq < 4; kq++) {
                 const int kg = sg * 4 + kq;
-                uint4 af[OB], bf[CB];
+                uint4 bf[CB];
 #pragma unroll
-                for (int ob = 0; ob < OB; ob++)
-                    af[ob] = *reinterpret_cast<const uint4 *>(stg + (ob * 32 + (lane & 31)) * SRS + (kq * 2 + (lane >> 5)) * 16);
-#pragma unroll
-                for (int cb = 0; cb < CB; cb++)
-                {
+                for (int cb = 0; cb < CB; cb++) {
                     const int row = cb * 32 + (lane & 31);
                     const int swz = sizeof(T) == 2 ? ((row >> 3) & 7) : 0;   // see interp_store
                     bf[cb] = *reinterpret_cast<const uint4 *>(&s_tile[tbuf][row * TRS + (((kg * 2 + (lane >> 5)) ^ swz) << 4)]);
@@ -584,7 +558,15 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                    for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], af[ob], bf[cb]);
+                    for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], ld[kq * 2 + ob], bf[cb]);
+                // refill: same k-group of the next stage (of the next tile after the last stage)
+                if (sg + 1 < NSTG) {
+#pragma unroll
+                    for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i, kg + 4, ob);
+                } else if (i + 1 < nmy) {
+#pragma unroll
+                    for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i + 1, kq, ob);
+                }
             }
         }
     };
@@ -592,6 +574,12 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
     // software pipeline over this workgroup's tiles: while the matrix cores take tile i, the corner
     // rows of tile i+1 are in flight and the corner weights of tile i+2 are computed
     if (nmy > 0) {
+        if (mma_wave) {
+#pragma unroll
+            for (int kq = 0; kq < 4; kq++)
+#pragma unroll
+                for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(0, kq, ob);
+        }
         coords(0, 0);
         __syncthreads();
         gather_issue(0);
@@ -678,6 +666,38 @@ __global__ void __launch_bounds__(256) cvt_grad_weight_kernel(const float *src, 
     }
 }
 
+// grad_out [N][Cout][P] -> MFMA fragments for the grad-weight kernel:
+//   goutp[wg][tile of kWMT positions][32-row block][k-group][lane] = 16 bytes =
+//   gout[wg*og + block*32 + lane%32][positions tile*kWMT + (2*kgroup + lane/32)*VEC + 0..VEC-1]
+// with positions numbered over the whole batch (m = b*P + p); rows past og and positions past N*P are zero.
+template <typename T>
+__global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp, TiledShape s, int ntile, int OBT, long total)
+{
+    constexpr int VEC = Elem<T>::VEC, NKGT = kWMT / (2 * VEC);
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int lane = (int)(i & 63);
+        long r = i >> 6;
+        const int kg = (int)(r % NKGT); r /= NKGT;
+        const int ob = (int)(r % OBT); r /= OBT;
+        const int tile = (int)(r % ntile);
+        const int wg = (int)(r / ntile);
+        const int ol = ob * 32 + (lane & 31);
+        const long m0 = (long)tile * kWMT + (2 * kg + (lane >> 5)) * VEC;
+        T e[VEC];
+#pragma unroll
+        for (int q = 0; q < VEC; q++) {
+            const long m = m0 + q;
+            T v = (T)0;
+            if (ol < s.og && m < s.M) {
+                const int b = (int)(m / s.P), p = (int)(m - (long)b * s.P);
+                v = gout[((long)b * s.Cout + wg * s.og + ol) * s.P + p];
+            }
+            e[q] = v;
+        }
+        reinterpret_cast<uint4 *>(goutp)[i] = *reinterpret_cast<const uint4 *>(e);
+    }
+}
+
 // gb[o] = sum_{b,p} gout[b,o,p]   (dconv3d_gpu.cu:1329)
 template <typename T>
 __global__ void __launch_bounds__(256) bias_grad_kernel(const T *gout, T *gb, int N, int Cout, int P)
@@ -724,9 +744,9 @@ bool d2c_tiled_bwd_data_supported(const TiledShape &s, int)
     return s.cg % s.cpg == 0;  // an offset group must lie inside one weight group
 }
 
-bool d2c_tiled_bwd_weight_supported(const TiledShape &s, int dtype)
+bool d2c_tiled_bwd_weight_supported(const TiledShape &, int)
 {
-    return s.P % (dtype == D2C_BF16 ? 8 : 4) == 0;
+    return true;   // the packed grad_out copy takes care of tiles that straddle samples or end early
 }
 
 // One pass reduces over all output channels of a weight group (the list-based grad_input needs that).
@@ -795,22 +815,35 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
     return D2C_OK;
 }
 
+// bytes of grad_out in fragment order (see pack_gout_kernel)
+size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype)
+{
+    const int vec = dtype == D2C_BF16 ? 8 : 4;
+    const long ntile = (s.M + kWMT - 1) / kWMT, OBT = (s.og + 63) / 64 * 2;
+    return (size_t)s.groups * ntile * OBT * (kWMT / (2 * vec)) * 64 * 16;
+}
+
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                                const void *mask, float *gwacc, void *gw, hipStream_t st)
+                                const void *mask, void *goutp, float *gwacc, void *gw, hipStream_t st)
 {
     const long nw = (long)s.Cout * s.cg * s.K;
-    {
-        D2cProfScope prof(D2C_PROF_PACK, st);
-        d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
-    }
     const int steps = s.nchunk * s.K;
     const int otiles = (s.og + 511) / 512;
     const int ntile = (s.M + kWMT - 1) / kWMT;
+    {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
+        const int OBT = (s.og + 63) / 64 * 2;
+        const long total = (long)s.groups * ntile * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
+        hipLaunchKernelGGL(pack_gout_kernel<T>, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const T *)gout, (T *)goutp, s,
+                           ntile, OBT, total);
+        if (int rc = d2c_check_launch("pack_gout_kernel")) return rc;
+    }
     int split = (512 + steps * otiles * s.groups - 1) / (steps * otiles * s.groups);
     if (split > ntile) split = ntile;
     if (split < 1) split = 1;
-    BwdWeightArgs a{s, gout, xcl, off, mask, gwacc, split};
+    BwdWeightArgs a{s, gout, xcl, off, mask, goutp, gwacc, split};
     {
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
         hipLaunchKernelGGL(tiled_bwd_weight_kernel<T>, dim3(steps, otiles, s.groups * split), dim3(kThreads), 0, st, a);
@@ -843,7 +876,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
                                               const void *, const void *, void *, float *, void *, void *, void *, \
                                               float *, hipStream_t);                                                        \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
-                                                const void *, float *, void *, hipStream_t);                      \
+                                                const void *, void *, float *, void *, hipStream_t);              \
     template int d2c_tiled_unpack_gx<T>(const TiledShape &, const float *, void *, hipStream_t);                   \
     template int d2c_tiled_bias_grad<T>(const TiledShape &, const void *, void *, hipStream_t);
 INST(bf16_t)
