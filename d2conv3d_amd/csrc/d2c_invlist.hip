@@ -11,10 +11,10 @@
 //      three fractions and its modulation;
 //   2. the grad-column values gcol[p, (k, chunk), c] are written once by the
 //      data kernel (in the element type of the call);
-//   3. one 8-lane group per (voxel, channel chunk) walks the lists of the 8 base
-//      voxels that can reach it, recomputes the corner weight, reads the gcol
-//      row segment and accumulates in registers; every grad_input element is
-//      written exactly once.
+//   3. one 8-lane group per (2 x 2 x 2 voxel cube, channel chunk) walks the
+//      lists of the 27 base voxels that can reach the cube, recomputes the
+//      corner weights, reads each gcol row segment once and accumulates in
+//      registers; every grad_input element is written exactly once.
 #include "d2c_mma.hpp"
 #include "d2c_tiled.hpp"
 
@@ -136,71 +136,111 @@ __global__ void set_total(const int *counts, int *starts, int n)
 }
 
 // ---- owner-computes accumulation ------------------------------------------
-// gcol layout: [chunk][tap][m = b*P + p][BKC] of T.  One 8-lane group per (voxel, chunk).
+// gcol layout: [chunk][tap][m = b*P + p][BKC] of T.
+// One 8-lane group per 2 x 2 x 2 cube of voxels (and channel chunk): the 27
+// base voxels that reach the cube are visited once each, and a grad-column row is read once for all the
+// voxels of the cube it contributes to (27 list visits and row reads per 8 voxels instead of 64).
+// Per axis, a base voxel at offset r in {0, 1, 2} from the cube's lower neighbour reaches cube voxel
+// a in {0, 1} with weight:  r = 0: (h, -),  r = 1: (1 - h, h),  r = 2: (-, 1 - h).
+// z and y offsets are compile-time (9 unrolled visits); the 3 base voxels along x are adjacent bins, one
+// contiguous range of entries, the x offset of an entry follows from its place in the range.
 template <typename T>
 __global__ void __launch_bounds__(256)
-gx_owner_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *entries, float *gxcl)
+gx_owner_cube_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *entries, float *gxcl)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
-    // a workgroup owns a compact 2 x 4 x 4 block of voxels: the 8 voxels that share a sample are then
-    // mostly served by one workgroup and the grad-column row is fetched once
-    const int sub = threadIdx.x & 7, vi = threadIdx.x >> 3;
+    const int sub = threadIdx.x & 7, ci = threadIdx.x >> 3;       // 32 cubes per workgroup: 2 x 4 x 4 of them
     const int cidx = blockIdx.y;                                  // channel chunk
-    const int nbx = (s.W + 3) / 4, nby = (s.H + 3) / 4, nbz = (s.D + 1) / 2;
-    int blk = xcd_swizzle(blockIdx.x, gridDim.x);                 // neighbouring blocks on the same XCD (L2)
+    const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
+    const int nbx = (ncx + 3) / 4, nby = (ncy + 3) / 4, nbz = (ncz + 1) / 2;
+    int blk = xcd_swizzle(blockIdx.x, gridDim.x);
     const int bx = blk % nbx; blk /= nbx;
     const int by = blk % nby; blk /= nby;
     const int bz = blk % nbz;
     const int b = blk / nbz;
-    const int x = bx * 4 + (vi & 3), y = by * 4 + ((vi >> 2) & 3), z = bz * 2 + (vi >> 4);
-    if (x >= s.W || y >= s.H || z >= s.D) return;
-    const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;   // voxel index over the batch
+    const int cx = bx * 4 + (ci & 3), cy = by * 4 + ((ci >> 2) & 3), cz = bz * 2 + (ci >> 4);
+    if (cx >= ncx || cy >= ncy || cz >= ncz) return;
+    const int x0 = cx * 2, y0 = cy * 2, z0 = cz * 2;
     const int g = (cidx * BKC) / s.cpg;
-    float acc[VEC];
+    float acc[2][2][2][VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; i++) acc[i] = 0.f;
+    for (int i = 0; i < 8 * VEC; i++) (&acc[0][0][0][0])[i] = 0.f;
     const T *gbase = gcol + ((long)cidx * s.K * s.M + (long)b * s.P) * BKC + sub * VEC;
-    // The base voxels (x-1) and (x) of one (z - dz, y - dy) row are neighbours in the bin order, so
-    // their lists form one contiguous range: 4 ranges per voxel, walked 4 entries at a time with all
-    // loads of a batch issued before their first use (entries past the end repeat the last one with
-    // weight 0).
-    // Order of the 4 ranges: by the parity of the base voxel's (z, y), so that the voxels that share a list
-    // (4 in z/y, and their x-neighbours) all walk it in the same quarter of the kernel, while its
-    // grad-column rows are still in the caches.
-#pragma unroll 1
-    for (int t = 0; t < 4; t++) {
-        const int dz = (z ^ (t >> 1)) & 1, dy = (y ^ t) & 1;
-        const int bin1 = bin_of(s, b, g, z - dz, y - dy, x - 1);   // dx = 1
-        const int e0 = starts[bin1], em = starts[bin1 + 1], e1 = starts[bin1 + 2];
-        for (int e = e0; e < e1; e += 4) {
-            uint4 q0[4], q1[4], row[4];
+    const int nxb = x0 + 1 < s.W ? 3 : 2;          // base voxels x0-1, x0, x0+1 (the last one only if it is a voxel)
+
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int ei = min(e + i, e1 - 1);
-                q0[i] = reinterpret_cast<const uint4 *>(entries + ei)[0];
-                q1[i] = reinterpret_cast<const uint4 *>(entries + ei)[1];
-            }
+    for (int rz = 0; rz < 3; rz++) {
+        const int zb = z0 - 1 + rz;
+        if (zb > s.D - 1) continue;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int p = (int)q0[i].x, k = (int)q0[i].y;
-                row[i] = *reinterpret_cast<const uint4 *>(gbase + ((long)k * s.M + p) * BKC);
-            }
+        for (int ry = 0; ry < 3; ry++) {
+            const int yb = y0 - 1 + ry;
+            if (yb > s.H - 1) continue;
+            const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
+            const int e0 = starts[bin1], em1 = starts[bin1 + 1], em2 = starts[bin1 + 2], e1 = starts[bin1 + nxb];
+            for (int e = e0; e < e1; e += 4) {
+                uint4 q0[4], q1[4], row[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float hz = __uint_as_float(q0[i].z), hy = __uint_as_float(q0[i].w);
-                const float hx = __uint_as_float(q1[i].x), al = __uint_as_float(q1[i].y);
-                const bool dx = e + i < em;      // entries of base voxel x-1 come first
-                float w = (dz ? hz : 1.f - hz) * (dy ? hy : 1.f - hy) * (dx ? hx : 1.f - hx) * al;
-                w = e + i < e1 ? w : 0.f;
-                const T *re = reinterpret_cast<const T *>(&row[i]);
+                for (int i = 0; i < 4; i++) {
+                    const int ei = min(e + i, e1 - 1);
+                    q0[i] = reinterpret_cast<const uint4 *>(entries + ei)[0];
+                    q1[i] = reinterpret_cast<const uint4 *>(entries + ei)[1];
+                }
 #pragma unroll
-                for (int j = 0; j < VEC; j++) acc[j] = fmaf(w, elem_to_f32<T>(re[j]), acc[j]);
+                for (int i = 0; i < 4; i++) {
+                    const int p = (int)q0[i].x, k = (int)q0[i].y;
+                    row[i] = *reinterpret_cast<const uint4 *>(gbase + ((long)k * s.M + p) * BKC);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float hz = __uint_as_float(q0[i].z), hy = __uint_as_float(q0[i].w);
+                    const float hx = __uint_as_float(q1[i].x);
+                    float al = __uint_as_float(q1[i].y);
+                    al = e + i < e1 ? al : 0.f;
+                    // x: offset 0 (base x0-1) reaches voxel c=0 with hx; 1 reaches (1-hx, hx); 2 reaches c=1 with 1-hx
+                    const bool r0 = e + i < em1, r2 = e + i >= em2;
+                    const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
+                    const float wx1 = r0 ? 0.f : (r2 ? 1.f - hx : hx);
+                    const T *re = reinterpret_cast<const T *>(&row[i]);
+                    float rv[VEC];
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) rv[j] = elem_to_f32<T>(re[j]);
+#pragma unroll
+                    for (int az = 0; az < 2; az++) {
+                        if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
+                        const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
+#pragma unroll
+                        for (int ay = 0; ay < 2; ay++) {
+                            if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
+                            const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
+                            const float wzy = wz * wy * al;
+                            const float w0 = wzy * wx0, w1 = wzy * wx1;
+#pragma unroll
+                            for (int j = 0; j < VEC; j++) {
+                                acc[az][ay][0][j] = fmaf(w0, rv[j], acc[az][ay][0][j]);
+                                acc[az][ay][1][j] = fmaf(w1, rv[j], acc[az][ay][1][j]);
+                            }
+                        }
+                    }
+                }
             }
         }
     }
-    float *o = gxcl + vg * s.Cin + cidx * BKC + sub * VEC;
 #pragma unroll
-    for (int i = 0; i < VEC; i += 4) *reinterpret_cast<float4 *>(o + i) = make_float4(acc[i], acc[i + 1], acc[i + 2], acc[i + 3]);
+    for (int az = 0; az < 2; az++)
+#pragma unroll
+        for (int ay = 0; ay < 2; ay++)
+#pragma unroll
+            for (int ax = 0; ax < 2; ax++) {
+                const int z = z0 + az, y = y0 + ay, x = x0 + ax;
+                if (z < s.D && y < s.H && x < s.W) {
+                    float *o = gxcl + ((long)b * s.vol + ((long)z * s.H + y) * s.W + x) * s.Cin + cidx * BKC + sub * VEC;
+#pragma unroll
+                    for (int i = 0; i < VEC; i += 4)
+                        *reinterpret_cast<float4 *>(o + i) = make_float4(acc[az][ay][ax][i], acc[az][ay][ax][i + 1],
+                                                                         acc[az][ay][ax][i + 2], acc[az][ay][ax][i + 3]);
+                }
+            }
 }
 
 // ---- owner-computes accumulation, channel-separated (depthwise) case ---------
@@ -265,7 +305,8 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
             for (int j = 0; j < kOwnCV; j++) acc[j] = 0.f;
 #pragma unroll 1
             for (int t4 = 0; t4 < 4; t4++) {
-                // ranges ordered by the parity of the base voxel's (z, y): see gx_owner_kernel
+                // ranges ordered by the parity of the base voxel's (z, y): the voxels that share a list (4 in z/y, and
+                // their x-neighbours) then walk it in the same quarter of the kernel, while it is still cached
                 const int dz = (z ^ (t4 >> 1)) & 1, dy = (y ^ t4) & 1;
                 const int bin1 = bin_of(s, b, g, z - dz, y - dy, x - 1);   // lists of base voxels x-1 and x are adjacent
                 const int e0 = starts[bin1], em = starts[bin1 + 1], e1 = starts[bin1 + 2];
@@ -351,9 +392,10 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
     D2cProfScope prof(D2C_PROF_GX_OWNER, st);
-    const long nblk = (long)s.N * ((s.D + 1) / 2) * ((s.H + 3) / 4) * ((s.W + 3) / 4);
+    const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
+    const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
     dim3 grid((unsigned)nblk, s.Cin / BKC);
-    hipLaunchKernelGGL(gx_owner_kernel<T>, grid, dim3(256), 0, st, s, (const T *)gcol, starts,
+    hipLaunchKernelGGL(gx_owner_cube_kernel<T>, grid, dim3(256), 0, st, s, (const T *)gcol, starts,
                        (const InvEntry *)entries, gxcl);
     return d2c_check_launch("gx_owner_kernel");
 }
