@@ -240,7 +240,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     const size_t es = d2c_elem_size(q.dtype);
     BwdWs w;
     w.xcl = 0;
-    w.wt = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
+    w.wt = d2c_align_up((size_t)s.N * s.vol * s.Cin * es + 256);   // input, then a 256-byte row of zeros
     const int omax = d2c_bwd_pass_channels(q.dtype);
     const int ogk = d2c_bwd_ogk(s.og < omax ? s.og : omax, q.dtype);
     w.gxcl = w.wt + d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * ogk * es);

@@ -11,7 +11,7 @@
 //   the weight group) stays in registers for the whole kernel; the weight
 //   operand of the step is staged in LDS; gcol never leaves the chip.
 //
-// Kernel 2 (tiled_bwd_weight_kernel), per workgroup one (tap, channel chunk)
+// Kernel 2 (tiled_bwd_weight_dma_kernel), per workgroup one (tap, channel chunk)
 // and all output channels, looping over position tiles:
 //     gW[o, c, k] += sum_pos gout[o, pos] * alpha * trilinear(x[c], pos)       (:1037-1088)
 //   The sampler writes its tile position-contiguous so that it is an MFMA
@@ -408,39 +408,58 @@ struct BwdWeightArgs {
     int split;      // position tiles are dealt round-robin to `split` workgroups per step
 };
 
-constexpr int kWMT = 128;  // positions per iteration
+constexpr int kWMT = 128;  // positions per tile of the packed grad_out copy
 
-template <typename T>
-__global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArgs a)
+// One workgroup = one (chunk, tap) step, all output channels of the weight group (8 worker wavefronts x 64
+// rows), looping over its share of the 64-position tiles.  The corner rows go global -> LDS by DMA loads
+// (no gather registers) and the coordinates are computed by a ninth wavefront: while the matrix cores take
+// tile `it`, tile it+1 is interpolated from LDS, the rows of tile it+2 are in flight and the table of tile
+// it+3 is computed.  Same roles and ring buffers as tiled_fwd_dma_kernel (d2c_tiled_fwd.hip).
+constexpr int kWDT = 64;                    // positions per iteration
+constexpr int kWRawPos = 8 * 128;           // raw bytes per position: 8 corner rows of 128 bytes
+
+struct BwdWeightDmaArgs {
+    BwdWeightArgs w;
+    unsigned zrow;       // byte offset (from xcl) of a 128-byte row of zeros: what dead corners read
+};
+
+template <typename T, bool AUX16>
+__global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(BwdWeightDmaArgs aa)
 {
+    constexpr int MT = kWDT;
     constexpr int VEC = Elem<T>::VEC;          // positions per 16-byte operand vector
     constexpr int BKC = 8 * VEC;               // channels per step (64 / 32)
     constexpr int CB = BKC / 32;
     constexpr int OB = 2;                      // 32-row blocks of output channels per wavefront
     constexpr int NT = 64 * 8;                 // output channels per workgroup
-    constexpr int TRS = kWMT * (int)sizeof(T) + 16;   // tile row stride: [channel][position]
-    constexpr int NITEM = kWMT * 8;            // gather items per tile: (position, 16-byte channel vector)
-    constexpr int ITEMS = NITEM / kThreads;
-    static_assert(ITEMS * kThreads == NITEM, "gather items divide evenly");
+    constexpr int TRS = MT * (int)sizeof(T) + 16;   // tile row stride: [channel][position]
+    constexpr int NKG = MT / (2 * VEC);        // k-groups per iteration (4 / 8)
+    constexpr int NKGP = kWMT / (2 * VEC);     // k-groups per tile of the packed grad_out copy
+    static_assert(MT * 8 == kThreads, "one (position, vector) item per worker thread");
 
-    __shared__ __align__(16) unsigned char s_tile[2][BKC * TRS];
-    __shared__ float s_w[2][8][kWMT];
-    __shared__ int s_idx[2][kWMT];
-    __shared__ int s_flag[2][kWMT];
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char *s_raw = smem;                                       // [2][MT][8 corners][128 B]
+    unsigned char *s_tile = s_raw + 2 * MT * kWRawPos;                 // [2][BKC][TRS]
+    float *s_w = reinterpret_cast<float *>(s_tile + 2 * BKC * TRS);    // [3][8][MT]
+    int *s_idx = reinterpret_cast<int *>(s_w + 3 * 8 * MT);            // [3][MT]
+    int *s_flag = s_idx + 3 * MT;                                      // [3][MT]
 
+    const BwdWeightArgs &a = aa.w;
     const TiledShape &s = a.s;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool worker = wave < 8;
     const int st = blockIdx.x;                 // step = chunk * K + tap
     const int otile = blockIdx.y;
     const int wg = blockIdx.z / a.split, sp = blockIdx.z % a.split;
     const int j = st / s.K, k = st - j * s.K;
     const int c0 = wg * s.cg + j * BKC;
     const int g = c0 / s.cpg;
-    const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;   // element strides of a step in z / y
-    const int ntile = (s.M + kWMT - 1) / kWMT;
+    const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;
+    const int ntile = (s.M + MT - 1) / MT;
     const int nmy = ntile > sp ? (ntile - sp + a.split - 1) / a.split : 0;   // tiles of this workgroup
-    const int o_base = otile * NT + wave * 64;   // first output channel (in the weight group) of this wavefront
-    const bool mma_wave = o_base < s.og;
+    const int o_base = otile * NT + wave * 64;
+    const bool mma_wave = worker && o_base < s.og;
 
     f32x16 acc[OB][CB];
 #pragma unroll
@@ -450,129 +469,139 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[ob][cb][r] = 0.f;
 
-    // corner weights of tile i's positions for this tap
-    auto coords = [&](int i, int buf) {
-        if (tid < kWMT) {
-            float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            int idx = 0;
-            unsigned live = 0;
-            const int m = (sp + i * a.split) * kWMT + tid;
-            if (m < s.M) {
-                const int b = m / s.P, p = m - b * s.P;
-                const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
-                float o0, o1, o2;
-                load_offsets(s, a.off, b, g, k, p, o0, o1, o2);
-                const float al = a.mask ? ld_aux(a.mask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt) : 1.f;
-                int bz, by, bx;
-                tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
-                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
-                live = t.live;
-                idx = (b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
-#pragma unroll
-                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
-            }
-#pragma unroll
-            for (int c = 0; c < 8; c++) s_w[buf][c][tid] = w[c];
-            s_idx[buf][tid] = idx;
-            s_flag[buf][tid] = (int)live;
-        }
-    };
-
-    // sample: one item = one position x one 16-byte vector of channels (8 lanes read one 128-byte corner row)
-    uint4 gv[ITEMS][8];
-    auto gather_issue = [&](int buf) {
-        const char *xb = reinterpret_cast<const char *>(a.xcl);
-#pragma unroll
-        for (int it = 0; it < ITEMS; it++) {
-            const int item = tid + it * kThreads;
-            const int pos = item >> 3, vec = item & 7;
-            const int idx = s_idx[buf][pos] + c0 + vec * VEC;
-            const unsigned live = (unsigned)s_flag[buf][pos];
-#pragma unroll
-            for (int c = 0; c < 8; c++) {
-                const unsigned o = (unsigned)(idx + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc + (c & 1) * s.Cin)
-                                   * (unsigned)sizeof(T);
-                gv[it][c] = ((live >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + o) : make_uint4(0, 0, 0, 0);
-            }
-        }
-    };
-    // interpolate, then store transposed ([channel][position]: the operand order of a reduction over
-    // positions).  bfloat16: the lanes of positions p and p^1 (8 lanes apart) swap values so that each
-    // writes whole 4-byte pairs of positions.
-    auto interp_store = [&](int cbuf, int tbuf) {
-#pragma unroll
-        for (int it = 0; it < ITEMS; it++) {
-            const int item = tid + it * kThreads;
-            const int pos = item >> 3, vec = item & 7;
-            VecAcc<T> acc;
-            acc.zero();
-#pragma unroll
-            for (int c = 0; c < 8; c++) acc.fma(s_w[cbuf][c][pos], gv[it][c]);
-            unsigned char *tb = &s_tile[tbuf][(vec * VEC) * TRS];
-            if constexpr (sizeof(T) == 2) {
-                const int odd = pos & 1;
-#pragma unroll
-                for (int e = 0; e < VEC; e++) {
-                    const float other = __shfl_xor(acc.a[e], 8, 64);     // same channel, position pos ^ 1
-                    if ((e & 1) == odd) {
-                        const uint32_t pr = odd ? pack_bf16x2(other, acc.a[e]) : pack_bf16x2(acc.a[e], other);
-                        // 16-byte chunks of a row are XOR-swizzled by its 8-channel group: the 8 vectors of a
-                        // position pair would otherwise all hit the same banks (rows 8 apart alias)
-                        *reinterpret_cast<uint32_t *>(tb + e * TRS + ((((pos >> 1) ^ (vec << 2))) << 2)) = pr;
-                    }
-                }
+    // --- coordinate wavefront: lane = position of tile i
+    const int ctid = tid - kThreads;
+    float craw[4];
+    int cb_ = 0, cp_ = 0;
+    bool cvalid = false;
+    auto coords_issue = [&](int i) {
+        if (worker) return;
+        const long m = (long)(sp + i * a.split) * MT + ctid;
+        cvalid = m < s.M;
+        if (cvalid) {
+            cb_ = (int)(m / s.P); cp_ = (int)(m - (long)cb_ * s.P);
+            const long ab = (((long)cb_ * s.G + g) * s.K + k) * s.P + cp_;
+            if (s.nd == 3) {
+                const long ob = 3 * ab - 2 * (long)cp_;
+                craw[0] = ld_auxT<AUX16>(a.off, ob);
+                craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
+                craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
             } else {
-#pragma unroll
-                for (int e = 0; e < VEC; e++) *reinterpret_cast<float *>(tb + e * TRS + pos * 4) = acc.a[e];
+                craw[0] = 0.f; craw[1] = 0.f;
+                craw[2] = ld_auxT<AUX16>(a.off, ab);
             }
+            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
+        }
+    };
+    auto coords_finish = [&](int buf) {   // of the tile whose offsets coords_issue requested last
+        if (worker) return;
+        float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        int idx = 0;
+        unsigned live = 0;
+        if (cvalid) {
+            const int ox = cp_ % s.Wo, oy = (cp_ / s.Wo) % s.Ho, oz = cp_ / (s.Wo * s.Ho);
+            int bz, by, bx;
+            tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
+            const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
+            live = t.live;
+            idx = (cb_ * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
+#pragma unroll
+            for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * craw[3] : 0.f;
+        }
+#pragma unroll
+        for (int c = 0; c < 8; c++) s_w[(buf * 8 + c) * MT + ctid] = w[c];
+        s_idx[buf * MT + ctid] = idx;
+        s_flag[buf * MT + ctid] = (int)live;
+    };
+
+    // --- corner rows of tile i -> s_raw[rbuf]: worker wavefront w requests positions 8w .. 8w+7
+    const int dcorner = lane >> 3, dvec = lane & 7;
+    const int dcoff = ((dcorner >> 2) & 1) * dzc + ((dcorner >> 1) & 1) * dyc + (dcorner & 1) * s.Cin;
+    auto dma_issue = [&](int rbuf, int tbuf) {
+        if (!worker) return;
+        const char *base = reinterpret_cast<const char *>(a.xcl);
+        const int vidx = s_idx[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const int vflag = s_flag[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+#pragma unroll
+        for (int i = 0; i < MT / 8; i++) {
+            const int pos = wave * (MT / 8) + i;
+            const int idx = __builtin_amdgcn_readlane(vidx, i);
+            const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
+            const unsigned o = ((live >> dcorner) & 1u)
+                                   ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
+                                   : aa.zrow + (unsigned)dvec * 16u;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + o),
+                                             (__attribute__((address_space(3))) void *)(s_raw + (rbuf * MT + pos) * kWRawPos),
+                                             16, 0, 0);
+        }
+    };
+    // --- interpolation, stored transposed ([channel][position]); thread = (position, 16-byte vector)
+    const int ipos = tid >> 3, ivec = tid & 7;
+    auto interp_store = [&](int rbuf, int tbuf, int dbuf) {
+        if (!worker) return;
+        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * kWRawPos + ivec * 16;
+        VecAcc<T> va;
+        va.zero();
+#pragma unroll
+        for (int c = 0; c < 8; c++)
+            va.fma(s_w[(tbuf * 8 + c) * MT + ipos], *reinterpret_cast<const uint4 *>(rp + c * 128));
+        unsigned char *tb = s_tile + dbuf * BKC * TRS + (ivec * VEC) * TRS;
+        if constexpr (sizeof(T) == 2) {
+            // lanes of positions p and p^1 (8 lanes apart) swap values, each writes 4-byte pairs of positions;
+            // 16-byte chunks of a row are XOR-swizzled by its 8-channel group (rows 8 apart alias in LDS)
+            const int odd = ipos & 1;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                const float other = __shfl_xor(va.a[e], 8, 64);
+                if ((e & 1) == odd) {
+                    const uint32_t pr = odd ? pack_bf16x2(other, va.a[e]) : pack_bf16x2(va.a[e], other);
+                    *reinterpret_cast<uint32_t *>(tb + e * TRS + ((((ipos >> 1) ^ (ivec << 2))) << 2)) = pr;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) *reinterpret_cast<float *>(tb + e * TRS + ipos * 4) = va.a[e];
         }
     };
 
-    // gW block += gout[o, pos] * tile[pos, c].  The gout operand comes from a copy of grad_out in MFMA
-    // fragment order (pack_gout_kernel): one coalesced 1 KiB load per fragment, straight into registers.
-    // Four k-groups (one "stage") are in flight: a slot is refilled with the fragment of the next stage as
-    // soon as the matrix cores have taken it.
-    constexpr int NKGT = kWMT / (2 * VEC);       // k-groups per tile
-    constexpr int NSTG = NKGT / 4;
-    const int OBT = (s.og + 63) / 64 * 2;        // 32-row blocks per weight group in the packed copy
+    // --- gW block += gout[o, pos] * tile[pos, c]; gout fragments straight from the packed copy
+    const int OBT = (s.og + 63) / 64 * 2;
+    const int ntp = (s.M + kWMT - 1) / kWMT;     // tiles of the packed copy (kWMT positions each)
     const uint4 *gp4 = reinterpret_cast<const uint4 *>(a.goutp);
     auto gfrag = [&](int i, int kg, int ob) {
-        const long tile = sp + (long)i * a.split;
-        return gp4[((((long)wg * ntile + tile) * OBT + (o_base >> 5) + ob) * NKGT + kg) * 64 + lane];
+        const long t64 = sp + (long)i * a.split;
+        const long tp = t64 / (kWMT / MT);
+        const int kgp = (int)(t64 % (kWMT / MT)) * NKG + kg;
+        return gp4[((((long)wg * ntp + tp) * OBT + (o_base >> 5) + ob) * NKGP + kgp) * 64 + lane];
     };
-    uint4 ld[8];
-    auto mma_tile = [&](int i, int tbuf) {
+    uint4 ld[8];   // four k-groups in flight; a slot is refilled as soon as the matrix cores have taken it
+    auto mma_tile = [&](int i, int dbuf) {
         if (!mma_wave) return;
 #pragma unroll
-        for (int sg = 0; sg < NSTG; sg++) {
+        for (int kg = 0; kg < NKG; kg++) {
+            const int kq = kg & 3;
+            uint4 bf[CB];
 #pragma unroll
-            for (int kq = 0; kq < 4; kq++) {
-                const int kg = sg * 4 + kq;
-                uint4 bf[CB];
+            for (int cb = 0; cb < CB; cb++) {
+                const int row = cb * 32 + (lane & 31);
+                const int swz = sizeof(T) == 2 ? ((row >> 3) & 7) : 0;
+                bf[cb] = *reinterpret_cast<const uint4 *>(s_tile + dbuf * BKC * TRS + row * TRS
+                                                          + (((kg * 2 + (lane >> 5)) ^ swz) << 4));
+            }
 #pragma unroll
-                for (int cb = 0; cb < CB; cb++) {
-                    const int row = cb * 32 + (lane & 31);
-                    const int swz = sizeof(T) == 2 ? ((row >> 3) & 7) : 0;   // see interp_store
-                    bf[cb] = *reinterpret_cast<const uint4 *>(&s_tile[tbuf][row * TRS + (((kg * 2 + (lane >> 5)) ^ swz) << 4)]);
-                }
+            for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                for (int ob = 0; ob < OB; ob++)
+                for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], ld[kq * 2 + ob], bf[cb]);
+            if (kg + 4 < NKG) {
 #pragma unroll
-                    for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], ld[kq * 2 + ob], bf[cb]);
-                // refill: same k-group of the next stage (of the next tile after the last stage)
-                if (sg + 1 < NSTG) {
+                for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i, kg + 4, ob);
+            } else if (i + 1 < nmy) {
 #pragma unroll
-                    for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i, kg + 4, ob);
-                } else if (i + 1 < nmy) {
-#pragma unroll
-                    for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i + 1, kq, ob);
-                }
+                for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i + 1, kg + 4 - NKG, ob);
             }
         }
     };
 
-    // software pipeline over this workgroup's tiles: while the matrix cores take tile i, the corner
-    // rows of tile i+1 are in flight and the corner weights of tile i+2 are computed
     if (nmy > 0) {
         if (mma_wave) {
 #pragma unroll
@@ -580,18 +609,33 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(0, kq, ob);
         }
-        coords(0, 0);
+        for (int q = 0; q < 3; q++) {
+            if (q < nmy) {
+                coords_issue(q);
+                coords_finish(q % 3);
+            }
+        }
         __syncthreads();
-        gather_issue(0);
-        if (nmy > 1) coords(1, 1);
-        interp_store(0, 0);
+        dma_issue(0, 0);
+        if (1 < nmy) dma_issue(1, 1);
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        for (int i = 0; i < nmy; i++) {
-            if (i + 1 < nmy) gather_issue((i + 1) & 1);
-            if (i + 2 < nmy) coords(i + 2, i & 1);
-            mma_tile(i, i & 1);
-            if (i + 1 < nmy) interp_store((i + 1) & 1, (i + 1) & 1);
-            __syncthreads();
+        interp_store(0, 0, 0);
+        if (3 < nmy) coords_issue(3);
+        if (worker) {
+            for (int it = 0; it < nmy; it++) {
+                __builtin_amdgcn_s_waitcnt(0);     // the transfers requested in the last iteration have landed
+                __syncthreads();
+                mma_tile(it, it & 1);
+                if (it + 2 < nmy) dma_issue(it & 1, (it + 2) % 3);
+                if (it + 1 < nmy) interp_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
+            }
+        } else {
+            for (int it = 0; it < nmy; it++) {
+                __syncthreads();
+                if (it + 3 < nmy) coords_finish(it % 3);   // offsets requested one iteration ago
+                if (it + 4 < nmy) coords_issue(it + 4);
+            }
         }
     }
 
@@ -608,6 +652,12 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_kernel(BwdWeightArg
                                   acc[ob][cb][r]);
                 }
     }
+}
+
+template <typename T> constexpr size_t bwd_weight_dma_lds()
+{
+    constexpr int BKC = 8 * Elem<T>::VEC;
+    return (size_t)2 * kWDT * kWRawPos + (size_t)2 * BKC * (kWDT * sizeof(T) + 16) + (size_t)3 * 10 * kWDT * 4;
 }
 
 // ============================================================ small kernels
@@ -830,25 +880,46 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     const long nw = (long)s.Cout * s.cg * s.K;
     const int steps = s.nchunk * s.K;
     const int otiles = (s.og + 511) / 512;
-    const int ntile = (s.M + kWMT - 1) / kWMT;
+    const int ntp = (s.M + kWMT - 1) / kWMT;     // tiles of the packed grad_out copy
+    const int ntile = (s.M + kWDT - 1) / kWDT;   // position tiles of the kernel
     {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
+        // the channels-last input is followed by a 256-byte row of zeros: what dead corners read
+        d2c_fill_zero((char *)const_cast<void *>(xcl) + (size_t)s.N * s.vol * s.Cin * sizeof(T), 256, st);
         const int OBT = (s.og + 63) / 64 * 2;
-        const long total = (long)s.groups * ntile * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
+        const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
         hipLaunchKernelGGL(pack_gout_kernel<T>, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const T *)gout, (T *)goutp, s,
-                           ntile, OBT, total);
+                           ntp, OBT, total);
         if (int rc = d2c_check_launch("pack_gout_kernel")) return rc;
     }
     int split = (512 + steps * otiles * s.groups - 1) / (steps * otiles * s.groups);
     if (split > ntile) split = ntile;
     if (split < 1) split = 1;
-    BwdWeightArgs a{s, gout, xcl, off, mask, goutp, gwacc, split};
+    BwdWeightDmaArgs a{{s, gout, xcl, off, mask, goutp, gwacc, split},
+                       (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T))};
     {
+        const dim3 grid(steps, otiles, s.groups * split);
+        constexpr size_t lds = bwd_weight_dma_lds<T>();
+        bool aux16 = false;
+        if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
-        hipLaunchKernelGGL(tiled_bwd_weight_kernel<T>, dim3(steps, otiles, s.groups * split), dim3(kThreads), 0, st, a);
+        if constexpr (sizeof(T) == 2) {
+            if (aux16) {
+                if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, true>,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+                    return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_weight_dma_kernel)");
+                hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, true>), grid, dim3(kThreads + 64), lds, st, a);
+            }
+        }
+        if (!aux16) {
+            if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+                return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_weight_dma_kernel)");
+            hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, false>), grid, dim3(kThreads + 64), lds, st, a);
+        }
     }
-    if (int rc = d2c_check_launch("tiled_bwd_weight_kernel")) return rc;
+    if (int rc = d2c_check_launch("tiled_bwd_weight_dma_kernel")) return rc;
     D2cProfScope prof(D2C_PROF_PACK, st);
     hipLaunchKernelGGL(cvt_grad_weight_kernel<T>, dim3(grid1d(nw)), dim3(256), 0, st, gwacc, (T *)gw, s, nw);
     return d2c_check_launch("cvt_grad_weight_kernel");
