@@ -225,11 +225,10 @@ bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 // grad_offset / grad_mask by the kernel of d2c_aux_grad.hip (from the grad-column rows): when the data kernel
-// makes whole rows in one pass and does not split its steps.
+// makes whole rows in one pass.
 bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
 {
-    return d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype)
-           && d2c_bwd_data_split(s, q.dtype) == 1;
+    return d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
 }
 
 struct BwdWs {
