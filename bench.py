@@ -104,7 +104,7 @@ def hbm_traffic_bytes(workload, kernel):
     try:
         for row in open(path):
             cells = [c.strip().strip("`") for c in row.split("|")]
-            if len(cells) > 4 and cells[1].startswith(kernel):
+            if len(cells) > 4 and cells[1].startswith(kernel[:-len("_kernel")] if kernel.endswith("_kernel") else kernel):
                 return int(float(cells[4]) * 1e6)
     except (OSError, ValueError):
         pass
@@ -237,7 +237,7 @@ def main():
     fam = {"mfma": "tiled", "depthwise": "dw", "generic": "generic"}[algo]
     names = {_lib.PROF_FWD: f"{fam}_fwd_kernel", _lib.PROF_BWD_DATA: f"{fam}_bwd_data_kernel",
              _lib.PROF_BWD_WEIGHT: f"{fam}_bwd_weight_kernel", _lib.PROF_GX_OWNER: "gx_owner_kernel",
-             _lib.PROF_PACK: "pack/clear/convert/lists"}
+             _lib.PROF_BWD_AUX: "aux_grad_kernel", _lib.PROF_PACK: "pack/clear/convert/lists"}
     if fam == "dw":
         names[_lib.PROF_BWD_DATA] = "dw_bwd_kernel"
     kern = {}
@@ -259,7 +259,13 @@ def main():
         P = 1
         for d in dims:
             P *= d
-        if dom == "gx_owner_kernel":
+        if dom == "aux_grad_kernel":
+            # the corner rows it gathers (8 per sample and chunk), the grad-column rows and the offset / mask
+            # tensors in and out, once each
+            K = 3 ** nd
+            nbytes = N * P * K * C * es * 9 + 2 * N * P * K * G * (nd + 1) * es
+            bound, ach = "hbm", nbytes / t_dom / 1e9
+        elif dom == "gx_owner_kernel":
             # every grad-column row (N*P*K*Cin elements), every list entry (32 B per sample) and every
             # grad_input element (fp32 accumulator) once
             K = 3 ** nd

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libd2conv.so")
 
 D2C_F32, D2C_F64, D2C_BF16 = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_MFMA, ALGO_DEPTHWISE = 0, 1, 2, 3
-PROF_FWD, PROF_BWD_DATA, PROF_BWD_WEIGHT, PROF_PACK, PROF_GX_OWNER = 0, 1, 2, 3, 4
+PROF_FWD, PROF_BWD_DATA, PROF_BWD_WEIGHT, PROF_PACK, PROF_GX_OWNER, PROF_BWD_AUX = 0, 1, 2, 3, 4, 5
 ALGO_NAMES = {ALGO_GENERIC: "generic", ALGO_MFMA: "mfma", ALGO_DEPTHWISE: "depthwise"}
 
 # every symbol that include/d2conv.h declares

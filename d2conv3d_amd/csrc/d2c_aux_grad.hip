@@ -259,7 +259,7 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     dim3 grid((ntile + kWavesPerBlock - 1) / kWavesPerBlock, s.G, s.K < kTapSplit ? s.K : kTapSplit);
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
-    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
+    D2cProfScope prof(D2C_PROF_BWD_AUX, st);
     if constexpr (sizeof(T) == 2) {
         if (aux16) hipLaunchKernelGGL((aux_grad_kernel<T, true>), grid, dim3(64 * kWavesPerBlock), 0, st, a);
     }

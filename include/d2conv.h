@@ -144,11 +144,12 @@ void d2c_set_algo_override(int algo);
  */
 enum {
     D2C_PROF_FWD = 0,         /* forward implicit-GEMM / depthwise kernel */
-    D2C_PROF_BWD_DATA = 1,    /* grad_input + grad_offset + grad_mask kernel */
+    D2C_PROF_BWD_DATA = 1,    /* grad-column product (+ grad_offset / grad_mask / scatter when fused) */
     D2C_PROF_BWD_WEIGHT = 2,  /* grad_weight kernel */
     D2C_PROF_PACK = 3,        /* layout changes, clears, conversions, sample lists (sum) */
     D2C_PROF_GX_OWNER = 4,    /* grad_input accumulation from the sample lists */
-    D2C_PROF_COUNT = 5
+    D2C_PROF_BWD_AUX = 5,     /* grad_offset / grad_mask from the grad-column rows */
+    D2C_PROF_COUNT = 6
 };
 void d2c_profile_enable(int on);
 void d2c_profile_reset(void);
