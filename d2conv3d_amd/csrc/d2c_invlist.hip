@@ -44,12 +44,10 @@ template <bool FILL>
 __global__ void __launch_bounds__(256)
 invlist_pass_kernel(TiledShape s, const void *off, const void *mask, int *counts, const int *starts, InvEntry *entries)
 {
-    const long total = (long)s.N * s.G * s.K * s.P;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-        const int p = (int)(i % s.P);
-        const int k = (int)((i / s.P) % s.K);
-        const int g = (int)((i / ((long)s.P * s.K)) % s.G);
-        const int b = (int)(i / ((long)s.P * s.K * s.G));
+    // grid = (position blocks, taps, samples x offset groups): no 64-bit index arithmetic per thread
+    const int k = blockIdx.y;
+    const int b = blockIdx.z / s.G, g = blockIdx.z - b * s.G;
+    for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < s.P; p += gridDim.x * blockDim.x) {
         const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
         float o0, o1, o2;
         load_offsets(s, off, b, g, k, p, o0, o1, o2);
@@ -371,9 +369,9 @@ int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, in
         return D2C_ERR_UNSUPPORTED;
     }
     const int nb = (int)nbl;
-    const long total = (long)s.N * s.G * s.K * s.P;
+    const dim3 pgrid(g1d(s.P, 4096), s.K, s.N * s.G);
     d2c_fill_zero(counts, (size_t)(nb + 1) * 4, st);
-    hipLaunchKernelGGL(invlist_pass_kernel<false>, dim3(g1d(total)), dim3(256), 0, st, s, off, mask, counts,
+    hipLaunchKernelGGL(invlist_pass_kernel<false>, pgrid, dim3(256), 0, st, s, off, mask, counts,
                        (const int *)nullptr, (InvEntry *)nullptr);
     const int nblk = (nb + kScanBlock - 1) / kScanBlock;
     hipLaunchKernelGGL(scan_block_sums, dim3(nblk), dim3(256), 0, st, counts, bsums, nb);
@@ -381,7 +379,7 @@ int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, in
     hipLaunchKernelGGL(scan_apply, dim3(nblk), dim3(256), 0, st, counts, bsums, starts, nb);
     hipLaunchKernelGGL(set_total, dim3(1), dim3(64), 0, st, counts, starts, nb);
     d2c_fill_zero(counts, (size_t)(nb + 1) * 4, st);   // reused as the per-bin cursor of the fill pass
-    hipLaunchKernelGGL(invlist_pass_kernel<true>, dim3(g1d(total)), dim3(256), 0, st, s, off, mask, counts, starts,
+    hipLaunchKernelGGL(invlist_pass_kernel<true>, pgrid, dim3(256), 0, st, s, off, mask, counts, starts,
                        (InvEntry *)entries);
     return d2c_check_launch("invlist_build");
 }
