@@ -48,6 +48,24 @@ int d2c_check_launch(const char *what)
     return D2C_ERR_LAUNCH;
 }
 
+int d2c_num_cus()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        d2c_set_error("hipGetDevice failed");
+        return 0;
+    }
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+        d2c_set_error("hipDeviceGetAttribute(multiprocessor count) failed");
+        return 0;
+    }
+    cached[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
 void d2c_prof_begin(int id, hipStream_t st)
 {
     if (!g_prof.on) return;

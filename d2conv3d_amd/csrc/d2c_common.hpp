@@ -122,6 +122,10 @@ static inline TapGeom make_geom(const d2c_conv3d_desc &q)
 void d2c_set_error(const char *fmt, ...);
 int d2c_check_launch(const char *what);
 
+// Compute units of the current device (persistent kernels launch one workgroup each); 0 if the query fails,
+// with the error text set.
+int d2c_num_cus();
+
 // Clears `bytes` (a multiple of 4) with a fill kernel; safe to record into a HIP graph.
 void d2c_fill_zero(void *p, size_t bytes, hipStream_t st);
 

@@ -141,9 +141,11 @@ FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.xcl = 0;
     w.wp = d2c_align_up((size_t)s.N * s.vol * s.Cin * es + 256);   // input, then a 256-byte row of zeros
     w.outacc = w.wp + d2c_align_up((size_t)s.groups * s.nchunk * s.K * s.ogp * bkc_of(q.dtype) * es);
-    // fp32 partial sums of the output, used only when the forward kernel splits its steps
+    // fp32 partial sums of the output, used only when the forward kernel splits its steps (as whole tiles of
+    // 64 positions x padded output channels in the DMA-gather kernel)
     w.total = w.outacc;
-    if (d2c_fwd_split(s) > 1) w.total += d2c_align_up((size_t)s.N * s.Cout * s.P * sizeof(float));
+    if (d2c_fwd_split(s) > 1)
+        w.total += d2c_align_up((size_t)((s.M + 63) / 64 * 64) * s.ogp * s.groups * sizeof(float));
     return w;
 }
 

@@ -37,6 +37,13 @@ struct FwdArgs {
     float *outacc;
     int nsplit;
     unsigned zrow;     // byte offset (from xcl) of a 128-byte row of zeros: what dead corners read
+    // Schedule of the DMA-gather kernel, whose workgroups are persistent (one per compute unit).  A work item is
+    // one (position tile, output tile, weight group) with all its steps.  Items [0, sk_full) are dealt whole,
+    // round-robin.  The remaining items, fewer than one round, have their steps cut into sk_cut equal ranges;
+    // the (range, item) pieces are dealt round-robin in range-major order, so that the workgroups running at
+    // one time are at about the same steps and share their weight fragments in L2.  The pieces add into
+    // `outacc`, here laid out [item - sk_full][output channel of the tile][position of the tile].
+    int sk_items, sk_full, sk_ntile, sk_otiles, sk_cut;
 };
 
 // Tiles that are neighbours in space go to the same XCD (workgroups are dealt
@@ -262,17 +269,64 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
 
 // ---------------------------------------------------------------------------
 // The same forward pass with the corner rows moved global -> LDS by DMA loads
-// (global_load_lds_dwordx4: no staging registers, so the rows of step s+2 are
-// in flight while step s runs on the matrix cores and step s+1 is interpolated).
-// One workgroup = 512 threads = 64 positions x NT output channels.  One DMA
+// (global_load_lds_dwordx4: no staging registers; the rows of step s+2 are
+// requested at the end of iteration s and are in flight over the barrier and
+// the matrix-core phase of iteration s+1).
+// One workgroup = 512 + 64 threads = 64 positions x NT output channels.  One DMA
 // instruction of a wavefront fetches the 8 corner rows (8 x 128 bytes) of one
 // position: lane = (corner, 16-byte vector); corners that are out of range or
 // cut off by the early-out read a row of zeros instead.
+//
+// Workgroups are persistent: each walks a list of segments (a work item and a
+// range of its steps, see FwdArgs) as ONE sequence of steps, so that the
+// pipeline stays full from one segment into the next; only the matrix-core
+// wavefronts notice a segment's end (they store or add their accumulators).
 constexpr int kDMT = 64;                   // positions per workgroup
 constexpr int kRawPos = 8 * kNV * 16;      // raw bytes per position: 8 corners x 128
 
+// Workgroup barrier that waits for this wavefront's LDS operations only: its global loads and DMA transfers
+// stay in flight across it (a __syncthreads() would wait for them as well).
+D2C_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+constexpr int kMaxSeg = 128;               // segments per workgroup (the launcher sizes the grid for this)
+
+// A position in the step sequence of a workgroup.  The segments are listed in LDS once, at the start; all
+// fields are uniform over the workgroup and live in scalar registers.
+struct SegWalk {
+    int seg;                      // index of the current segment
+    int item;                     // its work item, -1 past the end of the sequence
+    int st, st_hi;                // current step, end of the current segment
+    int tile, otile, wg;          // the item's position tile, output tile, weight group
+};
+D2C_DEV void seg_load(SegWalk &w, const int4 *s_seg, int nseg)
+{
+    if (w.seg < nseg) {
+        const int4 u = s_seg[2 * w.seg], v = s_seg[2 * w.seg + 1];
+        w.item = __builtin_amdgcn_readfirstlane(u.x);
+        w.st = __builtin_amdgcn_readfirstlane(u.y);
+        w.st_hi = __builtin_amdgcn_readfirstlane(u.z);
+        w.tile = __builtin_amdgcn_readfirstlane(v.x);
+        w.otile = __builtin_amdgcn_readfirstlane(v.y);
+        w.wg = __builtin_amdgcn_readfirstlane(v.z);
+    } else {
+        w.item = -1; w.st = 0; w.st_hi = 0x7fffffff;
+    }
+}
+// one step on; true when that entered a new segment
+D2C_DEV bool seg_advance(SegWalk &w, const int4 *s_seg, int nseg)
+{
+    if (++w.st < w.st_hi) return false;
+    w.seg++;
+    seg_load(w, s_seg, nseg);
+    return true;
+}
+
+// (The LDS regions are passed as restrict-qualified pointers: that gives their accesses alias scopes, without
+// which the compiler makes every LDS store wait for all DMA transfers in flight, whatever region they fill.)
 template <typename T, bool AUX16, int WAVES_O, int WAVES_P>
-__global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
+D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, unsigned char *__restrict__ s_tile,
+                          float *__restrict__ s_w, int *__restrict__ s_idx, int *__restrict__ s_flag,
+                          int4 *__restrict__ s_seg)
 {
     constexpr int MT = kDMT;
     constexpr int VEC = Elem<T>::VEC;
@@ -285,47 +339,67 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
     static_assert(MT * kNV == kThreads, "one (position, vector) item per thread");
     static_assert(WAVES_O * WAVES_P <= kThreads / 64 && PB >= 1, "MMA wave layout");
 
-    extern __shared__ __align__(16) unsigned char smem[];
-    unsigned char *s_raw = smem;                                   // [2][MT][8 corners][128 B]
-    unsigned char *s_tile = s_raw + 2 * MT * kRawPos;              // [2][MT][kRS]
-    float *s_w = reinterpret_cast<float *>(s_tile + 2 * MT * kRS); // [3][8][MT]
-    int *s_idx = reinterpret_cast<int *>(s_w + 3 * 8 * MT);        // [3][MT]
-    int *s_flag = s_idx + 3 * MT;                                  // [3][MT]
-
     const TiledShape &s = a.s;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
-    const int otile = blockIdx.y / a.nsplit, split = blockIdx.y - otile * a.nsplit, wg = blockIdx.z;
-    const int m0 = tile * MT;
     const int S = s.nchunk * s.K;
-    const int st_lo = (int)((long)S * split / a.nsplit);
-    const int st_hi = (int)((long)S * (split + 1) / a.nsplit);
     const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;
+
+    // --- the step sequence of this workgroup: its whole items, then its pieces of the last round's items
+    const int nwg = (int)gridDim.x;
+    const int bid = xcd_swizzle(blockIdx.x, nwg);
+    const int ntail = a.sk_items - a.sk_full, npiece = ntail * a.sk_cut;
+    const int nwhole_mine = bid < a.sk_full ? (a.sk_full - bid + nwg - 1) / nwg : 0;
+    const int npiece_mine = bid < npiece ? (npiece - bid + nwg - 1) / nwg : 0;
+    const int nseg = nwhole_mine + npiece_mine;        // <= kMaxSeg
+    if (nseg == 0) return;
+    if (tid < nseg) {
+        int item, lo, hi;
+        if (tid < nwhole_mine) {
+            item = bid + tid * nwg; lo = 0; hi = S;
+        } else {
+            const int piece = bid + (tid - nwhole_mine) * nwg, range = piece / ntail;
+            item = a.sk_full + (piece - range * ntail);
+            lo = (int)((long)S * range / a.sk_cut);
+            hi = (int)((long)S * (range + 1) / a.sk_cut);
+        }
+        s_seg[2 * tid] = make_int4(item, lo, hi, 0);
+        s_seg[2 * tid + 1] = make_int4(item % a.sk_ntile, (item / a.sk_ntile) % a.sk_otiles,
+                                       item / (a.sk_ntile * a.sk_otiles), 0);
+    }
+    __syncthreads();
+    int total = 0;
+    for (int q = 0; q < nseg; q++) total += __builtin_amdgcn_readfirstlane(s_seg[2 * q].z - s_seg[2 * q].y);
+    SegWalk w0;
+    w0.seg = 0;
+    seg_load(w0, s_seg, nseg);
 
     // --- coordinates: a ninth wavefront (one position per lane) that does nothing else, so that this
     // arithmetic runs beside the work of the other eight instead of in front of their barrier
     const bool cwave = wave == 8;        // coordinates
     const bool worker = wave < 8;
     const int ctid = tid - kThreads;
-    int cb = 0, cp = 0, coz = 0, coy = 0, cox = 0;
-    bool cvalid = false;
-    if (cwave) {
-        const int m = m0 + ctid;
-        cvalid = m < s.M;
-        if (cvalid) {
-            cb = m / s.P; cp = m - cb * s.P;
-            cox = cp % s.Wo; coy = (cp / s.Wo) % s.Ho; coz = cp / (s.Wo * s.Ho);
+    // The lane's position within a work item.  Offsets are requested (issue) one iteration before they are
+    // turned into a table row (finish), possibly across a segment boundary: one set of constants for each.
+    struct PosC { int b, p, oz, oy, ox; bool valid; };
+    auto pos_of = [&](const SegWalk &w) {
+        PosC c{0, 0, 0, 0, 0, false};
+        const int m = w.tile * MT + ctid;
+        c.valid = w.item >= 0 && m < s.M;
+        if (c.valid) {
+            c.b = m / s.P; c.p = m - c.b * s.P;
+            c.ox = c.p % s.Wo; c.oy = (c.p / s.Wo) % s.Ho; c.oz = c.p / (s.Wo * s.Ho);
         }
-    }
+        return c;
+    };
     float craw[4];
-    auto coords_issue = [&](int st) {
-        if (cwave && cvalid) {
-            const int j = st / s.K, k = st - j * s.K;
-            const int g = (wg * s.cg + j * BKC) / s.cpg;
-            const long ab = (((long)cb * s.G + g) * s.K + k) * s.P + cp;
+    auto coords_issue = [&](const SegWalk &w, const PosC &c) {
+        if (cwave && c.valid) {
+            const int j = w.st / s.K, k = w.st - j * s.K;
+            const int g = (w.wg * s.cg + j * BKC) / s.cpg;
+            const long ab = (((long)c.b * s.G + g) * s.K + k) * s.P + c.p;
             if (s.nd == 3) {
-                const long ob = 3 * ab - 2 * (long)cp;
+                const long ob = 3 * ab - 2 * (long)c.p;
                 craw[0] = ld_auxT<AUX16>(a.off, ob);
                 craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
                 craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
@@ -336,46 +410,49 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
         }
     };
-    auto coords_finish = [&](int st, int buf) {
+    auto coords_finish = [&](const SegWalk &w, const PosC &c, int buf) {
         if (cwave) {
-            float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            float wt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             int idx = 0;
             unsigned live = 0;
-            if (cvalid) {
-                const int k = st % s.K;
+            if (c.valid) {
+                const int k = w.st % s.K;
                 int bz, by, bx;
-                tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
+                tap_base(s.geo, k, c.oz, c.oy, c.ox, bz, by, bx);
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
                 live = t.live;
-                idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
+                idx = (c.b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
 #pragma unroll
-                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * craw[3] : 0.f;
+                for (int q = 0; q < 8; q++) wt[q] = ((live >> q) & 1u) ? tap3_weight(t, q) * craw[3] : 0.f;
             }
 #pragma unroll
-            for (int c = 0; c < 8; c++) s_w[(buf * 8 + c) * MT + ctid] = w[c];
+            for (int q = 0; q < 8; q++) s_w[(buf * 8 + q) * MT + ctid] = wt[q];
             s_idx[buf * MT + ctid] = idx;
             s_flag[buf * MT + ctid] = (int)live;
         }
     };
 
-    // --- corner rows of step st -> s_raw[rbuf]: worker wavefront w requests positions 8w .. 8w+7, one
+    // --- corner rows of a step -> s_raw[rbuf]: worker wavefront w requests positions 8w .. 8w+7, one
     // instruction per position, lane = (corner, 16-byte vector)
     const int dcorner = lane >> 3, dvec = lane & 7;
     const int dcoff = ((dcorner >> 2) & 1) * dzc + ((dcorner >> 1) & 1) * dyc + (dcorner & 1) * s.Cin;
-    auto dma_issue = [&](int st, int rbuf, int tbuf) {
+    auto dma_issue = [&](const SegWalk &w, int rbuf, int tbuf) {
         if (!worker) return;
-        const int j = st / s.K;
-        const int c0 = wg * s.cg + j * BKC;
+        const int j = w.st / s.K;
+        const int c0 = w.wg * s.cg + j * BKC;
         const char *base = reinterpret_cast<const char *>(a.xcl);
         // table entries of this wavefront's 8 positions: one LDS read (lane i holds position i), then
         // lane-indexed moves to scalar registers
         const int vidx = s_idx[tbuf * MT + wave * (MT / 8) + (lane & 7)];
         const int vflag = s_flag[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const unsigned vmask = w.item >= 0 ? 0xffu : 0u;
 #pragma unroll
         for (int i = 0; i < MT / 8; i++) {
             const int pos = wave * (MT / 8) + i;
             const int idx = __builtin_amdgcn_readlane(vidx, i);
-            const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
+            // (past the end of the sequence every lane fetches the row of zeros: the same number of transfers
+            // in every iteration, which lets the compiler count the loads in flight instead of waiting for all)
+            const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i) & vmask;
             const unsigned o = ((live >> dcorner) & 1u)
                                    ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
                                    : a.zrow + (unsigned)dvec * 16u;
@@ -410,11 +487,14 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
             for (int r = 0; r < 16; r++) acc[ob][pb][r] = 0.f;
     const uint4 *wp4 = reinterpret_cast<const uint4 *>(a.wp);
     uint4 af[NKG][OB];
-    auto wfrag = [&](int st, int kg, int ob) {
-        const long wbase = (((long)wg * S + st) * OBT + (otile * (NT / 32) + wave_o * OB)) * NKG * 64 + lane;
+    auto wfrag = [&](const SegWalk &w, int kg, int ob) {
+        // (past the end of the sequence: any valid address, the fragments are not used)
+        const int wgq = w.item >= 0 ? w.wg : 0, stq = w.item >= 0 ? w.st : 0, otq = w.item >= 0 ? w.otile : 0;
+        const long wbase = (((long)wgq * S + stq) * OBT + (otq * (NT / 32) + wave_o * OB)) * NKG * 64 + lane;
         return wp4[wbase + ((long)ob * NKG + kg) * 64];
     };
-    auto mma_step = [&](int st, int dbuf) {
+    // one step on the matrix cores; the weight fragments of the step after it (at `wn`) are fetched meanwhile
+    auto mma_step = [&](int dbuf, const SegWalk &wn) {
         if (!mma_wave) return;
         const unsigned char *tb = s_tile + (dbuf * MT + wave_p * WPOS + (lane & 31)) * kRS + (lane >> 5) * 16;
 #pragma unroll
@@ -427,96 +507,217 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
             for (int ob = 0; ob < OB; ob++)
 #pragma unroll
                 for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[kg][ob], bf[pb]);
-            if (st + 1 < st_hi) {
 #pragma unroll
-                for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(st + 1, kg, ob);
+            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(wn, kg, ob);
+        }
+    };
+    // end of a segment: whole items get bias, conversion and store; pieces of an item add into its fp32 tile
+    auto flush_acc = [&](const SegWalk &w) {
+        if (!mma_wave) return;
+        // (an opaque copy of the lane number: the address arithmetic below depends on nothing else that changes
+        // from step to step, and must not be computed ahead of the step loop and kept in registers)
+        int elane = lane;
+        asm volatile("" : "+v"(elane));
+        const int ot0 = wave_o * 64 + 4 * (elane >> 5);      // first output channel of this lane within the tile
+        const int nvalid = s.og - (w.otile * NT + ot0);       // channels from there on that exist
+        const int o0 = w.wg * s.og + w.otile * NT + ot0;
+        if (w.item >= a.sk_full) {
+            float *tp = a.outacc + ((long)(w.item - a.sk_full) * NT + ot0) * MT + wave_p * WPOS + (elane & 31);
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int oo = ob * 32 + 8 * (r >> 2) + (r & 3);
+                        if (oo < nvalid) atomicAdd(tp + oo * MT + pb * 32, acc[ob][pb][r]);
+                        acc[ob][pb][r] = 0.f;
+                    }
+        } else {
+            const T *bias = reinterpret_cast<const T *>(a.bias);
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++) {
+                const int m = w.tile * MT + wave_p * WPOS + pb * 32 + (elane & 31);
+                const bool ok = m < s.M;
+                const int b = m / s.P, p = m - b * s.P;
+                T *op = reinterpret_cast<T *>(a.out) + ((long)b * s.Cout + o0) * s.P + p;
+#pragma unroll
+                for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int oo = ob * 32 + 8 * (r >> 2) + (r & 3);
+                        if (ok && oo < nvalid) {
+                            float v = acc[ob][pb][r];
+                            if (bias) v += elem_to_f32<T>(bias[o0 + oo]);
+                            op[(long)oo * s.P] = f32_to_elem<T>(v);
+                        }
+                        acc[ob][pb][r] = 0.f;
+                    }
             }
         }
     };
 
-    // --- pipeline.  Iteration `it`: rows of step it+2 requested, step it on the matrix cores, step it+1
-    // interpolated, coordinates of step it+3 computed.  Corner tables rotate over 3 buffers, raw rows and
-    // tiles over 2.  Everything requested in one iteration has that whole iteration to arrive.
+    // --- pipeline.  Iteration `it` of the step sequence: step it on the matrix cores, step it+1 interpolated,
+    // rows of step it+2 requested, coordinates of step it+3 computed.  Corner tables rotate over 3 buffers,
+    // raw rows and tiles over 2.  A wavefront interpolates the positions whose rows it requested itself, so the
+    // rows need no barrier, only that wavefront's own wait.
+    SegWalk wc = w0;                  // coordinates: the step whose offsets are requested next
+    PosC pc = pos_of(wc);
     for (int q = 0; q < 3; q++) {
-        if (st_lo + q < st_hi) {
-            coords_issue(st_lo + q);
-            coords_finish(st_lo + q, (st_lo + q) % 3);
+        if (q < total) {
+            coords_issue(wc, pc);
+            coords_finish(wc, pc, q);
+            if (seg_advance(wc, s_seg, nseg)) pc = pos_of(wc);
         }
     }
+    SegWalk wf = wc;                  // coordinates: the step whose table row is computed next
+    PosC pf = pc;
+    SegWalk wm = w0, wn = w0, wd = w0;    // steps: on the matrix cores / after that one / rows requested next
+    seg_advance(wn, s_seg, nseg);
     if (mma_wave) {
 #pragma unroll
         for (int kg = 0; kg < NKG; kg++)
 #pragma unroll
-            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(st_lo, kg, ob);
+            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(wm, kg, ob);
     }
     __syncthreads();
-    dma_issue(st_lo, st_lo & 1, st_lo % 3);
-    if (st_lo + 1 < st_hi) dma_issue(st_lo + 1, (st_lo + 1) & 1, (st_lo + 1) % 3);
+    dma_issue(wd, 0, 0);
+    seg_advance(wd, s_seg, nseg);
+    if (1 < total) {
+        dma_issue(wd, 1, 1);
+        seg_advance(wd, s_seg, nseg);
+    }
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    interp_store(st_lo & 1, st_lo % 3, st_lo & 1);
-    if (st_lo + 3 < st_hi) coords_issue(st_lo + 3);
+    interp_store(0, 0, 0);
+    if (3 < total) {
+        coords_issue(wc, pc);
+        if (seg_advance(wc, s_seg, nseg)) pc = pos_of(wc);
+    }
     // One loop per role (separate register budgets), the same synchronisation point per iteration in each.
     if (worker) {
-        for (int it = st_lo; it < st_hi; it++) {
-            __builtin_amdgcn_s_waitcnt(0);     // the transfers requested in the last iteration have landed
-            __syncthreads();
-            mma_step(it, it & 1);
-            if (it + 2 < st_hi) dma_issue(it + 2, it & 1, (it + 2) % 3);
-            if (it + 1 < st_hi) interp_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
+        // (one inner loop per segment, so that the code that stores the accumulators stays out of the loop
+        // over steps; nothing but the accumulators knows where a segment ends)
+        int it = 0;
+        while (wm.item >= 0) {
+            for (; wm.st < wm.st_hi; wm.st++, it++) {
+                lds_barrier();
+                mma_step(it & 1, wn);
+                // The rows of step it+1, requested one iteration ago by this same wavefront (it interpolates the
+                // positions whose rows it requested), have had the barrier and the matrix-core phase to arrive;
+                // only the NKG * OB weight-fragment loads of mma_step are younger and may stay in flight.
+                static_assert(NKG * OB == 8, "the wait below counts the weight-fragment loads");
+                __builtin_amdgcn_s_waitcnt(0x0F78);     // vmcnt(8)
+                if (it + 1 < total) interp_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
+                dma_issue(wd, it & 1, (it + 2) % 3);
+                if (wd.item >= 0) seg_advance(wd, s_seg, nseg);
+                if (wn.item >= 0) seg_advance(wn, s_seg, nseg);
+            }
+            flush_acc(wm);
+            wm.seg++;
+            seg_load(wm, s_seg, nseg);
         }
     } else {
-        for (int it = st_lo; it < st_hi; it++) {
-            __syncthreads();
-            if (it + 3 < st_hi) coords_finish(it + 3, it % 3);   // offsets requested one iteration ago
-            if (it + 4 < st_hi) coords_issue(it + 4);
-        }
-    }
-
-    // --- epilogue: bias, convert, store
-    if (mma_wave) {
-        T *out = reinterpret_cast<T *>(a.out);
-        const T *bias = reinterpret_cast<const T *>(a.bias);
-#pragma unroll
-        for (int pb = 0; pb < PB; pb++) {
-            const int m = m0 + wave_p * WPOS + pb * 32 + (lane & 31);
-            if (m >= s.M) continue;
-            const int b = m / s.P, p = m - b * s.P;
-#pragma unroll
-            for (int ob = 0; ob < OB; ob++) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int ol = otile * NT + wave_o * 64 + ob * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    if (ol < s.og) {
-                        const int o = wg * s.og + ol;
-                        float v = acc[ob][pb][r];
-                        if (a.outacc) {
-                            atomicAdd(a.outacc + ((long)b * s.Cout + o) * s.P + p, v);
-                        } else {
-                            if (bias) v += elem_to_f32<T>(bias[o]);
-                            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(v);
-                        }
-                    }
-                }
+        for (int it = 0; it < total; it++) {
+            lds_barrier();
+            if (it + 3 < total) {                      // offsets requested one iteration ago
+                coords_finish(wf, pf, it % 3);
+                if (seg_advance(wf, s_seg, nseg)) pf = pos_of(wf);
+            }
+            if (it + 4 < total) {
+                coords_issue(wc, pc);
+                if (seg_advance(wc, s_seg, nseg)) pc = pos_of(wc);
             }
         }
     }
 }
 
-constexpr size_t kFwdDmaLds = (size_t)2 * kDMT * kRawPos + (size_t)2 * kDMT * kRS + (size_t)3 * 10 * kDMT * 4;
+template <typename T, bool AUX16, int WAVES_O, int WAVES_P>
+__global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
+{
+    constexpr int MT = kDMT;
+    // (separate arrays, not slices of one: the compiler then knows which of them a DMA transfer fills, and
+    // lets accesses to the others go ahead while transfers are in flight)
+    __shared__ __align__(16) unsigned char s_raw[2 * MT * kRawPos];   // [2][MT][8 corners][128 B]
+    __shared__ __align__(16) unsigned char s_tile[2 * MT * kRS];      // [2][MT][kRS]
+    __shared__ float s_w[3 * 8 * MT];                                 // [3][8][MT]
+    __shared__ int s_idx[3 * MT];                                     // [3][MT]
+    __shared__ int s_flag[3 * MT];                                    // [3][MT]
+    __shared__ int4 s_seg[2 * kMaxSeg];                               // [kMaxSeg][2]
+    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P>(a, s_raw, s_tile, s_w, s_idx, s_flag, s_seg);
+}
+
+// out = fp32 tile + bias for the items whose steps were shared out (see FwdArgs).  One block = 32 output
+// channels of one such item.
+template <typename T>
+__global__ void __launch_bounds__(256) fwd_dma_finish_kernel(FwdArgs a, int NT)
+{
+    constexpr int MT = kDMT;
+    const TiledShape &s = a.s;
+    const int item = a.sk_full + blockIdx.x;
+    const int tile = item % a.sk_ntile, otile = (item / a.sk_ntile) % a.sk_otiles, wg = item / (a.sk_ntile * a.sk_otiles);
+    const float *acc = a.outacc + (long)blockIdx.x * NT * MT;
+    const T *bias = reinterpret_cast<const T *>(a.bias);
+    T *out = reinterpret_cast<T *>(a.out);
+    for (int e = threadIdx.x; e < 32 * MT; e += 256) {
+        const int ot = blockIdx.y * 32 + e / MT, pl = e % MT;
+        const int ol = otile * NT + ot, m = tile * MT + pl;
+        if (ol < s.og && m < s.M) {
+            const int o = wg * s.og + ol, b = m / s.P, p = m - b * s.P;
+            float v = acc[(long)ot * MT + pl];
+            if (bias) v += elem_to_f32<T>(bias[o]);
+            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(v);
+        }
+    }
+}
 
 template <typename T, bool AUX16, int WO, int WP>
-int launch_fwd_dma(const FwdArgs &a, hipStream_t st)
+int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
 {
-    const int ntile = (a.s.M + kDMT - 1) / kDMT;
-    const int NT = 64 * WO;
-    if (hipFuncSetAttribute((const void *)tiled_fwd_dma_kernel<T, AUX16, WO, WP>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-        return d2c_check_launch("hipFuncSetAttribute(tiled_fwd_dma_kernel)");
-    dim3 grid(ntile, a.s.ogp / NT * a.nsplit, a.s.groups);
-    D2cProfScope prof(D2C_PROF_FWD, st);
-    hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP>), grid, dim3(kThreads + 64), kFwdDmaLds, st, a);
-    return d2c_check_launch("tiled_fwd_dma_kernel");
+    constexpr int NT = 64 * WO;
+    const int ncu = d2c_num_cus();
+    if (ncu <= 0) return D2C_ERR_LAUNCH;
+    a.sk_ntile = (a.s.M + kDMT - 1) / kDMT;
+    a.sk_otiles = a.s.ogp / NT;
+    a.sk_items = a.sk_ntile * a.sk_otiles * a.s.groups;
+    // The last, partial round: cut its items into the number of step ranges that is estimated to finish first
+    // (a piece costs its steps plus about two steps' time for adding its result).
+    // A workgroup lists at most kMaxSeg segments: very large problems get more workgroups than compute units
+    // (and no cut of their last round, which is a small part of them).
+    const int S = a.s.nchunk * a.s.K;
+    const int maxwhole = kMaxSeg / 2;
+    const int nwg_whole = a.sk_items > (long)ncu * maxwhole ? (a.sk_items + maxwhole - 1) / maxwhole : ncu;
+    const int tail = nwg_whole == ncu ? a.sk_items % ncu : 0;
+    a.sk_full = a.sk_items;
+    a.sk_cut = 1;
+    if (tail && outacc) {
+        long best = S;
+        for (int k = 2; k <= kMaxSeg / 2 && k <= S; k++) {
+            const long rounds = ((long)tail * k + ncu - 1) / ncu;
+            const long cost = rounds * ((S + k - 1) / k + 2);
+            if (cost < best) { best = cost; a.sk_cut = k; }
+        }
+        if (a.sk_cut > 1 && best * 10 < (long)S * 9) a.sk_full = a.sk_items - tail; else a.sk_cut = 1;
+    }
+    const int nshare = a.sk_items - a.sk_full;
+    a.outacc = nshare ? outacc : nullptr;
+    a.nsplit = 1;
+    if (nshare) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(outacc, (size_t)nshare * NT * kDMT * sizeof(float), st);
+    }
+    {
+        const int nwg = nshare ? ncu : (a.sk_items < nwg_whole ? a.sk_items : nwg_whole);
+        D2cProfScope prof(D2C_PROF_FWD, st);
+        hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        if (int rc = d2c_check_launch("tiled_fwd_dma_kernel")) return rc;
+    }
+    if (nshare) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        hipLaunchKernelGGL(fwd_dma_finish_kernel<T>, dim3(nshare, NT / 32), dim3(256), 0, st, a, NT);
+        return d2c_check_launch("fwd_dma_finish_kernel");
+    }
+    return 0;
 }
 
 // out = outacc + bias, in the element type of the output
@@ -575,6 +776,8 @@ int d2c_fwd_out_tile(int og, int M, int groups)
 // Workgroups per (position tile, output tile): 1 when the tiles alone fill the chip.
 int d2c_fwd_split(const TiledShape &s)
 {
+    // the DMA-gather kernel shares out the steps of its last round of work items, whatever their number
+    if (d2c_fwd_use_dma(s.og, s.M, s.groups)) return 2;
     const int mt = d2c_fwd_pos_tile(s.og, s.M, s.groups), nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
     const long wgs = (long)((s.M + mt - 1) / mt) * (s.ogp / nt) * s.groups;
     if (wgs >= 128) return 1;
@@ -587,25 +790,25 @@ template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
                          const void *bias, void *out, float *outacc, hipStream_t st)
 {
-    const int nsplit = outacc ? d2c_fwd_split(s) : 1;
+    const bool dma = d2c_fwd_use_dma(s.og, s.M, s.groups);
+    const int nsplit = (outacc && !dma) ? d2c_fwd_split(s) : 1;
     const long n = (long)s.N * s.Cout * s.P;
     // the channels-last input is followed by a row of zeros (see forward_t)
     const unsigned zrow = (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T));
-    FwdArgs a{s, xcl, off, mask, wp, bias, out, nsplit > 1 ? outacc : nullptr, nsplit, zrow};
+    FwdArgs a{s, xcl, off, mask, wp, bias, out, nsplit > 1 ? outacc : nullptr, nsplit, zrow, 0, 0, 0, 0, 1};
     if (nsplit > 1) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(outacc, (size_t)n * sizeof(float), st);
     }
     const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
-    const bool dma = d2c_fwd_use_dma(s.og, s.M, s.groups);
-    int rc;
+    int rc = 0;
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
     if (dma) {
         if constexpr (sizeof(T) == 2) {
-            if (aux16) rc = launch_fwd_dma<T, true, 8, 1>(a, st);
+            if (aux16) return launch_fwd_dma<T, true, 8, 1>(a, outacc, st);
         }
-        if (!aux16) rc = launch_fwd_dma<T, false, 8, 1>(a, st);
+        return launch_fwd_dma<T, false, 8, 1>(a, outacc, st);
     } else {
         if constexpr (sizeof(T) == 2) {
             if (aux16) rc = launch_fwd_cfg<T, true>(a, nt, st);
