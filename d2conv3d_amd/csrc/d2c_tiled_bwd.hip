@@ -820,7 +820,24 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
     const int omax = d2c_bwd_pass_channels(Elem<T>::DT);
-    const int nsplit = auxacc ? d2c_bwd_data_split(s, Elem<T>::DT) : 1;
+    int nsplit = auxacc ? d2c_bwd_data_split(s, Elem<T>::DT) : 1;
+    if (gcolbuf && !gxcl && !goff && !gmask) {
+        // Only the grad-column product is wanted: every (tile, step) writes its own part of the result, so the
+        // steps can be cut into ranges at no cost but the reload of the stationary operand.  Workgroups are
+        // dispatched range-major (blockIdx.z slowest), which keeps those running at one time on the same weight
+        // tiles; the cut is the one whose last round of workgroups is fullest.
+        const int ncu = d2c_num_cus();
+        if (ncu <= 0) return D2C_ERR_LAUNCH;
+        constexpr int MT = 32 * (8 / (BKC / 32));
+        const long items = (long)((s.M + MT - 1) / MT) * s.groups;
+        const int S = s.nchunk * s.K;
+        long best = ((items + ncu - 1) / ncu) * (S + 1);
+        nsplit = 1;
+        for (int k = 2; k <= 16 && k <= S; k++) {
+            const long cost = ((items * k + ncu - 1) / ncu) * ((S + k - 1) / k + 1);
+            if (cost < best) { best = cost; nsplit = k; }
+        }
+    }
     const long n_mask = (long)s.N * s.G * s.K * s.P, n_off = n_mask * s.nd;
     float *auxoff = nullptr, *auxmask = nullptr;
     if (nsplit > 1 && (goff || gmask)) {
@@ -893,9 +910,20 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
                            ntp, OBT, total);
         if (int rc = d2c_check_launch("pack_gout_kernel")) return rc;
     }
-    int split = (512 + steps * otiles * s.groups - 1) / (steps * otiles * s.groups);
-    if (split > ntile) split = ntile;
-    if (split < 1) split = 1;
+    // Position tiles of a step are dealt to `split` workgroups; one workgroup runs per compute unit at a time.
+    // The split is the one whose rounds of workgroups are estimated to finish first (a workgroup costs its tiles
+    // plus about six tiles' time for filling its pipeline and adding its result).
+    const int ncu = d2c_num_cus();
+    if (ncu <= 0) return D2C_ERR_LAUNCH;
+    int split = 1;
+    {
+        const long items = (long)steps * otiles * s.groups;
+        long best = -1;
+        for (int k = 1; k <= 32 && k <= ntile; k++) {
+            const long cost = ((items * k + ncu - 1) / ncu) * ((ntile + k - 1) / k + 6);
+            if (best < 0 || cost < best) { best = cost; split = k; }
+        }
+    }
     BwdWeightDmaArgs a{{s, gout, xcl, off, mask, goutp, gwacc, split},
                        (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T))};
     {
