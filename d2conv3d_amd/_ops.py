@@ -291,5 +291,6 @@ def set_algo_override(name):
 
 def set_grad_input_mode(mode):
     """Test hook: "lists" (default; grad_input gathered from per-voxel sample lists, every element
-    written once) or "atomics" (scatter with fp32 atomics like the reference)."""
-    _lib.load().d2c_set_grad_input_mode({"lists": 1, "atomics": 0}[mode])
+    written once), "atomics" (scatter with fp32 atomics like the reference), or an int n >= 2: lists of
+    at most n samples per voxel, the rest taking the overflow path."""
+    _lib.load().d2c_set_grad_input_mode(mode if isinstance(mode, int) else {"lists": 1, "atomics": 0}[mode])

@@ -44,6 +44,7 @@ struct AuxArgs {
     const void *gcol;    // [chunk][tap][N*P][BKC]
     void *goff, *gmask;  // or NULL
     int ntile;           // position tiles
+    SampleLists lists;   // counts != NULL: every live sample is filed in its bucket on the way (for grad_input)
 };
 
 template <typename T, bool AUX16>
@@ -98,6 +99,8 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     if (k_lo < k_hi) coords_issue(k_lo);
 
     for (int k = k_lo; k < k_hi; k++) {
+        int lbin = -1, lslot = 0;
+        float lhx = 0.f;
         // ---- corner table of the 64 positions for tap k
         {
             float fr[6] = {0, 0, 0, 0, 0, 0};
@@ -112,6 +115,13 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                 idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
                 unsigned inr = t.inrange, auxlive = t.live;
                 fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
+                if (a.lists.counts && t.live) {
+                    // a place in the sample's bucket is asked for now, the entry is written after the dot
+                    // products of this tap, when the answer has long arrived
+                    lbin = bin_of(s, cb, g, t.z0, t.y0, t.x0);
+                    lslot = lists_reserve(a.lists, lbin);
+                    lhx = t.hx;
+                }
                 if (s.nd == 1) {
                     // 1-D: both corners are gated by range only (dconv1d_gpu.cu:338-339), and at integer
                     // positions the low corner steps down by one while the high corner stays (:332-336);
@@ -243,6 +253,12 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                 }
             }
         }
+        if (lbin >= 0) {
+            InvEntry e;
+            e.p = cp; e.k = k; e.hz = s_tab[5][lane]; e.hy = s_tab[6][lane]; e.hx = lhx; e.alpha = s_tab[8][lane];
+            e.pad0 = 0; e.pad1 = 0;
+            lists_store(a.lists, lbin, lslot, e);
+        }
     }
 }
 
@@ -252,10 +268,10 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 // channel count is a multiple of the chunk width.
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, hipStream_t st)
+                        void *goff, void *gmask, const SampleLists *lists, hipStream_t st)
 {
     const int ntile = (s.M + kMT - 1) / kMT;
-    AuxArgs a{s, xcl, off, mask, gcol, goff, gmask, ntile};
+    AuxArgs a{s, xcl, off, mask, gcol, goff, gmask, ntile, lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}};
     dim3 grid((ntile + kWavesPerBlock - 1) / kWavesPerBlock, s.G, s.K < kTapSplit ? s.K : kTapSplit);
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
@@ -267,6 +283,6 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     return d2c_check_launch("aux_grad_kernel");
 }
 template int d2c_aux_grad_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                         void *, void *, hipStream_t);
+                                         void *, void *, const SampleLists *, hipStream_t);
 template int d2c_aux_grad_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                        void *, void *, hipStream_t);
+                                        void *, void *, const SampleLists *, hipStream_t);

@@ -18,6 +18,8 @@
 #include "d2c_mma.hpp"
 #include "d2c_tiled.hpp"
 
+int d2c_gx_mode();
+
 namespace {
 
 D2C_DEV int xcd_swizzle(int bid, int n)
@@ -27,17 +29,27 @@ D2C_DEV int xcd_swizzle(int bid, int n)
     return x * q + (x < r ? x : r) + idx;
 }
 
-struct alignas(16) InvEntry {
-    int p, k;              // output position inside the sample, tap
-    float hz, hy, hx;      // fractions z - floor(z), ...
-    float alpha;           // modulation
-    int pad0, pad1;
-};
-static_assert(sizeof(InvEntry) == 32, "two 16-byte loads per entry");
-
-D2C_DEV int bin_of(const TiledShape &s, int b, int g, int z0, int y0, int x0)
+// One pass over the samples that files them in the buckets (the offset / mask gradient kernel does the same
+// on its way when it runs, see d2c_aux_grad.hip).
+__global__ void __launch_bounds__(256)
+lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L)
 {
-    return (((b * s.G + g) * (s.D + 1) + (z0 + 1)) * (s.H + 1) + (y0 + 1)) * (s.W + 1) + (x0 + 1);
+    const int k = blockIdx.y;
+    const int b = blockIdx.z / s.G, g = blockIdx.z - b * s.G;
+    for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < s.P; p += gridDim.x * blockDim.x) {
+        const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
+        float o0, o1, o2;
+        load_offsets(s, off, b, g, k, p, o0, o1, o2);
+        int bz, by, bx;
+        tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
+        const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+        if (!t.live) continue;
+        InvEntry e;
+        e.p = p; e.k = k; e.hz = t.hz; e.hy = t.hy; e.hx = t.hx;
+        e.alpha = mask ? ld_aux(mask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt) : 1.f;
+        e.pad0 = 0; e.pad1 = 0;
+        lists_insert(L, bin_of(s, b, g, t.z0, t.y0, t.x0), e);
+    }
 }
 
 template <bool FILL>
@@ -144,7 +156,7 @@ __global__ void set_total(const int *counts, int *starts, int n)
 // contiguous range of entries, the x offset of an entry follows from its place in the range.
 template <typename T>
 __global__ void __launch_bounds__(256)
-gx_owner_cube_kernel(TiledShape s, const T *gcol, const int *starts, const InvEntry *entries, float *gxcl)
+gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
     const int sub = threadIdx.x & 7, ci = threadIdx.x >> 3;       // 32 cubes per workgroup: 2 x 4 x 4 of them
@@ -174,15 +186,20 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, const int *starts, const InvEn
         for (int ry = 0; ry < 3; ry++) {
             const int yb = y0 - 1 + ry;
             if (yb > s.H - 1) continue;
+            // the buckets of the (up to) three bins, walked as one range: [0, em1) | [em1, em2) | [em2, e1)
             const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
-            const int e0 = starts[bin1], em1 = starts[bin1 + 1], em2 = starts[bin1 + 2], e1 = starts[bin1 + nxb];
-            for (int e = e0; e < e1; e += 4) {
+            const int em1 = min(L.counts[bin1], L.cap);
+            const int em2 = em1 + min(L.counts[bin1 + 1], L.cap);
+            const int e1 = em2 + (nxb == 3 ? min(L.counts[bin1 + 2], L.cap) : 0);
+            const InvEntry *eb = L.entries + (long)bin1 * L.cap;
+            for (int e = 0; e < e1; e += 4) {
                 uint4 q0[4], q1[4], row[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int ei = min(e + i, e1 - 1);
-                    q0[i] = reinterpret_cast<const uint4 *>(entries + ei)[0];
-                    q1[i] = reinterpret_cast<const uint4 *>(entries + ei)[1];
+                    const int slot = ei < em1 ? ei : (ei < em2 ? ei - em1 + L.cap : ei - em2 + 2 * L.cap);
+                    q0[i] = reinterpret_cast<const uint4 *>(eb + slot)[0];
+                    q1[i] = reinterpret_cast<const uint4 *>(eb + slot)[1];
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -239,6 +256,42 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, const int *starts, const InvEn
                                                                          acc[az][ay][ax][i + 2], acc[az][ay][ax][i + 3]);
                 }
             }
+}
+
+// Samples that found their bucket full: added into grad_input with atomics, after the owner kernel has written
+// it.  One 8-lane group per (overflow entry, channel chunk of its offset group).
+template <typename T>
+__global__ void __launch_bounds__(256)
+gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
+    const int novf = min(L.counts[L.nbins], L.ovf_cap);
+    const int sub = threadIdx.x & 7;
+    const int cpc = s.cpg / BKC;
+    const long ngrp = (long)gridDim.x * 32, total = (long)novf * cpc;
+    for (long w = (long)blockIdx.x * 32 + (threadIdx.x >> 3); w < total; w += ngrp) {
+        const int i = (int)(w / cpc), jj = (int)(w - (long)i * cpc);
+        const InvEntry e = L.ovf[i];
+        int bin = e.pad0;
+        const int x0 = bin % (s.W + 1) - 1; bin /= s.W + 1;
+        const int y0 = bin % (s.H + 1) - 1; bin /= s.H + 1;
+        const int z0 = bin % (s.D + 1) - 1; bin /= s.D + 1;
+        const int g = bin % s.G, b = bin / s.G;
+        const int cidx = (g * s.cpg) / BKC + jj;
+        const uint4 row = *reinterpret_cast<const uint4 *>(gcol + (((long)cidx * s.K + e.k) * s.M + (long)b * s.P + e.p) * BKC
+                                                           + sub * VEC);
+        const T *re = reinterpret_cast<const T *>(&row);
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const int z = z0 + ((c >> 2) & 1), y = y0 + ((c >> 1) & 1), x = x0 + (c & 1);
+            if (z < 0 || z >= s.D || y < 0 || y >= s.H || x < 0 || x >= s.W) continue;
+            const float wgt = ((c & 4) ? e.hz : 1.f - e.hz) * ((c & 2) ? e.hy : 1.f - e.hy) * ((c & 1) ? e.hx : 1.f - e.hx)
+                              * e.alpha;
+            float *o = gxcl + ((long)b * s.vol + ((long)z * s.H + y) * s.W + x) * s.Cin + cidx * BKC + sub * VEC;
+#pragma unroll
+            for (int j = 0; j < VEC; j++) atomicAdd(o + j, wgt * elem_to_f32<T>(re[j]));
+        }
+    }
 }
 
 // ---- owner-computes accumulation, channel-separated (depthwise) case ---------
@@ -384,21 +437,70 @@ int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, in
     return d2c_check_launch("invlist_build");
 }
 
+// Bucket capacity: a power of two above 2.2 x the mean list length K * P / vol (8 .. 256), or what
+// d2c_set_grad_input_mode() asked for.
+int d2c_lists_cap(const TiledShape &s)
+{
+    const int forced = d2c_gx_mode();
+    if (forced >= 2) return forced;
+    const double mean = (double)s.K * s.P / s.vol;
+    int cap = 8;
+    while (cap < 256 && cap < 2.2 * mean) cap *= 2;
+    return cap;
+}
+void d2c_lists_ws(const TiledShape &s, size_t *counts, size_t *entries, size_t *ovf)
+{
+    const long nb = d2c_invlist_bins(s);
+    *counts = d2c_align_up((size_t)(nb + 1) * 4);
+    *entries = d2c_align_up((size_t)nb * d2c_lists_cap(s) * sizeof(InvEntry));
+    *ovf = d2c_align_up((size_t)s.N * s.G * s.K * s.P * sizeof(InvEntry));
+}
+// The lists over the three workspace regions sized by d2c_lists_ws; nbins == 0 when the shape is too large.
+SampleLists d2c_lists_make(const TiledShape &s, void *counts, void *entries, void *ovf)
+{
+    const long nb = d2c_invlist_bins(s), nsamp = (long)s.N * s.G * s.K * s.P;
+    SampleLists L{(int *)counts, (InvEntry *)entries, (InvEntry *)ovf, d2c_lists_cap(s), 0, 0};
+    if (nb < (1L << 31) - 1 && nsamp < (1L << 31)) {
+        L.nbins = (int)nb;
+        L.ovf_cap = (int)nsamp;
+    }
+    return L;
+}
+int d2c_lists_clear(const SampleLists &L, hipStream_t st)
+{
+    if (L.nbins == 0) {
+        d2c_set_error("too many sample bins");
+        return D2C_ERR_UNSUPPORTED;
+    }
+    D2cProfScope prof(D2C_PROF_PACK, st);
+    d2c_fill_zero(L.counts, (size_t)(L.nbins + 1) * 4, st);
+    return d2c_check_launch("lists_clear");
+}
+int d2c_lists_build(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st)
+{
+    if (int rc = d2c_lists_clear(L, st)) return rc;
+    D2cProfScope prof(D2C_PROF_PACK, st);
+    const dim3 pgrid(g1d(s.P, 4096), s.K, s.N * s.G);
+    hipLaunchKernelGGL(lists_pass_kernel, pgrid, dim3(256), 0, st, s, off, mask, L);
+    return d2c_check_launch("lists_pass_kernel");
+}
+
 template <typename T>
-int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts, const void *entries, float *gxcl,
-                        hipStream_t st)
+int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st)
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
     D2cProfScope prof(D2C_PROF_GX_OWNER, st);
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
     dim3 grid((unsigned)nblk, s.Cin / BKC);
-    hipLaunchKernelGGL(gx_owner_cube_kernel<T>, grid, dim3(256), 0, st, s, (const T *)gcol, starts,
-                       (const InvEntry *)entries, gxcl);
-    return d2c_check_launch("gx_owner_kernel");
+    hipLaunchKernelGGL(gx_owner_cube_kernel<T>, grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    if (int rc = d2c_check_launch("gx_owner_kernel")) return rc;
+    // the overflow entries, usually none (the kernel reads their number from device memory)
+    hipLaunchKernelGGL(gx_overflow_kernel<T>, dim3(512), dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    return d2c_check_launch("gx_overflow_kernel");
 }
-template int d2c_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const int *, const void *, float *, hipStream_t);
-template int d2c_gx_owner_launch<float>(const TiledShape &, const void *, const int *, const void *, float *, hipStream_t);
+template int d2c_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const SampleLists &, float *, hipStream_t);
+template int d2c_gx_owner_launch<float>(const TiledShape &, const void *, const SampleLists &, float *, hipStream_t);
 
 // Depthwise case: grad_input from the sample lists, the channels-last grad_out and the tap-major weights.
 template <typename T>

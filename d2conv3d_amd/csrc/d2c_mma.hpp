@@ -135,6 +135,47 @@ struct TiledShape {
     TapGeom geo;
 };
 
+// ---- sample lists: every live sample (b, g, k, p) filed under its base voxel floor(z, y, x) -------------------
+struct alignas(16) InvEntry {
+    int p, k;              // output position inside the sample, tap
+    float hz, hy, hx;      // fractions z - floor(z), ...
+    float alpha;           // modulation
+    int pad0, pad1;        // pad0: the bin, in entries of the overflow array
+};
+static_assert(sizeof(InvEntry) == 32, "two 16-byte loads per entry");
+
+// bins cover base voxels -1 .. size-1 per axis
+D2C_DEV int bin_of(const TiledShape &s, int b, int g, int z0, int y0, int x0)
+{
+    return (((b * s.G + g) * (s.D + 1) + (z0 + 1)) * (s.H + 1) + (y0 + 1)) * (s.W + 1) + (x0 + 1);
+}
+
+// Lists as buckets of fixed capacity, filled in one pass (a counter per bin; no counting pass, no scan).
+// A sample that finds its bucket full goes to one shared overflow array instead, which a separate kernel
+// adds into grad_input with atomics: rare for real offset fields (a bucket holds more than twice the mean
+// list), and correct however the samples crowd.
+struct SampleLists {
+    int *counts;         // [nbins] samples filed under the bin (may exceed cap); [nbins]: overflow entries
+    InvEntry *entries;   // [nbins][cap]
+    InvEntry *ovf;       // [ovf_cap]
+    int cap, nbins, ovf_cap;
+};
+// (in two steps, so that a caller can do other work while the counter's old value is on its way)
+D2C_DEV int lists_reserve(const SampleLists &L, int bin) { return atomicAdd(&L.counts[bin], 1); }
+D2C_DEV void lists_store(const SampleLists &L, int bin, int n, InvEntry e)
+{
+    if (n < L.cap) {
+        L.entries[(long)bin * L.cap + n] = e;
+    } else {
+        const int m = atomicAdd(&L.counts[L.nbins], 1);
+        if (m < L.ovf_cap) {
+            e.pad0 = bin;
+            L.ovf[m] = e;
+        }
+    }
+}
+D2C_DEV void lists_insert(const SampleLists &L, int bin, InvEntry e) { lists_store(L, bin, lists_reserve(L, bin), e); }
+
 // The three offsets (dz, dy, dx) of (b, g, k, p).  The 1-D operator stores one
 // offset per tap ([N, G*K, Lo], dconv1d_gpu.cu:40); it displaces along x only.
 D2C_DEV void load_offsets(const TiledShape &s, const void *off, int b, int g, int k, int p, float &o0, float &o1,

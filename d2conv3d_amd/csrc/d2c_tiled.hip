@@ -24,12 +24,15 @@ void d2c_invlist_ws(const TiledShape &s, size_t *counts, size_t *starts, size_t 
 int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, int *counts, int *starts, int *bsums,
                       void *entries, hipStream_t st);
 template <typename T>
-int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const int *starts, const void *entries, float *gxcl,
-                        hipStream_t st);
+int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st);
+void d2c_lists_ws(const TiledShape &s, size_t *counts, size_t *entries, size_t *ovf);
+SampleLists d2c_lists_make(const TiledShape &s, void *counts, void *entries, void *ovf);
+int d2c_lists_clear(const SampleLists &L, hipStream_t st);
+int d2c_lists_build(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
 int d2c_gx_mode();
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, hipStream_t st);
+                        void *goff, void *gmask, const SampleLists *lists, hipStream_t st);
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                                 const void *mask, void *goutp, float *gwacc, void *gw, hipStream_t st);
@@ -223,7 +226,7 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
 // channels in one pass of the data kernel.
 bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
 {
-    return d2c_gx_mode() == 1 && d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
+    return d2c_gx_mode() >= 1 && d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
 }
 
 // grad_offset / grad_mask by the kernel of d2c_aux_grad.hip (from the grad-column rows): when the data kernel
@@ -234,7 +237,7 @@ bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 struct BwdWs {
-    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, starts, bsums, entries, total;
+    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, total;
 };
 BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -252,19 +255,18 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.total = w.auxacc;
     if (d2c_bwd_data_split(s, q.dtype) > 1)
         w.total += d2c_align_up((size_t)s.N * s.G * s.K * s.P * (s.nd + 1) * sizeof(float));
-    w.gcol = w.counts = w.starts = w.bsums = w.entries = 0;
+    w.gcol = w.counts = w.entries = w.ovf = 0;
     if (use_lists(q, s) || use_aux_kernel(q, s)) {
         w.gcol = w.total;
         w.total = w.gcol + d2c_align_up((size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M * bkc_of(q.dtype) * es);
     }
     if (use_lists(q, s)) {
-        size_t c, st, bs, en;
-        d2c_invlist_ws(s, &c, &st, &bs, &en);
+        size_t c, en, ov;
+        d2c_lists_ws(s, &c, &en, &ov);
         w.counts = w.total;
-        w.starts = w.counts + c;
-        w.bsums = w.starts + st;
-        w.entries = w.bsums + bs;
-        w.total = w.entries + en;
+        w.entries = w.counts + c;
+        w.ovf = w.entries + en;
+        w.total = w.ovf + ov;
     }
     return w;
 }
@@ -287,7 +289,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             TiledShape so = s;
             so.Cin = s.Cout; so.vol = s.P;
             if (int rc = pack_input<T>(so, gout, base + d.goutcl, st)) return rc;
-            const bool lists = gx && d2c_gx_mode() == 1;
+            const bool lists = gx && d2c_gx_mode() >= 1;
             if (lists)
                 if (int rc = d2c_invlist_build(s, off, mask, (int *)(base + d.counts), (int *)(base + d.starts),
                                                (int *)(base + d.bsums), base + d.entries, st))
@@ -317,22 +319,24 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
             const bool lists = gx && use_lists(q, s);
             const bool auxk = (goff || gmask) && use_aux_kernel(q, s);
-            if (lists)
-                if (int rc = d2c_invlist_build(s, off, mask, (int *)(base + l.counts), (int *)(base + l.starts),
-                                               (int *)(base + l.bsums), base + l.entries, st))
-                    return rc;
+            // grad_input from sample lists: filled by the offset / mask gradient kernel on its way when that
+            // runs, by a pass of their own otherwise
+            SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
+            if (lists) {
+                L = d2c_lists_make(s, base + l.counts, base + l.entries, base + l.ovf);
+                if (int rc = auxk ? d2c_lists_clear(L, st) : d2c_lists_build(s, off, mask, L, st)) return rc;
+            }
             if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt,
                                                      lists ? nullptr : gxcl, (lists || auxk) ? base + l.gcol : nullptr,
                                                      auxk ? nullptr : goff, auxk ? nullptr : gmask,
                                                      (float *)(base + l.auxacc), st))
                 return rc;
             if (auxk)
-                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff, gmask, st))
+                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff, gmask,
+                                                    lists ? &L : nullptr, st))
                     return rc;
             if (lists)
-                if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, (const int *)(base + l.starts), base + l.entries,
-                                                    gxcl, st))
-                    return rc;
+                if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, L, gxcl, st)) return rc;
             if (gx)
                 if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
         } else {

@@ -157,7 +157,9 @@ int d2c_profile_read(int id, double *total_ms, int *launches);
 
 /* Test hook for the matrix-core backward pass: 1 (default) builds grad_input from
  * per-voxel sample lists, every element written once; 0 scatters with fp32 atomics
- * like the reference (dconv3d_gpu.cu:637).  Workspace sizes depend on the mode. */
+ * like the reference (dconv3d_gpu.cu:637).  A value n >= 2 is mode 1 with lists
+ * that hold at most n samples per voxel before the overflow path takes the rest
+ * (by default the capacity follows from the shape).  Workspace sizes depend on the mode. */
 void d2c_set_grad_input_mode(int mode);
 
 const char *d2c_last_error(void);

@@ -111,6 +111,36 @@ def test_grad_input_by_atomics_matches_lists(name, dtype, dev):
             assert rel_l2(grads[mode], eg[0]) < 2e-2, mode
 
 
+@pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cap", [2, 8])
+@pytest.mark.parametrize("want_aux", [True, False])
+def test_grad_input_when_sample_lists_overflow(name, dtype, cap, want_aux, dev):
+    # lists of tiny capacity: most samples take the overflow path (atomics after the owner kernel); with and
+    # without the offset / mask gradient, whose kernel files the samples on its way when it runs
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, dtype, seed=11)
+    eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+    _ops.set_grad_input_mode(cap)
+    try:
+        ts = [t.to(dev) if t is not None else None for t in (x, off, m, w, b)]
+        ts[0].requires_grad_(True)
+        if want_aux:
+            ts[1].requires_grad_(True)
+            if ts[2] is not None:
+                ts[2].requires_grad_(True)
+        d2c.deform_conv3d(*ts, s, p, d, groups, G).backward(gout.to(dev))
+    finally:
+        _ops.set_grad_input_mode("lists")
+    if dtype == torch.float32:
+        assert_close(ts[0].grad, eg[0], 1e-4, 1e-5 * max(1.0, eg[0].abs().max().item()), "grad_input")
+        if want_aux:
+            assert_close(ts[1].grad, eg[1], 1e-4, 1e-5 * max(1.0, eg[1].abs().max().item()), "grad_offset")
+    else:
+        assert rel_l2(ts[0].grad, eg[0]) < 2e-2
+        if want_aux:
+            assert rel_l2(ts[1].grad, eg[1]) < 2e-2
+
+
 def test_tiled_matches_generic_family(dev):
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make("c128_G2_o96", torch.float32, seed=3)
     ts = [t.to(dev) if t is not None else None for t in (x, off, m, w, b)]
