@@ -298,8 +298,8 @@ gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
 // gcol[p, k, c] = W[c, k] * gout[p, c] is one multiply, so no grad-column buffer
 // exists: the owner of a voxel reads the channels-last grad_out row of each
 // sample that reaches it and the weight row of its tap (staged in LDS).
-// A workgroup = kOwnVox voxels consecutive in x, 256 lanes each; a lane owns
-// kOwnCV consecutive channels (one vector load per lane and row).
+// A workgroup = kOwnVox 2 x 2 x 2 cubes of voxels consecutive in x, 256 lanes each;
+// a lane owns kOwnCV consecutive channels (one vector load per lane and row).
 constexpr int kOwnVox = 4, kOwnCV = 4, kOwnSlice = 256 * kOwnCV;
 
 template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
@@ -319,20 +319,26 @@ __global__ void __launch_bounds__(256 * kOwnVox)
 dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts, const InvEntry *entries,
                    float *gxcl, int w_in_lds)
 {
+    // One 256-lane group per 2 x 2 x 2 cube of voxels (kOwnVox cubes consecutive in x per workgroup, sharing the
+    // weights of the channel slice in LDS): the lists of the 27 base voxels that reach the cube are walked once
+    // each and a grad_out row is read once for all the voxels of the cube it contributes to, like
+    // gx_owner_cube_kernel does for the dense case.
     extern __shared__ __align__(16) unsigned char smem[];
     T *s_w = reinterpret_cast<T *>(smem);   // [K][kOwnSlice] weights of the channel slice
     const int t = threadIdx.x & 255;
     // wavefront-uniform quantities, kept in scalar registers
     const int vox = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
-    const int nbx = (s.W + kOwnVox - 1) / kOwnVox;
+    const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
+    const int nbx = (ncx + kOwnVox - 1) / kOwnVox;
     int blk = xcd_swizzle(blockIdx.x, gridDim.x);   // one contiguous part of the volume per XCD (L2)
     const int xb = blk % nbx; blk /= nbx;
-    const int y = blk % s.H; blk /= s.H;
-    const int z = blk % s.D;
-    const int b = blk / s.D;
-    const int x = xb * kOwnVox + vox;
-    const bool valid = x < s.W;
-    const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;
+    const int cy = blk % ncy; blk /= ncy;
+    const int cz = blk % ncz;
+    const int b = blk / ncz;
+    const int cx = xb * kOwnVox + vox;
+    const bool valid = cx < ncx;
+    const int x0 = cx * 2, y0 = cy * 2, z0 = cz * 2;
+    const int nxb = x0 + 1 < s.W ? 3 : 2;          // base voxels x0-1, x0, x0+1 (the last one only if it is a voxel)
     const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
     const T *grow = goutcl + (long)b * s.P * s.Cout;
 
@@ -351,42 +357,76 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
                 __syncthreads();
             }
             if (!valid || !cok) continue;
-            float acc[kOwnCV];
+            float acc[2][2][2][kOwnCV];
 #pragma unroll
-            for (int j = 0; j < kOwnCV; j++) acc[j] = 0.f;
-#pragma unroll 1
-            for (int t4 = 0; t4 < 4; t4++) {
-                // ranges ordered by the parity of the base voxel's (z, y): the voxels that share a list (4 in z/y, and
-                // their x-neighbours) then walk it in the same quarter of the kernel, while it is still cached
-                const int dz = (z ^ (t4 >> 1)) & 1, dy = (y ^ t4) & 1;
-                const int bin1 = bin_of(s, b, g, z - dz, y - dy, x - 1);   // lists of base voxels x-1 and x are adjacent
-                const int e0 = starts[bin1], em = starts[bin1 + 1], e1 = starts[bin1 + 2];
-                for (int e = e0; e < e1; e += 4) {
-                    float w[4];
-                    int kk[4];
-                    float go[4][kOwnCV];
+            for (int i = 0; i < 8 * kOwnCV; i++) (&acc[0][0][0][0])[i] = 0.f;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int ei = min(e + i, e1 - 1);
-                        const InvEntry q = entries[ei];
-                        const bool dx = e + i < em;
-                        const float wv = (dz ? q.hz : 1.f - q.hz) * (dy ? q.hy : 1.f - q.hy) * (dx ? q.hx : 1.f - q.hx)
-                                         * q.alpha;
-                        w[i] = e + i < e1 ? wv : 0.f;
-                        kk[i] = q.k;
-                        ld_vec4<T>(grow + (long)q.p * s.Cout + c, go[i]);
-                    }
+            for (int rz = 0; rz < 3; rz++) {
+                const int zb = z0 - 1 + rz;
+                if (zb > s.D - 1) continue;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        float wk[kOwnCV];
-                        if (w_in_lds) ld_vec4<T>(s_w + kk[i] * kOwnSlice + t * kOwnCV, wk);
-                        else ld_vec4<T>(wt + (long)kk[i] * s.Cin + c, wk);
+                for (int ry = 0; ry < 3; ry++) {
+                    const int yb = y0 - 1 + ry;
+                    if (yb > s.H - 1) continue;
+                    // the (up to) three base voxels along x are adjacent bins: one range of entries
+                    const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
+                    const int e0 = starts[bin1], em1 = starts[bin1 + 1], em2 = starts[bin1 + 2], e1 = starts[bin1 + nxb];
+                    for (int e = e0; e < e1; e += 4) {
+                        InvEntry q[4];
+                        float go[4][kOwnCV];
 #pragma unroll
-                        for (int j = 0; j < kOwnCV; j++) acc[j] = fmaf(w[i] * wk[j], go[i][j], acc[j]);
+                        for (int i = 0; i < 4; i++) {
+                            q[i] = entries[min(e + i, e1 - 1)];
+                            ld_vec4<T>(grow + (long)q[i].p * s.Cout + c, go[i]);
+                        }
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            float wk[kOwnCV];
+                            if (w_in_lds) ld_vec4<T>(s_w + q[i].k * kOwnSlice + t * kOwnCV, wk);
+                            else ld_vec4<T>(wt + (long)q[i].k * s.Cin + c, wk);
+                            const float al = e + i < e1 ? q[i].alpha : 0.f;
+                            float v[kOwnCV];
+#pragma unroll
+                            for (int jj = 0; jj < kOwnCV; jj++) v[jj] = wk[jj] * go[i][jj];
+                            // x: offset 0 (base x0-1) reaches voxel 0 with hx; 1 reaches (1-hx, hx); 2 reaches voxel 1 with 1-hx
+                            const float hz = q[i].hz, hy = q[i].hy, hx = q[i].hx;
+                            const bool r0 = e + i < em1, r2 = e + i >= em2;
+                            const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
+                            const float wx1 = r0 ? 0.f : (r2 ? 1.f - hx : hx);
+#pragma unroll
+                            for (int az = 0; az < 2; az++) {
+                                if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
+                                const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
+#pragma unroll
+                                for (int ay = 0; ay < 2; ay++) {
+                                    if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
+                                    const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
+                                    const float wzy = wz * wy * al;
+                                    const float w0 = wzy * wx0, w1 = wzy * wx1;
+#pragma unroll
+                                    for (int jj = 0; jj < kOwnCV; jj++) {
+                                        acc[az][ay][0][jj] = fmaf(w0, v[jj], acc[az][ay][0][jj]);
+                                        acc[az][ay][1][jj] = fmaf(w1, v[jj], acc[az][ay][1][jj]);
+                                    }
+                                }
+                            }
+                        }
                     }
                 }
             }
-            *reinterpret_cast<float4 *>(gxcl + vg * s.Cin + c) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+#pragma unroll
+            for (int az = 0; az < 2; az++)
+#pragma unroll
+                for (int ay = 0; ay < 2; ay++)
+#pragma unroll
+                    for (int ax = 0; ax < 2; ax++) {
+                        const int z = z0 + az, y = y0 + ay, x = x0 + ax;
+                        if (z < s.D && y < s.H && x < s.W) {
+                            const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;
+                            *reinterpret_cast<float4 *>(gxcl + vg * s.Cin + c) =
+                                make_float4(acc[az][ay][ax][0], acc[az][ay][ax][1], acc[az][ay][ax][2], acc[az][ay][ax][3]);
+                        }
+                    }
         }
     }
 }
@@ -514,7 +554,8 @@ int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *
     if (hipFuncSetAttribute((const void *)dw_gx_owner_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             160 * 1024) != hipSuccess)
         return d2c_check_launch("hipFuncSetAttribute(dw_gx_owner_kernel)");
-    const long nblk = (long)s.N * s.D * s.H * ((s.W + kOwnVox - 1) / kOwnVox);
+    const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
+    const long nblk = (long)s.N * ncz * ncy * ((ncx + kOwnVox - 1) / kOwnVox);
     hipLaunchKernelGGL(dw_gx_owner_kernel<T>, dim3((unsigned)nblk), dim3(256 * kOwnVox), lds, st, s, (const T *)goutcl,
                        (const T *)wt, starts, (const InvEntry *)entries, gxcl, w_in_lds);
     return d2c_check_launch("dw_gx_owner_kernel");
