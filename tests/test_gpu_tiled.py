@@ -114,10 +114,12 @@ def test_grad_input_by_atomics_matches_lists(name, dtype, dev):
 @pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("cap", [2, 8])
-@pytest.mark.parametrize("want_aux", [True, False])
-def test_grad_input_when_sample_lists_overflow(name, dtype, cap, want_aux, dev):
-    # lists of tiny capacity: most samples take the overflow path (atomics after the owner kernel); with and
-    # without the offset / mask gradient, whose kernel files the samples on its way when it runs
+@pytest.mark.parametrize("wanted", ["x", "x+aux", "all"])
+def test_grad_input_when_sample_lists_overflow(name, dtype, cap, wanted, dev):
+    # lists of tiny capacity: most samples take the overflow path (atomics after the owner kernel).  The samples
+    # are filed by the offset / mask gradient kernel when that runs ("x+aux", "all"), else by a pass of their
+    # own ("x")
+    want_aux = wanted != "x"
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, dtype, seed=11)
     eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
     _ops.set_grad_input_mode(cap)
@@ -128,6 +130,8 @@ def test_grad_input_when_sample_lists_overflow(name, dtype, cap, want_aux, dev):
             ts[1].requires_grad_(True)
             if ts[2] is not None:
                 ts[2].requires_grad_(True)
+        if wanted == "all":
+            ts[3].requires_grad_(True)
         d2c.deform_conv3d(*ts, s, p, d, groups, G).backward(gout.to(dev))
     finally:
         _ops.set_grad_input_mode("lists")
@@ -135,6 +139,8 @@ def test_grad_input_when_sample_lists_overflow(name, dtype, cap, want_aux, dev):
         assert_close(ts[0].grad, eg[0], 1e-4, 1e-5 * max(1.0, eg[0].abs().max().item()), "grad_input")
         if want_aux:
             assert_close(ts[1].grad, eg[1], 1e-4, 1e-5 * max(1.0, eg[1].abs().max().item()), "grad_offset")
+        if wanted == "all":
+            assert_close(ts[3].grad, eg[3], 1e-4, 1e-5 * max(1.0, eg[3].abs().max().item()), "grad_weight")
     else:
         assert rel_l2(ts[0].grad, eg[0]) < 2e-2
         if want_aux:
