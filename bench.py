@@ -185,15 +185,15 @@ def main():
     nf = f_fwd_ws(ctypes.byref(desc))
     nb = f_bwd_ws(ctypes.byref(desc)) if c["backward"] else 0
     ws = torch.empty(max(nf, nb, 256), dtype=torch.uint8, device=dev)
-    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    cur = [ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)]   # the stream the library launches on
     p = lambda t: ctypes.c_void_p(t.data_ptr())
 
     def forward():
-        _lib.check(f_fwd(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, stream), "forward")
+        _lib.check(f_fwd(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, cur[0]), "forward")
 
     def backward():
         _lib.check(f_bwd(ctypes.byref(desc), p(gout), p(x), p(off), p(m), p(w), p(gx), p(goff), p(gm), p(gw), p(gb),
-                         p(ws), nb, stream), "backward")
+                         p(ws), nb, cur[0]), "backward")
 
     def step():
         forward()
@@ -208,6 +208,28 @@ def main():
         step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # The same step captured once into a HIP graph and replayed (the library only enqueues kernels: no allocation,
+    # no memset node, no synchronisation).  Informational: what a launch-bound caller gains; `value` stays eager.
+    graph_ms = None
+    try:
+        graph = torch.cuda.CUDAGraph()
+        default_stream = cur[0]
+        with torch.cuda.graph(graph):
+            cur[0] = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+            step()
+        cur[0] = default_stream
+        for _ in range(2):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    except Exception as e:  # noqa: BLE001  (reported, never fatal: the eager figures above stand)
+        cur[0] = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        sys.stderr.write(f"bench.py: graph replay not measured: {e}\n")
 
     f_fwd_flops, b_fwd, b_bwd = algorithmic(name)
     nflops = (3 if c["backward"] else 1) * f_fwd_flops
@@ -293,6 +315,7 @@ def main():
                                f"groups={groups}, offset_groups={G}, bias, "
                                + ("bf16 in / fp32 accumulate" if dt == "bf16" else "fp32"),
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
+                   "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "algorithmic_gflop": round(nflops / 1e9, 2),
                    "algorithmic_mbytes": round((b_fwd + (b_bwd if c["backward"] else 0)) / 1e6, 1),
                    "frac_of_mfma_peak_whole_step": round(value / PEAK_TFLOPS[dt], 4),
