@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the D2Conv3D operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap]
 
 One step = one forward (+ one backward with all five gradients, except for
 the forward-only workload c1) of the modulated deformable convolution through
@@ -139,12 +139,61 @@ def cpu_baseline(name, torch):
     }
 
 
+def bench_size_map(args):
+    """The deformation producer in front of workload c2: predicted size map [2, 3, 8, 30, 54] -> ELU + 1 -> tap
+    offsets [2, 81, 8, 30, 54] and back (d2c_size_map_offsets_forward / _backward), against the torch formulation
+    of the reference (network/layers.py:171-181 + utils/grid.py:72-98) on the same GPU."""
+    import torch
+    from d2conv3d_amd.grid import offsets_from_size_map, size_map_offsets
+    from d2conv3d_amd.modules import _apply_size_activation
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    g = torch.Generator().manual_seed(1002)
+    raw = torch.randn(2, 3, 8, 30, 54, generator=g).to(dev).requires_grad_(True)
+    gout = torch.randn(2, 81, 8, 30, 54, generator=g).to(dev)
+
+    def fused():
+        raw.grad = None
+        size_map_offsets(raw, "xyz", (3, 3, 3), (1, 1, 1), "elu").backward(gout)
+
+    def stock():
+        raw.grad = None
+        offsets_from_size_map(_apply_size_activation("elu", raw), "xyz", (3, 3, 3), (1, 1, 1)).backward(gout)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms, ms_torch = timed(fused), timed(stock)
+    nbytes = 2 * (raw.numel() + gout.numel()) * 4          # each tensor once per direction
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    line = {
+        "metric": "size map -> offsets fwd+bwd GB/s (c2_sizemap) on 1 GPU", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "c2_sizemap: size map [2,3,8,30,54] -> ELU+1 -> offsets [2,81,8,30,54], forward + "
+                               "backward, through the autograd function (launch overhead included)",
+                   "torch_formulation_ms_per_step": round(ms_torch, 4), "algorithmic_mbytes": round(nbytes / 1e6, 2)},
+        "roofline": {"bound": "hbm", "kernel": "size_map_fwd_kernel + size_map_bwd_kernel", "achieved": round(gbs, 1),
+                     "peak": PEAK_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_GBS, 4), "traffic": None},
+    }
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -156,6 +205,8 @@ def main():
     lib = _lib.load()  # raises if the HIP library is missing: there is no fallback
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    if args.workload == "c2_sizemap":
+        return bench_size_map(args)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 

@@ -24,6 +24,7 @@ EXPORTS = (
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
     "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_last_error", "d2c_version",
     "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read",
+    "d2c_size_map_offsets_forward", "d2c_size_map_offsets_backward",
 )
 
 
@@ -32,6 +33,16 @@ class Conv3dDesc(ctypes.Structure):
         "N", "Cin", "Cout", "D", "H", "W", "kd", "kh", "kw", "sd", "sh", "sw",
         "pd", "ph", "pw", "dd", "dh", "dw", "groups", "offset_groups", "Do", "Ho", "Wo",
         "dtype", "aux_dtype")]
+
+
+SIZE_MAX_K = 16
+SIZE_MODES = {"xyz": 0, "xxz": 1, "xy": 2, "x": 3}
+SIZE_ACTIVATIONS = {"linear": 0, "elu": 1, "relu": 2, "relu_plus_one": 3}
+
+
+class SizeMapDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("N", "P", "kd", "kh", "kw", "mode", "activation", "dtype")] + [
+        (n, ctypes.c_float * SIZE_MAX_K) for n in ("base_z", "base_y", "base_x")]
 
 
 class Conv1dDesc(ctypes.Structure):
@@ -79,6 +90,9 @@ def load():
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int
     lib.d2c_set_grad_input_mode.argtypes, lib.d2c_set_grad_input_mode.restype = [ctypes.c_int], None
+    psm = ctypes.POINTER(SizeMapDesc)
+    lib.d2c_size_map_offsets_forward.argtypes, lib.d2c_size_map_offsets_forward.restype = [psm, vp, vp, vp], ctypes.c_int
+    lib.d2c_size_map_offsets_backward.argtypes, lib.d2c_size_map_offsets_backward.restype = [psm, vp, vp, vp, vp], ctypes.c_int
     lib.d2c_profile_enable.argtypes, lib.d2c_profile_enable.restype = [ctypes.c_int], None
     lib.d2c_profile_reset.argtypes, lib.d2c_profile_reset.restype = [], None
     lib.d2c_profile_read.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]

@@ -85,3 +85,83 @@ def offsets_from_size_map(size_map, *args, **kwargs):
     offsets = base * (size3.unsqueeze(1) - 1)                                           # [n, K, 3, d, h, w]
     n, _, d, h, w = size3.shape
     return offsets.reshape(n, -1, d, h, w)
+
+
+class _SizeMapOffsets(torch.autograd.Function):
+    """Size activation + offsets_from_size_map as one library kernel each way
+    (d2c_size_map_offsets_forward / _backward)."""
+
+    @staticmethod
+    def forward(ctx, size_raw, desc):
+        import ctypes
+        from . import _lib
+        lib = _lib.load()
+        size_raw = size_raw.contiguous()
+        n = size_raw.shape[0]
+        K = desc.kd * desc.kh * desc.kw
+        out = torch.empty((n, 3 * K) + tuple(size_raw.shape[2:]), dtype=size_raw.dtype, device=size_raw.device)
+        with torch.cuda.device(size_raw.device):
+            st = ctypes.c_void_p(torch.cuda.current_stream(size_raw.device).cuda_stream)
+            _lib.check(lib.d2c_size_map_offsets_forward(ctypes.byref(desc), ctypes.c_void_p(size_raw.data_ptr()),
+                                                        ctypes.c_void_p(out.data_ptr()), st), "size_map_offsets")
+        ctx.save_for_backward(size_raw)
+        ctx.desc = desc
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        import ctypes
+        from . import _lib
+        lib = _lib.load()
+        (size_raw,) = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        grad = torch.empty_like(size_raw)
+        with torch.cuda.device(size_raw.device):
+            st = ctypes.c_void_p(torch.cuda.current_stream(size_raw.device).cuda_stream)
+            _lib.check(lib.d2c_size_map_offsets_backward(ctypes.byref(ctx.desc), ctypes.c_void_p(size_raw.data_ptr()),
+                                                         ctypes.c_void_p(grad_out.data_ptr()),
+                                                         ctypes.c_void_p(grad.data_ptr()), st), "size_map_offsets backward")
+        return grad, None
+
+
+def size_map_offsets(size_raw, mode, kernel_shape=(3, 3, 3), dilation=(1, 1, 1), activation="linear"):
+    """offsets_from_size_map(size_activation(size_raw), mode, kernel_shape, dilation) in one kernel:
+    the deformation producer of the size-conditioned layers (network/layers.py:171-181 and
+    utils/grid.py:72-98) without the intermediate tensors and autograd nodes of the torch
+    formulation.  CUDA tensors, float32 or bfloat16; `size_raw` is the prediction BEFORE
+    the size activation.  Same values as the torch formulation (bit for bit in float32 except
+    for the exponential of the ELU)."""
+    from . import _lib
+    if not size_raw.is_cuda:
+        raise RuntimeError("size_map_offsets: CUDA tensors only (use offsets_from_size_map for CPU tensors)")
+    if size_raw.dtype not in (torch.float32, torch.bfloat16):
+        raise RuntimeError("size_map_offsets: float32 or bfloat16 only")
+    mode = mode.lower()
+    kernel_shape, dilation = _triple(kernel_shape), _triple(dilation)
+    want_c = {"xyz": 3, "xxz": 2, "xy": 2, "x": 1}[mode]
+    if size_raw.dim() < 3 or size_raw.shape[1] != want_c:
+        raise RuntimeError(f"size_map_offsets: mode '{mode}' wants {want_c} size channels, got {tuple(size_raw.shape)}")
+    if max(kernel_shape) > _lib.SIZE_MAX_K:
+        raise RuntimeError(f"size_map_offsets: kernel extents up to {_lib.SIZE_MAX_K}")
+    desc = _lib.SizeMapDesc()
+    desc.N = size_raw.shape[0]
+    desc.P = int(size_raw[0, 0].numel())
+    desc.kd, desc.kh, desc.kw = kernel_shape
+    desc.mode, desc.activation = _lib.SIZE_MODES[mode], _lib.SIZE_ACTIVATIONS[activation]
+    desc.dtype = _lib.D2C_BF16 if size_raw.dtype == torch.bfloat16 else _lib.D2C_F32
+    for name, d, k in zip(("base_z", "base_y", "base_x"), dilation, kernel_shape):
+        arr = getattr(desc, name)
+        for i, v in enumerate(_kernel_axis(d, k)):
+            arr[i] = v
+    return _SizeMapOffsets.apply(size_raw, desc)
+
+
+_AXIS_CACHE = {}
+
+
+def _kernel_axis(d, k):
+    """linspace(-d*(k//2), d*(k//2), k) exactly as get_kernel_grid computes it, as Python floats."""
+    key = (d, k)
+    if key not in _AXIS_CACHE:
+        _AXIS_CACHE[key] = torch.linspace(-d * (k // 2), d * (k // 2), k).tolist()
+    return _AXIS_CACHE[key]

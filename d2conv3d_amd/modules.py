@@ -15,7 +15,7 @@ from torch.nn.modules.utils import _triple
 from torch.utils.checkpoint import checkpoint
 
 from .deform_conv import DeformConv3d
-from .grid import offsets_from_size_map
+from .grid import offsets_from_size_map, size_map_offsets
 
 
 def _apply_size_activation(activation_mode, size_map):
@@ -164,28 +164,37 @@ class TemporalMDConv3d(_TemporalMixin, MDConv3d):
     pass
 
 
+def _size_offsets(layer, size_raw):
+    """Size activation + offsets_from_size_map: one library kernel each way for CUDA float32 / bfloat16
+    tensors (`fused_deformation`, on by default), the reference's torch formulation otherwise."""
+    if layer.fused_deformation and size_raw.is_cuda and size_raw.dtype in (torch.float32, torch.bfloat16):
+        return size_map_offsets(size_raw, layer._mode, layer.deform_conv.kernel_size, layer.deform_conv.dilation,
+                                layer.size_activation)
+    return offsets_from_size_map(_apply_size_activation(layer.size_activation, size_raw), layer._mode,
+                                 layer.deform_conv.kernel_size, layer.deform_conv.dilation)
+
+
 class _SizeConditionedD(DConv3d):
     """modules.py:123-159 / network/layers.py:184-230: the deformation branch
     predicts a dilation ("size") per location and axis subset; offsets follow
     from offsets_from_size_map.  Emits 3*K offset channels, i.e. offset_groups=1."""
     _size_channels = 1
     _mode = "x"
+    fused_deformation = True
 
     def _deform_channels(self):
         self.offset_channels = self._size_channels
         return self.offset_channels
 
     def _get_deformation(self, input):
-        size_map = _apply_size_activation(self.size_activation, self.deform_params(input))
-        offsets = offsets_from_size_map(size_map, self._mode, self.deform_conv.kernel_size,
-                                        self.deform_conv.dilation)
-        return offsets, None
+        return _size_offsets(self, self.deform_params(input)), None
 
 
 class _SizeConditionedMD(MDConv3d):
     """modules.py:162-219 / network/layers.py:233-313."""
     _size_channels = 1
     _mode = "x"
+    fused_deformation = True
 
     def _deform_channels(self):
         self.alpha_channels = self.offset_groups * self.num_kernel_points
@@ -195,10 +204,7 @@ class _SizeConditionedMD(MDConv3d):
     def _get_deformation(self, input):
         deformation = self.deform_params(input)
         size_map, alpha = torch.split(deformation, [self._size_channels, self.alpha_channels], dim=1)
-        size_map = _apply_size_activation(self.size_activation, size_map)
-        offsets = offsets_from_size_map(size_map, self._mode, self.deform_conv.kernel_size,
-                                        self.deform_conv.dilation)
-        return offsets, self.activation(alpha)
+        return _size_offsets(self, size_map), self.activation(alpha)
 
 
 class SizeConditionedDConv3d(_SizeConditionedD):

@@ -155,6 +155,36 @@ void d2c_profile_enable(int on);
 void d2c_profile_reset(void);
 int d2c_profile_read(int id, double *total_ms, int *launches);
 
+/* ---- dynamic-dilation front end -------------------------------------------------------
+ * The step in front of the operator in the size-conditioned layers: the predicted size map
+ * becomes tap offsets.  Replaces, in one kernel each way, the torch operations of
+ * network/layers.py:171-181 (_apply_size_activation), utils/grid.py:83-93 (axes the mode does
+ * not predict get size 1) and utils/grid.py:95-98 / dconv_native/grid.py:62-80
+ * (offsets_from_size_map):
+ *     offsets[n, 3*k + a, p] = base_a[k_a] * (act(size_raw)[n, channel(a), p] - 1),
+ *     k = (kz*kh + ky)*kw + kx;  base_a = linspace(-dil_a*(k_a/2), dil_a*(k_a/2), k_a), passed in.
+ * size_raw is [N, 3 | 2 | 2 | 1, P] for mode XYZ | XXZ (z, x; y = x) | XY (y, x) | X (y = x),
+ * offsets is [N, 3*K, P]; both in `dtype` (float32 or bfloat16).  The backward call turns
+ * grad_offsets into grad_size_raw (activation derivative included). */
+#define D2C_SIZE_MAX_K 16
+enum { D2C_SIZE_XYZ = 0, D2C_SIZE_XXZ = 1, D2C_SIZE_XY = 2, D2C_SIZE_X = 3 };
+enum {
+    D2C_SIZE_ACT_LINEAR = 0,        /* x */
+    D2C_SIZE_ACT_ELU = 1,           /* ELU(x) + 1 */
+    D2C_SIZE_ACT_RELU = 2,          /* ReLU(x + 1) */
+    D2C_SIZE_ACT_RELU_PLUS_ONE = 3  /* ReLU(x + 1e-3) + 1 */
+};
+typedef struct d2c_size_map_desc {
+    int32_t N, P;             /* samples, positions per sample (Do*Ho*Wo) */
+    int32_t kd, kh, kw;
+    int32_t mode, activation;
+    int32_t dtype;
+    float base_z[D2C_SIZE_MAX_K], base_y[D2C_SIZE_MAX_K], base_x[D2C_SIZE_MAX_K];
+} d2c_size_map_desc;
+int d2c_size_map_offsets_forward(const d2c_size_map_desc *desc, const void *size_raw, void *offsets, void *stream);
+int d2c_size_map_offsets_backward(const d2c_size_map_desc *desc, const void *size_raw, const void *grad_offsets,
+                                  void *grad_size_raw, void *stream);
+
 /* Test hook for the matrix-core backward pass: 1 (default) builds grad_input from
  * per-voxel sample lists, every element written once; 0 scatters with fp32 atomics
  * like the reference (dconv3d_gpu.cu:637).  A value n >= 2 is mode 1 with lists

@@ -71,3 +71,67 @@ def test_add_deformable_conv_replaces_and_keeps_weights(dev):
     # zero-initialised deformation: modulation 0.5 everywhere, dilation ELU(0)+1 = 1
     y = net2(x)
     assert y.shape == (1, 4, 4, 6, 6) and torch.isfinite(y).all()
+
+
+# ---- the deformation producer of the size-conditioned layers as library kernels ------------------------
+from d2conv3d_amd.grid import offsets_from_size_map, size_map_offsets  # noqa: E402
+
+
+@pytest.mark.parametrize("mode,channels", [("xyz", 3), ("xxz", 2), ("xy", 2), ("x", 1)])
+@pytest.mark.parametrize("activation", ["linear", "elu", "relu", "relu_plus_one"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_size_map_offsets_match_the_torch_formulation(mode, channels, activation, dtype, dev):
+    # network/layers.py:171-181 + utils/grid.py:72-98 in torch against d2c_size_map_offsets_forward / _backward;
+    # kernel (3, 5, 2) has an even extent (fractional kernel grid) and a non-unit dilation
+    g = torch.Generator().manual_seed(17)
+    raw = (torch.randn(2, channels, 3, 5, 6, generator=g) * 1.5).to(dev, dtype)
+    kernel, dilation = (3, 5, 2), (1, 2, 1)
+    a = raw.clone().requires_grad_(True)
+    b = raw.clone().requires_grad_(True)
+    ref = offsets_from_size_map(M._apply_size_activation(activation, a), mode, kernel, dilation)
+    out = size_map_offsets(b, mode, kernel, dilation, activation)
+    assert out.shape == ref.shape and out.dtype == ref.dtype
+    if dtype == torch.float32:
+        assert torch.allclose(out, ref, rtol=1e-6, atol=1e-6)
+    else:
+        assert torch.allclose(out.float(), ref.float(), rtol=1e-2, atol=1e-2)
+    go = torch.randn(ref.shape, generator=g).to(dev, dtype)
+    ref.backward(go)
+    out.backward(go)
+    if dtype == torch.float32:
+        assert torch.allclose(b.grad, a.grad, rtol=1e-5, atol=1e-5)
+    else:
+        # torch rounds every partial sum to bfloat16, the kernel accumulates in float32
+        scale = a.grad.float().abs().max().item()
+        assert torch.allclose(b.grad.float(), a.grad.float(), rtol=5e-2, atol=5e-2 * scale)
+
+
+@pytest.mark.parametrize("cls", ["XYZSizeConditionedMDConv3d", "XXZSizeConditionedDConv3d", "SizeConditionedMDConv3d"])
+def test_size_conditioned_layers_same_with_and_without_the_fused_producer(cls, dev):
+    torch.manual_seed(3)
+    layer = getattr(M, cls)(4, 6, 3, padding=1).to(dev)
+    with torch.no_grad():
+        layer.deform_params.weight.normal_(0, 0.3)
+        layer.deform_params.bias.normal_(0, 0.3)
+    x = torch.randn(2, 4, 5, 6, 7, device=dev)
+    outs, grads = [], []
+    for fused in (True, False):
+        layer.fused_deformation = fused
+        layer.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = layer(xi)
+        out.square().sum().backward()
+        outs.append(out.detach())
+        grads.append([xi.grad.clone(), layer.deform_params.weight.grad.clone()])
+    assert torch.allclose(outs[0], outs[1], rtol=1e-5, atol=1e-5)
+    for a, b in zip(*grads):
+        assert torch.allclose(a, b, rtol=1e-4, atol=1e-4 * max(1.0, b.abs().max().item()))
+
+
+def test_size_map_offsets_reject_bad_arguments(dev):
+    with pytest.raises(RuntimeError):
+        size_map_offsets(torch.zeros(1, 3, 2, 2, 2), "xyz")                       # CPU tensor
+    with pytest.raises(RuntimeError):
+        size_map_offsets(torch.zeros(1, 2, 2, 2, 2, device=dev), "xyz")           # wrong channel count
+    with pytest.raises(RuntimeError):
+        size_map_offsets(torch.zeros(1, 3, 2, 2, 2, device=dev, dtype=torch.float64), "xyz")
