@@ -14,8 +14,10 @@
 // Kernel 2 (tiled_bwd_weight_dma_kernel), per workgroup one (tap, channel chunk)
 // and all output channels, looping over position tiles:
 //     gW[o, c, k] += sum_pos gout[o, pos] * alpha * trilinear(x[c], pos)       (:1037-1088)
-//   The sampler writes its tile position-contiguous so that it is an MFMA
-//   operand as it lies.
+//   The reduction runs over positions, so the MFMA operand wants 8 consecutive
+//   positions of one channel per lane: the bfloat16 tile is stored as sampled
+//   ([position][channel]) and read with the transposing LDS load
+//   (ds_read_b64_tr_b16); the float tile is stored transposed.
 #include "d2c_mma.hpp"
 #include "d2c_tiled.hpp"
 
@@ -535,7 +537,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
                                              16, 0, 0);
         }
     };
-    // --- interpolation, stored transposed ([channel][position]); thread = (position, 16-byte vector)
+    // --- interpolation; thread = (position, 16-byte vector)
     const int ipos = tid >> 3, ivec = tid & 7;
     auto interp_store = [&](int rbuf, int tbuf, int dbuf) {
         if (!worker) return;
@@ -545,20 +547,14 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
 #pragma unroll
         for (int c = 0; c < 8; c++)
             va.fma(s_w[(tbuf * 8 + c) * MT + ipos], *reinterpret_cast<const uint4 *>(rp + c * 128));
-        unsigned char *tb = s_tile + dbuf * BKC * TRS + (ivec * VEC) * TRS;
         if constexpr (sizeof(T) == 2) {
-            // lanes of positions p and p^1 (8 lanes apart) swap values, each writes 4-byte pairs of positions;
-            // 16-byte chunks of a row are XOR-swizzled by its 8-channel group (rows 8 apart alias in LDS)
-            const int odd = ipos & 1;
-#pragma unroll
-            for (int e = 0; e < VEC; e++) {
-                const float other = __shfl_xor(va.a[e], 8, 64);
-                if ((e & 1) == odd) {
-                    const uint32_t pr = odd ? pack_bf16x2(other, va.a[e]) : pack_bf16x2(va.a[e], other);
-                    *reinterpret_cast<uint32_t *>(tb + e * TRS + ((((ipos >> 1) ^ (ivec << 2))) << 2)) = pr;
-                }
-            }
+            // bfloat16: the tile stays [position][channel] (one 16-byte store, rows of TRS bytes: MT == BKC);
+            // the matrix wavefronts read it with the transposing LDS load, see mma_tile
+            static_assert(sizeof(T) != 2 || MT == BKC, "tile rows of either orientation have the same length");
+            *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * TRS + ivec * 16) = va.pack();
         } else {
+            // float: stored transposed ([channel][position]), one element per store
+            unsigned char *tb = s_tile + dbuf * BKC * TRS + (ivec * VEC) * TRS;
 #pragma unroll
             for (int e = 0; e < VEC; e++) *reinterpret_cast<float *>(tb + e * TRS + ipos * 4) = va.a[e];
         }
@@ -581,12 +577,29 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
         for (int kg = 0; kg < NKG; kg++) {
             const int kq = kg & 3;
             uint4 bf[CB];
+            if constexpr (sizeof(T) == 2) {
+                // ds_read_b64_tr_b16: within 16 lanes, lane l element j comes from lane 4j + l/4, element l%4.
+                // Source lane (j, q) reads 4 channels of position +j; receiving lane (q, e) then holds channel
+                // 4q + e of 4 consecutive positions: two such loads make the 8 positions of an operand vector.
+                typedef short v4s __attribute__((ext_vector_type(4)));
+                const int l16 = lane & 15, g16 = lane >> 4;
 #pragma unroll
-            for (int cb = 0; cb < CB; cb++) {
-                const int row = cb * 32 + (lane & 31);
-                const int swz = sizeof(T) == 2 ? ((row >> 3) & 7) : 0;
-                bf[cb] = *reinterpret_cast<const uint4 *>(s_tile + dbuf * BKC * TRS + row * TRS
-                                                          + (((kg * 2 + (lane >> 5)) ^ swz) << 4));
+                for (int cb = 0; cb < CB; cb++) {
+                    const int pos = kg * 16 + (g16 >> 1) * 8 + (l16 >> 2);
+                    const int ch = cb * 32 + (g16 & 1) * 16 + (l16 & 3) * 4;
+                    const unsigned char *ap = s_tile + (dbuf * MT + pos) * TRS + ch * 2;
+                    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)ap);
+                    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(ap + 4 * TRS));
+                    const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+                    bf[cb] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+                }
+            } else {
+#pragma unroll
+                for (int cb = 0; cb < CB; cb++) {
+                    const int row = cb * 32 + (lane & 31);
+                    bf[cb] = *reinterpret_cast<const uint4 *>(s_tile + dbuf * BKC * TRS + row * TRS
+                                                              + ((kg * 2 + (lane >> 5)) << 4));
+                }
             }
 #pragma unroll
             for (int ob = 0; ob < OB; ob++)
@@ -750,20 +763,38 @@ __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp,
 
 // gb[o] = sum_{b,p} gout[b,o,p]   (dconv3d_gpu.cu:1329)
 template <typename T>
-__global__ void __launch_bounds__(256) bias_grad_kernel(const T *gout, T *gb, int N, int Cout, int P)
+__global__ void __launch_bounds__(1024) bias_grad_kernel(const T *gout, T *gb, int N, int Cout, int P)
 {
-    __shared__ float part[4];
+    // one workgroup of 16 wavefronts per output channel; 16-byte loads where the row allows them
+    constexpr int VEC = 16 / (int)sizeof(T);
+    __shared__ float part[16];
     const int o = blockIdx.x;
     float acc = 0.f;
     for (int b = 0; b < N; b++) {
         const T *row = gout + ((long)b * Cout + o) * P;
-        for (int p = threadIdx.x; p < P; p += 256) acc += elem_to_f32<T>(row[p]);
+        const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(row) & 15)) & 15) / sizeof(T));   // to 16-byte alignment
+        const int h = head < P ? head : P;
+        const int nvec = (P - h) / VEC;
+        if ((int)threadIdx.x < h) acc += elem_to_f32<T>(row[threadIdx.x]);
+        const uint4 *rv = reinterpret_cast<const uint4 *>(row + h);
+        for (int i = threadIdx.x; i < nvec; i += 1024) {
+            const uint4 v = rv[i];
+            const T *e = reinterpret_cast<const T *>(&v);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc += elem_to_f32<T>(e[j]);
+        }
+        for (int p = h + nvec * VEC + threadIdx.x; p < P; p += 1024) acc += elem_to_f32<T>(row[p]);
     }
 #pragma unroll
     for (int sft = 32; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft, 64);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
     __syncthreads();
-    if (threadIdx.x == 0) gb[o] = f32_to_elem<T>(part[0] + part[1] + part[2] + part[3]);
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) t += part[i];
+        gb[o] = f32_to_elem<T>(t);
+    }
 }
 
 // fp32 scratch of the split data kernel -> offset / mask gradient in its storage type
@@ -966,7 +997,7 @@ template <typename T>
 int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st)
 {
     D2cProfScope prof(D2C_PROF_PACK, st);
-    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(s.Cout), dim3(256), 0, st, (const T *)gout, (T *)gb, s.N, s.Cout, s.P);
+    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(s.Cout), dim3(1024), 0, st, (const T *)gout, (T *)gb, s.N, s.Cout, s.P);
     return d2c_check_launch("bias_grad_kernel");
 }
 
