@@ -151,6 +151,28 @@ def test_grad_input_when_sample_lists_overflow(name, dtype, cap, wanted, dev):
             assert rel_l2(ts[1].grad, eg[1]) < 2e-2
 
 
+@pytest.mark.parametrize("name", ["c64_g1", "c128_G2_o96", "dw64"])
+def test_integer_sampling_positions(name, dev):
+    # integer offsets (the state at zero-initialised offsets), with padding: samples sit exactly on voxels and
+    # exactly on the planes -1 and size, where the forward value is cut off by the early-out but the offset
+    # gradient still sees the in-range corners (dconv3d_gpu.cu:48-109 against :708-864)
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, torch.float32, seed=21)
+    g = torch.Generator().manual_seed(21)
+    ints = torch.randint(-2, 3, off.shape, generator=g).to(off.dtype)
+    keep = torch.rand(off.shape, generator=g) < 0.25            # a quarter of the offsets stay real-valued
+    off = torch.where(keep, off, ints)
+    off[:, : off.shape[1] // 3] = 0.0                             # and a third of the taps sit on their own voxel
+    ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+    out = d2c.deform_conv3d(*ts, s, p, d, groups, G)
+    exp = cpu.conv3d_forward(x, off, m, w, b, s, p, d, groups, G)
+    eg = cpu.conv3d_backward(gout, x, off, m, w, b is not None, s, p, d, groups, G)
+    out.backward(gout.to(dev))
+    assert_close(out, exp, 1e-4, 1e-5, "forward")
+    for n, t, e in zip(("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias"), ts, eg):
+        if t is not None:
+            assert_close(t.grad, e, 1e-4, 1e-5 * max(1.0, e.abs().max().item()), n)
+
+
 def test_tiled_matches_generic_family(dev):
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make("c128_G2_o96", torch.float32, seed=3)
     ts = [t.to(dev) if t is not None else None for t in (x, off, m, w, b)]
