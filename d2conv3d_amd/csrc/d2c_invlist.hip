@@ -495,6 +495,11 @@ void d2c_lists_ws(const TiledShape &s, size_t *counts, size_t *entries, size_t *
     *entries = d2c_align_up((size_t)nb * d2c_lists_cap(s) * sizeof(InvEntry));
     *ovf = d2c_align_up((size_t)s.N * s.G * s.K * s.P * sizeof(InvEntry));
 }
+// Bins and samples are counted in 32 bits; larger problems take the atomic scatter instead.
+bool d2c_lists_supported(const TiledShape &s)
+{
+    return d2c_invlist_bins(s) < (1L << 31) - 1 && (long)s.N * s.G * s.K * s.P < (1L << 31);
+}
 // The lists over the three workspace regions sized by d2c_lists_ws; nbins == 0 when the shape is too large.
 SampleLists d2c_lists_make(const TiledShape &s, void *counts, void *entries, void *ovf)
 {

@@ -28,6 +28,7 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists
 void d2c_lists_ws(const TiledShape &s, size_t *counts, size_t *entries, size_t *ovf);
 SampleLists d2c_lists_make(const TiledShape &s, void *counts, void *entries, void *ovf);
 int d2c_lists_clear(const SampleLists &L, hipStream_t st);
+bool d2c_lists_supported(const TiledShape &s);
 int d2c_lists_build(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
 int d2c_gx_mode();
 template <typename T>
@@ -226,7 +227,7 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
 // channels in one pass of the data kernel.
 bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
 {
-    return d2c_gx_mode() >= 1 && d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
+    return d2c_gx_mode() >= 1 && d2c_lists_supported(s) && d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
 }
 
 // grad_offset / grad_mask by the kernel of d2c_aux_grad.hip (from the grad-column rows): when the data kernel
@@ -289,7 +290,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             TiledShape so = s;
             so.Cin = s.Cout; so.vol = s.P;
             if (int rc = pack_input<T>(so, gout, base + d.goutcl, st)) return rc;
-            const bool lists = gx && d2c_gx_mode() >= 1;
+            const bool lists = gx && d2c_gx_mode() >= 1 && d2c_lists_supported(s);
             if (lists)
                 if (int rc = d2c_invlist_build(s, off, mask, (int *)(base + d.counts), (int *)(base + d.starts),
                                                (int *)(base + d.bsums), base + d.entries, st))
