@@ -493,10 +493,23 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         const long wbase = (((long)wgq * S + stq) * OBT + (otq * (NT / 32) + wave_o * OB)) * NKG * 64 + lane;
         return wp4[wbase + ((long)ob * NKG + kg) * 64];
     };
-    // one step on the matrix cores; the weight fragments of the step after it (at `wn`) are fetched meanwhile
-    auto mma_step = [&](int dbuf, const SegWalk &wn) {
-        if (!mma_wave) return;
+    // The vector-memory path of a CU takes one request of a wavefront at a time (1 KiB = 16 clocks) and a wavefront
+    // stalls at issue while the path is busy: requests issued back to back serialise with everything else the
+    // wavefront does.  So they are spread over the iteration: the DMA requests of step it+2 between the MFMAs of
+    // step it (in its first half, so that they have landed when the interpolation starts), the weight-fragment
+    // loads of step it+1 between the corners of the interpolation.
+    static_assert(WAVES_O * WAVES_P == 8 && NKG * OB == 8, "all workers are matrix wavefronts; a fragment per corner");
+    auto mma_dma_step = [&](int dbuf, const SegWalk &w, int rbuf, int tbuf) {
         const unsigned char *tb = s_tile + (dbuf * MT + wave_p * WPOS + (lane & 31)) * kRS + (lane >> 5) * 16;
+        const int j = w.st / s.K;
+        const int c0 = w.wg * s.cg + j * BKC;
+        const char *base = reinterpret_cast<const char *>(a.xcl);
+        // table entries of this wavefront's 8 positions: one LDS read (lane i holds position i), then
+        // lane-indexed moves to scalar registers
+        const int vidx = s_idx[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const int vflag = s_flag[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const unsigned vmask = w.item >= 0 ? 0xffu : 0u;     // past the end of the sequence: rows of zeros
+        constexpr int DPK = 4;                                // requests per k-group
 #pragma unroll
         for (int kg = 0; kg < NKG; kg++) {
             uint4 bf[PB];
@@ -508,8 +521,32 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
 #pragma unroll
                 for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[kg][ob], bf[pb]);
 #pragma unroll
-            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(wn, kg, ob);
+            for (int q = 0; q < DPK; q++) {
+                const int i = kg * DPK + q;
+                if (i >= MT / 8) break;
+                const int pos = wave * (MT / 8) + i;
+                const int idx = __builtin_amdgcn_readlane(vidx, i);
+                const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i) & vmask;
+                const unsigned o = ((live >> dcorner) & 1u)
+                                       ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
+                                       : a.zrow + (unsigned)dvec * 16u;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + o),
+                                                 (__attribute__((address_space(3))) void *)(s_raw + (rbuf * MT + pos) * kRawPos),
+                                                 16, 0, 0);
+            }
         }
+    };
+    // interpolation of one step; the weight fragments of that step (at `wn`) are fetched on the way
+    auto interp_wload_store = [&](int rbuf, int tbuf, int dbuf, const SegWalk &wn) {
+        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * kRawPos + ivec * 16;
+        VecAcc<T> va;
+        va.zero();
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            va.fma(s_w[(tbuf * 8 + c) * MT + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
+            af[c / OB][c % OB] = wfrag(wn, c / OB, c % OB);
+        }
+        *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = va.pack();
     };
     // end of a segment: whole items get bias, conversion and store; pieces of an item add into its fp32 tile
     auto flush_acc = [&](const SegWalk &w) {
@@ -557,8 +594,9 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         }
     };
 
-    // --- pipeline.  Iteration `it` of the step sequence: step it on the matrix cores, step it+1 interpolated,
-    // rows of step it+2 requested, coordinates of step it+3 computed.  Corner tables rotate over 3 buffers,
+    // --- pipeline.  Iteration `it` of the step sequence: step it on the matrix cores with the rows of step it+2
+    // requested on the way, step it+1 interpolated with its weight fragments requested on the way, coordinates
+    // of step it+3 computed.  Corner tables rotate over 3 buffers,
     // raw rows and tiles over 2.  A wavefront interpolates the positions whose rows it requested itself, so the
     // rows need no barrier, only that wavefront's own wait.
     SegWalk wc = w0;                  // coordinates: the step whose offsets are requested next
@@ -602,14 +640,12 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         while (wm.item >= 0) {
             for (; wm.st < wm.st_hi; wm.st++, it++) {
                 lds_barrier();
-                mma_step(it & 1, wn);
-                // The rows of step it+1, requested one iteration ago by this same wavefront (it interpolates the
-                // positions whose rows it requested), have had the barrier and the matrix-core phase to arrive;
-                // only the NKG * OB weight-fragment loads of mma_step are younger and may stay in flight.
-                static_assert(NKG * OB == 8, "the wait below counts the weight-fragment loads");
-                __builtin_amdgcn_s_waitcnt(0x0F78);     // vmcnt(8)
-                if (it + 1 < total) interp_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
-                dma_issue(wd, it & 1, (it + 2) % 3);
+                // everything this wavefront has in flight is due: the weight fragments of this step (requested
+                // during the last interpolation) and the rows of step it+1 (requested during the last matrix step)
+                __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
+                mma_dma_step(it & 1, wd, it & 1, (it + 2) % 3);
+                // (past the end of the sequence the interpolation works on stale rows into the tile nobody reads)
+                interp_wload_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1, wn);
                 if (wd.item >= 0) seg_advance(wd, s_seg, nseg);
                 if (wn.item >= 0) seg_advance(wn, s_seg, nseg);
             }
