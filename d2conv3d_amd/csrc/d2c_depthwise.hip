@@ -12,9 +12,9 @@
 //             gW[c,k]    += gout * alpha * trilinear                    (registers, then atomics)
 //
 // A workgroup owns a tile of output positions and a slice of 256 channels (one
-// 16-byte vector per lane of a wavefront).  The slice is the slow launch
-// dimension: at any time the whole chip works on one channel slice of the
-// input, which then stays in the L2 caches.  The corner weights of the tile are
+// 16-byte vector per lane of a wavefront); dw_tile() maps the workgroups so that
+// each XCD works on one channel slice of one batch element at a time, which
+// then stays in its L2.  The corner weights of the tile are
 // computed once into LDS and shared by the four wavefronts.
 #include "d2c_mma.hpp"
 #include "d2c_tiled.hpp"
@@ -43,14 +43,27 @@ struct DwArgs {
     float *gwacc;              // [K][C] fp32 accumulator (zeroed) or NULL
 };
 
-// Workgroups are dealt round-robin to the 8 XCDs; this gives each XCD one contiguous run of tiles, so that
-// its L2 sees a compact part of the input.
-D2C_DEV int xcd_swizzle(int bid, int n)
+// Tile of a workgroup: the combinations of xcd_unit() are (batch element, offset group, channel slice), so
+// the L2 of an XCD sees one channel slice of one batch element at a time (3.3 MB of the input for 256 fp32
+// channels of 8x15x27 voxels) and not, as with tiles dealt in launch order, all channels of the input.
+// Tiles do not straddle batch elements.
+struct DwTile {
+    int m0, m_end;   // positions [m0, m_end) of the flattened (batch, position) range
+    int y;           // offset group * slices + slice
+    bool ok;
+};
+D2C_DEV DwTile dw_tile(const TiledShape &s, int TP, int ny, int bid)
 {
-    const int x = bid & 7, idx = bid >> 3;
-    const int q = n >> 3, r = n & 7;
-    return x * q + (x < r ? x : r) + idx;
+    const XcdUnit u = xcd_unit(bid, s.N * ny, (s.P + TP - 1) / TP);
+    const int b = u.combo % s.N;
+    DwTile r;
+    r.y = u.combo / s.N;
+    r.ok = u.ok;
+    r.m0 = b * s.P + u.tile * TP;
+    r.m_end = min(r.m0 + TP, (b + 1) * s.P);
+    return r;
 }
+inline unsigned dw_grid(const TiledShape &s, int TP, int ny) { return xcd_unit_grid(s.N * ny, (s.P + TP - 1) / TP); }
 
 // View over dynamic LDS, one entry per (tap of the batch, position of the tile): the live corner
 // weights * alpha, the base voxel and live | inrange << 8; for the backward pass also the per-axis
@@ -81,7 +94,7 @@ constexpr size_t kDwLdsFwd = (size_t)10 * kFwdKB * kFwdTP * 4;
 constexpr size_t kDwLdsBwd = (size_t)17 * kBwdKB * kBwdTP * 4;
 
 template <bool BWD, int TP, int KB>
-D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<TP, KB> &t, int m0, int g, int k0, int kn)
+D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<TP, KB> &t, int m0, int m_end, int g, int k0, int kn)
 {
     const TiledShape &s = a.s;
     for (int task = threadIdx.x; task < kn * TP; task += kDwThreads) {
@@ -91,7 +104,7 @@ D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<TP, KB> &t, int m0, int g, 
         float fr[6] = {0, 0, 0, 0, 0, 0};
         float al = 0.f;
         int idx = 0, flag = 0;
-        if (m < s.M) {
+        if (m < m_end) {
             const int b = m / s.P, p = m - b * s.P;
             const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
             const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
@@ -146,10 +159,12 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
     const TiledShape &s = a.s;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * TP;
-    const int HW = s.H * s.W;
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
-    const int g = blockIdx.y / nsl, sl = blockIdx.y - g * nsl;
+    const DwTile tl = dw_tile(s, TP, s.G * nsl, blockIdx.x);
+    if (!tl.ok) return;
+    const int m0 = tl.m0, m_end = tl.m_end;
+    const int HW = s.H * s.W;
+    const int g = tl.y / nsl, sl = tl.y - g * nsl;
     const int cl = sl * kSlice + lane * kCV;      // first channel of this lane inside the offset group
     const bool cok = cl < s.cpg;
     const int c = g * s.cpg + (cok ? cl : 0);
@@ -165,7 +180,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
     for (int k0 = 0; k0 < s.K; k0 += KB) {
         const int kn = min(KB, s.K - k0);
         __syncthreads();
-        dw_coords<false, TP, KB>(a, taps, m0, g, k0, kn);
+        dw_coords<false, TP, KB>(a, taps, m0, m_end, g, k0, kn);
         __syncthreads();
         if (!cok) continue;
         for (int kk = 0; kk < kn; kk++) {
@@ -209,10 +224,10 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
     if (a.bias) ld4<T>(reinterpret_cast<const T *>(a.bias) + c, bv);
     T *out = reinterpret_cast<T *>(a.out);
     const int mf = m0 + wave * PW;
-    if (mf >= s.M) return;
+    if (mf >= m_end) return;
     const int bf = mf / s.P, pf = mf - bf * s.P;
     constexpr int EV = 16 / (int)sizeof(T);       // elements per 16-byte store
-    const bool fast = mf + PW <= s.M && pf + PW <= s.P && pf % EV == 0 && s.P % EV == 0;
+    const bool fast = mf + PW <= m_end && pf % EV == 0 && s.P % EV == 0;
     if (fast) {
 #pragma unroll
         for (int j = 0; j < kCV; j++) {
@@ -227,7 +242,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
 #pragma unroll
         for (int i = 0; i < PW; i++) {
             const int m = mf + i;
-            if (m < s.M) {
+            if (m < m_end) {
                 const int b = m / s.P, pp = m - b * s.P;
 #pragma unroll
                 for (int j = 0; j < kCV; j++)
@@ -268,10 +283,12 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
     const TiledShape &s = a.s;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int m0 = xcd_swizzle(blockIdx.x, gridDim.x) * TP;
-    const int HW = s.H * s.W;
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
-    const int g = blockIdx.y / nsl, sl = blockIdx.y - g * nsl;
+    const DwTile tl = dw_tile(s, TP, s.G * nsl, blockIdx.x);
+    if (!tl.ok) return;
+    const int m0 = tl.m0, m_end = tl.m_end;
+    const int HW = s.H * s.W;
+    const int g = tl.y / nsl, sl = tl.y - g * nsl;
     const int cl = sl * kSlice + lane * kCV;
     const bool cok = cl < s.cpg;       // lanes past the group still take part in the reductions
     const int c = g * s.cpg + (cok ? cl : 0);
@@ -283,7 +300,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
     for (int k0 = 0; k0 < s.K; k0 += KB) {
         const int kn = min(KB, s.K - k0);
         __syncthreads();
-        dw_coords<true, TP, KB>(a, taps, m0, g, k0, kn);
+        dw_coords<true, TP, KB>(a, taps, m0, m_end, g, k0, kn);
         __syncthreads();
         for (int kk = wave; kk < kn; kk += kDwThreads / 64) {
             float wv[kCV] = {0.f, 0.f, 0.f, 0.f};
@@ -296,7 +313,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
                 const unsigned inr = flag >> 8, live = flag & 0xffu;
                 if (!inr) continue;
                 const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
-                const int m = m0 + p;                     // m < M holds where inr != 0
+                const int m = m0 + p;                     // m < m_end holds where inr != 0
                 float go[kCV] = {0.f, 0.f, 0.f, 0.f};
                 if (cok) ld4<T>(goutcl + (long)m * s.Cout + c, go);
                 float gc[kCV];
@@ -434,7 +451,7 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
     DwArgs a{s, xcl, off, mask, wt, bias, out, nullptr, nullptr, nullptr, nullptr, nullptr};
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
     D2cProfScope prof(D2C_PROF_FWD, st);
-    hipLaunchKernelGGL(dw_fwd_kernel<T>, dim3((s.M + kFwdTP - 1) / kFwdTP, s.G * nsl), dim3(kDwThreads), kDwLdsFwd, st, a);
+    hipLaunchKernelGGL(dw_fwd_kernel<T>, dim3(dw_grid(s, kFwdTP, s.G * nsl)), dim3(kDwThreads), kDwLdsFwd, st, a);
     return d2c_check_launch("dw_fwd_kernel");
 }
 
@@ -462,8 +479,7 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
         if (hipFuncSetAttribute((const void *)dw_bwd_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)kDwLdsBwd) != hipSuccess)
             return d2c_check_launch("hipFuncSetAttribute(dw_bwd_kernel)");
-        hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3((s.M + kBwdTP - 1) / kBwdTP, s.G * nsl), dim3(kDwThreads), kDwLdsBwd, st,
-                           a);
+        hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3(dw_grid(s, kBwdTP, s.G * nsl)), dim3(kDwThreads), kDwLdsBwd, st, a);
     }
     if (int rc = d2c_check_launch("dw_bwd_kernel")) return rc;
     if (goff || gmask) {

@@ -298,9 +298,12 @@ gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
 // gcol[p, k, c] = W[c, k] * gout[p, c] is one multiply, so no grad-column buffer
 // exists: the owner of a voxel reads the channels-last grad_out row of each
 // sample that reaches it and the weight row of its tap (staged in LDS).
-// A workgroup = kOwnVox 2 x 2 x 2 cubes of voxels consecutive in x, 256 lanes each;
-// a lane owns kOwnCV consecutive channels (one vector load per lane and row).
-constexpr int kOwnVox = 4, kOwnCV = 4, kOwnSlice = 256 * kOwnCV;
+// A workgroup = kOwnVox 2 x 2 x 2 cubes of voxels consecutive in x, one wavefront
+// each, and a slice of kOwnSlice channels; a lane owns kOwnCV consecutive channels
+// (one vector load per lane and row).  xcd_unit() gives every XCD one channel slice
+// of one batch element at a time, so that the grad_out rows its workgroups gather
+// (6.6 MB for 256 fp32 channels of 8x15x27 positions) stay in its L2.
+constexpr int kOwnVox = 4, kOwnCV = 4, kOwnSlice = 64 * kOwnCV;
 
 template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
 {
@@ -315,120 +318,118 @@ template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256 * kOwnVox)
+__global__ void __launch_bounds__(64 * kOwnVox)
 dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts, const InvEntry *entries,
                    float *gxcl, int w_in_lds)
 {
-    // One 256-lane group per 2 x 2 x 2 cube of voxels (kOwnVox cubes consecutive in x per workgroup, sharing the
+    // One wavefront per 2 x 2 x 2 cube of voxels (kOwnVox cubes consecutive in x per workgroup, sharing the
     // weights of the channel slice in LDS): the lists of the 27 base voxels that reach the cube are walked once
     // each and a grad_out row is read once for all the voxels of the cube it contributes to, like
     // gx_owner_cube_kernel does for the dense case.
     extern __shared__ __align__(16) unsigned char smem[];
     T *s_w = reinterpret_cast<T *>(smem);   // [K][kOwnSlice] weights of the channel slice
-    const int t = threadIdx.x & 255;
+    const int t = threadIdx.x & 63;
     // wavefront-uniform quantities, kept in scalar registers
-    const int vox = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
+    const int vox = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const int nbx = (ncx + kOwnVox - 1) / kOwnVox;
-    int blk = xcd_swizzle(blockIdx.x, gridDim.x);   // one contiguous part of the volume per XCD (L2)
+    const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
+    const XcdUnit un = xcd_unit(blockIdx.x, s.N * s.G * nslice, ncz * ncy * nbx);
+    if (!un.ok) return;
+    const int b = un.combo % s.N;
+    const int g = (un.combo / s.N) / nslice, sl = (un.combo / s.N) % nslice;
+    int blk = un.tile;
     const int xb = blk % nbx; blk /= nbx;
-    const int cy = blk % ncy; blk /= ncy;
-    const int cz = blk % ncz;
-    const int b = blk / ncz;
+    const int cy = blk % ncy;
+    const int cz = blk / ncy;
     const int cx = xb * kOwnVox + vox;
     const bool valid = cx < ncx;
     const int x0 = cx * 2, y0 = cy * 2, z0 = cz * 2;
     const int nxb = x0 + 1 < s.W ? 3 : 2;          // base voxels x0-1, x0, x0+1 (the last one only if it is a voxel)
-    const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
     const T *grow = goutcl + (long)b * s.P * s.Cout;
 
-    for (int g = 0; g < s.G; g++) {
-        for (int sl = 0; sl < nslice; sl++) {
-            const int cl = sl * kOwnSlice + t * kOwnCV;   // first channel of this lane inside the offset group
-            const int c = g * s.cpg + cl;
-            const bool cok = cl < s.cpg;                  // cpg is a multiple of kOwnCV
-            if (w_in_lds) {
-                __syncthreads();
-                for (int i = threadIdx.x; i < s.K * kOwnSlice; i += 256 * kOwnVox) {
-                    const int k = i / kOwnSlice, cc = i - k * kOwnSlice;
-                    const int ch = sl * kOwnSlice + cc;
-                    s_w[i] = ch < s.cpg ? wt[(long)k * s.Cin + g * s.cpg + ch] : (T)0;
+    const int cl = sl * kOwnSlice + t * kOwnCV;   // first channel of this lane inside the offset group
+    const int c = g * s.cpg + cl;
+    const bool cok = cl < s.cpg;                  // cpg is a multiple of kOwnCV
+    if (w_in_lds) {
+        for (int i = threadIdx.x; i < s.K * kOwnSlice; i += 64 * kOwnVox) {
+            const int k = i / kOwnSlice, cc = i - k * kOwnSlice;
+            const int ch = sl * kOwnSlice + cc;
+            s_w[i] = ch < s.cpg ? wt[(long)k * s.Cin + g * s.cpg + ch] : (T)0;
+        }
+        __syncthreads();
+    }
+    if (!valid || !cok) return;
+    float acc[2][2][2][kOwnCV];
+#pragma unroll
+    for (int i = 0; i < 8 * kOwnCV; i++) (&acc[0][0][0][0])[i] = 0.f;
+#pragma unroll
+    for (int rz = 0; rz < 3; rz++) {
+        const int zb = z0 - 1 + rz;
+        if (zb > s.D - 1) continue;
+#pragma unroll
+        for (int ry = 0; ry < 3; ry++) {
+            const int yb = y0 - 1 + ry;
+            if (yb > s.H - 1) continue;
+            // the (up to) three base voxels along x are adjacent bins: one range of entries
+            const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
+            const int e0 = starts[bin1], em1 = starts[bin1 + 1], em2 = starts[bin1 + 2], e1 = starts[bin1 + nxb];
+            for (int e = e0; e < e1; e += 4) {
+                InvEntry q[4];
+                float go[4][kOwnCV];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    q[i] = entries[min(e + i, e1 - 1)];
+                    ld_vec4<T>(grow + (long)q[i].p * s.Cout + c, go[i]);
                 }
-                __syncthreads();
-            }
-            if (!valid || !cok) continue;
-            float acc[2][2][2][kOwnCV];
 #pragma unroll
-            for (int i = 0; i < 8 * kOwnCV; i++) (&acc[0][0][0][0])[i] = 0.f;
+                for (int i = 0; i < 4; i++) {
+                    float wk[kOwnCV];
+                    if (w_in_lds) ld_vec4<T>(s_w + q[i].k * kOwnSlice + t * kOwnCV, wk);
+                    else ld_vec4<T>(wt + (long)q[i].k * s.Cin + c, wk);
+                    const float al = e + i < e1 ? q[i].alpha : 0.f;
+                    float v[kOwnCV];
 #pragma unroll
-            for (int rz = 0; rz < 3; rz++) {
-                const int zb = z0 - 1 + rz;
-                if (zb > s.D - 1) continue;
+                    for (int jj = 0; jj < kOwnCV; jj++) v[jj] = wk[jj] * go[i][jj];
+                    // x: offset 0 (base x0-1) reaches voxel 0 with hx; 1 reaches (1-hx, hx); 2 reaches voxel 1 with 1-hx
+                    const float hz = q[i].hz, hy = q[i].hy, hx = q[i].hx;
+                    const bool r0 = e + i < em1, r2 = e + i >= em2;
+                    const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
+                    const float wx1 = r0 ? 0.f : (r2 ? 1.f - hx : hx);
 #pragma unroll
-                for (int ry = 0; ry < 3; ry++) {
-                    const int yb = y0 - 1 + ry;
-                    if (yb > s.H - 1) continue;
-                    // the (up to) three base voxels along x are adjacent bins: one range of entries
-                    const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
-                    const int e0 = starts[bin1], em1 = starts[bin1 + 1], em2 = starts[bin1 + 2], e1 = starts[bin1 + nxb];
-                    for (int e = e0; e < e1; e += 4) {
-                        InvEntry q[4];
-                        float go[4][kOwnCV];
+                    for (int az = 0; az < 2; az++) {
+                        if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
+                        const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            q[i] = entries[min(e + i, e1 - 1)];
-                            ld_vec4<T>(grow + (long)q[i].p * s.Cout + c, go[i]);
-                        }
+                        for (int ay = 0; ay < 2; ay++) {
+                            if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
+                            const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
+                            const float wzy = wz * wy * al;
+                            const float w0 = wzy * wx0, w1 = wzy * wx1;
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            float wk[kOwnCV];
-                            if (w_in_lds) ld_vec4<T>(s_w + q[i].k * kOwnSlice + t * kOwnCV, wk);
-                            else ld_vec4<T>(wt + (long)q[i].k * s.Cin + c, wk);
-                            const float al = e + i < e1 ? q[i].alpha : 0.f;
-                            float v[kOwnCV];
-#pragma unroll
-                            for (int jj = 0; jj < kOwnCV; jj++) v[jj] = wk[jj] * go[i][jj];
-                            // x: offset 0 (base x0-1) reaches voxel 0 with hx; 1 reaches (1-hx, hx); 2 reaches voxel 1 with 1-hx
-                            const float hz = q[i].hz, hy = q[i].hy, hx = q[i].hx;
-                            const bool r0 = e + i < em1, r2 = e + i >= em2;
-                            const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
-                            const float wx1 = r0 ? 0.f : (r2 ? 1.f - hx : hx);
-#pragma unroll
-                            for (int az = 0; az < 2; az++) {
-                                if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
-                                const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
-#pragma unroll
-                                for (int ay = 0; ay < 2; ay++) {
-                                    if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
-                                    const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
-                                    const float wzy = wz * wy * al;
-                                    const float w0 = wzy * wx0, w1 = wzy * wx1;
-#pragma unroll
-                                    for (int jj = 0; jj < kOwnCV; jj++) {
-                                        acc[az][ay][0][jj] = fmaf(w0, v[jj], acc[az][ay][0][jj]);
-                                        acc[az][ay][1][jj] = fmaf(w1, v[jj], acc[az][ay][1][jj]);
-                                    }
-                                }
+                            for (int jj = 0; jj < kOwnCV; jj++) {
+                                acc[az][ay][0][jj] = fmaf(w0, v[jj], acc[az][ay][0][jj]);
+                                acc[az][ay][1][jj] = fmaf(w1, v[jj], acc[az][ay][1][jj]);
                             }
                         }
                     }
                 }
             }
-#pragma unroll
-            for (int az = 0; az < 2; az++)
-#pragma unroll
-                for (int ay = 0; ay < 2; ay++)
-#pragma unroll
-                    for (int ax = 0; ax < 2; ax++) {
-                        const int z = z0 + az, y = y0 + ay, x = x0 + ax;
-                        if (z < s.D && y < s.H && x < s.W) {
-                            const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;
-                            *reinterpret_cast<float4 *>(gxcl + vg * s.Cin + c) =
-                                make_float4(acc[az][ay][ax][0], acc[az][ay][ax][1], acc[az][ay][ax][2], acc[az][ay][ax][3]);
-                        }
-                    }
         }
     }
+#pragma unroll
+    for (int az = 0; az < 2; az++)
+#pragma unroll
+        for (int ay = 0; ay < 2; ay++)
+#pragma unroll
+            for (int ax = 0; ax < 2; ax++) {
+                const int z = z0 + az, y = y0 + ay, x = x0 + ax;
+                if (z < s.D && y < s.H && x < s.W) {
+                    const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;
+                    *reinterpret_cast<float4 *>(gxcl + vg * s.Cin + c) =
+                        make_float4(acc[az][ay][ax][0], acc[az][ay][ax][1], acc[az][ay][ax][2], acc[az][ay][ax][3]);
+                }
+            }
 }
 
 inline unsigned g1d(long n, int cap = 16384)
@@ -560,8 +561,9 @@ int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *
                             160 * 1024) != hipSuccess)
         return d2c_check_launch("hipFuncSetAttribute(dw_gx_owner_kernel)");
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
-    const long nblk = (long)s.N * ncz * ncy * ((ncx + kOwnVox - 1) / kOwnVox);
-    hipLaunchKernelGGL(dw_gx_owner_kernel<T>, dim3((unsigned)nblk), dim3(256 * kOwnVox), lds, st, s, (const T *)goutcl,
+    const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
+    const unsigned nblk = xcd_unit_grid(s.N * s.G * nslice, ncz * ncy * ((ncx + kOwnVox - 1) / kOwnVox));
+    hipLaunchKernelGGL(dw_gx_owner_kernel<T>, dim3(nblk), dim3(64 * kOwnVox), lds, st, s, (const T *)goutcl,
                        (const T *)wt, starts, (const InvEntry *)entries, gxcl, w_in_lds);
     return d2c_check_launch("dw_gx_owner_kernel");
 }

@@ -150,6 +150,39 @@ D2C_DEV int bin_of(const TiledShape &s, int b, int g, int z0, int y0, int x0)
     return (((b * s.G + g) * (s.D + 1) + (z0 + 1)) * (s.H + 1) + (y0 + 1)) * (s.W + 1) + (x0 + 1);
 }
 
+// Mapping of a 1-D grid onto the 8 XCDs, each with an L2 of its own; workgroups are dealt to them round-robin.
+// The work is `ncombo` combinations (of batch element, channel slice, ...) of `tpb` tiles each.  It is cut
+// into units of (combination, part of its tiles), their number a multiple of 8, and unit u runs on XCD u % 8,
+// its tiles in order: the L2 of an XCD then holds the data of one combination at a time.  The grid is
+// xcd_unit_grid() workgroups; those with ok == false have no tile.
+struct XcdUnit {
+    int combo, tile;
+    bool ok;
+};
+__host__ __device__ inline int xcd_unit_parts(int ncombo)
+{
+    const int low = ncombo & -ncombo;   // largest power of two dividing ncombo
+    return low >= 8 ? 1 : 8 / low;
+}
+D2C_DEV XcdUnit xcd_unit(int bid, int ncombo, int tpb)
+{
+    const int parts = xcd_unit_parts(ncombo);
+    const int tpp = (tpb + parts - 1) / parts;      // tiles of a part
+    const int xcd = bid & 7, idx = bid >> 3;
+    const int j = idx / tpp, t = idx - j * tpp;
+    const int u = j * 8 + xcd;
+    XcdUnit r;
+    r.combo = u / parts;
+    r.tile = (u - r.combo * parts) * tpp + t;
+    r.ok = r.tile < tpb;
+    return r;
+}
+inline unsigned xcd_unit_grid(int ncombo, int tpb)
+{
+    const int parts = xcd_unit_parts(ncombo);
+    return (unsigned)(ncombo * parts * ((tpb + parts - 1) / parts));
+}
+
 // Lists as buckets of fixed capacity, filled in one pass (a counter per bin; no counting pass, no scan).
 // A sample that finds its bucket full goes to one shared overflow array instead, which a separate kernel
 // adds into grad_input with atomics: rare for real offset fields (a bucket holds more than twice the mean
