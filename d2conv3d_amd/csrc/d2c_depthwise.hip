@@ -255,6 +255,30 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
 // ----------------------------------------------------------------- backward
 // Sum of 4 per-lane values over the 64 lanes: after the exchange steps lane
 // group (lane>>4) holds the total of value (lane>>4) in all of its lanes.
+// Load of a lane's 4 channels from a wavefront-uniform row address plus the lane's byte offset.  The row
+// address is pinned to scalar registers, so that the load needs no 64-bit vector arithmetic.
+template <typename T> D2C_DEV void ld4_row(const T *row, unsigned lane_bytes, float *v)
+{
+    typedef const __attribute__((address_space(1))) char *gptr;
+    const unsigned long long a = reinterpret_cast<unsigned long long>(row);
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)a);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(a >> 32));
+    gptr p = (gptr)(((unsigned long long)hi << 32) | lo) + lane_bytes;
+    typedef float f32x4v __attribute__((ext_vector_type(4)));
+    typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
+    if constexpr (sizeof(T) == 4) {
+        const f32x4v t = *reinterpret_cast<const __attribute__((address_space(1))) f32x4v *>(p);
+        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+    } else {
+        const u32x2v t = *reinterpret_cast<const __attribute__((address_space(1))) u32x2v *>(p);
+        v[0] = __uint_as_float(t[0] << 16); v[1] = __uint_as_float(t[0] & 0xffff0000u);
+        v[2] = __uint_as_float(t[1] << 16); v[3] = __uint_as_float(t[1] & 0xffff0000u);
+    }
+}
+template <int CTRL> D2C_DEV float dpp_add(float v)
+{
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
 D2C_DEV float reduce4_over_wave(float v0, float v1, float v2, float v3, int lane)
 {
     // step 1: lanes with bit 5 set keep (v2, v3), others (v0, v1)
@@ -267,15 +291,16 @@ D2C_DEV float reduce4_over_wave(float v0, float v1, float v2, float v3, int lane
     const bool hi4 = lane & 16;
     float k = hi4 ? k1 : k0, sd = hi4 ? k0 : k1;
     k += __shfl_xor(sd, 16, 64);
-    k += __shfl_xor(k, 8, 64);
-    k += __shfl_xor(k, 4, 64);
-    k += __shfl_xor(k, 2, 64);
-    k += __shfl_xor(k, 1, 64);
+    // inside the rows of 16 lanes: neighbours of a quad, then rotations of the row by 4 and by 8 lanes
+    k = dpp_add<0xB1>(k);    // quad_perm [1, 0, 3, 2]
+    k = dpp_add<0x4E>(k);    // quad_perm [2, 3, 0, 1]
+    k = dpp_add<0x124>(k);   // row_ror 4
+    k = dpp_add<0x128>(k);   // row_ror 8
     return k;   // value index = (lane >> 5) * 2 + ((lane >> 4) & 1)
 }
 
 template <typename T>
-__global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
+__global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 wavefronts per SIMD: what the LDS allows
 {
     constexpr int TP = kBwdTP, KB = kBwdKB;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -306,41 +331,53 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
             float wv[kCV] = {0.f, 0.f, 0.f, 0.f};
             if (cok) ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
             float gwv[kCV] = {0.f, 0.f, 0.f, 0.f};
-            for (int p = 0; p < TP; p++) {
-                const int e = kk * TP + p;
-                // the table entry is the same for the whole wavefront: keep it in scalar registers
-                const unsigned flag = (unsigned)__builtin_amdgcn_readfirstlane(taps.flag[e]);
-                const unsigned inr = flag >> 8, live = flag & 0xffu;
-                if (!inr) continue;
-                const int idx = __builtin_amdgcn_readfirstlane(taps.idx[e]);
-                const int m = m0 + p;                     // m < m_end holds where inr != 0
-                float go[kCV] = {0.f, 0.f, 0.f, 0.f};
-                if (cok) ld4<T>(goutcl + (long)m * s.Cout + c, go);
-                float gc[kCV];
-#pragma unroll
-                for (int j = 0; j < kCV; j++) gc[j] = wv[j] * go[j];
-                float xv[8][kCV];
+            // table entries of the tap's positions: lane p holds those of position p; they are the same for the
+            // whole wavefront and are read out into scalar registers
+            const int vflag = taps.flag[kk * TP + (lane & (TP - 1))];
+            const int vidx = taps.idx[kk * TP + (lane & (TP - 1))];
+            // The rows of a position (grad_out and the 8 corners) are requested one position ahead of their use.
+            // Every request is made: a corner out of range reads voxel 0 and its dot product is dropped, a
+            // position past the tile reads the tile's last grad_out row and has no corner in range.  Lanes past
+            // the offset group read channel 0 on and hold a zero weight.
+            struct Rows {
+                float x[8][kCV], go[kCV];
+            };
+            unsigned cbytes = (unsigned)c * (unsigned)sizeof(T);
+            asm volatile("" : "+v"(cbytes));   // kept a plain 32-bit register: the offset operand of the loads
+            auto issue = [&](Rows &r, int p) {
+                const unsigned inr = (unsigned)__builtin_amdgcn_readlane(vflag, p) >> 8;
+                const int idx = __builtin_amdgcn_readlane(vidx, p);
+                const int m = min(m0 + p, m_end - 1);
+                // row address in scalar registers + the lane's byte offset
+                ld4_row<T>(goutcl + (size_t)m * s.Cout, cbytes, r.go);
 #pragma unroll
                 for (int cc = 0; cc < 8; cc++) {
-                    const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
-                    if (((inr >> cc) & 1u) && cok) {
-                        ld4<T>(xcl + (long)v * s.Cin + c, xv[cc]);
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < kCV; j++) xv[cc][j] = 0.f;
-                    }
+                    const int v = ((inr >> cc) & 1u) ? idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1) : 0;
+                    ld4_row<T>(xcl + (size_t)v * s.Cin, cbytes, r.x[cc]);
                 }
+            };
+            float stash = 0.f;
+            static_assert(TP == 16, "a row of 16 lanes per result");
+            auto compute = [&](const Rows &r, int p) {
+                const int e = kk * TP + p;
+                const unsigned flag = (unsigned)__builtin_amdgcn_readlane(vflag, p);
+                const unsigned inr = flag >> 8, live = flag & 0xffu;
+                if (!inr) return;
+                const int idx = __builtin_amdgcn_readlane(vidx, p);
+                float gc[kCV];
+#pragma unroll
+                for (int j = 0; j < kCV; j++) gc[j] = wv[j] * (cok ? r.go[j] : 0.f);
                 float dot[8];
                 float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int cc = 0; cc < 8; cc++) {
                     float d = 0.f;
 #pragma unroll
-                    for (int j = 0; j < kCV; j++) d = fmaf(gc[j], xv[cc][j], d);
+                    for (int j = 0; j < kCV; j++) d = fmaf(gc[j], r.x[cc][j], d);
                     if ((live >> cc) & 1u) {
                         const float wc = taps.w[cc][e];   // a_corner * alpha
 #pragma unroll
-                        for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, xv[cc][j], sv[j]);
+                        for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, r.x[cc][j], sv[j]);
                         if (a.gxcl && cok) {
                             const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
                             float *gp = a.gxcl + (long)v * s.Cin + c;
@@ -348,34 +385,68 @@ __global__ void __launch_bounds__(kDwThreads) dw_bwd_kernel(DwArgs a)
                             for (int j = 0; j < kCV; j++) atomicAdd(gp + j, wc * gc[j]);
                         }
                     }
-                    dot[cc] = d;
+                    dot[cc] = ((inr >> cc) & 1u) ? d : 0.f;
                 }
 #pragma unroll
-                for (int j = 0; j < kCV; j++) gwv[j] = fmaf(go[j], sv[j], gwv[j]);   // sv already holds alpha
+                for (int j = 0; j < kCV; j++) gwv[j] = fmaf(r.go[j], sv[j], gwv[j]);   // sv already holds alpha
                 if (want_aux) {
                     const float lz = taps.frac[0][e], ly = taps.frac[1][e], lx = taps.frac[2][e];
                     const float hz = taps.frac[3][e], hy = taps.frac[4][e], hx = taps.frac[5][e];
-                    float gz = 0.f, gy = 0.f, gxx = 0.f, gm = 0.f;
+                    // The four results are trilinear forms of the dot products; they are taken axis by axis
+                    // (x, then y, then z): interpolated sums and differences.
+                    float sx[4], dx[4];   // index = z * 2 + y
 #pragma unroll
-                    for (int cc = 0; cc < 8; cc++) {
-                        const float wz = (cc & 4) ? hz : lz, wy = (cc & 2) ? hy : ly, wx = (cc & 1) ? hx : lx;
-                        const float d = dot[cc];
-                        gz += ((cc & 4) ? d : -d) * (wy * wx);
-                        gy += ((cc & 2) ? d : -d) * (wz * wx);
-                        gxx += ((cc & 1) ? d : -d) * (wz * wy);
-                        if ((live >> cc) & 1u) gm += (wz * wy * wx) * d;
+                    for (int i = 0; i < 4; i++) {
+                        sx[i] = fmaf(hx, dot[2 * i + 1], lx * dot[2 * i]);
+                        dx[i] = dot[2 * i + 1] - dot[2 * i];
                     }
-                    // sums over the 256 channels of the slice; the other slices of the group add theirs
-                    const float r = reduce4_over_wave(gz, gy, gxx, gm, lane);
-                    if ((lane & 15) == 0) {
-                        const int which = (lane >> 5) * 2 + ((lane >> 4) & 1);
-                        const int b = m / s.P, pp = m - b * s.P;
-                        const long ab = (((long)b * s.G + g) * s.K + (k0 + kk)) * s.P + pp;
-                        if (which < 3) {
-                            if (a.auxoff) atomicAdd(a.auxoff + 3 * ab - 2 * (long)pp + which * (long)s.P, taps.alpha[e] * r);
-                        } else if (a.auxmask) {
-                            atomicAdd(a.auxmask + ab, r);
+                    float sxy[2], dy[2], sdx[2];   // index = z
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+                        sxy[i] = fmaf(hy, sx[2 * i + 1], ly * sx[2 * i]);
+                        dy[i] = sx[2 * i + 1] - sx[2 * i];
+                        sdx[i] = fmaf(hy, dx[2 * i + 1], ly * dx[2 * i]);
+                    }
+                    const float gz = sxy[1] - sxy[0];
+                    const float gy = fmaf(hz, dy[1], lz * dy[0]);
+                    const float gxx = fmaf(hz, sdx[1], lz * sdx[0]);
+                    float gm = fmaf(hz, sxy[1], lz * sxy[0]);
+                    if (live != inr) {
+                        // the modulation gradient takes the corners of the forward pass only
+                        gm = 0.f;
+#pragma unroll
+                        for (int cc = 0; cc < 8; cc++) {
+                            const float wz = (cc & 4) ? hz : lz, wy = (cc & 2) ? hy : ly, wx = (cc & 1) ? hx : lx;
+                            if ((live >> cc) & 1u) gm += (wz * wy * wx) * dot[cc];
                         }
+                    }
+                    // sums over the 256 channels of the slice; lane (which * 16 + p) keeps result `which` of
+                    // position p until all positions of the tap are done
+                    const float rs = reduce4_over_wave(gz, gy, gxx, gm, lane);
+                    const float val = lane < 48 ? taps.alpha[e] * rs : rs;
+                    stash = (lane & (TP - 1)) == p ? val : stash;
+                }
+            };
+            static_assert(TP % 2 == 0, "positions are worked on in pairs");
+            Rows ra, rb;
+            issue(ra, 0);
+            for (int p = 0; p < TP; p += 2) {
+                issue(rb, p + 1);
+                compute(ra, p);
+                issue(ra, min(p + 2, TP - 1));   // after the last pair: a repeat, not used
+                compute(rb, p + 1);
+            }
+            if (want_aux) {
+                // one atomic instruction per tap: 16 consecutive positions per result; the other channel slices
+                // of the offset group add theirs to the same places
+                const int which = lane >> 4, m = m0 + (lane & (TP - 1));
+                if (m < m_end) {
+                    const int b = m / s.P, pp = m - b * s.P;
+                    const long ab = (((long)b * s.G + g) * s.K + (k0 + kk)) * s.P + pp;
+                    if (which < 3) {
+                        if (a.auxoff) atomicAdd(a.auxoff + 3 * ab - 2 * (long)pp + which * (long)s.P, stash);
+                    } else if (a.auxmask) {
+                        atomicAdd(a.auxmask + ab, stash);
                     }
                 }
             }
