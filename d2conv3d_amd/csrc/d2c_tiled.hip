@@ -135,6 +135,49 @@ __global__ void __launch_bounds__(256) pack_weight_fwd_kernel(const T *w, T *wp,
     }
 }
 
+// The same re-layout through LDS: a workgroup takes kPackRows output channels of one channel chunk, whose
+// weights are runs of BKC * K consecutive elements in W, reads them with 16-byte loads and writes whole
+// 16-byte fragment vectors (kPackRows consecutive lanes each).  Needs a 16-byte aligned W and rows that fit LDS.
+constexpr int kPackRows = 16;
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_fwd_lds_kernel(const T *w, T *wp, TiledShape s)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, R = kPackRows;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int OBT = s.ogp / 32, S = s.nchunk * s.K;
+    int b = blockIdx.x;
+    const int part = b % (32 / R); b /= 32 / R;
+    const int obg = b % OBT; b /= OBT;
+    const int j = b % s.nchunk;
+    const int wg = b / s.nchunk;
+    const int run = BKC * s.K;                       // elements of a row
+    const int rs = run * (int)sizeof(T) + 4;         // LDS row stride in bytes (an odd number of banks)
+    const int ol0 = obg * 32 + part * R;
+    const int vpr = run * (int)sizeof(T) / 16;       // 16-byte vectors of a row
+    for (int i = threadIdx.x; i < R * vpr; i += 256) {
+        const int r = i / vpr, v = i - r * vpr;
+        const int ol = ol0 + r;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (ol < s.og)
+            val = *reinterpret_cast<const uint4 *>(
+                reinterpret_cast<const char *>(w + ((long)(wg * s.og + ol) * s.cg + j * BKC) * s.K) + (size_t)v * 16);
+        unsigned *d = reinterpret_cast<unsigned *>(smem + r * rs + v * 16);
+        d[0] = val.x; d[1] = val.y; d[2] = val.z; d[3] = val.w;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < s.K * 8 * R; i += 256) {
+        const int r = i % R, q = i / R;
+        const int khi = q & 7, k = q >> 3;           // khi = 2 * k-group + lane / 32
+        const T *src = reinterpret_cast<const T *>(smem + r * rs) + khi * VEC * s.K + k;
+        alignas(16) T tmp[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) tmp[e] = src[e * s.K];
+        const int lane = (khi & 1) * 32 + part * R + r;
+        const long vi = ((((long)wg * S + j * s.K + k) * OBT + obg) * 4 + (khi >> 1)) * 64 + lane;
+        *reinterpret_cast<uint4 *>(wp + vi * VEC) = *reinterpret_cast<const uint4 *>(tmp);
+    }
+}
+
 struct FwdWs {
     size_t xcl, wp, outacc, total;
 };
@@ -216,8 +259,14 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
     if (g > 8192) g = 8192;
     {
         D2cProfScope prof(D2C_PROF_PACK, st);
-        hipLaunchKernelGGL(pack_weight_fwd_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, (const T *)w,
-                           (T *)(base + l.wp), s, total);
+        const size_t lds = (size_t)kPackRows * ((size_t)bkc_of(q.dtype) * s.K * sizeof(T) + 4);
+        if (lds <= 64 * 1024 && reinterpret_cast<uintptr_t>(w) % 16 == 0)
+            hipLaunchKernelGGL(pack_weight_fwd_lds_kernel<T>,
+                               dim3((unsigned)(s.groups * s.nchunk * (s.ogp / 32) * (32 / kPackRows))), dim3(256), lds, st,
+                               (const T *)w, (T *)(base + l.wp), s);
+        else
+            hipLaunchKernelGGL(pack_weight_fwd_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, (const T *)w,
+                               (T *)(base + l.wp), s, total);
     }
     if (int rc = d2c_check_launch("pack_weight_fwd_kernel")) return rc;
     return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, (float *)(base + l.outacc), st);

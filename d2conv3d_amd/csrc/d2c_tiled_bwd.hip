@@ -693,6 +693,49 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
     }
 }
 
+// The same re-layout through LDS (needs a 16-byte aligned W): a workgroup takes a block of output channels
+// as wide as the padding unit of ogk (128 bytes of wt) and kPackCh channels of a chunk, whose weights are
+// runs of kPackCh * K consecutive elements in W, and writes 16-byte vectors of consecutive output channels.
+constexpr int kPackCh = 16;
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_bwd_lds_kernel(const T *w, T *wt, TiledShape s, int ogk, int o0,
+                                                                  int ogn)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, R = 128 / (int)sizeof(T), CB = BKC / kPackCh;
+    extern __shared__ __align__(16) unsigned char smem[];
+    int b = blockIdx.x;
+    const int cb = b % CB; b /= CB;
+    const int obk = b % (ogk / R); b /= ogk / R;
+    const int j = b % s.nchunk;
+    const int wg = b / s.nchunk;
+    const int run = kPackCh * s.K;                   // elements of a row
+    const int rs = run * (int)sizeof(T) + 4;         // LDS row stride in bytes (an odd number of banks)
+    const int vpr = run * (int)sizeof(T) / 16;
+    for (int i = threadIdx.x; i < R * vpr; i += 256) {
+        const int r = i / vpr, v = i - r * vpr;
+        const int oo = obk * R + r;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (oo < ogn)
+            val = *reinterpret_cast<const uint4 *>(
+                reinterpret_cast<const char *>(w + ((long)(wg * s.og + o0 + oo) * s.cg + j * BKC + cb * kPackCh) * s.K) +
+                (size_t)v * 16);
+        unsigned *d = reinterpret_cast<unsigned *>(smem + r * rs + v * 16);
+        d[0] = val.x; d[1] = val.y; d[2] = val.z; d[3] = val.w;
+    }
+    __syncthreads();
+    const int cpc = s.cpg / BKC;   // same step order as tiled_bwd_data_kernel
+    for (int i = threadIdx.x; i < s.K * kPackCh * (R / VEC); i += 256) {
+        const int ov = i % (R / VEC), q = i / (R / VEC);
+        const int cc = q % kPackCh, k = q / kPackCh;
+        alignas(16) T tmp[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) tmp[e] = reinterpret_cast<const T *>(smem + (ov * VEC + e) * rs)[cc * s.K + k];
+        const int st = ((j / cpc) * s.K + k) * cpc + j % cpc;
+        const long di = (((long)wg * s.K * s.nchunk + st) * BKC + cb * kPackCh + cc) * ogk + obk * R + ov * VEC;
+        *reinterpret_cast<uint4 *>(wt + di) = *reinterpret_cast<const uint4 *>(tmp);
+    }
+}
+
 // fp32 channels-last accumulator [N][vol][C] -> grad_input [N][C][vol] of type T
 template <typename T>
 __global__ void __launch_bounds__(256) unpack_grad_input_kernel(const float *gxcl, T *gx, int C, int vol)
@@ -726,6 +769,42 @@ __global__ void __launch_bounds__(256) cvt_grad_weight_kernel(const float *src, 
         const int o = (int)(i / ((long)s.K * s.cg));
         const int wg = o / s.og, ol = o - wg * s.og, j = cl / BKC, cc = cl - j * BKC;
         dst[i] = f32_to_elem<T>(src[(((long)wg * s.nchunk * s.K + j * s.K + k) * s.og + ol) * BKC + cc]);
+    }
+}
+
+// The same through LDS (needs a 16-byte aligned grad_weight): a workgroup takes kCvtRows output channels of one
+// channel chunk; per tap their accumulator rows are one contiguous piece, and in grad_weight they are runs
+// of BKC * K consecutive elements.
+constexpr int kCvtRows = 16;
+template <typename T>
+__global__ void __launch_bounds__(256) cvt_grad_weight_lds_kernel(const float *src, T *dst, TiledShape s)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, R = kCvtRows;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int nrb = (s.og + R - 1) / R;
+    int b = blockIdx.x;
+    const int rb = b % nrb; b /= nrb;
+    const int j = b % s.nchunk;
+    const int wg = b / s.nchunk;
+    const int run = BKC * s.K;
+    const int rs = run * (int)sizeof(T) + 16;        // LDS row stride in bytes
+    const int nr = min(R, s.og - rb * R);
+    // accumulator [tap][row][channel] -> LDS [row][channel][tap], converted
+    for (int i = threadIdx.x; i < s.K * nr * (BKC / 4); i += 256) {
+        const int c4 = i % (BKC / 4), q = i / (BKC / 4);
+        const int r = q % nr, k = q / nr;
+        const float4 v = *reinterpret_cast<const float4 *>(
+            src + (((long)wg * s.nchunk * s.K + j * s.K + k) * s.og + rb * R + r) * BKC + c4 * 4);
+        T *d = reinterpret_cast<T *>(smem + r * rs) + (c4 * 4) * s.K + k;
+        d[0] = f32_to_elem<T>(v.x); d[s.K] = f32_to_elem<T>(v.y);
+        d[2 * s.K] = f32_to_elem<T>(v.z); d[3 * s.K] = f32_to_elem<T>(v.w);
+    }
+    __syncthreads();
+    const int vpr = run * (int)sizeof(T) / 16;
+    for (int i = threadIdx.x; i < nr * vpr; i += 256) {
+        const int r = i / vpr, v = i - r * vpr;
+        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(dst + ((long)(wg * s.og + rb * R + r) * s.cg + j * BKC) * s.K) +
+                                   (size_t)v * 16) = *reinterpret_cast<const uint4 *>(smem + r * rs + v * 16);
     }
 }
 
@@ -889,8 +968,15 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
         {
             D2cProfScope prof(D2C_PROF_PACK, st);
-            hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w, (T *)wt,
-                               s, ogk, o0, ogn, total);
+            constexpr int R = 128 / (int)sizeof(T);
+            const size_t lds = (size_t)R * ((size_t)kPackCh * s.K * sizeof(T) + 4);
+            if (lds <= 64 * 1024 && reinterpret_cast<uintptr_t>(w) % 16 == 0)
+                hipLaunchKernelGGL(pack_weight_bwd_lds_kernel<T>,
+                                   dim3((unsigned)(s.groups * s.nchunk * (ogk / R) * (BKC / kPackCh))), dim3(256), lds, st,
+                                   (const T *)w, (T *)wt, s, ogk, o0, ogn);
+            else
+                hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w,
+                                   (T *)wt, s, ogk, o0, ogn, total);
         }
         if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
         BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0,
@@ -980,7 +1066,14 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     }
     if (int rc = d2c_check_launch("tiled_bwd_weight_dma_kernel")) return rc;
     D2cProfScope prof(D2C_PROF_PACK, st);
-    hipLaunchKernelGGL(cvt_grad_weight_kernel<T>, dim3(grid1d(nw)), dim3(256), 0, st, gwacc, (T *)gw, s, nw);
+    constexpr int BKC = 8 * Elem<T>::VEC;
+    const size_t cvt_lds = (size_t)kCvtRows * ((size_t)BKC * s.K * sizeof(T) + 16);
+    if (cvt_lds <= 64 * 1024 && reinterpret_cast<uintptr_t>(gw) % 16 == 0)
+        hipLaunchKernelGGL(cvt_grad_weight_lds_kernel<T>,
+                           dim3((unsigned)(s.groups * s.nchunk * ((s.og + kCvtRows - 1) / kCvtRows))), dim3(256), cvt_lds,
+                           st, gwacc, (T *)gw, s);
+    else
+        hipLaunchKernelGGL(cvt_grad_weight_kernel<T>, dim3(grid1d(nw)), dim3(256), 0, st, gwacc, (T *)gw, s, nw);
     return d2c_check_launch("cvt_grad_weight_kernel");
 }
 
