@@ -100,14 +100,17 @@ def algorithmic(name, N=None, dims=None):
 def hbm_traffic_bytes(workload, kernel):
     """HBM bytes per launch of `kernel`, from the committed rocprofv3 --pmc summary of the workload
     (FETCH_SIZE + WRITE_SIZE, calibrated on a plain copy kernel); None if not recorded."""
-    path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.md")
-    try:
-        for row in open(path):
-            cells = [c.strip().strip("`") for c in row.split("|")]
-            if len(cells) > 4 and cells[1].startswith(kernel[:-len("_kernel")] if kernel.endswith("_kernel") else kernel):
-                return int(float(cells[4]) * 1e6)
-    except (OSError, ValueError):
-        pass
+    import glob
+    stem = kernel[:-len("_kernel")] if kernel.endswith("_kernel") else kernel
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", f"{workload}_*.md"))):
+        try:
+            for row in open(path):
+                cells = [c.strip().strip("`") for c in row.split("|")]
+                # the traffic table: | kernel | fetch MB | write MB | total MB |
+                if len(cells) == 6 and cells[1].startswith(stem):
+                    return int(float(cells[4]) * 1e6)
+        except (OSError, ValueError):
+            pass
     return None
 
 

@@ -270,8 +270,9 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
 // ---------------------------------------------------------------------------
 // The same forward pass with the corner rows moved global -> LDS by DMA loads
 // (global_load_lds_dwordx4: no staging registers; the rows of step s+2 are
-// requested at the end of iteration s and are in flight over the barrier and
-// the matrix-core phase of iteration s+1).
+// requested during the matrix-core phase of iteration s, a few requests
+// between each pair of MFMAs, and are in flight over the interpolation of
+// step s+1 and the barrier).
 // One workgroup = 512 + 64 threads = 64 positions x NT output channels.  One DMA
 // instruction of a wavefront fetches the 8 corner rows (8 x 128 bytes) of one
 // position: lane = (corner, 16-byte vector); corners that are out of range or
