@@ -792,9 +792,9 @@ int launch_fwd_cfg(const FwdArgs &a, int nt, hipStream_t st)
 
 }  // namespace
 
-// Wide weight groups on problems with enough position tiles run the DMA-gather kernel (64-position tiles, all
-// 512 output channels per workgroup); everything else the register-gather kernel (128-position tiles).
-bool d2c_fwd_use_dma(int og, int M, int groups) { return og > 256 && (long)((M + kDMT - 1) / kDMT) * groups >= 128; }
+// Wide weight groups on problems with enough position tiles run the DMA-gather kernel (64-position tiles, 512 or
+// 256 output channels per workgroup); everything else the register-gather kernel (128-position tiles).
+bool d2c_fwd_use_dma(int og, int M, int groups) { return og > 128 && (long)((M + kDMT - 1) / kDMT) * groups >= 128; }
 
 int d2c_fwd_pos_tile(int og, int M, int groups) { return d2c_fwd_use_dma(og, M, groups) ? kDMT : kMT; }
 
@@ -803,7 +803,7 @@ int d2c_fwd_pos_tile(int og, int M, int groups) { return d2c_fwd_use_dma(og, M, 
 // tiles to occupy the chip.
 int d2c_fwd_out_tile(int og, int M, int groups)
 {
-    if (d2c_fwd_use_dma(og, M, groups)) return 512;
+    if (d2c_fwd_use_dma(og, M, groups)) return og > 256 ? 512 : 256;
     int nt = og > 256 ? 512 : (og > 128 ? 256 : (og > 64 ? 128 : 64));
     const int ntile = (M + kMT - 1) / kMT;
     while (nt > 64 && ntile * ((og + nt - 1) / nt) < 128) nt >>= 1;
@@ -842,10 +842,16 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
     if (dma) {
-        if constexpr (sizeof(T) == 2) {
-            if (aux16) return launch_fwd_dma<T, true, 8, 1>(a, outacc, st);
+        if (nt == 512) {
+            if constexpr (sizeof(T) == 2) {
+                if (aux16) return launch_fwd_dma<T, true, 8, 1>(a, outacc, st);
+            }
+            return launch_fwd_dma<T, false, 8, 1>(a, outacc, st);
         }
-        return launch_fwd_dma<T, false, 8, 1>(a, outacc, st);
+        if constexpr (sizeof(T) == 2) {
+            if (aux16) return launch_fwd_dma<T, true, 4, 2>(a, outacc, st);
+        }
+        return launch_fwd_dma<T, false, 4, 2>(a, outacc, st);
     } else {
         if constexpr (sizeof(T) == 2) {
             if (aux16) rc = launch_fwd_cfg<T, true>(a, nt, st);
