@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the D2Conv3D operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap|dwconv]
 
 One step = one forward (+ one backward with all five gradients, except for
 the forward-only workload c1) of the modulated deformable convolution through
@@ -191,12 +191,100 @@ def bench_size_map(args):
     print(json.dumps(line))
 
 
+def bench_dwconv(args):
+    """Plain depthwise conv3d (the reference's fast-depthwise-conv3d operator; backbone shape: 256 channels,
+    8x56x56, 3x3x3, stride 1, padding 1, float32), forward + backward through the C ABI with pre-allocated
+    buffers; torch's own grouped convolution (MIOpen) is timed beside it on the same GPU."""
+    import ctypes
+    import numpy as np
+    import torch
+    import torch.nn.functional as F
+    from d2conv3d_amd import _lib
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.load()
+    N, C, dims = 2, 256, (8, 56, 56)
+    g = torch.Generator().manual_seed(1006)
+    x = torch.randn(N, C, *dims, generator=g)
+    w = (torch.rand(C, 1, 3, 3, 3, generator=g) * 2 - 1) / 27 ** 0.5
+    b = (torch.rand(C, generator=g) * 2 - 1) / 27 ** 0.5
+    gout = torch.randn(N, C, *dims, generator=g)
+    xd, wd, bd, gd = (t.to(dev) for t in (x, w, b, gout))
+    desc = _lib.DwConv3dDesc(N, C, C, *dims, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, *dims, _lib.D2C_F32)
+    _lib.check(lib.d2c_dwconv3d_check(ctypes.byref(desc)), "check")
+    out, gx, gw, gb = torch.empty_like(xd), torch.empty_like(xd), torch.empty_like(wd), torch.empty_like(bd)
+    nws = lib.d2c_dwconv3d_backward_workspace_bytes(ctypes.byref(desc))
+    ws = torch.empty(max(nws, 256), dtype=torch.uint8, device=dev)
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def forward():
+        _lib.check(lib.d2c_dwconv3d_forward(ctypes.byref(desc), p(xd), p(wd), p(bd), p(out), st), "forward")
+
+    def backward():
+        _lib.check(lib.d2c_dwconv3d_backward(ctypes.byref(desc), p(gd), p(xd), p(wd), p(gx), p(gw), p(gb), p(ws), nws, st),
+                   "backward")
+
+    def step():
+        forward()
+        backward()
+
+    xt, wt, bt = (t.clone().requires_grad_(True) for t in (xd, wd, bd))
+
+    def stock():
+        xt.grad = wt.grad = bt.grad = None
+        F.conv3d(xt, wt, bt, 1, 1, 1, groups=C).backward(gd)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms, ms_f, ms_b, ms_torch = timed(step), timed(forward), timed(backward), timed(stock)
+    # parity of what was just timed, against torch's result on the same tensors (the reference's own check)
+    stock()
+    err = max(float((out - F.conv3d(xd, wd, bd, 1, 1, 1, groups=C)).abs().max()), float((gx - xt.grad).abs().max()),
+              float((gw - wt.grad).abs().max() / wt.grad.abs().max()), float((gb - bt.grad).abs().max() / bt.grad.abs().max()))
+    n_el = x.numel()
+    nbytes = 4 * (2 * n_el + 3 * n_el + 3 * w.numel() + 2 * b.numel())   # fwd: x, out; bwd: gout, x, gx; w, gw, b, gb
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    line = {
+        "metric": "plain depthwise conv3d fwd+bwd GB/s (dwconv) on 1 GPU", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "dwconv: depthwise conv3d fwd+bwd, N=2, C=256, 8x56x56, k3 s1 p1, bias, fp32",
+                   "forward_ms": round(ms_f, 4), "backward_ms": round(ms_b, 4),
+                   "torch_grouped_conv_ms_per_step": round(ms_torch, 4), "max_error_vs_torch": err,
+                   "algorithmic_mbytes": round(nbytes / 1e6, 1)},
+        "roofline": {"bound": "hbm", "kernel": "dwc_fwd_kernel + dwc_bwd_input_kernel + dwc_bwd_weight_kernel",
+                     "achieved": round(gbs, 1), "peak": PEAK_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_GBS, 4),
+                     "traffic": None},
+    }
+    if not args.no_cpu:
+        from oracle import dwconv
+        cx, cw, cb, cg = x[:1, :32].numpy(), w[:32].numpy(), b[:32].numpy(), gout[:1, :32].numpy()
+        t0 = time.perf_counter()
+        dwconv.forward(cx, cw, cb, (1, 1, 1), (1, 1, 1), (1, 1, 1))
+        dwconv.backward(cg, cx, cw, (1, 1, 1), (1, 1, 1), (1, 1, 1))
+        dt = time.perf_counter() - t0
+        line["cpu_baseline"] = {"value": round(nbytes / 16 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                                "sample": f"1 of 2 samples, 32 of 256 channels (1/16 of the workload), numpy float64: {dt:.2f} s"}
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -210,6 +298,8 @@ def main():
         sys.exit("bench.py: no GPU visible")
     if args.workload == "c2_sizemap":
         return bench_size_map(args)
+    if args.workload == "dwconv":
+        return bench_dwconv(args)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
@@ -253,6 +343,13 @@ def main():
         forward()
         if c["backward"]:
             backward()
+
+    taps = None
+    if nd == 3:
+        # how much of the offset field leaves the volume (outside the timed region)
+        from d2conv3d_amd.util import tap_statistics
+        st = tap_statistics((N, C, *dims), off, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), G)
+        taps = {k: round(st[k], 4) for k in ("dead", "partial", "corners_read")}
 
     for _ in range(args.warmup):
         step()
@@ -370,6 +467,7 @@ def main():
                                + ("bf16 in / fp32 accumulate" if dt == "bf16" else "fp32"),
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
+                   "taps_outside_volume": taps,
                    "algorithmic_gflop": round(nflops / 1e9, 2),
                    "algorithmic_mbytes": round((b_fwd + (b_bwd if c["backward"] else 0)) / 1e6, 1),
                    "frac_of_mfma_peak_whole_step": round(value / PEAK_TFLOPS[dt], 4),

@@ -14,6 +14,7 @@ from .modules import (
 )
 from .grid import offsets_from_size_map
 from .util import add_deformable_conv
+from .depthwise_conv import DepthwiseConv3d, depthwise_separable_conv3d, install_as_fast_depthwise_conv3d
 
 __all__ = [
     "deform_conv1d", "deform_conv3d", "DeformConv1d", "DeformConv3d", "DeformConvNd",
@@ -23,6 +24,7 @@ __all__ = [
     "XXZSizeConditionedDConv3d", "XXZSizeConditionedMDConv3d",
     "XYZSizeConditionedDConv3d", "XYZSizeConditionedMDConv3d",
     "offsets_from_size_map", "add_deformable_conv", "install_as_dconv_native",
+    "DepthwiseConv3d", "depthwise_separable_conv3d", "install_as_fast_depthwise_conv3d",
 ]
 
 

@@ -25,6 +25,7 @@ EXPORTS = (
     "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_last_error", "d2c_version",
     "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read",
     "d2c_size_map_offsets_forward", "d2c_size_map_offsets_backward",
+    "d2c_dwconv3d_check", "d2c_dwconv3d_backward_workspace_bytes", "d2c_dwconv3d_forward", "d2c_dwconv3d_backward",
 )
 
 
@@ -43,6 +44,12 @@ SIZE_ACTIVATIONS = {"linear": 0, "elu": 1, "relu": 2, "relu_plus_one": 3}
 class SizeMapDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("N", "P", "kd", "kh", "kw", "mode", "activation", "dtype")] + [
         (n, ctypes.c_float * SIZE_MAX_K) for n in ("base_z", "base_y", "base_x")]
+
+
+class DwConv3dDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "N", "C", "Cout", "D", "H", "W", "kd", "kh", "kw", "sd", "sh", "sw",
+        "pd", "ph", "pw", "dd", "dh", "dw", "Do", "Ho", "Wo", "dtype")]
 
 
 class Conv1dDesc(ctypes.Structure):
@@ -93,6 +100,12 @@ def load():
     psm = ctypes.POINTER(SizeMapDesc)
     lib.d2c_size_map_offsets_forward.argtypes, lib.d2c_size_map_offsets_forward.restype = [psm, vp, vp, vp], ctypes.c_int
     lib.d2c_size_map_offsets_backward.argtypes, lib.d2c_size_map_offsets_backward.restype = [psm, vp, vp, vp, vp], ctypes.c_int
+    pdw = ctypes.POINTER(DwConv3dDesc)
+    lib.d2c_dwconv3d_check.argtypes, lib.d2c_dwconv3d_check.restype = [pdw], ctypes.c_int
+    lib.d2c_dwconv3d_backward_workspace_bytes.argtypes = [pdw]
+    lib.d2c_dwconv3d_backward_workspace_bytes.restype = sz
+    lib.d2c_dwconv3d_forward.argtypes, lib.d2c_dwconv3d_forward.restype = [pdw] + [vp] * 5, ctypes.c_int
+    lib.d2c_dwconv3d_backward.argtypes, lib.d2c_dwconv3d_backward.restype = [pdw] + [vp] * 7 + [sz, vp], ctypes.c_int
     lib.d2c_profile_enable.argtypes, lib.d2c_profile_enable.restype = [ctypes.c_int], None
     lib.d2c_profile_reset.argtypes, lib.d2c_profile_reset.restype = [], None
     lib.d2c_profile_read.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]

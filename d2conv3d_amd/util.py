@@ -69,3 +69,27 @@ def dconv_replace_layer(conv_module, **kwargs):
 def add_deformable_conv(module, **kwargs):
     """util.py:62-63."""
     return replace_module(dconv_replace_layer, nn.Conv3d, module, **kwargs)
+
+
+def tap_statistics(input_shape, offset, kernel_size, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
+                   offset_groups=1):
+    """How much of an offset field samples outside the volume: the debug output the reference's trainer expects
+    from a `tools.hooks.oob_tracking` hook that its repository does not contain (trainer.py:99-101).
+
+    Counts come from the sampler's own bookkeeping (the set of corners the forward pass reads per tap,
+    dconv3d_gpu.cu:59-86), so they are exact for the kernel that runs.  Returns a dict:
+      taps            number of (sample, offset group, tap, position) sampling points
+      dead            fraction whose value is 0 by the early-out (no corner read)
+      partial         fraction read with at least one corner outside the volume
+      corners_read    fraction of all 8 * taps corner values that are read
+    """
+    import torch
+    from . import _ops
+    _, flags = _ops.conv3d_corner_index(tuple(input_shape), offset, tuple(kernel_size), tuple(stride), tuple(padding),
+                                        tuple(dilation), offset_groups)
+    n = flags.numel()
+    f = flags.to(torch.int32)
+    dead = int((f == 0).sum())
+    full = int((f == 255).sum())
+    bits = sum(((f >> c) & 1).sum() for c in range(8))
+    return {"taps": n, "dead": dead / n, "partial": (n - dead - full) / n, "corners_read": int(bits) / (8.0 * n)}

@@ -185,6 +185,34 @@ int d2c_size_map_offsets_forward(const d2c_size_map_desc *desc, const void *size
 int d2c_size_map_offsets_backward(const d2c_size_map_desc *desc, const void *size_raw, const void *grad_offsets,
                                   void *grad_size_raw, void *stream);
 
+/* ---- plain depthwise conv3d (no sampling) ------------------------------------------------
+ * The operator of the reference's second extension, ops/fast-depthwise-conv3d, which its
+ * backbone uses for the channel-separated 3x3x3 convolutions (network/backbone/resnet.py:110):
+ *   d2c_dwconv3d_forward   <- conv_depthwise3d_cuda           (csrc/grouped_conv3d.cu:22-92, 385-470)
+ *   d2c_dwconv3d_backward  <- conv_depthwise3d_backward_cuda  (csrc/grouped_conv3d.cu:93-276, 510-665)
+ *   d2c_dwconv3d_check     <- conv_depthwise_shape_check      (csrc/grouped_conv3d.cu:279-345)
+ * x [N,C,D,H,W], weight [Cout,1,kd,kh,kw] with Cout a multiple of C (output channel co reads
+ * input channel co / (Cout/C)), bias [Cout] or NULL, out [N,Cout,Do,Ho,Wo]; all in `dtype`
+ * (float32, float64 or bfloat16; sums in float32, float64 for float64).  In the backward call
+ * a NULL gradient pointer skips that gradient; grad_weight and grad_bias need the workspace. */
+typedef struct d2c_dwconv3d_desc {
+    int32_t N, C, Cout;
+    int32_t D, H, W;
+    int32_t kd, kh, kw;
+    int32_t sd, sh, sw;
+    int32_t pd, ph, pw;
+    int32_t dd, dh, dw;
+    int32_t Do, Ho, Wo;       /* must equal (in + 2p - (d(k-1)+1))/s + 1 */
+    int32_t dtype;
+} d2c_dwconv3d_desc;
+int d2c_dwconv3d_check(const d2c_dwconv3d_desc *desc);
+size_t d2c_dwconv3d_backward_workspace_bytes(const d2c_dwconv3d_desc *desc);
+int d2c_dwconv3d_forward(const d2c_dwconv3d_desc *desc, const void *x, const void *weight, const void *bias,
+                         void *out, void *stream);
+int d2c_dwconv3d_backward(const d2c_dwconv3d_desc *desc, const void *grad_out, const void *x, const void *weight,
+                          void *grad_x, void *grad_weight, void *grad_bias, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
 /* Test hook for the matrix-core backward pass: 1 (default) builds grad_input from
  * per-voxel sample lists, every element written once; 0 scatters with fp32 atomics
  * like the reference (dconv3d_gpu.cu:637).  A value n >= 2 is mode 1 with lists

@@ -111,3 +111,37 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.load()
+
+
+def test_plain_depthwise_boundary_without_gpu():
+    """d2c_dwconv3d_check mirrors conv_depthwise_shape_check (grouped_conv3d.cu:279-345); the Python surface
+    carries the reference's names (src/fast_depthwise_conv3d/__init__.py, conv.py:7-22) and rejects CPU tensors."""
+    import ctypes
+    lib = _lib.load()
+
+    def desc(**kw):
+        f = dict(N=2, C=4, Cout=8, D=6, H=7, W=8, kd=3, kh=3, kw=3, sd=1, sh=1, sw=1, pd=1, ph=1, pw=1, dd=1, dh=1, dw=1,
+                 Do=6, Ho=7, Wo=8, dtype=_lib.D2C_F32)
+        f.update(kw)
+        return _lib.DwConv3dDesc(*(f[n] for n, _ in _lib.DwConv3dDesc._fields_))
+
+    assert lib.d2c_dwconv3d_check(ctypes.byref(desc())) == 0
+    assert lib.d2c_dwconv3d_backward_workspace_bytes(ctypes.byref(desc())) >= 8 * 28 * 4
+    for bad, text in ((dict(Cout=6), "multiple of in channels"), (dict(sd=0), "stride should be at least 1"),
+                      (dict(pw=-1), "padding should be non-negative"), (dict(dh=0), "dilation should be at least 1"),
+                      (dict(D=2, pd=0, Do=0), "Output size should be positive"), (dict(Wo=9), "does not match"),
+                      (dict(dtype=7), "dtype")):
+        assert lib.d2c_dwconv3d_check(ctypes.byref(desc(**bad))) != 0
+        assert text in _lib.last_error()
+    assert lib.d2c_dwconv3d_backward_workspace_bytes(ctypes.byref(desc(Cout=6))) == 0
+
+    m = d2c.DepthwiseConv3d(4, 8, kernel_size=3, padding=1, groups=99)
+    assert isinstance(m, torch.nn.Conv3d) and m.groups == 4 and tuple(m.weight.shape) == (8, 1, 3, 3, 3)
+    with pytest.raises(RuntimeError, match="GPU"):
+        m(torch.randn(1, 4, 5, 5, 5))
+    with pytest.raises(RuntimeError, match="in_channels=1"):
+        d2c.depthwise_separable_conv3d(torch.randn(1, 4, 5, 5, 5), torch.randn(4, 2, 3, 3, 3), None, 1, 1, 1)
+    d2c.install_as_fast_depthwise_conv3d()
+    from fast_depthwise_conv3d import DepthwiseConv3d  # noqa: F401
+    import fast_depthwise_conv3d._ops as ops
+    assert callable(ops.depthwise_separable_conv3d)

@@ -135,3 +135,21 @@ def test_size_map_offsets_reject_bad_arguments(dev):
         size_map_offsets(torch.zeros(1, 2, 2, 2, 2, device=dev), "xyz")           # wrong channel count
     with pytest.raises(RuntimeError):
         size_map_offsets(torch.zeros(1, 3, 2, 2, 2, device=dev, dtype=torch.float64), "xyz")
+
+
+def test_tap_statistics_match_the_oracle(dev):
+    """Out-of-volume telemetry: the counts are those of the oracle's corner sets on the same offsets."""
+    from d2conv3d_amd.util import tap_statistics
+    from oracle import cpu
+    g = torch.Generator().manual_seed(11)
+    xshape, ks, stride, padding, dilation, G = (2, 8, 5, 9, 7), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 2
+    off = torch.randn(2, G * 81, 5, 9, 7, generator=g) * 2.0
+    _, ef = cpu.conv3d_corners(xshape, off, (8, 8) + ks, stride, padding, dilation, G)
+    ef = ef.to(torch.int32)
+    st = tap_statistics(xshape, off.to(dev), ks, stride, padding, dilation, G)
+    n = ef.numel()
+    assert st["taps"] == n
+    assert st["dead"] == int((ef == 0).sum()) / n
+    assert st["partial"] == int(((ef != 0) & (ef != 255)).sum()) / n
+    assert st["corners_read"] == sum(int(((ef >> c) & 1).sum()) for c in range(8)) / (8.0 * n)
+    assert 0.05 < st["dead"] < 0.6 and st["partial"] > 0.05     # the case does leave the volume

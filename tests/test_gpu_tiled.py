@@ -28,6 +28,7 @@ SHAPES = {
     # wide weight groups with many position tiles: the forward kernel that moves corner rows by DMA
     "c64_o320_big": (1, 64, 320, (7, 35, 34), 3, 1, 1, 1, 1, 1, True, True, 1.5),       # N*P = 8330: ragged
     "c128_groups2_o640_big": (1, 128, 640, (4, 32, 33), 3, 1, 1, 1, 2, 2, True, True, 2.0),
+    "c64_o200_big": (1, 64, 200, (7, 35, 34), 3, 1, 1, 1, 1, 1, True, True, 1.5),       # 256-wide output tile
     # the same kernel's schedule: three output tiles per position tile (399 work items on 256 compute units: one
     # whole round, the rest cut into step ranges), two weight groups with few position tiles (all items cut)
     "c64_o1100_big": (1, 64, 1100, (7, 35, 35), 3, 1, 1, 1, 1, 1, True, True, 1.5),

@@ -340,3 +340,36 @@ def test_1d_integer_position_rule():
     _, goff, gm, _, _ = cpu.conv1d_backward(gout, x, off, a, w, False, quirks=False)
     assert close(goff[0, 0], 0.5 * (xp[2:] - xp[1:-1]))
     assert close(gm[0, 0], x[0, 0])
+
+
+# ---------------------------------------------------------------- plain depthwise conv3d (oracle/dwconv.py)
+DW_CASES = [
+    # C, multiplier, kernel, stride, padding, dilation
+    (3, 1, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    (2, 2, (3, 3, 3), (2, 2, 2), (2, 2, 2), (2, 2, 2)),
+    (4, 3, (1, 3, 2), (1, 2, 1), (0, 1, 2), (1, 1, 2)),
+    (2, 1, (3, 3, 3), (2, 1, 2), (1, 1, 1), (1, 2, 1)),
+]
+
+
+@pytest.mark.parametrize("C,m,k,s,p,d", DW_CASES)
+def test_plain_depthwise_oracle_is_torch_grouped_conv(C, m, k, s, p, d):
+    """The library routine the reference's own test compares with (test_conv3d_depthwise.py:33-96): torch's grouped
+    convolution and its autograd, float64 on the CPU."""
+    from oracle import dwconv
+    g = torch.Generator().manual_seed(C * 7 + m)
+    x = torch.randn(2, C, 6, 7, 8, dtype=torch.float64, generator=g).requires_grad_(True)
+    w = torch.randn(C * m, 1, *k, dtype=torch.float64, generator=g).requires_grad_(True)
+    b = torch.randn(C * m, dtype=torch.float64, generator=g).requires_grad_(True)
+    out = F.conv3d(x, w, b, s, p, d, groups=C)
+    go = torch.randn(out.shape, dtype=torch.float64, generator=g)
+    out.backward(go)
+    eo = dwconv.forward(x.detach().numpy(), w.detach().numpy(), b.detach().numpy(), s, p, d)
+    gx, gw, gb = dwconv.backward(go.numpy(), x.detach().numpy(), w.detach().numpy(), s, p, d)
+    np.testing.assert_allclose(eo, out.detach().numpy(), rtol=0, atol=1e-12)
+    np.testing.assert_allclose(gx, x.grad.numpy(), rtol=0, atol=1e-12)
+    np.testing.assert_allclose(gw, w.grad.numpy(), rtol=0, atol=1e-12)
+    np.testing.assert_allclose(gb, b.grad.numpy(), rtol=0, atol=1e-12)
+    # without bias the forward value drops exactly the bias
+    np.testing.assert_allclose(dwconv.forward(x.detach().numpy(), w.detach().numpy(), None, s, p, d),
+                               F.conv3d(x, w, None, s, p, d, groups=C).detach().numpy(), rtol=0, atol=1e-12)
