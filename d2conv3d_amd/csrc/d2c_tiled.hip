@@ -109,6 +109,38 @@ __global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int
     }
 }
 
+// The same for bfloat16 with 16-byte accesses on both sides (2-byte accesses of 32 lanes move 64 bytes per
+// request): 64 x 64 element tiles; needs vol and C to be multiples of 8 and 16-byte aligned tensors.
+__global__ void __launch_bounds__(256) pack_input_bf16_kernel(const bf16_t *x, bf16_t *xcl, int C, int vol)
+{
+    constexpr int RS = 66;                             // LDS row stride in elements (33 words)
+    __shared__ bf16_t tile[64 * RS];                   // [v][c]
+    const int b = blockIdx.z, v0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+    const bf16_t *xb = x + (long)b * C * vol;
+    bf16_t *ob = xcl + (long)b * C * vol;
+    for (int i = threadIdx.x; i < 512; i += 256) {     // 64 channels x 8 vectors of 8 positions
+        const int c = c0 + i / 8, v = v0 + (i % 8) * 8;
+        if (c < C && v < vol) {                        // (vol % 8 == 0: the vector is inside or outside as a whole)
+            const uint4 q = *reinterpret_cast<const uint4 *>(xb + (long)c * vol + v);
+            const unsigned u[4] = {q.x, q.y, q.z, q.w};
+            bf16_t *t = tile + ((i % 8) * 8) * RS + i / 8;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                t[(2 * e) * RS] = (bf16_t)(u[e] & 0xffffu);
+                t[(2 * e + 1) * RS] = (bf16_t)(u[e] >> 16);
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 512; i += 256) {     // 64 positions x 8 vectors of 8 channels
+        const int v = v0 + i / 8, c = c0 + (i % 8) * 8;
+        if (c < C && v < vol) {
+            const unsigned *t = reinterpret_cast<const unsigned *>(tile + (i / 8) * RS + (i % 8) * 8);
+            *reinterpret_cast<uint4 *>(ob + (long)v * C + c) = make_uint4(t[0], t[1], t[2], t[3]);
+        }
+    }
+}
+
 // Forward weight operand in MFMA fragment order:
 //   wp[wg][step = chunk*K + k][o-block of 32][k-group][lane] = 16 bytes =
 //   W[wg*og + ob*32 + lane%32][chunk*BKC + (2*kg + lane/32)*VEC + 0..VEC-1][k]
@@ -201,6 +233,14 @@ int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st)
 {
     dim3 grid((s.vol + 31) / 32, (s.Cin + 31) / 32, s.N);
     D2cProfScope prof(D2C_PROF_PACK, st);
+    if constexpr (sizeof(T) == 2) {
+        if (s.vol % 8 == 0 && s.Cin % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+            reinterpret_cast<uintptr_t>(xcl) % 16 == 0) {
+            hipLaunchKernelGGL(pack_input_bf16_kernel, dim3((s.vol + 63) / 64, (s.Cin + 63) / 64, s.N), dim3(256), 0, st,
+                               (const bf16_t *)x, (bf16_t *)xcl, s.Cin, s.vol);
+            return d2c_check_launch("pack_input_bf16_kernel");
+        }
+    }
     hipLaunchKernelGGL(pack_input_kernel<T>, grid, dim3(256), 0, st, (const T *)x, (T *)xcl, s.Cin, s.vol);
     return d2c_check_launch("pack_input_kernel");
 }

@@ -758,6 +758,33 @@ __global__ void __launch_bounds__(256) unpack_grad_input_kernel(const float *gxc
     }
 }
 
+// The same for bfloat16 with 16-byte accesses on both sides: 64 x 64 element tiles; needs vol and C to be
+// multiples of 8 and a 16-byte aligned grad_input.
+__global__ void __launch_bounds__(256) unpack_grad_input_bf16_kernel(const float *gxcl, bf16_t *gx, int C, int vol)
+{
+    constexpr int RS = 66;                             // LDS row stride in elements (33 words)
+    __shared__ bf16_t tile[64 * RS];                   // [c][v]
+    const int b = blockIdx.z, v0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+    const float *ib = gxcl + (long)b * C * vol;
+    bf16_t *ob = gx + (long)b * C * vol;
+    for (int i = threadIdx.x; i < 1024; i += 256) {    // 64 positions x 16 vectors of 4 channels
+        const int v = v0 + i / 16, c = c0 + (i % 16) * 4;
+        if (c < C && v < vol) {
+            const float4 q = *reinterpret_cast<const float4 *>(ib + (long)v * C + c);
+            bf16_t *t = tile + ((i % 16) * 4) * RS + i / 16;
+            t[0] = f32_to_bf16(q.x); t[RS] = f32_to_bf16(q.y); t[2 * RS] = f32_to_bf16(q.z); t[3 * RS] = f32_to_bf16(q.w);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 512; i += 256) {     // 64 channels x 8 vectors of 8 positions
+        const int c = c0 + i / 8, v = v0 + (i % 8) * 8;
+        if (c < C && v < vol) {
+            const unsigned *t = reinterpret_cast<const unsigned *>(tile + (i / 8) * RS + (i % 8) * 8);
+            *reinterpret_cast<uint4 *>(ob + (long)c * vol + v) = make_uint4(t[0], t[1], t[2], t[3]);
+        }
+    }
+}
+
 // fp32 accumulator [group][chunk*K + tap][og][BKC] -> grad_weight [Cout][cg][K] of type T
 template <typename T>
 __global__ void __launch_bounds__(256) cvt_grad_weight_kernel(const float *src, T *dst, TiledShape s, long n)
@@ -1082,6 +1109,13 @@ int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStr
 {
     dim3 grid((s.vol + 31) / 32, (s.Cin + 31) / 32, s.N);
     D2cProfScope prof(D2C_PROF_PACK, st);
+    if constexpr (sizeof(T) == 2) {
+        if (s.vol % 8 == 0 && s.Cin % 8 == 0 && reinterpret_cast<uintptr_t>(gx) % 16 == 0) {
+            hipLaunchKernelGGL(unpack_grad_input_bf16_kernel, dim3((s.vol + 63) / 64, (s.Cin + 63) / 64, s.N), dim3(256), 0,
+                               st, gxcl, (bf16_t *)gx, s.Cin, s.vol);
+            return d2c_check_launch("unpack_grad_input_bf16_kernel");
+        }
+    }
     hipLaunchKernelGGL(unpack_grad_input_kernel<T>, grid, dim3(256), 0, st, gxcl, (T *)gx, s.Cin, s.vol);
     return d2c_check_launch("unpack_grad_input_kernel");
 }

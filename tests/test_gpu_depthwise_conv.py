@@ -154,3 +154,30 @@ def test_unaligned_tensors_take_the_scalar_kernels(dev):
     a = depthwise_separable_conv3d(x, w, None, 1, 1, 1)
     b = depthwise_separable_conv3d(x.clone(), w, None, 1, 1, 1)
     assert x.data_ptr() % 16 != 0 and torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_full_size_against_torch_grouped_conv(dtype, dev):
+    """The workload bench.py times (N=2, C=256, 8x56x56, 3^3, padding 1): too large for the numpy oracle, so the
+    reference's own check is used, torch's grouped convolution and its autograd on the same tensors (float32
+    arithmetic on bfloat16-rounded values for the bfloat16 case), plus grad_bias = sum of grad_out."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(1006)
+    N, C, dims = 2, 256, (8, 56, 56)
+    x = torch.randn(N, C, *dims, generator=g).to(dtype).to(dev)
+    w = ((torch.rand(C, 1, 3, 3, 3, generator=g) * 2 - 1) / 27 ** 0.5).to(dtype).to(dev)
+    b = ((torch.rand(C, generator=g) * 2 - 1) / 27 ** 0.5).to(dtype).to(dev)
+    go = torch.randn(N, C, *dims, generator=g).to(dtype).to(dev)
+    xs, ws, bs = (t.clone().requires_grad_(True) for t in (x, w, b))
+    out = depthwise_separable_conv3d(xs, ws, bs, 1, 1, 1)
+    out.backward(go)
+    xr, wr, br = (t.float().clone().requires_grad_(True) for t in (x, w, b))
+    ref = F.conv3d(xr, wr, br, 1, 1, 1, groups=C)
+    ref.backward(go.float())
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+
+    def rel(a, e):
+        return float((a.float() - e).abs().max() / e.abs().max())
+
+    assert rel(out, ref) < tol and rel(xs.grad, xr.grad) < tol and rel(ws.grad, wr.grad) < tol and rel(bs.grad, br.grad) < tol
+    assert rel(bs.grad, go.float().sum(dim=(0, 2, 3, 4))) < tol
