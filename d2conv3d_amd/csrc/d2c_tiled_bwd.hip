@@ -840,7 +840,8 @@ __global__ void __launch_bounds__(256) cvt_grad_weight_lds_kernel(const float *s
 //   gout[wg*og + block*32 + lane%32][positions tile*kWMT + (2*kgroup + lane/32)*VEC + 0..VEC-1]
 // with positions numbered over the whole batch (m = b*P + p); rows past og and positions past N*P are zero.
 template <typename T>
-__global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp, TiledShape s, int ntile, int OBT, long total)
+__global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp, TiledShape s, int ntile, int OBT, long total,
+                                                        bool vec)
 {
     constexpr int VEC = Elem<T>::VEC, NKGT = kWMT / (2 * VEC);
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
@@ -852,7 +853,17 @@ __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp,
         const int wg = (int)(r / ntile);
         const int ol = ob * 32 + (lane & 31);
         const long m0 = (long)tile * kWMT + (2 * kg + (lane >> 5)) * VEC;
-        T e[VEC];
+        alignas(16) T e[VEC];
+        if (vec) {
+            // P is a multiple of VEC: the VEC positions lie in one sample and are one aligned 16-byte piece of the row
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (ol < s.og && m0 < s.M) {
+                const int b = (int)(m0 / s.P), p = (int)(m0 - (long)b * s.P);
+                v = *reinterpret_cast<const uint4 *>(gout + ((long)b * s.Cout + wg * s.og + ol) * s.P + p);
+            }
+            reinterpret_cast<uint4 *>(goutp)[i] = v;
+            continue;
+        }
 #pragma unroll
         for (int q = 0; q < VEC; q++) {
             const long m = m0 + q;
@@ -1050,8 +1061,9 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         d2c_fill_zero((char *)const_cast<void *>(xcl) + (size_t)s.N * s.vol * s.Cin * sizeof(T), 256, st);
         const int OBT = (s.og + 63) / 64 * 2;
         const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
+        const bool vec = s.P % Elem<T>::VEC == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0;
         hipLaunchKernelGGL(pack_gout_kernel<T>, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const T *)gout, (T *)goutp, s,
-                           ntp, OBT, total);
+                           ntp, OBT, total, vec);
         if (int rc = d2c_check_launch("pack_gout_kernel")) return rc;
     }
     // Position tiles of a step are dealt to `split` workgroups; one workgroup runs per compute unit at a time.

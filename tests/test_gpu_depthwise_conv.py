@@ -177,7 +177,7 @@ def test_full_size_against_torch_grouped_conv(dtype, dev):
     tol = 1e-5 if dtype == torch.float32 else 2e-2
 
     def rel(a, e):
-        return float((a.float() - e).abs().max() / e.abs().max())
+        return float((a.detach().float() - e.detach()).abs().max() / e.detach().abs().max())
 
     assert rel(out, ref) < tol and rel(xs.grad, xr.grad) < tol and rel(ws.grad, wr.grad) < tol and rel(bs.grad, br.grad) < tol
     assert rel(bs.grad, go.float().sum(dim=(0, 2, 3, 4))) < tol
