@@ -267,3 +267,57 @@ def test_tiled_conv1d_integer_positions(quirks, dev):
     out.backward(gout.to(dev))
     for n, t, e in zip(("grad_input", "grad_offset", "grad_mask", "grad_weight"), ts, eg):
         assert_close(t.grad, e, 1e-4, 1e-5 * max(1.0, e.abs().max().item()), f"{n} quirks={quirks}")
+
+
+def _random_case(rng, depthwise):
+    """A random geometry that the matrix-core (or channel-separated) kernels accept."""
+    pick = lambda *v: v[int(rng.integers(len(v)))]
+    k = (pick(1, 3), pick(1, 3), pick(2, 3))
+    s = (pick(1, 2), pick(1, 1, 2), pick(1, 1, 2))
+    d = (pick(1, 2), pick(1, 1, 2), pick(1, 2))
+    p = tuple(int(rng.integers(0, 3)) for _ in range(3))
+    dims = tuple(int(rng.integers(dd * (kk - 1) + 1 + 1, dd * (kk - 1) + 1 + 9)) for kk, dd in zip(k, d))
+    N = pick(1, 2, 3)
+    if depthwise:
+        G = pick(1, 2, 4)
+        C = G * 4 * int(rng.integers(1, 70))
+        return N, C, C, dims, k, s, p, d, C, G, bool(rng.integers(2)), bool(rng.integers(2)), float(pick(0.5, 1.5, 3.0))
+    groups = pick(1, 1, 2)
+    G = groups * pick(1, 2)
+    Cin = 64 * G * pick(1, 2) if groups == 1 else 64 * G
+    Cout = groups * int(rng.integers(1, 300))
+    return N, Cin, Cout, dims, k, s, p, d, groups, G, bool(rng.integers(2)), bool(rng.integers(2)), float(pick(0.5, 1.5, 3.0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("depthwise", [False, True])
+def test_random_geometries_against_the_direct_kernels(depthwise, dtype, dev):
+    """Seeded random shapes, strides, paddings, dilations, groups and offset scales: the matrix-core / channel-separated
+    kernels against the direct kernels (one thread per element, checked against the oracle on the reference's test
+    matrix in test_gpu_reference_matrix.py) on the same tensors, forward and all gradients."""
+    import numpy as np
+    rng = np.random.default_rng(20240 + int(depthwise))
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    for case in range(10):
+        shape = _random_case(rng, depthwise)
+        SHAPES["_random"] = shape
+        try:
+            (x, off, m, w, b), gout, (s, p, d, groups, G) = make("_random", dtype, seed=100 + case)
+        finally:
+            del SHAPES["_random"]
+        res = []
+        for family in (None, "generic"):
+            ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+            _ops.set_algo_override(family)
+            try:
+                if family is None:
+                    assert _ops.conv3d_algo(ts[0], ts[1], ts[2], ts[3], s, p, d, groups, G) == \
+                        ("depthwise" if depthwise else "mfma"), shape
+                out = d2c.deform_conv3d(*ts, s, p, d, groups, G)
+                out.backward(gout.to(dev))
+            finally:
+                _ops.set_algo_override(None)
+            res.append([out.detach().float()] + [t.grad.float() for t in ts if t is not None])
+        for a, e in zip(*res):
+            scale = max(1.0, e.abs().max().item())
+            assert (a - e).abs().max().item() <= tol * scale, (shape, (a - e).abs().max().item(), scale)
