@@ -154,8 +154,8 @@ __global__ void set_total(const int *counts, int *starts, int n)
 // a in {0, 1} with weight:  r = 0: (h, -),  r = 1: (1 - h, h),  r = 2: (-, 1 - h).
 // z and y offsets are compile-time (9 unrolled visits); the 3 base voxels along x are adjacent bins, one
 // contiguous range of entries, the x offset of an entry follows from its place in the range.
-template <typename T>
-__global__ void __launch_bounds__(256)
+template <typename T, bool COMPACT>
+__global__ void __launch_bounds__(256, 4)   // registers for 4 wavefronts per SIMD
 gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
@@ -191,27 +191,30 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
             const int em1 = min(L.counts[bin1], L.cap);
             const int em2 = em1 + min(L.counts[bin1 + 1], L.cap);
             const int e1 = em2 + (nxb == 3 ? min(L.counts[bin1 + 2], L.cap) : 0);
-            const InvEntry *eb = L.entries + (long)bin1 * L.cap;
+            const uint4 *eb = reinterpret_cast<const uint4 *>(L.entries) + (long)bin1 * L.cap * (COMPACT ? 1 : 2);
             for (int e = 0; e < e1; e += 4) {
-                uint4 q0[4], q1[4], row[4];
+                InvEntry en[4];
+                uint4 row[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int ei = min(e + i, e1 - 1);
                     const int slot = ei < em1 ? ei : (ei < em2 ? ei - em1 + L.cap : ei - em2 + 2 * L.cap);
-                    q0[i] = reinterpret_cast<const uint4 *>(eb + slot)[0];
-                    q1[i] = reinterpret_cast<const uint4 *>(eb + slot)[1];
+                    if constexpr (COMPACT) {
+                        en[i] = unpack_entry(eb[slot]);
+                    } else {
+                        const uint4 q0 = eb[2 * slot], q1 = eb[2 * slot + 1];
+                        en[i].p = (int)q0.x; en[i].k = (int)q0.y;
+                        en[i].hz = __uint_as_float(q0.z); en[i].hy = __uint_as_float(q0.w);
+                        en[i].hx = __uint_as_float(q1.x); en[i].alpha = __uint_as_float(q1.y);
+                    }
                 }
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int p = (int)q0[i].x, k = (int)q0[i].y;
-                    row[i] = *reinterpret_cast<const uint4 *>(gbase + ((long)k * s.M + p) * BKC);
-                }
+                for (int i = 0; i < 4; i++)
+                    row[i] = *reinterpret_cast<const uint4 *>(gbase + ((long)en[i].k * s.M + en[i].p) * BKC);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const float hz = __uint_as_float(q0[i].z), hy = __uint_as_float(q0[i].w);
-                    const float hx = __uint_as_float(q1[i].x);
-                    float al = __uint_as_float(q1[i].y);
-                    al = e + i < e1 ? al : 0.f;
+                    const float hz = en[i].hz, hy = en[i].hy, hx = en[i].hx;
+                    const float al = e + i < e1 ? en[i].alpha : 0.f;
                     // x: offset 0 (base x0-1) reaches voxel c=0 with hx; 1 reaches (1-hx, hx); 2 reaches c=1 with 1-hx
                     const bool r0 = e + i < em1, r2 = e + i >= em2;
                     const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
@@ -489,11 +492,13 @@ int d2c_lists_cap(const TiledShape &s)
     while (cap < 256 && cap < 2.2 * mean) cap *= 2;
     return cap;
 }
-void d2c_lists_ws(const TiledShape &s, size_t *counts, size_t *entries, size_t *ovf)
+// 16-byte bucket entries: bfloat16 problems whose position and tap fit 24 + 8 bits
+bool d2c_lists_compact(const TiledShape &s, int dtype) { return dtype == D2C_BF16 && s.P < (1 << 24) && s.K < 256; }
+void d2c_lists_ws(const TiledShape &s, int dtype, size_t *counts, size_t *entries, size_t *ovf)
 {
     const long nb = d2c_invlist_bins(s);
     *counts = d2c_align_up((size_t)(nb + 1) * 4);
-    *entries = d2c_align_up((size_t)nb * d2c_lists_cap(s) * sizeof(InvEntry));
+    *entries = d2c_align_up((size_t)nb * d2c_lists_cap(s) * (d2c_lists_compact(s, dtype) ? 16 : sizeof(InvEntry)));
     *ovf = d2c_align_up((size_t)s.N * s.G * s.K * s.P * sizeof(InvEntry));
 }
 // Bins and samples are counted in 32 bits; larger problems take the atomic scatter instead.
@@ -502,10 +507,11 @@ bool d2c_lists_supported(const TiledShape &s)
     return d2c_invlist_bins(s) < (1L << 31) - 1 && (long)s.N * s.G * s.K * s.P < (1L << 31);
 }
 // The lists over the three workspace regions sized by d2c_lists_ws; nbins == 0 when the shape is too large.
-SampleLists d2c_lists_make(const TiledShape &s, void *counts, void *entries, void *ovf)
+SampleLists d2c_lists_make(const TiledShape &s, int dtype, void *counts, void *entries, void *ovf)
 {
     const long nb = d2c_invlist_bins(s), nsamp = (long)s.N * s.G * s.K * s.P;
-    SampleLists L{(int *)counts, (InvEntry *)entries, (InvEntry *)ovf, d2c_lists_cap(s), 0, 0};
+    SampleLists L{(int *)counts, (InvEntry *)entries, (InvEntry *)ovf, d2c_lists_cap(s), 0, 0,
+                  d2c_lists_compact(s, dtype) ? 1 : 0};
     if (nb < (1L << 31) - 1 && nsamp < (1L << 31)) {
         L.nbins = (int)nb;
         L.ovf_cap = (int)nsamp;
@@ -539,7 +545,8 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
     dim3 grid((unsigned)nblk, s.Cin / BKC);
-    hipLaunchKernelGGL(gx_owner_cube_kernel<T>, grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
     if (int rc = d2c_check_launch("gx_owner_kernel")) return rc;
     // the overflow entries, usually none (the kernel reads their number from device memory)
     hipLaunchKernelGGL(gx_overflow_kernel<T>, dim3(512), dim3(256), 0, st, s, (const T *)gcol, L, gxcl);

@@ -25,8 +25,8 @@ int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, in
                       void *entries, hipStream_t st);
 template <typename T>
 int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st);
-void d2c_lists_ws(const TiledShape &s, size_t *counts, size_t *entries, size_t *ovf);
-SampleLists d2c_lists_make(const TiledShape &s, void *counts, void *entries, void *ovf);
+void d2c_lists_ws(const TiledShape &s, int dtype, size_t *counts, size_t *entries, size_t *ovf);
+SampleLists d2c_lists_make(const TiledShape &s, int dtype, void *counts, void *entries, void *ovf);
 int d2c_lists_clear(const SampleLists &L, hipStream_t st);
 bool d2c_lists_supported(const TiledShape &s);
 int d2c_lists_build(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
@@ -352,7 +352,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     }
     if (use_lists(q, s)) {
         size_t c, en, ov;
-        d2c_lists_ws(s, &c, &en, &ov);
+        d2c_lists_ws(s, q.dtype, &c, &en, &ov);
         w.counts = w.total;
         w.entries = w.counts + c;
         w.ovf = w.entries + en;
@@ -413,7 +413,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             // runs, by a pass of their own otherwise
             SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
             if (lists) {
-                L = d2c_lists_make(s, base + l.counts, base + l.entries, base + l.ovf);
+                L = d2c_lists_make(s, Elem<T>::DT, base + l.counts, base + l.entries, base + l.ovf);
                 if (int rc = auxk ? d2c_lists_clear(L, st) : d2c_lists_build(s, off, mask, L, st)) return rc;
             }
             if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt,
