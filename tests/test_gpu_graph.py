@@ -63,3 +63,47 @@ def test_forward_backward_replays_from_a_graph(name, dtype, dev):
                 assert_close(a, e, 1e-4, 1e-5 * max(1.0, e.abs().max().item()), f"{name} replay {rep} {n}")
             else:
                 assert rel_l2(a, e) < 2e-2, (name, rep, n, rel_l2(a, e))
+
+
+def test_plain_depthwise_conv_replays_from_a_graph(dev):
+    """d2c_dwconv3d_forward / _backward under capture: its scratch is cleared by a fill kernel, not a memset node."""
+    from d2conv3d_amd.depthwise_conv import depthwise_separable_conv3d
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(2, 16, 5, 12, 16, generator=g).to(dev).requires_grad_(True)
+    w = (torch.randn(16, 1, 3, 3, 3, generator=g) / 5).to(dev).requires_grad_(True)
+    b = torch.randn(16, generator=g).to(dev).requires_grad_(True)
+    gout = torch.randn(2, 16, 5, 12, 16, generator=g).to(dev)
+    ts = [x, w, b]
+
+    def step():
+        for t in ts:
+            t.grad = None
+        out = depthwise_separable_conv3d(x, w, b, 1, 1, 1)
+        out.backward(gout)
+        return out
+
+    e_out = step().detach().clone()
+    e_grads = [t.grad.clone() for t in ts]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    for t in ts:
+        t.grad = None
+    with torch.cuda.graph(graph):
+        out = depthwise_separable_conv3d(x, w, b, 1, 1, 1)
+        out.backward(gout)
+    grads = [t.grad for t in ts]
+    for rep in range(3):
+        out.zero_()
+        for gr in grads:
+            gr.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_close(out, e_out, 1e-5, 1e-6, f"replay {rep} out")
+        for i, (a, e) in enumerate(zip(grads, e_grads)):
+            assert_close(a, e, 1e-5, 1e-5 * max(1.0, e.abs().max().item()), f"replay {rep} grad{i}")
