@@ -380,6 +380,212 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------
+// The grad-column product alone (grad_input comes from the sample lists, the offset / mask gradient from the
+// kernel of d2c_aux_grad.hip: the usual case).  Same tiling and operands as tiled_bwd_data_kernel, but the
+// weight tile is double-buffered: the DMA transfer of step s+1 is in flight while step s is on the matrix
+// cores, and where the registers allow it (up to 256 reduced channels per pass for bfloat16) the fragment reads
+// run ahead of the matrix instructions.  Two barriers per step, both waiting for LDS operations only.
+// Used where two weight tiles and the float grad-column block fit LDS, i.e. not for the widest bfloat16
+// reduction (512 channels: two 64 KB tiles + 35 KB): there a bfloat16 block in LDS (written by pairs of lanes
+// that swap values) made room, but with the stationary operand alone in 128 registers the compiler spills and
+// serialises read - wait - multiply, and the kernel ran 10 % slower than the single-buffered one (0.73 against
+// 0.66 ms at C3; with 4 wavefronts of 512 registers per workgroup: 1.0 ms).
+D2C_DEV void lds_only_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// at most `n` vector-memory operations of this wavefront still in flight
+D2C_DEV void wait_vm_at_most(int n)
+{
+    switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
+    case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    }
+}
+
+// (XOR over 8 piece positions.  Spreading the pieces over 16 positions, the 64 banks of this LDS, took the
+// bank-conflict cycles of the fragment reads from 50 M to 6 M per launch at C3 and made the kernel 5 % slower.)
+D2C_DEV int swizzle_of_row(int row) { return row & 7; }
+
+template <typename T, int NKG>
+__global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int NV = 8, BKC = NV * VEC;
+    constexpr int CB = BKC / 32;           // 32-channel blocks per step (2 for bf16, 1 for float)
+    constexpr int PBW = 8 / CB;            // 32-position blocks per workgroup
+    constexpr int MT = 32 * PBW;           // positions per workgroup (128 / 256)
+    constexpr int GRS = BKC * 4 + 16;      // gcol tile row stride (bytes), float
+    constexpr int NW = kThreads / 64;
+    constexpr int ITEMS = MT * NV / kThreads;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    const TiledShape &s = a.s;
+    const int rowB = a.ogk * (int)sizeof(T);
+    const int tileB = BKC * rowB;
+    unsigned char *s_wt = smem;                          // [2][BKC][rowB]
+    unsigned char *s_gcol = s_wt + 2 * tileB;            // [MT][GRS]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
+    const int wg = blockIdx.y;
+    const int m0 = tile * MT;
+    const int S = s.nchunk * s.K;
+    const int cb = wave % CB, pb = wave / CB;
+    const int nkg = a.ogk / (2 * VEC);
+    const int rp = rowB / 16;                            // 16-byte pieces per weight row (a multiple of 8)
+    const int ninstr = BKC * rp / 64;                    // DMA instructions per tile, dealt to the wavefronts
+    const int mine = ninstr > wave ? (ninstr - wave + NW - 1) / NW : 0;   // (at most 8: rows of 1 KiB)
+
+    // ---- stationary operand: gout[pos, o] of this wavefront's 32 positions
+    uint4 ga[NKG];
+    {
+        const int m = m0 + pb * 32 + (lane & 31);
+        const bool ok = m < s.M;
+        const int b = ok ? m / s.P : 0, p = ok ? m - b * s.P : 0;
+        const T *gp = reinterpret_cast<const T *>(a.gout) + ((long)b * s.Cout + wg * s.og + a.o0) * s.P + p;
+#pragma unroll
+        for (int kg = 0; kg < NKG; kg++) {
+            T e[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const int o = (kg * 2 + (lane >> 5)) * VEC + i;
+                e[i] = (ok && kg < nkg && o < a.ogn) ? gp[(long)o * s.P] : (T)0;
+            }
+            ga[kg] = *reinterpret_cast<uint4 *>(e);
+        }
+    }
+
+    // weight tile of step st: global -> LDS without passing through registers; one instruction of a wavefront
+    // moves 64 pieces to 1 KiB of consecutive LDS (lane i's piece lands at base + 16 i), so lane i fetches the
+    // piece that the swizzled layout wants there
+    auto dma_tile = [&](int st, int buf) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * rp;
+        for (int i = wave; i < ninstr; i += NW) {
+            const int pos = i * 64 + lane;
+            const int row = pos / rp, q = pos - row * rp;
+            const uint4 *g = src + row * rp + (q ^ swizzle_of_row(row));
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                             (__attribute__((address_space(3))) void *)(s_wt + buf * tileB + i * 1024), 16,
+                                             0, 0);
+        }
+    };
+
+    // byte offsets (inside a tile) of this lane's fragments of the first 8 k-groups
+    int woff[8];
+    {
+        const int wrow = cb * 32 + (lane & 31);
+        const int wsw = swizzle_of_row(wrow), wh = lane >> 5;
+#pragma unroll
+        for (int i = 0; i < 8; i++) woff[i] = wrow * rowB + (((i * 2 + wh) ^ wsw) << 4);
+    }
+
+    const int st_lo = (int)((long)S * blockIdx.z / gridDim.z), st_hi = (int)((long)S * (blockIdx.z + 1) / gridDim.z);
+    if (st_lo < st_hi) dma_tile(st_lo, 0);
+    for (int st = st_lo, it = 0; st < st_hi; st++, it++) {
+        // step order: offset group (outer), tap, chunk of the group (inner), as in tiled_bwd_data_kernel
+        const int cpc = s.cpg / BKC;
+        const int jj = st % cpc, k = (st / cpc) % s.K, gi = st / (cpc * s.K);
+        const int j = gi * cpc + jj;
+        const int c0 = wg * s.cg + j * BKC;
+        const bool more = st + 1 < st_hi;
+        if (more) dma_tile(st + 1, (it + 1) & 1);
+        // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
+        // flight (requests complete in order; the grad-column stores of the previous step are older)
+        wait_vm_at_most(more ? mine : 0);
+        lds_only_barrier();
+
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.f;
+        {
+            const unsigned char *wb = s_wt + (it & 1) * tileB;
+            if (NKG >= 8 && nkg == NKG && rp % 16 == 0) {
+                // The usual case, free of branches.  Fragment kg of this lane lies at piece (2 kg + wh) ^ wsw of its
+                // row: the pieces of 8 consecutive k-groups share a block of 16 and differ from the next 8 by a
+                // constant, so 8 lane addresses + immediate offsets address all of them; the reads run kPF
+                // fragments ahead of the matrix instructions that take them.
+                constexpr int kPF = 3;
+                uint4 bq[kPF + 1];
+#pragma unroll
+                for (int i = 0; i < kPF; i++) bq[i] = *reinterpret_cast<const uint4 *>(wb + woff[i & 7] + (i >> 3) * 256);
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    if (kg + kPF < NKG)
+                        bq[(kg + kPF) % (kPF + 1)] =
+                            *reinterpret_cast<const uint4 *>(wb + woff[(kg + kPF) & 7] + ((kg + kPF) >> 3) * 256);
+                    mma_kgroup<T>(acc, ga[kg], bq[kg % (kPF + 1)]);
+                }
+            } else {
+                const int wrow = cb * 32 + (lane & 31);
+                const unsigned char *wr = wb + wrow * rowB;
+                const int wsw = swizzle_of_row(wrow), wh = lane >> 5;
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    if (kg < nkg) {
+                        const uint4 bf = *reinterpret_cast<const uint4 *>(wr + (((kg * 2 + wh) ^ wsw) << 4));
+                        mma_kgroup<T>(acc, ga[kg], bf);
+                    }
+                }
+            }
+        }
+        // grad-column block -> LDS: lanes 0..31 / 32..63 each cover 32 consecutive channels
+        const int ch = cb * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int pl = pb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            *reinterpret_cast<float *>(s_gcol + pl * GRS + ch * 4) = acc[r];
+        }
+        lds_only_barrier();
+        // rows out to memory, 16 bytes per thread
+        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) {
+            const int item = tid + i * kThreads;
+            const int pos = item / NV, vec = item % NV;
+            const int m = m0 + pos;
+            if (m < s.M) {
+                const float *gp = reinterpret_cast<const float *>(s_gcol + pos * GRS + vec * VEC * 4);
+                uint4 o;
+                if constexpr (sizeof(T) == 2) {
+                    o = make_uint4(pack_bf16x2(gp[0], gp[1]), pack_bf16x2(gp[2], gp[3]), pack_bf16x2(gp[4], gp[5]),
+                                   pack_bf16x2(gp[6], gp[7]));
+                } else {
+                    o = *reinterpret_cast<const uint4 *>(gp);
+                }
+                *reinterpret_cast<uint4 *>(gb + (long)m * BKC + vec * VEC) = o;
+            }
+        }
+    }
+}
+
+template <typename T> size_t bwd_col_lds(int ogk)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
+    return (size_t)2 * BKC * ogk * sizeof(T) + (size_t)MT * (BKC * 4 + 16);
+}
+
+template <typename T, int NKG>
+int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st)
+{
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
+    const size_t lds = bwd_col_lds<T>(a.ogk);
+    if (hipFuncSetAttribute((const void *)tiled_bwd_col_kernel<T, NKG>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024) != hipSuccess)
+        return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_col_kernel)");
+    dim3 grid((a.s.M + MT - 1) / MT, a.s.groups, nsplit);
+    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
+    hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG>), grid, dim3(kThreads), lds, st, a);
+    return d2c_check_launch("tiled_bwd_col_kernel");
+}
+
 template <typename T> size_t bwd_data_lds(int ogk)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
@@ -1021,10 +1227,19 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                       auxoff, auxmask};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
-        if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, nsplit, st);
-        else if (nkg <= 8) rc = launch_bwd_data<T, 8>(a, nsplit, st);
-        else if (nkg <= 16) rc = launch_bwd_data<T, 16>(a, nsplit, st);
-        else rc = launch_bwd_data<T, 32>(a, nsplit, st);
+        // (the double-buffered kernel where two weight tiles and the float grad-column block fit LDS)
+        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk) <= 160 * 1024;
+        if (col_only) {
+            if (nkg <= 4) rc = launch_bwd_col<T, 4>(a, nsplit, st);
+            else if (nkg <= 8) rc = launch_bwd_col<T, 8>(a, nsplit, st);
+            else if (nkg <= 16) rc = launch_bwd_col<T, 16>(a, nsplit, st);
+            else rc = launch_bwd_col<T, 32>(a, nsplit, st);
+        } else {
+            if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, nsplit, st);
+            else if (nkg <= 8) rc = launch_bwd_data<T, 8>(a, nsplit, st);
+            else if (nkg <= 16) rc = launch_bwd_data<T, 16>(a, nsplit, st);
+            else rc = launch_bwd_data<T, 32>(a, nsplit, st);
+        }
         if (rc) return rc;
     }
     if (auxoff) {
