@@ -209,11 +209,26 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
             const int wrow = cb * 32 + (lane & 31);
             const unsigned char *wb = s_wt + wrow * rowB;
             const int wsw = wrow & 7, wh = lane >> 5;
+            if (NKG >= 8 && nkg == NKG && (rowB / 16) % 16 == 0) {
+                // The usual case, free of branches.  Fragment kg lies at piece (2 kg + wh) ^ wsw of the row: the pieces
+                // of 8 consecutive k-groups share a block of 16 and differ from the next 8 by a constant, so 8 lane
+                // addresses + immediate offsets address all of them (32 addresses would not fit the registers
+                // next to the stationary operand).
+                const unsigned char *wa[8];
 #pragma unroll
-            for (int kg = 0; kg < NKG; kg++) {
-                if (kg < nkg) {
-                    const uint4 bf = *reinterpret_cast<const uint4 *>(wb + (((kg * 2 + wh) ^ wsw) << 4));
+                for (int i = 0; i < 8; i++) wa[i] = wb + (((i * 2 + wh) ^ wsw) << 4);
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    const uint4 bf = *reinterpret_cast<const uint4 *>(wa[kg & 7] + (kg >> 3) * 256);
                     mma_kgroup<T>(acc, ga[kg], bf);
+                }
+            } else {
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    if (kg < nkg) {
+                        const uint4 bf = *reinterpret_cast<const uint4 *>(wb + (((kg * 2 + wh) ^ wsw) << 4));
+                        mma_kgroup<T>(acc, ga[kg], bf);
+                    }
                 }
             }
         }
@@ -382,15 +397,16 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 
 // ---------------------------------------------------------------------------
 // The grad-column product alone (grad_input comes from the sample lists, the offset / mask gradient from the
-// kernel of d2c_aux_grad.hip: the usual case).  Same tiling and operands as tiled_bwd_data_kernel, but the
-// weight tile is double-buffered: the DMA transfer of step s+1 is in flight while step s is on the matrix
-// cores, and where the registers allow it (up to 256 reduced channels per pass for bfloat16) the fragment reads
-// run ahead of the matrix instructions.  Two barriers per step, both waiting for LDS operations only.
-// Used where two weight tiles and the float grad-column block fit LDS, i.e. not for the widest bfloat16
-// reduction (512 channels: two 64 KB tiles + 35 KB): there a bfloat16 block in LDS (written by pairs of lanes
-// that swap values) made room, but with the stationary operand alone in 128 registers the compiler spills and
-// serialises read - wait - multiply, and the kernel ran 10 % slower than the single-buffered one (0.73 against
-// 0.66 ms at C3; with 4 wavefronts of 512 registers per workgroup: 1.0 ms).
+// kernel of d2c_aux_grad.hip: the usual case).  Same tiling and operands as tiled_bwd_data_kernel, without its
+// other duties, and with the fragment reads running ahead of the matrix instructions.  Where two weight tiles
+// and the float grad-column block fit LDS (DB: fp32 problems, bfloat16 with up to 256 reduced channels per pass)
+// the weight tile is double-buffered: the DMA transfer of step s+1 is in flight while step s is on the matrix
+// cores.  Two barriers per step, both waiting for LDS operations only.
+// The widest bfloat16 reduction (512 channels: one 64 KB tile + the 35 KB block) stays single-buffered: two
+// tiles next to a bfloat16 block (written by pairs of lanes that swap values) fit, but ran slower in every form
+// tried (0.71 - 0.75 ms against 0.58 ms at C3; as 4 wavefronts of 512 registers per workgroup 1.0 ms).  For it the
+// matrix step is scheduled by hand (mma8_bf16): with the stationary operand alone in 128 of its 256 registers the
+// compiler emits read - wait - multiply for every fragment.
 D2C_DEV void lds_only_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // at most `n` vector-memory operations of this wavefront still in flight
@@ -414,7 +430,53 @@ D2C_DEV void wait_vm_at_most(int n)
 // bank-conflict cycles of the fragment reads from 50 M to 6 M per launch at C3 and made the kernel 5 % slower.)
 D2C_DEV int swizzle_of_row(int row) { return row & 7; }
 
-template <typename T, int NKG>
+// Eight k-groups of the matrix step for bfloat16, scheduled by hand: the compiler, short of registers next to the
+// 128-register stationary operand, emits read - wait - multiply for every fragment; here the LDS reads run three
+// fragments ahead of the matrix instructions (four rotating fragment registers; a register is reloaded after the
+// matrix instruction that follows the one which read it).  `w0..w7` are the lane's LDS addresses of the 8 fragments,
+// OFF the byte offset of this block of 8.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+template <int OFF>
+D2C_DEV void mma8_bf16(f32x16 &acc, const uint4 *g, const unsigned *w)
+{
+    u32x4 b0, b1, b2, b3;
+    const u32x4 g0 = __builtin_bit_cast(u32x4, g[0]), g1 = __builtin_bit_cast(u32x4, g[1]),
+                g2 = __builtin_bit_cast(u32x4, g[2]), g3 = __builtin_bit_cast(u32x4, g[3]),
+                g4 = __builtin_bit_cast(u32x4, g[4]), g5 = __builtin_bit_cast(u32x4, g[5]),
+                g6 = __builtin_bit_cast(u32x4, g[6]), g7 = __builtin_bit_cast(u32x4, g[7]);
+    asm volatile(
+        "ds_read_b128 %[b0], %[w0] offset:%[off]\n\t"
+        "ds_read_b128 %[b1], %[w1] offset:%[off]\n\t"
+        "ds_read_b128 %[b2], %[w2] offset:%[off]\n\t"
+        "ds_read_b128 %[b3], %[w3] offset:%[off]\n\t"
+        "s_waitcnt lgkmcnt(3)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g0], %[b0], %[acc]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g1], %[b1], %[acc]\n\t"
+        "ds_read_b128 %[b0], %[w4] offset:%[off]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g2], %[b2], %[acc]\n\t"
+        "ds_read_b128 %[b1], %[w5] offset:%[off]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g3], %[b3], %[acc]\n\t"
+        "ds_read_b128 %[b2], %[w6] offset:%[off]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g4], %[b0], %[acc]\n\t"
+        "ds_read_b128 %[b3], %[w7] offset:%[off]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g5], %[b1], %[acc]\n\t"
+        "s_waitcnt lgkmcnt(1)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g6], %[b2], %[acc]\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[g7], %[b3], %[acc]\n\t"
+        : [acc] "+v"(acc), [b0] "=&v"(b0), [b1] "=&v"(b1), [b2] "=&v"(b2), [b3] "=&v"(b3)
+        : [g0] "v"(g0), [g1] "v"(g1), [g2] "v"(g2), [g3] "v"(g3), [g4] "v"(g4), [g5] "v"(g5), [g6] "v"(g6), [g7] "v"(g7),
+          [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]), [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]),
+          [w7] "v"(w[7]), [off] "n"(OFF)
+        : "memory");
+}
+
+template <typename T, int NKG, bool DB>
 __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
 {
     constexpr int VEC = Elem<T>::VEC;
@@ -430,8 +492,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     const TiledShape &s = a.s;
     const int rowB = a.ogk * (int)sizeof(T);
     const int tileB = BKC * rowB;
-    unsigned char *s_wt = smem;                          // [2][BKC][rowB]
-    unsigned char *s_gcol = s_wt + 2 * tileB;            // [MT][GRS]
+    unsigned char *s_wt = smem;                          // [DB ? 2 : 1][BKC][rowB]
+    unsigned char *s_gcol = s_wt + (DB ? 2 : 1) * tileB; // [MT][GRS]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
@@ -488,7 +550,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     }
 
     const int st_lo = (int)((long)S * blockIdx.z / gridDim.z), st_hi = (int)((long)S * (blockIdx.z + 1) / gridDim.z);
-    if (st_lo < st_hi) dma_tile(st_lo, 0);
+    if (DB && st_lo < st_hi) dma_tile(st_lo, 0);
     for (int st = st_lo, it = 0; st < st_hi; st++, it++) {
         // step order: offset group (outer), tap, chunk of the group (inner), as in tiled_bwd_data_kernel
         const int cpc = s.cpg / BKC;
@@ -496,32 +558,55 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
         const int j = gi * cpc + jj;
         const int c0 = wg * s.cg + j * BKC;
         const bool more = st + 1 < st_hi;
-        if (more) dma_tile(st + 1, (it + 1) & 1);
-        // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
-        // flight (requests complete in order; the grad-column stores of the previous step are older)
-        wait_vm_at_most(more ? mine : 0);
+        if constexpr (DB) {
+            if (more) dma_tile(st + 1, (it + 1) & 1);
+            // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
+            // flight (requests complete in order; the grad-column stores of the previous step are older)
+            wait_vm_at_most(more ? mine : 0);
+        } else {
+            // one tile buffer: every wavefront is past the matrix step of st-1 (the barrier behind it).  (Requesting
+            // the tile earlier, behind that barrier, so that it comes in while the rows go out, was 3 % slower.)
+            dma_tile(st, 0);
+            wait_vm_at_most(0);
+        }
         lds_only_barrier();
 
         f32x16 acc;
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = 0.f;
         {
-            const unsigned char *wb = s_wt + (it & 1) * tileB;
+            const unsigned char *wb = s_wt + (DB ? (it & 1) : 0) * tileB;
             if (NKG >= 8 && nkg == NKG && rp % 16 == 0) {
                 // The usual case, free of branches.  Fragment kg of this lane lies at piece (2 kg + wh) ^ wsw of its
                 // row: the pieces of 8 consecutive k-groups share a block of 16 and differ from the next 8 by a
                 // constant, so 8 lane addresses + immediate offsets address all of them; the reads run kPF
                 // fragments ahead of the matrix instructions that take them.
-                constexpr int kPF = 3;
-                uint4 bq[kPF + 1];
+                if constexpr (sizeof(T) == 2 && NKG == 32) {
+                    // (the accumulator was cleared by vector moves just now, and is read by vector instructions
+                    // right after: the waits that the compiler adds around its own matrix instructions)
+                    unsigned wl[8];
+                    const unsigned lbase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)wb;
 #pragma unroll
-                for (int i = 0; i < kPF; i++) bq[i] = *reinterpret_cast<const uint4 *>(wb + woff[i & 7] + (i >> 3) * 256);
+                    for (int i = 0; i < 8; i++) wl[i] = lbase + (unsigned)woff[i];
+                    asm volatile("s_nop 4" ::: "memory");
+                    mma8_bf16<0>(acc, ga, wl);
+                    mma8_bf16<256>(acc, ga + 8, wl);
+                    mma8_bf16<512>(acc, ga + 16, wl);
+                    mma8_bf16<768>(acc, ga + 24, wl);
+                    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc)::"memory");
+                } else {
+                    constexpr int kPF = 3;
+                    uint4 bq[kPF + 1];
 #pragma unroll
-                for (int kg = 0; kg < NKG; kg++) {
-                    if (kg + kPF < NKG)
-                        bq[(kg + kPF) % (kPF + 1)] =
-                            *reinterpret_cast<const uint4 *>(wb + woff[(kg + kPF) & 7] + ((kg + kPF) >> 3) * 256);
-                    mma_kgroup<T>(acc, ga[kg], bq[kg % (kPF + 1)]);
+                    for (int i = 0; i < kPF; i++)
+                        bq[i] = *reinterpret_cast<const uint4 *>(wb + woff[i & 7] + (i >> 3) * 256);
+#pragma unroll
+                    for (int kg = 0; kg < NKG; kg++) {
+                        if (kg + kPF < NKG)
+                            bq[(kg + kPF) % (kPF + 1)] =
+                                *reinterpret_cast<const uint4 *>(wb + woff[(kg + kPF) & 7] + ((kg + kPF) >> 3) * 256);
+                        mma_kgroup<T>(acc, ga[kg], bq[kg % (kPF + 1)]);
+                    }
                 }
             } else {
                 const int wrow = cb * 32 + (lane & 31);
@@ -566,23 +651,25 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     }
 }
 
-template <typename T> size_t bwd_col_lds(int ogk)
+template <typename T> size_t bwd_col_lds(int ogk, bool db)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
-    return (size_t)2 * BKC * ogk * sizeof(T) + (size_t)MT * (BKC * 4 + 16);
+    return (size_t)(db ? 2 : 1) * BKC * ogk * sizeof(T) + (size_t)MT * (BKC * 4 + 16);
 }
 
 template <typename T, int NKG>
 int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
-    const size_t lds = bwd_col_lds<T>(a.ogk);
-    if (hipFuncSetAttribute((const void *)tiled_bwd_col_kernel<T, NKG>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            160 * 1024) != hipSuccess)
+    const bool db = bwd_col_lds<T>(a.ogk, true) <= 160 * 1024;
+    const size_t lds = bwd_col_lds<T>(a.ogk, db);
+    const void *fn = db ? (const void *)tiled_bwd_col_kernel<T, NKG, true> : (const void *)tiled_bwd_col_kernel<T, NKG, false>;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
         return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_col_kernel)");
     dim3 grid((a.s.M + MT - 1) / MT, a.s.groups, nsplit);
     D2cProfScope prof(D2C_PROF_BWD_DATA, st);
-    hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG>), grid, dim3(kThreads), lds, st, a);
+    if (db) hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, true>), grid, dim3(kThreads), lds, st, a);
+    else hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, false>), grid, dim3(kThreads), lds, st, a);
     return d2c_check_launch("tiled_bwd_col_kernel");
 }
 
@@ -1227,8 +1314,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                       auxoff, auxmask};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
-        // (the double-buffered kernel where two weight tiles and the float grad-column block fit LDS)
-        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk) <= 160 * 1024;
+        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
         if (col_only) {
             if (nkg <= 4) rc = launch_bwd_col<T, 4>(a, nsplit, st);
             else if (nkg <= 8) rc = launch_bwd_col<T, 8>(a, nsplit, st);
