@@ -285,7 +285,7 @@ def _random_case(rng, depthwise):
     groups = pick(1, 1, 2)
     G = groups * pick(1, 2)
     Cin = 64 * G * pick(1, 2) if groups == 1 else 64 * G
-    Cout = groups * int(rng.integers(1, 300))
+    Cout = G * int(rng.integers(1, 300 // G + 1))      # a multiple of groups and of the offset groups
     return N, Cin, Cout, dims, k, s, p, d, groups, G, bool(rng.integers(2)), bool(rng.integers(2)), float(pick(0.5, 1.5, 3.0))
 
 
@@ -294,12 +294,15 @@ def _random_case(rng, depthwise):
 def test_random_geometries_against_the_direct_kernels(depthwise, dtype, dev):
     """Seeded random shapes, strides, paddings, dilations, groups and offset scales: the matrix-core / channel-separated
     kernels against the direct kernels (one thread per element, checked against the oracle on the reference's test
-    matrix in test_gpu_reference_matrix.py) on the same tensors, forward and all gradients."""
+    matrix in test_gpu_reference_matrix.py) on the same tensors, forward and all gradients.  D2C_RANDOM_CASES in the
+    environment widens the sweep (10 by default); each case is printed before it runs."""
+    import os
     import numpy as np
     rng = np.random.default_rng(20240 + int(depthwise))
     tol = 1e-4 if dtype == torch.float32 else 2e-2
-    for case in range(10):
+    for case in range(int(os.environ.get("D2C_RANDOM_CASES", "10"))):
         shape = _random_case(rng, depthwise)
+        print(f"random case {case} depthwise={depthwise} {dtype}: {shape}", flush=True)
         SHAPES["_random"] = shape
         try:
             (x, off, m, w, b), gout, (s, p, d, groups, G) = make("_random", dtype, seed=100 + case)
