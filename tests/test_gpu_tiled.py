@@ -324,3 +324,46 @@ def test_random_geometries_against_the_direct_kernels(depthwise, dtype, dev):
         for a, e in zip(*res):
             scale = max(1.0, e.abs().max().item())
             assert (a - e).abs().max().item() <= tol * scale, (shape, (a - e).abs().max().item(), scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_random_geometries_1d_against_the_direct_kernels(dtype, dev):
+    """The 1-D operator on seeded random lengths, kernel sizes, strides, paddings, dilations and groups: matrix-core
+    kernels against the direct kernels on the same tensors, forward and all gradients (D2C_RANDOM_CASES widens
+    the sweep)."""
+    import os
+    import numpy as np
+    rng = np.random.default_rng(777)
+    pick = lambda *v: v[int(rng.integers(len(v)))]
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    for case in range(int(os.environ.get("D2C_RANDOM_CASES", "10"))):
+        k, st, d = pick(1, 2, 3, 5), pick(1, 1, 2, 3), pick(1, 1, 2, 3)
+        pad = int(rng.integers(0, 4))
+        L = int(rng.integers(d * (k - 1) + 2, d * (k - 1) + 90))
+        groups = pick(1, 1, 2)
+        G = groups * pick(1, 2)
+        Cin = 64 * G * pick(1, 2) if groups == 1 else 64 * G
+        Cout = G * int(rng.integers(1, 300 // G + 1))
+        shape = (pick(1, 2, 5), Cin, Cout, L, k, st, pad, d, groups, G, bool(rng.integers(2)), bool(rng.integers(2)),
+                 float(pick(0.5, 1.5, 3.0)))
+        print(f"random 1-D case {case} {dtype}: {shape}", flush=True)
+        SHAPES_1D["_random"] = shape
+        try:
+            (x, off, m, w, b), gout, (s, p, d, groups, G) = make1d("_random", dtype, seed=300 + case)
+        finally:
+            del SHAPES_1D["_random"]
+        res = []
+        for family in (None, "generic"):
+            ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+            _ops.set_algo_override(family)
+            try:
+                if family is None:
+                    assert _ops.conv1d_algo(ts[0], ts[1], ts[2], ts[3], s, p, d, groups, G) == "mfma", shape
+                out = d2c.deform_conv1d(*ts, s, p, d, groups, G)
+                out.backward(gout.to(dev))
+            finally:
+                _ops.set_algo_override(None)
+            res.append([out.detach().float()] + [t.grad.float() for t in ts if t is not None])
+        for a, e in zip(*res):
+            scale = max(1.0, e.abs().max().item())
+            assert (a - e).abs().max().item() <= tol * scale, (shape, (a - e).abs().max().item(), scale)
