@@ -80,6 +80,28 @@ def test_shapes(dtype, case, dev):
     _run(dev, dtype, *case, seed=3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+def test_random_geometries(dtype, dev):
+    """Seeded random sizes, filters, strides, paddings, dilations and depth multipliers against the oracle; widths
+    are drawn so that the vector, the blocked and the element-per-thread kernels all get cases (D2C_RANDOM_CASES
+    in the environment widens the sweep; each case is printed before it runs)."""
+    import os
+    rng = np.random.default_rng(4242)
+    pick = lambda *v: v[int(rng.integers(len(v)))]
+    for case in range(int(os.environ.get("D2C_RANDOM_CASES", "12"))):
+        k = (pick(1, 3, 3), pick(1, 3, 3), pick(1, 2, 3, 3, 5))
+        s = (pick(1, 1, 2), pick(1, 1, 2), pick(1, 1, 1, 2))
+        d = (pick(1, 1, 2), pick(1, 1, 2), pick(1, 1, 2))
+        p = tuple(int(rng.integers(0, 3)) for _ in range(3))
+        dims = [int(rng.integers(dd * (kk - 1) + 1, dd * (kk - 1) + 1 + 8)) for kk, dd in zip(k, d)]
+        if rng.integers(2):
+            dims[2] = max(dims[2], 4 * int(rng.integers(1, 36)))      # widths that are multiples of 4, up to 140
+        shape = (pick(1, 2, 3), int(rng.integers(1, 20)), pick(1, 1, 2, 3), tuple(dims), k, s, p, d,
+                 bool(rng.integers(2)))
+        print(f"random case {case} {dtype}: {shape}", flush=True)
+        _run(dev, dtype, *shape, seed=500 + case)
+
+
 def test_many_positions_per_channel(dev):
     """More items than one launch covers in one pass of its grid-stride loops, and several shares in grad_weight."""
     _run(dev, torch.float32, 1, 2, 1, (16, 64, 130), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), True, seed=5)
