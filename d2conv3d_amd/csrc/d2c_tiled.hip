@@ -87,10 +87,20 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0)
     return s;
 }
 
+// The tiled kernels let dead corners read a 256-byte row of zeros that follows the channels-last input; the first
+// workgroup of the pack kernel writes it (the batch size is the grid's z extent; C is a multiple of the channel
+// chunk there, so the row is 128-byte aligned).
+template <typename T> D2C_DEV void pack_zero_row(T *xcl, int C, int vol, int zero_row)
+{
+    if (zero_row && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < 64)
+        reinterpret_cast<unsigned *>(xcl + (long)gridDim.z * C * vol)[threadIdx.x] = 0u;
+}
+
 // x [N][C][vol] -> xcl [N][vol][C]  (32 x 32 element tiles through LDS)
 template <typename T>
-__global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int C, int vol)
+__global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int C, int vol, int zero_row)
 {
+    pack_zero_row(xcl, C, vol, zero_row);
     __shared__ T tile[32][33];
     const int b = blockIdx.z, v0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
@@ -111,8 +121,9 @@ __global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int
 
 // The same for bfloat16 with 16-byte accesses on both sides (2-byte accesses of 32 lanes move 64 bytes per
 // request): 64 x 64 element tiles; needs vol and C to be multiples of 8 and 16-byte aligned tensors.
-__global__ void __launch_bounds__(256) pack_input_bf16_kernel(const bf16_t *x, bf16_t *xcl, int C, int vol)
+__global__ void __launch_bounds__(256) pack_input_bf16_kernel(const bf16_t *x, bf16_t *xcl, int C, int vol, int zero_row)
 {
+    pack_zero_row(xcl, C, vol, zero_row);
     constexpr int RS = 66;                             // LDS row stride in elements (33 words)
     __shared__ bf16_t tile[64 * RS];                   // [v][c]
     const int b = blockIdx.z, v0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
@@ -229,7 +240,7 @@ FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 template <typename T>
-int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st)
+int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st, bool zero_row = false)
 {
     dim3 grid((s.vol + 31) / 32, (s.Cin + 31) / 32, s.N);
     D2cProfScope prof(D2C_PROF_PACK, st);
@@ -237,11 +248,11 @@ int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st)
         if (s.vol % 8 == 0 && s.Cin % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
             reinterpret_cast<uintptr_t>(xcl) % 16 == 0) {
             hipLaunchKernelGGL(pack_input_bf16_kernel, dim3((s.vol + 63) / 64, (s.Cin + 63) / 64, s.N), dim3(256), 0, st,
-                               (const bf16_t *)x, (bf16_t *)xcl, s.Cin, s.vol);
+                               (const bf16_t *)x, (bf16_t *)xcl, s.Cin, s.vol, (int)zero_row);
             return d2c_check_launch("pack_input_bf16_kernel");
         }
     }
-    hipLaunchKernelGGL(pack_input_kernel<T>, grid, dim3(256), 0, st, (const T *)x, (T *)xcl, s.Cin, s.vol);
+    hipLaunchKernelGGL(pack_input_kernel<T>, grid, dim3(256), 0, st, (const T *)x, (T *)xcl, s.Cin, s.vol, (int)zero_row);
     return d2c_check_launch("pack_input_kernel");
 }
 
@@ -289,11 +300,7 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
         return d2c_depthwise_forward<T>(s, base + d.xcl, off, mask, w, base + d.wt, bias, out, st);
     }
     const FwdWs l = fwd_ws(q, s);
-    if (int rc = pack_input<T>(s, x, base + l.xcl, st)) return rc;
-    {
-        D2cProfScope prof(D2C_PROF_PACK, st);
-        d2c_fill_zero(base + l.xcl + (size_t)s.N * s.vol * s.Cin * sizeof(T), 256, st);   // what dead corners read
-    }
+    if (int rc = pack_input<T>(s, x, base + l.xcl, st, true)) return rc;   // with the row of zeros behind it
     const long total = (long)s.groups * s.nchunk * s.K * (s.ogp / 32) * 4 * 64;
     long g = (total + 255) / 256;
     if (g > 8192) g = 8192;
@@ -403,7 +410,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         return D2C_OK;
     }
     const BwdWs l = bwd_ws(q, s);
-    if (int rc = pack_input<T>(s, x, base + l.xcl, st)) return rc;
+    if (int rc = pack_input<T>(s, x, base + l.xcl, st, true)) return rc;   // with the row of zeros behind it
     if (gx || goff || gmask) {
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;

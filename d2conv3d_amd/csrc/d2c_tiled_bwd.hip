@@ -1358,8 +1358,8 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
-        // the channels-last input is followed by a 256-byte row of zeros: what dead corners read
-        d2c_fill_zero((char *)const_cast<void *>(xcl) + (size_t)s.N * s.vol * s.Cin * sizeof(T), 256, st);
+        // (the channels-last input is followed by a 256-byte row of zeros, written by the kernel that packed it:
+        // what dead corners read)
         const int OBT = (s.og + 63) / 64 * 2;
         const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
         const bool vec = s.P % Elem<T>::VEC == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0;
