@@ -89,10 +89,13 @@ def _unify(input, offset, alpha, weight, bias):
 
 
 class _DeformConv3dFunction(torch.autograd.Function):
-    """DeformConv3dFunction of dconv3d.h:70-186."""
+    """DeformConv3dFunction of dconv3d.h:70-186.  `relu_scale` > 0 (not in the reference) makes the forward
+    kernels store relu_scale * max(out, 0) -- the activation that follows the convolution, fused into their last
+    step; the backward pass then starts from grad_out * relu_scale where the stored output is positive."""
 
     @staticmethod
-    def forward(ctx, input, offset, alpha, weight, bias, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, offset_groups):
+    def forward(ctx, input, offset, alpha, weight, bias, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, offset_groups,
+                relu_scale=0.0):
         lib = _lib.load()
         input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
         alpha = alpha.contiguous() if alpha is not None else None
@@ -101,7 +104,8 @@ class _DeformConv3dFunction(torch.autograd.Function):
         Cout, _, kd, kh, kw = weight.shape
         Do, Ho, Wo = offset.shape[2:]
         desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, sd, sh, sw, pd, ph, pw, dd, dh, dw,
-                               groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype])
+                               groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype],
+                               _lib.EPILOGUE_RELU if relu_scale > 0 else _lib.EPILOGUE_NONE, float(relu_scale) or 1.0)
         _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d")
         dev = input.device
         out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
@@ -111,18 +115,21 @@ class _DeformConv3dFunction(torch.autograd.Function):
             rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha), _ptr(weight),
                                         _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d forward")
-        ctx.save_for_backward(input, offset, alpha, weight, bias)
+        ctx.save_for_backward(input, offset, alpha, weight, bias, out if relu_scale > 0 else None)
         ctx.desc = desc
+        ctx.relu_scale = float(relu_scale)
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_out):
         lib = _lib.load()
-        input, offset, alpha, weight, bias = ctx.saved_tensors
+        input, offset, alpha, weight, bias, out = ctx.saved_tensors
         desc = ctx.desc
         dev = input.device
         grad_out = grad_out.contiguous().to(input.dtype)
+        if out is not None:    # gradient with respect to the value before the fused activation
+            grad_out = torch.where(out > 0, grad_out * ctx.relu_scale, torch.zeros_like(grad_out))
         need = ctx.needs_input_grad
         gx = torch.empty_like(input) if need[0] else None
         goff = torch.empty_like(offset) if need[1] else None
@@ -136,18 +143,19 @@ class _DeformConv3dFunction(torch.autograd.Function):
                                          _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
                                          _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d backward")
-        return (gx, goff, galpha, gw, gb) + (None,) * 11
+        return (gx, goff, galpha, gw, gb) + (None,) * 12
 
 
 def deform_conv3d(input, offset, alpha, weight, bias, stride_d, stride_h, stride_w, pad_d, pad_h, pad_w,
-                  dilation_d, dilation_h, dilation_w, groups, offset_groups):
-    """deform_conv3d of dconv3d.h:188-226; `alpha` and `bias` may be None."""
+                  dilation_d, dilation_h, dilation_w, groups, offset_groups, relu_scale=0.0):
+    """deform_conv3d of dconv3d.h:188-226; `alpha` and `bias` may be None.  `relu_scale` > 0 fuses
+    relu_scale * relu(.) into the store of the output (see _DeformConv3dFunction)."""
     _check_common(3, input, offset, alpha, weight, bias, groups, offset_groups)
     input, offset, alpha, weight, bias = _unify(input, offset, alpha, weight, bias)
     return _DeformConv3dFunction.apply(
         input, offset, alpha, weight, bias, int(stride_d), int(stride_h), int(stride_w),
         int(pad_d), int(pad_h), int(pad_w), int(dilation_d), int(dilation_h), int(dilation_w),
-        int(groups), int(offset_groups))
+        int(groups), int(offset_groups), float(relu_scale))
 
 
 class _DeformConv1dFunction(torch.autograd.Function):

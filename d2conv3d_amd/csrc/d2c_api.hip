@@ -201,6 +201,9 @@ int d2c_conv3d_check(const d2c_conv3d_desc *q)
                     && (long)q->N * q->offset_groups * 3 * K * P < (1L << 31)
                     && (long)q->Cout * (q->Cin / q->groups) * K < (1L << 31),
                 "tensor with 2^31 or more elements is not supported");
+    D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || q->epilogue == D2C_EPILOGUE_RELU, "unknown epilogue %d", q->epilogue);
+    D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || (q->epilogue_scale > 0.f && q->epilogue_scale < 3.0e38f),
+                "epilogue_scale must be positive and finite");
     return D2C_OK;
 }
 

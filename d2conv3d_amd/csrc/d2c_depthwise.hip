@@ -234,7 +234,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
             T *o = out + ((long)bf * s.Cout + c + j) * s.P + pf;
             alignas(16) T e[PW];
 #pragma unroll
-            for (int i = 0; i < PW; i++) e[i] = f32_to_elem<T>(acc[i][j] + bv[j]);
+            for (int i = 0; i < PW; i++) e[i] = f32_to_elem<T>(d2c_epilogue(acc[i][j] + bv[j], s.act, s.act_scale));
 #pragma unroll
             for (int q = 0; q < PW / EV; q++) reinterpret_cast<uint4 *>(o)[q] = reinterpret_cast<const uint4 *>(e)[q];
         }
@@ -246,7 +246,7 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
                 const int b = m / s.P, pp = m - b * s.P;
 #pragma unroll
                 for (int j = 0; j < kCV; j++)
-                    out[((long)b * s.Cout + c + j) * s.P + pp] = f32_to_elem<T>(acc[i][j] + bv[j]);
+                    out[((long)b * s.Cout + c + j) * s.P + pp] = f32_to_elem<T>(d2c_epilogue(acc[i][j] + bv[j], s.act, s.act_scale));
             }
         }
     }

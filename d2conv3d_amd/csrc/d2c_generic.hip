@@ -20,6 +20,8 @@ inline int grid_for(long n, int block = kBlock)
 struct Shape3 {
     int N, Cin, Cout, D, H, W, K, G, groups, Do, Ho, Wo;
     int dt, adt;
+    int act;            // forward epilogue: 0 none, 1 act_scale * max(v, 0)
+    float act_scale;
     long P, vol;
     TapGeom geo;
 };
@@ -30,6 +32,7 @@ inline Shape3 shape_of(const d2c_conv3d_desc &q)
     s.N = q.N; s.Cin = q.Cin; s.Cout = q.Cout; s.D = q.D; s.H = q.H; s.W = q.W;
     s.K = q.kd * q.kh * q.kw; s.G = q.offset_groups; s.groups = q.groups;
     s.Do = q.Do; s.Ho = q.Ho; s.Wo = q.Wo; s.dt = q.dtype; s.adt = q.aux_dtype;
+    s.act = q.epilogue; s.act_scale = q.epilogue_scale;
     s.P = (long)q.Do * q.Ho * q.Wo; s.vol = (long)q.D * q.H * q.W;
     s.geo = make_geom(q);
     return s;
@@ -103,6 +106,7 @@ generic_fwd3d(Shape3 s, const void *x, const void *off, const void *mask, const 
             }
         }
         if (bias) acc += ld_as<CT>(bias, o, s.dt);
+        if (s.act) acc = (acc < (CT)0 ? (CT)0 : acc) * (CT)s.act_scale;
         st_as<CT>(out, idx, s.dt, acc);
     }
 }

@@ -132,8 +132,18 @@ struct TiledShape {
     int M;                // N * P
     int nd;               // 3, or 1 for the 1-D operator mapped onto a 1 x 1 x L volume
     int quirks;           // 1-D only: integer-position rule of dconv1d_gpu.cu:332-336 in grad_offset / grad_mask
+    int act;              // forward epilogue: 0 none, 1 act_scale * max(v, 0)
+    float act_scale;
     TapGeom geo;
 };
+
+// The forward kernels' last step before a value is stored (NaN stays NaN, as in torch's relu).
+__host__ __device__ inline float d2c_epilogue(float v, int act, float scale)
+{
+    // branch-free: without activation the floor is -inf and the factor 1 (v * 1 is exact)
+    const float lo = act ? 0.f : -__builtin_inff(), sc = act ? scale : 1.f;
+    return (v < lo ? lo : v) * sc;
+}
 
 // ---- sample lists: every live sample (b, g, k, p) filed under its base voxel floor(z, y, x) -------------------
 struct alignas(16) InvEntry {

@@ -257,7 +257,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
                             atomicAdd(a.outacc + ((long)b * s.Cout + o) * s.P + p, v);
                         } else {
                             if (bias) v += elem_to_f32<T>(bias[o]);
-                            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(v);
+                            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(d2c_epilogue(v, s.act, s.act_scale));
                         }
                     }
                 }
@@ -587,7 +587,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                         if (ok && oo < nvalid) {
                             float v = acc[ob][pb][r];
                             if (bias) v += elem_to_f32<T>(bias[o0 + oo]);
-                            op[(long)oo * s.P] = f32_to_elem<T>(v);
+                            op[(long)oo * s.P] = f32_to_elem<T>(d2c_epilogue(v, s.act, s.act_scale));
                         }
                         acc[ob][pb][r] = 0.f;
                     }
@@ -703,7 +703,7 @@ __global__ void __launch_bounds__(256) fwd_dma_finish_kernel(FwdArgs a, int NT)
             const int o = wg * s.og + ol, b = m / s.P, p = m - b * s.P;
             float v = acc[(long)ot * MT + pl];
             if (bias) v += elem_to_f32<T>(bias[o]);
-            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(v);
+            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(d2c_epilogue(v, s.act, s.act_scale));
         }
     }
 }
@@ -757,14 +757,15 @@ int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
     return 0;
 }
 
-// out = outacc + bias, in the element type of the output
+// out = epilogue(outacc + bias), in the element type of the output
 template <typename T>
-__global__ void __launch_bounds__(256) fwd_finish_kernel(const float *acc, const T *bias, T *out, int Cout, int P, long n)
+__global__ void __launch_bounds__(256) fwd_finish_kernel(const float *acc, const T *bias, T *out, int Cout, int P, long n,
+                                                         int act, float act_scale)
 {
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
         float v = acc[i];
         if (bias) v += elem_to_f32<T>(bias[(i / P) % Cout]);
-        out[i] = f32_to_elem<T>(v);
+        out[i] = f32_to_elem<T>(d2c_epilogue(v, act, act_scale));
     }
 }
 
@@ -863,7 +864,7 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
     if (g > 8192) g = 8192;
     D2cProfScope prof(D2C_PROF_PACK, st);
     hipLaunchKernelGGL(fwd_finish_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, outacc, (const T *)bias, (T *)out,
-                       s.Cout, s.P, n);
+                       s.Cout, s.P, n, s.act, s.act_scale);
     return d2c_check_launch("fwd_finish_kernel");
 }
 template int d2c_tiled_fwd_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,

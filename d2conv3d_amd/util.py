@@ -71,6 +71,35 @@ def add_deformable_conv(module, **kwargs):
     return replace_module(dconv_replace_layer, nn.Conv3d, module, **kwargs)
 
 
+SCALED_RELU = 1.71285855    # network/layers.py:409-411
+
+
+def fuse_output_activation(module):
+    """Folds the activation that follows a deformable convolution into the convolution's forward kernels: in
+    every nn.Sequential under `module` a D2Conv layer directly followed by nn.ReLU or by a ScaledReLU
+    (network/layers.py:414-419; recognised by its class name) -- the `_conv` blocks of the reference's
+    refinement modules, network/modules/refinement.py:38-43 -- keeps its place, the activation becomes
+    nn.Identity and the layer's DeformConv3d stores scale * relu(out) itself.  Returns the number of fused pairs.
+    State-dict keys do not change (neither activation has parameters)."""
+    fused = 0
+    for seq in [m for m in module.modules() if isinstance(m, nn.Sequential)]:
+        names = list(seq._modules)
+        for a, b in zip(names, names[1:]):
+            conv, act = seq._modules[a], seq._modules[b]
+            if not isinstance(conv, _m._DConvBase) or conv.deform_conv.output_relu_scale is not None:
+                continue
+            if isinstance(act, nn.ReLU):
+                scale = 1.0
+            elif type(act).__name__ == "ScaledReLU":
+                scale = SCALED_RELU
+            else:
+                continue
+            conv.deform_conv.output_relu_scale = scale
+            seq._modules[b] = nn.Identity()
+            fused += 1
+    return fused
+
+
 def tap_statistics(input_shape, offset, kernel_size, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
                    offset_groups=1):
     """How much of an offset field samples outside the volume: the debug output the reference's trainer expects

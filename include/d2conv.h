@@ -62,6 +62,9 @@ enum {
     D2C_ALGO_DEPTHWISE = 3  /* groups == Cin == Cout, bandwidth kernels */
 };
 
+#define D2C_EPILOGUE_NONE 0
+#define D2C_EPILOGUE_RELU 1
+
 typedef struct d2c_conv3d_desc {
     int32_t N, Cin, Cout;
     int32_t D, H, W;
@@ -72,6 +75,13 @@ typedef struct d2c_conv3d_desc {
     int32_t groups, offset_groups;
     int32_t Do, Ho, Wo;   /* spatial size of offset / mask / out as passed by the caller */
     int32_t dtype, aux_dtype;
+    /* What the forward kernels do to a value (bias included) before they store it: nothing, or
+     * epilogue_scale * max(value, 0) -- the ReLU / ScaledReLU that follows every deformable convolution of the
+     * reference's refinement modules (network/modules/refinement.py:38-43, network/layers.py:409-419), saving the
+     * separate pass over the output.  The backward call ignores these fields: it expects the gradient with respect
+     * to the value before the activation (grad_out * epilogue_scale where out > 0, else 0). */
+    int32_t epilogue;     /* D2C_EPILOGUE_NONE or D2C_EPILOGUE_RELU */
+    float epilogue_scale;
 } d2c_conv3d_desc;
 
 typedef struct d2c_conv1d_desc {

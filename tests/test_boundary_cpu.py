@@ -55,6 +55,12 @@ def test_conv3d_check_accepts_and_rejects():
     assert lib.d2c_conv3d_check(ctypes.byref(_desc(dtype=7))) != 0
     assert lib.d2c_conv3d_check(ctypes.byref(_desc(dtype=0, aux_dtype=2))) != 0
     assert lib.d2c_conv3d_check(ctypes.byref(_desc(dtype=2, aux_dtype=0))) == 0
+    # the forward epilogue: none, or a ReLU with a positive finite scale
+    assert lib.d2c_conv3d_check(ctypes.byref(_desc(epilogue=_lib.EPILOGUE_RELU, epilogue_scale=1.71285855))) == 0
+    assert lib.d2c_conv3d_check(ctypes.byref(_desc(epilogue=5, epilogue_scale=1.0))) != 0
+    assert "unknown epilogue" in _lib.last_error()
+    assert lib.d2c_conv3d_check(ctypes.byref(_desc(epilogue=_lib.EPILOGUE_RELU, epilogue_scale=0.0))) != 0
+    assert lib.d2c_conv3d_check(ctypes.byref(_desc(epilogue=_lib.EPILOGUE_RELU, epilogue_scale=float("inf")))) != 0
 
 
 def test_workspace_queries_run_without_gpu():
