@@ -41,6 +41,20 @@ struct AuxArgs {
     SampleLists lists;   // counts != NULL: every live sample is filed in its bucket on the way (for grad_input)
 };
 
+// Sum over the 8 lanes of a position without LDS traffic: neighbours of a quad, the other pair of the quad, then
+// the other quad of the 8 (row_half_mirror: lane i reads lane 7 - i of its half row; all lanes of a quad hold the
+// same value by then).
+template <int CTRL> D2C_DEV float dpp_add(float v)
+{
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+D2C_DEV float sum_over_8_lanes(float v)
+{
+    v = dpp_add<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+    v = dpp_add<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+    return dpp_add<0x141>(v); // row_half_mirror
+}
+
 template <typename T, bool AUX16>
 __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a)
 {
@@ -222,13 +236,10 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                         gxx += ((c & 1) ? d : -d) * (wz * wy);
                         if ((live >> c) & 1u) gm += (wz * wy * wx) * d;
                     }
-#pragma unroll
-                    for (int sft = 1; sft < 8; sft <<= 1) {
-                        gz += __shfl_xor(gz, sft, 64);
-                        gy += __shfl_xor(gy, sft, 64);
-                        gxx += __shfl_xor(gxx, sft, 64);
-                        gm += __shfl_xor(gm, sft, 64);
-                    }
+                    gz = sum_over_8_lanes(gz);
+                    gy = sum_over_8_lanes(gy);
+                    gxx = sum_over_8_lanes(gxx);
+                    gm = sum_over_8_lanes(gm);
                     g_acc[r][0] += gz; g_acc[r][1] += gy; g_acc[r][2] += gxx; g_acc[r][3] += gm;
                 }
             }
