@@ -27,8 +27,10 @@ constexpr int kWavesPerBlock = 4;
 constexpr int kMT = 64;                    // positions per wavefront
 constexpr int kTab = 9;                    // table words per position: idx, flag, lz ly lx hz hy hx, alpha
 constexpr int kRounds = 1;                 // rounds whose loads are in flight together
-constexpr int kTapSplit = 9;               // wavefronts per (tile, group), each with its share of the taps (many short
-                                           // tasks balance better than few long ones: 0.49 ms against 0.59 ms at 1)
+constexpr int kTapSplit = 27;              // wavefronts per (tile, group), each with its share of the taps: many short
+                                           // tasks balance better than few long ones (C=512, 8 groups, 27 taps:
+                                           // 0.67 ms at 3 shares, 0.57 at 9, 0.54 at 27; one group of 256 channels
+                                           // on 207360 positions: 2.65 / 2.11 / 1.75 ms)
 
 struct AuxArgs {
     TiledShape s;
@@ -68,13 +70,16 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     float (*s_tab)[MT] = s_tab_all[wib];
     // wavefront task = (tile, offset group, tap share).  Workgroups are dealt round-robin to the 8 XCDs, each
     // with an L2 of its own: an XCD works on one part of the positions (tiles that are neighbours in space
-    // share its L2), block after block of one offset group, then the next group, then the next tap share.
-    // It keeps its part from tap share to tap share, whose corner rows are the same ones, and moves to another
-    // part with every offset group (measured: 7 % faster with 8 groups than keeping the part).
+    // share its L2).  Its sequence of workgroups: the tap shares of a block of tiles one after the other (their
+    // corner rows are the same ones), then the next block of the part, and only then the next offset group, with
+    // another part (measured at 8 groups, C=512: 0.65 -> 0.57 ms against tap shares outermost, where the rows of
+    // a block were long gone from L2 when its next share came round).  Groups are taken last to first: the
+    // grad-column rows of the last groups are the ones the kernel in front wrote last, and what the memory-side
+    // cache still holds of them is read first (0.590 -> 0.576 ms).
     const int nblk = (a.ntile + kWavesPerBlock - 1) / kWavesPerBlock, nblk_p = (nblk + 7) / 8;
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    const int g = (idx / nblk_p) % s.G, share = idx / (nblk_p * s.G);
-    const int blk = ((xcd + 3 * g) & 7) * nblk_p + idx % nblk_p;
+    const int share = idx % a.nshare, g = s.G - 1 - idx / (nblk_p * a.nshare);
+    const int blk = ((xcd + 3 * g) & 7) * nblk_p + (idx / a.nshare) % nblk_p;
     if (blk >= nblk) return;
     const int tile = blk * kWavesPerBlock + wib;
     if (tile >= a.ntile) return;

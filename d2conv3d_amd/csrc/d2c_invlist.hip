@@ -160,10 +160,17 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
     const int sub = threadIdx.x & 7, ci = threadIdx.x >> 3;       // 32 cubes per workgroup: 2 x 4 x 4 of them
-    const int cidx = blockIdx.y;                                  // channel chunk
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const int nbx = (ncx + 3) / 4, nby = (ncy + 3) / 4, nbz = (ncz + 1) / 2;
-    int blk = xcd_swizzle(blockIdx.x, gridDim.x);
+    // Workgroups are dealt round-robin to the 8 XCDs.  An XCD takes a contiguous range of the blocks of cubes
+    // (neighbours in space share bins and grad-column rows in its L2) and, block by block, the channel chunks one
+    // after the other: the chunks of one offset group walk the same lists, which then come from L2.
+    const int nblk = s.N * nbz * nby * nbx, nch = s.Cin / BKC;
+    const int xcd = blockIdx.x & 7, uidx = blockIdx.x >> 3;
+    const int bq = nblk >> 3, br = nblk & 7;
+    const int cidx = uidx % nch, bi = uidx / nch;                 // channel chunk, block within the XCD's range
+    if (bi >= bq + (xcd < br ? 1 : 0)) return;
+    int blk = xcd * bq + (xcd < br ? xcd : br) + bi;
     const int bx = blk % nbx; blk /= nbx;
     const int by = blk % nby; blk /= nby;
     const int bz = blk % nbz;
@@ -544,7 +551,7 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists
     D2cProfScope prof(D2C_PROF_GX_OWNER, st);
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
-    dim3 grid((unsigned)nblk, s.Cin / BKC);
+    dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * (s.Cin / BKC)));    // see the kernel's unit mapping
     if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
     else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
     if (int rc = d2c_check_launch("gx_owner_kernel")) return rc;
