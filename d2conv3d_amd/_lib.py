@@ -18,7 +18,7 @@ ALGO_NAMES = {ALGO_GENERIC: "generic", ALGO_MFMA: "mfma", ALGO_DEPTHWISE: "depth
 EXPORTS = (
     "d2c_output_size", "d2c_conv3d_check", "d2c_conv3d_algo",
     "d2c_conv3d_forward_workspace_bytes", "d2c_conv3d_backward_workspace_bytes",
-    "d2c_conv3d_forward", "d2c_conv3d_backward",
+    "d2c_conv3d_forward", "d2c_conv3d_backward", "d2c_conv3d_forward_static", "d2c_static_workspace_bytes",
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
@@ -96,6 +96,8 @@ def load():
         f = getattr(lib, f"d2c_{name}_backward")
         f.argtypes, f.restype = [p] + [vp] * 11 + [sz, vp], ctypes.c_int
     lib.d2c_conv3d_algo.argtypes, lib.d2c_conv3d_algo.restype = [p3], ctypes.c_int
+    lib.d2c_conv3d_forward_static.argtypes, lib.d2c_conv3d_forward_static.restype = [p3] + [vp] * 7, ctypes.c_int
+    lib.d2c_static_workspace_bytes.argtypes, lib.d2c_static_workspace_bytes.restype = [], sz
     lib.d2c_conv1d_algo.argtypes, lib.d2c_conv1d_algo.restype = [p1], ctypes.c_int
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int

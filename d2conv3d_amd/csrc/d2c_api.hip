@@ -8,6 +8,12 @@
 #include <mutex>
 #include <vector>
 
+// Workspace of d2c_conv3d_forward_static: a device array that is part of the library's image, so the call that
+// uses it asks the runtime for no memory.  Every GPU the library runs on holds its own copy (at its own
+// address) until the process ends.  In host code the name is only a handle for hipGetSymbolAddress; the
+// address that kernels and copies get is the one looked up per device below.
+static __device__ __align__(256) unsigned char scratch[D2C_STATIC_WORKSPACE_BYTES];
+
 namespace {
 thread_local char g_err[512] = "";
 std::atomic<uint64_t> g_max_intermediate{1ull << 32};  // dconv3d_gpu.cu:12
@@ -27,6 +33,32 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n)
 {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
         p[i] = 0u;
+}
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Address of the current device's copy of `scratch` (looked up once per device, with that device current).
+int static_scratch(void **out)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        d2c_set_error("hipGetDevice failed or device index out of range");
+        return D2C_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            d2c_set_error("hipGetSymbolAddress(static workspace) on device %d: %s", dev, hipGetErrorString(e));
+            return D2C_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return D2C_OK;
 }
 }  // namespace
 
@@ -288,6 +320,29 @@ int d2c_conv3d_forward(const d2c_conv3d_desc *q, const void *x, const void *offs
     hipStream_t st = (hipStream_t)stream;
     if (a == D2C_ALGO_GENERIC) return d2c_generic_conv3d_forward(*q, x, offset, mask, weight, bias, out, st);
     if (int rc = check_ws(d2c_tiled_forward_ws(*q), ws, ws_bytes)) return rc;
+    return d2c_tiled_forward(*q, x, offset, mask, weight, bias, out, ws, st);
+}
+
+size_t d2c_static_workspace_bytes(void) { return (size_t)D2C_STATIC_WORKSPACE_BYTES; }
+
+int d2c_conv3d_forward_static(const d2c_conv3d_desc *q, const void *x, const void *offset, const void *mask,
+                              const void *weight, const void *bias, void *out, void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!x || !offset || !weight || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    const int a = choose_algo(*q, false);
+    if (a < 0) return D2C_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (a == D2C_ALGO_GENERIC) return d2c_generic_conv3d_forward(*q, x, offset, mask, weight, bias, out, st);
+    const size_t need = d2c_tiled_forward_ws(*q);
+    if (need > (size_t)D2C_STATIC_WORKSPACE_BYTES) {
+        d2c_set_error("d2c_conv3d_forward_static: this description needs %zu bytes of workspace, the static one holds "
+                      "%zu; use d2c_conv3d_forward with a caller-provided workspace",
+                      need, (size_t)D2C_STATIC_WORKSPACE_BYTES);
+        return D2C_ERR_WORKSPACE;
+    }
+    void *ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
     return d2c_tiled_forward(*q, x, offset, mask, weight, bias, out, ws, st);
 }
 

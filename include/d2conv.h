@@ -105,6 +105,23 @@ int d2c_conv3d_forward(const d2c_conv3d_desc *desc, const void *x, const void *o
                        const void *mask, const void *weight, const void *bias, void *out,
                        void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * d2c_conv3d_forward without a workspace argument and without any allocation.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory around the call: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The scratch memory is an array of
+ * D2C_STATIC_WORKSPACE_BYTES inside the library's device image (each GPU the library runs on holds its own
+ * copy until the process ends); the call makes no hipMalloc / hipFree and uses no allocating library routine.
+ * A description whose d2c_conv3d_forward_workspace_bytes() exceeds that size is refused with
+ * D2C_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (different streams or threads) race; serialise them.  Otherwise identical to d2c_conv3d_forward
+ * (same kernels, same results).  Instrumentation (d2c_profile_enable) must be off: it creates events.
+ */
+#define D2C_STATIC_WORKSPACE_BYTES (32u << 20)
+size_t d2c_static_workspace_bytes(void);
+int d2c_conv3d_forward_static(const d2c_conv3d_desc *desc, const void *x, const void *offset,
+                              const void *mask, const void *weight, const void *bias, void *out,
+                              void *stream);
+
 int d2c_conv3d_backward(const d2c_conv3d_desc *desc, const void *grad_out, const void *x,
                         const void *offset, const void *mask, const void *weight,
                         void *grad_x, void *grad_offset, void *grad_mask, void *grad_weight,
