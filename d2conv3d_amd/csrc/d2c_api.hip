@@ -257,6 +257,7 @@ int d2c_conv1d_check(const d2c_conv1d_desc *q)
     D2C_REQUIRE(lo > 0, "computed output size %d must be positive", lo);
     D2C_REQUIRE(q->Lo == lo, "offset output dims do not match computed dims. Got: %d but expected: %d", q->Lo, lo);
     D2C_REQUIRE((long)q->N * q->Cin * q->L < (1L << 31) && (long)q->N * q->Cout * lo < (1L << 31)
+                    && (long)q->N * q->offset_groups * q->k * lo < (1L << 31)
                     && (long)q->Cout * (q->Cin / q->groups) * q->k < (1L << 31),
                 "tensor with 2^31 or more elements is not supported");
     return D2C_OK;

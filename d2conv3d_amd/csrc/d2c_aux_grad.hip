@@ -14,7 +14,8 @@
 //
 // One wavefront = 64 output positions of one offset group and a share of the
 // taps.  Per tap: lane = position computes the corner table of the 64 positions
-// into a private LDS patch; then, per channel chunk of the group, 8 rounds of
+// (kept in registers, read across lanes with ds_bpermute: no LDS is allocated);
+// then, per channel chunk of the group, 8 rounds of
 // lane = (position, 16-byte vector): 8 corner vectors + 1 grad-column vector ->
 // 8 dot products -> the 4 results (linear in the dots) -> sum over the 8 lanes
 // of the position.
@@ -62,12 +63,16 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 {
     constexpr int MT = kMT;
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
-    __shared__ float s_tab_all[kWavesPerBlock][kTab][MT];
-
     const TiledShape &s = a.s;
     const int lane = threadIdx.x & 63;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    float (*s_tab)[MT] = s_tab_all[wib];
+    // The corner table of the 64 positions of a tap lives in registers (lane = position) and is read by the
+    // lanes of the dot-product role with ds_bpermute: the kernel allocates no LDS, so its workgroups fit on a
+    // compute unit next to a kernel that fills the LDS.
+    float tab[kTab];
+    auto tab_of = [&](int i, int pos) {
+        return __int_as_float(__builtin_amdgcn_ds_bpermute(pos << 2, __float_as_int(tab[i])));
+    };
     // wavefront task = (tile, offset group, tap share).  Workgroups are dealt round-robin to the 8 XCDs, each
     // with an L2 of its own: an XCD works on one part of the positions (tiles that are neighbours in space
     // share its L2).  Its sequence of workgroups: the tap shares of a block of tiles one after the other (their
@@ -162,15 +167,11 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                 }
                 flag |= (int)((inr << 8) | (auxlive << 24));
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the reads of the previous tap are done
-            __builtin_amdgcn_wave_barrier();
-            s_tab[0][lane] = __int_as_float(idx);
-            s_tab[1][lane] = __int_as_float(flag);
+            tab[0] = __int_as_float(idx);
+            tab[1] = __int_as_float(flag);
 #pragma unroll
-            for (int c = 0; c < 6; c++) s_tab[2 + c][lane] = fr[c];
-            s_tab[8][lane] = al;
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
+            for (int c = 0; c < 6; c++) tab[2 + c] = fr[c];
+            tab[8] = al;
             if (k + 1 < k_hi) coords_issue(k + 1);
         }
 
@@ -189,8 +190,8 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 #pragma unroll
                 for (int r = 0; r < kRounds; r++) {
                     const int pos = (rp * kRounds + r) * 8 + rpos;
-                    const int idx = __float_as_int(s_tab[0][pos]);
-                    const unsigned flag = (unsigned)__float_as_int(s_tab[1][pos]);
+                    const int idx = __float_as_int(tab_of(0, pos));
+                    const unsigned flag = (unsigned)__float_as_int(tab_of(1, pos));
                     const unsigned inr = (flag >> 8) & 0xffu;
                     const int qshift = (flag >> 16) & 1;
                     const int ib = idx + c0 + ivec * VEC;
@@ -207,7 +208,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 #pragma unroll
                 for (int r = 0; r < kRounds; r++) {
                     const int pos = (rp * kRounds + r) * 8 + rpos;
-                    const unsigned live = (unsigned)__float_as_int(s_tab[1][pos]) >> 24;
+                    const unsigned live = (unsigned)__float_as_int(tab_of(1, pos)) >> 24;
                     float dot[8];
                     if constexpr (sizeof(T) == 2) {
                         const bf16x2_t g0 = __builtin_bit_cast(bf16x2_t, gq[r].x), g1 = __builtin_bit_cast(bf16x2_t, gq[r].y);
@@ -229,8 +230,8 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                         }
                     }
                     // the four results are linear in the 8 dots: combine per lane, then sum over the 8 lanes
-                    const float lz = s_tab[2][pos], ly = s_tab[3][pos], lx = s_tab[4][pos];
-                    const float hz = s_tab[5][pos], hy = s_tab[6][pos], hx = s_tab[7][pos];
+                    const float lz = tab_of(2, pos), ly = tab_of(3, pos), lx = tab_of(4, pos);
+                    const float hz = tab_of(5, pos), hy = tab_of(6, pos), hx = tab_of(7, pos);
                     float gz = 0.f, gy = 0.f, gxx = 0.f, gm = 0.f;
 #pragma unroll
                     for (int c = 0; c < 8; c++) {
@@ -249,13 +250,17 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                 }
             }
             // ---- results of tap k for the positions of these rounds
+            // (every lane takes part in the exchange: a lane that is switched off supplies zeros)
+            float al_r[kRounds];
+#pragma unroll
+            for (int r = 0; r < kRounds; r++) al_r[r] = tab_of(8, (rp * kRounds + r) * 8 + rpos);
             if (ivec == 0) {
 #pragma unroll
                 for (int r = 0; r < kRounds; r++) {
                     const int pos = (rp * kRounds + r) * 8 + rpos;
                     const int m = m0 + pos;
                     if (m < s.M) {
-                        const float al = s_tab[8][pos];
+                        const float al = al_r[r];
                         const int b = m / s.P, p = m - b * s.P;
                         const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
                         if (a.goff && s.nd == 3) {
@@ -273,7 +278,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
         }
         if (lbin >= 0) {
             InvEntry e;
-            e.p = cp; e.k = k; e.hz = s_tab[5][lane]; e.hy = s_tab[6][lane]; e.hx = lhx; e.alpha = s_tab[8][lane];
+            e.p = cp; e.k = k; e.hz = tab[5]; e.hy = tab[6]; e.hx = lhx; e.alpha = tab[8];
             e.pad0 = 0; e.pad1 = 0;
             lists_store(a.lists, lbin, lslot, e);
         }
