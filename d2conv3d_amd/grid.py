@@ -109,6 +109,7 @@ class _SizeMapOffsets(torch.autograd.Function):
         return out
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, grad_out):
         import ctypes
         from . import _lib

@@ -16,8 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "..", ".."))
 sys.path.insert(0, os.path.join(HERE, ".."))
 
-from oracle import cpu, dwconv  # noqa: E402
-from d2conv3d_amd.grid import offsets_from_size_map  # noqa: E402
+from oracle import cpu, dwconv, sizemap  # noqa: E402
 
 CASES_3D = {
     # name: (N, Cin, Cout, dims, kernel, stride, padding, dilation, groups, offset groups, mask, bias, offset scale)
@@ -63,11 +62,14 @@ def case_1d():
                 geometry=np.array([s, p, d, groups, G]))
 
 
-def case_size_map():
-    g = torch.Generator().manual_seed(77)
-    size = torch.rand(2, 3, 2, 3, 4, generator=g, dtype=torch.float64) * 3.5 + 0.5
-    return dict(size=size, offsets=offsets_from_size_map(size, "xyz", (3, 3, 3), (1, 2, 1)),
-                geometry=np.array([3, 3, 3, 1, 2, 1]))
+def case_size_map(mode, channels, kernel, dilation, seed):
+    # from the numpy closed form of oracle/sizemap.py (pinned by tests/test_size_map_pins.py), not from the package
+    g = torch.Generator().manual_seed(seed)
+    size = torch.rand(2, channels, 2, 3, 4, generator=g, dtype=torch.float64) * 3.5 + 0.5
+    go = torch.randn(2, 3 * kernel[0] * kernel[1] * kernel[2], 2, 3, 4, generator=g, dtype=torch.float64)
+    return dict(size=size, offsets=sizemap.offsets(size.numpy(), mode, kernel, dilation), grad_offsets=go,
+                grad_size=sizemap.offsets_backward(go.numpy(), mode, kernel, dilation),
+                geometry=np.array([*kernel, *dilation]))
 
 
 def case_dwconv():
@@ -92,5 +94,8 @@ if __name__ == "__main__":
     for name in CASES_3D:
         save(name, case_3d(name))
     save("conv1d_groups", case_1d())
-    save("size_map_xyz", case_size_map())
+    save("size_map_xyz", case_size_map("xyz", 3, (3, 3, 3), (1, 2, 1), 77))
+    save("size_map_xxz", case_size_map("xxz", 2, (3, 5, 2), (1, 2, 1), 78))
+    save("size_map_xy", case_size_map("xy", 2, (3, 3, 3), (1, 1, 1), 79))
+    save("size_map_x", case_size_map("x", 1, (1, 3, 3), (1, 1, 2), 80))
     save("dwconv3d_multiplier2", case_dwconv())

@@ -50,9 +50,14 @@ def test_oracle_reproduces_conv1d():
 def test_size_map_and_plain_depthwise_fixtures_on_the_cpu():
     from d2conv3d_amd.grid import offsets_from_size_map
     from oracle import dwconv
-    c = load("size_map_xyz")
-    g = c["geometry"]
-    assert_close(offsets_from_size_map(c["size"], "xyz", tuple(g[0:3]), tuple(g[3:6])), c["offsets"], 0, 1e-12, "offsets")
+    for mode in ("xyz", "xxz", "xy", "x"):
+        c = load("size_map_" + mode)
+        g = c["geometry"]
+        size = c["size"].clone().requires_grad_(True)
+        off = offsets_from_size_map(size, mode, tuple(g[0:3]), tuple(g[3:6]))
+        assert_close(off, c["offsets"], 0, 1e-12, f"offsets ({mode})")
+        off.backward(c["grad_offsets"])
+        assert_close(size.grad, c["grad_size"], 0, 1e-12, f"grad_size ({mode})")
     c = load("dwconv3d_multiplier2")
     g = c["geometry"]
     s, p, d = tuple(g[0:3]), tuple(g[3:6]), tuple(g[6:9])
@@ -104,10 +109,14 @@ def test_gpu_matches_conv1d_fixture(dtype, dev):
 def test_gpu_matches_size_map_and_plain_depthwise_fixtures(dev):
     from d2conv3d_amd.depthwise_conv import depthwise_separable_conv3d
     from d2conv3d_amd.grid import size_map_offsets
-    c = load("size_map_xyz")
-    g = c["geometry"]
-    got = size_map_offsets(c["size"].float().to(dev), "xyz", tuple(g[0:3]), tuple(g[3:6]), "linear")
-    assert_close(got, c["offsets"], 1e-5, 1e-6, "offsets")
+    for mode in ("xyz", "xxz", "xy", "x"):
+        c = load("size_map_" + mode)
+        g = c["geometry"]
+        size = c["size"].float().to(dev).requires_grad_(True)
+        got = size_map_offsets(size, mode, tuple(g[0:3]), tuple(g[3:6]), "linear")
+        assert_close(got, c["offsets"], 1e-5, 1e-6, f"offsets ({mode})")
+        got.backward(c["grad_offsets"].float().to(dev))
+        assert_close(size.grad, c["grad_size"], 1e-5, 1e-5, f"grad_size ({mode})")
     c = load("dwconv3d_multiplier2")
     g = c["geometry"]
     s, p, d = tuple(g[0:3]), tuple(g[3:6]), tuple(g[6:9])

@@ -10,8 +10,12 @@ C5b included, size-independent properties are checked as well:
   adjoints:  <op(x), g> = <x, grad_input(g)> = <w, grad_weight(g)> (bias excluded), evaluated at g = op(x);
 * grad_bias = sum of grad_out.
 
-float32: 1e-4 relative / 1e-5 absolute, scaled by the tensor's magnitude for
-the long sums.  bfloat16: 2e-2 relative (L2 over the tensor).
+float32: the literal gate (1e-4 relative / 1e-5 absolute) against the float64
+oracle on the same values where float32 sums can meet it, else at most three
+times the float32 oracle's own excess over it (both figures are printed per
+tensor), and 1e-4 relative / 1e-5 absolute scaled by the tensor's magnitude
+against the float32 oracle.  bfloat16: 2e-2 relative, over the tensor (L2) and
+element-wise against the tensor's scale.
 """
 import os
 import sys
@@ -47,6 +51,13 @@ def _run(c, dev, x, off, m, w, b, gout=None):
     return out.detach(), [t.grad if t is not None else None for t in ts]
 
 
+def literal_gate_excess(actual, exact):
+    """max over the tensor of |actual - exact| / (1e-5 + 1e-4 |exact|): <= 1 means the literal float32 gate
+    (1e-4 relative / 1e-5 absolute, no scaling) holds against the float64 result."""
+    a, e = actual.detach().double().cpu(), exact.double()
+    return ((a - e).abs() / (1e-5 + 1e-4 * e.abs())).max().item()
+
+
 @pytest.mark.parametrize("name", ["c1", "c5a", "c4", "c2_f32", "c2_bf16", "c3"])
 def test_full_size_against_oracle(name, dev):
     c, x, off, m, w, b, gout = _tensors(name)
@@ -59,12 +70,54 @@ def test_full_size_against_oracle(name, dev):
     if c["backward"]:
         e = bwd(f(gout), f(x), f(off), f(m), f(w), True, 1, 1, 1, c["groups"], c["G"])
         pairs += [(n, g, ee) for n, g, ee in zip(names, grads, e)]
-    for n, a, ee in pairs:
+    exact = None
+    if c["dt"] == "f32":
+        # the same float32 values in float64 arithmetic: what both float32 computations approximate
+        dd = lambda t: t.double()
+        exact = [fwd(dd(x), dd(off), dd(m), dd(w), dd(b), 1, 1, 1, c["groups"], c["G"])]
+        if c["backward"]:
+            exact += list(bwd(dd(gout), dd(x), dd(off), dd(m), dd(w), True, 1, 1, 1, c["groups"], c["G"]))
+    for i, (n, a, ee) in enumerate(pairs):
         if c["dt"] == "f32":
+            # Literal gate first, against the float64 result.  Long float32 sums (the gradients of the large
+            # workloads add 10^4 - 10^5 terms) miss it whatever their order: where the float32 oracle, the
+            # reference's own summation order, misses it too, the kernels may miss it by at most three times as much.
+            hip, o32 = literal_gate_excess(a, exact[i]), literal_gate_excess(ee, exact[i])
+            print(f"literal 1e-4/1e-5 gate, {name} {n}: kernels {hip:.3g}, float32 oracle {o32:.3g} "
+                  f"(max |exact| {exact[i].abs().max().item():.3g})", flush=True)
+            assert hip <= max(1.0, 3.0 * o32), (name, n, hip, o32)
             scale = max(1.0, ee.abs().max().item())
             assert_close(a, ee, 1e-4, 1e-5 * scale, f"{name} {n}")
         else:
             assert rel_l2(a, ee) < 2e-2, (name, n, rel_l2(a, ee))
+            assert_close(a, ee, 2e-2, 2e-2 * ee.abs().max().item(), f"{name} {n}")
+
+
+def test_long_clip_backward_against_oracle(dev):
+    """The long-clip volume of workload c5b (32 x 60 x 108 = 207360 positions, bfloat16, one offset group) with
+    64 channels, which the oracle finishes in seconds: all five gradients, i.e. the grad-column rows, the offset /
+    mask gradient and the sample lists at the full number of positions."""
+    g = torch.Generator().manual_seed(1505)
+    N, C, dims = 1, 64, (32, 60, 108)
+    x = torch.randn(N, C, *dims, generator=g).bfloat16()
+    bound = 1.0 / (C * 27) ** 0.5
+    w = ((torch.rand(C, C, 3, 3, 3, generator=g) * 2 - 1) * bound).bfloat16()
+    b = ((torch.rand(C, generator=g) * 2 - 1) * bound).bfloat16()
+    off = torch.randn(N, 81, *dims, generator=g)
+    m = torch.sigmoid(torch.randn(N, 27, *dims, generator=g))
+    gout = torch.randn(N, C, *dims, generator=g).bfloat16()
+    ts = [t.to(dev).requires_grad_(True) for t in (x, off, m, w, b)]
+    from d2conv3d_amd import _ops
+    assert _ops.conv3d_algo(ts[0], ts[1], ts[2], ts[3], (1, 1, 1), (1, 1, 1), (1, 1, 1), 1, 1) == "mfma"
+    out = d2c.deform_conv3d(*ts, 1, 1, 1, 1, 1)
+    out.backward(gout.to(dev))
+    f = lambda t: t.float()
+    e_out = cpu.conv3d_forward(f(x), off, m, f(w), f(b), 1, 1, 1, 1, 1)
+    e = cpu.conv3d_backward(f(gout), f(x), off, m, f(w), True, 1, 1, 1, 1, 1)
+    for n, a, ee in [("out", out, e_out)] + list(zip(("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias"),
+                                                     [t.grad for t in ts], e)):
+        assert rel_l2(a, ee) < 2e-2, (n, rel_l2(a, ee))
+        assert_close(a, ee, 2e-2, 2e-2 * ee.abs().max().item(), n)
 
 
 @pytest.mark.parametrize("name", ["c2_bf16", "c3", "c4", "c5a", "c5b"])

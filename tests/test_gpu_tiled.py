@@ -21,6 +21,9 @@ SHAPES = {
     "c64_g1": (2, 64, 64, (4, 6, 7), 3, 1, 1, 1, 1, 1, True, True, 1.0),
     "c128_G2_o96": (1, 128, 96, (3, 6, 9), 3, 1, 1, 1, 1, 2, True, True, 2.0),
     "c128_groups2": (2, 128, 192, (3, 5, 6), 3, 1, 1, 1, 2, 2, False, True, 1.5),
+    # an offset group that spans both weight groups: the grad-column kernel cannot keep such a group on chip, the
+    # direct kernels compute grad_input / grad_offset / grad_mask beside the matrix-core grad_weight kernel
+    "c128_groups2_G1": (1, 128, 64, (3, 5, 6), 3, 1, 1, 1, 2, 1, True, True, 1.5),
     "c64_o320_nomask": (1, 64, 320, (3, 5, 5), 3, 1, 1, 1, 1, 1, True, False, 1.0),
     "c64_o600": (1, 64, 600, (2, 5, 5), (1, 3, 3), 1, (0, 1, 1), 1, 1, 1, True, True, 1.0),
     "c64_stride_dil": (2, 64, 64, (5, 9, 8), 3, (1, 2, 1), (1, 2, 2), (1, 2, 1), 1, 1, True, True, 1.0),
@@ -283,23 +286,35 @@ def _random_case(rng, depthwise):
         C = G * 4 * int(rng.integers(1, 70))
         return N, C, C, dims, k, s, p, d, C, G, bool(rng.integers(2)), bool(rng.integers(2)), float(pick(0.5, 1.5, 3.0))
     groups = pick(1, 1, 2)
-    G = groups * pick(1, 2)
-    Cin = 64 * G * pick(1, 2) if groups == 1 else 64 * G
-    Cout = G * int(rng.integers(1, 300 // G + 1))      # a multiple of groups and of the offset groups
+    G = pick(1, groups, 2 * groups)                    # fewer, as many or more offset groups than weight groups
+    unit = 64 * max(G, groups)                         # channels per weight group and per offset group: multiples of 64
+    Cin = unit * pick(1, 2) if groups == 1 else unit
+    m = G * groups // (2 if G % 2 == 0 and groups % 2 == 0 else 1)   # Cout: a multiple of groups and of the offset groups
+    Cout = m * int(rng.integers(1, 300 // m + 1))
     return N, Cin, Cout, dims, k, s, p, d, groups, G, bool(rng.integers(2)), bool(rng.integers(2)), float(pick(0.5, 1.5, 3.0))
+
+
+def _check_against_oracle(res, exp, dtype, shape, family):
+    """Forward value and gradients of one kernel family against the oracle's: float32 1e-4 relative / 1e-5
+    absolute (the absolute part scaled by the tensor's magnitude: the gradients are long sums), bfloat16 2e-2 of
+    the tensor's scale."""
+    for i, (a, e) in enumerate(zip(res, exp)):
+        scale = max(1.0, e.abs().max().item())
+        err = (a.cpu().float() - e).abs()
+        bound = (1e-5 * scale + 1e-4 * e.abs()) if dtype == torch.float32 else torch.full_like(e, 2e-2 * scale)
+        assert bool((err <= bound).all()), (shape, family, i, err.max().item(), scale)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("depthwise", [False, True])
-def test_random_geometries_against_the_direct_kernels(depthwise, dtype, dev):
-    """Seeded random shapes, strides, paddings, dilations, groups and offset scales: the matrix-core / channel-separated
-    kernels against the direct kernels (one thread per element, checked against the oracle on the reference's test
-    matrix in test_gpu_reference_matrix.py) on the same tensors, forward and all gradients.  D2C_RANDOM_CASES in the
-    environment widens the sweep (10 by default); each case is printed before it runs."""
+def test_random_geometries_against_the_oracle(depthwise, dtype, dev):
+    """Seeded random shapes, strides, paddings, dilations, weight / offset groups and offset scales: the matrix-core
+    / channel-separated kernels AND the direct kernels (one thread per element), each against the CPU oracle on
+    the same tensors, forward and all gradients.  D2C_RANDOM_CASES in the environment widens the sweep (10 by
+    default); each case is printed before it runs."""
     import os
     import numpy as np
     rng = np.random.default_rng(20240 + int(depthwise))
-    tol = 1e-4 if dtype == torch.float32 else 2e-2
     for case in range(int(os.environ.get("D2C_RANDOM_CASES", "10"))):
         shape = _random_case(rng, depthwise)
         print(f"random case {case} depthwise={depthwise} {dtype}: {shape}", flush=True)
@@ -308,7 +323,9 @@ def test_random_geometries_against_the_direct_kernels(depthwise, dtype, dev):
             (x, off, m, w, b), gout, (s, p, d, groups, G) = make("_random", dtype, seed=100 + case)
         finally:
             del SHAPES["_random"]
-        res = []
+        e_out = cpu.conv3d_forward(f32(x), off, m, f32(w), f32(b), s, p, d, groups, G)
+        eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+        exp = [e_out] + [e for e in eg if e is not None]
         for family in (None, "generic"):
             ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
             _ops.set_algo_override(family)
@@ -320,22 +337,19 @@ def test_random_geometries_against_the_direct_kernels(depthwise, dtype, dev):
                 out.backward(gout.to(dev))
             finally:
                 _ops.set_algo_override(None)
-            res.append([out.detach().float()] + [t.grad.float() for t in ts if t is not None])
-        for a, e in zip(*res):
-            scale = max(1.0, e.abs().max().item())
-            assert (a - e).abs().max().item() <= tol * scale, (shape, (a - e).abs().max().item(), scale)
+            res = [out.detach().float()] + [t.grad.float() for t in ts if t is not None]
+            _check_against_oracle(res, exp, dtype, shape, family or "tiled")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_random_geometries_1d_against_the_direct_kernels(dtype, dev):
+def test_random_geometries_1d_against_the_oracle(dtype, dev):
     """The 1-D operator on seeded random lengths, kernel sizes, strides, paddings, dilations and groups: matrix-core
-    kernels against the direct kernels on the same tensors, forward and all gradients (D2C_RANDOM_CASES widens
-    the sweep)."""
+    kernels and direct kernels, each against the CPU oracle on the same tensors, forward and all gradients
+    (D2C_RANDOM_CASES widens the sweep)."""
     import os
     import numpy as np
     rng = np.random.default_rng(777)
     pick = lambda *v: v[int(rng.integers(len(v)))]
-    tol = 1e-4 if dtype == torch.float32 else 2e-2
     for case in range(int(os.environ.get("D2C_RANDOM_CASES", "10"))):
         k, st, d = pick(1, 2, 3, 5), pick(1, 1, 2, 3), pick(1, 1, 2, 3)
         pad = int(rng.integers(0, 4))
@@ -352,7 +366,9 @@ def test_random_geometries_1d_against_the_direct_kernels(dtype, dev):
             (x, off, m, w, b), gout, (s, p, d, groups, G) = make1d("_random", dtype, seed=300 + case)
         finally:
             del SHAPES_1D["_random"]
-        res = []
+        e_out = cpu.conv1d_forward(f32(x), off, m, f32(w), f32(b), s, p, d, groups, G)
+        eg = cpu.conv1d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+        exp = [e_out] + [e for e in eg if e is not None]
         for family in (None, "generic"):
             ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
             _ops.set_algo_override(family)
@@ -363,7 +379,5 @@ def test_random_geometries_1d_against_the_direct_kernels(dtype, dev):
                 out.backward(gout.to(dev))
             finally:
                 _ops.set_algo_override(None)
-            res.append([out.detach().float()] + [t.grad.float() for t in ts if t is not None])
-        for a, e in zip(*res):
-            scale = max(1.0, e.abs().max().item())
-            assert (a - e).abs().max().item() <= tol * scale, (shape, (a - e).abs().max().item(), scale)
+            res = [out.detach().float()] + [t.grad.float() for t in ts if t is not None]
+            _check_against_oracle(res, exp, dtype, shape, family or "tiled")
