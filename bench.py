@@ -52,9 +52,10 @@ PEAK_GBS = 8000.0
 CPU_CROP = {"c5b": (1, (16, 60, 108))}
 
 
-def make_inputs(name, torch, crop=None):
+def make_inputs(name, torch, crop=None, want_size=False):
     """Seeded synthetic tensors of the workload (generated on the CPU so that the CPU leg and the GPU see the
-    same numbers).  `crop` = (N, dims) replaces the batch and spatial size for the CPU sample."""
+    same numbers).  `crop` = (N, dims) replaces the batch and spatial size for the CPU sample.  `want_size`
+    appends the dilation map that the offsets were expanded from (None for workloads with free offsets)."""
     from d2conv3d_amd.grid import offsets_from_size_map
     c = WORKLOADS[name]
     N, dims = (c["N"], c["dims"]) if crop is None else crop
@@ -66,6 +67,7 @@ def make_inputs(name, torch, crop=None):
     bound = 1.0 / (C // groups * K) ** 0.5
     w = (torch.rand(C, C // groups, *ks, generator=g) * 2 - 1) * bound
     b = (torch.rand(C, generator=g) * 2 - 1) * bound
+    size = None
     if c["off"][0] == "dilation":
         _, lo, hi = c["off"]
         size = torch.rand(N, 3, *dims, generator=g) * (hi - lo) + lo
@@ -74,7 +76,7 @@ def make_inputs(name, torch, crop=None):
         off = torch.randn(N, G * nd * K, *dims, generator=g) * c["off"][1]
     m = torch.sigmoid(torch.randn(N, G * K, *dims, generator=g))
     gout = torch.randn(N, C, *dims, generator=g)
-    return x, off, m, w, b, gout
+    return (x, off, m, w, b, gout, size) if want_size else (x, off, m, w, b, gout)
 
 
 def algorithmic(name, N=None, dims=None):
@@ -286,6 +288,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--expanded-offsets", action="store_true",
+                    help="dynamic-dilation workloads (c2_*): expand the dilation map to an offsets tensor first "
+                         "and time the ordinary operator on it, instead of handing the map to the operator")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this operator path is measured on ONE GPU only (--gpus 1); "
@@ -306,10 +311,18 @@ def main():
     name = args.workload
     c = WORKLOADS[name]
     N, C, dims, G, groups, dt, nd = c["N"], c["C"], c["dims"], c["G"], c["groups"], c["dt"], c["nd"]
-    x, off, m, w, b, gout = make_inputs(name, torch)
+    x, off, m, w, b, gout, size = make_inputs(name, torch, want_size=True)
     tdt = torch.bfloat16 if dt == "bf16" else torch.float32
     x, w, b, gout, off, m = (t.to(dev, tdt).contiguous() for t in (x, w, b, gout, off, m))
     code = _lib.D2C_BF16 if dt == "bf16" else _lib.D2C_F32
+    # Dynamic-dilation workloads hand the dilation map itself to the operator (d2c_conv3d_sized_*: the sampler
+    # forms the tap offsets, no [N, 81, ...] tensor exists) unless --expanded-offsets asks for the two-step form.
+    sized = size is not None and not args.expanded_offsets
+    if sized:
+        from d2conv3d_amd.grid import size_map_desc
+        size = size.to(dev, tdt).contiguous()
+        sdesc = size_map_desc(size, "xyz", (3, 3, 3), (1, 1, 1), "linear")
+        gsize = torch.empty_like(size)
     if nd == 3:
         T_, H_, W_ = dims
         desc = _lib.Conv3dDesc(N, C, C, T_, H_, W_, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, groups, G, T_, H_, W_,
@@ -332,10 +345,24 @@ def main():
     cur = [ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)]   # the stream the library launches on
     p = lambda t: ctypes.c_void_p(t.data_ptr())
 
+    if sized:
+        nf = lib.d2c_conv3d_sized_forward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+        nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+        ws = torch.empty(max(nf, nb, 256), dtype=torch.uint8, device=dev)
+
     def forward():
+        if sized:
+            _lib.check(lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), p(x), p(size), p(m), p(w),
+                                                    p(b), p(out), p(ws), nf, cur[0]), "forward")
+            return
         _lib.check(f_fwd(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, cur[0]), "forward")
 
     def backward():
+        if sized:
+            _lib.check(lib.d2c_conv3d_sized_backward(ctypes.byref(desc), ctypes.byref(sdesc), p(gout), p(x), p(size),
+                                                     p(m), p(w), p(gx), p(gsize), p(gm), p(gw), p(gb), p(ws), nb,
+                                                     cur[0]), "backward")
+            return
         _lib.check(f_bwd(ctypes.byref(desc), p(gout), p(x), p(off), p(m), p(w), p(gx), p(goff), p(gm), p(gw), p(gb),
                          p(ws), nb, cur[0]), "backward")
 
@@ -465,6 +492,8 @@ def main():
         "config": {"workload": f"{name}: {what}, N={N}, Cin=Cout={C}, {'x'.join(map(str, dims))}, k3 p1, "
                                f"groups={groups}, offset_groups={G}, bias, "
                                + ("bf16 in / fp32 accumulate" if dt == "bf16" else "fp32"),
+                   "offsets": ("formed in the sampler from the dilation map [N,3,T,H,W] (d2c_conv3d_sized_*)" if sized
+                               else "offsets tensor [N,3*K*G,T,H,W]"),
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "taps_outside_volume": taps,

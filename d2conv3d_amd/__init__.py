@@ -3,7 +3,7 @@ dynamic-dilation conv3d and deformable conv1d, forward and backward, as
 hand-written HIP kernels for gfx950 behind the Python surface of the
 reference's `dconv_native` package (ops/dconv-native/src/dconv_native).
 """
-from .deform_conv import deform_conv1d, deform_conv3d
+from .deform_conv import deform_conv1d, deform_conv3d, deform_conv3d_sized
 from .deform_conv import DeformConv1d, DeformConv3d, DeformConvNd
 from .modules import (
     DConv3d, MDConv3d, SpatialDConv3d, SpatialMDConv3d, TemporalDConv3d, TemporalMDConv3d,
@@ -17,7 +17,7 @@ from .util import add_deformable_conv
 from .depthwise_conv import DepthwiseConv3d, depthwise_separable_conv3d, install_as_fast_depthwise_conv3d
 
 __all__ = [
-    "deform_conv1d", "deform_conv3d", "DeformConv1d", "DeformConv3d", "DeformConvNd",
+    "deform_conv1d", "deform_conv3d", "deform_conv3d_sized", "DeformConv1d", "DeformConv3d", "DeformConvNd",
     "DConv3d", "MDConv3d", "SpatialDConv3d", "SpatialMDConv3d", "TemporalDConv3d", "TemporalMDConv3d",
     "SizeConditionedDConv3d", "SizeConditionedMDConv3d",
     "XYSizeConditionedDConv3d", "XYSizeConditionedMDConv3d",

@@ -25,6 +25,8 @@ EXPORTS = (
     "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_last_error", "d2c_version",
     "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read",
     "d2c_size_map_offsets_forward", "d2c_size_map_offsets_backward",
+    "d2c_conv3d_sized_forward_workspace_bytes", "d2c_conv3d_sized_backward_workspace_bytes",
+    "d2c_conv3d_sized_forward", "d2c_conv3d_sized_backward",
     "d2c_dwconv3d_check", "d2c_dwconv3d_backward_workspace_bytes", "d2c_dwconv3d_forward", "d2c_dwconv3d_backward",
 )
 
@@ -105,6 +107,11 @@ def load():
     psm = ctypes.POINTER(SizeMapDesc)
     lib.d2c_size_map_offsets_forward.argtypes, lib.d2c_size_map_offsets_forward.restype = [psm, vp, vp, vp], ctypes.c_int
     lib.d2c_size_map_offsets_backward.argtypes, lib.d2c_size_map_offsets_backward.restype = [psm, vp, vp, vp, vp], ctypes.c_int
+    for d in ("forward", "backward"):
+        f = getattr(lib, f"d2c_conv3d_sized_{d}_workspace_bytes")
+        f.argtypes, f.restype = [p3, psm], sz
+    lib.d2c_conv3d_sized_forward.argtypes, lib.d2c_conv3d_sized_forward.restype = [p3, psm] + [vp] * 7 + [sz, vp], ctypes.c_int
+    lib.d2c_conv3d_sized_backward.argtypes, lib.d2c_conv3d_sized_backward.restype = [p3, psm] + [vp] * 11 + [sz, vp], ctypes.c_int
     pdw = ctypes.POINTER(DwConv3dDesc)
     lib.d2c_dwconv3d_check.argtypes, lib.d2c_dwconv3d_check.restype = [pdw], ctypes.c_int
     lib.d2c_dwconv3d_backward_workspace_bytes.argtypes = [pdw]

@@ -158,6 +158,89 @@ def deform_conv3d(input, offset, alpha, weight, bias, stride_d, stride_h, stride
         int(groups), int(offset_groups), float(relu_scale))
 
 
+class _DeformConv3dSizedFunction(torch.autograd.Function):
+    """The deformable convolution of the size-conditioned layers (network/layers.py:184-313) with the predicted size
+    map as its input: size activation, expansion to tap offsets (utils/grid.py:72-98) and the operator itself in
+    d2c_conv3d_sized_forward / _backward.  No offsets tensor and no gradient of one exist where the matrix-core
+    kernels serve the call."""
+
+    @staticmethod
+    def forward(ctx, input, size_raw, alpha, weight, bias, mode, activation, stride, padding, dilation, groups,
+                relu_scale=0.0):
+        from .grid import size_map_desc
+        lib = _lib.load()
+        input, size_raw, weight = input.contiguous(), size_raw.contiguous(), weight.contiguous()
+        alpha = alpha.contiguous() if alpha is not None else None
+        bias = bias.contiguous() if bias is not None else None
+        N, Cin, D, H, W = input.shape
+        Cout, _, kd, kh, kw = weight.shape
+        Do, Ho, Wo = size_raw.shape[2:]
+        desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, *stride, *padding, *dilation, groups, 1, Do, Ho, Wo,
+                               _DT[input.dtype], _DT[size_raw.dtype],
+                               _lib.EPILOGUE_RELU if relu_scale > 0 else _lib.EPILOGUE_NONE, float(relu_scale) or 1.0)
+        sdesc = size_map_desc(size_raw, mode, (kd, kh, kw), dilation, activation)
+        _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d_sized")
+        dev = input.device
+        out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
+        with torch.cuda.device(dev):
+            nb = lib.d2c_conv3d_sized_forward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+            ws = _workspace(nb, dev)
+            rc = lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input), _ptr(size_raw),
+                                              _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
+        _lib.check(rc, "deform_conv3d_sized forward")
+        ctx.save_for_backward(input, size_raw, alpha, weight, bias, out if relu_scale > 0 else None)
+        ctx.desc, ctx.sdesc = desc, sdesc
+        ctx.relu_scale = float(relu_scale)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        lib = _lib.load()
+        input, size_raw, alpha, weight, bias, out = ctx.saved_tensors
+        desc, sdesc = ctx.desc, ctx.sdesc
+        dev = input.device
+        grad_out = grad_out.contiguous().to(input.dtype)
+        if out is not None:    # gradient with respect to the value before the fused activation
+            grad_out = torch.where(out > 0, grad_out * ctx.relu_scale, torch.zeros_like(grad_out))
+        need = ctx.needs_input_grad
+        gx = torch.empty_like(input) if need[0] else None
+        gsize = torch.empty_like(size_raw) if need[1] else None
+        galpha = torch.empty_like(alpha) if (alpha is not None and need[2]) else None
+        gw = torch.empty_like(weight) if need[3] else None
+        gb = torch.empty_like(bias) if (bias is not None and need[4]) else None
+        with torch.cuda.device(dev):
+            nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+            ws = _workspace(nb, dev)
+            rc = lib.d2c_conv3d_sized_backward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(grad_out), _ptr(input),
+                                               _ptr(size_raw), _ptr(alpha), _ptr(weight), _ptr(gx), _ptr(gsize),
+                                               _ptr(galpha), _ptr(gw), _ptr(gb), _ptr(ws), nb, _stream(dev))
+        _lib.check(rc, "deform_conv3d_sized backward")
+        return (gx, gsize, galpha, gw, gb) + (None,) * 7
+
+
+def deform_conv3d_sized(input, size_raw, alpha, weight, bias, mode, activation, stride, padding, dilation, groups=1,
+                        relu_scale=0.0):
+    """Deformable convolution whose tap offsets follow from a predicted size map:
+    deform_conv3d(input, offsets_from_size_map(size_activation(size_raw), mode, kernel, dilation), alpha, ...)
+    of network/layers.py:184-313 as one operator.  `size_raw` [N, 3|2|2|1, Do, Ho, Wo] for mode xyz|xxz|xy|x."""
+    from torch.nn.modules.utils import _triple
+    stride, padding, dilation = (tuple(int(v) for v in _triple(t)) for t in (stride, padding, dilation))
+    mode = mode.lower()
+    want_c = {"xyz": 3, "xxz": 2, "xy": 2, "x": 1}[mode]
+    K = weight.shape[2] * weight.shape[3] * weight.shape[4]
+    if size_raw.dim() != 5 or size_raw.shape[1] != want_c:
+        raise RuntimeError(f"deform_conv3d_sized: mode '{mode}' wants {want_c} size channels, got {tuple(size_raw.shape)}")
+    if not size_raw.is_cuda or size_raw.device != input.device:
+        raise RuntimeError("deform_conv3d_sized: size_raw must be on the input's GPU")
+    # the operator's own checks, with (a view shaped like) the offsets tensor the size map stands for
+    stand_in = size_raw.new_empty(1).expand((size_raw.shape[0], 3 * K) + tuple(size_raw.shape[2:]))
+    _check_common(3, input, stand_in, alpha, weight, bias, groups, 1)
+    input, size_raw, alpha, weight, bias = _unify(input, size_raw, alpha, weight, bias)
+    return _DeformConv3dSizedFunction.apply(input, size_raw, alpha, weight, bias, mode, activation, stride, padding,
+                                            dilation, int(groups), float(relu_scale))
+
+
 class _DeformConv1dFunction(torch.autograd.Function):
     """DeformConv1dFunction of dconv1d.h:69-159."""
 

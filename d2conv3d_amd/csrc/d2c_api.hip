@@ -364,6 +364,89 @@ int d2c_conv3d_backward(const d2c_conv3d_desc *q, const void *gout, const void *
     return d2c_tiled_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws, st);
 }
 
+// ---- the operator fed by a size map (dynamic dilation) ----
+// Where the matrix-core kernels can form the offsets themselves the map goes straight to them; otherwise it is
+// expanded into the front of the workspace by d2c_size_map_offsets_forward and the ordinary call runs behind it
+// (and d2c_size_map_offsets_backward folds the offset gradient back).
+static int sized_check(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!z) { d2c_set_error("null size-map description"); return D2C_ERR_SHAPE; }
+    D2C_REQUIRE(q->offset_groups == 1, "a size map drives one offset group (3K offset channels), got offset_groups = %d",
+                q->offset_groups);
+    D2C_REQUIRE(z->N == q->N && z->P == q->Do * q->Ho * q->Wo && z->kd == q->kd && z->kh == q->kh && z->kw == q->kw,
+                "size-map description does not match the convolution (N, output positions, kernel extents)");
+    D2C_REQUIRE(q->kd <= D2C_SIZE_MAX_K && q->kh <= D2C_SIZE_MAX_K && q->kw <= D2C_SIZE_MAX_K,
+                "size map: kernel extents at most %d", D2C_SIZE_MAX_K);
+    D2C_REQUIRE(z->mode >= D2C_SIZE_XYZ && z->mode <= D2C_SIZE_X && z->activation >= D2C_SIZE_ACT_LINEAR
+                    && z->activation <= D2C_SIZE_ACT_RELU_PLUS_ONE, "size map: unknown mode or activation");
+    if (q->dtype == D2C_F64 || z->dtype != q->aux_dtype) {
+        d2c_set_error("size map: float32 or bfloat16 in the element type of the mask (aux_dtype)");
+        return D2C_ERR_DTYPE;
+    }
+    return D2C_OK;
+}
+static size_t expanded_offsets_bytes(const d2c_conv3d_desc &q)
+{
+    const size_t K = (size_t)q.kd * q.kh * q.kw, P = (size_t)q.Do * q.Ho * q.Wo;
+    return d2c_align_up((size_t)q.N * 3 * K * P * d2c_elem_size(q.aux_dtype));
+}
+static bool sized_fused(const d2c_conv3d_desc &q, bool backward)
+{
+    const int a = choose_algo(q, true);
+    return a == D2C_ALGO_MFMA && d2c_tiled_sized_supported(q, backward);
+}
+
+size_t d2c_conv3d_sized_forward_workspace_bytes(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
+{
+    if (sized_check(q, z) != D2C_OK) return 0;
+    if (sized_fused(*q, false)) return d2c_tiled_forward_ws(*q);
+    return expanded_offsets_bytes(*q) + d2c_conv3d_forward_workspace_bytes(q);
+}
+
+size_t d2c_conv3d_sized_backward_workspace_bytes(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
+{
+    if (sized_check(q, z) != D2C_OK) return 0;
+    if (sized_fused(*q, true)) return d2c_tiled_backward_ws(*q, z);
+    return 2 * expanded_offsets_bytes(*q) + d2c_conv3d_backward_workspace_bytes(q);
+}
+
+int d2c_conv3d_sized_forward(const d2c_conv3d_desc *q, const d2c_size_map_desc *z, const void *x, const void *size_raw,
+                             const void *mask, const void *weight, const void *bias, void *out, void *ws,
+                             size_t ws_bytes, void *stream)
+{
+    if (int rc = sized_check(q, z)) return rc;
+    if (!x || !size_raw || !weight || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (choose_algo(*q, false) < 0) return D2C_ERR_UNSUPPORTED;
+    if (int rc = check_ws(d2c_conv3d_sized_forward_workspace_bytes(q, z), ws, ws_bytes)) return rc;
+    if (sized_fused(*q, false))
+        return d2c_tiled_forward(*q, x, size_raw, mask, weight, bias, out, ws, (hipStream_t)stream, z);
+    const size_t ob = expanded_offsets_bytes(*q);
+    if (int rc = d2c_size_map_offsets_forward(z, size_raw, ws, stream)) return rc;
+    return d2c_conv3d_forward(q, x, ws, mask, weight, bias, out, (char *)ws + ob, ws_bytes - ob, stream);
+}
+
+int d2c_conv3d_sized_backward(const d2c_conv3d_desc *q, const d2c_size_map_desc *z, const void *gout, const void *x,
+                              const void *size_raw, const void *mask, const void *weight, void *gx, void *gsize,
+                              void *gmask, void *gw, void *gb, void *ws, size_t ws_bytes, void *stream)
+{
+    if (int rc = sized_check(q, z)) return rc;
+    if (!gout || !x || !size_raw || !weight) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (choose_algo(*q, false) < 0) return D2C_ERR_UNSUPPORTED;
+    if (int rc = check_ws(d2c_conv3d_sized_backward_workspace_bytes(q, z), ws, ws_bytes)) return rc;
+    if (sized_fused(*q, true))
+        return d2c_tiled_backward(*q, gout, x, size_raw, mask, weight, gx, gsize, gmask, gw, gb, ws,
+                                  (hipStream_t)stream, z);
+    const size_t ob = expanded_offsets_bytes(*q);
+    char *off = (char *)ws, *goff = off + ob;
+    if (int rc = d2c_size_map_offsets_forward(z, size_raw, off, stream)) return rc;
+    if (int rc = d2c_conv3d_backward(q, gout, x, off, mask, weight, gx, gsize ? goff : nullptr, gmask, gw, gb,
+                                     goff + ob, ws_bytes - 2 * ob, stream))
+        return rc;
+    if (gsize) return d2c_size_map_offsets_backward(z, size_raw, goff, gsize, stream);
+    return D2C_OK;
+}
+
 int d2c_conv3d_corner_index(const d2c_conv3d_desc *q, const void *offset, int32_t *base, uint8_t *flags,
                             void *stream)
 {

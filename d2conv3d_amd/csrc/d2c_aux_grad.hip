@@ -39,6 +39,7 @@ struct AuxArgs {
     const void *off, *mask;
     const void *gcol;    // [chunk][tap][N*P][BKC]
     void *goff, *gmask;  // or NULL
+    float *gsize;        // size-map source: fp32 sums [N][3][P] of d(loss)/d(size) per axis (zeroed), instead of goff
     int ntile;           // position tiles
     int nshare;          // tap shares
     SampleLists lists;   // counts != NULL: every live sample is filed in its bucket on the way (for grad_input)
@@ -111,14 +112,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     auto coords_issue = [&](int k) {
         if (cvalid) {
             const long ab = (((long)cb * s.G + g) * s.K + k) * s.P + cp;
-            if (s.nd == 3) {
-                const long ob = 3 * ab - 2 * (long)cp;
-                craw[0] = ld_auxT<AUX16>(a.off, ob);
-                craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
-                craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
-            } else {
-                craw[2] = ld_auxT<AUX16>(a.off, ab);
-            }
+            tap_offsets_issue<AUX16>(s, a.off, cb, g, k, cp, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
         }
     };
@@ -133,6 +127,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
             float al = 0.f;
             int idx = 0, flag = 0;
             if (cvalid) {
+                tap_offsets_finish<AUX16>(s, k, craw);
                 const float o0 = craw[0], o1 = craw[1], o2 = craw[2];
                 al = craw[3];
                 int bz, by, bx;
@@ -263,7 +258,16 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                         const float al = al_r[r];
                         const int b = m / s.P, p = m - b * s.P;
                         const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
-                        if (a.goff && s.nd == 3) {
+                        if (a.gsize) {
+                            // size-map source: d(offset_a) / d(size_a) = base_a[k_a]; the taps of a position add up
+                            // (fp32 atomics into [N][3][P], finished by size_grad_finish_kernel)
+                            const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
+#pragma unroll
+                            for (int ax = 0; ax < 3; ax++)
+                                if (axis_channel(s.ss.mode, ax) >= 0)
+                                    atomicAdd(a.gsize + ((long)b * 3 + ax) * s.P + p,
+                                              s.ss.base[ax][kq[ax]] * (al * g_acc[r][ax]));
+                        } else if (a.goff && s.nd == 3) {
                             const long ob = 3 * ab - 2 * (long)p;
                             st_aux(a.goff, ob, s.adt, al * g_acc[r][0]);
                             st_aux(a.goff, ob + s.P, s.adt, al * g_acc[r][1]);
@@ -295,7 +299,8 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
 {
     const int ntile = (s.M + kMT - 1) / kMT;
     const int nshare = s.K < kTapSplit ? s.K : kTapSplit;
-    AuxArgs a{s, xcl, off, mask, gcol, goff, gmask, ntile, nshare,
+    // (with the size-map source `goff` is the fp32 accumulator of the size gradient)
+    AuxArgs a{s, xcl, off, mask, gcol, s.ss.on ? nullptr : goff, gmask, s.ss.on ? (float *)goff : nullptr, ntile, nshare,
               lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}};
     dim3 grid((unsigned)(8 * (((ntile + kWavesPerBlock - 1) / kWavesPerBlock + 7) / 8) * s.G * nshare));
     bool aux16 = false;

@@ -12,6 +12,7 @@
 //   B: lane l holds col  n = l % 32, same k-slice
 //   D: lane l holds col  n = l % 32, rows m = 8*(r/4) + 4*(l/32) + r%4 for r = 0..15
 #pragma once
+#include <type_traits>
 #include "d2c_common.hpp"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -119,6 +120,84 @@ D2C_DEV void st_aux(void *p, long i, int adt, float v)
     else reinterpret_cast<bf16_t *>(p)[i] = f32_to_bf16(v);
 }
 
+// ---- tap offsets formed from a predicted size map (the dynamic-dilation layers) --------------------------------
+// When SizeSrc::on is set, the `off` argument of the tiled kernels is not the [N, 3K, P] offsets tensor but the raw
+// size prediction [N, channels(mode), P], and a tap's offsets are formed where they are needed:
+//     off_a = base_a[k_a] * (act(raw_a) - 1)      (network/layers.py:171-181, utils/grid.py:72-98)
+// with every intermediate rounded to the storage type, i.e. bit for bit what the expanding kernel of
+// d2c_sizemap.hip (and the torch formulation) would have stored.  One offset group only (the reference's
+// size-conditioned layers predict 3K offset channels, network/layers.py:184-313).
+struct SizeSrc {
+    int on;                               // 1: `off` is the raw map; 2: `off` is (size - 1) per axis, float [N][3][P],
+                                          //    made from the raw map by one small kernel in front (backward pass)
+    int mode, act;                        // D2C_SIZE_*, D2C_SIZE_ACT_*
+    float base[3][D2C_SIZE_MAX_K];        // kernel-grid axes z, y, x
+};
+
+// channel of the raw map that feeds axis a (0 z, 1 y, 2 x), or -1 for "size 1"
+D2C_DEV int axis_channel(int mode, int a)
+{
+    switch (mode) {
+    case D2C_SIZE_XYZ: return a;
+    case D2C_SIZE_XXZ: return a == 0 ? 0 : 1;
+    case D2C_SIZE_XY: return a == 0 ? -1 : a - 1;
+    default: return a == 0 ? -1 : 0;   // D2C_SIZE_X
+    }
+}
+__host__ __device__ inline int mode_channels(int mode) { return mode == D2C_SIZE_XYZ ? 3 : (mode == D2C_SIZE_X ? 1 : 2); }
+
+// value rounded to the storage type, as a tensor between two torch operations would be
+template <typename T> D2C_DEV float rnd(float v);
+template <> D2C_DEV float rnd<float>(float v) { return v; }
+template <> D2C_DEV float rnd<bf16_t>(float v)
+{
+    // (the hardware conversion, round to nearest even like f32_to_bf16: two instructions)
+    typedef float f32x2_ __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_ __attribute__((ext_vector_type(2)));
+    const f32x2_ t = {v, 0.f};
+    return __uint_as_float(__builtin_bit_cast(uint32_t, __builtin_convertvector(t, bf16x2_)) << 16);
+}
+
+// network/layers.py:171-181, operation by operation
+template <typename T> D2C_DEV float size_act(int act, float x)
+{
+    switch (act) {
+    case D2C_SIZE_ACT_ELU: return rnd<T>(rnd<T>(x > 0.f ? x : expf(x) - 1.f) + 1.f);
+    case D2C_SIZE_ACT_RELU: return fmaxf(rnd<T>(x + 1.f), 0.f);
+    case D2C_SIZE_ACT_RELU_PLUS_ONE: return rnd<T>(fmaxf(rnd<T>(x + 1e-3f), 0.f) + 1.f);
+    default: return x;
+    }
+}
+D2C_DEV float size_act_grad(int act, float x)
+{
+    switch (act) {
+    case D2C_SIZE_ACT_ELU: return x > 0.f ? 1.f : expf(x);
+    case D2C_SIZE_ACT_RELU: return x + 1.f > 0.f ? 1.f : 0.f;
+    case D2C_SIZE_ACT_RELU_PLUS_ONE: return x + 1e-3f > 0.f ? 1.f : 0.f;
+    default: return 1.f;
+    }
+}
+
+// Exact n / d for 0 <= n < 2^31 by a multiplication: with l = ceil(log2 d) and m = ceil(2^(31 + l) / d) (which
+// fits 32 bits), floor(m * n / 2^(31 + l)) = floor(n / d).  A 32-bit integer division costs ~35 vector
+// instructions, a 64-bit one well over a hundred: too much for code that runs once per (tile, tap).
+struct FastDiv {
+    unsigned m;
+    int sh;        // l - 1, or -1 for d == 1
+    int d;
+};
+inline FastDiv make_fastdiv(int d)
+{
+    FastDiv f{0u, -1, d};
+    if (d <= 1) return f;
+    int l = 0;
+    while ((1ll << l) < d) l++;
+    f.m = (unsigned)(((1ull << (31 + l)) + (unsigned long long)d - 1) / (unsigned long long)d);
+    f.sh = l - 1;
+    return f;
+}
+D2C_DEV int fdiv(int n, const FastDiv &f) { return f.sh < 0 ? n : (int)(__umulhi((unsigned)n, f.m) >> f.sh); }
+
 // Geometry of the tiled kernels.  Channels are walked in chunks of BKC = 8*VEC
 // (64 bf16 / 32 float): one chunk never straddles an offset group or a weight
 // group, so all of its channels share the 8 corner positions of a tap.
@@ -135,7 +214,62 @@ struct TiledShape {
     int act;              // forward epilogue: 0 none, 1 act_scale * max(v, 0)
     float act_scale;
     TapGeom geo;
+    SizeSrc ss;           // offsets formed from a size map instead of read from a tensor
+    FastDiv dP, dHW, dW;  // divisions by P, Ho * Wo and Wo
 };
+
+// The three values a sampling point needs, requested early (issue) and turned into offsets late (finish):
+// the offsets themselves, or the raw sizes of the position (0 for an axis the mode does not predict).
+template <bool AUX16>
+D2C_DEV void tap_offsets_issue(const TiledShape &s, const void *off, int b, int g, int k, int p, float *c)
+{
+    if (s.ss.on == 2) {
+        const float *f = reinterpret_cast<const float *>(off) + (long)b * 3 * s.P + p;
+        c[0] = f[0]; c[1] = f[s.P]; c[2] = f[2 * (long)s.P];
+        return;
+    }
+    if (s.ss.on) {
+        const int nc = mode_channels(s.ss.mode);
+#pragma unroll
+        for (int ax = 0; ax < 3; ax++) {
+            const int ch = axis_channel(s.ss.mode, ax);
+            c[ax] = ch < 0 ? 0.f : ld_auxT<AUX16>(off, ((long)b * nc + ch) * s.P + p);
+        }
+        return;
+    }
+    const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
+    if (s.nd == 3) {
+        const long ob = 3 * ab - 2 * (long)p;   // ((b*G+g)*K+k)*3*P + p
+        c[0] = ld_auxT<AUX16>(off, ob);
+        c[1] = ld_auxT<AUX16>(off, ob + s.P);
+        c[2] = ld_auxT<AUX16>(off, ob + 2 * (long)s.P);
+    } else {
+        c[0] = 0.f; c[1] = 0.f;
+        c[2] = ld_auxT<AUX16>(off, ab);
+    }
+}
+// size map: raw sizes of a position -> (size - 1) per axis, the part of a tap's offsets that all taps share
+template <bool AUX16> D2C_DEV void size_minus_one(const TiledShape &s, float *c)
+{
+    typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+#pragma unroll
+    for (int ax = 0; ax < 3; ax++)
+        c[ax] = axis_channel(s.ss.mode, ax) < 0 ? 0.f : rnd<AT>(size_act<AT>(s.ss.act, c[ax]) - 1.f);
+}
+// ... and from there the offsets of tap k
+template <bool AUX16> D2C_DEV void size_tap_offsets(const TiledShape &s, int k, const float *sm1, float *o)
+{
+    typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+    const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
+#pragma unroll
+    for (int ax = 0; ax < 3; ax++) o[ax] = rnd<AT>(rnd<AT>(s.ss.base[ax][kq[ax]]) * sm1[ax]);
+}
+template <bool AUX16> D2C_DEV void tap_offsets_finish(const TiledShape &s, int k, float *c)
+{
+    if (!s.ss.on) return;
+    if (s.ss.on == 1) size_minus_one<AUX16>(s, c);
+    size_tap_offsets<AUX16>(s, k, c, c);
+}
 
 // The forward kernels' last step before a value is stored (NaN stays NaN, as in torch's relu).
 __host__ __device__ inline float d2c_epilogue(float v, int act, float scale)
@@ -248,6 +382,18 @@ D2C_DEV void lists_insert(const SampleLists &L, int bin, InvEntry e) { lists_sto
 D2C_DEV void load_offsets(const TiledShape &s, const void *off, int b, int g, int k, int p, float &o0, float &o1,
                           float &o2)
 {
+    if (s.ss.on) {
+        float c[3];
+        if (s.adt == D2C_BF16) {
+            tap_offsets_issue<true>(s, off, b, g, k, p, c);
+            tap_offsets_finish<true>(s, k, c);
+        } else {
+            tap_offsets_issue<false>(s, off, b, g, k, p, c);
+            tap_offsets_finish<false>(s, k, c);
+        }
+        o0 = c[0]; o1 = c[1]; o2 = c[2];
+        return;
+    }
     if (s.nd == 3) {
         const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
         o0 = ld_aux(off, ob, s.adt);

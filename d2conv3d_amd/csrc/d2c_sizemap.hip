@@ -24,41 +24,6 @@ struct SizeMapArgs {
     void *graw;          // backward: [N][channels][P] out
 };
 
-// channel of the raw map that feeds axis a (0 z, 1 y, 2 x), or -1 for "size 1"
-D2C_DEV int axis_channel(int mode, int a)
-{
-    switch (mode) {
-    case D2C_SIZE_XYZ: return a;
-    case D2C_SIZE_XXZ: return a == 0 ? 0 : 1;
-    case D2C_SIZE_XY: return a == 0 ? -1 : a - 1;
-    default: return a == 0 ? -1 : 0;   // D2C_SIZE_X
-    }
-}
-D2C_DEV int mode_channels(int mode) { return mode == D2C_SIZE_XYZ ? 3 : (mode == D2C_SIZE_X ? 1 : 2); }
-
-// value rounded to the storage type, as a tensor between two torch operations would be
-template <typename T> D2C_DEV float rnd(float v) { return elem_to_f32<T>(f32_to_elem<T>(v)); }
-
-// network/layers.py:171-181, operation by operation
-template <typename T> D2C_DEV float size_act(int act, float x)
-{
-    switch (act) {
-    case D2C_SIZE_ACT_ELU: return rnd<T>(rnd<T>(x > 0.f ? x : expf(x) - 1.f) + 1.f);
-    case D2C_SIZE_ACT_RELU: return fmaxf(rnd<T>(x + 1.f), 0.f);
-    case D2C_SIZE_ACT_RELU_PLUS_ONE: return rnd<T>(fmaxf(rnd<T>(x + 1e-3f), 0.f) + 1.f);
-    default: return x;
-    }
-}
-D2C_DEV float size_act_grad(int act, float x)
-{
-    switch (act) {
-    case D2C_SIZE_ACT_ELU: return x > 0.f ? 1.f : expf(x);
-    case D2C_SIZE_ACT_RELU: return x + 1.f > 0.f ? 1.f : 0.f;
-    case D2C_SIZE_ACT_RELU_PLUS_ONE: return x + 1e-3f > 0.f ? 1.f : 0.f;
-    default: return 1.f;
-    }
-}
-
 template <typename T>
 __global__ void __launch_bounds__(256) size_map_fwd_kernel(SizeMapArgs a)
 {

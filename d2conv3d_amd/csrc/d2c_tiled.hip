@@ -54,6 +54,8 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
                            const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc,
                            void *gw, hipStream_t st);
 
+static bool mfma_channels_ok(const d2c_conv3d_desc &q);
+
 namespace {
 
 inline int vec_of(int dtype) { return dtype == D2C_BF16 ? 8 : 4; }
@@ -71,9 +73,17 @@ d2c_conv3d_desc as_3d(const d2c_conv1d_desc &q)
     return r;
 }
 
-TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0)
+TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0, const d2c_size_map_desc *sz = nullptr)
 {
     TiledShape s;
+    s.ss.on = sz ? 1 : 0;
+    s.ss.mode = sz ? sz->mode : 0;
+    s.ss.act = sz ? sz->activation : 0;
+    for (int i = 0; i < D2C_SIZE_MAX_K; i++) {
+        s.ss.base[0][i] = sz ? sz->base_z[i] : 0.f;
+        s.ss.base[1][i] = sz ? sz->base_y[i] : 0.f;
+        s.ss.base[2][i] = sz ? sz->base_x[i] : 0.f;
+    }
     s.nd = nd; s.quirks = quirks;
     s.N = q.N; s.Cin = q.Cin; s.Cout = q.Cout; s.D = q.D; s.H = q.H; s.W = q.W;
     s.K = q.kd * q.kh * q.kw; s.G = q.offset_groups; s.groups = q.groups;
@@ -83,6 +93,7 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0)
     s.adt = q.aux_dtype;
     s.act = q.epilogue; s.act_scale = q.epilogue_scale;
     s.P = q.Do * q.Ho * q.Wo; s.vol = q.D * q.H * q.W; s.M = q.N * s.P;
+    s.dP = make_fastdiv(s.P); s.dHW = make_fastdiv(q.Ho * q.Wo); s.dW = make_fastdiv(q.Wo);
     const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
     s.ogp = (s.og + nt - 1) / nt * nt;
     s.geo = make_geom(q);
@@ -223,6 +234,49 @@ __global__ void __launch_bounds__(256) pack_weight_fwd_lds_kernel(const T *w, T 
     }
 }
 
+// Size-map source, backward: fp32 sums per axis [N][3][P] -> gradient of the raw size prediction [N][channels][P]
+// (the axes a channel feeds add up; times the derivative of the size activation), in the storage type of the map.
+template <bool AUX16>
+__global__ void __launch_bounds__(256) size_grad_finish_kernel(TiledShape s, const float *acc, const void *raw, void *graw)
+{
+    const int nc = mode_channels(s.ss.mode);
+    const long total = (long)s.N * s.P;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long n = i / s.P, p = i - n * s.P;
+        for (int c = 0; c < nc; c++) {
+            float v = 0.f;
+#pragma unroll
+            for (int ax = 0; ax < 3; ax++)
+                if (axis_channel(s.ss.mode, ax) == c) v += acc[(n * 3 + ax) * s.P + p];
+            const long ri = (n * nc + c) * s.P + p;
+            v *= size_act_grad(s.ss.act, ld_auxT<AUX16>(raw, ri));
+            if constexpr (AUX16) reinterpret_cast<bf16_t *>(graw)[ri] = f32_to_bf16(v);
+            else reinterpret_cast<float *>(graw)[ri] = v;
+        }
+    }
+}
+
+// Size-map source, backward: raw map -> (size - 1) per axis as float [N][3][P] (0 for an axis the mode does not
+// predict), once per call: the kernels of the backward pass form a tap's offsets from it per (tile, tap).
+template <bool AUX16>
+__global__ void __launch_bounds__(256) size_minus_one_kernel(TiledShape s, const void *raw, float *sm1)
+{
+    const int nc = mode_channels(s.ss.mode);
+    const long total = (long)s.N * s.P;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long n = i / s.P, p = i - n * s.P;
+        float c[3];
+#pragma unroll
+        for (int ax = 0; ax < 3; ax++) {
+            const int ch = axis_channel(s.ss.mode, ax);
+            c[ax] = ch < 0 ? 0.f : ld_auxT<AUX16>(raw, (n * nc + ch) * s.P + p);
+        }
+        size_minus_one<AUX16>(s, c);
+#pragma unroll
+        for (int ax = 0; ax < 3; ax++) sm1[(n * 3 + ax) * s.P + p] = c[ax];
+    }
+}
+
 struct FwdWs {
     size_t xcl, wp, outacc, total;
 };
@@ -292,9 +346,9 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 
 template <typename T>
 int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
-              const void *bias, void *out, void *ws, hipStream_t st, int nd = 3)
+              const void *bias, void *out, void *ws, hipStream_t st, int nd = 3, const d2c_size_map_desc *sz = nullptr)
 {
-    const TiledShape s = tiled_shape(q, nd, 0);
+    const TiledShape s = tiled_shape(q, nd, 0, sz);
     char *base = (char *)ws;
     if (nd == 3 && is_depthwise(q)) {
         const DwWs d = dw_ws(q, s);
@@ -336,7 +390,7 @@ bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 struct BwdWs {
-    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, total;
+    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, gsacc, sm1, total;
 };
 BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -367,17 +421,23 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
         w.ovf = w.entries + en;
         w.total = w.ovf + ov;
     }
+    // size-map source: fp32 sums of the size gradient per axis
+    w.gsacc = w.total;
+    if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
+    w.sm1 = w.total;       // ... and (size - 1) per axis
+    if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
     return w;
 }
 
 template <typename T>
 int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off, const void *mask,
                const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws, hipStream_t st,
-               int nd = 3, int quirks = 0)
+               int nd = 3, int quirks = 0, const d2c_size_map_desc *sz = nullptr)
 {
-    const TiledShape s = tiled_shape(q, nd, quirks);
+    TiledShape s = tiled_shape(q, nd, quirks, sz);
     char *base = (char *)ws;
     if (!mask) gmask = nullptr;
+    const void *size_raw = off;   // (size-map source; `off` becomes the per-axis (size - 1) below)
     if (nd == 3 && is_depthwise(q)) {
         const DwWs d = dw_ws(q, s);
         if (int rc = pack_input<T>(s, x, base + d.xcl, st)) return rc;
@@ -413,6 +473,19 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
     }
     const BwdWs l = bwd_ws(q, s);
     if (int rc = pack_input<T>(s, x, base + l.xcl, st, true)) return rc;   // with the row of zeros behind it
+    if (s.ss.on) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        long gr = ((long)s.N * s.P + 255) / 256;
+        if (gr > 8192) gr = 8192;
+        float *sm1 = (float *)(base + l.sm1);
+        if (s.adt == D2C_BF16)
+            hipLaunchKernelGGL(size_minus_one_kernel<true>, dim3((unsigned)gr), dim3(256), 0, st, s, size_raw, sm1);
+        else
+            hipLaunchKernelGGL(size_minus_one_kernel<false>, dim3((unsigned)gr), dim3(256), 0, st, s, size_raw, sm1);
+        if (int rc = d2c_check_launch("size_minus_one_kernel")) return rc;
+        s.ss.on = 2;
+        off = sm1;
+    }
     if (gx || goff || gmask) {
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
@@ -420,6 +493,14 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             const bool auxk = (goff || gmask) && use_aux_kernel(q, s);
             // grad_input from sample lists: filled by the offset / mask gradient kernel on its way when that
             // runs, by a pass of their own otherwise
+            // size-map source: `goff` is the gradient of the raw size map; the offset / mask gradient kernel adds
+            // into fp32 sums per axis, which a finishing kernel folds into it
+            void *goff_k = goff;
+            if (s.ss.on && goff) {
+                goff_k = base + l.gsacc;
+                D2cProfScope prof(D2C_PROF_PACK, st);
+                d2c_fill_zero(goff_k, (size_t)s.N * 3 * s.P * sizeof(float), st);
+            }
             SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
             if (lists) {
                 L = d2c_lists_make(s, Elem<T>::DT, base + l.counts, base + l.entries, base + l.ovf);
@@ -431,9 +512,21 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                                                      (float *)(base + l.auxacc), st))
                 return rc;
             if (auxk)
-                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff, gmask,
+                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff_k, gmask,
                                                     lists ? &L : nullptr, st))
                     return rc;
+            if (s.ss.on && goff) {
+                D2cProfScope prof(D2C_PROF_PACK, st);
+                long gr = ((long)s.N * s.P + 255) / 256;
+                if (gr > 8192) gr = 8192;
+                if (s.adt == D2C_BF16)
+                    hipLaunchKernelGGL(size_grad_finish_kernel<true>, dim3((unsigned)gr), dim3(256), 0, st, s,
+                                       (const float *)goff_k, size_raw, goff);
+                else
+                    hipLaunchKernelGGL(size_grad_finish_kernel<false>, dim3((unsigned)gr), dim3(256), 0, st, s,
+                                       (const float *)goff_k, size_raw, goff);
+                if (int rc = d2c_check_launch("size_grad_finish_kernel")) return rc;
+            }
             if (lists)
                 if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, L, gxcl, st)) return rc;
             if (gx)
@@ -525,23 +618,33 @@ size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q)
     return is_depthwise(q) ? dw_ws(q, s).total_fwd : fwd_ws(q, s).total;
 }
 
-size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q)
+size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q, const d2c_size_map_desc *sz)
 {
-    const TiledShape s = tiled_shape(q);
+    const TiledShape s = tiled_shape(q, 3, 0, sz);
     return is_depthwise(q) ? dw_ws(q, s).total_bwd : bwd_ws(q, s).total;
 }
 
-int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
-                      const void *bias, void *out, void *ws, hipStream_t st)
+// The matrix-core kernels can form the offsets from a size map themselves; the backward pass then needs the
+// offset / mask gradient kernel (one pass over the output channels of a weight group).
+bool d2c_tiled_sized_supported(const d2c_conv3d_desc &q, bool backward)
 {
-    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st);
-    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st);
+    if (q.offset_groups != 1 || is_depthwise(q) || !mfma_channels_ok(q)) return false;
+    if (!backward) return true;
+    return use_aux_kernel(q, tiled_shape(q));
+}
+
+int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
+                      const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz)
+{
+    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 3, sz);
+    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 3, sz);
 }
 
 int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
                        const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
-                       void *ws, hipStream_t st)
+                       void *ws, hipStream_t st, const d2c_size_map_desc *sz)
 {
-    if (q.dtype == D2C_BF16) return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st);
-    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st);
+    if (q.dtype == D2C_BF16)
+        return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz);
+    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz);
 }

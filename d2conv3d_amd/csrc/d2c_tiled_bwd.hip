@@ -774,29 +774,36 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
         const long m = (long)(sp + i * a.split) * MT + ctid;
         cvalid = m < s.M;
         if (cvalid) {
-            cb_ = (int)(m / s.P); cp_ = (int)(m - (long)cb_ * s.P);
+            cb_ = fdiv((int)m, s.dP); cp_ = (int)m - cb_ * s.P;      // (m < N * P < 2^31)
             const long ab = (((long)cb_ * s.G + g) * s.K + k) * s.P + cp_;
-            if (s.nd == 3) {
-                const long ob = 3 * ab - 2 * (long)cp_;
-                craw[0] = ld_auxT<AUX16>(a.off, ob);
-                craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
-                craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
-            } else {
-                craw[0] = 0.f; craw[1] = 0.f;
-                craw[2] = ld_auxT<AUX16>(a.off, ab);
-            }
+            tap_offsets_issue<AUX16>(s, a.off, cb_, g, k, cp_, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
         }
     };
+    float sbase[3] = {0.f, 0.f, 0.f};   // kernel-grid coordinates of this workgroup's tap (size-map source)
+    if (s.ss.on) {
+        typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+        const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
+#pragma unroll
+        for (int ax = 0; ax < 3; ax++) sbase[ax] = rnd<AT>(s.ss.base[ax][kq[ax]]);
+    }
     auto coords_finish = [&](int buf) {   // of the tile whose offsets coords_issue requested last
         if (worker) return;
         float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         int idx = 0;
         unsigned live = 0;
         if (cvalid) {
-            const int ox = cp_ % s.Wo, oy = (cp_ / s.Wo) % s.Ho, oz = cp_ / (s.Wo * s.Ho);
+            const int oz = fdiv(cp_, s.dHW), rem = cp_ - oz * (s.Wo * s.Ho);
+            const int oy = fdiv(rem, s.dW), ox = rem - oy * s.Wo;
             int bz, by, bx;
             tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
+            if (s.ss.on) {
+                // size-map source: offsets = base_a[k_a] * (size_a - 1); the tap is this workgroup's own
+                typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+                if (s.ss.on == 1) size_minus_one<AUX16>(s, craw);
+#pragma unroll
+                for (int ax = 0; ax < 3; ax++) craw[ax] = rnd<AT>(sbase[ax] * craw[ax]);
+            }
             const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
             live = t.live;
             idx = (cb_ * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
@@ -937,9 +944,17 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
                 if (it + 1 < nmy) interp_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
             }
         } else {
+            // (the coordinate wavefront shares its SIMD with two worker wavefronts and is the one the iteration
+            // waits for when the matrix work per tile is small: it issues ahead of them)
+            __builtin_amdgcn_s_setprio(2);
             for (int it = 0; it < nmy; it++) {
-                __syncthreads();
-                if (it + 3 < nmy) coords_finish(it % 3);   // offsets requested one iteration ago
+                // (a barrier that waits for this wavefront's LDS stores only: the offsets it requested stay in
+                // flight across it and are waited for where they are used, a whole iteration after the request)
+                lds_only_barrier();
+                if (it + 3 < nmy) {
+                    __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0)
+                    coords_finish(it % 3);
+                }
                 if (it + 4 < nmy) coords_issue(it + 4);
             }
         }

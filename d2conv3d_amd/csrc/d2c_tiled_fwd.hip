@@ -103,15 +103,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
         if (tid < MT && cvalid) {
             const int j = st / s.K, k = st - j * s.K;
             const int g = (wg * s.cg + j * BKC) / s.cpg;
-            if (s.nd == 3) {
-                const long ob = (((long)cb * s.G + g) * s.K + k) * 3 * s.P + cp;
-                craw[0] = ld_auxT<AUX16>(a.off, ob);
-                craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
-                craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
-            } else {
-                craw[0] = 0.f; craw[1] = 0.f;
-                craw[2] = ld_auxT<AUX16>(a.off, (((long)cb * s.G + g) * s.K + k) * s.P + cp);
-            }
+            tap_offsets_issue<AUX16>(s, a.off, cb, g, k, cp, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, (((long)cb * s.G + g) * s.K + k) * s.P + cp) : 1.f;
         }
     };
@@ -124,6 +116,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
                 const int k = st % s.K;
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
+                tap_offsets_finish<AUX16>(s, k, craw);
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
                 live = t.live;
                 idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
@@ -382,14 +375,20 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     const int ctid = tid - kThreads;
     // The lane's position within a work item.  Offsets are requested (issue) one iteration before they are
     // turned into a table row (finish), possibly across a segment boundary: one set of constants for each.
-    struct PosC { int b, p, oz, oy, ox; bool valid; };
+    // (size-map source: the part of the offsets that the taps of a position share, size - 1 per axis, is formed
+    // here once per work item; a step then costs three multiplications and no load)
+    struct PosC { int b, p, oz, oy, ox; bool valid; float sm1[3]; };
     auto pos_of = [&](const SegWalk &w) {
-        PosC c{0, 0, 0, 0, 0, false};
+        PosC c{0, 0, 0, 0, 0, false, {0.f, 0.f, 0.f}};
         const int m = w.tile * MT + ctid;
         c.valid = w.item >= 0 && m < s.M;
         if (c.valid) {
             c.b = m / s.P; c.p = m - c.b * s.P;
             c.ox = c.p % s.Wo; c.oy = (c.p / s.Wo) % s.Ho; c.oz = c.p / (s.Wo * s.Ho);
+            if (s.ss.on && cwave) {
+                tap_offsets_issue<AUX16>(s, a.off, c.b, 0, 0, c.p, c.sm1);
+                size_minus_one<AUX16>(s, c.sm1);
+            }
         }
         return c;
     };
@@ -399,15 +398,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
             const int j = w.st / s.K, k = w.st - j * s.K;
             const int g = (w.wg * s.cg + j * BKC) / s.cpg;
             const long ab = (((long)c.b * s.G + g) * s.K + k) * s.P + c.p;
-            if (s.nd == 3) {
-                const long ob = 3 * ab - 2 * (long)c.p;
-                craw[0] = ld_auxT<AUX16>(a.off, ob);
-                craw[1] = ld_auxT<AUX16>(a.off, ob + s.P);
-                craw[2] = ld_auxT<AUX16>(a.off, ob + 2 * (long)s.P);
-            } else {
-                craw[0] = 0.f; craw[1] = 0.f;
-                craw[2] = ld_auxT<AUX16>(a.off, ab);
-            }
+            if (!s.ss.on) tap_offsets_issue<AUX16>(s, a.off, c.b, g, k, c.p, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
         }
     };
@@ -420,6 +411,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 const int k = w.st % s.K;
                 int bz, by, bx;
                 tap_base(s.geo, k, c.oz, c.oy, c.ox, bz, by, bx);
+                if (s.ss.on) size_tap_offsets<AUX16>(s, k, c.sm1, craw);
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
                 live = t.live;
                 idx = (c.b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000

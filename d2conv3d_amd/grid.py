@@ -144,17 +144,23 @@ def size_map_offsets(size_raw, mode, kernel_shape=(3, 3, 3), dilation=(1, 1, 1),
         raise RuntimeError(f"size_map_offsets: mode '{mode}' wants {want_c} size channels, got {tuple(size_raw.shape)}")
     if max(kernel_shape) > _lib.SIZE_MAX_K:
         raise RuntimeError(f"size_map_offsets: kernel extents up to {_lib.SIZE_MAX_K}")
+    return _SizeMapOffsets.apply(size_raw, size_map_desc(size_raw, mode, kernel_shape, dilation, activation))
+
+
+def size_map_desc(size_raw, mode, kernel_shape, dilation, activation):
+    """The d2c_size_map_desc of a raw size map [N, channels(mode), *spatial]."""
+    from . import _lib
     desc = _lib.SizeMapDesc()
     desc.N = size_raw.shape[0]
     desc.P = int(size_raw[0, 0].numel())
     desc.kd, desc.kh, desc.kw = kernel_shape
-    desc.mode, desc.activation = _lib.SIZE_MODES[mode], _lib.SIZE_ACTIVATIONS[activation]
+    desc.mode, desc.activation = _lib.SIZE_MODES[mode.lower()], _lib.SIZE_ACTIVATIONS[activation]
     desc.dtype = _lib.D2C_BF16 if size_raw.dtype == torch.bfloat16 else _lib.D2C_F32
     for name, d, k in zip(("base_z", "base_y", "base_x"), dilation, kernel_shape):
         arr = getattr(desc, name)
         for i, v in enumerate(_kernel_axis(d, k)):
             arr[i] = v
-    return _SizeMapOffsets.apply(size_raw, desc)
+    return desc
 
 
 _AXIS_CACHE = {}

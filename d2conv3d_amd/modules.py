@@ -14,7 +14,7 @@ import torch.nn.functional as F
 from torch.nn.modules.utils import _triple
 from torch.utils.checkpoint import checkpoint
 
-from .deform_conv import DeformConv3d
+from .deform_conv import DeformConv3d, deform_conv3d_sized
 from .grid import offsets_from_size_map, size_map_offsets
 
 
@@ -164,9 +164,25 @@ class TemporalMDConv3d(_TemporalMixin, MDConv3d):
     pass
 
 
+def _sized_forward(layer, input):
+    """forward() of the size-conditioned layers with `fused_deformation = True` (the default) on CUDA tensors: the
+    predicted size map goes to the operator as it is (deform_conv3d_sized); no [N, 3K, ...] offsets tensor and no
+    autograd graph of its expansion exist.  Returns None where that does not apply (CPU tensors, float64)."""
+    if layer.fused_deformation is not True or not input.is_cuda or input.dtype == torch.float64:
+        return None
+    deform_input = input if layer.norm is None else layer.norm(input)
+    if layer.checkpoint_deformation and torch.is_grad_enabled():
+        size_raw, alpha = checkpoint(layer._get_size_and_alpha, deform_input, use_reentrant=False)
+    else:
+        size_raw, alpha = layer._get_size_and_alpha(deform_input)
+    dc = layer.deform_conv
+    return deform_conv3d_sized(input, size_raw, alpha, dc.weight, dc.bias, layer._mode, layer.size_activation,
+                               dc.stride, dc.padding, dc.dilation, dc.groups, output_relu=dc.output_relu_scale)
+
+
 def _size_offsets(layer, size_raw):
-    """Size activation + offsets_from_size_map: one library kernel each way for CUDA float32 / bfloat16
-    tensors (`fused_deformation`, on by default), the reference's torch formulation otherwise."""
+    """Size activation + offsets_from_size_map as tensors: one library kernel each way for CUDA float32 / bfloat16
+    tensors (`fused_deformation = "expand"`), the reference's torch formulation otherwise."""
     if layer.fused_deformation and size_raw.is_cuda and size_raw.dtype in (torch.float32, torch.bfloat16):
         return size_map_offsets(size_raw, layer._mode, layer.deform_conv.kernel_size, layer.deform_conv.dilation,
                                 layer.size_activation)
@@ -189,6 +205,13 @@ class _SizeConditionedD(DConv3d):
     def _get_deformation(self, input):
         return _size_offsets(self, self.deform_params(input)), None
 
+    def _get_size_and_alpha(self, input):
+        return self.deform_params(input), None
+
+    def forward(self, input):
+        out = _sized_forward(self, input)
+        return out if out is not None else super().forward(input)
+
 
 class _SizeConditionedMD(MDConv3d):
     """modules.py:162-219 / network/layers.py:233-313."""
@@ -205,6 +228,15 @@ class _SizeConditionedMD(MDConv3d):
         deformation = self.deform_params(input)
         size_map, alpha = torch.split(deformation, [self._size_channels, self.alpha_channels], dim=1)
         return _size_offsets(self, size_map), self.activation(alpha)
+
+    def _get_size_and_alpha(self, input):
+        deformation = self.deform_params(input)
+        size_map, alpha = torch.split(deformation, [self._size_channels, self.alpha_channels], dim=1)
+        return size_map, self.activation(alpha)
+
+    def forward(self, input):
+        out = _sized_forward(self, input)
+        return out if out is not None else super().forward(input)
 
 
 class SizeConditionedDConv3d(_SizeConditionedD):

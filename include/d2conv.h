@@ -212,6 +212,25 @@ int d2c_size_map_offsets_forward(const d2c_size_map_desc *desc, const void *size
 int d2c_size_map_offsets_backward(const d2c_size_map_desc *desc, const void *size_raw, const void *grad_offsets,
                                   void *grad_size_raw, void *stream);
 
+/* The deformable convolution fed by the size map itself (no counterpart as ONE call in the reference: it replaces
+ * network/layers.py:171-181 + utils/grid.py:72-98 + deform_conv3d_forward/backward_cuda for the size-conditioned
+ * layers, network/layers.py:184-313).  `size_raw` [N, 3|2|2|1, Do, Ho, Wo] is the prediction before the size
+ * activation, in the element type `aux_dtype` of the mask; the convolution description must have
+ * offset_groups == 1 and `sdesc` the same N, kernel extents and P = Do*Ho*Wo.  Where the matrix-core kernels serve
+ * the description, the sampler forms base_a[k_a] * (act(size_raw) - 1) where it needs a tap's offsets and no
+ * [N, 3K, P] offsets tensor (nor its gradient) exists; other descriptions expand the map inside the workspace
+ * and run the ordinary kernels.  Results equal d2c_size_map_offsets_forward followed by d2c_conv3d_forward (bit
+ * for bit in the forward pass).  `grad_size_raw` (may be NULL) has the shape of size_raw. */
+size_t d2c_conv3d_sized_forward_workspace_bytes(const d2c_conv3d_desc *desc, const d2c_size_map_desc *sdesc);
+size_t d2c_conv3d_sized_backward_workspace_bytes(const d2c_conv3d_desc *desc, const d2c_size_map_desc *sdesc);
+int d2c_conv3d_sized_forward(const d2c_conv3d_desc *desc, const d2c_size_map_desc *sdesc, const void *x,
+                             const void *size_raw, const void *mask, const void *weight, const void *bias, void *out,
+                             void *workspace, size_t workspace_bytes, void *stream);
+int d2c_conv3d_sized_backward(const d2c_conv3d_desc *desc, const d2c_size_map_desc *sdesc, const void *grad_out,
+                              const void *x, const void *size_raw, const void *mask, const void *weight, void *grad_x,
+                              void *grad_size_raw, void *grad_mask, void *grad_weight, void *grad_bias,
+                              void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- plain depthwise conv3d (no sampling) ------------------------------------------------
  * The operator of the reference's second extension, ops/fast-depthwise-conv3d, which its
  * backbone uses for the channel-separated 3x3x3 convolutions (network/backbone/resnet.py:110):

@@ -93,6 +93,38 @@ def test_full_size_against_oracle(name, dev):
             assert_close(a, ee, 2e-2, 2e-2 * ee.abs().max().item(), f"{name} {n}")
 
 
+@pytest.mark.parametrize("name", ["c2_f32", "c2_bf16"])
+def test_full_size_dilation_map_into_the_operator(name, dev):
+    """Workload C2 the way bench.py times it: the dilation map [2, 3, 8, 30, 54] goes into the operator
+    (deform_conv3d_sized), no offsets tensor exists.  Against the oracle on the expanded offsets; the expected
+    gradient of the map is the transpose of the expansion (oracle/sizemap.py) applied to the oracle's grad_offset."""
+    import numpy as np
+    from oracle import sizemap
+    c = bench.WORKLOADS[name]
+    x, off, m, w, b, gout, size = bench.make_inputs(name, torch, want_size=True)
+    f = lambda t: t.float()
+    if c["dt"] == "bf16":
+        x, w, b, gout, m, size = (t.bfloat16() for t in (x, w, b, gout, m, size))
+        # the offsets the sampler forms from a bfloat16 map: the torch formulation in bfloat16
+        from d2conv3d_amd.grid import offsets_from_size_map
+        off = offsets_from_size_map(size, "xyz", (3, 3, 3), (1, 1, 1))
+    else:
+        assert np.array_equal(off.numpy(), sizemap.offsets(size.double().numpy(), "xyz").astype(np.float32))
+    ts = [t.to(dev).requires_grad_(True) for t in (x, size, m, w, b)]
+    out = d2c.deform_conv3d_sized(*ts, "xyz", "linear", 1, 1, 1, 1)
+    out.backward(gout.to(dev))
+    e_out = cpu.conv3d_forward(f(x), f(off), f(m), f(w), f(b), 1, 1, 1, 1, 1)
+    e = list(cpu.conv3d_backward(f(gout), f(x), f(off), f(m), f(w), True, 1, 1, 1, 1, 1))
+    e[1] = torch.from_numpy(sizemap.offsets_backward(e[1].double().numpy(), "xyz")).float()
+    names = ["grad_input", "grad_size", "grad_mask", "grad_weight", "grad_bias"]
+    for n, a, ee in [("out", out, e_out)] + list(zip(names, [t.grad for t in ts], e)):
+        if c["dt"] == "f32":
+            assert_close(a, ee, 1e-4, 1e-5 * max(1.0, ee.abs().max().item()), f"{name} {n}")
+        else:
+            assert rel_l2(a, ee) < 2e-2, (name, n, rel_l2(a, ee))
+            assert_close(a, ee, 2e-2, 2e-2 * ee.abs().max().item(), f"{name} {n}")
+
+
 def test_long_clip_backward_against_oracle(dev):
     """The long-clip volume of workload c5b (32 x 60 x 108 = 207360 positions, bfloat16, one offset group) with
     64 channels, which the oracle finishes in seconds: all five gradients, i.e. the grad-column rows, the offset /

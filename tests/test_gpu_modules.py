@@ -115,7 +115,9 @@ def test_size_conditioned_layers_same_with_and_without_the_fused_producer(cls, d
         layer.deform_params.bias.normal_(0, 0.3)
     x = torch.randn(2, 4, 5, 6, 7, device=dev)
     outs, grads = [], []
-    for fused in (True, False):
+    # True: the size map goes into the operator (deform_conv3d_sized); "expand": offsets tensor made by the library's
+    # expansion kernel; False: the reference's torch formulation
+    for fused in (True, "expand", False):
         layer.fused_deformation = fused
         layer.zero_grad()
         xi = x.clone().requires_grad_(True)
@@ -123,9 +125,10 @@ def test_size_conditioned_layers_same_with_and_without_the_fused_producer(cls, d
         out.square().sum().backward()
         outs.append(out.detach())
         grads.append([xi.grad.clone(), layer.deform_params.weight.grad.clone()])
-    assert torch.allclose(outs[0], outs[1], rtol=1e-5, atol=1e-5)
-    for a, b in zip(*grads):
-        assert torch.allclose(a, b, rtol=1e-4, atol=1e-4 * max(1.0, b.abs().max().item()))
+    for i in (0, 1):
+        assert torch.allclose(outs[i], outs[2], rtol=1e-5, atol=1e-5)
+        for a, b in zip(grads[i], grads[2]):
+            assert torch.allclose(a, b, rtol=1e-4, atol=1e-4 * max(1.0, b.abs().max().item()))
 
 
 def test_size_map_offsets_reject_bad_arguments(dev):
