@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the D2Conv3D operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap|dwconv]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap|dwconv|c3_norm]
 
 One step = one forward (+ one backward with all five gradients, except for
 the forward-only workload c1) of the modulated deformable convolution through
@@ -193,6 +193,81 @@ def bench_size_map(args):
     print(json.dumps(line))
 
 
+def bench_conv_act_norm(args):
+    """The `_conv` block of the reference's refinement modules (network/modules/refinement.py:38-43) at the size of
+    workload c3: Sequential(MDConv3d-style operator, ReLU, GroupNorm(32)), forward + backward, as the fused block
+    of util.fuse_conv_act_norm (activation and per-channel sums in the convolution's forward kernel, GroupNorm in one
+    pass from them) against the plain sequence (the same operator, then torch's relu and group_norm)."""
+    import copy
+    import torch
+    import torch.nn as nn
+    from d2conv3d_amd import util
+    from d2conv3d_amd.deform_conv import DeformConv3d
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    x, off, m, w, b, gout = (t.to(dev, torch.bfloat16) for t in make_inputs("c3", torch))
+
+    class Block(nn.Module):          # offsets / mask given (the deformation branch is not part of this measurement)
+        def __init__(self):
+            super().__init__()
+            self.deform_conv = DeformConv3d(512, 512, 3, padding=1, offset_groups=8)
+            self.norm = nn.GroupNorm(32, 512)
+            self.fused = False
+
+        def forward(self, x, off, m):
+            dc = self.deform_conv
+            if not self.fused:
+                return self.norm(torch.relu(dc(x, off, m)))
+            from d2conv3d_amd import _ops
+            dc.output_relu_scale, dc.keep_output_stats = 1.0, True
+            out = dc(x, off, m)
+            return _ops.group_norm_from_stats(out, dc.last_output_stats, self.norm.weight, self.norm.bias, 32, self.norm.eps)
+
+    net = Block().to(dev, torch.bfloat16)
+    with torch.no_grad():
+        net.deform_conv.weight.copy_(w)
+        net.deform_conv.bias.copy_(b)
+    xs = x.clone().requires_grad_(True)
+    offs, ms = off.clone().requires_grad_(True), m.clone().requires_grad_(True)
+
+    def step():
+        net.zero_grad(set_to_none=True)
+        xs.grad = offs.grad = ms.grad = None
+        net(xs, offs, ms).backward(gout)
+
+    def timed():
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    net.fused = False
+    ms_plain = timed()
+    y_plain = net(xs, offs, ms).detach().float()
+    net.fused = True
+    ms_fused = timed()
+    y_fused = net(xs, offs, ms).detach().float()
+    err = float((y_fused - y_plain).norm() / y_plain.norm())
+    f_fwd, _, _ = algorithmic("c3")
+    value = 3 * f_fwd / (ms_fused * 1e-3) / 1e12
+    line = {
+        "metric": "mdconv3d + ReLU + GroupNorm block fwd+bwd effective TFLOP/s (c3_norm) on 1 GPU", "value": round(value, 3),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_fused, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "c3_norm: Sequential(modulated deformable conv3d of workload c3, ReLU, GroupNorm(32)) "
+                               "forward + backward through the autograd functions (allocations included), fused block",
+                   "plain_sequence_ms_per_step": round(ms_plain, 4), "relative_l2_fused_vs_plain": err},
+        "roofline": None,
+    }
+    print(json.dumps(line))
+
+
 def bench_dwconv(args):
     """Plain depthwise conv3d (the reference's fast-depthwise-conv3d operator; backbone shape: 256 channels,
     8x56x56, 3x3x3, stride 1, padding 1, float32), forward + backward through the C ABI with pre-allocated
@@ -286,7 +361,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv", "c3_norm"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--expanded-offsets", action="store_true",
                     help="dynamic-dilation workloads (c2_*): expand the dilation map to an offsets tensor first "
@@ -305,6 +380,8 @@ def main():
         return bench_size_map(args)
     if args.workload == "dwconv":
         return bench_dwconv(args)
+    if args.workload == "c3_norm":
+        return bench_conv_act_norm(args)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 

@@ -27,6 +27,8 @@ EXPORTS = (
     "d2c_size_map_offsets_forward", "d2c_size_map_offsets_backward",
     "d2c_conv3d_sized_forward_workspace_bytes", "d2c_conv3d_sized_backward_workspace_bytes",
     "d2c_conv3d_sized_forward", "d2c_conv3d_sized_backward",
+    "d2c_conv3d_forward_stats_workspace_bytes", "d2c_conv3d_forward_stats", "d2c_channel_stats",
+    "d2c_group_norm_forward", "d2c_group_norm_backward_workspace_bytes", "d2c_group_norm_backward",
     "d2c_dwconv3d_check", "d2c_dwconv3d_backward_workspace_bytes", "d2c_dwconv3d_forward", "d2c_dwconv3d_backward",
 )
 
@@ -49,6 +51,10 @@ SIZE_ACTIVATIONS = {"linear": 0, "elu": 1, "relu": 2, "relu_plus_one": 3}
 class SizeMapDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("N", "P", "kd", "kh", "kw", "mode", "activation", "dtype")] + [
         (n, ctypes.c_float * SIZE_MAX_K) for n in ("base_z", "base_y", "base_x")]
+
+
+class GroupNormDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("N", "C", "P", "groups", "dtype")] + [("eps", ctypes.c_float)]
 
 
 class DwConv3dDesc(ctypes.Structure):
@@ -112,6 +118,15 @@ def load():
         f.argtypes, f.restype = [p3, psm], sz
     lib.d2c_conv3d_sized_forward.argtypes, lib.d2c_conv3d_sized_forward.restype = [p3, psm] + [vp] * 7 + [sz, vp], ctypes.c_int
     lib.d2c_conv3d_sized_backward.argtypes, lib.d2c_conv3d_sized_backward.restype = [p3, psm] + [vp] * 11 + [sz, vp], ctypes.c_int
+    pgn = ctypes.POINTER(GroupNormDesc)
+    lib.d2c_conv3d_forward_stats_workspace_bytes.argtypes = [p3, psm]
+    lib.d2c_conv3d_forward_stats_workspace_bytes.restype = sz
+    lib.d2c_conv3d_forward_stats.argtypes, lib.d2c_conv3d_forward_stats.restype = [p3, psm] + [vp] * 8 + [sz, vp], ctypes.c_int
+    lib.d2c_channel_stats.argtypes, lib.d2c_channel_stats.restype = [pgn, vp, vp, vp], ctypes.c_int
+    lib.d2c_group_norm_forward.argtypes, lib.d2c_group_norm_forward.restype = [pgn] + [vp] * 6, ctypes.c_int
+    lib.d2c_group_norm_backward_workspace_bytes.argtypes = [pgn]
+    lib.d2c_group_norm_backward_workspace_bytes.restype = sz
+    lib.d2c_group_norm_backward.argtypes, lib.d2c_group_norm_backward.restype = [pgn] + [vp] * 8 + [sz, vp], ctypes.c_int
     pdw = ctypes.POINTER(DwConv3dDesc)
     lib.d2c_dwconv3d_check.argtypes, lib.d2c_dwconv3d_check.restype = [pdw], ctypes.c_int
     lib.d2c_dwconv3d_backward_workspace_bytes.argtypes = [pdw]

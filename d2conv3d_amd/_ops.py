@@ -95,7 +95,7 @@ class _DeformConv3dFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, offset, alpha, weight, bias, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, offset_groups,
-                relu_scale=0.0):
+                relu_scale=0.0, want_stats=False):
         lib = _lib.load()
         input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
         alpha = alpha.contiguous() if alpha is not None else None
@@ -109,20 +109,30 @@ class _DeformConv3dFunction(torch.autograd.Function):
         _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d")
         dev = input.device
         out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
+        stats = torch.empty((N, Cout, 2), dtype=torch.float32, device=dev) if want_stats else None
         with torch.cuda.device(dev):
-            nb = lib.d2c_conv3d_forward_workspace_bytes(ctypes.byref(desc))
+            nb = (lib.d2c_conv3d_forward_stats_workspace_bytes(ctypes.byref(desc), None) if want_stats
+                  else lib.d2c_conv3d_forward_workspace_bytes(ctypes.byref(desc)))
             ws = _workspace(nb, dev)
-            rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha), _ptr(weight),
-                                        _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
+            if want_stats:
+                rc = lib.d2c_conv3d_forward_stats(ctypes.byref(desc), None, _ptr(input), _ptr(offset), _ptr(alpha),
+                                                  _ptr(weight), _ptr(bias), _ptr(out), _ptr(stats), _ptr(ws), nb,
+                                                  _stream(dev))
+            else:
+                rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha), _ptr(weight),
+                                            _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d forward")
         ctx.save_for_backward(input, offset, alpha, weight, bias, out if relu_scale > 0 else None)
         ctx.desc = desc
         ctx.relu_scale = float(relu_scale)
+        if want_stats:
+            ctx.mark_non_differentiable(stats)
+            return out, stats
         return out
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, grad_out):
+    def backward(ctx, grad_out, _grad_stats=None):
         lib = _lib.load()
         input, offset, alpha, weight, bias, out = ctx.saved_tensors
         desc = ctx.desc
@@ -143,19 +153,21 @@ class _DeformConv3dFunction(torch.autograd.Function):
                                          _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
                                          _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d backward")
-        return (gx, goff, galpha, gw, gb) + (None,) * 12
+        return (gx, goff, galpha, gw, gb) + (None,) * 13
 
 
 def deform_conv3d(input, offset, alpha, weight, bias, stride_d, stride_h, stride_w, pad_d, pad_h, pad_w,
-                  dilation_d, dilation_h, dilation_w, groups, offset_groups, relu_scale=0.0):
+                  dilation_d, dilation_h, dilation_w, groups, offset_groups, relu_scale=0.0, want_stats=False):
     """deform_conv3d of dconv3d.h:188-226; `alpha` and `bias` may be None.  `relu_scale` > 0 fuses
-    relu_scale * relu(.) into the store of the output (see _DeformConv3dFunction)."""
+    relu_scale * relu(.) into the store of the output (see _DeformConv3dFunction).  `want_stats` also returns the
+    float32 [N, Cout, 2] sums and sums of squares of the stored output per (sample, channel), added up by the
+    forward kernels where they store (the statistics a GroupNorm behind the convolution needs)."""
     _check_common(3, input, offset, alpha, weight, bias, groups, offset_groups)
     input, offset, alpha, weight, bias = _unify(input, offset, alpha, weight, bias)
     return _DeformConv3dFunction.apply(
         input, offset, alpha, weight, bias, int(stride_d), int(stride_h), int(stride_w),
         int(pad_d), int(pad_h), int(pad_w), int(dilation_d), int(dilation_h), int(dilation_w),
-        int(groups), int(offset_groups), float(relu_scale))
+        int(groups), int(offset_groups), float(relu_scale), bool(want_stats))
 
 
 class _DeformConv3dSizedFunction(torch.autograd.Function):
@@ -166,7 +178,7 @@ class _DeformConv3dSizedFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, size_raw, alpha, weight, bias, mode, activation, stride, padding, dilation, groups,
-                relu_scale=0.0):
+                relu_scale=0.0, want_stats=False):
         from .grid import size_map_desc
         lib = _lib.load()
         input, size_raw, weight = input.contiguous(), size_raw.contiguous(), weight.contiguous()
@@ -182,20 +194,31 @@ class _DeformConv3dSizedFunction(torch.autograd.Function):
         _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d_sized")
         dev = input.device
         out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
+        stats = torch.empty((N, Cout, 2), dtype=torch.float32, device=dev) if want_stats else None
         with torch.cuda.device(dev):
-            nb = lib.d2c_conv3d_sized_forward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+            nb = (lib.d2c_conv3d_forward_stats_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc)) if want_stats
+                  else lib.d2c_conv3d_sized_forward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc)))
             ws = _workspace(nb, dev)
-            rc = lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input), _ptr(size_raw),
-                                              _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
+            if want_stats:
+                rc = lib.d2c_conv3d_forward_stats(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input), _ptr(size_raw),
+                                                  _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out), _ptr(stats),
+                                                  _ptr(ws), nb, _stream(dev))
+            else:
+                rc = lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input), _ptr(size_raw),
+                                                  _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nb,
+                                                  _stream(dev))
         _lib.check(rc, "deform_conv3d_sized forward")
         ctx.save_for_backward(input, size_raw, alpha, weight, bias, out if relu_scale > 0 else None)
         ctx.desc, ctx.sdesc = desc, sdesc
         ctx.relu_scale = float(relu_scale)
+        if want_stats:
+            ctx.mark_non_differentiable(stats)
+            return out, stats
         return out
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, grad_out):
+    def backward(ctx, grad_out, _grad_stats=None):
         lib = _lib.load()
         input, size_raw, alpha, weight, bias, out = ctx.saved_tensors
         desc, sdesc = ctx.desc, ctx.sdesc
@@ -216,11 +239,11 @@ class _DeformConv3dSizedFunction(torch.autograd.Function):
                                                _ptr(size_raw), _ptr(alpha), _ptr(weight), _ptr(gx), _ptr(gsize),
                                                _ptr(galpha), _ptr(gw), _ptr(gb), _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d_sized backward")
-        return (gx, gsize, galpha, gw, gb) + (None,) * 7
+        return (gx, gsize, galpha, gw, gb) + (None,) * 8
 
 
 def deform_conv3d_sized(input, size_raw, alpha, weight, bias, mode, activation, stride, padding, dilation, groups=1,
-                        relu_scale=0.0):
+                        relu_scale=0.0, want_stats=False):
     """Deformable convolution whose tap offsets follow from a predicted size map:
     deform_conv3d(input, offsets_from_size_map(size_activation(size_raw), mode, kernel, dilation), alpha, ...)
     of network/layers.py:184-313 as one operator.  `size_raw` [N, 3|2|2|1, Do, Ho, Wo] for mode xyz|xxz|xy|x."""
@@ -238,7 +261,75 @@ def deform_conv3d_sized(input, size_raw, alpha, weight, bias, mode, activation, 
     _check_common(3, input, stand_in, alpha, weight, bias, groups, 1)
     input, size_raw, alpha, weight, bias = _unify(input, size_raw, alpha, weight, bias)
     return _DeformConv3dSizedFunction.apply(input, size_raw, alpha, weight, bias, mode, activation, stride, padding,
-                                            dilation, int(groups), float(relu_scale))
+                                            dilation, int(groups), float(relu_scale), bool(want_stats))
+
+
+class _GroupNormFromStats(torch.autograd.Function):
+    """torch.nn.functional.group_norm on the output of a convolution whose forward kernels already added up the
+    per-(sample, channel) sums (d2c_conv3d_forward_stats): d2c_group_norm_forward / _backward."""
+
+    @staticmethod
+    def forward(ctx, x, stats, weight, bias, groups, eps):
+        lib = _lib.load()
+        x = x.contiguous()
+        N, C = x.shape[:2]
+        P = x[0, 0].numel()
+        desc = _lib.GroupNormDesc(N, C, P, groups, _DT[x.dtype], eps)
+        weight = weight.to(x.dtype).contiguous() if weight is not None else None
+        bias = bias.to(x.dtype).contiguous() if bias is not None else None
+        y = torch.empty_like(x)
+        with torch.cuda.device(x.device):
+            rc = lib.d2c_group_norm_forward(ctypes.byref(desc), _ptr(x), _ptr(stats), _ptr(weight), _ptr(bias), _ptr(y),
+                                            _stream(x.device))
+        _lib.check(rc, "group_norm forward")
+        ctx.save_for_backward(x, stats, weight)
+        ctx.desc = desc
+        ctx.has_affine = (weight is not None, bias is not None)
+        return y
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_y):
+        lib = _lib.load()
+        x, stats, weight = ctx.saved_tensors
+        desc = ctx.desc
+        grad_y = grad_y.contiguous().to(x.dtype)
+        need = ctx.needs_input_grad
+        gx = torch.empty_like(x) if need[0] else None
+        gw = torch.empty(desc.C, dtype=x.dtype, device=x.device) if (ctx.has_affine[0] and need[2]) else None
+        gb = torch.empty(desc.C, dtype=x.dtype, device=x.device) if (ctx.has_affine[1] and need[3]) else None
+        with torch.cuda.device(x.device):
+            nb = lib.d2c_group_norm_backward_workspace_bytes(ctypes.byref(desc))
+            ws = _workspace(nb, x.device)
+            rc = lib.d2c_group_norm_backward(ctypes.byref(desc), _ptr(grad_y), _ptr(x), _ptr(stats), _ptr(weight),
+                                             _ptr(gx), _ptr(gw), _ptr(gb), _ptr(ws), nb, _stream(x.device))
+        _lib.check(rc, "group_norm backward")
+        return gx, None, gw, gb, None, None
+
+
+def group_norm_from_stats(x, stats, weight, bias, groups, eps=1e-5):
+    """GroupNorm of `x` [N, C, *spatial] (CUDA, float32 or bfloat16) from `stats` [N, C, 2] = per (sample, channel)
+    sum and sum of squares of x in float32, as the convolutions return them with want_stats."""
+    if not x.is_cuda or x.dtype not in (torch.float32, torch.bfloat16):
+        raise RuntimeError("group_norm_from_stats: CUDA float32 / bfloat16 tensors only")
+    if stats.shape != (x.shape[0], x.shape[1], 2) or stats.dtype != torch.float32 or stats.device != x.device:
+        raise RuntimeError(f"group_norm_from_stats: stats must be float32 [N, C, 2] on the input's GPU, got {tuple(stats.shape)}")
+    if x.shape[1] % groups != 0:
+        raise RuntimeError("group_norm_from_stats: groups must divide the channel count")
+    return _GroupNormFromStats.apply(x, stats.contiguous(), weight, bias, int(groups), float(eps))
+
+
+def channel_stats(x):
+    """float32 [N, C, 2]: per (sample, channel) sum and sum of squares of x (d2c_channel_stats)."""
+    lib = _lib.load()
+    x = x.contiguous()
+    N, C = x.shape[:2]
+    desc = _lib.GroupNormDesc(N, C, x[0, 0].numel(), 1, _DT[x.dtype], 0.0)
+    stats = torch.empty((N, C, 2), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.d2c_channel_stats(ctypes.byref(desc), _ptr(x), _ptr(stats), _stream(x.device))
+    _lib.check(rc, "channel_stats")
+    return stats
 
 
 class _DeformConv1dFunction(torch.autograd.Function):

@@ -447,6 +447,39 @@ int d2c_conv3d_sized_backward(const d2c_conv3d_desc *q, const d2c_size_map_desc 
     return D2C_OK;
 }
 
+static bool stats_fused(const d2c_conv3d_desc &q, const d2c_size_map_desc *z)
+{
+    return choose_algo(q, true) == D2C_ALGO_MFMA && d2c_tiled_forward_fills_stats(q) && (!z || sized_fused(q, false));
+}
+
+size_t d2c_conv3d_forward_stats_workspace_bytes(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
+{
+    if ((z ? sized_check(q, z) : d2c_conv3d_check(q)) != D2C_OK) return 0;
+    if (stats_fused(*q, z)) return d2c_tiled_forward_ws(*q, true);
+    return z ? d2c_conv3d_sized_forward_workspace_bytes(q, z) : d2c_conv3d_forward_workspace_bytes(q);
+}
+
+int d2c_conv3d_forward_stats(const d2c_conv3d_desc *q, const d2c_size_map_desc *z, const void *x, const void *offset,
+                             const void *mask, const void *weight, const void *bias, void *out, float *chan_stats,
+                             void *ws, size_t ws_bytes, void *stream)
+{
+    if (int rc = z ? sized_check(q, z) : d2c_conv3d_check(q)) return rc;
+    if (!x || !offset || !weight || !out || !chan_stats) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (q->dtype == D2C_F64) { d2c_set_error("output statistics: float32 or bfloat16 only"); return D2C_ERR_DTYPE; }
+    const int a = choose_algo(*q, false);
+    if (a < 0) return D2C_ERR_UNSUPPORTED;
+    // the kernels that add the sums up on their way: matrix-core family, offsets from a tensor or formed in the sampler
+    if (stats_fused(*q, z)) {
+        if (int rc = check_ws(d2c_tiled_forward_ws(*q, true), ws, ws_bytes)) return rc;
+        return d2c_tiled_forward(*q, x, offset, mask, weight, bias, out, ws, (hipStream_t)stream, z, chan_stats);
+    }
+    if (int rc = z ? d2c_conv3d_sized_forward(q, z, x, offset, mask, weight, bias, out, ws, ws_bytes, stream)
+                   : d2c_conv3d_forward(q, x, offset, mask, weight, bias, out, ws, ws_bytes, stream))
+        return rc;
+    const d2c_group_norm_desc g{q->N, q->Cout, q->Do * q->Ho * q->Wo, 1, q->dtype, 0.f};
+    return d2c_channel_stats(&g, out, chan_stats, stream);
+}
+
 int d2c_conv3d_corner_index(const d2c_conv3d_desc *q, const void *offset, int32_t *base, uint8_t *flags,
                             void *stream)
 {

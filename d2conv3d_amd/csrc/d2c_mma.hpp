@@ -260,9 +260,12 @@ template <bool AUX16> D2C_DEV void size_minus_one(const TiledShape &s, float *c)
 template <bool AUX16> D2C_DEV void size_tap_offsets(const TiledShape &s, int k, const float *sm1, float *o)
 {
     typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
-    const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
-#pragma unroll
-    for (int ax = 0; ax < 3; ax++) o[ax] = rnd<AT>(rnd<AT>(s.ss.base[ax][kq[ax]]) * sm1[ax]);
+    const int kz = k / (s.geo.kw * s.geo.kh), ky = (k / s.geo.kw) % s.geo.kh, kx = k % s.geo.kw;
+    const float b0 = s.ss.base[0][kz], b1 = s.ss.base[1][ky], b2 = s.ss.base[2][kx];
+    const float s0 = sm1[0], s1 = sm1[1], s2 = sm1[2];
+    o[0] = rnd<AT>(rnd<AT>(b0) * s0);
+    o[1] = rnd<AT>(rnd<AT>(b1) * s1);
+    o[2] = rnd<AT>(rnd<AT>(b2) * s2);
 }
 template <bool AUX16> D2C_DEV void tap_offsets_finish(const TiledShape &s, int k, float *c)
 {

@@ -7,7 +7,9 @@
 int d2c_fwd_out_tile(int og, int M, int groups);
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
-                         const void *bias, void *out, float *outacc, hipStream_t st);
+                         const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part);
+bool d2c_fwd_fills_stats(const TiledShape &s);
+size_t d2c_fwd_stats_ws(const TiledShape &s);
 int d2c_fwd_split(const TiledShape &s);
 
 bool d2c_tiled_bwd_data_supported(const TiledShape &s, int dtype);
@@ -346,7 +348,8 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 
 template <typename T>
 int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
-              const void *bias, void *out, void *ws, hipStream_t st, int nd = 3, const d2c_size_map_desc *sz = nullptr)
+              const void *bias, void *out, void *ws, hipStream_t st, int nd = 3, const d2c_size_map_desc *sz = nullptr,
+              float *stats = nullptr)
 {
     const TiledShape s = tiled_shape(q, nd, 0, sz);
     char *base = (char *)ws;
@@ -372,7 +375,9 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
                                (T *)(base + l.wp), s, total);
     }
     if (int rc = d2c_check_launch("pack_weight_fwd_kernel")) return rc;
-    return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, (float *)(base + l.outacc), st);
+    // (the per-tile sums of the output statistics go behind everything else in the workspace)
+    return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, (float *)(base + l.outacc), st,
+                                   stats, stats ? (float *)(base + l.total) : nullptr);
 }
 
 // grad_input by sample lists (see d2c_invlist.hip) needs the whole reduction over output
@@ -612,10 +617,11 @@ bool d2c_tiled_supported(const d2c_conv3d_desc &q)
 
 int d2c_tiled_algo(const d2c_conv3d_desc &q) { return is_depthwise(q) ? D2C_ALGO_DEPTHWISE : D2C_ALGO_MFMA; }
 
-size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q)
+size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q, bool with_stats)
 {
     const TiledShape s = tiled_shape(q);
-    return is_depthwise(q) ? dw_ws(q, s).total_fwd : fwd_ws(q, s).total;
+    if (is_depthwise(q)) return dw_ws(q, s).total_fwd;
+    return fwd_ws(q, s).total + (with_stats && d2c_fwd_fills_stats(s) ? d2c_fwd_stats_ws(s) : 0);
 }
 
 size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q, const d2c_size_map_desc *sz)
@@ -634,10 +640,16 @@ bool d2c_tiled_sized_supported(const d2c_conv3d_desc &q, bool backward)
 }
 
 int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
-                      const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz)
+                      const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz, float *stats)
 {
-    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 3, sz);
-    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 3, sz);
+    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats);
+    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats);
+}
+
+// The forward kernels of this description add up per-channel statistics of the output on their way.
+bool d2c_tiled_forward_fills_stats(const d2c_conv3d_desc &q)
+{
+    return !is_depthwise(q) && mfma_channels_ok(q) && d2c_fwd_fills_stats(tiled_shape(q));
 }
 
 int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,

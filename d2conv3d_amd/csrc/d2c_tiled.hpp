@@ -5,13 +5,17 @@
 
 bool d2c_tiled_supported(const d2c_conv3d_desc &q);
 int d2c_tiled_algo(const d2c_conv3d_desc &q);  // D2C_ALGO_MFMA or D2C_ALGO_DEPTHWISE
-size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q);
+size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q, bool with_stats = false);
 // `sz` != nullptr: the offsets are formed from a raw size map (`off` is that map [N, channels(mode), P], `goff` the
 // gradient with respect to it); only where d2c_tiled_sized_supported() says so.
 size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q, const d2c_size_map_desc *sz = nullptr);
 bool d2c_tiled_sized_supported(const d2c_conv3d_desc &q, bool backward);
+// `stats` != nullptr (only where d2c_tiled_forward_fills_stats() says so): fp32 [N][Cout][2], the sum and the sum of
+// squares of the stored output per (sample, channel).
+bool d2c_tiled_forward_fills_stats(const d2c_conv3d_desc &q);
 int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
-                      const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz = nullptr);
+                      const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz = nullptr,
+                      float *stats = nullptr);
 int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
                        const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
                        void *ws, hipStream_t st, const d2c_size_map_desc *sz = nullptr);

@@ -44,6 +44,12 @@ struct FwdArgs {
     // one time are at about the same steps and share their weight fragments in L2.  The pieces add into
     // `outacc`, here laid out [item - sk_full][output channel of the tile][position of the tile].
     int sk_items, sk_full, sk_ntile, sk_otiles, sk_cut;
+    // Statistics for a normalisation behind the convolution (GroupNorm), or NULL: the sum and the sum of squares of
+    // the values as stored, per position tile and output channel, fp32 [position tile][2][Cout][2] -- a tile of 64
+    // positions lies in one sample or straddles two (slot 0: the sample of its first position, slot 1: the next
+    // one); every entry has exactly one writer (no atomics: they would all land on the same few cache lines), and
+    // stats_reduce_kernel adds the tiles of a sample up.  Filled by the DMA-gather kernel and its finishing kernel.
+    float *stats;
 };
 
 // Tiles that are neighbours in space go to the same XCD (workgroups are dealt
@@ -377,17 +383,19 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     // turned into a table row (finish), possibly across a segment boundary: one set of constants for each.
     // (size-map source: the part of the offsets that the taps of a position share, size - 1 per axis, is formed
     // here once per work item; a step then costs three multiplications and no load)
-    struct PosC { int b, p, oz, oy, ox; bool valid; float sm1[3]; };
+    struct PosC { int b, p, oz, oy, ox; bool valid; float s0, s1, s2; };
     auto pos_of = [&](const SegWalk &w) {
-        PosC c{0, 0, 0, 0, 0, false, {0.f, 0.f, 0.f}};
+        PosC c{0, 0, 0, 0, 0, false, 0.f, 0.f, 0.f};
         const int m = w.tile * MT + ctid;
         c.valid = w.item >= 0 && m < s.M;
         if (c.valid) {
             c.b = m / s.P; c.p = m - c.b * s.P;
             c.ox = c.p % s.Wo; c.oy = (c.p / s.Wo) % s.Ho; c.oz = c.p / (s.Wo * s.Ho);
             if (s.ss.on && cwave) {
-                tap_offsets_issue<AUX16>(s, a.off, c.b, 0, 0, c.p, c.sm1);
-                size_minus_one<AUX16>(s, c.sm1);
+                float t[3];
+                tap_offsets_issue<AUX16>(s, a.off, c.b, 0, 0, c.p, t);
+                size_minus_one<AUX16>(s, t);
+                c.s0 = t[0]; c.s1 = t[1]; c.s2 = t[2];
             }
         }
         return c;
@@ -411,7 +419,10 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 const int k = w.st % s.K;
                 int bz, by, bx;
                 tap_base(s.geo, k, c.oz, c.oy, c.ox, bz, by, bx);
-                if (s.ss.on) size_tap_offsets<AUX16>(s, k, c.sm1, craw);
+                if (s.ss.on) {
+                    const float t[3] = {c.s0, c.s1, c.s2};
+                    size_tap_offsets<AUX16>(s, k, t, craw);
+                }
                 const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
                 live = t.live;
                 idx = (c.b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
@@ -563,6 +574,56 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                         if (oo < nvalid) atomicAdd(tp + oo * MT + pb * 32, acc[ob][pb][r]);
                         acc[ob][pb][r] = 0.f;
                     }
+        } else if (a.stats) {
+            // the same stores, and on the way the sum and the sum of squares of the stored values per output channel
+            // and sample slot: over the positions a lane holds, then over the 32 lanes of its half
+            const T *bias = reinterpret_cast<const T *>(a.bias);
+            const int b_lo = (w.tile * MT) / s.P;
+            bool okq[PB], hiq[PB];
+            T *opq[PB];
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++) {
+                const int m = w.tile * MT + wave_p * WPOS + pb * 32 + (elane & 31);
+                okq[pb] = m < s.M;
+                const int b = m / s.P;
+                hiq[pb] = b != b_lo;
+                opq[pb] = reinterpret_cast<T *>(a.out) + ((long)b * s.Cout + o0) * s.P + (m - b * s.P);
+            }
+            float *sp = a.stats + ((long)w.tile * 2 * s.Cout + o0) * 2;
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int oo = ob * 32 + 8 * (r >> 2) + (r & 3);
+                    float q4[4] = {0.f, 0.f, 0.f, 0.f};     // slot 0: sum, sum of squares; slot 1 likewise
+#pragma unroll
+                    for (int pb = 0; pb < PB; pb++) {
+                        if (okq[pb] && oo < nvalid) {
+                            float v = acc[ob][pb][r];
+                            if (bias) v += elem_to_f32<T>(bias[o0 + oo]);
+                            const T sv = f32_to_elem<T>(d2c_epilogue(v, s.act, s.act_scale));
+                            opq[pb][(long)oo * s.P] = sv;
+                            const float fv = elem_to_f32<T>(sv);
+                            q4[0] += hiq[pb] ? 0.f : fv; q4[1] += hiq[pb] ? 0.f : fv * fv;
+                            q4[2] += hiq[pb] ? fv : 0.f; q4[3] += hiq[pb] ? fv * fv : 0.f;
+                        }
+                        acc[ob][pb][r] = 0.f;
+                    }
+#pragma unroll
+                    for (int d = 1; d < 32; d <<= 1)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) q4[i] += __shfl_xor(q4[i], d, 64);
+                    if ((elane & 31) == 0 && oo < nvalid) {
+                        if (WAVES_P == 1) {
+                            sp[oo * 2] = q4[0]; sp[oo * 2 + 1] = q4[1];
+                            sp[(s.Cout + oo) * 2] = q4[2]; sp[(s.Cout + oo) * 2 + 1] = q4[3];
+                        } else {
+                            // (several wavefronts share a channel's positions: the slots were zeroed)
+                            atomicAdd(sp + oo * 2, q4[0]); atomicAdd(sp + oo * 2 + 1, q4[1]);
+                            atomicAdd(sp + (s.Cout + oo) * 2, q4[2]); atomicAdd(sp + (s.Cout + oo) * 2 + 1, q4[3]);
+                        }
+                    }
+                }
         } else {
             const T *bias = reinterpret_cast<const T *>(a.bias);
 #pragma unroll
@@ -691,16 +752,53 @@ __global__ void __launch_bounds__(256) fwd_dma_finish_kernel(FwdArgs a, int NT)
     const float *acc = a.outacc + (long)blockIdx.x * NT * MT;
     const T *bias = reinterpret_cast<const T *>(a.bias);
     T *out = reinterpret_cast<T *>(a.out);
+    const int b_lo = (tile * MT) / s.P;
+    static_assert(MT == 64, "one wavefront = the positions of one channel");
     for (int e = threadIdx.x; e < 32 * MT; e += 256) {
         const int ot = blockIdx.y * 32 + e / MT, pl = e % MT;
         const int ol = otile * NT + ot, m = tile * MT + pl;
-        if (ol < s.og && m < s.M) {
-            const int o = wg * s.og + ol, b = m / s.P, p = m - b * s.P;
+        float fv = 0.f;
+        const bool ok = ol < s.og && m < s.M;
+        const int o = wg * s.og + ol, b = ok ? m / s.P : b_lo, p = m - b * s.P;
+        if (ok) {
             float v = acc[(long)ot * MT + pl];
             if (bias) v += elem_to_f32<T>(bias[o]);
-            out[((long)b * s.Cout + o) * s.P + p] = f32_to_elem<T>(d2c_epilogue(v, s.act, s.act_scale));
+            const T sv = f32_to_elem<T>(d2c_epilogue(v, s.act, s.act_scale));
+            out[((long)b * s.Cout + o) * s.P + p] = sv;
+            fv = elem_to_f32<T>(sv);
+        }
+        if (a.stats) {
+            // (e / MT is uniform over a wavefront: its 64 lanes are the positions of one channel)
+            const bool hi = b != b_lo;
+            float q4[4] = {hi ? 0.f : fv, hi ? 0.f : fv * fv, hi ? fv : 0.f, hi ? fv * fv : 0.f};
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1)
+#pragma unroll
+                for (int i = 0; i < 4; i++) q4[i] += __shfl_xor(q4[i], d, 64);
+            if (pl == 0 && ol < s.og) {
+                float *sp = a.stats + ((long)tile * 2 * s.Cout + o) * 2;
+                sp[0] = q4[0]; sp[1] = q4[1];
+                sp[s.Cout * 2] = q4[2]; sp[s.Cout * 2 + 1] = q4[3];
+            }
         }
     }
+}
+
+// chan_stats[n][c] = sums over the position tiles of sample n (see FwdArgs::stats); one thread per (n, c)
+__global__ void __launch_bounds__(256) stats_reduce_kernel(const float *part, float *chan_stats, int N, int Cout, int P, int M)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N * Cout) return;
+    const int n = i / Cout, c = i - n * Cout;
+    const int t_lo = (int)(((long)n * P) / kDMT), t_hi = (int)((min((long)(n + 1) * P, (long)M) - 1) / kDMT);
+    float s0 = 0.f, s1 = 0.f;
+    for (int t = t_lo; t <= t_hi; t++) {
+        const int slot = n - (t * kDMT) / P;           // 0, or 1 for the tile that began in the sample before
+        const float *q = part + (((long)t * 2 + slot) * Cout + c) * 2;
+        s0 += q[0]; s1 += q[1];
+    }
+    chan_stats[2 * i] = s0;
+    chan_stats[2 * i + 1] = s1;
 }
 
 template <typename T, bool AUX16, int WO, int WP>
@@ -819,16 +917,31 @@ int d2c_fwd_split(const TiledShape &s)
     return (int)(want < S ? want : S);
 }
 
+// Whether the forward kernels of this shape add up per-channel statistics themselves (FwdArgs::stats): the
+// DMA-gather kernel, on samples of at least one position tile (a tile then meets at most two samples).
+bool d2c_fwd_fills_stats(const TiledShape &s) { return d2c_fwd_use_dma(s.og, s.M, s.groups) && s.P >= kDMT; }
+size_t d2c_fwd_stats_ws(const TiledShape &s)
+{
+    return d2c_align_up((size_t)((s.M + kDMT - 1) / kDMT) * 2 * s.Cout * 2 * sizeof(float));
+}
+
+// `stats` / `stats_part`: the [N][Cout][2] result and the per-tile scratch of d2c_fwd_stats_ws() bytes, or NULL.
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
-                         const void *bias, void *out, float *outacc, hipStream_t st)
+                         const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part)
 {
     const bool dma = d2c_fwd_use_dma(s.og, s.M, s.groups);
     const int nsplit = (outacc && !dma) ? d2c_fwd_split(s) : 1;
     const long n = (long)s.N * s.Cout * s.P;
     // the channels-last input is followed by a row of zeros (see forward_t)
     const unsigned zrow = (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T));
-    FwdArgs a{s, xcl, off, mask, wp, bias, out, nsplit > 1 ? outacc : nullptr, nsplit, zrow, 0, 0, 0, 0, 1};
+    FwdArgs a{s, xcl, off, mask, wp, bias, out, nsplit > 1 ? outacc : nullptr, nsplit, zrow, 0, 0, 0, 0, 1,
+              (dma && stats) ? stats_part : nullptr};
+    if (a.stats && d2c_fwd_out_tile(s.og, s.M, s.groups) != 512) {
+        // (the 256-channel tile has two wavefronts per channel, which add into their slots)
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(a.stats, d2c_fwd_stats_ws(s), st);
+    }
     if (nsplit > 1) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(outacc, (size_t)n * sizeof(float), st);
@@ -840,14 +953,20 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
     if (dma) {
         if (nt == 512) {
             if constexpr (sizeof(T) == 2) {
-                if (aux16) return launch_fwd_dma<T, true, 8, 1>(a, outacc, st);
+                if (aux16) rc = launch_fwd_dma<T, true, 8, 1>(a, outacc, st);
             }
-            return launch_fwd_dma<T, false, 8, 1>(a, outacc, st);
+            if (!aux16) rc = launch_fwd_dma<T, false, 8, 1>(a, outacc, st);
+        } else {
+            if constexpr (sizeof(T) == 2) {
+                if (aux16) rc = launch_fwd_dma<T, true, 4, 2>(a, outacc, st);
+            }
+            if (!aux16) rc = launch_fwd_dma<T, false, 4, 2>(a, outacc, st);
         }
-        if constexpr (sizeof(T) == 2) {
-            if (aux16) return launch_fwd_dma<T, true, 4, 2>(a, outacc, st);
-        }
-        return launch_fwd_dma<T, false, 4, 2>(a, outacc, st);
+        if (rc || !a.stats) return rc;
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        hipLaunchKernelGGL(stats_reduce_kernel, dim3((unsigned)((s.N * s.Cout + 255) / 256)), dim3(256), 0, st, a.stats,
+                           stats, s.N, s.Cout, s.P, s.M);
+        return d2c_check_launch("stats_reduce_kernel");
     } else {
         if constexpr (sizeof(T) == 2) {
             if (aux16) rc = launch_fwd_cfg<T, true>(a, nt, st);
@@ -863,6 +982,6 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
     return d2c_check_launch("fwd_finish_kernel");
 }
 template int d2c_tiled_fwd_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                          const void *, void *, float *, hipStream_t);
+                                          const void *, void *, float *, hipStream_t, float *, float *);
 template int d2c_tiled_fwd_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                         const void *, void *, float *, hipStream_t);
+                                         const void *, void *, float *, hipStream_t, float *, float *);

@@ -176,8 +176,12 @@ def _sized_forward(layer, input):
     else:
         size_raw, alpha = layer._get_size_and_alpha(deform_input)
     dc = layer.deform_conv
-    return deform_conv3d_sized(input, size_raw, alpha, dc.weight, dc.bias, layer._mode, layer.size_activation,
-                               dc.stride, dc.padding, dc.dilation, dc.groups, output_relu=dc.output_relu_scale)
+    out = deform_conv3d_sized(input, size_raw, alpha, dc.weight, dc.bias, layer._mode, layer.size_activation,
+                              dc.stride, dc.padding, dc.dilation, dc.groups, output_relu=dc.output_relu_scale,
+                              output_stats=dc.keep_output_stats)
+    if dc.keep_output_stats:
+        out, dc.last_output_stats = out
+    return out
 
 
 def _size_offsets(layer, size_raw):

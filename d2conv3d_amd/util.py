@@ -1,6 +1,7 @@
 """nn.Conv3d -> deformable layer replacement, mirroring
 ops/dconv-native/src/dconv_native/util.py and utils/replace.py:11-82.
 """
+import torch
 import torch.nn as nn
 
 from .modules import *  # noqa: F401,F403  (the reference's util.py re-exports the layer classes)
@@ -96,6 +97,51 @@ def fuse_output_activation(module):
                 continue
             conv.deform_conv.output_relu_scale = scale
             seq._modules[b] = nn.Identity()
+            fused += 1
+    return fused
+
+
+class ConvActGroupNorm(nn.Sequential):
+    """Sequential(deformable convolution, ReLU | ScaledReLU | Identity, GroupNorm) -- the `_conv` block of the
+    reference's refinement modules (network/modules/refinement.py:38-43) -- run as two kernels' worth of passes:
+    the convolution applies the activation where it stores its output and adds up the per-channel sums on the
+    way, and the normalisation is one pass over the output from those sums (no statistics pass).  Children keep
+    their places and names, so state-dict keys do not change.  CPU / float64 inputs take the plain sequence."""
+
+    def forward(self, input):
+        conv, act, norm = self[0], self[1], self[2]
+        dc = conv.deform_conv
+        if not input.is_cuda or input.dtype == torch.float64:
+            return norm(act(conv(input)))
+        from . import _ops
+        dc.keep_output_stats = True
+        try:
+            out = conv(input)            # the activation is folded into the convolution (output_relu_scale)
+            stats = dc.last_output_stats
+        finally:
+            dc.keep_output_stats = False
+            dc.last_output_stats = None
+        return _ops.group_norm_from_stats(out, stats, norm.weight, norm.bias, norm.num_groups, norm.eps)
+
+
+def fuse_conv_act_norm(module):
+    """Turns every nn.Sequential of exactly (D2Conv layer, nn.ReLU | ScaledReLU | nn.Identity, nn.GroupNorm) under
+    `module` into a ConvActGroupNorm (in place: same children, same state-dict keys).  Returns their number."""
+    fused = 0
+    fuse_output_activation(module)
+    for parent in list(module.modules()):
+        for name, seq in list(parent.named_children()):
+            if type(seq) is not nn.Sequential or len(seq) != 3:
+                continue
+            conv, act, norm = seq[0], seq[1], seq[2]
+            if not (isinstance(conv, _m._DConvBase) and isinstance(norm, nn.GroupNorm)):
+                continue
+            if not (isinstance(act, nn.Identity) and conv.deform_conv.output_relu_scale is not None):
+                continue
+            block = ConvActGroupNorm()
+            for n, child in seq.named_children():
+                block.add_module(n, child)
+            setattr(parent, name, block)
             fused += 1
     return fused
 

@@ -231,6 +231,37 @@ int d2c_conv3d_sized_backward(const d2c_conv3d_desc *desc, const d2c_size_map_de
                               void *grad_size_raw, void *grad_mask, void *grad_weight, void *grad_bias,
                               void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- normalisation behind the convolution ------------------------------------------------------------------
+ * Every deformable convolution of the reference's refinement modules is followed by an activation and a
+ * GroupNorm (network/modules/refinement.py:38-43: Sequential(ConvType, ActivationType, NormType)).
+ * d2c_conv3d_forward_stats is d2c_conv3d_forward (sdesc == NULL, `offset` = the offsets tensor) or
+ * d2c_conv3d_sized_forward (sdesc != NULL, `offset` = the raw size map) that also returns
+ *     chan_stats[n][c] = (sum_p out[n,c,p], sum_p out[n,c,p]^2)        float32 [N][Cout][2],
+ * of the values as stored (bias and epilogue applied, rounded to `dtype`).  The matrix-core kernels for wide
+ * weight groups add these sums up where they store the output (per position tile, without atomics; a small kernel
+ * adds the tiles of a sample up); other descriptions run d2c_channel_stats behind the convolution.  Workspace:
+ * d2c_conv3d_forward_stats_workspace_bytes().
+ * d2c_group_norm_forward / _backward are torch.nn.functional.group_norm and its gradients (biased variance,
+ * var = sumsq / m - mean^2 in float32) from such statistics: one pass over x each way plus a reduction pass for the
+ * backward sums; gamma, beta (may be NULL: 1, 0) and their gradients in `dtype`. */
+typedef struct d2c_group_norm_desc {
+    int32_t N, C, P;          /* samples, channels, positions per channel */
+    int32_t groups;           /* normalisation groups; must divide C */
+    int32_t dtype;            /* D2C_F32 or D2C_BF16 */
+    float eps;
+} d2c_group_norm_desc;
+size_t d2c_conv3d_forward_stats_workspace_bytes(const d2c_conv3d_desc *desc, const d2c_size_map_desc *sdesc);
+int d2c_conv3d_forward_stats(const d2c_conv3d_desc *desc, const d2c_size_map_desc *sdesc, const void *x,
+                             const void *offset, const void *mask, const void *weight, const void *bias, void *out,
+                             float *chan_stats, void *workspace, size_t workspace_bytes, void *stream);
+int d2c_channel_stats(const d2c_group_norm_desc *desc, const void *x, float *chan_stats, void *stream);
+int d2c_group_norm_forward(const d2c_group_norm_desc *desc, const void *x, const float *chan_stats, const void *gamma,
+                           const void *beta, void *y, void *stream);
+size_t d2c_group_norm_backward_workspace_bytes(const d2c_group_norm_desc *desc);
+int d2c_group_norm_backward(const d2c_group_norm_desc *desc, const void *grad_y, const void *x,
+                            const float *chan_stats, const void *gamma, void *grad_x, void *grad_gamma,
+                            void *grad_beta, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- plain depthwise conv3d (no sampling) ------------------------------------------------
  * The operator of the reference's second extension, ops/fast-depthwise-conv3d, which its
  * backbone uses for the channel-separated 3x3x3 convolutions (network/backbone/resnet.py:110):
