@@ -363,6 +363,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv", "c3_norm"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--offset-axes", type=int, default=7,
+                    help="mask of the axes the offsets displace along (1 z, 2 y, 4 x): 6 = the Spatial layers, 1 = the "
+                         "Temporal layers of the reference (3-D matrix-core workloads only; default all three)")
     ap.add_argument("--expanded-offsets", action="store_true",
                     help="dynamic-dilation workloads (c2_*): expand the dilation map to an offsets tensor first "
                          "and time the ordinary operator on it, instead of handing the map to the operator")
@@ -403,7 +406,7 @@ def main():
     if nd == 3:
         T_, H_, W_ = dims
         desc = _lib.Conv3dDesc(N, C, C, T_, H_, W_, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, groups, G, T_, H_, W_,
-                               code, code)
+                               code, code, 0, 1.0, args.offset_axes)
         kind = "conv3d"
         algo = _lib.ALGO_NAMES[lib.d2c_conv3d_algo(ctypes.byref(desc))]
     else:
@@ -571,6 +574,7 @@ def main():
                                + ("bf16 in / fp32 accumulate" if dt == "bf16" else "fp32"),
                    "offsets": ("formed in the sampler from the dilation map [N,3,T,H,W] (d2c_conv3d_sized_*)" if sized
                                else "offsets tensor [N,3*K*G,T,H,W]"),
+                   "offset_axes": args.offset_axes,
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "taps_outside_volume": taps,

@@ -37,7 +37,7 @@ class Conv3dDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "N", "Cin", "Cout", "D", "H", "W", "kd", "kh", "kw", "sd", "sh", "sw",
         "pd", "ph", "pw", "dd", "dh", "dw", "groups", "offset_groups", "Do", "Ho", "Wo",
-        "dtype", "aux_dtype", "epilogue")] + [("epilogue_scale", ctypes.c_float)]
+        "dtype", "aux_dtype", "epilogue")] + [("epilogue_scale", ctypes.c_float), ("offset_axes", ctypes.c_int32)]
 
 
 EPILOGUE_NONE, EPILOGUE_RELU = 0, 1

@@ -95,7 +95,7 @@ class _DeformConv3dFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, offset, alpha, weight, bias, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, offset_groups,
-                relu_scale=0.0, want_stats=False):
+                relu_scale=0.0, want_stats=False, offset_axes=7):
         lib = _lib.load()
         input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
         alpha = alpha.contiguous() if alpha is not None else None
@@ -105,7 +105,8 @@ class _DeformConv3dFunction(torch.autograd.Function):
         Do, Ho, Wo = offset.shape[2:]
         desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, sd, sh, sw, pd, ph, pw, dd, dh, dw,
                                groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype],
-                               _lib.EPILOGUE_RELU if relu_scale > 0 else _lib.EPILOGUE_NONE, float(relu_scale) or 1.0)
+                               _lib.EPILOGUE_RELU if relu_scale > 0 else _lib.EPILOGUE_NONE, float(relu_scale) or 1.0,
+                               int(offset_axes))
         _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d")
         dev = input.device
         out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
@@ -153,21 +154,24 @@ class _DeformConv3dFunction(torch.autograd.Function):
                                          _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
                                          _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d backward")
-        return (gx, goff, galpha, gw, gb) + (None,) * 13
+        return (gx, goff, galpha, gw, gb) + (None,) * 14
 
 
 def deform_conv3d(input, offset, alpha, weight, bias, stride_d, stride_h, stride_w, pad_d, pad_h, pad_w,
-                  dilation_d, dilation_h, dilation_w, groups, offset_groups, relu_scale=0.0, want_stats=False):
+                  dilation_d, dilation_h, dilation_w, groups, offset_groups, relu_scale=0.0, want_stats=False,
+                  offset_axes=7):
     """deform_conv3d of dconv3d.h:188-226; `alpha` and `bias` may be None.  `relu_scale` > 0 fuses
     relu_scale * relu(.) into the store of the output (see _DeformConv3dFunction).  `want_stats` also returns the
     float32 [N, Cout, 2] sums and sums of squares of the stored output per (sample, channel), added up by the
-    forward kernels where they store (the statistics a GroupNorm behind the convolution needs)."""
+    forward kernels where they store (the statistics a GroupNorm behind the convolution needs).  `offset_axes`: mask
+    of the axes (1 z, 2 y, 4 x) the offsets displace along; the others are taken as zero and their gradient
+    channels come back zero (matrix-core kernels only, see conv3d_algo)."""
     _check_common(3, input, offset, alpha, weight, bias, groups, offset_groups)
     input, offset, alpha, weight, bias = _unify(input, offset, alpha, weight, bias)
     return _DeformConv3dFunction.apply(
         input, offset, alpha, weight, bias, int(stride_d), int(stride_h), int(stride_w),
         int(pad_d), int(pad_h), int(pad_w), int(dilation_d), int(dilation_h), int(dilation_w),
-        int(groups), int(offset_groups), float(relu_scale), bool(want_stats))
+        int(groups), int(offset_groups), float(relu_scale), bool(want_stats), int(offset_axes))
 
 
 class _DeformConv3dSizedFunction(torch.autograd.Function):

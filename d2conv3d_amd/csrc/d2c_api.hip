@@ -233,6 +233,7 @@ int d2c_conv3d_check(const d2c_conv3d_desc *q)
                     && (long)q->N * q->offset_groups * 3 * K * P < (1L << 31)
                     && (long)q->Cout * (q->Cin / q->groups) * K < (1L << 31),
                 "tensor with 2^31 or more elements is not supported");
+    D2C_REQUIRE(q->offset_axes >= 0 && q->offset_axes <= 7, "offset_axes must be a mask of the axes z, y, x (0 .. 7)");
     D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || q->epilogue == D2C_EPILOGUE_RELU, "unknown epilogue %d", q->epilogue);
     D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || (q->epilogue_scale > 0.f && q->epilogue_scale < 3.0e38f),
                 "epilogue_scale must be positive and finite");
@@ -263,7 +264,21 @@ int d2c_conv1d_check(const d2c_conv1d_desc *q)
     return D2C_OK;
 }
 
+static int choose_algo_any_axes(const d2c_conv3d_desc &q, bool quiet);
+
+// fixed offset axes (the Spatial / Temporal layers) are served by the matrix-core kernels only
 static int choose_algo(const d2c_conv3d_desc &q, bool quiet)
+{
+    const int a = choose_algo_any_axes(q, quiet);
+    const bool fixed_axis = (q.offset_axes & 7) != 0 && (q.offset_axes & 7) != 7;
+    if (a >= 0 && fixed_axis && a != D2C_ALGO_MFMA) {
+        if (!quiet) d2c_set_error("offset_axes = %d is served by the matrix-core kernels only", q.offset_axes);
+        return -1;
+    }
+    return a;
+}
+
+static int choose_algo_any_axes(const d2c_conv3d_desc &q, bool quiet)
 {
     const int forced = g_algo_override.load();
     const bool tiled_ok = d2c_tiled_supported(q);

@@ -132,7 +132,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                 al = craw[3];
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
-                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+                const Tap3<float> t = tiled_tap3(s, bz, by, bx, o0, o1, o2);
                 idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
                 unsigned inr = t.inrange, auxlive = t.live;
                 fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
@@ -269,9 +269,9 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                                               s.ss.base[ax][kq[ax]] * (al * g_acc[r][ax]));
                         } else if (a.goff && s.nd == 3) {
                             const long ob = 3 * ab - 2 * (long)p;
-                            st_aux(a.goff, ob, s.adt, al * g_acc[r][0]);
-                            st_aux(a.goff, ob + s.P, s.adt, al * g_acc[r][1]);
-                            st_aux(a.goff, ob + 2 * (long)s.P, s.adt, al * g_acc[r][2]);
+                            st_aux(a.goff, ob, s.adt, (s.axes & 1) ? al * g_acc[r][0] : 0.f);
+                            st_aux(a.goff, ob + s.P, s.adt, (s.axes & 2) ? al * g_acc[r][1] : 0.f);
+                            st_aux(a.goff, ob + 2 * (long)s.P, s.adt, (s.axes & 4) ? al * g_acc[r][2] : 0.f);
                         } else if (a.goff) {
                             st_aux(a.goff, ab, s.adt, al * g_acc[r][2]);
                         }

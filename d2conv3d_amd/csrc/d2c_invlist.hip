@@ -42,7 +42,7 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
         load_offsets(s, off, b, g, k, p, o0, o1, o2);
         int bz, by, bx;
         tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
-        const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+        const Tap3<float> t = tiled_tap3(s, bz, by, bx, o0, o1, o2);
         if (!t.live) continue;
         InvEntry e;
         e.p = p; e.k = k; e.hz = t.hz; e.hy = t.hy; e.hx = t.hx;
@@ -65,7 +65,7 @@ invlist_pass_kernel(TiledShape s, const void *off, const void *mask, int *counts
         load_offsets(s, off, b, g, k, p, o0, o1, o2);
         int bz, by, bx;
         tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
-        const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+        const Tap3<float> t = tiled_tap3(s, bz, by, bx, o0, o1, o2);
         if (!t.live) continue;
         const int bin = bin_of(s, b, g, t.z0, t.y0, t.x0);
         const int n = atomicAdd(&counts[bin], 1);

@@ -214,9 +214,20 @@ struct TiledShape {
     int act;              // forward epilogue: 0 none, 1 act_scale * max(v, 0)
     float act_scale;
     TapGeom geo;
+    int axes;             // bit a set: sampling points are displaced along axis a (0 z, 1 y, 2 x); 7 = all
+    unsigned keep;        // corners that can have a non-zero weight: with an axis fixed, those on its near plane
     SizeSrc ss;           // offsets formed from a size map instead of read from a tensor
     FastDiv dP, dHW, dW;  // divisions by P, Ho * Wo and Wo
 };
+
+// make_tap3 for the tiled kernels: corners that a fixed axis leaves with weight zero are not fetched.
+D2C_DEV Tap3<float> tiled_tap3(const TiledShape &s, int bz, int by, int bx, float oz, float oy, float ox)
+{
+    Tap3<float> t = make_tap3<float>(bz, by, bx, oz, oy, ox, s.D, s.H, s.W);
+    t.live &= s.keep;
+    t.inrange &= s.keep;
+    return t;
+}
 
 // The three values a sampling point needs, requested early (issue) and turned into offsets late (finish):
 // the offsets themselves, or the raw sizes of the position (0 for an axis the mode does not predict).
@@ -240,9 +251,12 @@ D2C_DEV void tap_offsets_issue(const TiledShape &s, const void *off, int b, int 
     const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
     if (s.nd == 3) {
         const long ob = 3 * ab - 2 * (long)p;   // ((b*G+g)*K+k)*3*P + p
-        c[0] = ld_auxT<AUX16>(off, ob);
-        c[1] = ld_auxT<AUX16>(off, ob + s.P);
-        c[2] = ld_auxT<AUX16>(off, ob + 2 * (long)s.P);
+        // (all three are requested, a fixed axis is dropped by a select: no branches between the loads)
+        const float v0 = ld_auxT<AUX16>(off, ob), v1 = ld_auxT<AUX16>(off, ob + s.P);
+        const float v2 = ld_auxT<AUX16>(off, ob + 2 * (long)s.P);
+        c[0] = (s.axes & 1) ? v0 : 0.f;
+        c[1] = (s.axes & 2) ? v1 : 0.f;
+        c[2] = (s.axes & 4) ? v2 : 0.f;
     } else {
         c[0] = 0.f; c[1] = 0.f;
         c[2] = ld_auxT<AUX16>(off, ab);
@@ -399,9 +413,9 @@ D2C_DEV void load_offsets(const TiledShape &s, const void *off, int b, int g, in
     }
     if (s.nd == 3) {
         const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
-        o0 = ld_aux(off, ob, s.adt);
-        o1 = ld_aux(off, ob + s.P, s.adt);
-        o2 = ld_aux(off, ob + 2 * (long)s.P, s.adt);
+        o0 = (s.axes & 1) ? ld_aux(off, ob, s.adt) : 0.f;
+        o1 = (s.axes & 2) ? ld_aux(off, ob + s.P, s.adt) : 0.f;
+        o2 = (s.axes & 4) ? ld_aux(off, ob + 2 * (long)s.P, s.adt) : 0.f;
     } else {
         o0 = 0.f; o1 = 0.f;
         o2 = ld_aux(off, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt);

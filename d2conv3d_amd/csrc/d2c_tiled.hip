@@ -71,7 +71,7 @@ d2c_conv3d_desc as_3d(const d2c_conv1d_desc &q)
     r.kd = 1; r.kh = 1; r.kw = q.k; r.sd = 1; r.sh = 1; r.sw = q.s; r.pd = 0; r.ph = 0; r.pw = q.p;
     r.dd = 1; r.dh = 1; r.dw = q.d; r.groups = q.groups; r.offset_groups = q.offset_groups;
     r.Do = 1; r.Ho = 1; r.Wo = q.Lo; r.dtype = q.dtype; r.aux_dtype = q.aux_dtype;
-    r.epilogue = D2C_EPILOGUE_NONE; r.epilogue_scale = 1.f;
+    r.epilogue = D2C_EPILOGUE_NONE; r.epilogue_scale = 1.f; r.offset_axes = 0;
     return r;
 }
 
@@ -95,6 +95,11 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0, con
     s.adt = q.aux_dtype;
     s.act = q.epilogue; s.act_scale = q.epilogue_scale;
     s.P = q.Do * q.Ho * q.Wo; s.vol = q.D * q.H * q.W; s.M = q.N * s.P;
+    s.axes = (nd == 3 && (q.offset_axes & 7)) ? (q.offset_axes & 7) : 7;
+    s.keep = 0xffu;
+    if (!(s.axes & 1)) s.keep &= 0x0fu;     // z fixed: dz = 0 corners
+    if (!(s.axes & 2)) s.keep &= 0x33u;     // y fixed: dy = 0
+    if (!(s.axes & 4)) s.keep &= 0x55u;     // x fixed: dx = 0
     s.dP = make_fastdiv(s.P); s.dHW = make_fastdiv(q.Ho * q.Wo); s.dW = make_fastdiv(q.Wo);
     const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
     s.ogp = (s.og + nt - 1) / nt * nt;

@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                 al = a.mask ? ld_aux(a.mask, (((long)cbatch * s.G + g) * s.K + k) * s.P + cp, s.adt) : 1.f;
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
-                const Tap3<float> t = make_tap3<float>(bz, by, bx, o0, o1, o2, s.D, s.H, s.W);
+                const Tap3<float> t = tiled_tap3(s, bz, by, bx, o0, o1, o2);
                 idx = (cbatch * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
                 unsigned inr = t.inrange, auxlive = t.live;
                 fr[0] = t.lz; fr[1] = t.ly; fr[2] = t.lx; fr[3] = t.hz; fr[4] = t.hy; fr[5] = t.hx;
@@ -368,7 +368,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                                 if (a.goff && s.nd == 3) {
                                     const long ob = 3 * ab - 2 * (long)p;
 #pragma unroll
-                                    for (int ax = 0; ax < 3; ax++) atomicAdd(a.auxoff + ob + ax * (long)s.P, g_acc[i][ax]);
+                                    for (int ax = 0; ax < 3; ax++)
+                                        if ((s.axes >> ax) & 1) atomicAdd(a.auxoff + ob + ax * (long)s.P, g_acc[i][ax]);
                                 } else if (a.goff) {
                                     atomicAdd(a.auxoff + ab, g_acc[i][2]);
                                 }
@@ -378,7 +379,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 #pragma unroll
                                 for (int ax = 0; ax < 3; ax++) {
                                     const long oi = ob + ax * (long)s.P;
-                                    st_aux(a.goff, oi, s.adt, g_acc[i][ax] + (a.add_aux ? ld_aux(a.goff, oi, s.adt) : 0.f));
+                                    st_aux(a.goff, oi, s.adt, ((s.axes >> ax) & 1)
+                                               ? g_acc[i][ax] + (a.add_aux ? ld_aux(a.goff, oi, s.adt) : 0.f) : 0.f);
                                 }
                             } else if (a.goff) {
                                 st_aux(a.goff, ab, s.adt, g_acc[i][2] + (a.add_aux ? ld_aux(a.goff, ab, s.adt) : 0.f));
@@ -804,7 +806,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
 #pragma unroll
                 for (int ax = 0; ax < 3; ax++) craw[ax] = rnd<AT>(sbase[ax] * craw[ax]);
             }
-            const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
+            const Tap3<float> t = tiled_tap3(s, bz, by, bx, craw[0], craw[1], craw[2]);
             live = t.live;
             idx = (cb_ * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
 #pragma unroll

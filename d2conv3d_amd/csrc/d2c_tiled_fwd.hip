@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
                 tap_offsets_finish<AUX16>(s, k, craw);
-                const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
+                const Tap3<float> t = tiled_tap3(s, bz, by, bx, craw[0], craw[1], craw[2]);
                 live = t.live;
                 idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
 #pragma unroll
@@ -423,7 +423,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                     const float t[3] = {c.s0, c.s1, c.s2};
                     size_tap_offsets<AUX16>(s, k, t, craw);
                 }
-                const Tap3<float> t = make_tap3<float>(bz, by, bx, craw[0], craw[1], craw[2], s.D, s.H, s.W);
+                const Tap3<float> t = tiled_tap3(s, bz, by, bx, craw[0], craw[1], craw[2]);
                 live = t.live;
                 idx = (c.b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
 #pragma unroll

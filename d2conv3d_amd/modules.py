@@ -129,23 +129,53 @@ class MDConv3d(_DConvBase):
             nn.init.zeros_(self.deform_params.bias)
 
 
-class _SpatialMixin:
+def _fixed_axes_in_kernel(layer, input, offsets, alpha):
+    """Whether the operator itself can hold the offsets of some axes at zero (descriptor field offset_axes: the
+    matrix-core kernels then skip those offset channels and the corners that get weight zero) instead of the
+    reference's overwrite of a cloned offsets tensor."""
+    if not layer.fixed_axes_in_kernel or not input.is_cuda or input.dtype not in (torch.float32, torch.bfloat16):
+        return False
+    from . import _ops
+    dc = layer.deform_conv
+    return _ops.conv3d_algo(input, offsets, alpha, dc.weight, dc.stride, dc.padding, dc.dilation, dc.groups,
+                            dc.offset_groups) == "mfma"
+
+
+class _AxesMixin:
+    """dconv_native/modules.py:87-120: the Spatial layers do not displace along the temporal axis (offset channels
+    0, 3, 6, ... zero), the Temporal layers displace along it only."""
+    _offset_axes = 7              # 1 z | 2 y | 4 x
+    fixed_axes_in_kernel = True
+
+    def forward(self, input):
+        deform_input = input if self.norm is None else self.norm(input)
+        if self.checkpoint_deformation and torch.is_grad_enabled():
+            offsets, alpha = checkpoint(super()._get_deformation, deform_input, use_reentrant=False)
+        else:
+            offsets, alpha = super()._get_deformation(deform_input)
+        if _fixed_axes_in_kernel(self, input, offsets, alpha):
+            return self.deform_conv(input, offsets, alpha, offset_axes=self._offset_axes)
+        offsets = offsets.clone()
+        for a in range(3):
+            if not (self._offset_axes >> a) & 1:
+                offsets[:, a::3] = 0
+        return self.deform_conv(input, offsets, alpha)
+
     def _get_deformation(self, input):
-        # modules.py:87-101: no displacement along the temporal axis
         offsets, alpha = super()._get_deformation(input)
         offsets = offsets.clone()
-        offsets[:, ::3] = 0
+        for a in range(3):
+            if not (self._offset_axes >> a) & 1:
+                offsets[:, a::3] = 0
         return offsets, alpha
 
 
-class _TemporalMixin:
-    def _get_deformation(self, input):
-        # modules.py:104-120: displacement along the temporal axis only
-        offsets, alpha = super()._get_deformation(input)
-        offsets = offsets.clone()
-        offsets[:, 1::3] = 0
-        offsets[:, 2::3] = 0
-        return offsets, alpha
+class _SpatialMixin(_AxesMixin):
+    _offset_axes = 6
+
+
+class _TemporalMixin(_AxesMixin):
+    _offset_axes = 1
 
 
 class SpatialDConv3d(_SpatialMixin, DConv3d):

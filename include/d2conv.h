@@ -82,6 +82,14 @@ typedef struct d2c_conv3d_desc {
      * to the value before the activation (grad_out * epilogue_scale where out > 0, else 0). */
     int32_t epilogue;     /* D2C_EPILOGUE_NONE or D2C_EPILOGUE_RELU */
     float epilogue_scale;
+    /* Which axes the sampling points are displaced along: bit 0 = z (temporal), bit 1 = y, bit 2 = x; 0 means all
+     * three.  For a cleared axis the offsets are taken as zero whatever the tensor holds, and its grad_offset
+     * channels come back zero: the Spatial (y, x: 6) and Temporal (z: 1) layers of the reference, which overwrite
+     * those channels of a cloned offsets tensor (dconv_native/modules.py:87-120).  With an axis fixed a sampling
+     * point sits on a voxel plane of it and the four corners on the far plane have weight zero; the kernels do not
+     * fetch them.  Served by the matrix-core kernels only: other descriptions answer D2C_ERR_UNSUPPORTED (zero the
+     * channels in a copy of the tensor instead). */
+    int32_t offset_axes;
 } d2c_conv3d_desc;
 
 typedef struct d2c_conv1d_desc {
