@@ -59,7 +59,7 @@ D2C_DEV float sum_over_8_lanes(float v)
     return dpp_add<0x141>(v); // row_half_mirror
 }
 
-template <typename T, bool AUX16>
+template <typename T, bool AUX16, bool SIZED>
 __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a)
 {
     constexpr int MT = kMT;
@@ -112,7 +112,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     auto coords_issue = [&](int k) {
         if (cvalid) {
             const long ab = (((long)cb * s.G + g) * s.K + k) * s.P + cp;
-            tap_offsets_issue<AUX16>(s, a.off, cb, g, k, cp, craw);
+            tap_offsets_issue<AUX16, SIZED>(s, a.off, cb, g, k, cp, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
         }
     };
@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
             float al = 0.f;
             int idx = 0, flag = 0;
             if (cvalid) {
-                tap_offsets_finish<AUX16>(s, k, craw);
+                tap_offsets_finish<AUX16, SIZED>(s, k, craw);
                 const float o0 = craw[0], o1 = craw[1], o2 = craw[2];
                 al = craw[3];
                 int bz, by, bx;
@@ -258,7 +258,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                         const float al = al_r[r];
                         const int b = m / s.P, p = m - b * s.P;
                         const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
-                        if (a.gsize) {
+                        if (SIZED && a.gsize) {
                             // size-map source: d(offset_a) / d(size_a) = base_a[k_a]; the taps of a position add up
                             // (fp32 atomics into [N][3][P], finished by size_grad_finish_kernel)
                             const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
@@ -306,10 +306,17 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
     D2cProfScope prof(D2C_PROF_BWD_AUX, st);
+    const dim3 blk(64 * kWavesPerBlock);
     if constexpr (sizeof(T) == 2) {
-        if (aux16) hipLaunchKernelGGL((aux_grad_kernel<T, true>), grid, dim3(64 * kWavesPerBlock), 0, st, a);
+        if (aux16) {
+            if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, true, true>), grid, blk, 0, st, a);
+            else hipLaunchKernelGGL((aux_grad_kernel<T, true, false>), grid, blk, 0, st, a);
+        }
     }
-    if (!aux16) hipLaunchKernelGGL((aux_grad_kernel<T, false>), grid, dim3(64 * kWavesPerBlock), 0, st, a);
+    if (!aux16) {
+        if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, false, true>), grid, blk, 0, st, a);
+        else hipLaunchKernelGGL((aux_grad_kernel<T, false, false>), grid, blk, 0, st, a);
+    }
     return d2c_check_launch("aux_grad_kernel");
 }
 template int d2c_aux_grad_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,

@@ -231,15 +231,17 @@ D2C_DEV Tap3<float> tiled_tap3(const TiledShape &s, int bz, int by, int bx, floa
 
 // The three values a sampling point needs, requested early (issue) and turned into offsets late (finish):
 // the offsets themselves, or the raw sizes of the position (0 for an axis the mode does not predict).
-template <bool AUX16>
+// (SIZED is a compile-time property of the kernels: the ones that read an offsets tensor carry none of the size-map
+// code, which would cost their coordinate wavefronts, the critical ones at small tiles, several per cent)
+template <bool AUX16, bool SIZED>
 D2C_DEV void tap_offsets_issue(const TiledShape &s, const void *off, int b, int g, int k, int p, float *c)
 {
-    if (s.ss.on == 2) {
-        const float *f = reinterpret_cast<const float *>(off) + (long)b * 3 * s.P + p;
-        c[0] = f[0]; c[1] = f[s.P]; c[2] = f[2 * (long)s.P];
-        return;
-    }
-    if (s.ss.on) {
+    if constexpr (SIZED) {
+        if (s.ss.on == 2) {
+            const float *f = reinterpret_cast<const float *>(off) + (long)b * 3 * s.P + p;
+            c[0] = f[0]; c[1] = f[s.P]; c[2] = f[2 * (long)s.P];
+            return;
+        }
         const int nc = mode_channels(s.ss.mode);
 #pragma unroll
         for (int ax = 0; ax < 3; ax++) {
@@ -281,11 +283,12 @@ template <bool AUX16> D2C_DEV void size_tap_offsets(const TiledShape &s, int k, 
     o[1] = rnd<AT>(rnd<AT>(b1) * s1);
     o[2] = rnd<AT>(rnd<AT>(b2) * s2);
 }
-template <bool AUX16> D2C_DEV void tap_offsets_finish(const TiledShape &s, int k, float *c)
+template <bool AUX16, bool SIZED> D2C_DEV void tap_offsets_finish(const TiledShape &s, int k, float *c)
 {
-    if (!s.ss.on) return;
-    if (s.ss.on == 1) size_minus_one<AUX16>(s, c);
-    size_tap_offsets<AUX16>(s, k, c, c);
+    if constexpr (SIZED) {
+        if (s.ss.on == 1) size_minus_one<AUX16>(s, c);
+        size_tap_offsets<AUX16>(s, k, c, c);
+    }
 }
 
 // The forward kernels' last step before a value is stored (NaN stays NaN, as in torch's relu).
@@ -402,11 +405,11 @@ D2C_DEV void load_offsets(const TiledShape &s, const void *off, int b, int g, in
     if (s.ss.on) {
         float c[3];
         if (s.adt == D2C_BF16) {
-            tap_offsets_issue<true>(s, off, b, g, k, p, c);
-            tap_offsets_finish<true>(s, k, c);
+            tap_offsets_issue<true, true>(s, off, b, g, k, p, c);
+            tap_offsets_finish<true, true>(s, k, c);
         } else {
-            tap_offsets_issue<false>(s, off, b, g, k, p, c);
-            tap_offsets_finish<false>(s, k, c);
+            tap_offsets_issue<false, true>(s, off, b, g, k, p, c);
+            tap_offsets_finish<false, true>(s, k, c);
         }
         o0 = c[0]; o1 = c[1]; o2 = c[2];
         return;

@@ -720,7 +720,7 @@ struct BwdWeightDmaArgs {
     unsigned zrow;       // byte offset (from xcl) of a 128-byte row of zeros: what dead corners read
 };
 
-template <typename T, bool AUX16>
+template <typename T, bool AUX16, bool SIZED>
 __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(BwdWeightDmaArgs aa)
 {
     constexpr int MT = kWDT;
@@ -746,7 +746,10 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool worker = wave < 8;
-    const int st = blockIdx.x;                 // step = chunk * K + tap
+    // step = chunk * K + tap.  Workgroups are dealt round-robin to the 8 XCDs; an XCD takes a contiguous range of
+    // the steps, i.e. the taps of one or two channel chunks: its L2 then holds the corner rows of those channels only
+    // (one eighth of the input at 8 chunks) instead of all of them
+    const int st = xcd_swizzle(blockIdx.x, gridDim.x);
     const int otile = blockIdx.y;
     const int wg = blockIdx.z / a.split, sp = blockIdx.z % a.split;
     const int j = st / s.K, k = st - j * s.K;
@@ -778,12 +781,12 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
         if (cvalid) {
             cb_ = fdiv((int)m, s.dP); cp_ = (int)m - cb_ * s.P;      // (m < N * P < 2^31)
             const long ab = (((long)cb_ * s.G + g) * s.K + k) * s.P + cp_;
-            tap_offsets_issue<AUX16>(s, a.off, cb_, g, k, cp_, craw);
+            tap_offsets_issue<AUX16, SIZED>(s, a.off, cb_, g, k, cp_, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
         }
     };
     float sbase[3] = {0.f, 0.f, 0.f};   // kernel-grid coordinates of this workgroup's tap (size-map source)
-    if (s.ss.on) {
+    if constexpr (SIZED) {
         typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
         const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
 #pragma unroll
@@ -799,7 +802,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
             const int oy = fdiv(rem, s.dW), ox = rem - oy * s.Wo;
             int bz, by, bx;
             tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
-            if (s.ss.on) {
+            if constexpr (SIZED) {
                 // size-map source: offsets = base_a[k_a] * (size_a - 1); the tap is this workgroup's own
                 typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
                 if (s.ss.on == 1) size_minus_one<AUX16>(s, craw);
@@ -1406,20 +1409,23 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         bool aux16 = false;
         if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
-        if constexpr (sizeof(T) == 2) {
-            if (aux16) {
-                if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, true>,
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-                    return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_weight_dma_kernel)");
-                hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, true>), grid, dim3(kThreads + 64), lds, st, a);
-            }
-        }
-        if (!aux16) {
-            if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, false>,
+        auto go = [&](auto aux_c, auto sized_c) -> bool {
+            constexpr bool A16 = decltype(aux_c)::value, SZ = decltype(sized_c)::value;
+            if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, A16, SZ>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-                return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_weight_dma_kernel)");
-            hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, false>), grid, dim3(kThreads + 64), lds, st, a);
+                return false;
+            hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, A16, SZ>), grid, dim3(kThreads + 64), lds, st, a);
+            return true;
+        };
+        const bool sized = s.ss.on != 0;
+        bool ok;
+        if constexpr (sizeof(T) == 2) {
+            if (aux16) ok = sized ? go(std::true_type{}, std::true_type{}) : go(std::true_type{}, std::false_type{});
+            else ok = sized ? go(std::false_type{}, std::true_type{}) : go(std::false_type{}, std::false_type{});
+        } else {
+            ok = sized ? go(std::false_type{}, std::true_type{}) : go(std::false_type{}, std::false_type{});
         }
+        if (!ok) return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_weight_dma_kernel)");
     }
     if (int rc = d2c_check_launch("tiled_bwd_weight_dma_kernel")) return rc;
     D2cProfScope prof(D2C_PROF_PACK, st);

@@ -61,7 +61,7 @@ D2C_DEV int xcd_swizzle(int bid, int n)
     return x * q + (x < r ? x : r) + idx;
 }
 
-template <typename T, bool AUX16, int MT, int WAVES_O, int WAVES_P>
+template <typename T, bool AUX16, int MT, int WAVES_O, int WAVES_P, bool SIZED>
 __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
 {
     constexpr int VEC = Elem<T>::VEC;
@@ -109,7 +109,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
         if (tid < MT && cvalid) {
             const int j = st / s.K, k = st - j * s.K;
             const int g = (wg * s.cg + j * BKC) / s.cpg;
-            tap_offsets_issue<AUX16>(s, a.off, cb, g, k, cp, craw);
+            tap_offsets_issue<AUX16, SIZED>(s, a.off, cb, g, k, cp, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, (((long)cb * s.G + g) * s.K + k) * s.P + cp) : 1.f;
         }
     };
@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
                 const int k = st % s.K;
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
-                tap_offsets_finish<AUX16>(s, k, craw);
+                tap_offsets_finish<AUX16, SIZED>(s, k, craw);
                 const Tap3<float> t = tiled_tap3(s, bz, by, bx, craw[0], craw[1], craw[2]);
                 live = t.live;
                 idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
@@ -323,7 +323,7 @@ D2C_DEV bool seg_advance(SegWalk &w, const int4 *s_seg, int nseg)
 
 // (The LDS regions are passed as restrict-qualified pointers: that gives their accesses alias scopes, without
 // which the compiler makes every LDS store wait for all DMA transfers in flight, whatever region they fill.)
-template <typename T, bool AUX16, int WAVES_O, int WAVES_P>
+template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED>
 D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, unsigned char *__restrict__ s_tile,
                           float *__restrict__ s_w, int *__restrict__ s_idx, int *__restrict__ s_flag,
                           int4 *__restrict__ s_seg)
@@ -391,9 +391,9 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         if (c.valid) {
             c.b = m / s.P; c.p = m - c.b * s.P;
             c.ox = c.p % s.Wo; c.oy = (c.p / s.Wo) % s.Ho; c.oz = c.p / (s.Wo * s.Ho);
-            if (s.ss.on && cwave) {
+            if (SIZED && cwave) {
                 float t[3];
-                tap_offsets_issue<AUX16>(s, a.off, c.b, 0, 0, c.p, t);
+                tap_offsets_issue<AUX16, true>(s, a.off, c.b, 0, 0, c.p, t);
                 size_minus_one<AUX16>(s, t);
                 c.s0 = t[0]; c.s1 = t[1]; c.s2 = t[2];
             }
@@ -406,7 +406,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
             const int j = w.st / s.K, k = w.st - j * s.K;
             const int g = (w.wg * s.cg + j * BKC) / s.cpg;
             const long ab = (((long)c.b * s.G + g) * s.K + k) * s.P + c.p;
-            if (!s.ss.on) tap_offsets_issue<AUX16>(s, a.off, c.b, g, k, c.p, craw);
+            if constexpr (!SIZED) tap_offsets_issue<AUX16, false>(s, a.off, c.b, g, k, c.p, craw);
             craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
         }
     };
@@ -419,7 +419,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 const int k = w.st % s.K;
                 int bz, by, bx;
                 tap_base(s.geo, k, c.oz, c.oy, c.ox, bz, by, bx);
-                if (s.ss.on) {
+                if constexpr (SIZED) {
                     const float t[3] = {c.s0, c.s1, c.s2};
                     size_tap_offsets<AUX16>(s, k, t, craw);
                 }
@@ -725,7 +725,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     }
 }
 
-template <typename T, bool AUX16, int WAVES_O, int WAVES_P>
+template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED>
 __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
 {
     constexpr int MT = kDMT;
@@ -737,7 +737,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
     __shared__ int s_idx[3 * MT];                                     // [3][MT]
     __shared__ int s_flag[3 * MT];                                    // [3][MT]
     __shared__ int4 s_seg[2 * kMaxSeg];                               // [kMaxSeg][2]
-    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P>(a, s_raw, s_tile, s_w, s_idx, s_flag, s_seg);
+    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P, SIZED>(a, s_raw, s_tile, s_w, s_idx, s_flag, s_seg);
 }
 
 // out = fp32 tile + bias for the items whose steps were shared out (see FwdArgs).  One block = 32 output
@@ -804,6 +804,7 @@ __global__ void __launch_bounds__(256) stats_reduce_kernel(const float *part, fl
 template <typename T, bool AUX16, int WO, int WP>
 int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
 {
+    const bool sized = a.s.ss.on != 0;
     constexpr int NT = 64 * WO;
     const int ncu = d2c_num_cus();
     if (ncu <= 0) return D2C_ERR_LAUNCH;
@@ -839,7 +840,8 @@ int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
     {
         const int nwg = nshare ? ncu : (a.sk_items < nwg_whole ? a.sk_items : nwg_whole);
         D2cProfScope prof(D2C_PROF_FWD, st);
-        hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        else hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         if (int rc = d2c_check_launch("tiled_fwd_dma_kernel")) return rc;
     }
     if (nshare) {
@@ -869,7 +871,8 @@ int launch_fwd(const FwdArgs &a, hipStream_t st)
     const int NT = 64 * WO;
     dim3 grid(ntile, a.s.ogp / NT * a.nsplit, a.s.groups);
     D2cProfScope prof(D2C_PROF_FWD, st);
-    hipLaunchKernelGGL((tiled_fwd_kernel<T, AUX16, MT, WO, WP>), grid, dim3(kThreads), 0, st, a);
+    if (a.s.ss.on) hipLaunchKernelGGL((tiled_fwd_kernel<T, AUX16, MT, WO, WP, true>), grid, dim3(kThreads), 0, st, a);
+    else hipLaunchKernelGGL((tiled_fwd_kernel<T, AUX16, MT, WO, WP, false>), grid, dim3(kThreads), 0, st, a);
     return d2c_check_launch("tiled_fwd_kernel");
 }
 
