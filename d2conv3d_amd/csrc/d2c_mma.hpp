@@ -205,6 +205,7 @@ struct TiledShape {
     int N, Cin, Cout, D, H, W, K, G, groups, Do, Ho, Wo;
     int cg, og, cpg;      // channels per weight group (in / out), per offset group
     int nchunk;           // chunks per weight group = cg / BKC
+    int bkc, cpc;         // channels per chunk (BKC); consecutive chunks of a weight group that share an offset group
     int ogp;              // og rounded up to the output tile width
     int adt;
     int P, vol;           // output positions / input voxels per sample
@@ -289,6 +290,102 @@ template <bool AUX16, bool SIZED> D2C_DEV void tap_offsets_finish(const TiledSha
         if (s.ss.on == 1) size_minus_one<AUX16>(s, c);
         size_tap_offsets<AUX16>(s, k, c, c);
     }
+}
+
+// ---- the coordinate wavefront of the DMA-gather kernels ---------------------------------------------------------
+// One wavefront per workgroup turns sampling points into table rows (8 corner weights, the element offset of corner
+// 000, the corners to fetch); an iteration of the workgroup cannot end before its row is written, so this code is
+// written for instruction count: no integer division, no branch, loop constants in vector registers (a scalar
+// register that is spilled costs a vector instruction per use), corners dropped through their axis factor.
+struct CoordConst {
+    float Df, Hf, Wf, Dm1, Hm1, Wm1;      // extents, and extents - 1, as float
+    int H, W, Cin;
+    unsigned ax0, ax1, ax2;               // all ones where the offsets displace along the axis, else 0
+    unsigned keep;
+};
+// value of lane l (uniform) of a float register
+D2C_DEV float lane_value(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+D2C_DEV void opaque_v(float &v) { asm volatile("" : "+v"(v)); }
+D2C_DEV void opaque_v(int &v) { asm volatile("" : "+v"(v)); }
+D2C_DEV void opaque_v(unsigned &v) { asm volatile("" : "+v"(v)); }
+D2C_DEV CoordConst coord_const(const TiledShape &s)
+{
+    CoordConst c;
+    c.Df = (float)s.D; c.Hf = (float)s.H; c.Wf = (float)s.W;
+    c.Dm1 = (float)(s.D - 1); c.Hm1 = (float)(s.H - 1); c.Wm1 = (float)(s.W - 1);
+    c.H = s.H; c.W = s.W; c.Cin = s.Cin;
+    // (the 1-D operator has one offset component, which the loads deliver in all three slots: x keeps it)
+    const int axes = s.nd == 3 ? s.axes : 4;
+    c.ax0 = (axes & 1) ? ~0u : 0u; c.ax1 = (axes & 2) ? ~0u : 0u; c.ax2 = (axes & 4) ? ~0u : 0u;
+    c.keep = s.keep;
+    opaque_v(c.Df); opaque_v(c.Hf); opaque_v(c.Wf); opaque_v(c.Dm1); opaque_v(c.Hm1); opaque_v(c.Wm1);
+    opaque_v(c.H); opaque_v(c.W); opaque_v(c.Cin);
+    opaque_v(c.ax0); opaque_v(c.ax1); opaque_v(c.ax2); opaque_v(c.keep);
+    return c;
+}
+
+// Offsets of one sampling point, requested from (uniform address) + (32-bit offset of the lane): the address
+// arithmetic stays in scalar registers.  `ub`: first component of the (sample, group, tap) row of the lane with
+// offset 0; `cstride`: bytes between components (0 for the one-component offsets of the 1-D operator, whose value is
+// then read three times and kept as the x component).
+template <bool AUX16> D2C_DEV float ld_aux_at(const char *ub, unsigned lane_bytes)
+{
+    if constexpr (AUX16) return bf16_to_f32(*reinterpret_cast<const bf16_t *>(ub + lane_bytes));
+    else return *reinterpret_cast<const float *>(ub + lane_bytes);
+}
+template <bool AUX16>
+D2C_DEV void coord_offsets_issue(const char *ub, long cstride, unsigned lane_bytes, float *c)
+{
+    c[0] = ld_aux_at<AUX16>(ub, lane_bytes);
+    c[1] = ld_aux_at<AUX16>(ub + cstride, lane_bytes);
+    c[2] = ld_aux_at<AUX16>(ub + 2 * cstride, lane_bytes);
+}
+D2C_DEV void coord_offsets_select(const CoordConst &cc, float *c)
+{
+    c[0] = __uint_as_float(__float_as_uint(c[0]) & cc.ax0);
+    c[1] = __uint_as_float(__float_as_uint(c[1]) & cc.ax1);
+    c[2] = __uint_as_float(__float_as_uint(c[2]) & cc.ax2);
+}
+
+// Table row of the sampling point (z, y, x) with modulation m; `ok` false (a lane without a position) gives a row
+// that fetches nothing.  Bit for bit the weights of make_tap3 / tap3_weight times m for the corners that are live
+// there, zero for the others:
+//   * a point outside (-1, extent) on any axis, or not a number, has no live corner (make_tap3's `out` / `finite`);
+//     inside, floor(z) lies in [-1, D-1], so corner 0 of the axis is in range iff floor(z) >= 0 and corner 1 iff
+//     floor(z) < D - 1, and no clamp is needed before the conversion to int;
+//   * a corner out of range gets weight zero through its axis factor (the factors of the live corners are untouched,
+//     and so are their products, in tap3_weight's order);
+//   * m of a point without live corner is dropped (0 * NaN would be NaN; with a live corner all eight products end
+//     in the same sum, where a NaN modulation shows up in either formulation).
+struct CornerRow {
+    float w[8];
+    int idx;              // element offset of corner 000 in the channels-last input (only live corners are fetched)
+    unsigned live;
+};
+D2C_DEV CornerRow corner_row(const CoordConst &cc, float z, float y, float x, float m, int vox0, bool ok)
+{
+    CornerRow r;
+    // (bitwise: one chain of compare masks, no branch)
+    const bool in = ok & (z > -1.f) & (z < cc.Df) & (y > -1.f) & (y < cc.Hf) & (x > -1.f) & (x < cc.Wf);
+    const float zs = in ? z : 0.f, ys = in ? y : 0.f, xs = in ? x : 0.f, ms = in ? m : 0.f;
+    const float fz = floorf(zs), fy = floorf(ys), fx = floorf(xs);
+    const float hz = zs - fz, hy = ys - fy, hx = xs - fx;
+    const float lz = (fz + 1.f) - zs, ly = (fy + 1.f) - ys, lx = (fx + 1.f) - xs;
+    const bool z0 = in & (fz >= 0.f), z1 = in & (fz < cc.Dm1);
+    const bool y0 = in & (fy >= 0.f), y1 = in & (fy < cc.Hm1);
+    const bool x0 = in & (fx >= 0.f), x1 = in & (fx < cc.Wm1);
+    r.live = ((z0 ? 0x0Fu : 0u) | (z1 ? 0xF0u : 0u)) & ((y0 ? 0x33u : 0u) | (y1 ? 0xCCu : 0u))
+             & ((x0 ? 0x55u : 0u) | (x1 ? 0xAAu : 0u)) & cc.keep;
+    const float az[2] = {z0 ? lz : 0.f, z1 ? hz : 0.f};
+    const float ay[2] = {y0 ? ly : 0.f, y1 ? hy : 0.f};
+    const float ax[2] = {x0 ? lx : 0.f, x1 ? hx : 0.f};
+#pragma unroll
+    for (int q = 0; q < 8; q++) r.w[q] = ((az[q >> 2] * ay[(q >> 1) & 1]) * ax[q & 1]) * ms;
+    // (24-bit multiplications: the kernels that use this take shapes with D * H and W below 2^23 only; the last
+    // product is a full one)
+    const int iz = (int)fz, iy = (int)fy, ix = (int)fx;
+    r.idx = (vox0 + __mul24(__mul24(iz, cc.H) + iy, cc.W) + ix) * cc.Cin;
+    return r;
 }
 
 // The forward kernels' last step before a value is stored (NaN stays NaN, as in torch's relu).

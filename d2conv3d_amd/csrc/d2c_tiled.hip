@@ -92,6 +92,8 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0, con
     s.Do = q.Do; s.Ho = q.Ho; s.Wo = q.Wo;
     s.cg = q.Cin / q.groups; s.og = q.Cout / q.groups; s.cpg = q.Cin / q.offset_groups;
     s.nchunk = s.cg / bkc_of(q.dtype);
+    s.bkc = bkc_of(q.dtype);
+    s.cpc = (s.cg < s.cpg ? s.cg : s.cpg) / s.bkc;
     s.adt = q.aux_dtype;
     s.act = q.epilogue; s.act_scale = q.epilogue_scale;
     s.P = q.Do * q.Ho * q.Wo; s.vol = q.D * q.H * q.W; s.M = q.N * s.P;
@@ -571,6 +573,10 @@ static bool mfma_channels_ok(const d2c_conv3d_desc &q)
     if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
     // the tiled kernels address the channels-last input with 32-bit byte offsets
     if ((size_t)q.N * q.Cin * q.D * q.H * q.W * d2c_elem_size(q.dtype) + 256 >= (1ull << 32)) return false;
+    // ... form voxel indices with 24-bit multiplications (corner_row), and address the offsets of the (at most two)
+    // samples a position tile meets with 32-bit byte offsets from the first one
+    if ((long)q.D * q.H >= (1 << 23) || q.W >= (1 << 23)) return false;
+    if ((size_t)2 * q.offset_groups * q.kd * q.kh * q.kw * 3 * q.Do * q.Ho * q.Wo * 4 >= (1ull << 32)) return false;
     const int bkc = bkc_of(q.dtype);
     const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
     return cg % bkc == 0 && cpg % bkc == 0;

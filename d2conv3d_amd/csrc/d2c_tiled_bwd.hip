@@ -738,8 +738,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     unsigned char *s_raw = smem;                                       // [2][MT][8 corners][128 B]
     unsigned char *s_tile = s_raw + 2 * MT * kWRawPos;                 // [2][BKC][TRS]
     float *s_w = reinterpret_cast<float *>(s_tile + 2 * BKC * TRS);    // [3][8][MT]
-    int *s_idx = reinterpret_cast<int *>(s_w + 3 * 8 * MT);            // [3][MT]
-    int *s_flag = s_idx + 3 * MT;                                      // [3][MT]
+    int2 *s_if = reinterpret_cast<int2 *>(s_w + 3 * 8 * MT);           // [3][MT] (offset of corner 000, live corners)
 
     const BwdWeightArgs &a = aa.w;
     const TiledShape &s = a.s;
@@ -769,56 +768,65 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[ob][cb][r] = 0.f;
 
-    // --- coordinate wavefront: lane = position of tile i
+    // --- coordinate wavefront: lane = position of tile i.  The tap is the workgroup's own: its constants are formed
+    // once; an iteration takes the position apart (multiplications, no division) and builds the table row.
     const int ctid = tid - kThreads;
-    float craw[4];
+    typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+    const CoordConst cc = coord_const(s);
+    const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
+    // where the tap sits relative to (o * stride), as float
+    float tapf[3] = {(float)(kq[0] * s.geo.dd - s.geo.pd), (float)(kq[1] * s.geo.dh - s.geo.ph),
+                     (float)(kq[2] * s.geo.dw - s.geo.pw)};
+    opaque_v(tapf[0]); opaque_v(tapf[1]); opaque_v(tapf[2]);
+    float sbase[3] = {0.f, 0.f, 0.f};   // kernel-grid coordinates of the tap (size-map source)
+    if constexpr (SIZED) {
+#pragma unroll
+        for (int ax = 0; ax < 3; ax++) sbase[ax] = rnd<AT>(s.ss.base[ax][kq[ax]]);
+    }
+    const long cstride = s.nd == 3 ? (long)s.P * (long)sizeof(AT) : 0;
+    const long off_tap = (long)(s.nd == 3 ? 3 : 1) * s.P * (long)sizeof(AT);   // bytes per (sample, group, tap)
+    const long mask_tap = (long)s.P * (long)sizeof(AT);
+    const unsigned off_sample = (unsigned)(s.G * s.K) * (unsigned)off_tap, mask_sample = (unsigned)(s.G * s.K) * (unsigned)mask_tap;
+    float craw[4] = {0.f, 0.f, 0.f, 1.f};
     int cb_ = 0, cp_ = 0;
     bool cvalid = false;
     auto coords_issue = [&](int i) {
         if (worker) return;
-        const long m = (long)(sp + i * a.split) * MT + ctid;
+        const int m0 = (sp + i * a.split) * MT;                 // (m < N * P < 2^31)
+        const int m = m0 + ctid;
         cvalid = m < s.M;
-        if (cvalid) {
-            cb_ = fdiv((int)m, s.dP); cp_ = (int)m - cb_ * s.P;      // (m < N * P < 2^31)
-            const long ab = (((long)cb_ * s.G + g) * s.K + k) * s.P + cp_;
-            tap_offsets_issue<AUX16, SIZED>(s, a.off, cb_, g, k, cp_, craw);
-            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
+        // (a lane without a position reads what the tile's first position reads)
+        const int mq = cvalid ? m : m0;
+        const int b_lo = fdiv(m0, s.dP);                        // uniform: the tile's first sample
+        cb_ = fdiv(mq, s.dP); cp_ = mq - cb_ * s.P;
+        if constexpr (SIZED) {
+            tap_offsets_issue<AUX16, true>(s, a.off, cb_, g, k, cp_, craw);
+        } else {
+            const char *ub = reinterpret_cast<const char *>(a.off) + ((long)(b_lo * s.G + g) * s.K + k) * off_tap;
+            coord_offsets_issue<AUX16>(ub, cstride, (unsigned)(cb_ - b_lo) * off_sample + (unsigned)cp_ * (unsigned)sizeof(AT), craw);
+        }
+        if (a.mask) {
+            const char *um = reinterpret_cast<const char *>(a.mask) + ((long)(b_lo * s.G + g) * s.K + k) * mask_tap;
+            craw[3] = ld_aux_at<AUX16>(um, (unsigned)(cb_ - b_lo) * mask_sample + (unsigned)cp_ * (unsigned)sizeof(AT));
         }
     };
-    float sbase[3] = {0.f, 0.f, 0.f};   // kernel-grid coordinates of this workgroup's tap (size-map source)
-    if constexpr (SIZED) {
-        typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
-        const int kq[3] = {k / (s.geo.kw * s.geo.kh), (k / s.geo.kw) % s.geo.kh, k % s.geo.kw};
-#pragma unroll
-        for (int ax = 0; ax < 3; ax++) sbase[ax] = rnd<AT>(s.ss.base[ax][kq[ax]]);
-    }
     auto coords_finish = [&](int buf) {   // of the tile whose offsets coords_issue requested last
         if (worker) return;
-        float w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        int idx = 0;
-        unsigned live = 0;
-        if (cvalid) {
-            const int oz = fdiv(cp_, s.dHW), rem = cp_ - oz * (s.Wo * s.Ho);
-            const int oy = fdiv(rem, s.dW), ox = rem - oy * s.Wo;
-            int bz, by, bx;
-            tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
-            if constexpr (SIZED) {
-                // size-map source: offsets = base_a[k_a] * (size_a - 1); the tap is this workgroup's own
-                typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
-                if (s.ss.on == 1) size_minus_one<AUX16>(s, craw);
+        const int oz = fdiv(cp_, s.dHW), rem = cp_ - oz * (s.Wo * s.Ho);
+        const int oy = fdiv(rem, s.dW), ox = rem - oy * s.Wo;
+        if constexpr (SIZED) {
+            // size-map source: offsets = base_a[k_a] * (size_a - 1); the tap is this workgroup's own
+            if (s.ss.on == 1) size_minus_one<AUX16>(s, craw);
 #pragma unroll
-                for (int ax = 0; ax < 3; ax++) craw[ax] = rnd<AT>(sbase[ax] * craw[ax]);
-            }
-            const Tap3<float> t = tiled_tap3(s, bz, by, bx, craw[0], craw[1], craw[2]);
-            live = t.live;
-            idx = (cb_ * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
-#pragma unroll
-            for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * craw[3] : 0.f;
+            for (int ax = 0; ax < 3; ax++) craw[ax] = rnd<AT>(sbase[ax] * craw[ax]);
         }
+        coord_offsets_select(cc, craw);
+        const CornerRow r = corner_row(cc, ((float)__mul24(oz, s.geo.sd) + tapf[0]) + craw[0],
+                                       ((float)__mul24(oy, s.geo.sh) + tapf[1]) + craw[1],
+                                       ((float)__mul24(ox, s.geo.sw) + tapf[2]) + craw[2], craw[3], cb_ * s.vol, cvalid);
 #pragma unroll
-        for (int c = 0; c < 8; c++) s_w[(buf * 8 + c) * MT + ctid] = w[c];
-        s_idx[buf * MT + ctid] = idx;
-        s_flag[buf * MT + ctid] = (int)live;
+        for (int c = 0; c < 8; c++) s_w[(buf * 8 + c) * MT + ctid] = r.w[c];
+        s_if[buf * MT + ctid] = make_int2(r.idx, (int)r.live);
     };
 
     // --- corner rows of tile i -> s_raw[rbuf]: worker wavefront w requests positions 8w .. 8w+7
@@ -827,8 +835,8 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     auto dma_issue = [&](int rbuf, int tbuf) {
         if (!worker) return;
         const char *base = reinterpret_cast<const char *>(a.xcl);
-        const int vidx = s_idx[tbuf * MT + wave * (MT / 8) + (lane & 7)];
-        const int vflag = s_flag[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const int2 vif = s_if[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const int vidx = vif.x, vflag = vif.y;
 #pragma unroll
         for (int i = 0; i < MT / 8; i++) {
             const int pos = wave * (MT / 8) + i;
@@ -949,9 +957,8 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
                 if (it + 1 < nmy) interp_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
             }
         } else {
-            // (the coordinate wavefront shares its SIMD with two worker wavefronts and is the one the iteration
-            // waits for when the matrix work per tile is small: it issues ahead of them)
-            __builtin_amdgcn_s_setprio(2);
+            // (at default priority: issuing ahead of the two worker wavefronts of its SIMD paid while this code was
+            // three times as long; with the short version it costs 5 - 8 %)
             for (int it = 0; it < nmy; it++) {
                 // (a barrier that waits for this wavefront's LDS stores only: the offsets it requested stay in
                 // flight across it and are waited for where they are used, a whole iteration after the request)

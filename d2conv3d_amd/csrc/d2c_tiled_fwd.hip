@@ -292,13 +292,20 @@ constexpr int kMaxSeg = 128;               // segments per workgroup (the launch
 
 // A position in the step sequence of a workgroup.  The segments are listed in LDS once, at the start; all
 // fields are uniform over the workgroup and live in scalar registers.
+//
+// Step order within a work item: offset group (outer), tap, chunk of that offset group (inner), so that the chunks
+// that share the sampling points of a (group, tap) follow each other and the coordinate wavefront computes a table
+// once for all of them.  The walker counts chunk, tap and group along (no division per step).
 struct SegWalk {
     int seg;                      // index of the current segment
     int item;                     // its work item, -1 past the end of the sequence
     int st, st_hi;                // current step, end of the current segment
     int tile, otile, wg;          // the item's position tile, output tile, weight group
+    int j, k, g;                  // the step's chunk within the weight group, tap, offset group
+    int jj;                       // chunk within the offset group
+    bool fresh;                   // first step of its (group, tap) in this segment: sampling points not seen yet
 };
-D2C_DEV void seg_load(SegWalk &w, const int4 *s_seg, int nseg)
+D2C_DEV void seg_load(SegWalk &w, const int4 *s_seg, int nseg, const TiledShape &s)
 {
     if (w.seg < nseg) {
         const int4 u = s_seg[2 * w.seg], v = s_seg[2 * w.seg + 1];
@@ -308,16 +315,32 @@ D2C_DEV void seg_load(SegWalk &w, const int4 *s_seg, int nseg)
         w.tile = __builtin_amdgcn_readfirstlane(v.x);
         w.otile = __builtin_amdgcn_readfirstlane(v.y);
         w.wg = __builtin_amdgcn_readfirstlane(v.z);
+        const int t = w.st / s.cpc, gi = t / s.K;
+        w.jj = w.st - t * s.cpc;
+        w.k = t - gi * s.K;
+        w.j = gi * s.cpc + w.jj;
+        w.g = (w.wg * s.cg + w.j * s.bkc) / s.cpg;
     } else {
         w.item = -1; w.st = 0; w.st_hi = 0x7fffffff;
+        w.j = 0; w.k = 0; w.g = 0; w.jj = 0;
     }
+    w.fresh = true;
 }
 // one step on; true when that entered a new segment
-D2C_DEV bool seg_advance(SegWalk &w, const int4 *s_seg, int nseg)
+D2C_DEV bool seg_advance(SegWalk &w, const int4 *s_seg, int nseg, const TiledShape &s)
 {
-    if (++w.st < w.st_hi) return false;
+    if (++w.st < w.st_hi) {
+        if (++w.jj < s.cpc) {
+            w.j++; w.fresh = false;
+        } else {
+            w.jj = 0; w.fresh = true;
+            if (++w.k < s.K) w.j -= s.cpc - 1;
+            else { w.k = 0; w.j++; w.g++; }
+        }
+        return false;
+    }
     w.seg++;
-    seg_load(w, s_seg, nseg);
+    seg_load(w, s_seg, nseg, s);
     return true;
 }
 
@@ -325,8 +348,8 @@ D2C_DEV bool seg_advance(SegWalk &w, const int4 *s_seg, int nseg)
 // which the compiler makes every LDS store wait for all DMA transfers in flight, whatever region they fill.)
 template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED>
 D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, unsigned char *__restrict__ s_tile,
-                          float *__restrict__ s_w, int *__restrict__ s_idx, int *__restrict__ s_flag,
-                          int4 *__restrict__ s_seg)
+                          float *__restrict__ s_w, int2 *__restrict__ s_if,
+                          int *__restrict__ s_meta, int4 *__restrict__ s_seg)
 {
     constexpr int MT = kDMT;
     constexpr int VEC = Elem<T>::VEC;
@@ -343,6 +366,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int S = s.nchunk * s.K;
+    const int OBT = s.ogp / 32;
     const int dzc = s.H * s.W * s.Cin, dyc = s.W * s.Cin;
 
     // --- the step sequence of this workgroup: its whole items, then its pieces of the last round's items
@@ -372,7 +396,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     for (int q = 0; q < nseg; q++) total += __builtin_amdgcn_readfirstlane(s_seg[2 * q].z - s_seg[2 * q].y);
     SegWalk w0;
     w0.seg = 0;
-    seg_load(w0, s_seg, nseg);
+    seg_load(w0, s_seg, nseg, s);
 
     // --- coordinates: a ninth wavefront (one position per lane) that does nothing else, so that this
     // arithmetic runs beside the work of the other eight instead of in front of their barrier
@@ -380,59 +404,115 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     const bool worker = wave < 8;
     const int ctid = tid - kThreads;
     // The lane's position within a work item.  Offsets are requested (issue) one iteration before they are
-    // turned into a table row (finish), possibly across a segment boundary: one set of constants for each.
+    // turned into a table row (finish).
     // (size-map source: the part of the offsets that the taps of a position share, size - 1 per axis, is formed
     // here once per work item; a step then costs three multiplications and no load)
-    struct PosC { int b, p, oz, oy, ox; bool valid; float s0, s1, s2; };
+    typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+    const CoordConst cc = coord_const(s);
+    const int ncomp = s.nd == 3 ? 3 : 1;                               // offset components per tap
+    const long cstride = s.nd == 3 ? (long)s.P * (long)sizeof(AT) : 0;
+    const long off_tap = (long)ncomp * s.P * (long)sizeof(AT);         // bytes per (sample, group, tap) of the offsets
+    const long mask_tap = (long)s.P * (long)sizeof(AT);                // ... of the mask
+    // Lane l of the coordinate wavefront keeps the constants of tap l (taps 64 and up are computed when met):
+    // where the tap sits in the kernel, as float, and for the size-map source its kernel-grid coordinates.
+    float tap_z = 0.f, tap_y = 0.f, tap_x = 0.f, tap_bz = 0.f, tap_by = 0.f, tap_bx = 0.f;
+    auto tap_consts = [&](int k, float &tz, float &ty, float &tx, float &bz, float &by, float &bx) {
+        const int kx = k % s.geo.kw, ky = (k / s.geo.kw) % s.geo.kh, kz = k / (s.geo.kw * s.geo.kh);
+        tz = (float)(kz * s.geo.dd); ty = (float)(ky * s.geo.dh); tx = (float)(kx * s.geo.dw);
+        if constexpr (SIZED) {
+            bz = rnd<AT>(s.ss.base[0][kz]); by = rnd<AT>(s.ss.base[1][ky]); bx = rnd<AT>(s.ss.base[2][kx]);
+        }
+    };
+    if (cwave && ctid < s.K) tap_consts(ctid, tap_z, tap_y, tap_x, tap_bz, tap_by, tap_bx);
+    struct PosC {
+        float fz, fy, fx;          // o * stride - pad per axis, as float
+        int vox0;                  // voxel index of the sample's origin
+        unsigned aoff, moff;       // byte offsets of (sample - first sample of the tile, position) in offsets / mask
+        bool valid;
+        float s0, s1, s2;
+    };
+    const char *off_item = nullptr, *mask_item = nullptr;      // uniform: the tile's first sample
     auto pos_of = [&](const SegWalk &w) {
-        PosC c{0, 0, 0, 0, 0, false, 0.f, 0.f, 0.f};
-        const int m = w.tile * MT + ctid;
+        PosC c{0.f, 0.f, 0.f, 0, 0u, 0u, false, 0.f, 0.f, 0.f};
+        const int m0 = w.item >= 0 ? w.tile * MT : 0;
+        const int b_lo = fdiv(m0, s.dP);
+        off_item = reinterpret_cast<const char *>(a.off) + (long)b_lo * s.G * s.K * off_tap;
+        mask_item = reinterpret_cast<const char *>(a.mask) + (long)b_lo * s.G * s.K * mask_tap;
+        const int m = m0 + ctid;
         c.valid = w.item >= 0 && m < s.M;
         if (c.valid) {
-            c.b = m / s.P; c.p = m - c.b * s.P;
-            c.ox = c.p % s.Wo; c.oy = (c.p / s.Wo) % s.Ho; c.oz = c.p / (s.Wo * s.Ho);
+            const int b = fdiv(m, s.dP), p = m - b * s.P;
+            const int oz = fdiv(p, s.dHW), rem = p - oz * (s.Wo * s.Ho);
+            const int oy = fdiv(rem, s.dW), ox = rem - oy * s.Wo;
+            c.fz = (float)(oz * s.geo.sd - s.geo.pd);
+            c.fy = (float)(oy * s.geo.sh - s.geo.ph);
+            c.fx = (float)(ox * s.geo.sw - s.geo.pw);
+            c.vox0 = b * s.vol;
+            // (a lane without a position keeps offset 0: its loads read the tile's first position)
+            c.aoff = (unsigned)(b - b_lo) * (unsigned)(s.G * s.K) * (unsigned)off_tap + (unsigned)p * (unsigned)sizeof(AT);
+            c.moff = (unsigned)(b - b_lo) * (unsigned)(s.G * s.K) * (unsigned)mask_tap + (unsigned)p * (unsigned)sizeof(AT);
             if (SIZED && cwave) {
                 float t[3];
-                tap_offsets_issue<AUX16, true>(s, a.off, c.b, 0, 0, c.p, t);
+                tap_offsets_issue<AUX16, true>(s, a.off, b, 0, 0, p, t);
                 size_minus_one<AUX16>(s, t);
                 c.s0 = t[0]; c.s1 = t[1]; c.s2 = t[2];
             }
         }
         return c;
     };
-    float craw[4];
+    float craw[4] = {0.f, 0.f, 0.f, 1.f};
     auto coords_issue = [&](const SegWalk &w, const PosC &c) {
-        if (cwave && c.valid) {
-            const int j = w.st / s.K, k = w.st - j * s.K;
-            const int g = (w.wg * s.cg + j * BKC) / s.cpg;
-            const long ab = (((long)c.b * s.G + g) * s.K + k) * s.P + c.p;
-            if constexpr (!SIZED) tap_offsets_issue<AUX16, false>(s, a.off, c.b, g, k, c.p, craw);
-            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
+        if (cwave && w.fresh) {
+            const int gk = w.g * s.K + w.k;
+            if constexpr (!SIZED) coord_offsets_issue<AUX16>(off_item + gk * off_tap, cstride, c.aoff, craw);
+            if (a.mask) craw[3] = ld_aux_at<AUX16>(mask_item + gk * mask_tap, c.moff);
         }
     };
     auto coords_finish = [&](const SegWalk &w, const PosC &c, int buf) {
-        if (cwave) {
-            float wt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            int idx = 0;
-            unsigned live = 0;
-            if (c.valid) {
-                const int k = w.st % s.K;
-                int bz, by, bx;
-                tap_base(s.geo, k, c.oz, c.oy, c.ox, bz, by, bx);
+        if (cwave && !w.fresh) {
+            // same sampling points as the step before (another chunk of the offset group): its table, copied
+            const int pbuf = (buf + 2) % 3;
+#pragma unroll
+            for (int q = 0; q < 8; q++) s_w[(buf * 8 + q) * MT + ctid] = s_w[(pbuf * 8 + q) * MT + ctid];
+            s_if[buf * MT + ctid] = s_if[pbuf * MT + ctid];
+        } else if (cwave) {
+            float tz, ty, tx, bz = 0.f, by = 0.f, bx = 0.f;
+            if (w.k < 64) {
+                tz = lane_value(tap_z, w.k);
+                ty = lane_value(tap_y, w.k);
+                tx = lane_value(tap_x, w.k);
                 if constexpr (SIZED) {
-                    const float t[3] = {c.s0, c.s1, c.s2};
-                    size_tap_offsets<AUX16>(s, k, t, craw);
+                    bz = lane_value(tap_bz, w.k);
+                    by = lane_value(tap_by, w.k);
+                    bx = lane_value(tap_bx, w.k);
                 }
-                const Tap3<float> t = tiled_tap3(s, bz, by, bx, craw[0], craw[1], craw[2]);
-                live = t.live;
-                idx = (c.b * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
-#pragma unroll
-                for (int q = 0; q < 8; q++) wt[q] = ((live >> q) & 1u) ? tap3_weight(t, q) * craw[3] : 0.f;
+            } else {
+                tap_consts(w.k, tz, ty, tx, bz, by, bx);
             }
+            if constexpr (SIZED) {
+                craw[0] = rnd<AT>(bz * c.s0); craw[1] = rnd<AT>(by * c.s1); craw[2] = rnd<AT>(bx * c.s2);
+            }
+            coord_offsets_select(cc, craw);
+            const CornerRow r = corner_row(cc, (c.fz + tz) + craw[0], (c.fy + ty) + craw[1], (c.fx + tx) + craw[2],
+                                           craw[3], c.vox0, c.valid);
 #pragma unroll
-            for (int q = 0; q < 8; q++) s_w[(buf * 8 + q) * MT + ctid] = wt[q];
-            s_idx[buf * MT + ctid] = idx;
-            s_flag[buf * MT + ctid] = (int)live;
+            for (int q = 0; q < 8; q++) s_w[(buf * 8 + q) * MT + ctid] = r.w[q];
+            s_if[buf * MT + ctid] = make_int2(r.idx, (int)r.live);
+        }
+        // what the workers need to know of the step: its first input channel and where its weight fragments start
+        // (they walk no step sequence of their own)
+        if (cwave && ctid == 0) {
+            s_meta[buf * 4] = w.wg * s.cg + w.j * BKC;
+            s_meta[buf * 4 + 1] = (w.wg * S + w.j * s.K + w.k) * OBT + w.otile * (NT / 32);
+        }
+    };
+    // a table that fetches rows of zeros: steps past the end of a sequence shorter than the pipeline
+    auto coords_none = [&](int buf) {
+        if (cwave) {
+#pragma unroll
+            for (int q = 0; q < 8; q++) s_w[(buf * 8 + q) * MT + ctid] = 0.f;
+            s_if[buf * MT + ctid] = make_int2(0, 0);
+            if (ctid == 0) { s_meta[buf * 4] = 0; s_meta[buf * 4 + 1] = 0; }
         }
     };
 
@@ -440,23 +520,22 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     // instruction per position, lane = (corner, 16-byte vector)
     const int dcorner = lane >> 3, dvec = lane & 7;
     const int dcoff = ((dcorner >> 2) & 1) * dzc + ((dcorner >> 1) & 1) * dyc + (dcorner & 1) * s.Cin;
-    auto dma_issue = [&](const SegWalk &w, int rbuf, int tbuf) {
+    // (past the end of the sequence the tables are those of three steps before, or the ones of coords_none: the
+    // same number of transfers in every iteration, which lets the compiler count the loads in flight instead of
+    // waiting for all)
+    auto dma_issue = [&](int rbuf, int tbuf) {
         if (!worker) return;
-        const int j = w.st / s.K;
-        const int c0 = w.wg * s.cg + j * BKC;
+        const int c0 = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4]);
         const char *base = reinterpret_cast<const char *>(a.xcl);
         // table entries of this wavefront's 8 positions: one LDS read (lane i holds position i), then
         // lane-indexed moves to scalar registers
-        const int vidx = s_idx[tbuf * MT + wave * (MT / 8) + (lane & 7)];
-        const int vflag = s_flag[tbuf * MT + wave * (MT / 8) + (lane & 7)];
-        const unsigned vmask = w.item >= 0 ? 0xffu : 0u;
+        const int2 vif = s_if[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const int vidx = vif.x, vflag = vif.y;
 #pragma unroll
         for (int i = 0; i < MT / 8; i++) {
             const int pos = wave * (MT / 8) + i;
             const int idx = __builtin_amdgcn_readlane(vidx, i);
-            // (past the end of the sequence every lane fetches the row of zeros: the same number of transfers
-            // in every iteration, which lets the compiler count the loads in flight instead of waiting for all)
-            const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i) & vmask;
+            const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
             const unsigned o = ((live >> dcorner) & 1u)
                                    ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
                                    : a.zrow + (unsigned)dvec * 16u;
@@ -481,7 +560,6 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     // --- MMA role
     const bool mma_wave = wave < WAVES_O * WAVES_P;
     const int wave_o = wave % WAVES_O, wave_p = wave / WAVES_O;
-    const int OBT = s.ogp / 32;
     f32x16 acc[OB][PB];
 #pragma unroll
     for (int ob = 0; ob < OB; ob++)
@@ -491,10 +569,9 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
             for (int r = 0; r < 16; r++) acc[ob][pb][r] = 0.f;
     const uint4 *wp4 = reinterpret_cast<const uint4 *>(a.wp);
     uint4 af[NKG][OB];
-    auto wfrag = [&](const SegWalk &w, int kg, int ob) {
-        // (past the end of the sequence: any valid address, the fragments are not used)
-        const int wgq = w.item >= 0 ? w.wg : 0, stq = w.item >= 0 ? w.st : 0, otq = w.item >= 0 ? w.otile : 0;
-        const long wbase = (((long)wgq * S + stq) * OBT + (otq * (NT / 32) + wave_o * OB)) * NKG * 64 + lane;
+    // (wstep: the table's entry for the step; past the end of the sequence a stale one, the fragments are not used)
+    auto wfrag = [&](int wstep, int kg, int ob) {
+        const long wbase = ((long)wstep + wave_o * OB) * NKG * 64 + lane;
         return wp4[wbase + ((long)ob * NKG + kg) * 64];
     };
     // The vector-memory path of a CU takes one request of a wavefront at a time (1 KiB = 16 clocks) and a wavefront
@@ -503,16 +580,14 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     // step it (in its first half, so that they have landed when the interpolation starts), the weight-fragment
     // loads of step it+1 between the corners of the interpolation.
     static_assert(WAVES_O * WAVES_P == 8 && NKG * OB == 8, "all workers are matrix wavefronts; a fragment per corner");
-    auto mma_dma_step = [&](int dbuf, const SegWalk &w, int rbuf, int tbuf) {
+    auto mma_dma_step = [&](int dbuf, int rbuf, int tbuf) {
         const unsigned char *tb = s_tile + (dbuf * MT + wave_p * WPOS + (lane & 31)) * kRS + (lane >> 5) * 16;
-        const int j = w.st / s.K;
-        const int c0 = w.wg * s.cg + j * BKC;
+        const int c0 = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4]);
         const char *base = reinterpret_cast<const char *>(a.xcl);
         // table entries of this wavefront's 8 positions: one LDS read (lane i holds position i), then
         // lane-indexed moves to scalar registers
-        const int vidx = s_idx[tbuf * MT + wave * (MT / 8) + (lane & 7)];
-        const int vflag = s_flag[tbuf * MT + wave * (MT / 8) + (lane & 7)];
-        const unsigned vmask = w.item >= 0 ? 0xffu : 0u;     // past the end of the sequence: rows of zeros
+        const int2 vif = s_if[tbuf * MT + wave * (MT / 8) + (lane & 7)];
+        const int vidx = vif.x, vflag = vif.y;
         constexpr int DPK = 4;                                // requests per k-group
 #pragma unroll
         for (int kg = 0; kg < NKG; kg++) {
@@ -530,7 +605,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 if (i >= MT / 8) break;
                 const int pos = wave * (MT / 8) + i;
                 const int idx = __builtin_amdgcn_readlane(vidx, i);
-                const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i) & vmask;
+                const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
                 const unsigned o = ((live >> dcorner) & 1u)
                                        ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
                                        : a.zrow + (unsigned)dvec * 16u;
@@ -540,15 +615,16 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
             }
         }
     };
-    // interpolation of one step; the weight fragments of that step (at `wn`) are fetched on the way
-    auto interp_wload_store = [&](int rbuf, int tbuf, int dbuf, const SegWalk &wn) {
+    // interpolation of one step; the weight fragments of that step are fetched on the way
+    auto interp_wload_store = [&](int rbuf, int tbuf, int dbuf) {
         const unsigned char *rp = s_raw + (rbuf * MT + ipos) * kRawPos + ivec * 16;
+        const int wstep = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4 + 1]);
         VecAcc<T> va;
         va.zero();
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             va.fma(s_w[(tbuf * 8 + c) * MT + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
-            af[c / OB][c % OB] = wfrag(wn, c / OB, c % OB);
+            af[c / OB][c % OB] = wfrag(wstep, c / OB, c % OB);
         }
         *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = va.pack();
     };
@@ -653,38 +729,34 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     // of step it+3 computed.  Corner tables rotate over 3 buffers,
     // raw rows and tiles over 2.  A wavefront interpolates the positions whose rows it requested itself, so the
     // rows need no barrier, only that wavefront's own wait.
-    SegWalk wc = w0;                  // coordinates: the step whose offsets are requested next
+    SegWalk wc = w0;                  // coordinates: the step whose table is computed next (its offsets are requested
+                                      // one iteration before)
     PosC pc = pos_of(wc);
     for (int q = 0; q < 3; q++) {
         if (q < total) {
             coords_issue(wc, pc);
             coords_finish(wc, pc, q);
-            if (seg_advance(wc, s_seg, nseg)) pc = pos_of(wc);
+            if (seg_advance(wc, s_seg, nseg, s)) pc = pos_of(wc);
+        } else {
+            coords_none(q);
         }
     }
-    SegWalk wf = wc;                  // coordinates: the step whose table row is computed next
-    PosC pf = pc;
-    SegWalk wm = w0, wn = w0, wd = w0;    // steps: on the matrix cores / after that one / rows requested next
-    seg_advance(wn, s_seg, nseg);
+    SegWalk wm = w0;                  // the step on the matrix cores
+    __syncthreads();
     if (mma_wave) {
+        const int wstep = __builtin_amdgcn_readfirstlane(s_meta[1]);
 #pragma unroll
         for (int kg = 0; kg < NKG; kg++)
 #pragma unroll
-            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(wm, kg, ob);
+            for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(wstep, kg, ob);
     }
-    __syncthreads();
-    dma_issue(wd, 0, 0);
-    seg_advance(wd, s_seg, nseg);
-    if (1 < total) {
-        dma_issue(wd, 1, 1);
-        seg_advance(wd, s_seg, nseg);
-    }
+    dma_issue(0, 0);
+    dma_issue(1, 1);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     interp_store(0, 0, 0);
     if (3 < total) {
         coords_issue(wc, pc);
-        if (seg_advance(wc, s_seg, nseg)) pc = pos_of(wc);
     }
     // One loop per role (separate register budgets), the same synchronisation point per iteration in each.
     if (worker) {
@@ -697,29 +769,25 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 // everything this wavefront has in flight is due: the weight fragments of this step (requested
                 // during the last interpolation) and the rows of step it+1 (requested during the last matrix step)
                 __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
-                mma_dma_step(it & 1, wd, it & 1, (it + 2) % 3);
+                mma_dma_step(it & 1, it & 1, (it + 2) % 3);
                 // (past the end of the sequence the interpolation works on stale rows into the tile nobody reads)
-                interp_wload_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1, wn);
-                if (wd.item >= 0) seg_advance(wd, s_seg, nseg);
-                if (wn.item >= 0) seg_advance(wn, s_seg, nseg);
+                interp_wload_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
             }
             flush_acc(wm);
             wm.seg++;
-            seg_load(wm, s_seg, nseg);
+            seg_load(wm, s_seg, nseg, s);
         }
     } else {
-        // (the coordinate wavefront issues ahead of the two workers it shares a SIMD with: measured -6 % on the
-        // 512-channel tile (C = 512, 8 x 30 x 54: 0.78 -> 0.73 ms), +3 % on the 256-channel one, so only there)
-        if constexpr (WAVES_O == 8) __builtin_amdgcn_s_setprio(2);
+        // (at default priority: with its short instruction sequence, issuing ahead of the two workers of its SIMD
+        // costs 3 % on the 512-channel tile and gains nothing on the 256-channel one)
         for (int it = 0; it < total; it++) {
             lds_barrier();
             if (it + 3 < total) {                      // offsets requested one iteration ago
-                coords_finish(wf, pf, it % 3);
-                if (seg_advance(wf, s_seg, nseg)) pf = pos_of(wf);
+                coords_finish(wc, pc, it % 3);
+                if (seg_advance(wc, s_seg, nseg, s)) pc = pos_of(wc);
             }
             if (it + 4 < total) {
                 coords_issue(wc, pc);
-                if (seg_advance(wc, s_seg, nseg)) pc = pos_of(wc);
             }
         }
     }
@@ -734,10 +802,10 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
     __shared__ __align__(16) unsigned char s_raw[2 * MT * kRawPos];   // [2][MT][8 corners][128 B]
     __shared__ __align__(16) unsigned char s_tile[2 * MT * kRS];      // [2][MT][kRS]
     __shared__ float s_w[3 * 8 * MT];                                 // [3][8][MT]
-    __shared__ int s_idx[3 * MT];                                     // [3][MT]
-    __shared__ int s_flag[3 * MT];                                    // [3][MT]
+    __shared__ int2 s_if[3 * MT];                                     // [3][MT] (offset of corner 000, live corners)
+    __shared__ int s_meta[3 * 4];                                     // [3][first channel, weight-fragment row]
     __shared__ int4 s_seg[2 * kMaxSeg];                               // [kMaxSeg][2]
-    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P, SIZED>(a, s_raw, s_tile, s_w, s_idx, s_flag, s_seg);
+    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P, SIZED>(a, s_raw, s_tile, s_w, s_if, s_meta, s_seg);
 }
 
 // out = fp32 tile + bias for the items whose steps were shared out (see FwdArgs).  One block = 32 output
