@@ -100,9 +100,11 @@ def algorithmic(name, N=None, dims=None):
 
 
 def hbm_traffic_bytes(workload, kernel):
-    """HBM bytes per launch of `kernel`, from the committed rocprofv3 --pmc summary of the workload
-    (FETCH_SIZE + WRITE_SIZE, calibrated on a plain copy kernel); None if not recorded."""
+    """(HBM bytes per launch of `kernel`, where the figure comes from): read from the committed rocprofv3 --pmc
+    summary of the workload (FETCH_SIZE + WRITE_SIZE, calibrated on a plain copy kernel), i.e. NOT measured in this
+    run; (None, None) if not recorded."""
     import glob
+    import subprocess
     stem = kernel[:-len("_kernel")] if kernel.endswith("_kernel") else kernel
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", f"{workload}_*.md"))):
         try:
@@ -110,10 +112,19 @@ def hbm_traffic_bytes(workload, kernel):
                 cells = [c.strip().strip("`") for c in row.split("|")]
                 # the traffic table: | kernel | fetch MB | write MB | total MB |
                 if len(cells) == 6 and cells[1].startswith(stem):
-                    return int(float(cells[4]) * 1e6)
+                    rel = os.path.relpath(path, ROOT)
+                    src = f"{rel} (committed rocprofv3 --pmc summary, not measured in this run)"
+                    try:
+                        h = subprocess.run(["git", "-C", ROOT, "log", "-1", "--format=%h", "--", rel],
+                                           capture_output=True, text=True, timeout=10).stdout.strip()
+                        if h:
+                            src = f"{rel} @ {h} (committed rocprofv3 --pmc summary, not measured in this run)"
+                    except (OSError, subprocess.SubprocessError):
+                        pass
+                    return int(float(cells[4]) * 1e6), src
         except (OSError, ValueError):
             pass
-    return None
+    return None, None
 
 
 def cpu_baseline(name, torch):
@@ -533,7 +544,7 @@ def main():
     roofline = None
     if dom:
         kms = {k: round(v, 4) for k, v in kern.items()}
-        traffic = hbm_traffic_bytes(name, dom)
+        traffic, traffic_source = hbm_traffic_bytes(name, dom)
         t_dom = main_k[dom] * 1e-3
         es = 2 if dt == "bf16" else 4
         P = 1
@@ -560,7 +571,24 @@ def main():
             bound, ach = "mfma", f_fwd_flops / t_dom / 1e12
         peak, unit = (PEAK_GBS, "GB/s") if bound == "hbm" else (PEAK_TFLOPS[dt], "TFLOP/s")
         roofline = {"bound": bound, "kernel": dom, "achieved": round(ach, 2), "peak": peak, "unit": unit,
-                    "frac": round(ach / peak, 4), "traffic": traffic, "kernel_ms": kms}
+                    "frac": round(ach / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
+                    "kernel_ms": kms}
+
+    # Depthwise kernels: the corner rows they pull through the vector-memory path of the compute units (L1), which
+    # is what bounds them (64 bytes per clock and compute unit; 256 units at 2.4 GHz), beside the HBM figure above.
+    roofline_l1 = None
+    if fam == "dw" and nd == 3:
+        peak_l1 = 64 * 256 * 2.4  # GB/s
+        npos, esz = dims[0] * dims[1] * dims[2], (2 if dt == "bf16" else 4)
+        rows = N * npos * 27 * 8 * C * esz          # 8 corner values per tap and channel
+        per = {"dw_fwd_kernel": rows, "dw_bwd_kernel": rows + N * npos * 27 * C * esz}   # + the grad_out value per tap
+        roofline_l1 = {"bound": "l1", "peak": round(peak_l1, 1), "unit": "GB/s",
+                       "peak_source": "64 B/clk/CU x 256 CUs x 2.4 GHz (vector-memory path)", "kernels": {}}
+        for kname, nbytes in per.items():
+            if kname in kern:
+                gbs = nbytes / (kern[kname] * 1e-3) / 1e9
+                roofline_l1["kernels"][kname] = {"bytes": nbytes, "ms": round(kern[kname], 4),
+                                                 "achieved": round(gbs, 1), "frac": round(gbs / peak_l1, 4)}
 
     what = "modulated deformable conv%dd %s" % (nd, "fwd+bwd" if c["backward"] else "fwd")
     line = {
@@ -585,6 +613,8 @@ def main():
                                                         / (ms * 1e-3) / 1e9 / PEAK_GBS, 4)},
         "roofline": roofline,
     }
+    if roofline_l1:
+        line["roofline_l1"] = roofline_l1
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(name, torch)
     print(json.dumps(line))

@@ -23,10 +23,44 @@ def _stream(dev):
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
 
+# One workspace tensor per (device, stream), grown when a call needs more and handed to every call on that stream:
+# the kernels of a stream run one after the other, so they can share it, and a training step does not allocate (and
+# hold in the caching allocator, beside whatever else is cached) its largest workspace anew per layer call.  Calls
+# recorded into a HIP graph take a tensor of their own from the graph's pool, as any other tensor made under capture.
+_WS_CACHE = {}
+_WS_CACHE_ON = [True]
+
+
 def _workspace(nbytes, dev):
     if nbytes == 0:
         return None
-    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    if not _WS_CACHE_ON[0] or torch.cuda.is_current_stream_capturing():
+        return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    dev = torch.device(dev)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    key = (index, torch.cuda.current_stream(dev).cuda_stream)
+    ws = _WS_CACHE.get(key)
+    if ws is None or ws.numel() < nbytes:
+        _WS_CACHE.pop(key, None)      # (the old one goes back to the allocator before the new one is asked for)
+        ws = None
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _WS_CACHE[key] = ws
+    return ws
+
+
+def _release_workspaces():
+    """Drops the cached workspace tensors (they return to torch's caching allocator)."""
+    _WS_CACHE.clear()
+
+
+def _set_workspace_caching(on):
+    _WS_CACHE_ON[0] = bool(on)
+    if not on:
+        _WS_CACHE.clear()
+
+
+def _workspace_bytes_cached():
+    return {k: v.numel() for k, v in _WS_CACHE.items()}
 
 
 def _check_common(nd, input, offset, alpha, weight, bias, groups, offset_groups):
@@ -417,6 +451,10 @@ def _set_max_intermediate_elements(m):
 config = types.SimpleNamespace(
     get_max_intermediate_elements=_get_max_intermediate_elements,
     set_max_intermediate_elements=_set_max_intermediate_elements,
+    # not in the reference: the workspace tensors this layer keeps per (device, stream)
+    release_workspaces=_release_workspaces,
+    set_workspace_caching=_set_workspace_caching,
+    cached_workspace_bytes=_workspace_bytes_cached,
 )
 
 

@@ -416,9 +416,10 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
     w.goutp = w.gwacc + d2c_align_up((size_t)s.Cout * s.cg * s.K * sizeof(float));
     w.auxacc = w.goutp + d2c_align_up(d2c_bwd_goutp_bytes(s, q.dtype));
-    // fp32 scratch of the offset / mask gradient, used only when the data kernel splits its steps
+    // fp32 scratch of the offset / mask gradient, used when the data kernel splits its steps or reduces the output
+    // channels in several passes (the partial sums then add up in fp32, whatever the storage type of the result)
     w.total = w.auxacc;
-    if (d2c_bwd_data_split(s, q.dtype) > 1)
+    if (d2c_bwd_data_split(s, q.dtype) > 1 || !d2c_tiled_bwd_single_pass(s, q.dtype))
         w.total += d2c_align_up((size_t)s.N * s.G * s.K * s.P * (s.nd + 1) * sizeof(float));
     w.gcol = w.counts = w.entries = w.ovf = 0;
     if (use_lists(q, s) || use_aux_kernel(q, s)) {

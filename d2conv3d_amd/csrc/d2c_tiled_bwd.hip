@@ -1,15 +1,20 @@
-// Backward pass on the matrix cores, without a column buffer.
+// Backward pass on the matrix cores.
 //
-// Kernel 1 (tiled_bwd_data_kernel), per workgroup a tile of output positions,
-// per step one (tap, channel chunk):
+// Kernel 1, per workgroup a tile of output positions, per step one (tap, channel chunk):
 //     gcol[pos, c]  = sum_o gout[pos, o] * W[o, c, k]                (MFMA; dconv3d_gpu.cu:976-1000)
+//   The gout operand of a wavefront (its 32 positions x all output channels of the weight group) stays in registers
+//   for the whole kernel; the weight operand of the step is staged in LDS.
+//   tiled_bwd_col_kernel (the usual path) writes the grad-column rows to a buffer [chunk][tap][position][BKC] in
+//   device memory, which two kernels of their own read back: the offset / mask gradient (d2c_aux_grad.hip) and
+//   grad_input from per-voxel sample lists (d2c_invlist.hip).  This round trip through memory (N*P*K*Cin elements
+//   written once, read twice) is the price of running those two without the barriers and the register budget of
+//   the matrix kernel.
+//   tiled_bwd_data_kernel (shapes the other path does not take: several passes over the output channels, no sample
+//   lists) consumes the rows where they are made:
 //     gx[corner, c] += a_corner * alpha * gcol[pos, c]               (atomics; :593-642)
 //     dot[corner]    = sum_c gcol[pos, c] * x[corner, c]
 //     gmask          = sum_corner a_corner * dot[corner]             (:837-839)
 //     goff_axis      = alpha * sum_corner (d a_corner / d axis) * dot[corner]   (:708-754, :848-858)
-//   The gout operand of a wavefront (its 32 positions x all output channels of
-//   the weight group) stays in registers for the whole kernel; the weight
-//   operand of the step is staged in LDS; gcol never leaves the chip.
 //
 // Kernel 2 (tiled_bwd_weight_dma_kernel), per workgroup one (tap, channel chunk)
 // and all output channels, looping over position tiles:
@@ -1334,7 +1339,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
     }
     const long n_mask = (long)s.N * s.G * s.K * s.P, n_off = n_mask * s.nd;
     float *auxoff = nullptr, *auxmask = nullptr;
-    if (nsplit > 1 && (goff || gmask)) {
+    if ((nsplit > 1 || s.og > omax) && (goff || gmask) && auxacc) {
         auxoff = auxacc;
         auxmask = auxacc + n_off;
         D2cProfScope prof(D2C_PROF_PACK, st);

@@ -164,9 +164,15 @@ int d2c_conv3d_corner_index(const d2c_conv3d_desc *desc, const void *offset, int
 uint64_t d2c_get_max_intermediate_elements(void);
 void d2c_set_max_intermediate_elements(uint64_t m);
 
-/* Test hook: force a kernel family (D2C_ALGO_*; D2C_ALGO_AUTO restores the
- * default choice).  A forced family that cannot serve a description makes the
- * call fail with D2C_ERR_UNSUPPORTED. */
+/* Test hook, not for production callers: force a kernel family (D2C_ALGO_*;
+ * D2C_ALGO_AUTO restores the default choice).  A forced family that cannot
+ * serve a description makes the call fail with D2C_ERR_UNSUPPORTED.  The
+ * setting is one per process (an atomic; every device and thread sees it) and
+ * both the *_workspace_bytes queries and the calls read it: changing it from
+ * another thread between a query and its call makes that call fail with
+ * D2C_ERR_WORKSPACE at worst, never write out of bounds, but the hook is not
+ * meant to be flipped while calls are in flight.  The same holds for
+ * d2c_set_grad_input_mode() below. */
 void d2c_set_algo_override(int algo);
 
 /*
@@ -302,7 +308,8 @@ int d2c_dwconv3d_backward(const d2c_dwconv3d_desc *desc, const void *grad_out, c
  * per-voxel sample lists, every element written once; 0 scatters with fp32 atomics
  * like the reference (dconv3d_gpu.cu:637).  A value n >= 2 is mode 1 with lists
  * that hold at most n samples per voxel before the overflow path takes the rest
- * (by default the capacity follows from the shape).  Workspace sizes depend on the mode. */
+ * (by default the capacity follows from the shape).  Workspace sizes depend on the mode.
+ * One setting per process, for tests only (see d2c_set_algo_override). */
 void d2c_set_grad_input_mode(int mode);
 
 const char *d2c_last_error(void);
