@@ -227,16 +227,21 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                     // the four results are linear in the 8 dots: combine per lane, then sum over the 8 lanes
                     const float lz = tab_of(2, pos), ly = tab_of(3, pos), lx = tab_of(4, pos);
                     const float hz = tab_of(5, pos), hy = tab_of(6, pos), hx = tab_of(7, pos);
-                    float gz = 0.f, gy = 0.f, gxx = 0.f, gm = 0.f;
+                    // axis by axis (31 operations instead of ~80 for the eight corners one by one): along x the
+                    // differences and the interpolated values of the four (z, y) edges, then along y, then z.
+                    // (Corners out of range have dot 0.  The modulation gradient counts live corners only, and a
+                    // point has either all of its in-range corners live or none: see make_tap3.)
+                    float ex[4], sx[4];
 #pragma unroll
-                    for (int c = 0; c < 8; c++) {
-                        const float wz = (c & 4) ? hz : lz, wy = (c & 2) ? hy : ly, wx = (c & 1) ? hx : lx;
-                        const float d = dot[c];
-                        gz += ((c & 4) ? d : -d) * (wy * wx);
-                        gy += ((c & 2) ? d : -d) * (wz * wx);
-                        gxx += ((c & 1) ? d : -d) * (wz * wy);
-                        if ((live >> c) & 1u) gm += (wz * wy * wx) * d;
+                    for (int e = 0; e < 4; e++) {
+                        ex[e] = dot[2 * e + 1] - dot[2 * e];
+                        sx[e] = fmaf(hx, dot[2 * e + 1], lx * dot[2 * e]);
                     }
+                    float gxx = fmaf(hz, fmaf(hy, ex[3], ly * ex[2]), lz * fmaf(hy, ex[1], ly * ex[0]));
+                    const float sy0 = fmaf(hy, sx[1], ly * sx[0]), sy1 = fmaf(hy, sx[3], ly * sx[2]);
+                    float gy = fmaf(hz, sx[3] - sx[2], lz * (sx[1] - sx[0]));
+                    float gz = sy1 - sy0;
+                    float gm = live ? fmaf(hz, sy1, lz * sy0) : 0.f;
                     gz = sum_over_8_lanes(gz);
                     gy = sum_over_8_lanes(gy);
                     gxx = sum_over_8_lanes(gxx);
