@@ -136,22 +136,34 @@ def cpu_baseline(name, torch):
     if c["dt"] == "bf16":
         x, w, b, gout, off, m = (t.bfloat16().float() for t in (x, w, b, gout, off, m))
     fwd, bwd = (cpu.conv3d_forward, cpu.conv3d_backward) if c["nd"] == 3 else (cpu.conv1d_forward, cpu.conv1d_backward)
-    reps = 1
-    t0 = time.perf_counter()
-    while True:
+    # timed iterations until 5 s have passed (at most 200); the figure is the median iteration when there are at
+    # least five of them (after one untimed warm-up iteration), else the mean
+    def once():
         fwd(x, off, m, w, b, 1, 1, 1, c["groups"], c["G"])
         if c["backward"]:
             bwd(gout, x, off, m, w, True, 1, 1, 1, c["groups"], c["G"])
-        dt = time.perf_counter() - t0
-        if dt > 5.0 or reps >= 200:
+    times = []
+    t_start = time.perf_counter()
+    while True:
+        t0 = time.perf_counter()
+        once()
+        t1 = time.perf_counter()
+        times.append(t1 - t0)
+        if t1 - t_start > 5.0 or len(times) >= 201:
             break
-        reps += 1
+    if len(times) >= 6:
+        timed = sorted(times[1:])
+        per_iter, stat = timed[len(timed) // 2], "median"
+    else:
+        timed = times
+        per_iter, stat = sum(times) / len(times), "mean"
     f_fwd, _, _ = algorithmic(name, x.shape[0], tuple(x.shape[2:]))
-    flops = (3 if c["backward"] else 1) * f_fwd * reps
+    flops = (3 if c["backward"] else 1) * f_fwd
     what = "full workload" if crop is None else f"same layer on N={crop[0]}, {'x'.join(map(str, crop[1]))} positions"
     return {
-        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu.num_threads(), "kind": "port",
-        "sample": f"{what}, fp32, {'forward+backward' if c['backward'] else 'forward'} x{reps}: {dt:.2f} s",
+        "value": flops / per_iter / 1e12, "unit": "TFLOP/s", "cores": cpu.num_threads(), "kind": "port",
+        "sample": f"{what}, fp32, {'forward+backward' if c['backward'] else 'forward'}: {stat} of {len(timed)} "
+                  f"iterations = {per_iter * 1e3:.2f} ms ({sum(times):.2f} s of CPU work)",
     }
 
 
@@ -377,6 +389,11 @@ def main():
     ap.add_argument("--offset-axes", type=int, default=7,
                     help="mask of the axes the offsets displace along (1 z, 2 y, 4 x): 6 = the Spatial layers, 1 = the "
                          "Temporal layers of the reference (3-D matrix-core workloads only; default all three)")
+    ap.add_argument("--grad-input-mode", type=int, default=1, choices=[0, 1],
+                    help="matrix-core backward: 1 (default) grad-column rows through device memory, offset / mask "
+                         "gradient and grad_input (from sample lists) as kernels of their own; 0 everything inside "
+                         "the grad-column kernel, grad_input scattered with atomics (the reference's formulation; for "
+                         "comparison)")
     ap.add_argument("--expanded-offsets", action="store_true",
                     help="dynamic-dilation workloads (c2_*): expand the dilation map to an offsets tensor first "
                          "and time the ordinary operator on it, instead of handing the map to the operator")
@@ -388,6 +405,7 @@ def main():
     import torch
     from d2conv3d_amd import _lib
     lib = _lib.load()  # raises if the HIP library is missing: there is no fallback
+    lib.d2c_set_grad_input_mode(args.grad_input_mode)
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     if args.workload == "c2_sizemap":
@@ -603,6 +621,7 @@ def main():
                    "offsets": ("formed in the sampler from the dilation map [N,3,T,H,W] (d2c_conv3d_sized_*)" if sized
                                else "offsets tensor [N,3*K*G,T,H,W]"),
                    "offset_axes": args.offset_axes,
+                   "grad_input_mode": args.grad_input_mode,
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "taps_outside_volume": taps,
