@@ -221,6 +221,18 @@ struct TiledShape {
     FastDiv dP, dHW, dW;  // divisions by P, Ho * Wo and Wo
 };
 
+// With offsets fixed along some axes only the corners on the near side of those axes can have weight: 2^(free axes) of
+// them.  Slot j of those is the corner whose bits are the bits of j spread over the free axes (corner bit 2 = z,
+// 1 = y, 0 = x; `axes` bit 0 = z free, 1 = y, 2 = x).
+__host__ __device__ inline int corner_of_slot(int j, int axes)
+{
+    int c = 0;
+    if (axes & 4) { c |= (j & 1); j >>= 1; }          // x
+    if (axes & 2) { c |= (j & 1) << 1; j >>= 1; }     // y
+    if (axes & 1) { c |= (j & 1) << 2; }              // z
+    return c;
+}
+
 // make_tap3 for the tiled kernels: corners that a fixed axis leaves with weight zero are not fetched.
 D2C_DEV Tap3<float> tiled_tap3(const TiledShape &s, int bz, int by, int bx, float oz, float oy, float ox)
 {

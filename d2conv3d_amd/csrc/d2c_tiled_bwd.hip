@@ -730,16 +730,18 @@ constexpr int kWMT = 128;  // positions per tile of the packed grad_out copy
 // tile `it`, tile it+1 is interpolated from LDS, the rows of tile it+2 are in flight and the table of tile
 // it+3 is computed.  Same roles and ring buffers as tiled_fwd_dma_kernel (d2c_tiled_fwd.hip).
 constexpr int kWDT = 64;                    // positions per iteration
-constexpr int kWRawPos = 8 * 128;           // raw bytes per position: 8 corner rows of 128 bytes
 
 struct BwdWeightDmaArgs {
     BwdWeightArgs w;
     unsigned zrow;       // byte offset (from xcl) of a 128-byte row of zeros: what dead corners read
 };
 
-template <typename T, bool AUX16, bool SIZED>
+// NC: corner rows per sampling point, 8, or 4 / 2 when offsets along one / two axes are fixed (see fwd_dma_body).
+template <typename T, bool AUX16, bool SIZED, int NC>
 __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(BwdWeightDmaArgs aa)
 {
+    constexpr int RAWPOS = NC * 128;           // raw bytes per position
+    constexpr int PPI = 8 / NC;                // positions per DMA instruction
     constexpr int MT = kWDT;
     constexpr int VEC = Elem<T>::VEC;          // positions per 16-byte operand vector
     constexpr int BKC = 8 * VEC;               // channels per step (64 / 32)
@@ -753,7 +755,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
 
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *s_raw = smem;                                       // [2][MT][8 corners][128 B]
-    unsigned char *s_tile = s_raw + 2 * MT * kWRawPos;                 // [2][BKC][TRS]
+    unsigned char *s_tile = s_raw + 2 * MT * RAWPOS;                   // [2][BKC][TRS]
     float *s_w = reinterpret_cast<float *>(s_tile + 2 * BKC * TRS);    // [3][8][MT]
     int2 *s_if = reinterpret_cast<int2 *>(s_w + 3 * 8 * MT);           // [3][MT] (offset of corner 000, live corners)
 
@@ -861,7 +863,9 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     };
 
     // --- corner rows of tile i -> s_raw[rbuf]: worker wavefront w requests positions 8w .. 8w+7
-    const int dcorner = lane >> 3, dvec = lane & 7;
+    // (with fewer than 8 corners an instruction covers 8 / NC positions: lane = (position, corner slot, vector))
+    const int dslot = (lane >> 3) % NC, dsub = (lane >> 3) / NC, dvec = lane & 7;
+    const int dcorner = NC == 8 ? dslot : corner_of_slot(dslot, s.axes);
     const int dcoff = ((dcorner >> 2) & 1) * dzc + ((dcorner >> 1) & 1) * dyc + (dcorner & 1) * s.Cin;
     auto dma_issue = [&](int rbuf, int tbuf) {
         if (!worker) return;
@@ -869,28 +873,38 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
         const int2 vif = s_if[tbuf * MT + wave * (MT / 8) + (lane & 7)];
         const int vidx = vif.x, vflag = vif.y;
 #pragma unroll
-        for (int i = 0; i < MT / 8; i++) {
-            const int pos = wave * (MT / 8) + i;
-            const int idx = __builtin_amdgcn_readlane(vidx, i);
-            const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
+        for (int i = 0; i < MT / 8 / PPI; i++) {
+            const int pos0 = wave * (MT / 8) + i * PPI;
+            int idx;
+            unsigned live;
+            if constexpr (PPI == 1) {
+                idx = __builtin_amdgcn_readlane(vidx, i);
+                live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
+            } else {
+                idx = __builtin_amdgcn_ds_bpermute((i * PPI + dsub) << 2, vidx);
+                live = (unsigned)__builtin_amdgcn_ds_bpermute((i * PPI + dsub) << 2, vflag);
+            }
             const unsigned o = ((live >> dcorner) & 1u)
                                    ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
                                    : aa.zrow + (unsigned)dvec * 16u;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + o),
-                                             (__attribute__((address_space(3))) void *)(s_raw + (rbuf * MT + pos) * kWRawPos),
+                                             (__attribute__((address_space(3))) void *)(s_raw + (rbuf * MT + pos0) * RAWPOS),
                                              16, 0, 0);
         }
     };
     // --- interpolation; thread = (position, 16-byte vector)
     const int ipos = tid >> 3, ivec = tid & 7;
+    int wslot[NC];      // row of the weight table that belongs to corner slot c
+#pragma unroll
+    for (int c = 0; c < NC; c++) wslot[c] = (NC == 8 ? c : corner_of_slot(c, s.axes)) * MT;
     auto interp_store = [&](int rbuf, int tbuf, int dbuf) {
         if (!worker) return;
-        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * kWRawPos + ivec * 16;
+        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16;
         VecAcc<T> va;
         va.zero();
 #pragma unroll
-        for (int c = 0; c < 8; c++)
-            va.fma(s_w[(tbuf * 8 + c) * MT + ipos], *reinterpret_cast<const uint4 *>(rp + c * 128));
+        for (int c = 0; c < NC; c++)
+            va.fma(s_w[tbuf * 8 * MT + wslot[c] + ipos], *reinterpret_cast<const uint4 *>(rp + c * 128));
         if constexpr (sizeof(T) == 2) {
             // bfloat16: the tile stays [position][channel] (one 16-byte store, rows of TRS bytes: MT == BKC);
             // the matrix wavefronts read it with the transposing LDS load, see mma_tile
@@ -1018,10 +1032,10 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     }
 }
 
-template <typename T> constexpr size_t bwd_weight_dma_lds()
+template <typename T, int NC> constexpr size_t bwd_weight_dma_lds()
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
-    return (size_t)2 * kWDT * kWRawPos + (size_t)2 * BKC * (kWDT * sizeof(T) + 16) + (size_t)3 * 10 * kWDT * 4;
+    return (size_t)2 * kWDT * NC * 128 + (size_t)2 * BKC * (kWDT * sizeof(T) + 16) + (size_t)3 * 10 * kWDT * 4;
 }
 
 // ============================================================ small kernels
@@ -1497,19 +1511,29 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
                        (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T))};
     {
         const dim3 grid((unsigned)(items * (nmain + ntail)));
-        constexpr size_t lds = bwd_weight_dma_lds<T>();
         bool aux16 = false;
         if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
-        auto go = [&](auto aux_c, auto sized_c) -> bool {
+        auto go_nc = [&](auto aux_c, auto sized_c, auto nc_c) -> bool {
             constexpr bool A16 = decltype(aux_c)::value, SZ = decltype(sized_c)::value;
-            if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, A16, SZ>,
+            constexpr int NC = decltype(nc_c)::value;
+            constexpr size_t lds = bwd_weight_dma_lds<T, NC>();
+            if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, A16, SZ, NC>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
                 return false;
-            hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, A16, SZ>), grid, dim3(kThreads + 64), lds, st, a);
+            hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, A16, SZ, NC>), grid, dim3(kThreads + 64), lds, st, a);
             return true;
         };
         const bool sized = s.ss.on != 0;
+        // offsets fixed along one / two axes: 4 / 2 corner rows per sampling point (offsets-tensor source only)
+        const int nfree = (s.nd == 3 && !sized) ? __builtin_popcount(s.axes & 7) : 3;
+        auto go = [&](auto aux_c, auto sized_c) -> bool {
+            if constexpr (!decltype(sized_c)::value) {
+                if (nfree == 2) return go_nc(aux_c, sized_c, std::integral_constant<int, 4>{});
+                if (nfree == 1) return go_nc(aux_c, sized_c, std::integral_constant<int, 2>{});
+            }
+            return go_nc(aux_c, sized_c, std::integral_constant<int, 8>{});
+        };
         bool ok;
         if constexpr (sizeof(T) == 2) {
             if (aux16) ok = sized ? go(std::true_type{}, std::true_type{}) : go(std::true_type{}, std::false_type{});

@@ -282,7 +282,6 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
 // pipeline stays full from one segment into the next; only the matrix-core
 // wavefronts notice a segment's end (they store or add their accumulators).
 constexpr int kDMT = 64;                   // positions per workgroup
-constexpr int kRawPos = 8 * kNV * 16;      // raw bytes per position: 8 corners x 128
 
 // Workgroup barrier that waits for this wavefront's LDS operations only: its global loads and DMA transfers
 // stay in flight across it (a __syncthreads() would wait for them as well).
@@ -346,7 +345,9 @@ D2C_DEV bool seg_advance(SegWalk &w, const int4 *s_seg, int nseg, const TiledSha
 
 // (The LDS regions are passed as restrict-qualified pointers: that gives their accesses alias scopes, without
 // which the compiler makes every LDS store wait for all DMA transfers in flight, whatever region they fill.)
-template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED>
+// NC: corner rows fetched and interpolated per sampling point: 8, or 4 / 2 when offsets along one / two axes are fixed
+// (TiledShape::axes; the corners on the far side of a fixed axis have weight zero and no slot at all).
+template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED, int NC>
 D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, unsigned char *__restrict__ s_tile,
                           float *__restrict__ s_w, int2 *__restrict__ s_if,
                           int *__restrict__ s_meta, int4 *__restrict__ s_seg)
@@ -361,6 +362,8 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     constexpr int NKG = kNV / 2;          // k-groups per step
     static_assert(MT * kNV == kThreads, "one (position, vector) item per thread");
     static_assert(WAVES_O * WAVES_P <= kThreads / 64 && PB >= 1, "MMA wave layout");
+    constexpr int RAWPOS = NC * kNV * 16;   // raw bytes per position
+    constexpr int PPI = 8 / NC;             // positions per DMA instruction
 
     const TiledShape &s = a.s;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -518,42 +521,57 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
 
     // --- corner rows of a step -> s_raw[rbuf]: worker wavefront w requests positions 8w .. 8w+7, one
     // instruction per position, lane = (corner, 16-byte vector)
-    const int dcorner = lane >> 3, dvec = lane & 7;
+    // (with fewer than 8 corners an instruction covers 8 / NC positions: lane = (position, corner slot, vector); slot j
+    // is the corner whose bits are those of j spread over the free axes)
+    const int dslot = (lane >> 3) % NC, dsub = (lane >> 3) / NC, dvec = lane & 7;
+    const int dcorner = NC == 8 ? dslot : corner_of_slot(dslot, s.axes);
     const int dcoff = ((dcorner >> 2) & 1) * dzc + ((dcorner >> 1) & 1) * dyc + (dcorner & 1) * s.Cin;
+    // one request: the rows of position(s) wave * 8 + i * PPI (+ dsub); `vidx` / `vflag` hold the table entries of the
+    // wavefront's 8 positions (lane i: position i)
+    auto dma_request = [&](int i, int vidx, int vflag, int c0, int rbuf) {
+        const char *base = reinterpret_cast<const char *>(a.xcl);
+        const int pos0 = wave * (MT / 8) + i * PPI;
+        int idx;
+        unsigned live;
+        if constexpr (PPI == 1) {
+            idx = __builtin_amdgcn_readlane(vidx, i);
+            live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
+        } else {
+            idx = __builtin_amdgcn_ds_bpermute((i * PPI + dsub) << 2, vidx);
+            live = (unsigned)__builtin_amdgcn_ds_bpermute((i * PPI + dsub) << 2, vflag);
+        }
+        const unsigned o = ((live >> dcorner) & 1u)
+                               ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
+                               : a.zrow + (unsigned)dvec * 16u;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + o),
+                                         (__attribute__((address_space(3))) void *)(s_raw + (rbuf * MT + pos0) * RAWPOS),
+                                         16, 0, 0);
+    };
     // (past the end of the sequence the tables are those of three steps before, or the ones of coords_none: the
     // same number of transfers in every iteration, which lets the compiler count the loads in flight instead of
     // waiting for all)
     auto dma_issue = [&](int rbuf, int tbuf) {
         if (!worker) return;
         const int c0 = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4]);
-        const char *base = reinterpret_cast<const char *>(a.xcl);
         // table entries of this wavefront's 8 positions: one LDS read (lane i holds position i), then
         // lane-indexed moves to scalar registers
         const int2 vif = s_if[tbuf * MT + wave * (MT / 8) + (lane & 7)];
-        const int vidx = vif.x, vflag = vif.y;
 #pragma unroll
-        for (int i = 0; i < MT / 8; i++) {
-            const int pos = wave * (MT / 8) + i;
-            const int idx = __builtin_amdgcn_readlane(vidx, i);
-            const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
-            const unsigned o = ((live >> dcorner) & 1u)
-                                   ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
-                                   : a.zrow + (unsigned)dvec * 16u;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + o),
-                                             (__attribute__((address_space(3))) void *)(s_raw + (rbuf * MT + pos) * kRawPos),
-                                             16, 0, 0);
-        }
+        for (int i = 0; i < MT / 8 / PPI; i++) dma_request(i, vif.x, vif.y, c0, rbuf);
     };
     // --- interpolation: thread = (position, 16-byte vector)
     const int ipos = tid >> 3, ivec = tid & 7;
+    int wslot[NC];      // row of the weight table that belongs to corner slot c
+#pragma unroll
+    for (int c = 0; c < NC; c++) wslot[c] = (NC == 8 ? c : corner_of_slot(c, s.axes)) * MT;
     auto interp_store = [&](int rbuf, int tbuf, int dbuf) {
         if (!worker) return;
-        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * kRawPos + ivec * 16;
+        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16;
         VecAcc<T> acc;
         acc.zero();
 #pragma unroll
-        for (int c = 0; c < 8; c++)
-            acc.fma(s_w[(tbuf * 8 + c) * MT + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
+        for (int c = 0; c < NC; c++)
+            acc.fma(s_w[tbuf * 8 * MT + wslot[c] + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
         *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = acc.pack();
     };
 
@@ -583,11 +601,9 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     auto mma_dma_step = [&](int dbuf, int rbuf, int tbuf) {
         const unsigned char *tb = s_tile + (dbuf * MT + wave_p * WPOS + (lane & 31)) * kRS + (lane >> 5) * 16;
         const int c0 = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4]);
-        const char *base = reinterpret_cast<const char *>(a.xcl);
         // table entries of this wavefront's 8 positions: one LDS read (lane i holds position i), then
         // lane-indexed moves to scalar registers
         const int2 vif = s_if[tbuf * MT + wave * (MT / 8) + (lane & 7)];
-        const int vidx = vif.x, vflag = vif.y;
         constexpr int DPK = 4;                                // requests per k-group
 #pragma unroll
         for (int kg = 0; kg < NKG; kg++) {
@@ -602,28 +618,21 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
 #pragma unroll
             for (int q = 0; q < DPK; q++) {
                 const int i = kg * DPK + q;
-                if (i >= MT / 8) break;
-                const int pos = wave * (MT / 8) + i;
-                const int idx = __builtin_amdgcn_readlane(vidx, i);
-                const unsigned live = (unsigned)__builtin_amdgcn_readlane(vflag, i);
-                const unsigned o = ((live >> dcorner) & 1u)
-                                       ? (unsigned)(idx + c0 + dcoff + dvec * VEC) * (unsigned)sizeof(T)
-                                       : a.zrow + (unsigned)dvec * 16u;
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + o),
-                                                 (__attribute__((address_space(3))) void *)(s_raw + (rbuf * MT + pos) * kRawPos),
-                                                 16, 0, 0);
+                if (i >= MT / 8 / PPI) break;
+                dma_request(i, vif.x, vif.y, c0, rbuf);
             }
         }
     };
     // interpolation of one step; the weight fragments of that step are fetched on the way
     auto interp_wload_store = [&](int rbuf, int tbuf, int dbuf) {
-        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * kRawPos + ivec * 16;
+        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16;
         const int wstep = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4 + 1]);
         VecAcc<T> va;
         va.zero();
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-            va.fma(s_w[(tbuf * 8 + c) * MT + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
+            if (c < NC)
+                va.fma(s_w[tbuf * 8 * MT + wslot[c < NC ? c : 0] + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
             af[c / OB][c % OB] = wfrag(wstep, c / OB, c % OB);
         }
         *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = va.pack();
@@ -793,19 +802,19 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     }
 }
 
-template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED>
+template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED, int NC>
 __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
 {
     constexpr int MT = kDMT;
     // (separate arrays, not slices of one: the compiler then knows which of them a DMA transfer fills, and
     // lets accesses to the others go ahead while transfers are in flight)
-    __shared__ __align__(16) unsigned char s_raw[2 * MT * kRawPos];   // [2][MT][8 corners][128 B]
+    __shared__ __align__(16) unsigned char s_raw[2 * MT * NC * kNV * 16];   // [2][MT][NC corners][128 B]
     __shared__ __align__(16) unsigned char s_tile[2 * MT * kRS];      // [2][MT][kRS]
     __shared__ float s_w[3 * 8 * MT];                                 // [3][8][MT]
     __shared__ int2 s_if[3 * MT];                                     // [3][MT] (offset of corner 000, live corners)
     __shared__ int s_meta[3 * 4];                                     // [3][first channel, weight-fragment row]
     __shared__ int4 s_seg[2 * kMaxSeg];                               // [kMaxSeg][2]
-    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P, SIZED>(a, s_raw, s_tile, s_w, s_if, s_meta, s_seg);
+    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P, SIZED, NC>(a, s_raw, s_tile, s_w, s_if, s_meta, s_seg);
 }
 
 // out = fp32 tile + bias for the items whose steps were shared out (see FwdArgs).  One block = 32 output
@@ -908,8 +917,12 @@ int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
     {
         const int nwg = nshare ? ncu : (a.sk_items < nwg_whole ? a.sk_items : nwg_whole);
         D2cProfScope prof(D2C_PROF_FWD, st);
-        if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
-        else hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        // offsets fixed along one / two axes (the layers that deform in space or in time only): 4 / 2 corner rows
+        const int nfree = a.s.nd == 3 ? __builtin_popcount(a.s.axes & 7) : 3;
+        if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        else if (nfree == 2) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 4>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        else if (nfree == 1) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 2>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        else hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 8>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         if (int rc = d2c_check_launch("tiled_fwd_dma_kernel")) return rc;
     }
     if (nshare) {
