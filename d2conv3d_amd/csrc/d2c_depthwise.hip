@@ -459,11 +459,18 @@ __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 
     }
 }
 
-// fp32 accumulator -> offset / mask gradient in its storage type
-__global__ void __launch_bounds__(256) dw_aux_finish_kernel(const float *src, void *dst, int adt, long n)
+// fp32 accumulators (offset part, then mask part) -> offset / mask gradient in their storage type; a NULL
+// destination is skipped
+__global__ void __launch_bounds__(256) dw_aux_finish_kernel(const float *src, void *goff, void *gmask, int adt, long n_off,
+                                                            long n_mask)
 {
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
-        st_aux(dst, i, adt, src[i]);
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n_off + n_mask; i += (long)gridDim.x * blockDim.x) {
+        if (i < n_off) {
+            if (goff) st_aux(goff, i, adt, src[i]);
+        } else if (gmask) {
+            st_aux(gmask, i - n_off, adt, src[i]);
+        }
+    }
 }
 
 // W[c][0][k] -> wt[k][c]
@@ -527,11 +534,12 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
 }
 
 // `goutcl` is the channels-last copy of grad_out.  `gxcl` NULL: grad_input is not wanted here (or comes
-// from the sample lists afterwards); otherwise it is accumulated with atomics.
+// from the sample lists afterwards); otherwise it is accumulated with atomics.  `cleared`: the caller has zeroed
+// `gwacc` and `auxacc` (together with its other scratch, in one launch).
 template <typename T>
 int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
                            const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc,
-                           void *gw, hipStream_t st)
+                           void *gw, hipStream_t st, bool cleared)
 {
     const long n_mask = (long)s.N * s.G * s.K * s.P, n_off = 3 * n_mask;
     float *auxoff = goff ? auxacc : nullptr, *auxmask = gmask ? auxacc + n_off : nullptr;
@@ -540,8 +548,8 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
         hipLaunchKernelGGL(dw_pack_weight_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, (const T *)w,
                            (T *)wt, s.Cin, s.K);
         if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
-        if (gwacc) d2c_fill_zero(gwacc, (size_t)s.Cin * s.K * sizeof(float), st);
-        if (goff || gmask) d2c_fill_zero(auxacc, (size_t)(n_off + n_mask) * sizeof(float), st);
+        if (gwacc && !cleared) d2c_fill_zero(gwacc, (size_t)s.Cin * s.K * sizeof(float), st);
+        if ((goff || gmask) && !cleared) d2c_fill_zero(auxacc, (size_t)(n_off + n_mask) * sizeof(float), st);
     }
     DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, goutcl, gxcl, auxoff, auxmask, gwacc};
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
@@ -555,9 +563,9 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
     if (int rc = d2c_check_launch("dw_bwd_kernel")) return rc;
     if (goff || gmask) {
         D2cProfScope prof(D2C_PROF_PACK, st);
-        if (goff) hipLaunchKernelGGL(dw_aux_finish_kernel, dim3(g1d(n_off)), dim3(256), 0, st, auxoff, goff, s.adt, n_off);
-        if (gmask)
-            hipLaunchKernelGGL(dw_aux_finish_kernel, dim3(g1d(n_mask)), dim3(256), 0, st, auxmask, gmask, s.adt, n_mask);
+        // (one launch for both: the two fp32 arrays follow each other)
+        hipLaunchKernelGGL(dw_aux_finish_kernel, dim3(g1d(n_off + n_mask)), dim3(256), 0, st, auxacc, goff, gmask, s.adt,
+                           n_off, n_mask);
         if (int rc = d2c_check_launch("dw_aux_finish_kernel")) return rc;
     }
     if (gwacc && gw) {
@@ -575,6 +583,6 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
                                           void *, const void *, void *, hipStream_t);                                \
     template int d2c_depthwise_backward<T>(const TiledShape &, const void *, const void *, const void *,             \
                                            const void *, const void *, void *, float *, void *, void *, float *,     \
-                                           float *, void *, hipStream_t);
+                                           float *, void *, hipStream_t, bool);
 INST(bf16_t)
 INST(float)

@@ -7,8 +7,9 @@
 // turned around:
 //
 //   1. every live sample (b, g, k, p) is filed under its base voxel
-//      floor(z, y, x) (counting sort: count, scan, fill), with its tap, its
-//      three fractions and its modulation;
+//      floor(z, y, x) (a bucket of fixed capacity per voxel, filled in one pass;
+//      what does not fit goes to an overflow array), with its tap, its three
+//      fractions and its modulation;
 //   2. the grad-column values gcol[p, (k, chunk), c] are written once by the
 //      data kernel (in the element type of the call);
 //   3. one 8-lane group per (2 x 2 x 2 voxel cube, channel chunk) walks the
@@ -50,99 +51,6 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
         e.pad0 = 0; e.pad1 = 0;
         lists_insert(L, bin_of(s, b, g, t.z0, t.y0, t.x0), e);
     }
-}
-
-template <bool FILL>
-__global__ void __launch_bounds__(256)
-invlist_pass_kernel(TiledShape s, const void *off, const void *mask, int *counts, const int *starts, InvEntry *entries)
-{
-    // grid = (position blocks, taps, samples x offset groups): no 64-bit index arithmetic per thread
-    const int k = blockIdx.y;
-    const int b = blockIdx.z / s.G, g = blockIdx.z - b * s.G;
-    for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < s.P; p += gridDim.x * blockDim.x) {
-        const int ox = p % s.Wo, oy = (p / s.Wo) % s.Ho, oz = p / (s.Wo * s.Ho);
-        float o0, o1, o2;
-        load_offsets(s, off, b, g, k, p, o0, o1, o2);
-        int bz, by, bx;
-        tap_base(s.geo, k, oz, oy, ox, bz, by, bx);
-        const Tap3<float> t = tiled_tap3(s, bz, by, bx, o0, o1, o2);
-        if (!t.live) continue;
-        const int bin = bin_of(s, b, g, t.z0, t.y0, t.x0);
-        const int n = atomicAdd(&counts[bin], 1);
-        if (FILL) {
-            InvEntry e;
-            e.p = p; e.k = k; e.hz = t.hz; e.hy = t.hy; e.hx = t.hx;
-            e.alpha = mask ? ld_aux(mask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt) : 1.f;
-            e.pad0 = 0; e.pad1 = 0;
-            entries[starts[bin] + n] = e;
-        }
-    }
-}
-
-// exclusive prefix sum of `n` ints in three launches (1024 elements per block)
-constexpr int kScanBlock = 1024;
-__global__ void __launch_bounds__(256) scan_block_sums(const int *in, int *bsum, int n)
-{
-    __shared__ int part[4];
-    const int base = blockIdx.x * kScanBlock;
-    int acc = 0;
-    for (int i = threadIdx.x; i < kScanBlock; i += 256) acc += (base + i < n) ? in[base + i] : 0;
-#pragma unroll
-    for (int sft = 32; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft, 64);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) bsum[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
-}
-__global__ void __launch_bounds__(256) scan_of_sums(int *bsum, int nb)
-{
-    // one workgroup, sequential over chunks of 256 block sums
-    __shared__ int buf[256];
-    __shared__ int carry;
-    if (threadIdx.x == 0) carry = 0;
-    __syncthreads();
-    for (int base = 0; base < nb; base += 256) {
-        const int i = base + threadIdx.x;
-        const int v = i < nb ? bsum[i] : 0;
-        buf[threadIdx.x] = v;
-        __syncthreads();
-        for (int d = 1; d < 256; d <<= 1) {   // Hillis-Steele inclusive scan
-            const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
-            __syncthreads();
-            buf[threadIdx.x] += t;
-            __syncthreads();
-        }
-        if (i < nb) bsum[i] = carry + buf[threadIdx.x] - v;
-        __syncthreads();
-        if (threadIdx.x == 255) carry += buf[255];
-        __syncthreads();
-    }
-}
-__global__ void __launch_bounds__(256) scan_apply(const int *in, const int *bsum, int *out, int n)
-{
-    // sequential-per-thread scan of 4 elements, then a block scan of the 256 partial sums
-    __shared__ int buf[256];
-    const int base = blockIdx.x * kScanBlock + threadIdx.x * 4;
-    int v[4], s = 0;
-#pragma unroll
-    for (int j = 0; j < 4; j++) { v[j] = (base + j < n) ? in[base + j] : 0; s += v[j]; }
-    buf[threadIdx.x] = s;
-    __syncthreads();
-    for (int d = 1; d < 256; d <<= 1) {
-        const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
-        __syncthreads();
-        buf[threadIdx.x] += t;
-        __syncthreads();
-    }
-    int run = bsum[blockIdx.x] + buf[threadIdx.x] - s;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        if (base + j < n) out[base + j] = run;
-        run += v[j];
-    }
-}
-__global__ void set_total(const int *counts, int *starts, int n)
-{
-    if (threadIdx.x == 0 && blockIdx.x == 0) starts[n] = n > 0 ? starts[n - 1] + counts[n - 1] : 0;
 }
 
 // ---- owner-computes accumulation ------------------------------------------
@@ -329,8 +237,7 @@ template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
 
 template <typename T>
 __global__ void __launch_bounds__(64 * kOwnVox)
-dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts, const InvEntry *entries,
-                   float *gxcl, int w_in_lds)
+dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, SampleLists L, float *gxcl, int w_in_lds)
 {
     // One wavefront per 2 x 2 x 2 cube of voxels (kOwnVox cubes consecutive in x per workgroup, sharing the
     // weights of the channel slice in LDS): the lists of the 27 base voxels that reach the cube are walked once
@@ -381,45 +288,50 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
         for (int ry = 0; ry < 3; ry++) {
             const int yb = y0 - 1 + ry;
             if (yb > s.H - 1) continue;
-            // the (up to) three base voxels along x are adjacent bins: one range of entries
+            // the (up to) three base voxels along x are adjacent bins; each has its bucket
             const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
-            const int e0 = starts[bin1], em1 = starts[bin1 + 1], em2 = starts[bin1 + 2], e1 = starts[bin1 + nxb];
-            for (int e = e0; e < e1; e += 4) {
-                InvEntry q[4];
-                float go[4][kOwnCV];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    q[i] = entries[min(e + i, e1 - 1)];
-                    ld_vec4<T>(grow + (long)q[i].p * s.Cout + c, go[i]);
-                }
+            for (int rx = 0; rx < 3; rx++) {
+                if (rx >= nxb) continue;
+                const int bin = bin1 + rx;
+                const int n = min(L.counts[bin], L.cap);
+                const InvEntry *entries = L.entries + (long)bin * L.cap;
+                for (int e = 0; e < n; e += 4) {
+                    InvEntry q[4];
+                    float go[4][kOwnCV];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    float wk[kOwnCV];
-                    if (w_in_lds) ld_vec4<T>(s_w + q[i].k * kOwnSlice + t * kOwnCV, wk);
-                    else ld_vec4<T>(wt + (long)q[i].k * s.Cin + c, wk);
-                    const float al = e + i < e1 ? q[i].alpha : 0.f;
-                    float v[kOwnCV];
+                    for (int i = 0; i < 4; i++) {
+                        q[i] = entries[min(e + i, n - 1)];
+                        ld_vec4<T>(grow + (long)q[i].p * s.Cout + c, go[i]);
+                    }
 #pragma unroll
-                    for (int jj = 0; jj < kOwnCV; jj++) v[jj] = wk[jj] * go[i][jj];
-                    // x: offset 0 (base x0-1) reaches voxel 0 with hx; 1 reaches (1-hx, hx); 2 reaches voxel 1 with 1-hx
-                    const float hz = q[i].hz, hy = q[i].hy, hx = q[i].hx;
-                    const bool r0 = e + i < em1, r2 = e + i >= em2;
-                    const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
-                    const float wx1 = r0 ? 0.f : (r2 ? 1.f - hx : hx);
+                    for (int i = 0; i < 4; i++) {
+                        float wk[kOwnCV];
+                        if (w_in_lds) ld_vec4<T>(s_w + q[i].k * kOwnSlice + t * kOwnCV, wk);
+                        else ld_vec4<T>(wt + (long)q[i].k * s.Cin + c, wk);
+                        const float al = e + i < n ? q[i].alpha : 0.f;
+                        float v[kOwnCV];
 #pragma unroll
-                    for (int az = 0; az < 2; az++) {
-                        if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
-                        const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
+                        for (int jj = 0; jj < kOwnCV; jj++) v[jj] = wk[jj] * go[i][jj];
+                        // x: base x0-1 reaches voxel 0 with hx; x0 reaches (1-hx, hx); x0+1 reaches voxel 1 with 1-hx
+                        const float hz = q[i].hz, hy = q[i].hy, hx = q[i].hx;
+                        const float wx0 = rx == 0 ? hx : (rx == 2 ? 0.f : 1.f - hx);
+                        const float wx1 = rx == 0 ? 0.f : (rx == 2 ? 1.f - hx : hx);
 #pragma unroll
-                        for (int ay = 0; ay < 2; ay++) {
-                            if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
-                            const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
-                            const float wzy = wz * wy * al;
-                            const float w0 = wzy * wx0, w1 = wzy * wx1;
+                        for (int az = 0; az < 2; az++) {
+                            if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
+                            const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
 #pragma unroll
-                            for (int jj = 0; jj < kOwnCV; jj++) {
-                                acc[az][ay][0][jj] = fmaf(w0, v[jj], acc[az][ay][0][jj]);
-                                acc[az][ay][1][jj] = fmaf(w1, v[jj], acc[az][ay][1][jj]);
+                            for (int ay = 0; ay < 2; ay++) {
+                                if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
+                                const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
+                                const float wzy = wz * wy * al;
+                                const float w0 = wzy * wx0, w1 = wzy * wx1;
+#pragma unroll
+                                for (int jj = 0; jj < kOwnCV; jj++) {
+                                    if (rx != 2) acc[az][ay][0][jj] = fmaf(w0, v[jj], acc[az][ay][0][jj]);
+                                    if (rx != 0) acc[az][ay][1][jj] = fmaf(w1, v[jj], acc[az][ay][1][jj]);
+                                }
                             }
                         }
                     }
@@ -442,6 +354,43 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, const int *starts
             }
 }
 
+// The samples that found their bucket full (usually none), added with atomics: one 64-lane group per (entry, 256
+// channels of its offset group), a lane owns kOwnCV channels.
+template <typename T>
+__global__ void __launch_bounds__(256)
+dw_gx_overflow_kernel(TiledShape s, const T *goutcl, const T *wt, SampleLists L, float *gxcl)
+{
+    const int novf = min(L.counts[L.nbins], L.ovf_cap);
+    const int t = threadIdx.x & 63;
+    const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
+    const long ngrp = (long)gridDim.x * 4, total = (long)novf * nslice;
+    for (long w = (long)blockIdx.x * 4 + (threadIdx.x >> 6); w < total; w += ngrp) {
+        const int i = (int)(w / nslice), sl = (int)(w - (long)i * nslice);
+        const InvEntry e = L.ovf[i];
+        int bin = e.pad0;
+        const int x0 = bin % (s.W + 1) - 1; bin /= s.W + 1;
+        const int y0 = bin % (s.H + 1) - 1; bin /= s.H + 1;
+        const int z0 = bin % (s.D + 1) - 1; bin /= s.D + 1;
+        const int g = bin % s.G, b = bin / s.G;
+        const int cl = sl * kOwnSlice + t * kOwnCV;
+        if (cl >= s.cpg) continue;
+        const int c = g * s.cpg + cl;
+        float go[kOwnCV], wk[kOwnCV];
+        ld_vec4<T>(goutcl + ((long)b * s.P + e.p) * s.Cout + c, go);
+        ld_vec4<T>(wt + (long)e.k * s.Cin + c, wk);
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int z = z0 + ((q >> 2) & 1), y = y0 + ((q >> 1) & 1), x = x0 + (q & 1);
+            if (z < 0 || z >= s.D || y < 0 || y >= s.H || x < 0 || x >= s.W) continue;
+            const float wgt = ((q & 4) ? e.hz : 1.f - e.hz) * ((q & 2) ? e.hy : 1.f - e.hy) * ((q & 1) ? e.hx : 1.f - e.hx)
+                              * e.alpha;
+            float *o = gxcl + ((long)b * s.vol + ((long)z * s.H + y) * s.W + x) * s.Cin + c;
+#pragma unroll
+            for (int j = 0; j < kOwnCV; j++) atomicAdd(o + j, wgt * (wk[j] * go[j]));
+        }
+    }
+}
+
 inline unsigned g1d(long n, int cap = 16384)
 {
     long g = (n + 255) / 256;
@@ -452,41 +401,6 @@ inline unsigned g1d(long n, int cap = 16384)
 
 // ------------------------------------------------------------------ host
 long d2c_invlist_bins(const TiledShape &s) { return (long)s.N * s.G * (s.D + 1) * (s.H + 1) * (s.W + 1); }
-
-// workspace pieces (bytes), in this order: counts | starts | block sums | entries
-void d2c_invlist_ws(const TiledShape &s, size_t *counts, size_t *starts, size_t *bsums, size_t *entries)
-{
-    const long nb = d2c_invlist_bins(s);
-    *counts = d2c_align_up((size_t)(nb + 1) * 4);
-    *starts = d2c_align_up((size_t)(nb + 1) * 4);
-    *bsums = d2c_align_up((size_t)((nb + kScanBlock - 1) / kScanBlock + 1) * 4);
-    *entries = d2c_align_up((size_t)s.N * s.G * s.K * s.P * sizeof(InvEntry));
-}
-
-int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, int *counts, int *starts, int *bsums,
-                      void *entries, hipStream_t st)
-{
-    D2cProfScope prof(D2C_PROF_PACK, st);
-    const long nbl = d2c_invlist_bins(s);
-    if (nbl >= (1L << 31) - kScanBlock) {
-        d2c_set_error("too many sample bins");
-        return D2C_ERR_UNSUPPORTED;
-    }
-    const int nb = (int)nbl;
-    const dim3 pgrid(g1d(s.P, 4096), s.K, s.N * s.G);
-    d2c_fill_zero(counts, (size_t)(nb + 1) * 4, st);
-    hipLaunchKernelGGL(invlist_pass_kernel<false>, pgrid, dim3(256), 0, st, s, off, mask, counts,
-                       (const int *)nullptr, (InvEntry *)nullptr);
-    const int nblk = (nb + kScanBlock - 1) / kScanBlock;
-    hipLaunchKernelGGL(scan_block_sums, dim3(nblk), dim3(256), 0, st, counts, bsums, nb);
-    hipLaunchKernelGGL(scan_of_sums, dim3(1), dim3(256), 0, st, bsums, nblk);
-    hipLaunchKernelGGL(scan_apply, dim3(nblk), dim3(256), 0, st, counts, bsums, starts, nb);
-    hipLaunchKernelGGL(set_total, dim3(1), dim3(64), 0, st, counts, starts, nb);
-    d2c_fill_zero(counts, (size_t)(nb + 1) * 4, st);   // reused as the per-bin cursor of the fill pass
-    hipLaunchKernelGGL(invlist_pass_kernel<true>, pgrid, dim3(256), 0, st, s, off, mask, counts, starts,
-                       (InvEntry *)entries);
-    return d2c_check_launch("invlist_build");
-}
 
 // Bucket capacity: a power of two above 2.2 x the mean list length K * P / vol (8 .. 256), or what
 // d2c_set_grad_input_mode() asked for.
@@ -535,9 +449,19 @@ int d2c_lists_clear(const SampleLists &L, hipStream_t st)
     d2c_fill_zero(L.counts, (size_t)(L.nbins + 1) * 4, st);
     return d2c_check_launch("lists_clear");
 }
+int d2c_lists_fill(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
 int d2c_lists_build(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st)
 {
     if (int rc = d2c_lists_clear(L, st)) return rc;
+    return d2c_lists_fill(s, off, mask, L, st);
+}
+// ... the same on counts that the caller has cleared
+int d2c_lists_fill(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st)
+{
+    if (L.nbins == 0) {
+        d2c_set_error("too many sample bins");
+        return D2C_ERR_UNSUPPORTED;
+    }
     D2cProfScope prof(D2C_PROF_PACK, st);
     const dim3 pgrid(g1d(s.P, 4096), s.K, s.N * s.G);
     hipLaunchKernelGGL(lists_pass_kernel, pgrid, dim3(256), 0, st, s, off, mask, L);
@@ -564,8 +488,8 @@ template int d2c_gx_owner_launch<float>(const TiledShape &, const void *, const 
 
 // Depthwise case: grad_input from the sample lists, the channels-last grad_out and the tap-major weights.
 template <typename T>
-int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const int *starts,
-                           const void *entries, float *gxcl, hipStream_t st)
+int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const SampleLists &L, float *gxcl,
+                           hipStream_t st)
 {
     D2cProfScope prof(D2C_PROF_GX_OWNER, st);
     size_t lds = (size_t)s.K * kOwnSlice * sizeof(T);
@@ -578,10 +502,14 @@ int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *
     const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
     const unsigned nblk = xcd_unit_grid(s.N * s.G * nslice, ncz * ncy * ((ncx + kOwnVox - 1) / kOwnVox));
     hipLaunchKernelGGL(dw_gx_owner_kernel<T>, dim3(nblk), dim3(64 * kOwnVox), lds, st, s, (const T *)goutcl,
-                       (const T *)wt, starts, (const InvEntry *)entries, gxcl, w_in_lds);
-    return d2c_check_launch("dw_gx_owner_kernel");
+                       (const T *)wt, L, gxcl, w_in_lds);
+    if (int rc = d2c_check_launch("dw_gx_owner_kernel")) return rc;
+    // the overflow entries, usually none (the kernel reads their number from device memory)
+    hipLaunchKernelGGL(dw_gx_overflow_kernel<T>, dim3(256), dim3(256), 0, st, s, (const T *)goutcl, (const T *)wt, L, gxcl);
+    return d2c_check_launch("dw_gx_overflow_kernel");
 }
-template int d2c_dw_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const void *, const int *, const void *,
-                                            float *, hipStream_t);
-template int d2c_dw_gx_owner_launch<float>(const TiledShape &, const void *, const void *, const int *, const void *,
-                                           float *, hipStream_t);
+template int d2c_dw_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const void *, const SampleLists &, float *,
+                                            hipStream_t);
+template int d2c_dw_gx_owner_launch<float>(const TiledShape &, const void *, const void *, const SampleLists &, float *,
+                                           hipStream_t);
+

@@ -22,9 +22,6 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
                               void *gmask, float *auxacc, hipStream_t st);
 int d2c_bwd_data_split(const TiledShape &s, int dtype);
-void d2c_invlist_ws(const TiledShape &s, size_t *counts, size_t *starts, size_t *bsums, size_t *entries);
-int d2c_invlist_build(const TiledShape &s, const void *off, const void *mask, int *counts, int *starts, int *bsums,
-                      void *entries, hipStream_t st);
 template <typename T>
 int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st);
 void d2c_lists_ws(const TiledShape &s, int dtype, size_t *counts, size_t *entries, size_t *ovf);
@@ -32,6 +29,7 @@ SampleLists d2c_lists_make(const TiledShape &s, int dtype, void *counts, void *e
 int d2c_lists_clear(const SampleLists &L, hipStream_t st);
 bool d2c_lists_supported(const TiledShape &s);
 int d2c_lists_build(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
+int d2c_lists_fill(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
 int d2c_gx_mode();
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
@@ -49,12 +47,12 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
                           void *wt, const void *bias, void *out, hipStream_t st);
 template <typename T> int d2c_depthwise_pack_weight(const TiledShape &s, const void *w, void *wt, hipStream_t st);
 template <typename T>
-int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const int *starts,
-                           const void *entries, float *gxcl, hipStream_t st);
+int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const SampleLists &L, float *gxcl,
+                           hipStream_t st);
 template <typename T>
 int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
                            const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc,
-                           void *gw, hipStream_t st);
+                           void *gw, hipStream_t st, bool cleared);
 
 static bool mfma_channels_ok(const d2c_conv3d_desc &q);
 
@@ -328,9 +326,9 @@ bool is_depthwise(const d2c_conv3d_desc &q)
 }
 
 // depthwise workspace: channels-last input | weights [K][C] | grad_input accumulator | grad_weight accumulator |
-// channels-last grad_out | sample lists (counts, starts, block sums, entries)
+// channels-last grad_out | sample lists (bucket counts, buckets of 32-byte entries, overflow array)
 struct DwWs {
-    size_t xcl, wt, gxcl, gwacc, auxacc, goutcl, counts, starts, bsums, entries, total_fwd, total_bwd;
+    size_t xcl, wt, gxcl, gwacc, auxacc, goutcl, counts, entries, ovf, total_fwd, total_bwd;
 };
 DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -342,14 +340,14 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.gxcl = w.total_fwd;
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
     w.auxacc = w.gwacc + d2c_align_up((size_t)s.K * s.Cin * sizeof(float));
-    w.goutcl = w.auxacc + d2c_align_up((size_t)s.N * s.G * s.K * s.P * 4 * sizeof(float));
-    w.counts = w.goutcl + d2c_align_up((size_t)s.N * s.P * s.Cout * es);
-    size_t c, st, bs, en;
-    d2c_invlist_ws(s, &c, &st, &bs, &en);
-    w.starts = w.counts + c;
-    w.bsums = w.starts + st;
-    w.entries = w.bsums + bs;
-    w.total_bwd = w.entries + en;
+    // (grad_weight sums, offset / mask gradient sums and bucket counts follow each other: one clear)
+    size_t c, en, ov;
+    d2c_lists_ws(s, D2C_F32, &c, &en, &ov);      // (32-byte entries whatever the element type)
+    w.counts = w.auxacc + d2c_align_up((size_t)s.N * s.G * s.K * s.P * 4 * sizeof(float));
+    w.goutcl = w.counts + c;
+    w.entries = w.goutcl + d2c_align_up((size_t)s.N * s.P * s.Cout * es);
+    w.ovf = w.entries + en;
+    w.total_bwd = w.ovf + ov;
     return w;
 }
 
@@ -462,21 +460,25 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             so.Cin = s.Cout; so.vol = s.P;
             if (int rc = pack_input<T>(so, gout, base + d.goutcl, st)) return rc;
             const bool lists = gx && d2c_gx_mode() >= 1 && d2c_lists_supported(s);
-            if (lists)
-                if (int rc = d2c_invlist_build(s, off, mask, (int *)(base + d.counts), (int *)(base + d.starts),
-                                               (int *)(base + d.bsums), base + d.entries, st))
-                    return rc;
+            {
+                // grad_weight sums, offset / mask gradient sums, bucket counts: cleared together
+                D2cProfScope prof(D2C_PROF_PACK, st);
+                d2c_fill_zero(base + d.gwacc, d.goutcl - d.gwacc, st);
+            }
+            SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
+            if (lists) {
+                L = d2c_lists_make(s, D2C_F32, base + d.counts, base + d.entries, base + d.ovf);
+                if (int rc = d2c_lists_fill(s, off, mask, L, st)) return rc;
+            }
             if (goff || gmask || gw || !lists)
                 if (int rc = d2c_depthwise_backward<T>(s, base + d.goutcl, base + d.xcl, off, mask, w, base + d.wt,
                                                       lists ? nullptr : gxcl, goff, gmask, (float *)(base + d.auxacc),
-                                                      gwacc, gw, st))
+                                                      gwacc, gw, st, true))
                     return rc;
             if (lists) {
                 if (!(goff || gmask || gw))
                     if (int rc = d2c_depthwise_pack_weight<T>(s, w, base + d.wt, st)) return rc;
-                if (int rc = d2c_dw_gx_owner_launch<T>(s, base + d.goutcl, base + d.wt, (const int *)(base + d.starts),
-                                                       base + d.entries, gxcl, st))
-                    return rc;
+                if (int rc = d2c_dw_gx_owner_launch<T>(s, base + d.goutcl, base + d.wt, L, gxcl, st)) return rc;
             }
             if (gx)
                 if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;

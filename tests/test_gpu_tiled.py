@@ -119,7 +119,7 @@ def test_grad_input_by_atomics_matches_lists(name, dtype, dev):
             assert rel_l2(grads[mode], eg[0]) < 2e-2, mode
 
 
-@pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail"])
+@pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail", "dw64", "dw96_G3_nomask"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("cap", [2, 8])
 @pytest.mark.parametrize("wanted", ["x", "x+aux", "all"])
