@@ -304,6 +304,29 @@ template <bool AUX16, bool SIZED> D2C_DEV void tap_offsets_finish(const TiledSha
     }
 }
 
+// ---- LDS reads of rows that DMA transfers (global_load_lds) filled --------------------------------------------------
+// The compiler makes every LDS read wait for all DMA transfers in flight into the same array (it cannot tell the
+// half being read from the half being filled), i.e. it drains the requests just issued for a later tile before the
+// rows of this one are read.  These reads are hidden from it (inline assembly); the kernels wait for the transfers
+// they need themselves (vmcnt) and for the reads with lds_rows_wait(), through which the values must pass before
+// they are used.
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+template <int OFF> D2C_DEV u32x4_t lds_row_read(unsigned lds_addr)
+{
+    u32x4_t v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(OFF));
+    return v;
+}
+D2C_DEV void lds_rows_wait(u32x4_t &a, u32x4_t &b, u32x4_t &c, u32x4_t &d)
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+D2C_DEV void lds_rows_wait(u32x4_t &a, u32x4_t &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
+D2C_DEV unsigned lds_address(const void *p)
+{
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const void *)p;
+}
+
 // ---- the coordinate wavefront of the DMA-gather kernels ---------------------------------------------------------
 // One wavefront per workgroup turns sampling points into table rows (8 corner weights, the element offset of corner
 // 000, the corners to fetch); an iteration of the workgroup cannot end before its row is written, so this code is

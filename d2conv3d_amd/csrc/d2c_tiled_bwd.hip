@@ -899,12 +899,34 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     for (int c = 0; c < NC; c++) wslot[c] = (NC == 8 ? c : corner_of_slot(c, s.axes)) * MT;
     auto interp_store = [&](int rbuf, int tbuf, int dbuf) {
         if (!worker) return;
-        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16;
+        // (the rows are read behind the compiler's back, see lds_row_read: the transfers just requested for tile
+        // i + 2 stay in flight while tile i + 1 is interpolated)
+        const unsigned rp = lds_address(s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16);
         VecAcc<T> va;
         va.zero();
+        if constexpr (NC == 2) {
+            u32x4_t r0 = lds_row_read<0>(rp), r1 = lds_row_read<128>(rp);
+            const float w0 = s_w[tbuf * 8 * MT + wslot[0] + ipos], w1 = s_w[tbuf * 8 * MT + wslot[1] + ipos];
+            lds_rows_wait(r0, r1);
+            va.fma(w0, __builtin_bit_cast(uint4, r0));
+            va.fma(w1, __builtin_bit_cast(uint4, r1));
+        } else {
 #pragma unroll
-        for (int c = 0; c < NC; c++)
-            va.fma(s_w[tbuf * 8 * MT + wslot[c] + ipos], *reinterpret_cast<const uint4 *>(rp + c * 128));
+            for (int h = 0; h < NC / 4; h++) {
+                u32x4_t r0 = h ? lds_row_read<512>(rp) : lds_row_read<0>(rp);
+                u32x4_t r1 = h ? lds_row_read<640>(rp) : lds_row_read<128>(rp);
+                u32x4_t r2 = h ? lds_row_read<768>(rp) : lds_row_read<256>(rp);
+                u32x4_t r3 = h ? lds_row_read<896>(rp) : lds_row_read<384>(rp);
+                float w[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) w[c] = s_w[tbuf * 8 * MT + wslot[h * 4 + c] + ipos];
+                lds_rows_wait(r0, r1, r2, r3);
+                va.fma(w[0], __builtin_bit_cast(uint4, r0));
+                va.fma(w[1], __builtin_bit_cast(uint4, r1));
+                va.fma(w[2], __builtin_bit_cast(uint4, r2));
+                va.fma(w[3], __builtin_bit_cast(uint4, r3));
+            }
+        }
         if constexpr (sizeof(T) == 2) {
             // bfloat16: the tile stays [position][channel] (one 16-byte store, rows of TRS bytes: MT == BKC);
             // the matrix wavefronts read it with the transposing LDS load, see mma_tile

@@ -564,15 +564,48 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     int wslot[NC];      // row of the weight table that belongs to corner slot c
 #pragma unroll
     for (int c = 0; c < NC; c++) wslot[c] = (NC == 8 ? c : corner_of_slot(c, s.axes)) * MT;
+    // (the rows are read behind the compiler's back, see lds_row_read: the transfers requested during the matrix
+    // step, for the step after the one interpolated here, stay in flight; `between(c)` runs after corner slot c)
+    auto interp_rows = [&](int rbuf, int tbuf, auto between) {
+        const unsigned rp = lds_address(s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16);
+        VecAcc<T> va;
+        va.zero();
+        if constexpr (NC == 2) {
+            u32x4_t r0 = lds_row_read<0>(rp), r1 = lds_row_read<kNV * 16>(rp);
+            const float w0 = s_w[tbuf * 8 * MT + wslot[0] + ipos], w1 = s_w[tbuf * 8 * MT + wslot[1] + ipos];
+            lds_rows_wait(r0, r1);
+            va.fma(w0, __builtin_bit_cast(uint4, r0));
+            between(0);
+            va.fma(w1, __builtin_bit_cast(uint4, r1));
+            between(1);
+        } else {
+#pragma unroll
+            for (int h = 0; h < NC / 4; h++) {
+                constexpr int R = kNV * 16;
+                u32x4_t r0 = h ? lds_row_read<4 * R>(rp) : lds_row_read<0>(rp);
+                u32x4_t r1 = h ? lds_row_read<5 * R>(rp) : lds_row_read<R>(rp);
+                u32x4_t r2 = h ? lds_row_read<6 * R>(rp) : lds_row_read<2 * R>(rp);
+                u32x4_t r3 = h ? lds_row_read<7 * R>(rp) : lds_row_read<3 * R>(rp);
+                float w[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) w[c] = s_w[tbuf * 8 * MT + wslot[h * 4 + c] + ipos];
+                lds_rows_wait(r0, r1, r2, r3);
+                va.fma(w[0], __builtin_bit_cast(uint4, r0));
+                between(h * 4);
+                va.fma(w[1], __builtin_bit_cast(uint4, r1));
+                between(h * 4 + 1);
+                va.fma(w[2], __builtin_bit_cast(uint4, r2));
+                between(h * 4 + 2);
+                va.fma(w[3], __builtin_bit_cast(uint4, r3));
+                between(h * 4 + 3);
+            }
+        }
+        return va;
+    };
     auto interp_store = [&](int rbuf, int tbuf, int dbuf) {
         if (!worker) return;
-        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16;
-        VecAcc<T> acc;
-        acc.zero();
-#pragma unroll
-        for (int c = 0; c < NC; c++)
-            acc.fma(s_w[tbuf * 8 * MT + wslot[c] + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
-        *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = acc.pack();
+        VecAcc<T> va = interp_rows(rbuf, tbuf, [](int) {});
+        *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = va.pack();
     };
 
     // --- MMA role
@@ -625,16 +658,11 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     };
     // interpolation of one step; the weight fragments of that step are fetched on the way
     auto interp_wload_store = [&](int rbuf, int tbuf, int dbuf) {
-        const unsigned char *rp = s_raw + (rbuf * MT + ipos) * RAWPOS + ivec * 16;
         const int wstep = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4 + 1]);
-        VecAcc<T> va;
-        va.zero();
+        VecAcc<T> va = interp_rows(rbuf, tbuf, [&](int c) {
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            if (c < NC)
-                va.fma(s_w[tbuf * 8 * MT + wslot[c < NC ? c : 0] + ipos], *reinterpret_cast<const uint4 *>(rp + c * (kNV * 16)));
-            af[c / OB][c % OB] = wfrag(wstep, c / OB, c % OB);
-        }
+            for (int f = c * (8 / NC); f < (c + 1) * (8 / NC); f++) af[f / OB][f % OB] = wfrag(wstep, f / OB, f % OB);
+        });
         *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = va.pack();
     };
     // end of a segment: whole items get bias, conversion and store; pieces of an item add into its fp32 tile
