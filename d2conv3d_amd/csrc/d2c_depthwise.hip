@@ -450,48 +450,44 @@ __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 
                     }
                 }
             }
-            if (a.gwacc && cok) {
-                float *gw = a.gwacc + (long)(k0 + kk) * s.Cin + c;
+            if (a.gwacc) {
+                // A lane holds 4 consecutive channels; atomics issued that way touch every 64-byte line of the slice's
+                // 1 KiB four times.  The values change lanes first (lane l of instruction j takes channel 64 j + l),
+                // so that an instruction covers 256 consecutive bytes: a quarter of the memory-side operations.
+                static_assert(kCV == 4 && kSlice == 256, "4 x 64 channels per wavefront");
+                float *gw = a.gwacc + (long)(k0 + kk) * s.Cin + g * s.cpg + sl * kSlice;
 #pragma unroll
-                for (int j = 0; j < kCV; j++) atomicAdd(gw + j, gwv[j]);
+                for (int j = 0; j < 4; j++) {
+                    const int src = (16 * j + (lane >> 2)) << 2;
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        v[e] = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(gwv[e])));
+                    const float val = (lane & 2) ? ((lane & 1) ? v[3] : v[2]) : ((lane & 1) ? v[1] : v[0]);
+                    if (sl * kSlice + j * 64 + lane < s.cpg) atomicAdd(gw + j * 64 + lane, val);
+                }
             }
         }
     }
 }
 
-// fp32 accumulators (offset part, then mask part) -> offset / mask gradient in their storage type; a NULL
-// destination is skipped
-__global__ void __launch_bounds__(256) dw_aux_finish_kernel(const float *src, void *goff, void *gmask, int adt, long n_off,
-                                                            long n_mask)
+// What follows the backward kernel, as one launch: the fp32 sums (offset part, then mask part) -> offset / mask gradient
+// in their storage type (a NULL destination is skipped), and gwacc[k][c] (fp32) -> gw[c][0][k]
+template <typename T>
+__global__ void __launch_bounds__(256) dw_finish_kernel(const float *src, void *goff, void *gmask, int adt, long n_off,
+                                                        long n_mask, const float *gwacc, T *gw, int C, int K)
 {
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n_off + n_mask; i += (long)gridDim.x * blockDim.x) {
+    const long n_aux = n_off + n_mask, n = n_aux + (gw ? (long)C * K : 0);
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
         if (i < n_off) {
             if (goff) st_aux(goff, i, adt, src[i]);
-        } else if (gmask) {
-            st_aux(gmask, i - n_off, adt, src[i]);
+        } else if (i < n_aux) {
+            if (gmask) st_aux(gmask, i - n_off, adt, src[i]);
+        } else {
+            const long q = i - n_aux;
+            const int k = (int)(q % K), c = (int)(q / K);
+            gw[q] = f32_to_elem<T>(gwacc[(long)k * C + c]);
         }
-    }
-}
-
-// W[c][0][k] -> wt[k][c]
-template <typename T>
-__global__ void __launch_bounds__(256) dw_pack_weight_kernel(const T *w, T *wt, int C, int K)
-{
-    const long n = (long)C * K;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
-        const int c = (int)(i % C), k = (int)(i / C);
-        wt[i] = w[(long)c * K + k];
-    }
-}
-
-// gwacc[k][c] (fp32) -> gw[c][0][k]
-template <typename T>
-__global__ void __launch_bounds__(256) dw_unpack_gw_kernel(const float *gwacc, T *gw, int C, int K)
-{
-    const long n = (long)C * K;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
-        const int k = (int)(i % K), c = (int)(i / K);
-        gw[i] = f32_to_elem<T>(gwacc[(long)k * C + c]);
     }
 }
 
@@ -509,23 +505,11 @@ bool d2c_depthwise_supported(const TiledShape &s)
     return s.cg == 1 && s.og == 1 && s.cpg % kCV == 0;
 }
 
-template <typename T> int d2c_depthwise_pack_weight(const TiledShape &s, const void *w, void *wt, hipStream_t st)
-{
-    D2cProfScope prof(D2C_PROF_PACK, st);
-    hipLaunchKernelGGL(dw_pack_weight_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, (const T *)w, (T *)wt,
-                       s.Cin, s.K);
-    return d2c_check_launch("dw_pack_weight_kernel");
-}
-
+// `wt`: the weights as [K][C] (see dw_prepare_kernel)
 template <typename T>
-int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *w,
-                          void *wt, const void *bias, void *out, hipStream_t st)
+int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wt,
+                          const void *bias, void *out, hipStream_t st)
 {
-    {
-        D2cProfScope prof(D2C_PROF_PACK, st);
-        hipLaunchKernelGGL(dw_pack_weight_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, (const T *)w,
-                           (T *)wt, s.Cin, s.K);
-    }
     DwArgs a{s, xcl, off, mask, wt, bias, out, nullptr, nullptr, nullptr, nullptr, nullptr};
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
     D2cProfScope prof(D2C_PROF_FWD, st);
@@ -533,23 +517,19 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
     return d2c_check_launch("dw_fwd_kernel");
 }
 
-// `goutcl` is the channels-last copy of grad_out.  `gxcl` NULL: grad_input is not wanted here (or comes
-// from the sample lists afterwards); otherwise it is accumulated with atomics.  `cleared`: the caller has zeroed
-// `gwacc` and `auxacc` (together with its other scratch, in one launch).
+// `goutcl` is the channels-last copy of grad_out, `wt` the weights as [K][C].  `gxcl` NULL: grad_input is not wanted
+// here (or comes from the sample lists afterwards); otherwise it is accumulated with atomics.  The caller has zeroed
+// `gwacc` and `auxacc`.
 template <typename T>
 int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
-                           const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc,
-                           void *gw, hipStream_t st, bool cleared)
+                           const void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc, void *gw,
+                           hipStream_t st)
 {
     const long n_mask = (long)s.N * s.G * s.K * s.P, n_off = 3 * n_mask;
     float *auxoff = goff ? auxacc : nullptr, *auxmask = gmask ? auxacc + n_off : nullptr;
-    {
+    if (gxcl) {
         D2cProfScope prof(D2C_PROF_PACK, st);
-        hipLaunchKernelGGL(dw_pack_weight_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, (const T *)w,
-                           (T *)wt, s.Cin, s.K);
-        if (gxcl) d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
-        if (gwacc && !cleared) d2c_fill_zero(gwacc, (size_t)s.Cin * s.K * sizeof(float), st);
-        if ((goff || gmask) && !cleared) d2c_fill_zero(auxacc, (size_t)(n_off + n_mask) * sizeof(float), st);
+        d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
     }
     DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, goutcl, gxcl, auxoff, auxmask, gwacc};
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
@@ -561,28 +541,23 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
         hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3(dw_grid(s, kBwdTP, s.G * nsl)), dim3(kDwThreads), kDwLdsBwd, st, a);
     }
     if (int rc = d2c_check_launch("dw_bwd_kernel")) return rc;
-    if (goff || gmask) {
+    const bool want_gw = gwacc && gw;
+    if (goff || gmask || want_gw) {
         D2cProfScope prof(D2C_PROF_PACK, st);
-        // (one launch for both: the two fp32 arrays follow each other)
-        hipLaunchKernelGGL(dw_aux_finish_kernel, dim3(g1d(n_off + n_mask)), dim3(256), 0, st, auxacc, goff, gmask, s.adt,
-                           n_off, n_mask);
-        if (int rc = d2c_check_launch("dw_aux_finish_kernel")) return rc;
-    }
-    if (gwacc && gw) {
-        D2cProfScope prof(D2C_PROF_PACK, st);
-        hipLaunchKernelGGL(dw_unpack_gw_kernel<T>, dim3(g1d((long)s.Cin * s.K)), dim3(256), 0, st, gwacc, (T *)gw,
-                           s.Cin, s.K);
-        return d2c_check_launch("dw_unpack_gw_kernel");
+        const long n_aux = (goff || gmask) ? n_off + n_mask : 0;
+        hipLaunchKernelGGL(dw_finish_kernel<T>, dim3(g1d(n_aux + (want_gw ? (long)s.Cin * s.K : 0))), dim3(256), 0, st,
+                           auxacc, goff, gmask, s.adt, (goff || gmask) ? n_off : 0, (goff || gmask) ? n_mask : 0, gwacc,
+                           want_gw ? (T *)gw : nullptr, s.Cin, s.K);
+        return d2c_check_launch("dw_finish_kernel");
     }
     return D2C_OK;
 }
 
 #define INST(T)                                                                                                      \
-    template int d2c_depthwise_pack_weight<T>(const TiledShape &, const void *, void *, hipStream_t);                \
     template int d2c_depthwise_forward<T>(const TiledShape &, const void *, const void *, const void *, const void *, \
-                                          void *, const void *, void *, hipStream_t);                                \
+                                          const void *, void *, hipStream_t);                                        \
     template int d2c_depthwise_backward<T>(const TiledShape &, const void *, const void *, const void *,             \
-                                           const void *, const void *, void *, float *, void *, void *, float *,     \
-                                           float *, void *, hipStream_t, bool);
+                                           const void *, const void *, float *, void *, void *, float *, float *,    \
+                                           void *, hipStream_t);
 INST(bf16_t)
 INST(float)

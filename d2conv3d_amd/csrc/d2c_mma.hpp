@@ -304,6 +304,40 @@ template <bool AUX16, bool SIZED> D2C_DEV void tap_offsets_finish(const TiledSha
     }
 }
 
+// ---- bias gradient of one output channel by a workgroup of NT threads: gb[o] = sum_{b,p} gout[b,o,p]
+// (16-byte loads where the row allows them)
+template <typename T, int NT> D2C_DEV void bias_grad_body(const T *gout, T *gb, int N, int Cout, int P, int o)
+{
+    constexpr int VEC = 16 / (int)sizeof(T);
+    __shared__ float part[NT / 64];
+    float acc = 0.f;
+    for (int b = 0; b < N; b++) {
+        const T *row = gout + ((long)b * Cout + o) * P;
+        const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(row) & 15)) & 15) / sizeof(T));   // to 16-byte alignment
+        const int h = head < P ? head : P;
+        const int nvec = (P - h) / VEC;
+        if ((int)threadIdx.x < h) acc += elem_to_f32<T>(row[threadIdx.x]);
+        const uint4 *rv = reinterpret_cast<const uint4 *>(row + h);
+        for (int i = threadIdx.x; i < nvec; i += NT) {
+            const uint4 v = rv[i];
+            const T *e = reinterpret_cast<const T *>(&v);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc += elem_to_f32<T>(e[j]);
+        }
+        for (int p = h + nvec * VEC + threadIdx.x; p < P; p += NT) acc += elem_to_f32<T>(row[p]);
+    }
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < NT / 64; i++) t += part[i];
+        gb[o] = f32_to_elem<T>(t);
+    }
+}
+
 // ---- LDS reads of rows that DMA transfers (global_load_lds) filled --------------------------------------------------
 // The compiler makes every LDS read wait for all DMA transfers in flight into the same array (it cannot tell the
 // half being read from the half being filled), i.e. it drains the requests just issued for a later tile before the

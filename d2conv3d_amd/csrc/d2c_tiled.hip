@@ -43,16 +43,15 @@ template <typename T> int d2c_tiled_bias_grad(const TiledShape &s, const void *g
 
 bool d2c_depthwise_supported(const TiledShape &s);
 template <typename T>
-int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *w,
-                          void *wt, const void *bias, void *out, hipStream_t st);
-template <typename T> int d2c_depthwise_pack_weight(const TiledShape &s, const void *w, void *wt, hipStream_t st);
+int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wt,
+                          const void *bias, void *out, hipStream_t st);
 template <typename T>
 int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const SampleLists &L, float *gxcl,
                            hipStream_t st);
 template <typename T>
 int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *xcl, const void *off, const void *mask,
-                           const void *w, void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc,
-                           void *gw, hipStream_t st, bool cleared);
+                           const void *wt, float *gxcl, void *goff, void *gmask, float *auxacc, float *gwacc, void *gw,
+                           hipStream_t st);
 
 static bool mfma_channels_ok(const d2c_conv3d_desc &q);
 
@@ -116,16 +115,11 @@ template <typename T> D2C_DEV void pack_zero_row(T *xcl, int C, int vol, int zer
         reinterpret_cast<unsigned *>(xcl + (long)gridDim.z * C * vol)[threadIdx.x] = 0u;
 }
 
-// x [N][C][vol] -> xcl [N][vol][C]  (32 x 32 element tiles through LDS)
-template <typename T>
-__global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int C, int vol, int zero_row)
+// x [C][vol] -> xcl [vol][C] of one batch element: a 32 x 32 element tile through LDS
+template <typename T> D2C_DEV void pack_tile32(const T *xb, T *ob, int C, int vol, int v0, int c0)
 {
-    pack_zero_row(xcl, C, vol, zero_row);
     __shared__ T tile[32][33];
-    const int b = blockIdx.z, v0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    const T *xb = x + (long)b * C * vol;
-    T *ob = xcl + (long)b * C * vol;
 #pragma unroll
     for (int i = 0; i < 32; i += 8) {
         const int c = c0 + ty + i, v = v0 + tx;
@@ -140,15 +134,11 @@ __global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int
 }
 
 // The same for bfloat16 with 16-byte accesses on both sides (2-byte accesses of 32 lanes move 64 bytes per
-// request): 64 x 64 element tiles; needs vol and C to be multiples of 8 and 16-byte aligned tensors.
-__global__ void __launch_bounds__(256) pack_input_bf16_kernel(const bf16_t *x, bf16_t *xcl, int C, int vol, int zero_row)
+// request): a 64 x 64 element tile; needs vol and C to be multiples of 8 and 16-byte aligned tensors.
+D2C_DEV void pack_tile64_bf16(const bf16_t *xb, bf16_t *ob, int C, int vol, int v0, int c0)
 {
-    pack_zero_row(xcl, C, vol, zero_row);
     constexpr int RS = 66;                             // LDS row stride in elements (33 words)
     __shared__ bf16_t tile[64 * RS];                   // [v][c]
-    const int b = blockIdx.z, v0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-    const bf16_t *xb = x + (long)b * C * vol;
-    bf16_t *ob = xcl + (long)b * C * vol;
     for (int i = threadIdx.x; i < 512; i += 256) {     // 64 channels x 8 vectors of 8 positions
         const int c = c0 + i / 8, v = v0 + (i % 8) * 8;
         if (c < C && v < vol) {                        // (vol % 8 == 0: the vector is inside or outside as a whole)
@@ -170,6 +160,78 @@ __global__ void __launch_bounds__(256) pack_input_bf16_kernel(const bf16_t *x, b
             *reinterpret_cast<uint4 *>(ob + (long)v * C + c) = make_uint4(t[0], t[1], t[2], t[3]);
         }
     }
+}
+
+// x [N][C][vol] -> xcl [N][vol][C]
+template <typename T>
+__global__ void __launch_bounds__(256) pack_input_kernel(const T *x, T *xcl, int C, int vol, int zero_row)
+{
+    pack_zero_row(xcl, C, vol, zero_row);
+    const long bo = (long)blockIdx.z * C * vol;
+    pack_tile32<T>(x + bo, xcl + bo, C, vol, blockIdx.x * 32, blockIdx.y * 32);
+}
+
+__global__ void __launch_bounds__(256) pack_input_bf16_kernel(const bf16_t *x, bf16_t *xcl, int C, int vol, int zero_row)
+{
+    pack_zero_row(xcl, C, vol, zero_row);
+    const long bo = (long)blockIdx.z * C * vol;
+    pack_tile64_bf16(x + bo, xcl + bo, C, vol, blockIdx.x * 64, blockIdx.y * 64);
+}
+
+// Everything a depthwise call needs before its main kernels, as one launch: up to two tensors to channels-last (the
+// input, grad_out), the weights W[c][0][k] -> wt[k][c], a range of the workspace cleared, the bias gradient.  A
+// workgroup finds its job from its index; jobs a call does not need have no workgroups.
+struct DwPrepArgs {
+    struct Pack {
+        const void *src;
+        void *dst;
+        int C, vol, wide;     // wide: 64 x 64 bfloat16 tiles (see pack_tile64_bf16)
+        int nbx, nby, nblk;   // tiles along vol and C; workgroups of the job (tiles x batch)
+    } pack[2];
+    const void *w;
+    void *wt;
+    int wC, wK, nblk_w;
+    uint32_t *zero;
+    size_t zero_words;
+    int nblk_z;
+    const void *gout;          // bias gradient: one workgroup per channel
+    void *gb;
+    int bN, bC, bP, nblk_b;
+};
+template <typename T> __global__ void __launch_bounds__(256) dw_prepare_kernel(DwPrepArgs a)
+{
+    int b = blockIdx.x;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const DwPrepArgs::Pack &pk = a.pack[j];
+        if (b < pk.nblk) {
+            const int bx = b % pk.nbx, by = (b / pk.nbx) % pk.nby;
+            const long bo = (long)(b / (pk.nbx * pk.nby)) * pk.C * pk.vol;
+            if constexpr (sizeof(T) == 2) {
+                if (pk.wide) {
+                    pack_tile64_bf16((const bf16_t *)pk.src + bo, (bf16_t *)pk.dst + bo, pk.C, pk.vol, bx * 64, by * 64);
+                    return;
+                }
+            }
+            pack_tile32<T>((const T *)pk.src + bo, (T *)pk.dst + bo, pk.C, pk.vol, bx * 32, by * 32);
+            return;
+        }
+        b -= pk.nblk;
+    }
+    if (b < a.nblk_w) {
+        const T *w = (const T *)a.w;
+        T *wt = (T *)a.wt;
+        const int n = a.wC * a.wK;
+        for (int i = b * 256 + threadIdx.x; i < n; i += a.nblk_w * 256) wt[i] = w[(i % a.wC) * a.wK + i / a.wC];
+        return;
+    }
+    b -= a.nblk_w;
+    if (b < a.nblk_z) {
+        for (size_t i = (size_t)b * 256 + threadIdx.x; i < a.zero_words; i += (size_t)a.nblk_z * 256) a.zero[i] = 0u;
+        return;
+    }
+    b -= a.nblk_z;
+    if (b < a.nblk_b) bias_grad_body<T, 256>((const T *)a.gout, (T *)a.gb, a.bN, a.bC, a.bP, b);
 }
 
 // Forward weight operand in MFMA fragment order:
@@ -319,6 +381,35 @@ int pack_input(const TiledShape &s, const void *x, void *xcl, hipStream_t st, bo
     return d2c_check_launch("pack_input_kernel");
 }
 
+// The jobs of dw_prepare_kernel for one call (gout == nullptr: no grad_out copy; zero_bytes == 0: nothing to clear;
+// gb == nullptr: no bias gradient).
+template <typename T>
+int dw_prepare(const TiledShape &s, const void *x, void *xcl, const void *gout, void *goutcl, const void *w, void *wt,
+               void *zero, size_t zero_bytes, void *gb, hipStream_t st)
+{
+    DwPrepArgs a{};
+    auto job = [&](DwPrepArgs::Pack &pk, const void *src, void *dst, int C, int vol) {
+        pk.src = src; pk.dst = dst; pk.C = C; pk.vol = vol;
+        pk.wide = sizeof(T) == 2 && vol % 8 == 0 && C % 8 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+        const int tl = pk.wide ? 64 : 32;
+        pk.nbx = (vol + tl - 1) / tl; pk.nby = (C + tl - 1) / tl;
+        pk.nblk = pk.nbx * pk.nby * s.N;
+    };
+    job(a.pack[0], x, xcl, s.Cin, s.vol);
+    if (gout) job(a.pack[1], gout, goutcl, s.Cout, s.P);
+    a.w = w; a.wt = wt; a.wC = s.Cin; a.wK = s.K;
+    a.nblk_w = std::min((s.Cin * s.K + 255) / 256, 1024);
+    a.zero = (uint32_t *)zero; a.zero_words = zero_bytes / 4;
+    a.nblk_z = (int)std::min<size_t>((a.zero_words + 1023) / 1024, 2048);
+    a.gout = gout; a.gb = gb; a.bN = s.N; a.bC = s.Cout; a.bP = s.P;
+    a.nblk_b = (gb && gout) ? s.Cout : 0;
+    const long nblk = (long)a.pack[0].nblk + a.pack[1].nblk + a.nblk_w + a.nblk_z + a.nblk_b;
+    D2cProfScope prof(D2C_PROF_PACK, st);
+    hipLaunchKernelGGL(dw_prepare_kernel<T>, dim3((unsigned)nblk), dim3(256), 0, st, a);
+    return d2c_check_launch("dw_prepare_kernel");
+}
+
 bool is_depthwise(const d2c_conv3d_desc &q)
 {
     if (q.dtype != D2C_BF16 && q.dtype != D2C_F32) return false;
@@ -360,8 +451,8 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
     char *base = (char *)ws;
     if (nd == 3 && is_depthwise(q)) {
         const DwWs d = dw_ws(q, s);
-        if (int rc = pack_input<T>(s, x, base + d.xcl, st)) return rc;
-        return d2c_depthwise_forward<T>(s, base + d.xcl, off, mask, w, base + d.wt, bias, out, st);
+        if (int rc = dw_prepare<T>(s, x, base + d.xcl, nullptr, nullptr, w, base + d.wt, nullptr, 0, nullptr, st)) return rc;
+        return d2c_depthwise_forward<T>(s, base + d.xcl, off, mask, base + d.wt, bias, out, st);
     }
     const FwdWs l = fwd_ws(q, s);
     if (int rc = pack_input<T>(s, x, base + l.xcl, st, true)) return rc;   // with the row of zeros behind it
@@ -451,39 +542,32 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
     const void *size_raw = off;   // (size-map source; `off` becomes the per-axis (size - 1) below)
     if (nd == 3 && is_depthwise(q)) {
         const DwWs d = dw_ws(q, s);
-        if (int rc = pack_input<T>(s, x, base + d.xcl, st)) return rc;
         float *gxcl = gx ? (float *)(base + d.gxcl) : nullptr;
         float *gwacc = gw ? (float *)(base + d.gwacc) : nullptr;
-        if (gx || goff || gmask || gw) {
-            // grad_out channels-last: [N][P][C]
-            TiledShape so = s;
-            so.Cin = s.Cout; so.vol = s.P;
-            if (int rc = pack_input<T>(so, gout, base + d.goutcl, st)) return rc;
+        const bool grads = gx || goff || gmask || gw;
+        // one launch: input and grad_out channels-last ([N][P][C]), the weights [K][C], the clear of the grad_weight sums,
+        // offset / mask gradient sums and bucket counts (which follow each other), the bias gradient
+        if (!grads) return gb ? d2c_tiled_bias_grad<T>(s, gout, gb, st) : D2C_OK;
+        if (int rc = dw_prepare<T>(s, x, base + d.xcl, gout, base + d.goutcl, w, base + d.wt,
+                                   grads ? base + d.gwacc : nullptr, grads ? d.goutcl - d.gwacc : 0, gb, st))
+            return rc;
+        if (grads) {
             const bool lists = gx && d2c_gx_mode() >= 1 && d2c_lists_supported(s);
-            {
-                // grad_weight sums, offset / mask gradient sums, bucket counts: cleared together
-                D2cProfScope prof(D2C_PROF_PACK, st);
-                d2c_fill_zero(base + d.gwacc, d.goutcl - d.gwacc, st);
-            }
             SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
             if (lists) {
                 L = d2c_lists_make(s, D2C_F32, base + d.counts, base + d.entries, base + d.ovf);
                 if (int rc = d2c_lists_fill(s, off, mask, L, st)) return rc;
             }
             if (goff || gmask || gw || !lists)
-                if (int rc = d2c_depthwise_backward<T>(s, base + d.goutcl, base + d.xcl, off, mask, w, base + d.wt,
+                if (int rc = d2c_depthwise_backward<T>(s, base + d.goutcl, base + d.xcl, off, mask, base + d.wt,
                                                       lists ? nullptr : gxcl, goff, gmask, (float *)(base + d.auxacc),
-                                                      gwacc, gw, st, true))
+                                                      gwacc, gw, st))
                     return rc;
-            if (lists) {
-                if (!(goff || gmask || gw))
-                    if (int rc = d2c_depthwise_pack_weight<T>(s, w, base + d.wt, st)) return rc;
+            if (lists)
                 if (int rc = d2c_dw_gx_owner_launch<T>(s, base + d.goutcl, base + d.wt, L, gxcl, st)) return rc;
-            }
             if (gx)
                 if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
         }
-        if (gb) return d2c_tiled_bias_grad<T>(s, gout, gb, st);
         return D2C_OK;
     }
     const BwdWs l = bwd_ws(q, s);

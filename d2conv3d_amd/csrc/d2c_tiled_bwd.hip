@@ -1265,40 +1265,11 @@ __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp,
     }
 }
 
-// gb[o] = sum_{b,p} gout[b,o,p]   (dconv3d_gpu.cu:1329)
+// gb[o] = sum_{b,p} gout[b,o,p]   (dconv3d_gpu.cu:1329): one workgroup of 16 wavefronts per output channel
 template <typename T>
 __global__ void __launch_bounds__(1024) bias_grad_kernel(const T *gout, T *gb, int N, int Cout, int P)
 {
-    // one workgroup of 16 wavefronts per output channel; 16-byte loads where the row allows them
-    constexpr int VEC = 16 / (int)sizeof(T);
-    __shared__ float part[16];
-    const int o = blockIdx.x;
-    float acc = 0.f;
-    for (int b = 0; b < N; b++) {
-        const T *row = gout + ((long)b * Cout + o) * P;
-        const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(row) & 15)) & 15) / sizeof(T));   // to 16-byte alignment
-        const int h = head < P ? head : P;
-        const int nvec = (P - h) / VEC;
-        if ((int)threadIdx.x < h) acc += elem_to_f32<T>(row[threadIdx.x]);
-        const uint4 *rv = reinterpret_cast<const uint4 *>(row + h);
-        for (int i = threadIdx.x; i < nvec; i += 1024) {
-            const uint4 v = rv[i];
-            const T *e = reinterpret_cast<const T *>(&v);
-#pragma unroll
-            for (int j = 0; j < VEC; j++) acc += elem_to_f32<T>(e[j]);
-        }
-        for (int p = h + nvec * VEC + threadIdx.x; p < P; p += 1024) acc += elem_to_f32<T>(row[p]);
-    }
-#pragma unroll
-    for (int sft = 32; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft, 64);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float t = 0.f;
-#pragma unroll
-        for (int i = 0; i < 16; i++) t += part[i];
-        gb[o] = f32_to_elem<T>(t);
-    }
+    bias_grad_body<T, 1024>(gout, gb, N, Cout, P, blockIdx.x);
 }
 
 // fp32 scratch of the split data kernel -> offset / mask gradient in its storage type
