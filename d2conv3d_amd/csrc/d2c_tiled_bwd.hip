@@ -489,6 +489,10 @@ D2C_DEV void mma8_bf16(f32x16 &acc, const uint4 *g, const unsigned *w)
         : "memory");
 }
 
+// Row stride (bytes) of the float grad-column block in LDS.  bfloat16 problems: unpadded, 128 rows of 256 bytes =
+// 32 KiB, which leaves room for two 64 KiB weight tiles (512 reduced channels) in the 160 KiB of a workgroup.
+template <typename T> constexpr int col_row_stride() { return 8 * Elem<T>::VEC * 4 + (sizeof(T) == 2 ? 0 : 16); }
+
 template <typename T, int NKG, bool DB>
 __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
 {
@@ -497,7 +501,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     constexpr int CB = BKC / 32;           // 32-channel blocks per step (2 for bf16, 1 for float)
     constexpr int PBW = 8 / CB;            // 32-position blocks per workgroup
     constexpr int MT = 32 * PBW;           // positions per workgroup (128 / 256)
-    constexpr int GRS = BKC * 4 + 16;      // gcol tile row stride (bytes), float
+    constexpr int GRS = col_row_stride<T>();   // gcol tile row stride (bytes), float
     constexpr int NW = kThreads / 64;
     constexpr int ITEMS = MT * NV / kThreads;
 
@@ -541,17 +545,24 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     // weight tile of step st: global -> LDS without passing through registers; one instruction of a wavefront
     // moves 64 pieces to 1 KiB of consecutive LDS (lane i's piece lands at base + 16 i), so lane i fetches the
     // piece that the swizzled layout wants there
-    auto dma_tile = [&](int st, int buf) {
+    auto dma_piece = [&](int st, int buf, int i) {       // instruction i of the tile
         const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * rp;
-        for (int i = wave; i < ninstr; i += NW) {
-            const int pos = i * 64 + lane;
-            const int row = pos / rp, q = pos - row * rp;
-            const uint4 *g = src + row * rp + (q ^ swizzle_of_row(row));
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
-                                             (__attribute__((address_space(3))) void *)(s_wt + buf * tileB + i * 1024), 16,
-                                             0, 0);
-        }
+        const int pos = i * 64 + lane;
+        const int row = pos / rp, q = pos - row * rp;
+        const uint4 *g = src + row * rp + (q ^ swizzle_of_row(row));
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                         (__attribute__((address_space(3))) void *)(s_wt + buf * tileB + i * 1024), 16,
+                                         0, 0);
     };
+    auto dma_tile = [&](int st, int buf) {
+        for (int i = wave; i < ninstr; i += NW) dma_piece(st, buf, i);
+    };
+    // Where the matrix step is the hand-scheduled one (see below), the requests for the next tile are spread between
+    // its four blocks of matrix instructions: a wavefront stalls at the issue of a vector-memory instruction while the
+    // path is busy, and eight requests in a row in front of the matrix step hold it up for most of the transfer.
+    constexpr bool HAND = sizeof(T) == 2 && NKG % 8 == 0;     // matrix step scheduled by hand (mma8_bf16)
+    constexpr bool SPREAD = DB && HAND;
+    const bool spread = SPREAD && nkg == NKG && rp % 16 == 0;
 
     // byte offsets (inside a tile) of this lane's fragments of the first 8 k-groups
     int woff[8];
@@ -572,10 +583,15 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
         const int c0 = wg * s.cg + j * BKC;
         const bool more = st + 1 < st_hi;
         if constexpr (DB) {
-            if (more) dma_tile(st + 1, (it + 1) & 1);
-            // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
-            // flight (requests complete in order; the grad-column stores of the previous step are older)
-            wait_vm_at_most(more ? mine : 0);
+            if (spread) {
+                // (tile st was requested during the matrix step of st-1)
+                wait_vm_at_most(0);
+            } else {
+                if (more) dma_tile(st + 1, (it + 1) & 1);
+                // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
+                // flight (requests complete in order; the grad-column stores of the previous step are older)
+                wait_vm_at_most(more ? mine : 0);
+            }
         } else {
             // one tile buffer: every wavefront is past the matrix step of st-1 (the barrier behind it).  (Requesting
             // the tile earlier, behind that barrier, so that it comes in while the rows go out, was 3 % slower.)
@@ -594,7 +610,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 // row: the pieces of 8 consecutive k-groups share a block of 16 and differ from the next 8 by a
                 // constant, so 8 lane addresses + immediate offsets address all of them; the reads run kPF
                 // fragments ahead of the matrix instructions that take them.
-                if constexpr (sizeof(T) == 2 && NKG == 32) {
+                if constexpr (HAND) {
                     // (the accumulator was cleared by vector moves just now, and is read by vector instructions
                     // right after: the waits that the compiler adds around its own matrix instructions)
                     unsigned wl[8];
@@ -602,10 +618,28 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
 #pragma unroll
                     for (int i = 0; i < 8; i++) wl[i] = lbase + (unsigned)woff[i];
                     asm volatile("s_nop 4" ::: "memory");
+                    auto next_tile = [&](int q) {      // requests 2q, 2q+1 of this wavefront for tile st+1
+                        if constexpr (SPREAD) {
+                            if (more) {
+                                const int i0 = wave + 2 * q * NW, i1 = i0 + NW;
+                                if (i0 < ninstr) dma_piece(st + 1, (it + 1) & 1, i0);
+                                if (i1 < ninstr) dma_piece(st + 1, (it + 1) & 1, i1);
+                            }
+                        }
+                    };
+                    // (a tile has 2 requests per wavefront for every 8 k-groups)
                     mma8_bf16<0>(acc, ga, wl);
-                    mma8_bf16<256>(acc, ga + 8, wl);
-                    mma8_bf16<512>(acc, ga + 16, wl);
-                    mma8_bf16<768>(acc, ga + 24, wl);
+                    next_tile(0);
+                    if constexpr (NKG >= 16) {
+                        mma8_bf16<256>(acc, ga + 8, wl);
+                        next_tile(1);
+                    }
+                    if constexpr (NKG >= 32) {
+                        mma8_bf16<512>(acc, ga + 16, wl);
+                        next_tile(2);
+                        mma8_bf16<768>(acc, ga + 24, wl);
+                        next_tile(3);
+                    }
                     asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc)::"memory");
                 } else {
                     constexpr int kPF = 3;
@@ -667,7 +701,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
 template <typename T> size_t bwd_col_lds(int ogk, bool db)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
-    return (size_t)(db ? 2 : 1) * BKC * ogk * sizeof(T) + (size_t)MT * (BKC * 4 + 16);
+    return (size_t)(db ? 2 : 1) * BKC * ogk * sizeof(T) + (size_t)MT * col_row_stride<T>();
 }
 
 template <typename T, int NKG>
