@@ -447,10 +447,11 @@ D2C_DEV int swizzle_of_row(int row) { return row & 7; }
 // 128-register stationary operand, emits read - wait - multiply for every fragment; here the LDS reads run three
 // fragments ahead of the matrix instructions (four rotating fragment registers; a register is reloaded after the
 // matrix instruction that follows the one which read it).  `w0..w7` are the lane's LDS addresses of the 8 fragments,
-// OFF the byte offset of this block of 8.
+// OFF the byte offset of this block of 8.  The fragments from LDS are the first operand, the stationary `g` the
+// second: the product comes out transposed (lane = column of `g`, i.e. position).
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 template <int OFF>
-D2C_DEV void mma8_bf16(f32x16 &acc, const uint4 *g, const unsigned *w)
+D2C_DEV void mma8_bf16_t(f32x16 &acc, const uint4 *g, const unsigned *w)
 {
     u32x4 b0, b1, b2, b3;
     const u32x4 g0 = __builtin_bit_cast(u32x4, g[0]), g1 = __builtin_bit_cast(u32x4, g[1]),
@@ -463,25 +464,25 @@ D2C_DEV void mma8_bf16(f32x16 &acc, const uint4 *g, const unsigned *w)
         "ds_read_b128 %[b2], %[w2] offset:%[off]\n\t"
         "ds_read_b128 %[b3], %[w3] offset:%[off]\n\t"
         "s_waitcnt lgkmcnt(3)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g0], %[b0], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b0], %[g0], %[acc]\n\t"
         "s_waitcnt lgkmcnt(2)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g1], %[b1], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b1], %[g1], %[acc]\n\t"
         "ds_read_b128 %[b0], %[w4] offset:%[off]\n\t"
         "s_waitcnt lgkmcnt(2)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g2], %[b2], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b2], %[g2], %[acc]\n\t"
         "ds_read_b128 %[b1], %[w5] offset:%[off]\n\t"
         "s_waitcnt lgkmcnt(2)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g3], %[b3], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b3], %[g3], %[acc]\n\t"
         "ds_read_b128 %[b2], %[w6] offset:%[off]\n\t"
         "s_waitcnt lgkmcnt(2)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g4], %[b0], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b0], %[g4], %[acc]\n\t"
         "ds_read_b128 %[b3], %[w7] offset:%[off]\n\t"
         "s_waitcnt lgkmcnt(2)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g5], %[b1], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b1], %[g5], %[acc]\n\t"
         "s_waitcnt lgkmcnt(1)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g6], %[b2], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b2], %[g6], %[acc]\n\t"
         "s_waitcnt lgkmcnt(0)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[acc], %[g7], %[b3], %[acc]\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[acc], %[b3], %[g7], %[acc]\n\t"
         : [acc] "+v"(acc), [b0] "=&v"(b0), [b1] "=&v"(b1), [b2] "=&v"(b2), [b3] "=&v"(b3)
         : [g0] "v"(g0), [g1] "v"(g1), [g2] "v"(g2), [g3] "v"(g3), [g4] "v"(g4), [g5] "v"(g5), [g6] "v"(g6), [g7] "v"(g7),
           [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]), [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]),
@@ -560,14 +561,25 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     // Where the matrix step is the hand-scheduled one (see below), the requests for the next tile are spread between
     // its four blocks of matrix instructions: a wavefront stalls at the issue of a vector-memory instruction while the
     // path is busy, and eight requests in a row in front of the matrix step hold it up for most of the transfer.
-    constexpr bool HAND = sizeof(T) == 2 && NKG % 8 == 0;     // matrix step scheduled by hand (mma8_bf16)
+    constexpr bool HAND = sizeof(T) == 2 && NKG % 8 == 0;     // matrix step scheduled by hand (mma8_bf16_t)
     constexpr bool SPREAD = DB && HAND;
     const bool spread = SPREAD && nkg == NKG && rp % 16 == 0;
+    const bool full_tile = m0 + MT <= s.M;                    // every lane stores its rows: a fixed number of stores
 
     // byte offsets (inside a tile) of this lane's fragments of the first 8 k-groups
+    // Hand-scheduled path: the product is taken transposed, lane = position and the 16 accumulator registers = 16
+    // channels, and the lane's weight row is chosen such that these are two runs of 8 consecutive channels
+    // (register r = 4 i + j holds matrix row 8 i + 4 h + j, h = lane / 32: rows 8 i + 4 h' + j take the channels
+    // 8 h' + 4 i + j for i < 2 and 16 + 8 h' + 4 (i - 2) + j above).  The rows then go from the registers to memory,
+    // 16 bytes per lane and store, without a pass through LDS and without a second barrier per step.
+    const bool direct = HAND && nkg == NKG && rp % 16 == 0;
     int woff[8];
     {
-        const int wrow = cb * 32 + (lane & 31);
+        int wrow = cb * 32 + (lane & 31);
+        if (direct) {
+            const int ml = lane & 31, i = ml >> 3, hq = (ml >> 2) & 1, j = ml & 3;
+            wrow = cb * 32 + (i < 2 ? 8 * hq + 4 * i + j : 16 + 8 * hq + 4 * (i - 2) + j);
+        }
         const int wsw = swizzle_of_row(wrow), wh = lane >> 5;
 #pragma unroll
         for (int i = 0; i < 8; i++) woff[i] = wrow * rowB + (((i * 2 + wh) ^ wsw) << 4);
@@ -584,8 +596,9 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
         const bool more = st + 1 < st_hi;
         if constexpr (DB) {
             if (spread) {
-                // (tile st was requested during the matrix step of st-1)
-                wait_vm_at_most(0);
+                // (tile st was requested during the matrix step of st-1; the two stores of that step's rows are
+                // younger and may stay in flight)
+                wait_vm_at_most(full_tile ? 2 : 0);
             } else {
                 if (more) dma_tile(st + 1, (it + 1) & 1);
                 // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
@@ -628,16 +641,16 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                         }
                     };
                     // (a tile has 2 requests per wavefront for every 8 k-groups)
-                    mma8_bf16<0>(acc, ga, wl);
+                    mma8_bf16_t<0>(acc, ga, wl);
                     next_tile(0);
                     if constexpr (NKG >= 16) {
-                        mma8_bf16<256>(acc, ga + 8, wl);
+                        mma8_bf16_t<256>(acc, ga + 8, wl);
                         next_tile(1);
                     }
                     if constexpr (NKG >= 32) {
-                        mma8_bf16<512>(acc, ga + 16, wl);
+                        mma8_bf16_t<512>(acc, ga + 16, wl);
                         next_tile(2);
-                        mma8_bf16<768>(acc, ga + 24, wl);
+                        mma8_bf16_t<768>(acc, ga + 24, wl);
                         next_tile(3);
                     }
                     asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc)::"memory");
@@ -668,6 +681,24 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 }
             }
         }
+        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
+        if (direct) {
+            if constexpr (HAND) {
+                const int m = m0 + pb * 32 + (lane & 31);
+                if (m < s.M) {
+                    T *row = gb + (long)m * BKC + cb * 32 + 8 * (lane >> 5);
+                    *reinterpret_cast<uint4 *>(row) =
+                        make_uint4(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
+                                   pack_bf16x2(acc[6], acc[7]));
+                    *reinterpret_cast<uint4 *>(row + 16) =
+                        make_uint4(pack_bf16x2(acc[8], acc[9]), pack_bf16x2(acc[10], acc[11]),
+                                   pack_bf16x2(acc[12], acc[13]), pack_bf16x2(acc[14], acc[15]));
+                }
+                // (one tile buffer: the next transfer must not start before every wavefront has read this tile)
+                if constexpr (!DB) lds_only_barrier();
+            }
+            continue;
+        }
         // grad-column block -> LDS: lanes 0..31 / 32..63 each cover 32 consecutive channels
         const int ch = cb * 32 + (lane & 31);
 #pragma unroll
@@ -677,7 +708,6 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
         }
         lds_only_barrier();
         // rows out to memory, 16 bytes per thread
-        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
 #pragma unroll
         for (int i = 0; i < ITEMS; i++) {
             const int item = tid + i * kThreads;
