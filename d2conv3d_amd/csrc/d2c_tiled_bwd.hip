@@ -435,6 +435,13 @@ D2C_DEV void wait_vm_at_most(int n)
     case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
     case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
     case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+    case 9: __builtin_amdgcn_s_waitcnt(0x0F79); break;
+    case 10: __builtin_amdgcn_s_waitcnt(0x0F7A); break;
+    case 11: __builtin_amdgcn_s_waitcnt(0x0F7B); break;
+    case 12: __builtin_amdgcn_s_waitcnt(0x0F7C); break;
+    case 13: __builtin_amdgcn_s_waitcnt(0x0F7D); break;
+    case 14: __builtin_amdgcn_s_waitcnt(0x0F7E); break;
+    case 15: __builtin_amdgcn_s_waitcnt(0x0F7F); break;
     default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
     }
 }
@@ -728,6 +735,141 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     }
 }
 
+// The grad-column product for bfloat16 reductions of 128, 256, 384 or 512 channels: one workgroup = 256 positions
+// (a wavefront keeps the grad_out rows of 32 of them, its stationary operand), a step = 32 channels of one tap, i.e.
+// half a channel chunk; the weight half-tiles ([32 channels][ogk], 32 KiB at 512) go through a ring of kColRing LDS
+// buffers and are requested kColAhead steps before their use, one request per wavefront between two blocks of 8
+// matrix instructions.  Against the 128-position / 64-channel shape of tiled_bwd_col_kernel: half the weight
+// traffic per product, and a transfer has three steps to arrive instead of one (the loaded latency of a tile is
+// about a whole step of that kernel, which waited for it at every step).  The product is taken transposed and
+// stored from the registers (see mma8_bf16_t and the `direct` path of tiled_bwd_col_kernel).
+constexpr int kColRing = 4, kColAhead = 3;
+template <int NB>   // blocks of 8 k-groups: ogk = 128 NB
+__global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a)
+{
+    typedef bf16_t T;
+    constexpr int VEC = 8, BKC = 64, HC = 32, MT = 256, NKG = 8 * NB, NW = kThreads / 64;
+    constexpr int R = NB;                    // requests per wavefront and half-tile (32 rows x ogk / 8 pieces / 64 / 8)
+    static_assert(kColAhead < kColRing && kColRing == 4, "a buffer is refilled a step after its last reader at the earliest");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const TiledShape &s = a.s;
+    const int rowB = a.ogk * (int)sizeof(T), tileB = HC * rowB, rp = rowB / 16;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
+    const int wg = blockIdx.y;
+    const int m0 = tile * MT;
+    const int S = s.nchunk * s.K, S2 = 2 * S;
+    const bool full_tile = m0 + MT <= s.M;
+
+    // ---- stationary operand: gout[pos, o] of this wavefront's 32 positions
+    uint4 ga[NKG];
+    {
+        const int m = m0 + wave * 32 + (lane & 31);
+        const bool ok = m < s.M;
+        const int b = ok ? m / s.P : 0, p = ok ? m - b * s.P : 0;
+        const T *gp = reinterpret_cast<const T *>(a.gout) + ((long)b * s.Cout + wg * s.og + a.o0) * s.P + p;
+#pragma unroll
+        for (int kg = 0; kg < NKG; kg++) {
+            T e[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const int o = (kg * 2 + (lane >> 5)) * VEC + i;
+                e[i] = (ok && o < a.ogn) ? gp[(long)o * s.P] : (T)0;
+            }
+            ga[kg] = *reinterpret_cast<uint4 *>(e);
+        }
+    }
+
+    // request q (0 .. R-1) of this wavefront for half-tile h2 (= 2 * step + half, in the order of the data kernel's
+    // steps) into ring buffer `buf`: 64 pieces of 16 bytes to 1 KiB of consecutive LDS, lane i fetching the piece
+    // that the swizzled layout wants there
+    int psrc[R];      // (which piece of a half-tile the lane fetches does not change from step to step)
+#pragma unroll
+    for (int q = 0; q < R; q++) {
+        const int pos = (wave + q * NW) * 64 + lane;
+        const int row = pos / rp, pc = pos - row * rp;
+        psrc[q] = row * rp + (pc ^ swizzle_of_row(row));
+    }
+    auto dma_piece = [&](int h2, int buf, int q) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + (((long)wg * S + (h2 >> 1)) * BKC + (h2 & 1) * HC) * rp;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + psrc[q]),
+                                         (__attribute__((address_space(3))) void *)(smem + buf * tileB + (wave + q * NW) * 1024),
+                                         16, 0, 0);
+    };
+
+    // LDS addresses of this lane's fragments of the first 8 k-groups in the ring buffer of the current step; the lane's
+    // weight row is the one that makes its 16 accumulator registers two runs of 8 consecutive channels
+    unsigned woff[8];
+    {
+        const int ml = lane & 31, i = ml >> 3, hq = (ml >> 2) & 1, j = ml & 3;
+        const int wrow = i < 2 ? 8 * hq + 4 * i + j : 16 + 8 * hq + 4 * (i - 2) + j;
+        const int wsw = swizzle_of_row(wrow), wh = lane >> 5;
+        const unsigned lbase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
+#pragma unroll
+        for (int q = 0; q < 8; q++) woff[q] = lbase + (unsigned)(wrow * rowB + (((q * 2 + wh) ^ wsw) << 4));
+    }
+
+    const int lo = (int)((long)S2 * blockIdx.z / gridDim.z), hi = (int)((long)S2 * (blockIdx.z + 1) / gridDim.z);
+    if (lo >= hi) return;
+    // (past the end of the range the last half-tile is requested again, into buffers nobody reads: the same number
+    // of requests in every step, which the counted waits below rely on)
+#pragma unroll
+    for (int d = 0; d < kColAhead; d++)
+#pragma unroll
+        for (int q = 0; q < R; q++) dma_piece(min(lo + d, hi - 1), d, q);
+
+    const int cpc2 = 2 * (s.cpg / BKC);        // half-steps per (offset group, tap)
+    for (int h2 = lo, it = 0; h2 < hi; h2++, it++) {
+        // step order: offset group (outer), tap, chunk of the group, half (inner)
+        const int jj2 = h2 % cpc2, k = (h2 / cpc2) % s.K, gi = h2 / (cpc2 * s.K);
+        const int j = gi * (cpc2 >> 1) + (jj2 >> 1), half = jj2 & 1;
+        // Half-tile `it` has landed when no more of this wavefront's operations are in flight than it has issued
+        // since: the requests of the kColAhead - 1 half-tiles behind it, and the 2 stores of each step since then
+        // (only counted when every wavefront of the workgroup stores in every step).
+        wait_vm_at_most((kColAhead - 1) * R + ((full_tile && it >= kColAhead) ? 2 * kColAhead : 0));
+        lds_only_barrier();
+
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.f;
+        const int nx = min(h2 + kColAhead, hi - 1), nbuf = (it + kColAhead) & (kColRing - 1);
+        asm volatile("s_nop 4" ::: "memory");
+        mma8_bf16_t<0>(acc, ga, woff);
+        dma_piece(nx, nbuf, 0);
+        if constexpr (NB >= 2) {
+            mma8_bf16_t<256>(acc, ga + 8, woff);
+            dma_piece(nx, nbuf, 1);
+        }
+        if constexpr (NB >= 3) {
+            mma8_bf16_t<512>(acc, ga + 16, woff);
+            dma_piece(nx, nbuf, 2);
+        }
+        if constexpr (NB >= 4) {
+            mma8_bf16_t<768>(acc, ga + 24, woff);
+            dma_piece(nx, nbuf, 3);
+        }
+        asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc)::"memory");
+        // (the fragment addresses move on to the next buffer of the ring)
+        const unsigned adv = ((it + 1) & (kColRing - 1)) ? (unsigned)tileB : (unsigned)(-(kColRing - 1) * tileB);
+#pragma unroll
+        for (int q = 0; q < 8; q++) woff[q] += adv;
+
+        const int c0 = wg * s.cg + j * BKC;
+        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
+        const int m = m0 + wave * 32 + (lane & 31);
+        if (m < s.M) {
+            T *row = gb + (long)m * BKC + half * HC + 8 * (lane >> 5);
+            *reinterpret_cast<uint4 *>(row) =
+                make_uint4(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
+                           pack_bf16x2(acc[6], acc[7]));
+            *reinterpret_cast<uint4 *>(row + 16) =
+                make_uint4(pack_bf16x2(acc[8], acc[9]), pack_bf16x2(acc[10], acc[11]), pack_bf16x2(acc[12], acc[13]),
+                           pack_bf16x2(acc[14], acc[15]));
+        }
+    }
+    wait_vm_at_most(0);     // (transfers into this workgroup's LDS must not outlive it)
+}
+
 template <typename T> size_t bwd_col_lds(int ogk, bool db)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
@@ -748,6 +890,29 @@ int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st)
     if (db) hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, true>), grid, dim3(kThreads), lds, st, a);
     else hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, false>), grid, dim3(kThreads), lds, st, a);
     return d2c_check_launch("tiled_bwd_col_kernel");
+}
+
+constexpr int kCol32MT = 256;
+bool bwd_col32_ok(int ogk, int ogn, int dtype) { return dtype == D2C_BF16 && ogk % 128 == 0 && ogk <= 512 && ogn > 0; }
+int launch_bwd_col32(const BwdDataArgs &a, int nsplit, hipStream_t st)
+{
+    const size_t lds = (size_t)kColRing * 32 * a.ogk * 2;
+    const dim3 grid((a.s.M + kCol32MT - 1) / kCol32MT, a.s.groups, nsplit);
+    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
+    auto go = [&](auto nb_c) -> int {
+        constexpr int NB = decltype(nb_c)::value;
+        if (hipFuncSetAttribute((const void *)tiled_bwd_col32_kernel<NB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024) != hipSuccess)
+            return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_col32_kernel)");
+        hipLaunchKernelGGL((tiled_bwd_col32_kernel<NB>), grid, dim3(kThreads), lds, st, a);
+        return d2c_check_launch("tiled_bwd_col32_kernel");
+    };
+    switch (a.ogk / 128) {
+    case 1: return go(std::integral_constant<int, 1>{});
+    case 2: return go(std::integral_constant<int, 2>{});
+    case 3: return go(std::integral_constant<int, 3>{});
+    default: return go(std::integral_constant<int, 4>{});
+    }
 }
 
 template <typename T> size_t bwd_data_lds(int ogk)
@@ -1398,13 +1563,16 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         // tiles; the cut is the one whose last round of workgroups is fullest.
         const int ncu = d2c_num_cus();
         if (ncu <= 0) return D2C_ERR_LAUNCH;
-        constexpr int MT = 32 * (8 / (BKC / 32));
+        // (the 256-position kernel of bfloat16 problems walks half-steps; reloading its stationary operand costs
+        // about two of them)
+        const bool c32 = s.og <= omax && bwd_col32_ok(d2c_bwd_ogk(s.og, Elem<T>::DT), s.og, Elem<T>::DT);
+        const int MT = c32 ? kCol32MT : 32 * (8 / (BKC / 32));
         const long items = (long)((s.M + MT - 1) / MT) * s.groups;
-        const int S = s.nchunk * s.K;
-        long best = ((items + ncu - 1) / ncu) * (S + 1);
+        const int S = s.nchunk * s.K * (c32 ? 2 : 1), reload = c32 ? 2 : 1;
+        long best = ((items + ncu - 1) / ncu) * (S + reload);
         nsplit = 1;
         for (int k = 2; k <= 16 && k <= S; k++) {
-            const long cost = ((items * k + ncu - 1) / ncu) * ((S + k - 1) / k + 1);
+            const long cost = ((items * k + ncu - 1) / ncu) * ((S + k - 1) / k + reload);
             if (cost < best) { best = cost; nsplit = k; }
         }
     }
@@ -1444,7 +1612,9 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
         const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
-        if (col_only) {
+        if (col_only && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
+            rc = launch_bwd_col32(a, nsplit, st);
+        } else if (col_only) {
             if (nkg <= 4) rc = launch_bwd_col<T, 4>(a, nsplit, st);
             else if (nkg <= 8) rc = launch_bwd_col<T, 8>(a, nsplit, st);
             else if (nkg <= 16) rc = launch_bwd_col<T, 16>(a, nsplit, st);
