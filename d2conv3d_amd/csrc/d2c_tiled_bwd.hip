@@ -4,7 +4,7 @@
 //     gcol[pos, c]  = sum_o gout[pos, o] * W[o, c, k]                (MFMA; dconv3d_gpu.cu:976-1000)
 //   The gout operand of a wavefront (its 32 positions x all output channels of the weight group) stays in registers
 //   for the whole kernel; the weight operand of the step is staged in LDS.
-//   tiled_bwd_col_kernel (the usual path) writes the grad-column rows to a buffer [chunk][tap][position][BKC] in
+//   tiled_bwd_col32_kernel / tiled_bwd_col_kernel (the usual path) write the grad-column rows to a buffer [chunk][tap][position][BKC] in
 //   device memory, which two kernels of their own read back: the offset / mask gradient (d2c_aux_grad.hip) and
 //   grad_input from per-voxel sample lists (d2c_invlist.hip).  This round trip through memory (N*P*K*Cin elements
 //   written once, read twice) is the price of running those two without the barriers and the register budget of
@@ -410,16 +410,12 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 
 // ---------------------------------------------------------------------------
 // The grad-column product alone (grad_input comes from the sample lists, the offset / mask gradient from the
-// kernel of d2c_aux_grad.hip: the usual case).  Same tiling and operands as tiled_bwd_data_kernel, without its
-// other duties, and with the fragment reads running ahead of the matrix instructions.  Where two weight tiles
-// and the float grad-column block fit LDS (DB: fp32 problems, bfloat16 with up to 256 reduced channels per pass)
-// the weight tile is double-buffered: the DMA transfer of step s+1 is in flight while step s is on the matrix
-// cores.  Two barriers per step, both waiting for LDS operations only.
-// The widest bfloat16 reduction (512 channels: one 64 KB tile + the 35 KB block) stays single-buffered: two
-// tiles next to a bfloat16 block (written by pairs of lanes that swap values) fit, but ran slower in every form
-// tried (0.71 - 0.75 ms against 0.58 ms at C3; as 4 wavefronts of 512 registers per workgroup 1.0 ms).  For it the
-// matrix step is scheduled by hand (mma8_bf16): with the stationary operand alone in 128 of its 256 registers the
-// compiler emits read - wait - multiply for every fragment.
+// kernel of d2c_aux_grad.hip: the usual case).  tiled_bwd_col_kernel: same tiling and operands as
+// tiled_bwd_data_kernel, without its other duties, and with the fragment reads running ahead of the matrix
+// instructions.  Where two weight tiles and the float grad-column block fit LDS (DB) the weight tile is
+// double-buffered: the DMA transfer of step s+1 is in flight while step s is on the matrix cores.  Two barriers
+// per step, both waiting for LDS operations only.  It serves float problems and the bfloat16 reductions that are
+// no multiple of 128 channels; the others take tiled_bwd_col32_kernel further down.
 D2C_DEV void lds_only_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // at most `n` vector-memory operations of this wavefront still in flight
@@ -450,8 +446,9 @@ D2C_DEV void wait_vm_at_most(int n)
 // bank-conflict cycles of the fragment reads from 50 M to 6 M per launch at C3 and made the kernel 5 % slower.)
 D2C_DEV int swizzle_of_row(int row) { return row & 7; }
 
-// Eight k-groups of the matrix step for bfloat16, scheduled by hand: the compiler, short of registers next to the
-// 128-register stationary operand, emits read - wait - multiply for every fragment; here the LDS reads run three
+// Eight k-groups of the matrix step for bfloat16, scheduled by hand: the compiler, short of registers next to a
+// 128-register stationary operand, emits read - wait - multiply for every fragment, and it makes LDS reads that it
+// sees wait for every DMA transfer in flight into the same array; here the LDS reads run three
 // fragments ahead of the matrix instructions (four rotating fragment registers; a register is reloaded after the
 // matrix instruction that follows the one which read it).  `w0..w7` are the lane's LDS addresses of the 8 fragments,
 // OFF the byte offset of this block of 8.  The fragments from LDS are the first operand, the stationary `g` the
@@ -553,40 +550,22 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
     // weight tile of step st: global -> LDS without passing through registers; one instruction of a wavefront
     // moves 64 pieces to 1 KiB of consecutive LDS (lane i's piece lands at base + 16 i), so lane i fetches the
     // piece that the swizzled layout wants there
-    auto dma_piece = [&](int st, int buf, int i) {       // instruction i of the tile
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * rp;
-        const int pos = i * 64 + lane;
-        const int row = pos / rp, q = pos - row * rp;
-        const uint4 *g = src + row * rp + (q ^ swizzle_of_row(row));
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
-                                         (__attribute__((address_space(3))) void *)(s_wt + buf * tileB + i * 1024), 16,
-                                         0, 0);
-    };
     auto dma_tile = [&](int st, int buf) {
-        for (int i = wave; i < ninstr; i += NW) dma_piece(st, buf, i);
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * rp;
+        for (int i = wave; i < ninstr; i += NW) {
+            const int pos = i * 64 + lane;
+            const int row = pos / rp, q = pos - row * rp;
+            const uint4 *g = src + row * rp + (q ^ swizzle_of_row(row));
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                             (__attribute__((address_space(3))) void *)(s_wt + buf * tileB + i * 1024), 16,
+                                             0, 0);
+        }
     };
-    // Where the matrix step is the hand-scheduled one (see below), the requests for the next tile are spread between
-    // its four blocks of matrix instructions: a wavefront stalls at the issue of a vector-memory instruction while the
-    // path is busy, and eight requests in a row in front of the matrix step hold it up for most of the transfer.
-    constexpr bool HAND = sizeof(T) == 2 && NKG % 8 == 0;     // matrix step scheduled by hand (mma8_bf16_t)
-    constexpr bool SPREAD = DB && HAND;
-    const bool spread = SPREAD && nkg == NKG && rp % 16 == 0;
-    const bool full_tile = m0 + MT <= s.M;                    // every lane stores its rows: a fixed number of stores
 
     // byte offsets (inside a tile) of this lane's fragments of the first 8 k-groups
-    // Hand-scheduled path: the product is taken transposed, lane = position and the 16 accumulator registers = 16
-    // channels, and the lane's weight row is chosen such that these are two runs of 8 consecutive channels
-    // (register r = 4 i + j holds matrix row 8 i + 4 h + j, h = lane / 32: rows 8 i + 4 h' + j take the channels
-    // 8 h' + 4 i + j for i < 2 and 16 + 8 h' + 4 (i - 2) + j above).  The rows then go from the registers to memory,
-    // 16 bytes per lane and store, without a pass through LDS and without a second barrier per step.
-    const bool direct = HAND && nkg == NKG && rp % 16 == 0;
     int woff[8];
     {
-        int wrow = cb * 32 + (lane & 31);
-        if (direct) {
-            const int ml = lane & 31, i = ml >> 3, hq = (ml >> 2) & 1, j = ml & 3;
-            wrow = cb * 32 + (i < 2 ? 8 * hq + 4 * i + j : 16 + 8 * hq + 4 * (i - 2) + j);
-        }
+        const int wrow = cb * 32 + (lane & 31);
         const int wsw = swizzle_of_row(wrow), wh = lane >> 5;
 #pragma unroll
         for (int i = 0; i < 8; i++) woff[i] = wrow * rowB + (((i * 2 + wh) ^ wsw) << 4);
@@ -602,16 +581,10 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
         const int c0 = wg * s.cg + j * BKC;
         const bool more = st + 1 < st_hi;
         if constexpr (DB) {
-            if (spread) {
-                // (tile st was requested during the matrix step of st-1; the two stores of that step's rows are
-                // younger and may stay in flight)
-                wait_vm_at_most(full_tile ? 2 : 0);
-            } else {
-                if (more) dma_tile(st + 1, (it + 1) & 1);
-                // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
-                // flight (requests complete in order; the grad-column stores of the previous step are older)
-                wait_vm_at_most(more ? mine : 0);
-            }
+            if (more) dma_tile(st + 1, (it + 1) & 1);
+            // this wavefront's pieces of tile st have landed when only its requests for tile st+1 are still in
+            // flight (requests complete in order; the grad-column stores of the previous step are older)
+            wait_vm_at_most(more ? mine : 0);
         } else {
             // one tile buffer: every wavefront is past the matrix step of st-1 (the barrier behind it).  (Requesting
             // the tile earlier, behind that barrier, so that it comes in while the rows go out, was 3 % slower.)
@@ -630,50 +603,17 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 // row: the pieces of 8 consecutive k-groups share a block of 16 and differ from the next 8 by a
                 // constant, so 8 lane addresses + immediate offsets address all of them; the reads run kPF
                 // fragments ahead of the matrix instructions that take them.
-                if constexpr (HAND) {
-                    // (the accumulator was cleared by vector moves just now, and is read by vector instructions
-                    // right after: the waits that the compiler adds around its own matrix instructions)
-                    unsigned wl[8];
-                    const unsigned lbase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)wb;
+                constexpr int kPF = 3;
+                uint4 bq[kPF + 1];
 #pragma unroll
-                    for (int i = 0; i < 8; i++) wl[i] = lbase + (unsigned)woff[i];
-                    asm volatile("s_nop 4" ::: "memory");
-                    auto next_tile = [&](int q) {      // requests 2q, 2q+1 of this wavefront for tile st+1
-                        if constexpr (SPREAD) {
-                            if (more) {
-                                const int i0 = wave + 2 * q * NW, i1 = i0 + NW;
-                                if (i0 < ninstr) dma_piece(st + 1, (it + 1) & 1, i0);
-                                if (i1 < ninstr) dma_piece(st + 1, (it + 1) & 1, i1);
-                            }
-                        }
-                    };
-                    // (a tile has 2 requests per wavefront for every 8 k-groups)
-                    mma8_bf16_t<0>(acc, ga, wl);
-                    next_tile(0);
-                    if constexpr (NKG >= 16) {
-                        mma8_bf16_t<256>(acc, ga + 8, wl);
-                        next_tile(1);
-                    }
-                    if constexpr (NKG >= 32) {
-                        mma8_bf16_t<512>(acc, ga + 16, wl);
-                        next_tile(2);
-                        mma8_bf16_t<768>(acc, ga + 24, wl);
-                        next_tile(3);
-                    }
-                    asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc)::"memory");
-                } else {
-                    constexpr int kPF = 3;
-                    uint4 bq[kPF + 1];
+                for (int i = 0; i < kPF; i++)
+                    bq[i] = *reinterpret_cast<const uint4 *>(wb + woff[i & 7] + (i >> 3) * 256);
 #pragma unroll
-                    for (int i = 0; i < kPF; i++)
-                        bq[i] = *reinterpret_cast<const uint4 *>(wb + woff[i & 7] + (i >> 3) * 256);
-#pragma unroll
-                    for (int kg = 0; kg < NKG; kg++) {
-                        if (kg + kPF < NKG)
-                            bq[(kg + kPF) % (kPF + 1)] =
-                                *reinterpret_cast<const uint4 *>(wb + woff[(kg + kPF) & 7] + ((kg + kPF) >> 3) * 256);
-                        mma_kgroup<T>(acc, ga[kg], bq[kg % (kPF + 1)]);
-                    }
+                for (int kg = 0; kg < NKG; kg++) {
+                    if (kg + kPF < NKG)
+                        bq[(kg + kPF) % (kPF + 1)] =
+                            *reinterpret_cast<const uint4 *>(wb + woff[(kg + kPF) & 7] + ((kg + kPF) >> 3) * 256);
+                    mma_kgroup<T>(acc, ga[kg], bq[kg % (kPF + 1)]);
                 }
             } else {
                 const int wrow = cb * 32 + (lane & 31);
@@ -688,24 +628,6 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 }
             }
         }
-        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
-        if (direct) {
-            if constexpr (HAND) {
-                const int m = m0 + pb * 32 + (lane & 31);
-                if (m < s.M) {
-                    T *row = gb + (long)m * BKC + cb * 32 + 8 * (lane >> 5);
-                    *reinterpret_cast<uint4 *>(row) =
-                        make_uint4(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
-                                   pack_bf16x2(acc[6], acc[7]));
-                    *reinterpret_cast<uint4 *>(row + 16) =
-                        make_uint4(pack_bf16x2(acc[8], acc[9]), pack_bf16x2(acc[10], acc[11]),
-                                   pack_bf16x2(acc[12], acc[13]), pack_bf16x2(acc[14], acc[15]));
-                }
-                // (one tile buffer: the next transfer must not start before every wavefront has read this tile)
-                if constexpr (!DB) lds_only_barrier();
-            }
-            continue;
-        }
         // grad-column block -> LDS: lanes 0..31 / 32..63 each cover 32 consecutive channels
         const int ch = cb * 32 + (lane & 31);
 #pragma unroll
@@ -715,6 +637,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
         }
         lds_only_barrier();
         // rows out to memory, 16 bytes per thread
+        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
 #pragma unroll
         for (int i = 0; i < ITEMS; i++) {
             const int item = tid + i * kThreads;
@@ -742,7 +665,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
 // matrix instructions.  Against the 128-position / 64-channel shape of tiled_bwd_col_kernel: half the weight
 // traffic per product, and a transfer has three steps to arrive instead of one (the loaded latency of a tile is
 // about a whole step of that kernel, which waited for it at every step).  The product is taken transposed and
-// stored from the registers (see mma8_bf16_t and the `direct` path of tiled_bwd_col_kernel).
+// stored from the registers: the lane's weight row is chosen such that its 16 accumulator registers are two runs
+// of 8 consecutive channels (see mma8_bf16_t).
 constexpr int kColRing = 4, kColAhead = 3;
 template <int NB>   // blocks of 8 k-groups: ogk = 128 NB
 __global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a)
