@@ -389,6 +389,10 @@ def main():
     ap.add_argument("--offset-axes", type=int, default=7,
                     help="mask of the axes the offsets displace along (1 z, 2 y, 4 x): 6 = the Spatial layers, 1 = the "
                          "Temporal layers of the reference (3-D matrix-core workloads only; default all three)")
+    ap.add_argument("--grad-weight-mode", type=int, default=1, choices=[0, 1],
+                    help="matrix-core backward of bfloat16 problems: 1 (default) grad_weight as a matrix product over "
+                         "the sampled columns that the offset / mask gradient kernel writes; 0 the grad-weight kernel "
+                         "samples the input again")
     ap.add_argument("--grad-input-mode", type=int, default=1, choices=[0, 1],
                     help="matrix-core backward: 1 (default) grad-column rows through device memory, offset / mask "
                          "gradient and grad_input (from sample lists) as kernels of their own; 0 everything inside "
@@ -406,6 +410,7 @@ def main():
     from d2conv3d_amd import _lib
     lib = _lib.load()  # raises if the HIP library is missing: there is no fallback
     lib.d2c_set_grad_input_mode(args.grad_input_mode)
+    lib.d2c_set_grad_weight_mode(args.grad_weight_mode)
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     if args.workload == "c2_sizemap":
@@ -621,7 +626,7 @@ def main():
                    "offsets": ("formed in the sampler from the dilation map [N,3,T,H,W] (d2c_conv3d_sized_*)" if sized
                                else "offsets tensor [N,3*K*G,T,H,W]"),
                    "offset_axes": args.offset_axes,
-                   "grad_input_mode": args.grad_input_mode,
+                   "grad_input_mode": args.grad_input_mode, "grad_weight_mode": args.grad_weight_mode,
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "taps_outside_volume": taps,

@@ -22,7 +22,7 @@ EXPORTS = (
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
-    "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_last_error", "d2c_version",
+    "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_set_grad_weight_mode", "d2c_last_error", "d2c_version",
     "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read",
     "d2c_size_map_offsets_forward", "d2c_size_map_offsets_backward",
     "d2c_conv3d_sized_forward_workspace_bytes", "d2c_conv3d_sized_backward_workspace_bytes",
@@ -110,6 +110,7 @@ def load():
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int
     lib.d2c_set_grad_input_mode.argtypes, lib.d2c_set_grad_input_mode.restype = [ctypes.c_int], None
+    lib.d2c_set_grad_weight_mode.argtypes, lib.d2c_set_grad_weight_mode.restype = [ctypes.c_int], None
     psm = ctypes.POINTER(SizeMapDesc)
     lib.d2c_size_map_offsets_forward.argtypes, lib.d2c_size_map_offsets_forward.restype = [psm, vp, vp, vp], ctypes.c_int
     lib.d2c_size_map_offsets_backward.argtypes, lib.d2c_size_map_offsets_backward.restype = [psm, vp, vp, vp, vp], ctypes.c_int

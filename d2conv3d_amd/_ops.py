@@ -513,6 +513,13 @@ def set_algo_override(name):
     _lib.load().d2c_set_algo_override(code)
 
 
+def set_grad_weight_mode(mode):
+    """Test hook for bfloat16 problems on the matrix-core kernels: "columns" (default; grad_weight as a matrix
+    product over the sampled columns that the offset / mask gradient kernel writes) or "resample" (the
+    grad-weight kernel samples the input again)."""
+    _lib.load().d2c_set_grad_weight_mode(mode if isinstance(mode, int) else {"columns": 1, "resample": 0}[mode])
+
+
 def set_grad_input_mode(mode):
     """Test hook: "lists" (default; grad_input gathered from per-voxel sample lists, every element
     written once), "atomics" (scatter with fp32 atomics like the reference), or an int n >= 2: lists of

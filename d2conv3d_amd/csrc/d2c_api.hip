@@ -19,6 +19,7 @@ thread_local char g_err[512] = "";
 std::atomic<uint64_t> g_max_intermediate{1ull << 32};  // dconv3d_gpu.cu:12
 std::atomic<int> g_algo_override{D2C_ALGO_AUTO};
 std::atomic<int> g_gx_mode{1};
+std::atomic<int> g_gw_mode{1};
 
 struct ProfState {
     std::mutex mu;
@@ -63,6 +64,7 @@ int static_scratch(void **out)
 }  // namespace
 
 int d2c_gx_mode() { return g_gx_mode.load(); }
+int d2c_col_weight_mode() { return g_gw_mode.load(); }
 
 void d2c_set_error(const char *fmt, ...)
 {
@@ -150,6 +152,7 @@ uint64_t d2c_get_max_intermediate_elements(void) { return g_max_intermediate.loa
 void d2c_set_max_intermediate_elements(uint64_t m) { g_max_intermediate.store(m); }
 void d2c_set_algo_override(int algo) { g_algo_override.store(algo); }
 void d2c_set_grad_input_mode(int mode) { g_gx_mode.store(mode > 0 ? mode : 0); }
+void d2c_set_grad_weight_mode(int mode) { g_gw_mode.store(mode ? 1 : 0); }
 
 void d2c_profile_enable(int on)
 {

@@ -43,6 +43,8 @@ struct AuxArgs {
     int ntile;           // position tiles
     int nshare;          // tap shares
     SampleLists lists;   // counts != NULL: every live sample is filed in its bucket on the way (for grad_input)
+    void *col;           // COL: the sampled columns [chunk][tap][mpad][BKC] (what the forward pass multiplied with W),
+    long mpad;           //      rows of all `ntile` position tiles (zeros past the last position)
 };
 
 // Sum over the 8 lanes of a position without LDS traffic: neighbours of a quad, the other pair of the quad, then
@@ -59,7 +61,10 @@ D2C_DEV float sum_over_8_lanes(float v)
     return dpp_add<0x141>(v); // row_half_mirror
 }
 
-template <typename T, bool AUX16, bool SIZED>
+// COL: the kernel also writes the sampled, modulated columns alpha * sum_corner a_corner * x[corner, c] of every
+// (position, tap, channel) -- the corner vectors are in its registers anyway -- so that the grad-weight product
+// can run as a plain matrix product over them (tiled_bwd_weight_col_kernel) instead of sampling the input again.
+template <typename T, bool AUX16, bool SIZED, bool COL>
 __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a)
 {
     constexpr int MT = kMT;
@@ -118,6 +123,11 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     };
     if (k_lo < k_hi) coords_issue(k_lo);
 
+    // COL: a column vector is stored one round late, right behind the loads of the next round: those loads are
+    // then older than the store, and the wait for them leaves the store in flight for a whole round
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 pend_v = {0u, 0u, 0u, 0u};
+    u32x4 *pend_p = nullptr;
     for (int k = k_lo; k < k_hi; k++) {
         int lbin = -1, lslot = 0;
         float lhx = 0.f;
@@ -200,10 +210,33 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                     gq[r] = inr ? *reinterpret_cast<const uint4 *>(gcb + ((grow + m) * BKC + ivec * VEC) * (long)sizeof(T))
                                 : make_uint4(0, 0, 0, 0);
                 }
+                if constexpr (COL) {
+                    // (a streaming store: written once, read by another kernel much later; it leaves the rows that
+                    // this kernel gathers in the L2)
+                    if (pend_p) __builtin_nontemporal_store(pend_v, pend_p);
+                }
 #pragma unroll
                 for (int r = 0; r < kRounds; r++) {
                     const int pos = (rp * kRounds + r) * 8 + rpos;
                     const unsigned live = (unsigned)__float_as_int(tab_of(1, pos)) >> 24;
+                    if constexpr (COL) {
+                        // corner weights as in the forward pass (dconv3d_gpu.cu:88-95: wz * wy * wx, then the
+                        // modulation); a point that is not live contributes nothing, corners out of range read zeros
+                        // (the exchange first, with every lane taking part, then the choice)
+                        const float al_pos = tab_of(8, pos);
+                        const float alv = live ? al_pos : 0.f;
+                        const float cz[2] = {tab_of(2, pos), tab_of(5, pos)}, cy[2] = {tab_of(3, pos), tab_of(6, pos)};
+                        const float cx[2] = {tab_of(4, pos), tab_of(7, pos)};
+                        VecAcc<T> va;
+                        va.zero();
+#pragma unroll
+                        for (int c = 0; c < 8; c++)
+                            va.fma(((cz[c >> 2] * cy[(c >> 1) & 1]) * cx[c & 1]) * alv, xv[r][c]);
+                        const uint4 cv = va.pack();
+                        pend_v = u32x4{cv.x, cv.y, cv.z, cv.w};
+                        pend_p = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(a.col)
+                            + ((((long)(c0 / BKC) * s.K + k) * a.mpad + m0 + pos) * BKC + ivec * VEC) * (long)sizeof(T));
+                    }
                     float dot[8];
                     if constexpr (sizeof(T) == 2) {
                         const bf16x2_t g0 = __builtin_bit_cast(bf16x2_t, gq[r].x), g1 = __builtin_bit_cast(bf16x2_t, gq[r].y);
@@ -292,6 +325,9 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
             lists_store(a.lists, lbin, lslot, e);
         }
     }
+    if constexpr (COL) {
+        if (pend_p) __builtin_nontemporal_store(pend_v, pend_p);
+    }
 }
 
 }  // namespace
@@ -300,31 +336,46 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 // channel count is a multiple of the chunk width.
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, const SampleLists *lists, hipStream_t st)
+                        void *goff, void *gmask, const SampleLists *lists, void *col, hipStream_t st)
 {
     const int ntile = (s.M + kMT - 1) / kMT;
     const int nshare = s.K < kTapSplit ? s.K : kTapSplit;
     // (with the size-map source `goff` is the fp32 accumulator of the size gradient)
     AuxArgs a{s, xcl, off, mask, gcol, s.ss.on ? nullptr : goff, gmask, s.ss.on ? (float *)goff : nullptr, ntile, nshare,
-              lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}};
+              lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}, col, (long)ntile * kMT};
     dim3 grid((unsigned)(8 * (((ntile + kWavesPerBlock - 1) / kWavesPerBlock + 7) / 8) * s.G * nshare));
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
     D2cProfScope prof(D2C_PROF_BWD_AUX, st);
     const dim3 blk(64 * kWavesPerBlock);
     if constexpr (sizeof(T) == 2) {
+        // (the sampled columns are written for bfloat16 problems in three dimensions only, see d2c_bwd_weight_from_col)
+        if (col && s.nd == 3) {
+            if (aux16) {
+                if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, true, true, true>), grid, blk, 0, st, a);
+                else hipLaunchKernelGGL((aux_grad_kernel<T, true, false, true>), grid, blk, 0, st, a);
+            } else {
+                if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, false, true, true>), grid, blk, 0, st, a);
+                else hipLaunchKernelGGL((aux_grad_kernel<T, false, false, true>), grid, blk, 0, st, a);
+            }
+            return d2c_check_launch("aux_grad_kernel");
+        }
         if (aux16) {
-            if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, true, true>), grid, blk, 0, st, a);
-            else hipLaunchKernelGGL((aux_grad_kernel<T, true, false>), grid, blk, 0, st, a);
+            if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, true, true, false>), grid, blk, 0, st, a);
+            else hipLaunchKernelGGL((aux_grad_kernel<T, true, false, false>), grid, blk, 0, st, a);
         }
     }
+    if (col && (sizeof(T) != 2 || s.nd != 3)) {
+        d2c_set_error("aux_grad_kernel: sampled columns are written for bfloat16 problems in three dimensions only");
+        return D2C_ERR_LAUNCH;
+    }
     if (!aux16) {
-        if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, false, true>), grid, blk, 0, st, a);
-        else hipLaunchKernelGGL((aux_grad_kernel<T, false, false>), grid, blk, 0, st, a);
+        if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, false, true, false>), grid, blk, 0, st, a);
+        else hipLaunchKernelGGL((aux_grad_kernel<T, false, false, false>), grid, blk, 0, st, a);
     }
     return d2c_check_launch("aux_grad_kernel");
 }
 template int d2c_aux_grad_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                         void *, void *, const SampleLists *, hipStream_t);
+                                         void *, void *, const SampleLists *, void *, hipStream_t);
 template int d2c_aux_grad_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                        void *, void *, const SampleLists *, hipStream_t);
+                                        void *, void *, const SampleLists *, void *, hipStream_t);

@@ -31,12 +31,15 @@ bool d2c_lists_supported(const TiledShape &s);
 int d2c_lists_build(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
 int d2c_lists_fill(const TiledShape &s, const void *off, const void *mask, const SampleLists &L, hipStream_t st);
 int d2c_gx_mode();
+int d2c_col_weight_mode();
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, const SampleLists *lists, hipStream_t st);
+                        void *goff, void *gmask, const SampleLists *lists, void *col, hipStream_t st);
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                                const void *mask, void *goutp, float *gwacc, void *gw, hipStream_t st);
+                                const void *mask, void *goutp, float *gwacc, void *gw, const void *col, hipStream_t st);
+bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype);
+size_t d2c_bwd_col_bytes(const TiledShape &s);
 size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype);
 template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
 template <typename T> int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st);
@@ -490,8 +493,15 @@ bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
     return d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_single_pass(s, q.dtype);
 }
 
+// grad_weight as a matrix product over sampled columns that the offset / mask gradient kernel writes on its way
+// (needs that kernel to run: the caller wants grad_offset or grad_mask)
+bool use_col_weight(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    return d2c_col_weight_mode() && use_aux_kernel(q, s) && d2c_bwd_weight_from_col(s, q.dtype);
+}
+
 struct BwdWs {
-    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, gsacc, sm1, total;
+    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, gsacc, sm1, col, total;
 };
 BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
@@ -528,6 +538,8 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
     w.sm1 = w.total;       // ... and (size - 1) per axis
     if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
+    w.col = w.total;       // sampled columns for the grad-weight product
+    if (use_col_weight(q, s)) w.total += d2c_align_up(d2c_bwd_col_bytes(s));
     return w;
 }
 
@@ -585,6 +597,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         s.ss.on = 2;
         off = sm1;
     }
+    bool gw_from_col = false;
     if (gx || goff || gmask) {
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
@@ -610,9 +623,10 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                                                      auxk ? nullptr : goff, auxk ? nullptr : gmask,
                                                      (float *)(base + l.auxacc), st))
                 return rc;
+            gw_from_col = gw && auxk && use_col_weight(q, s);
             if (auxk)
                 if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff_k, gmask,
-                                                    lists ? &L : nullptr, st))
+                                                    lists ? &L : nullptr, gw_from_col ? base + l.col : nullptr, st))
                     return rc;
             if (s.ss.on && goff) {
                 D2cProfScope prof(D2C_PROF_PACK, st);
@@ -641,7 +655,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
             if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc),
-                                                       gw, st))
+                                                       gw, gw_from_col ? base + l.col : nullptr, st))
                 return rc;
         } else {
             if (int rc = d2c_generic_conv3d_backward(q, gout, x, off, mask, w, nullptr, nullptr, nullptr, gw, nullptr,

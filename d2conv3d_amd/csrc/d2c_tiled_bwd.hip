@@ -1207,6 +1207,196 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     }
 }
 
+// ============================================================ kernel 2b
+// grad_weight as a plain matrix product over the sampled columns that the offset / mask gradient kernel left in
+// device memory (aux_grad_kernel<.., COL>; bfloat16 problems):
+//     gW[o, (chunk, tap, c)] += sum_pos gout[o, pos] * col[chunk][tap][pos][c]
+// One workgroup = one tap and kColChunks channel chunks (128 columns), all output channels of the weight group (8
+// wavefronts x 64 rows), looping over its piece of the 64-position tiles.  No sampling here: the input is not read
+// again, there is no coordinate wavefront and no interpolation.  The column tiles (2 x 8 KiB per step) go through
+// registers into a double-buffered LDS tile (one 16-byte load and one LDS store per lane and tile, requested a step
+// ahead), the grad_out fragments come straight from the fragment-ordered copy, a step ahead as well.  All loads are
+// ordinary ones, so the compiler counts its waits; the barrier waits for LDS operations only.  Twice the columns per
+// grad_out fragment of tiled_bwd_weight_dma_kernel: half the fragment traffic per product.
+constexpr int kColChunks = 2;
+
+struct BwdWeightColArgs {
+    TiledShape s;
+    const void *col;     // [chunk][tap][mpad][64]
+    const void *goutp;   // grad_out in MFMA fragment order, see pack_gout_kernel
+    float *gwacc;        // as in BwdWeightArgs
+    long mpad;           // rows per (chunk, tap) of `col`: whole 64-position tiles
+    int otiles, nmain, main_len, ntail, tail_len;   // as in BwdWeightArgs
+};
+
+__global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeightColArgs a)
+{
+    typedef bf16_t T;
+    constexpr int MT = kWDT, VEC = 8, BKC = 64, NCH = kColChunks, CB = NCH * (BKC / 32), OB = 2, NT = 64 * 8;
+    constexpr int TRS = MT * (int)sizeof(T) + 16;   // tile row stride: [position][channel]
+    constexpr int NKG = MT / (2 * VEC);        // k-groups per iteration
+    constexpr int NKGP = kWMT / (2 * VEC);     // k-groups per tile of the packed grad_out copy
+    static_assert(MT * 8 == kThreads, "one (position, vector) item per thread and column tile");
+    __shared__ __align__(16) unsigned char s_tile[2 * NCH * MT * TRS];
+
+    const TiledShape &s = a.s;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ntile = (s.M + MT - 1) / MT;
+    const int npair = s.nchunk / NCH;
+    const int nstep = npair * s.K;
+    const int nitem = s.groups * a.otiles * nstep;
+    int item, t_lo, nmy, t_step;
+    if ((int)blockIdx.x < nitem * a.nmain) {
+        item = blockIdx.x % nitem;
+        t_lo = blockIdx.x / nitem;
+        t_step = a.nmain;
+        const int nt = min(ntile, a.nmain * a.main_len);
+        nmy = nt > t_lo ? (nt - t_lo + t_step - 1) / t_step : 0;
+    } else {
+        const int id = blockIdx.x - nitem * a.nmain;
+        item = id % nitem;
+        t_lo = a.nmain * a.main_len + id / nitem;
+        t_step = a.ntail;
+        nmy = ntile > t_lo ? (ntile - t_lo + t_step - 1) / t_step : 0;
+    }
+    if (nmy <= 0) return;
+    const int st = item % nstep, otile = (item / nstep) % a.otiles, wg = item / (nstep * a.otiles);
+    const int jp = st / s.K, k = st - jp * s.K;
+    const int o_base = otile * NT + wave * 64;
+    const bool mma_wave = o_base < s.og;
+
+    f32x16 acc[OB][CB];
+#pragma unroll
+    for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[ob][cb][r] = 0.f;
+
+    // --- column tiles: thread = (position, 16-byte vector) of each of the two tiles
+    static_assert(NCH == 2, "the two tiles of a step are named variables below");
+    const int ipos = tid >> 3, ivec = tid & 7;
+    const long chunk0 = (long)wg * s.nchunk + jp * NCH;
+    const uint4 *const colp0 = reinterpret_cast<const uint4 *>(a.col) + ((chunk0 * s.K + k) * a.mpad + ipos) * (BKC / VEC) + ivec;
+    const uint4 *const colp1 = colp0 + (long)s.K * a.mpad * (BKC / VEC);
+    // (past the end of the piece the last tile is requested again: the same loads in every iteration, no branches
+    // around them, so that the values stay in registers and the compiler's waits count)
+    // column tiles in flight: the odd tile (crO) and the even tile (crE) after the one on the matrix cores; a pair of
+    // registers is refilled, for the tile three steps on, as soon as it has been written to LDS: two whole steps for
+    // a tile to arrive from device memory
+    uint4 crO0, crO1, crE0, crE1;
+    auto col_row0 = [&](int i) { return (long)(t_lo + min(i, nmy - 1) * t_step) * MT * (BKC / VEC); };
+    unsigned char *const st_p = s_tile + ipos * TRS + ivec * 16;
+
+    // --- gW block += gout[o, pos] * tile[pos, c]; gout fragments straight from the packed copy
+    const int OBT = (s.og + 63) / 64 * 2;
+    const int ntp = (s.M + kWMT - 1) / kWMT;     // tiles of the packed copy (kWMT positions each)
+    // (a wavefront without output channels reads the first one's fragments in the prologue, and none after that)
+    const uint4 *gp4 = reinterpret_cast<const uint4 *>(a.goutp) + (((long)wg * ntp * OBT + (mma_wave ? o_base >> 5 : 0)) * NKGP) * 64 + lane;
+    auto gfrag_p = [&](int i) {     // fragment (k-group 0, row block 0) of tile i of this piece
+        const long t64 = t_lo + (long)min(i, nmy - 1) * t_step;
+        const long tp = t64 / (kWMT / MT);
+        const int kgp = (int)(t64 % (kWMT / MT)) * NKG;
+        return gp4 + ((tp * OBT) * NKGP + kgp) * 64;
+    };
+    // the fragments of two tiles in flight (even / odd iterations); a slot is refilled, for the tile after next, as
+    // soon as the matrix cores have taken it: two whole steps for a fragment to arrive
+    uint4 ldA[2 * NKG], ldB[2 * NKG];
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    const int l16 = lane & 15, g16 = lane >> 4;
+    // this lane's part of the transposing reads: position (g16 >> 1) * 8 + (l16 >> 2), channel (g16 & 1) * 16 + (l16 & 3) * 4
+    const unsigned char *const rd_p = s_tile + ((g16 >> 1) * 8 + (l16 >> 2)) * TRS + ((g16 & 1) * 16 + (l16 & 3) * 4) * 2;
+
+    {
+        const uint4 *g0 = gfrag_p(0), *g1 = gfrag_p(1);
+#pragma unroll
+        for (int kg = 0; kg < NKG; kg++)
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++) ldA[kg * 2 + ob] = g0[(ob * NKGP + kg) * 64];
+#pragma unroll
+        for (int kg = 0; kg < NKG; kg++)
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++) ldB[kg * 2 + ob] = g1[(ob * NKGP + kg) * 64];
+        const long r0 = col_row0(0), r1 = col_row0(1), r2 = col_row0(2);
+        crE0 = colp0[r0];
+        crE1 = colp1[r0];
+        crO0 = colp0[r1];
+        crO1 = colp1[r1];
+        *reinterpret_cast<uint4 *>(st_p) = crE0;
+        *reinterpret_cast<uint4 *>(st_p + MT * TRS) = crE1;
+        crE0 = colp0[r2];
+        crE1 = colp1[r2];
+    }
+    lds_only_barrier();
+    // Wavefronts without output channels (weight groups of fewer than 512) only move the column tiles.  Each role has
+    // a loop of its own: a wait that served both would have to assume the fewer loads in flight.
+    auto run = [&](auto mma_c) {
+        constexpr bool MMA = decltype(mma_c)::value;
+        auto step = [&](int it, uint4(&ld)[2 * NKG], uint4 &cr0, uint4 &cr1) {
+            const int dbuf = it & 1;
+            if constexpr (MMA) {
+                const uint4 *gn = gfrag_p(it + 2);
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    uint4 bf[CB];
+                    // ds_read_b64_tr_b16, as in tiled_bwd_weight_dma_kernel: two loads make the 8 positions of an
+                    // operand vector
+#pragma unroll
+                    for (int cb = 0; cb < CB; cb++) {
+                        const unsigned char *ap = rd_p + ((dbuf * NCH + (cb >> 1)) * MT + kg * 16) * TRS + (cb & 1) * 64;
+                        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)ap);
+                        const v4s hi =
+                            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(ap + 4 * TRS));
+                        const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+                        bf[cb] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+                    }
+#pragma unroll
+                    for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+                        for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], ld[kg * 2 + ob], bf[cb]);
+#pragma unroll
+                    for (int ob = 0; ob < OB; ob++) ld[kg * 2 + ob] = gn[(ob * NKGP + kg) * 64];
+                    // (the requests stay behind the matrix instructions of their k-group)
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            // (the other buffer was last read in the iteration before, which every wavefront has left)
+            *reinterpret_cast<uint4 *>(st_p + ((dbuf ^ 1) * NCH * MT) * TRS) = cr0;
+            *reinterpret_cast<uint4 *>(st_p + ((dbuf ^ 1) * NCH + 1) * MT * TRS) = cr1;
+            const long r3 = col_row0(it + 3);
+            cr0 = colp0[r3];
+            cr1 = colp1[r3];
+            lds_only_barrier();
+        };
+        // pairs of steps, then the odd one out: no branch inside the loop (see above)
+        int it = 0;
+        for (; it + 1 < nmy; it += 2) {
+            step(it, ldA, crO0, crO1);
+            step(it + 1, ldB, crE0, crE1);
+        }
+        if (it < nmy) step(it, ldA, crO0, crO1);
+    };
+    if (mma_wave) run(std::true_type{});
+    else run(std::false_type{});
+
+    if (mma_wave) {
+#pragma unroll
+        for (int ob = 0; ob < OB; ob++)
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) {
+                const int stw = (jp * NCH + (cb >> 1)) * s.K + k;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int ol = o_base + ob * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (ol < s.og)
+                        atomicAdd(a.gwacc + (((long)wg * s.nchunk * s.K + stw) * s.og + ol) * BKC + (cb & 1) * 32 + (lane & 31),
+                                  acc[ob][cb][r]);
+                }
+            }
+    }
+}
+
 template <typename T, int NC> constexpr size_t bwd_weight_dma_lds()
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
@@ -1629,9 +1819,22 @@ static GwPieces gw_pieces(long items, int ntile, int ncu)
     return r;
 }
 
+// grad_weight from the sampled columns (tiled_bwd_weight_col_kernel): bfloat16 problems in three dimensions whose
+// weight groups hold whole sets of kColChunks channel chunks.
+bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype)
+{
+    return dtype == D2C_BF16 && s.nd == 3 && s.nchunk % kColChunks == 0;
+}
+// bytes of the sampled columns [chunk][tap][whole 64-position tiles][64]
+size_t d2c_bwd_col_bytes(const TiledShape &s)
+{
+    const long ntile = (s.M + kWDT - 1) / kWDT;
+    return (size_t)(s.Cin / 64) * s.K * ntile * kWDT * 64 * 2;
+}
+
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                                const void *mask, void *goutp, float *gwacc, void *gw, hipStream_t st)
+                                const void *mask, void *goutp, float *gwacc, void *gw, const void *col, hipStream_t st)
 {
     const long nw = (long)s.Cout * s.cg * s.K;
     const int steps = s.nchunk * s.K;
@@ -1655,12 +1858,20 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     // first.
     const int ncu = d2c_num_cus();
     if (ncu <= 0) return D2C_ERR_LAUNCH;
-    const long items = (long)steps * otiles * s.groups;
+    bool from_col = false;
+    if constexpr (sizeof(T) == 2) from_col = col != nullptr;
+    const long items = (long)(from_col ? steps / kColChunks : steps) * otiles * s.groups;
     const GwPieces pc = gw_pieces(items, ntile, ncu);
     const int nmain = pc.nmain, main_len = pc.main_len, ntail = pc.ntail, tail_len = pc.tail_len;
+    if (from_col) {
+        BwdWeightColArgs c{s, col, goutp, gwacc, (long)ntile * kWDT, otiles, nmain, main_len, ntail, tail_len};
+        D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
+        hipLaunchKernelGGL(tiled_bwd_weight_col_kernel, dim3((unsigned)(items * (nmain + ntail))), dim3(kThreads), 0, st, c);
+        if (int rc = d2c_check_launch("tiled_bwd_weight_col_kernel")) return rc;
+    }
     BwdWeightDmaArgs a{{s, gout, xcl, off, mask, goutp, gwacc, otiles, nmain, main_len, ntail, tail_len},
                        (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T))};
-    {
+    if (!from_col) {
         const dim3 grid((unsigned)(items * (nmain + ntail)));
         bool aux16 = false;
         if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
@@ -1736,7 +1947,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
                                               const void *, const void *, void *, float *, void *, void *, void *, \
                                               float *, hipStream_t);                                                        \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
-                                                const void *, void *, float *, void *, hipStream_t);              \
+                                                const void *, void *, float *, void *, const void *, hipStream_t); \
     template int d2c_tiled_unpack_gx<T>(const TiledShape &, const float *, void *, hipStream_t);                   \
     template int d2c_tiled_bias_grad<T>(const TiledShape &, const void *, void *, hipStream_t);
 INST(bf16_t)

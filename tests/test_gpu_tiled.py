@@ -36,6 +36,10 @@ SHAPES = {
     # whole round, the rest cut into step ranges), two weight groups with few position tiles (all items cut)
     "c64_o1100_big": (1, 64, 1100, (7, 35, 35), 3, 1, 1, 1, 1, 1, True, True, 1.5),
     "c128_groups2_o1280_mid": (1, 128, 1280, (5, 41, 41), (1, 3, 3), 1, (0, 1, 1), 1, 2, 2, True, True, 1.0),
+    # weight groups of two and four channel chunks (bfloat16: grad_weight as a matrix product over the sampled
+    # columns, two chunks per workgroup), ragged last position tile, all 512 / some of the output channels of a pass
+    "c256_G2_o512_tail": (1, 256, 512, (3, 7, 7), 3, 1, 1, 1, 1, 2, True, True, 1.5),
+    "c256_groups2_G4_o384": (2, 256, 384, (3, 5, 6), 3, 1, 1, 1, 2, 4, False, False, 1.5),
     # channel-separated (groups == Cin == Cout)
     "dw64": (2, 64, 64, (4, 6, 7), 3, 1, 1, 1, 64, 1, True, True, 1.5),
     "dw96_G3_nomask": (1, 96, 96, (3, 5, 9), 3, 1, 1, 1, 96, 3, False, False, 1.0),
@@ -95,6 +99,38 @@ def test_tiled_forward_backward(name, dtype, dev):
                 assert t.grad.dtype == t.dtype
                 assert rel_l2(t.grad, e) < 2e-2, (n, rel_l2(t.grad, e))
                 assert_close(t.grad, e, 2e-2, 2e-2 * e.abs().max().item(), n)
+
+
+@pytest.mark.parametrize("name", ["c128_G2_o96", "c256_G2_o512_tail", "c256_groups2_G4_o384"])
+@pytest.mark.parametrize("wanted", ["all", "w+offset", "w"])
+def test_grad_weight_from_columns_matches_resampling(name, wanted, dev):
+    # bfloat16 grad_weight two ways: as a matrix product over the sampled columns that the offset / mask gradient
+    # kernel writes on its way (when that kernel runs: grad_offset or grad_mask wanted), or by sampling the input
+    # again in the grad-weight kernel; both against the oracle
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, torch.bfloat16, seed=5)
+    eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+    got = {}
+    for mode in ("columns", "resample"):
+        _ops.set_grad_weight_mode(mode)
+        try:
+            ts = [t.to(dev) if t is not None else None for t in (x, off, m, w, b)]
+            ts[3].requires_grad_(True)
+            if wanted != "w":
+                ts[1].requires_grad_(True)
+            if wanted == "all":
+                ts[0].requires_grad_(True)
+                if ts[2] is not None:
+                    ts[2].requires_grad_(True)
+            d2c.deform_conv3d(*ts, s, p, d, groups, G).backward(gout.to(dev))
+            got[mode] = ts[3].grad
+        finally:
+            _ops.set_grad_weight_mode("columns")
+        assert rel_l2(got[mode], eg[3]) < 2e-2, (mode, rel_l2(got[mode], eg[3]))
+        assert_close(got[mode], eg[3], 2e-2, 2e-2 * eg[3].abs().max().item(), f"grad_weight ({mode})")
+        if wanted != "w":
+            assert rel_l2(ts[1].grad, eg[1]) < 2e-2, mode
+    # the two differ by the rounding of the columns to bfloat16 at most (both round them before the product)
+    assert rel_l2(got["columns"], got["resample"].float().cpu()) < 1e-2
 
 
 @pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail", "dw64", "dw96_G3_nomask",
