@@ -574,10 +574,14 @@ def main():
         for d in dims:
             P *= d
         if dom == "aux_grad_kernel":
-            # the corner rows it gathers (8 per sample and chunk), the grad-column rows and the offset / mask
-            # tensors in and out, once each
+            # every tensor it has to move once: the grad-column rows in, the sampled columns out (bfloat16 problems
+            # whose grad_weight runs over them), the input, offsets and modulation in, their gradients out, one list
+            # entry (16 / 32 B) per sample
             K = 3 ** nd
-            nbytes = N * P * K * C * es * 9 + 2 * N * P * K * G * (nd + 1) * es
+            rows = N * P * K * C * es
+            cols = rows if (dt == "bf16" and nd == 3 and args.grad_weight_mode == 1 and (C // groups) % 128 == 0) else 0
+            aux = N * P * K * G * (nd + 1) * (2 if dt == "bf16" else 4)
+            nbytes = rows + cols + N * P * C * es + 2 * aux + N * P * K * G * (16 if dt == "bf16" else 32)
             bound, ach = "hbm", nbytes / t_dom / 1e9
         elif dom == "gx_owner_kernel":
             # every grad-column row (N*P*K*Cin elements), every list entry (32 B per sample) and every

@@ -1233,7 +1233,9 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
 {
     typedef bf16_t T;
     constexpr int MT = kWDT, VEC = 8, BKC = 64, NCH = kColChunks, CB = NCH * (BKC / 32), OB = 2, NT = 64 * 8;
-    constexpr int TRS = MT * (int)sizeof(T) + 16;   // tile row stride: [position][channel]
+    // tile row stride ([position][channel]): 64 bytes more than a row, so that the 64-byte segments of four consecutive
+    // rows, which 32 lanes of a transposing read fetch together, fall into different quarters of the 64 banks
+    constexpr int TRS = MT * (int)sizeof(T) + 64;
     constexpr int NKG = MT / (2 * VEC);        // k-groups per iteration
     constexpr int NKGP = kWMT / (2 * VEC);     // k-groups per tile of the packed grad_out copy
     static_assert(MT * 8 == kThreads, "one (position, vector) item per thread and column tile");
@@ -1765,11 +1767,11 @@ constexpr int kGwPieceCost = 10;     // what a workgroup costs beside its tiles 
 struct GwPieces {
     int nmain, main_len, ntail, tail_len;
 };
-static GwPieces gw_pieces(long items, int ntile, int ncu)
+static GwPieces gw_pieces(long items, int ntile, int ncu, int max_main = 1)
 {
     static std::mutex mu;
-    static std::map<std::tuple<long, int, int>, GwPieces> memo;
-    const auto key = std::make_tuple(items, ntile, ncu);
+    static std::map<std::tuple<long, int, int, int>, GwPieces> memo;
+    const auto key = std::make_tuple(items, ntile, ncu, max_main);
     {
         std::lock_guard<std::mutex> lock(mu);
         const auto it = memo.find(key);
@@ -1806,12 +1808,15 @@ static GwPieces gw_pieces(long items, int ntile, int ncu)
     // 8 % ahead of the deal to 7 on paper, 5 % faster; with two main pieces per item, at 108 items x 405 and
     // 108 x 3240 tiles, 9 % and 1 % ahead on paper, 9 % and 25 % slower: the workgroups of an item drift apart and
     // share less in L2.)
+    // (tiled_bwd_weight_col_kernel, which gathers nothing, takes up to `max_main` main pieces per item: fewer pieces
+    // than the round-robin deal needs for the same balance, and every piece ends in fp32 atomics of its whole block)
     const long ideal = (items * (ntile + kGwPieceCost) + ncu - 1) / ncu;
-    if (2 * ideal > ntile && ideal < ntile) {
-        for (int ml = (int)(ideal - ideal / 8); ml <= (int)(ideal + ideal / 8) && ml < ntile; ml += 1 + (int)ideal / 64) {
-            if (2 * ml <= ntile) continue;
-            const int rest = ntile - ml;
-            for (int f = 1; f <= 4; f++) consider(1, ml, f, (rest + f - 1) / f, 0);
+    for (int nm = 1; nm <= max_main; nm++) {
+        if (!((nm + 1) * ideal > ntile && nm * ideal < ntile)) continue;
+        for (int ml = (int)(ideal - ideal / 8); ml <= (int)(ideal + ideal / 8) && nm * ml < ntile; ml += 1 + (int)ideal / 64) {
+            if ((nm + 1) * ml <= ntile) continue;
+            const int rest = ntile - nm * ml;
+            for (int f = 1; f <= 4; f++) consider(nm, ml, f, (rest + f - 1) / f, 0);
         }
     }
     std::lock_guard<std::mutex> lock(mu);
@@ -1861,7 +1866,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     bool from_col = false;
     if constexpr (sizeof(T) == 2) from_col = col != nullptr;
     const long items = (long)(from_col ? steps / kColChunks : steps) * otiles * s.groups;
-    const GwPieces pc = gw_pieces(items, ntile, ncu);
+    const GwPieces pc = gw_pieces(items, ntile, ncu, from_col ? 4 : 1);
     const int nmain = pc.nmain, main_len = pc.main_len, ntail = pc.ntail, tail_len = pc.tail_len;
     if (from_col) {
         BwdWeightColArgs c{s, col, goutp, gwacc, (long)ntile * kWDT, otiles, nmain, main_len, ntail, tail_len};
