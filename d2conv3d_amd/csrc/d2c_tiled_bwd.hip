@@ -16,7 +16,11 @@
 //     gmask          = sum_corner a_corner * dot[corner]             (:837-839)
 //     goff_axis      = alpha * sum_corner (d a_corner / d axis) * dot[corner]   (:708-754, :848-858)
 //
-// Kernel 2 (tiled_bwd_weight_dma_kernel), per workgroup one (tap, channel chunk)
+// Kernel 2b (tiled_bwd_weight_col_kernel; bfloat16 problems whose offset / mask gradient kernel runs): grad_weight as
+// a plain matrix product over the sampled columns which that kernel writes on its way -- the backward pass samples
+// the input once.
+//
+// Kernel 2 (tiled_bwd_weight_dma_kernel; everything else), per workgroup one (tap, channel chunk)
 // and all output channels, looping over position tiles:
 //     gW[o, c, k] += sum_pos gout[o, pos] * alpha * trilinear(x[c], pos)       (:1037-1088)
 //   The reduction runs over positions, so the MFMA operand wants 8 consecutive
