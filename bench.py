@@ -389,9 +389,10 @@ def main():
     ap.add_argument("--offset-axes", type=int, default=7,
                     help="mask of the axes the offsets displace along (1 z, 2 y, 4 x): 6 = the Spatial layers, 1 = the "
                          "Temporal layers of the reference (3-D matrix-core workloads only; default all three)")
-    ap.add_argument("--grad-weight-mode", type=int, default=1, choices=[0, 1],
+    ap.add_argument("--grad-weight-mode", type=int, default=1, choices=[0, 1, 2],
                     help="matrix-core backward of bfloat16 problems: 1 (default) grad_weight as a matrix product over "
-                         "the sampled columns that the offset / mask gradient kernel writes; 0 the grad-weight kernel "
+                         "the sampled columns that the offset / mask gradient kernel writes; 2 the same with the columns "
+                         "written over the grad-column rows (no buffer of their own); 0 the grad-weight kernel "
                          "samples the input again")
     ap.add_argument("--grad-input-mode", type=int, default=1, choices=[0, 1],
                     help="matrix-core backward: 1 (default) grad-column rows through device memory, offset / mask "
@@ -579,7 +580,7 @@ def main():
             # entry (16 / 32 B) per sample
             K = 3 ** nd
             rows = N * P * K * C * es
-            cols = rows if (dt == "bf16" and nd == 3 and args.grad_weight_mode == 1 and (C // groups) % 128 == 0) else 0
+            cols = rows if (dt == "bf16" and nd == 3 and args.grad_weight_mode >= 1 and (C // groups) % 128 == 0) else 0
             aux = N * P * K * G * (nd + 1) * (2 if dt == "bf16" else 4)
             nbytes = rows + cols + N * P * C * es + 2 * aux + N * P * K * G * (16 if dt == "bf16" else 32)
             bound, ach = "hbm", nbytes / t_dom / 1e9

@@ -152,7 +152,7 @@ uint64_t d2c_get_max_intermediate_elements(void) { return g_max_intermediate.loa
 void d2c_set_max_intermediate_elements(uint64_t m) { g_max_intermediate.store(m); }
 void d2c_set_algo_override(int algo) { g_algo_override.store(algo); }
 void d2c_set_grad_input_mode(int mode) { g_gx_mode.store(mode > 0 ? mode : 0); }
-void d2c_set_grad_weight_mode(int mode) { g_gw_mode.store(mode ? 1 : 0); }
+void d2c_set_grad_weight_mode(int mode) { g_gw_mode.store(mode < 0 ? 0 : (mode > 2 ? 2 : mode)); }
 
 void d2c_profile_enable(int on)
 {

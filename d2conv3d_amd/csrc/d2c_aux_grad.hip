@@ -44,7 +44,8 @@ struct AuxArgs {
     int nshare;          // tap shares
     SampleLists lists;   // counts != NULL: every live sample is filed in its bucket on the way (for grad_input)
     void *col;           // COL: the sampled columns [chunk][tap][mpad][BKC] (what the forward pass multiplied with W),
-    long mpad;           //      rows of all `ntile` position tiles (zeros past the last position)
+    long mpad;           //      rows of all `ntile` position tiles (zeros past the last position); or, in place of the
+                         //      grad-column rows (`col` == `gcol`, which nobody reads after this kernel then): N*P rows
 };
 
 // Sum over the 8 lanes of a position without LDS traffic: neighbours of a quad, the other pair of the quad, then
@@ -234,8 +235,10 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                             va.fma(((cz[c >> 2] * cy[(c >> 1) & 1]) * cx[c & 1]) * alv, xv[r][c]);
                         const uint4 cv = va.pack();
                         pend_v = u32x4{cv.x, cv.y, cv.z, cv.w};
-                        pend_p = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(a.col)
-                            + ((((long)(c0 / BKC) * s.K + k) * a.mpad + m0 + pos) * BKC + ivec * VEC) * (long)sizeof(T));
+                        pend_p = m0 + pos < a.mpad
+                                     ? reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(a.col)
+                                           + ((((long)(c0 / BKC) * s.K + k) * a.mpad + m0 + pos) * BKC + ivec * VEC) * (long)sizeof(T))
+                                     : nullptr;
                     }
                     float dot[8];
                     if constexpr (sizeof(T) == 2) {
@@ -336,13 +339,13 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 // channel count is a multiple of the chunk width.
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, const SampleLists *lists, void *col, hipStream_t st)
+                        void *goff, void *gmask, const SampleLists *lists, void *col, bool col_in_place, hipStream_t st)
 {
     const int ntile = (s.M + kMT - 1) / kMT;
     const int nshare = s.K < kTapSplit ? s.K : kTapSplit;
     // (with the size-map source `goff` is the fp32 accumulator of the size gradient)
     AuxArgs a{s, xcl, off, mask, gcol, s.ss.on ? nullptr : goff, gmask, s.ss.on ? (float *)goff : nullptr, ntile, nshare,
-              lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}, col, (long)ntile * kMT};
+              lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}, col, col_in_place ? (long)s.M : (long)ntile * kMT};
     dim3 grid((unsigned)(8 * (((ntile + kWavesPerBlock - 1) / kWavesPerBlock + 7) / 8) * s.G * nshare));
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
@@ -376,6 +379,6 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     return d2c_check_launch("aux_grad_kernel");
 }
 template int d2c_aux_grad_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                         void *, void *, const SampleLists *, void *, hipStream_t);
+                                         void *, void *, const SampleLists *, void *, bool, hipStream_t);
 template int d2c_aux_grad_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                        void *, void *, const SampleLists *, void *, hipStream_t);
+                                        void *, void *, const SampleLists *, void *, bool, hipStream_t);

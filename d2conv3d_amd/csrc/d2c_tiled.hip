@@ -34,10 +34,11 @@ int d2c_gx_mode();
 int d2c_col_weight_mode();
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, const SampleLists *lists, void *col, hipStream_t st);
+                        void *goff, void *gmask, const SampleLists *lists, void *col, bool col_in_place, hipStream_t st);
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                                const void *mask, void *goutp, float *gwacc, void *gw, const void *col, hipStream_t st);
+                                const void *mask, void *goutp, float *gwacc, void *gw, const void *col, long col_rows,
+                                hipStream_t st);
 bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype);
 size_t d2c_bwd_col_bytes(const TiledShape &s);
 size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype);
@@ -499,6 +500,9 @@ bool use_col_weight(const d2c_conv3d_desc &q, const TiledShape &s)
 {
     return d2c_col_weight_mode() && use_aux_kernel(q, s) && d2c_bwd_weight_from_col(s, q.dtype);
 }
+// ... written over the grad-column rows (mode 2): grad_input is taken from those rows first, from sample lists
+// that a pass of their own files
+bool col_in_place(const d2c_conv3d_desc &q, const TiledShape &s) { return d2c_col_weight_mode() == 2 && use_col_weight(q, s); }
 
 struct BwdWs {
     size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, gsacc, sm1, col, total;
@@ -523,7 +527,9 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.gcol = w.counts = w.entries = w.ovf = 0;
     if (use_lists(q, s) || use_aux_kernel(q, s)) {
         w.gcol = w.total;
-        w.total = w.gcol + d2c_align_up((size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M * bkc_of(q.dtype) * es);
+        // (+ 64 rows behind the last one: what the last tile of the grad-weight product reads when the columns took
+        // the rows' place)
+        w.total = w.gcol + d2c_align_up(((size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M + 64) * bkc_of(q.dtype) * es);
     }
     if (use_lists(q, s)) {
         size_t c, en, ov;
@@ -539,7 +545,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.sm1 = w.total;       // ... and (size - 1) per axis
     if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
     w.col = w.total;       // sampled columns for the grad-weight product
-    if (use_col_weight(q, s)) w.total += d2c_align_up(d2c_bwd_col_bytes(s));
+    if (use_col_weight(q, s) && !col_in_place(q, s)) w.total += d2c_align_up(d2c_bwd_col_bytes(s));
     return w;
 }
 
@@ -597,7 +603,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         s.ss.on = 2;
         off = sm1;
     }
-    bool gw_from_col = false;
+    bool gw_from_col = false, gw_in_place = false;
     if (gx || goff || gmask) {
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
@@ -613,20 +619,32 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                 D2cProfScope prof(D2C_PROF_PACK, st);
                 d2c_fill_zero(goff_k, (size_t)s.N * 3 * s.P * sizeof(float), st);
             }
+            gw_from_col = gw && auxk && use_col_weight(q, s);
+            // (the sampled columns over the grad-column rows: grad_input has to be done with the rows before the
+            // offset / mask gradient kernel runs, so the samples are filed by a pass of their own)
+            gw_in_place = gw_from_col && col_in_place(q, s);
             SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
             if (lists) {
                 L = d2c_lists_make(s, Elem<T>::DT, base + l.counts, base + l.entries, base + l.ovf);
-                if (int rc = auxk ? d2c_lists_clear(L, st) : d2c_lists_build(s, off, mask, L, st)) return rc;
+                if (int rc = (auxk && !gw_in_place) ? d2c_lists_clear(L, st) : d2c_lists_build(s, off, mask, L, st)) return rc;
             }
             if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt,
                                                      lists ? nullptr : gxcl, (lists || auxk) ? base + l.gcol : nullptr,
                                                      auxk ? nullptr : goff, auxk ? nullptr : gmask,
                                                      (float *)(base + l.auxacc), st))
                 return rc;
-            gw_from_col = gw && auxk && use_col_weight(q, s);
+            if (lists && gw_in_place)
+                if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, L, gxcl, st)) return rc;
+            if (gw_in_place) {
+                D2cProfScope prof(D2C_PROF_PACK, st);
+                d2c_fill_zero(base + l.gcol + (size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M * bkc_of(q.dtype) * sizeof(T),
+                              (size_t)64 * bkc_of(q.dtype) * sizeof(T), st);
+            }
             if (auxk)
                 if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff_k, gmask,
-                                                    lists ? &L : nullptr, gw_from_col ? base + l.col : nullptr, st))
+                                                    (lists && !gw_in_place) ? &L : nullptr,
+                                                    gw_from_col ? (gw_in_place ? base + l.gcol : base + l.col) : nullptr,
+                                                    gw_in_place, st))
                     return rc;
             if (s.ss.on && goff) {
                 D2cProfScope prof(D2C_PROF_PACK, st);
@@ -640,7 +658,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                                        (const float *)goff_k, size_raw, goff);
                 if (int rc = d2c_check_launch("size_grad_finish_kernel")) return rc;
             }
-            if (lists)
+            if (lists && !gw_in_place)
                 if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, L, gxcl, st)) return rc;
             if (gx)
                 if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
@@ -655,7 +673,8 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
             if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc),
-                                                       gw, gw_from_col ? base + l.col : nullptr, st))
+                                                       gw, gw_from_col ? (gw_in_place ? base + l.gcol : base + l.col) : nullptr,
+                                                       gw_in_place ? (long)s.M : (long)((s.M + 63) / 64) * 64, st))
                 return rc;
         } else {
             if (int rc = d2c_generic_conv3d_backward(q, gout, x, off, mask, w, nullptr, nullptr, nullptr, gw, nullptr,

@@ -1229,7 +1229,9 @@ struct BwdWeightColArgs {
     const void *col;     // [chunk][tap][mpad][64]
     const void *goutp;   // grad_out in MFMA fragment order, see pack_gout_kernel
     float *gwacc;        // as in BwdWeightArgs
-    long mpad;           // rows per (chunk, tap) of `col`: whole 64-position tiles
+    long mpad;           // rows per (chunk, tap) of `col`: whole 64-position tiles, or N*P when the columns took the place
+                         // of the grad-column rows (the last tile then reads into the next block, or the zeroed pad
+                         // behind the last one: finite values that meet the zero tail of the grad_out copy)
     int otiles, nmain, main_len, ntail, tail_len;   // as in BwdWeightArgs
 };
 
@@ -1843,7 +1845,8 @@ size_t d2c_bwd_col_bytes(const TiledShape &s)
 
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
-                                const void *mask, void *goutp, float *gwacc, void *gw, const void *col, hipStream_t st)
+                                const void *mask, void *goutp, float *gwacc, void *gw, const void *col, long col_rows,
+                                hipStream_t st)
 {
     const long nw = (long)s.Cout * s.cg * s.K;
     const int steps = s.nchunk * s.K;
@@ -1873,7 +1876,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     const GwPieces pc = gw_pieces(items, ntile, ncu, from_col ? 4 : 1);
     const int nmain = pc.nmain, main_len = pc.main_len, ntail = pc.ntail, tail_len = pc.tail_len;
     if (from_col) {
-        BwdWeightColArgs c{s, col, goutp, gwacc, (long)ntile * kWDT, otiles, nmain, main_len, ntail, tail_len};
+        BwdWeightColArgs c{s, col, goutp, gwacc, col_rows, otiles, nmain, main_len, ntail, tail_len};
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
         hipLaunchKernelGGL(tiled_bwd_weight_col_kernel, dim3((unsigned)(items * (nmain + ntail))), dim3(kThreads), 0, st, c);
         if (int rc = d2c_check_launch("tiled_bwd_weight_col_kernel")) return rc;
@@ -1956,7 +1959,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
                                               const void *, const void *, void *, float *, void *, void *, void *, \
                                               float *, hipStream_t);                                                        \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
-                                                const void *, void *, float *, void *, const void *, hipStream_t); \
+                                                const void *, void *, float *, void *, const void *, long, hipStream_t); \
     template int d2c_tiled_unpack_gx<T>(const TiledShape &, const float *, void *, hipStream_t);                   \
     template int d2c_tiled_bias_grad<T>(const TiledShape &, const void *, void *, hipStream_t);
 INST(bf16_t)

@@ -312,14 +312,17 @@ int d2c_dwconv3d_backward(const d2c_dwconv3d_desc *desc, const void *grad_out, c
  * One setting per process, for tests only (see d2c_set_algo_override). */
 void d2c_set_grad_input_mode(int mode);
 
-/* Test hook for the matrix-core backward pass of bfloat16 problems: 1 (default)
+/* Hook for the matrix-core backward pass of bfloat16 problems: 1 (default)
  * lets the offset / mask gradient kernel write the sampled columns, over which
  * grad_weight then runs as a plain matrix product (the reference's formulation,
  * dconv3d_gpu.cu:1037-1088, with the column buffer filled by the kernel that has
- * the corner values in registers anyway); 0 makes the grad-weight kernel sample
- * the input again, which is also what happens whenever the caller wants neither
- * grad_offset nor grad_mask.  Workspace sizes depend on the mode.  One setting
- * per process, for tests only (see d2c_set_algo_override). */
+ * the corner values in registers anyway); 2 is the same with the columns written
+ * over the grad-column rows (no buffer of their own: the workspace of mode 0;
+ * grad_input is then taken from the rows first, from sample lists that a pass
+ * of their own files, which costs part of the gain); 0 makes the grad-weight
+ * kernel sample the input again, which is also what happens whenever the caller
+ * wants neither grad_offset nor grad_mask.  Workspace sizes depend on the mode.
+ * One setting per process (see d2c_set_algo_override). */
 void d2c_set_grad_weight_mode(int mode);
 
 const char *d2c_last_error(void);

@@ -110,7 +110,7 @@ def test_grad_weight_from_columns_matches_resampling(name, wanted, dev):
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, torch.bfloat16, seed=5)
     eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
     got = {}
-    for mode in ("columns", "resample"):
+    for mode in ("columns", "in_place", "resample"):
         _ops.set_grad_weight_mode(mode)
         try:
             ts = [t.to(dev) if t is not None else None for t in (x, off, m, w, b)]
@@ -129,8 +129,13 @@ def test_grad_weight_from_columns_matches_resampling(name, wanted, dev):
         assert_close(got[mode], eg[3], 2e-2, 2e-2 * eg[3].abs().max().item(), f"grad_weight ({mode})")
         if wanted != "w":
             assert rel_l2(ts[1].grad, eg[1]) < 2e-2, mode
+        if wanted == "all":
+            assert rel_l2(ts[0].grad, eg[0]) < 2e-2, mode
+            if ts[2] is not None:
+                assert rel_l2(ts[2].grad, eg[2]) < 2e-2, mode
     # the two differ by the rounding of the columns to bfloat16 at most (both round them before the product)
     assert rel_l2(got["columns"], got["resample"].float().cpu()) < 1e-2
+    assert rel_l2(got["in_place"], got["columns"].float().cpu()) < 1e-3
 
 
 @pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail", "dw64", "dw96_G3_nomask",
