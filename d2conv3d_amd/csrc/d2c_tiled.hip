@@ -267,7 +267,7 @@ __global__ void __launch_bounds__(256) pack_weight_fwd_kernel(const T *w, T *wp,
 // The same re-layout through LDS: a workgroup takes kPackRows output channels of one channel chunk, whose
 // weights are runs of BKC * K consecutive elements in W, reads them with 16-byte loads and writes whole
 // 16-byte fragment vectors (kPackRows consecutive lanes each).  Needs a 16-byte aligned W and rows that fit LDS.
-constexpr int kPackRows = 16;
+constexpr int kPackRows = 8;
 template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_fwd_lds_kernel(const T *w, T *wp, TiledShape s)
 {

@@ -1434,7 +1434,7 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
 // The same re-layout through LDS (needs a 16-byte aligned W): a workgroup takes a block of output channels
 // as wide as the padding unit of ogk (128 bytes of wt) and kPackCh channels of a chunk, whose weights are
 // runs of kPackCh * K consecutive elements in W, and writes 16-byte vectors of consecutive output channels.
-constexpr int kPackCh = 16;
+constexpr int kPackCh = 8;
 template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_bwd_lds_kernel(const T *w, T *wt, TiledShape s, int ogk, int o0,
                                                                   int ogn)
@@ -1540,7 +1540,7 @@ __global__ void __launch_bounds__(256) cvt_grad_weight_kernel(const float *src, 
 // The same through LDS (needs a 16-byte aligned grad_weight): a workgroup takes kCvtRows output channels of one
 // channel chunk; per tap their accumulator rows are one contiguous piece, and in grad_weight they are runs
 // of BKC * K consecutive elements.
-constexpr int kCvtRows = 16;
+constexpr int kCvtRows = 4;
 template <typename T>
 __global__ void __launch_bounds__(256) cvt_grad_weight_lds_kernel(const float *src, T *dst, TiledShape s)
 {
