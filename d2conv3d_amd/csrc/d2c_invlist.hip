@@ -62,8 +62,11 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
 // a in {0, 1} with weight:  r = 0: (h, -),  r = 1: (1 - h, h),  r = 2: (-, 1 - h).
 // z and y offsets are compile-time (9 unrolled visits); the 3 base voxels along x are adjacent bins, one
 // contiguous range of entries, the x offset of an entry follows from its place in the range.
-template <typename T, bool COMPACT>
-__global__ void __launch_bounds__(256, 4)   // registers for 4 wavefronts per SIMD
+// EB: list entries (and grad-column rows) requested together by a group of lanes: 4 at registers for 4 wavefronts per
+// SIMD, or 8 at registers for 2 -- more rows in flight per lane, which pays where the problem does not fill the
+// compute units with wavefronts anyway (see d2c_gx_owner_launch).
+template <typename T, bool COMPACT, int EB>
+__global__ void __launch_bounds__(256, EB == 4 ? 4 : 2)
 gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
@@ -107,11 +110,11 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
             const int em2 = em1 + min(L.counts[bin1 + 1], L.cap);
             const int e1 = em2 + (nxb == 3 ? min(L.counts[bin1 + 2], L.cap) : 0);
             const uint4 *eb = reinterpret_cast<const uint4 *>(L.entries) + (long)bin1 * L.cap * (COMPACT ? 1 : 2);
-            for (int e = 0; e < e1; e += 4) {
-                InvEntry en[4];
-                uint4 row[4];
+            for (int e = 0; e < e1; e += EB) {
+                InvEntry en[EB];
+                uint4 row[EB];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < EB; i++) {
                     const int ei = min(e + i, e1 - 1);
                     const int slot = ei < em1 ? ei : (ei < em2 ? ei - em1 + L.cap : ei - em2 + 2 * L.cap);
                     if constexpr (COMPACT) {
@@ -124,10 +127,10 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < EB; i++)
                     row[i] = *reinterpret_cast<const uint4 *>(gbase + ((long)en[i].k * s.M + en[i].p) * BKC);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < EB; i++) {
                     const float hz = en[i].hz, hy = en[i].hy, hx = en[i].hx;
                     const float al = e + i < e1 ? en[i].alpha : 0.f;
                     // x: offset 0 (base x0-1) reaches voxel c=0 with hx; 1 reaches (1-hx, hx); 2 reaches c=1 with 1-hx
@@ -476,8 +479,18 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
     dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * (s.Cin / BKC)));    // see the kernel's unit mapping
-    if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
-    else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    // Eight rows in flight per group of lanes where several channel chunks of an offset group walk the same lists
+    // (bfloat16): the lists then come from L2 and the rows' latency is what the kernel waits for (N=2, C=256, one
+    // offset group: 0.30 -> 0.23 ms; 207360 positions: 1.78 -> 1.59 ms).  With one chunk per offset group (C=512 in 8
+    // groups: 0.40 -> 0.45 ms) and for float problems (0.39 -> 0.41 ms) the wavefront lost per SIMD costs more.
+    const int eb = (sizeof(T) == 2 && s.cpg / BKC >= 2) ? 8 : 4;
+    if (eb == 8) {
+        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    } else {
+        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    }
     if (int rc = d2c_check_launch("gx_owner_kernel")) return rc;
     // the overflow entries, usually none (the kernel reads their number from device memory)
     hipLaunchKernelGGL(gx_overflow_kernel<T>, dim3(512), dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
