@@ -40,6 +40,9 @@ SHAPES = {
     # columns, two chunks per workgroup), ragged last position tile, all 512 / some of the output channels of a pass
     "c256_G2_o512_tail": (1, 256, 512, (3, 7, 7), 3, 1, 1, 1, 1, 2, True, True, 1.5),
     "c256_groups2_G4_o384": (2, 256, 384, (3, 5, 6), 3, 1, 1, 1, 2, 4, False, False, 1.5),
+    # four chunks per weight group, 200 output channels: half of the grad-weight product's wavefronts have no output
+    # channels and only move column tiles; the last slice of output channels is ragged
+    "c256_G1_o200": (2, 256, 200, (3, 6, 7), 3, 1, 1, 1, 1, 1, True, True, 1.5),
     # channel-separated (groups == Cin == Cout)
     "dw64": (2, 64, 64, (4, 6, 7), 3, 1, 1, 1, 64, 1, True, True, 1.5),
     "dw96_G3_nomask": (1, 96, 96, (3, 5, 9), 3, 1, 1, 1, 96, 3, False, False, 1.0),
@@ -101,7 +104,7 @@ def test_tiled_forward_backward(name, dtype, dev):
                 assert_close(t.grad, e, 2e-2, 2e-2 * e.abs().max().item(), n)
 
 
-@pytest.mark.parametrize("name", ["c128_G2_o96", "c256_G2_o512_tail", "c256_groups2_G4_o384"])
+@pytest.mark.parametrize("name", ["c128_G2_o96", "c256_G2_o512_tail", "c256_groups2_G4_o384", "c256_G1_o200"])
 @pytest.mark.parametrize("wanted", ["all", "w+offset", "w"])
 def test_grad_weight_from_columns_matches_resampling(name, wanted, dev):
     # bfloat16 grad_weight two ways: as a matrix product over the sampled columns that the offset / mask gradient
