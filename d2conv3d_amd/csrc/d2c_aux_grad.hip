@@ -208,8 +208,8 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                         xv[r][c] = ((inr >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + o) : make_uint4(0, 0, 0, 0);
                     }
                     const int m = m0 + pos;
-                    gq[r] = inr ? *reinterpret_cast<const uint4 *>(gcb + ((grow + m) * BKC + ivec * VEC) * (long)sizeof(T))
-                                : make_uint4(0, 0, 0, 0);
+                    // (the grad-column row: read once by this kernel)
+                    gq[r] = inr ? ld_stream16(gcb + ((grow + m) * BKC + ivec * VEC) * (long)sizeof(T)) : make_uint4(0, 0, 0, 0);
                 }
                 if constexpr (COL) {
                     // (a streaming store: written once, read by another kernel much later; it leaves the rows that

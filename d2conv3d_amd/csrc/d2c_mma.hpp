@@ -345,6 +345,13 @@ template <typename T, int NT> D2C_DEV void bias_grad_body(const T *gout, T *gb, 
 // they need themselves (vmcnt) and for the reads with lds_rows_wait(), through which the values must pass before
 // they are used.
 typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+// 16 bytes of a buffer that the kernel reads once, front to back (grad-column rows, sampled columns): a streaming load,
+// so that the lines do not push the rows that are gathered again and again out of the L2.
+D2C_DEV uint4 ld_stream16(const void *p)
+{
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 template <int OFF> D2C_DEV u32x4_t lds_row_read(unsigned lds_addr)
 {
     u32x4_t v;

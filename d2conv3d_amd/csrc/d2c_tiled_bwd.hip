@@ -1327,14 +1327,14 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
 #pragma unroll
             for (int ob = 0; ob < OB; ob++) ldB[kg * 2 + ob] = g1[(ob * NKGP + kg) * 64];
         const long r0 = col_row0(0), r1 = col_row0(1), r2 = col_row0(2);
-        crE0 = colp0[r0];
-        crE1 = colp1[r0];
-        crO0 = colp0[r1];
-        crO1 = colp1[r1];
+        crE0 = ld_stream16(colp0 + r0);
+        crE1 = ld_stream16(colp1 + r0);
+        crO0 = ld_stream16(colp0 + r1);
+        crO1 = ld_stream16(colp1 + r1);
         *reinterpret_cast<uint4 *>(st_p) = crE0;
         *reinterpret_cast<uint4 *>(st_p + MT * TRS) = crE1;
-        crE0 = colp0[r2];
-        crE1 = colp1[r2];
+        crE0 = ld_stream16(colp0 + r2);
+        crE1 = ld_stream16(colp1 + r2);
     }
     lds_only_barrier();
     // Wavefronts without output channels (weight groups of fewer than 512) only move the column tiles.  Each role has
@@ -1373,8 +1373,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
             *reinterpret_cast<uint4 *>(st_p + ((dbuf ^ 1) * NCH * MT) * TRS) = cr0;
             *reinterpret_cast<uint4 *>(st_p + ((dbuf ^ 1) * NCH + 1) * MT * TRS) = cr1;
             const long r3 = col_row0(it + 3);
-            cr0 = colp0[r3];
-            cr1 = colp1[r3];
+            cr0 = ld_stream16(colp0 + r3);
+            cr1 = ld_stream16(colp1 + r3);
             lds_only_barrier();
         };
         // pairs of steps, then the odd one out: no branch inside the loop (see above)
