@@ -49,7 +49,7 @@ WORKLOADS = {
 PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 PEAK_GBS = 8000.0
 # largest sample the CPU leg runs (the oracle does ~0.09 TFLOP/s on 16 cores): N and leading dim cut down to this
-CPU_CROP = {"c5b": (1, (16, 60, 108))}
+CPU_CROP = {"c3": (1, (8, 30, 54)), "c5b": (1, (8, 60, 108))}
 
 
 def make_inputs(name, torch, crop=None, want_size=False):
@@ -136,34 +136,30 @@ def cpu_baseline(name, torch):
     if c["dt"] == "bf16":
         x, w, b, gout, off, m = (t.bfloat16().float() for t in (x, w, b, gout, off, m))
     fwd, bwd = (cpu.conv3d_forward, cpu.conv3d_backward) if c["nd"] == 3 else (cpu.conv1d_forward, cpu.conv1d_backward)
-    # timed iterations until 5 s have passed (at most 200); the figure is the median iteration when there are at
-    # least five of them (after one untimed warm-up iteration), else the mean
+    # one untimed warm-up iteration, then timed iterations until at least three are done and 5 s have passed (at
+    # most 200); the figure is their median
     def once():
         fwd(x, off, m, w, b, 1, 1, 1, c["groups"], c["G"])
         if c["backward"]:
             bwd(gout, x, off, m, w, True, 1, 1, 1, c["groups"], c["G"])
+    t_start = time.perf_counter()
+    once()
+    t_warm = time.perf_counter() - t_start
     times = []
     t_start = time.perf_counter()
-    while True:
+    while len(times) < 3 or (time.perf_counter() - t_start < 5.0 and len(times) < 200):
         t0 = time.perf_counter()
         once()
-        t1 = time.perf_counter()
-        times.append(t1 - t0)
-        if t1 - t_start > 5.0 or len(times) >= 201:
-            break
-    if len(times) >= 6:
-        timed = sorted(times[1:])
-        per_iter, stat = timed[len(timed) // 2], "median"
-    else:
-        timed = times
-        per_iter, stat = sum(times) / len(times), "mean"
+        times.append(time.perf_counter() - t0)
+    timed = sorted(times)
+    per_iter, stat = timed[len(timed) // 2], "median"
     f_fwd, _, _ = algorithmic(name, x.shape[0], tuple(x.shape[2:]))
     flops = (3 if c["backward"] else 1) * f_fwd
     what = "full workload" if crop is None else f"same layer on N={crop[0]}, {'x'.join(map(str, crop[1]))} positions"
     return {
         "value": flops / per_iter / 1e12, "unit": "TFLOP/s", "cores": cpu.num_threads(), "kind": "port",
         "sample": f"{what}, fp32, {'forward+backward' if c['backward'] else 'forward'}: {stat} of {len(timed)} "
-                  f"iterations = {per_iter * 1e3:.2f} ms ({sum(times):.2f} s of CPU work)",
+                  f"iterations after one warm-up = {per_iter * 1e3:.2f} ms ({sum(times) + t_warm:.2f} s of CPU work)",
     }
 
 
@@ -550,57 +546,67 @@ def main():
     torch.cuda.synchronize()
     lib.d2c_profile_enable(0)
     fam = {"mfma": "tiled", "depthwise": "dw", "generic": "generic"}[algo]
-    names = {_lib.PROF_FWD: f"{fam}_fwd_kernel", _lib.PROF_BWD_DATA: f"{fam}_bwd_data_kernel",
-             _lib.PROF_BWD_WEIGHT: f"{fam}_bwd_weight_kernel", _lib.PROF_GX_OWNER: "gx_owner_kernel",
-             _lib.PROF_BWD_AUX: "aux_grad_kernel", _lib.PROF_PACK: "pack/clear/convert/lists"}
-    if fam == "dw":
-        names[_lib.PROF_BWD_DATA] = "dw_bwd_kernel"
-    kern = {}
-    for kid, kname in names.items():
+    # per-kernel time under the name a profiler trace shows (the library reports which kernel it launched)
+    ids = {_lib.PROF_FWD: "fwd", _lib.PROF_BWD_DATA: "bwd_data", _lib.PROF_BWD_WEIGHT: "bwd_weight",
+           _lib.PROF_GX_OWNER: "gx_owner", _lib.PROF_BWD_AUX: "bwd_aux", _lib.PROF_PACK: "pack"}
+    kern, role = {}, {}
+    for kid, r in ids.items():
         tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
         lib.d2c_profile_read(kid, ctypes.byref(tot), ctypes.byref(cnt))
         if cnt.value:
+            kname = "pack/clear/convert/lists" if r == "pack" else (lib.d2c_profile_kernel_name(kid).decode() or r)
             kern[kname] = tot.value / nprof  # ms per step spent in this kernel (all launches of it)
+            role[kname] = r
 
-    # the kernel that takes the most time, against the roofline that bounds it
-    main_k = {k: v for k, v in kern.items() if not k.startswith("pack")}
-    dom = max(main_k, key=main_k.get) if main_k else None
+    es = 2 if dt == "bf16" else 4
+    P = 1
+    for d in dims:
+        P *= d
+    K = 3 ** nd
+    kms = {k: round(v, 4) for k, v in kern.items()}
     roofline = None
-    if dom:
-        kms = {k: round(v, 4) for k, v in kern.items()}
+    gemm_k = {k: v for k, v in kern.items() if role[k] in ("fwd", "bwd_data", "bwd_weight")}
+    main_k = {k: v for k, v in kern.items() if role[k] != "pack"}
+    if c["bound"] == "mfma" and gemm_k:
+        # the longest kernel that carries one of the three GEMMs (2*N*P*Cout*(Cin/groups)*K flop each)
+        dom = max(gemm_k, key=gemm_k.get)
+        ach = f_fwd_flops / (gemm_k[dom] * 1e-3) / 1e12
         traffic, traffic_source = hbm_traffic_bytes(name, dom)
-        t_dom = main_k[dom] * 1e-3
-        es = 2 if dt == "bf16" else 4
-        P = 1
-        for d in dims:
-            P *= d
-        if dom == "aux_grad_kernel":
-            # every tensor it has to move once: the grad-column rows in, the sampled columns out (bfloat16 problems
-            # whose grad_weight runs over them), the input, offsets and modulation in, their gradients out, one list
-            # entry (16 / 32 B) per sample
-            K = 3 ** nd
-            rows = N * P * K * C * es
-            cols = rows if (dt == "bf16" and nd == 3 and args.grad_weight_mode >= 1 and (C // groups) % 128 == 0) else 0
-            aux = N * P * K * G * (nd + 1) * (2 if dt == "bf16" else 4)
-            nbytes = rows + cols + N * P * C * es + 2 * aux + N * P * K * G * (16 if dt == "bf16" else 32)
-            bound, ach = "hbm", nbytes / t_dom / 1e9
-        elif dom == "gx_owner_kernel":
-            # every grad-column row (N*P*K*Cin elements), every list entry (32 B per sample) and every
-            # grad_input element (fp32 accumulator) once
-            K = 3 ** nd
-            nbytes = N * P * K * C * es + N * P * K * G * 32 + N * C * P * 4
-            bound, ach = "hbm", nbytes / t_dom / 1e9
-        elif c["bound"] == "hbm":
-            # every tensor of that direction once
-            nbytes = b_fwd if dom.endswith("fwd_kernel") else b_bwd
-            bound, ach = "hbm", nbytes / t_dom / 1e9
-        else:
-            # each of the three matrix kernels carries one GEMM of f_fwd flops
-            bound, ach = "mfma", f_fwd_flops / t_dom / 1e12
-        peak, unit = (PEAK_GBS, "GB/s") if bound == "hbm" else (PEAK_TFLOPS[dt], "TFLOP/s")
-        roofline = {"bound": bound, "kernel": dom, "achieved": round(ach, 2), "peak": peak, "unit": unit,
-                    "frac": round(ach / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
+        roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 2), "peak": PEAK_TFLOPS[dt],
+                    "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dt], 4), "traffic": traffic,
+                    "traffic_source": traffic_source, "algorithmic_gflop_per_launch": round(f_fwd_flops / 1e9, 2),
+                    "whole_step_frac": round(value / PEAK_TFLOPS[dt], 4), "kernel_ms": kms}
+    elif main_k:
+        # bandwidth-bound workloads: the longest kernel against every tensor of its direction once
+        dom = max(main_k, key=main_k.get)
+        nbytes = b_fwd if role[dom] == "fwd" else b_bwd
+        ach = nbytes / (main_k[dom] * 1e-3) / 1e9
+        traffic, traffic_source = hbm_traffic_bytes(name, dom)
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(ach, 2), "peak": PEAK_GBS, "unit": "GB/s",
+                    "frac": round(ach / PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                    "algorithmic_mbytes_per_launch": round(nbytes / 1e6, 1),
+                    "whole_step_frac": round((b_fwd + (b_bwd if c["backward"] else 0)) / (ms * 1e-3) / 1e9 / PEAK_GBS, 4),
                     "kernel_ms": kms}
+
+    # The gather kernels of the matrix-core backward carry no GEMM; what they move is mostly the library's own
+    # intermediates (grad-column rows, sampled columns, sample lists), i.e. internal traffic, not tensors of the
+    # operator: reported apart from `roofline`, never as a fraction of a peak over algorithmic bytes.
+    internal = None
+    if fam == "tiled":
+        rows = N * P * K * C * es
+        per = {}
+        for kname, r in role.items():
+            if r == "bwd_aux":
+                cols = rows if (dt == "bf16" and nd == 3 and args.grad_weight_mode >= 1 and (C // groups) % 128 == 0) else 0
+                aux = N * P * K * G * (nd + 1) * es
+                per[kname] = rows + cols + N * P * C * es + 2 * aux + N * P * K * G * (16 if dt == "bf16" else 32)
+            elif r == "gx_owner":
+                per[kname] = rows + N * P * K * G * (16 if dt == "bf16" else 32) + N * C * P * 4
+        if per:
+            internal = {"note": "internal traffic: grad-column rows, sampled columns and sample lists of the library "
+                                "plus the operator's tensors these kernels touch, each counted once",
+                        "kernels": {k: {"ms": round(kern[k], 4), "internal_mbytes": round(v / 1e6, 1),
+                                        "gbytes_per_s": round(v / (kern[k] * 1e-3) / 1e9, 1)} for k, v in per.items()}}
 
     # Depthwise kernels: the corner rows they pull through the vector-memory path of the compute units (L1), which
     # is what bounds them (64 bytes per clock and compute unit; 256 units at 2.4 GHz), beside the HBM figure above.
@@ -609,7 +615,8 @@ def main():
         peak_l1 = 64 * 256 * 2.4  # GB/s
         npos, esz = dims[0] * dims[1] * dims[2], (2 if dt == "bf16" else 4)
         rows = N * npos * 27 * 8 * C * esz          # 8 corner values per tap and channel
-        per = {"dw_fwd_kernel": rows, "dw_bwd_kernel": rows + N * npos * 27 * C * esz}   # + the grad_out value per tap
+        per = {"dw_fwd_kernel": rows, "dw_bwd_kernel": rows + N * npos * 27 * C * esz,   # + the grad_out value per tap
+               "dw_gx_owner_kernel": N * npos * 27 * (32 + C * esz) + N * npos * C * 4}  # list entry + grad_out row per sample, grad_input once
         roofline_l1 = {"bound": "l1", "peak": round(peak_l1, 1), "unit": "GB/s",
                        "peak_source": "64 B/clk/CU x 256 CUs x 2.4 GHz (vector-memory path)", "kernels": {}}
         for kname, nbytes in per.items():
@@ -637,6 +644,7 @@ def main():
                    "taps_outside_volume": taps,
                    "algorithmic_gflop": round(nflops / 1e9, 2),
                    "algorithmic_mbytes": round((b_fwd + (b_bwd if c["backward"] else 0)) / 1e6, 1),
+                   "backward_workspace_mbytes": round(nb / 1e6, 1), "forward_workspace_mbytes": round(nf / 1e6, 1),
                    "frac_of_mfma_peak_whole_step": round(value / PEAK_TFLOPS[dt], 4),
                    "frac_of_hbm_peak_whole_step": round((b_fwd + (b_bwd if c["backward"] else 0))
                                                         / (ms * 1e-3) / 1e9 / PEAK_GBS, 4)},
@@ -644,6 +652,8 @@ def main():
     }
     if roofline_l1:
         line["roofline_l1"] = roofline_l1
+    if internal:
+        line["gather_kernels"] = internal
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(name, torch)
     print(json.dumps(line))

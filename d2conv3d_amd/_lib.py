@@ -23,7 +23,7 @@ EXPORTS = (
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
     "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_set_grad_weight_mode", "d2c_last_error", "d2c_version",
-    "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read",
+    "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read", "d2c_profile_kernel_name",
     "d2c_size_map_offsets_forward", "d2c_size_map_offsets_backward",
     "d2c_conv3d_sized_forward_workspace_bytes", "d2c_conv3d_sized_backward_workspace_bytes",
     "d2c_conv3d_sized_forward", "d2c_conv3d_sized_backward",
@@ -138,6 +138,7 @@ def load():
     lib.d2c_profile_reset.argtypes, lib.d2c_profile_reset.restype = [], None
     lib.d2c_profile_read.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]
     lib.d2c_profile_read.restype = ctypes.c_int
+    lib.d2c_profile_kernel_name.argtypes, lib.d2c_profile_kernel_name.restype = [ctypes.c_int], ctypes.c_char_p
     _lib = lib
     return lib
 

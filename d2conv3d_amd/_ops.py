@@ -483,15 +483,17 @@ def conv3d_corner_index(input_shape, offset, kernel_size, stride=(1, 1, 1), padd
 
 
 def conv3d_algo(input, offset, alpha, weight, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
-                groups=1, offset_groups=1):
-    """Name of the kernel family ("generic", "mfma", "depthwise") these arguments are served by."""
+                groups=1, offset_groups=1, offset_axes=7):
+    """Name of the kernel family ("generic", "mfma", "depthwise") these arguments are served by; "invalid" when
+    none takes them (a partial `offset_axes` on a shape the matrix-core kernels do not serve in both directions)."""
     lib = _lib.load()
     input, offset, alpha, weight, _ = _unify(input, offset, alpha, weight, None)
     N, Cin, D, H, W = input.shape
     Cout, _, kd, kh, kw = weight.shape
     Do, Ho, Wo = offset.shape[2:]
     desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, *stride, *padding, *dilation,
-                           groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype])
+                           groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype],
+                           _lib.EPILOGUE_NONE, 1.0, int(offset_axes))
     return _lib.ALGO_NAMES.get(lib.d2c_conv3d_algo(ctypes.byref(desc)), "invalid")
 
 

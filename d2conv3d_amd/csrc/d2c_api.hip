@@ -28,7 +28,12 @@ struct ProfState {
     hipEvent_t open_start[D2C_PROF_COUNT] = {};
     double total_ms[D2C_PROF_COUNT] = {};
     int launches[D2C_PROF_COUNT] = {};
+    const char *name[D2C_PROF_COUNT] = {};
 } g_prof;
+
+struct LdsGrant { const void *fn; int dev, bytes; };
+std::mutex g_lds_mu;
+std::vector<LdsGrant> g_lds_grants;
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n)
 {
@@ -100,10 +105,31 @@ int d2c_num_cus()
     return n;
 }
 
-void d2c_prof_begin(int id, hipStream_t st)
+int d2c_allow_lds(const void *kernel, int bytes, const char *what)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        d2c_set_error("hipGetDevice failed");
+        return D2C_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lk(g_lds_mu);
+    for (const LdsGrant &g : g_lds_grants)
+        if (g.fn == kernel && g.dev == dev && g.bytes >= bytes) return D2C_OK;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) {
+        d2c_set_error("hipFuncSetAttribute(%s, dynamic LDS %d): %s", what, bytes, hipGetErrorString(e));
+        (void)hipGetLastError();
+        return D2C_ERR_LAUNCH;
+    }
+    g_lds_grants.push_back({kernel, dev, bytes});
+    return D2C_OK;
+}
+
+void d2c_prof_begin(int id, hipStream_t st, const char *name)
 {
     if (!g_prof.on) return;
     std::lock_guard<std::mutex> lk(g_prof.mu);
+    if (name) g_prof.name[id] = name;
     hipEvent_t e;
     if (hipEventCreate(&e) != hipSuccess) return;
     (void)hipEventRecord(e, st);
@@ -181,7 +207,15 @@ void d2c_profile_reset(void)
         prof_drain(i);
         g_prof.total_ms[i] = 0.0;
         g_prof.launches[i] = 0;
+        g_prof.name[i] = nullptr;
     }
+}
+
+const char *d2c_profile_kernel_name(int id)
+{
+    if (id < 0 || id >= D2C_PROF_COUNT) return "";
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    return g_prof.name[id] ? g_prof.name[id] : "";
 }
 
 int d2c_profile_read(int id, double *total_ms, int *launches)
@@ -274,8 +308,10 @@ static int choose_algo(const d2c_conv3d_desc &q, bool quiet)
 {
     const int a = choose_algo_any_axes(q, quiet);
     const bool fixed_axis = (q.offset_axes & 7) != 0 && (q.offset_axes & 7) != 7;
-    if (a >= 0 && fixed_axis && a != D2C_ALGO_MFMA) {
-        if (!quiet) d2c_set_error("offset_axes = %d is served by the matrix-core kernels only", q.offset_axes);
+    if (a >= 0 && fixed_axis && (a != D2C_ALGO_MFMA || !d2c_tiled_axes_supported(q))) {
+        if (!quiet)
+            d2c_set_error("offset_axes = %d is served by the matrix-core kernels only (in both directions: offset "
+                          "groups must lie inside weight groups)", q.offset_axes);
         return -1;
     }
     return a;

@@ -349,7 +349,7 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     dim3 grid((unsigned)(8 * (((ntile + kWavesPerBlock - 1) / kWavesPerBlock + 7) / 8) * s.G * nshare));
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
-    D2cProfScope prof(D2C_PROF_BWD_AUX, st);
+    D2cProfScope prof(D2C_PROF_BWD_AUX, st, "aux_grad_kernel");
     const dim3 blk(64 * kWavesPerBlock);
     if constexpr (sizeof(T) == 2) {
         // (the sampled columns are written for bfloat16 problems in three dimensions only, see d2c_bwd_weight_from_col)

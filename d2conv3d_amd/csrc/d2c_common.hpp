@@ -130,13 +130,18 @@ int d2c_num_cus();
 void d2c_fill_zero(void *p, size_t bytes, hipStream_t st);
 
 // Event bracket around a kernel launch when instrumentation is on (see d2c_profile_enable).
-void d2c_prof_begin(int id, hipStream_t st);
+// `name` (a string literal): the kernel launched inside the bracket, reported by d2c_profile_kernel_name().
+void d2c_prof_begin(int id, hipStream_t st, const char *name = nullptr);
 void d2c_prof_end(int id, hipStream_t st);
 struct D2cProfScope {
     int id; hipStream_t st;
-    D2cProfScope(int i, hipStream_t s) : id(i), st(s) { d2c_prof_begin(id, st); }
+    D2cProfScope(int i, hipStream_t s, const char *name = nullptr) : id(i), st(s) { d2c_prof_begin(id, st, name); }
     ~D2cProfScope() { d2c_prof_end(id, st); }
 };
+
+// Raises a kernel's dynamic-LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize); the runtime is asked once
+// per (kernel, device), later calls only look the pair up.  Returns D2C_OK or D2C_ERR_LAUNCH with the error text set.
+int d2c_allow_lds(const void *kernel, int bytes, const char *what);
 
 static inline size_t d2c_align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 

@@ -512,7 +512,7 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
 {
     DwArgs a{s, xcl, off, mask, wt, bias, out, nullptr, nullptr, nullptr, nullptr, nullptr};
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
-    D2cProfScope prof(D2C_PROF_FWD, st);
+    D2cProfScope prof(D2C_PROF_FWD, st, "dw_fwd_kernel");
     hipLaunchKernelGGL(dw_fwd_kernel<T>, dim3(dw_grid(s, kFwdTP, s.G * nsl)), dim3(kDwThreads), kDwLdsFwd, st, a);
     return d2c_check_launch("dw_fwd_kernel");
 }
@@ -534,10 +534,8 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
     DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, goutcl, gxcl, auxoff, auxmask, gwacc};
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
     {
-        D2cProfScope prof(D2C_PROF_BWD_DATA, st);
-        if (hipFuncSetAttribute((const void *)dw_bwd_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)kDwLdsBwd) != hipSuccess)
-            return d2c_check_launch("hipFuncSetAttribute(dw_bwd_kernel)");
+        if (int rc = d2c_allow_lds((const void *)dw_bwd_kernel<T>, (int)kDwLdsBwd, "dw_bwd_kernel")) return rc;
+        D2cProfScope prof(D2C_PROF_BWD_DATA, st, "dw_bwd_kernel");
         hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3(dw_grid(s, kBwdTP, s.G * nsl)), dim3(kDwThreads), kDwLdsBwd, st, a);
     }
     if (int rc = d2c_check_launch("dw_bwd_kernel")) return rc;

@@ -73,32 +73,44 @@ template <typename T> __global__ void __launch_bounds__(kGnThreads) channel_stat
     }
 }
 
-// mean and 1 / sqrt(var + eps) of the group that channel c of sample n belongs to
+// mean and 1 / sqrt(var + eps) of a group from the sums over its (C / groups) * P values.  The per-channel fp32 sums
+// are combined, and the variance sum_sq / m - mean^2 is taken, in double: with |mean| far above the standard
+// deviation the two terms agree in their leading digits and a float difference would lose the variance.
+D2C_DEV void moments_from_sums(double s, double sq, double m, float eps, float &mean, float &rstd)
+{
+    const double mu = s / m;
+    const double var = fmax(sq / m - mu * mu, 0.0);
+    mean = (float)mu;
+    rstd = (float)(1.0 / sqrt(var + (double)eps));
+}
+
+// mean and rstd of the group that channel c of sample n belongs to
 D2C_DEV void group_moments(const GnArgs &a, int n, int c, float &mean, float &rstd)
 {
     const int cpg = a.q.C / a.q.groups, g = c / cpg;
     const float *st = a.stats + ((long)n * a.q.C + g * cpg) * 2;
-    float s = 0.f, sq = 0.f;
-    for (int i = 0; i < cpg; i++) { s += st[2 * i]; sq += st[2 * i + 1]; }
-    const float m = (float)cpg * (float)a.q.P;
-    mean = s / m;
-    const float var = fmaxf(sq / m - mean * mean, 0.f);
-    rstd = 1.f / sqrtf(var + a.q.eps);
+    double s = 0.0, sq = 0.0;
+    for (int i = 0; i < cpg; i++) { s += (double)st[2 * i]; sq += (double)st[2 * i + 1]; }
+    moments_from_sums(s, sq, (double)cpg * (double)a.q.P, a.q.eps, mean, rstd);
 }
 
 // the same by all threads of a workgroup together
-D2C_DEV void group_moments_block(const GnArgs &a, int n, int c, float &mean, float &rstd, float *red)
+D2C_DEV void group_moments_block(const GnArgs &a, int n, int c, float &mean, float &rstd, float *)
 {
+    __shared__ double redd[2][kGnThreads / 64];
     const int cpg = a.q.C / a.q.groups, g = c / cpg;
     const float *st = a.stats + ((long)n * a.q.C + g * cpg) * 2;
-    float s = 0.f, sq = 0.f;
-    for (int i = threadIdx.x; i < cpg; i += kGnThreads) { s += st[2 * i]; sq += st[2 * i + 1]; }
-    s = block_sum(s, red);
-    sq = block_sum(sq, red);
-    const float m = (float)cpg * (float)a.q.P;
-    mean = s / m;
-    const float var = fmaxf(sq / m - mean * mean, 0.f);
-    rstd = 1.f / sqrtf(var + a.q.eps);
+    double s = 0.0, sq = 0.0;
+    for (int i = threadIdx.x; i < cpg; i += kGnThreads) { s += (double)st[2 * i]; sq += (double)st[2 * i + 1]; }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) { s += __shfl_xor(s, d, 64); sq += __shfl_xor(sq, d, 64); }
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) { redd[0][threadIdx.x >> 6] = s; redd[1][threadIdx.x >> 6] = sq; }
+    __syncthreads();
+    s = sq = 0.0;
+#pragma unroll
+    for (int i = 0; i < kGnThreads / 64; i++) { s += redd[0][i]; sq += redd[1][i]; }
+    moments_from_sums(s, sq, (double)cpg * (double)a.q.P, a.q.eps, mean, rstd);
 }
 
 template <typename T> __global__ void __launch_bounds__(kGnThreads) gn_fwd_kernel(GnArgs a)

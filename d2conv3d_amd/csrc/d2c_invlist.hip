@@ -475,7 +475,7 @@ template <typename T>
 int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st)
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
-    D2cProfScope prof(D2C_PROF_GX_OWNER, st);
+    D2cProfScope prof(D2C_PROF_GX_OWNER, st, "gx_owner_cube_kernel");
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
     dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * (s.Cin / BKC)));    // see the kernel's unit mapping
@@ -504,13 +504,11 @@ template <typename T>
 int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const SampleLists &L, float *gxcl,
                            hipStream_t st)
 {
-    D2cProfScope prof(D2C_PROF_GX_OWNER, st);
+    if (int rc = d2c_allow_lds((const void *)dw_gx_owner_kernel<T>, 160 * 1024, "dw_gx_owner_kernel")) return rc;
+    D2cProfScope prof(D2C_PROF_GX_OWNER, st, "dw_gx_owner_kernel");
     size_t lds = (size_t)s.K * kOwnSlice * sizeof(T);
     const int w_in_lds = lds <= 144 * 1024;
     if (!w_in_lds) lds = 0;
-    if (hipFuncSetAttribute((const void *)dw_gx_owner_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            160 * 1024) != hipSuccess)
-        return d2c_check_launch("hipFuncSetAttribute(dw_gx_owner_kernel)");
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
     const unsigned nblk = xcd_unit_grid(s.N * s.G * nslice, ncz * ncy * ((ncx + kOwnVox - 1) / kOwnVox));

@@ -748,6 +748,15 @@ bool d2c_tiled_supported(const d2c_conv3d_desc &q)
 
 int d2c_tiled_algo(const d2c_conv3d_desc &q) { return is_depthwise(q) ? D2C_ALGO_DEPTHWISE : D2C_ALGO_MFMA; }
 
+// Offsets held at zero along some axes (offset_axes) are honoured by the tiled kernels only: every part of the
+// backward pass has to stay on them too, or the direct kernels that take over would sample with the unzeroed offsets.
+bool d2c_tiled_axes_supported(const d2c_conv3d_desc &q)
+{
+    if (is_depthwise(q) || !mfma_channels_ok(q)) return false;
+    const TiledShape s = tiled_shape(q);
+    return d2c_tiled_bwd_data_supported(s, q.dtype) && d2c_tiled_bwd_weight_supported(s, q.dtype);
+}
+
 size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q, bool with_stats)
 {
     const TiledShape s = tiled_shape(q);

@@ -5,6 +5,8 @@
 
 bool d2c_tiled_supported(const d2c_conv3d_desc &q);
 int d2c_tiled_algo(const d2c_conv3d_desc &q);  // D2C_ALGO_MFMA or D2C_ALGO_DEPTHWISE
+// whether a description with some offset axes fixed (offset_axes != 7) stays on the tiled kernels in both directions
+bool d2c_tiled_axes_supported(const d2c_conv3d_desc &q);
 size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q, bool with_stats = false);
 // `sz` != nullptr: the offsets are formed from a raw size map (`off` is that map [N, channels(mode), P], `goff` the
 // gradient with respect to it); only where d2c_tiled_sized_supported() says so.

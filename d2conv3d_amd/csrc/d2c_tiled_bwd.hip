@@ -811,10 +811,9 @@ int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st)
     const bool db = bwd_col_lds<T>(a.ogk, true) <= 160 * 1024;
     const size_t lds = bwd_col_lds<T>(a.ogk, db);
     const void *fn = db ? (const void *)tiled_bwd_col_kernel<T, NKG, true> : (const void *)tiled_bwd_col_kernel<T, NKG, false>;
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-        return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_col_kernel)");
+    if (int rc = d2c_allow_lds(fn, 160 * 1024, "tiled_bwd_col_kernel")) return rc;
     dim3 grid((a.s.M + MT - 1) / MT, a.s.groups, nsplit);
-    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
+    D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_col_kernel");
     if (db) hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, true>), grid, dim3(kThreads), lds, st, a);
     else hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, false>), grid, dim3(kThreads), lds, st, a);
     return d2c_check_launch("tiled_bwd_col_kernel");
@@ -826,12 +825,10 @@ int launch_bwd_col32(const BwdDataArgs &a, int nsplit, hipStream_t st)
 {
     const size_t lds = (size_t)kColRing * 32 * a.ogk * 2;
     const dim3 grid((a.s.M + kCol32MT - 1) / kCol32MT, a.s.groups, nsplit);
-    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
     auto go = [&](auto nb_c) -> int {
         constexpr int NB = decltype(nb_c)::value;
-        if (hipFuncSetAttribute((const void *)tiled_bwd_col32_kernel<NB>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess)
-            return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_col32_kernel)");
+        if (int rc = d2c_allow_lds((const void *)tiled_bwd_col32_kernel<NB>, 160 * 1024, "tiled_bwd_col32_kernel")) return rc;
+        D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_col32_kernel");
         hipLaunchKernelGGL((tiled_bwd_col32_kernel<NB>), grid, dim3(kThreads), lds, st, a);
         return d2c_check_launch("tiled_bwd_col32_kernel");
     };
@@ -854,11 +851,9 @@ int launch_bwd_data(const BwdDataArgs &a, int nsplit, hipStream_t st)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
     const size_t lds = bwd_data_lds<T>(a.ogk);
-    if (hipFuncSetAttribute((const void *)tiled_bwd_data_kernel<T, NKG>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            160 * 1024) != hipSuccess)
-        return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_data_kernel)");
+    if (int rc = d2c_allow_lds((const void *)tiled_bwd_data_kernel<T, NKG>, 160 * 1024, "tiled_bwd_data_kernel")) return rc;
     dim3 grid((a.s.M + MT - 1) / MT, a.s.groups, nsplit);
-    D2cProfScope prof(D2C_PROF_BWD_DATA, st);
+    D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_data_kernel");
     hipLaunchKernelGGL((tiled_bwd_data_kernel<T, NKG>), grid, dim3(kThreads), lds, st, a);
     return d2c_check_launch("tiled_bwd_data_kernel");
 }
@@ -1877,7 +1872,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     const int nmain = pc.nmain, main_len = pc.main_len, ntail = pc.ntail, tail_len = pc.tail_len;
     if (from_col) {
         BwdWeightColArgs c{s, col, goutp, gwacc, col_rows, otiles, nmain, main_len, ntail, tail_len};
-        D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
+        D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st, "tiled_bwd_weight_col_kernel");
         hipLaunchKernelGGL(tiled_bwd_weight_col_kernel, dim3((unsigned)(items * (nmain + ntail))), dim3(kThreads), 0, st, c);
         if (int rc = d2c_check_launch("tiled_bwd_weight_col_kernel")) return rc;
     }
@@ -1887,13 +1882,13 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         const dim3 grid((unsigned)(items * (nmain + ntail)));
         bool aux16 = false;
         if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
-        D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st);
+        D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st, "tiled_bwd_weight_dma_kernel");
         auto go_nc = [&](auto aux_c, auto sized_c, auto nc_c) -> bool {
             constexpr bool A16 = decltype(aux_c)::value, SZ = decltype(sized_c)::value;
             constexpr int NC = decltype(nc_c)::value;
             constexpr size_t lds = bwd_weight_dma_lds<T, NC>();
-            if (hipFuncSetAttribute((const void *)tiled_bwd_weight_dma_kernel<T, A16, SZ, NC>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            if (d2c_allow_lds((const void *)tiled_bwd_weight_dma_kernel<T, A16, SZ, NC>, 160 * 1024,
+                              "tiled_bwd_weight_dma_kernel") != D2C_OK)
                 return false;
             hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, A16, SZ, NC>), grid, dim3(kThreads + 64), lds, st, a);
             return true;
@@ -1915,7 +1910,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         } else {
             ok = sized ? go(std::false_type{}, std::true_type{}) : go(std::false_type{}, std::false_type{});
         }
-        if (!ok) return d2c_check_launch("hipFuncSetAttribute(tiled_bwd_weight_dma_kernel)");
+        if (!ok) return D2C_ERR_LAUNCH;   // (d2c_allow_lds has set the error text)
     }
     if (int rc = d2c_check_launch("tiled_bwd_weight_dma_kernel")) return rc;
     D2cProfScope prof(D2C_PROF_PACK, st);

@@ -944,7 +944,7 @@ int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
     }
     {
         const int nwg = nshare ? ncu : (a.sk_items < nwg_whole ? a.sk_items : nwg_whole);
-        D2cProfScope prof(D2C_PROF_FWD, st);
+        D2cProfScope prof(D2C_PROF_FWD, st, "tiled_fwd_dma_kernel");
         // offsets fixed along one / two axes (the layers that deform in space or in time only): 4 / 2 corner rows
         const int nfree = a.s.nd == 3 ? __builtin_popcount(a.s.axes & 7) : 3;
         if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
@@ -979,7 +979,7 @@ int launch_fwd(const FwdArgs &a, hipStream_t st)
     const int ntile = (a.s.M + MT - 1) / MT;
     const int NT = 64 * WO;
     dim3 grid(ntile, a.s.ogp / NT * a.nsplit, a.s.groups);
-    D2cProfScope prof(D2C_PROF_FWD, st);
+    D2cProfScope prof(D2C_PROF_FWD, st, "tiled_fwd_kernel");
     if (a.s.ss.on) hipLaunchKernelGGL((tiled_fwd_kernel<T, AUX16, MT, WO, WP, true>), grid, dim3(kThreads), 0, st, a);
     else hipLaunchKernelGGL((tiled_fwd_kernel<T, AUX16, MT, WO, WP, false>), grid, dim3(kThreads), 0, st, a);
     return d2c_check_launch("tiled_fwd_kernel");

@@ -138,7 +138,7 @@ def _fixed_axes_in_kernel(layer, input, offsets, alpha):
     from . import _ops
     dc = layer.deform_conv
     return _ops.conv3d_algo(input, offsets, alpha, dc.weight, dc.stride, dc.padding, dc.dilation, dc.groups,
-                            dc.offset_groups) == "mfma"
+                            dc.offset_groups, offset_axes=layer._offset_axes) == "mfma"
 
 
 class _AxesMixin:

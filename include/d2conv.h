@@ -195,6 +195,9 @@ enum {
 void d2c_profile_enable(int on);
 void d2c_profile_reset(void);
 int d2c_profile_read(int id, double *total_ms, int *launches);
+/* Name of the kernel last launched under `id` since the last reset ("" if none): the name a profiler trace
+ * shows, without template arguments. */
+const char *d2c_profile_kernel_name(int id);
 
 /* ---- dynamic-dilation front end -------------------------------------------------------
  * The step in front of the operator in the size-conditioned layers: the predicted size map

@@ -65,6 +65,67 @@ def test_fixed_offset_axes_need_the_matrix_core_kernels(dev):
         d2c.deform_conv3d(*(t.to(dev) for t in (x, off, m, w, b)), 1, 1, 1, 1, 1, offset_axes=9)
 
 
+def test_fixed_offset_axes_refused_where_the_backward_would_leave_the_matrix_core_kernels(dev):
+    """An offset group that spans several weight groups (groups=2, offset_groups=1): the backward pass of such a
+    shape runs on the direct kernels, which know nothing of offset_axes, so the operator refuses the field as a
+    whole instead of sampling with unzeroed offsets in one direction."""
+    from d2conv3d_amd import _ops
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(1, 128, 3, 5, 6, generator=g).to(dev)
+    w = (torch.randn(128, 64, 3, 3, 3, generator=g) * 0.02).to(dev)
+    off = torch.randn(1, 81, 3, 5, 6, generator=g).to(dev)
+    m = torch.rand(1, 27, 3, 5, 6, generator=g).to(dev)
+    assert _ops.conv3d_algo(x, off, m, w, (1, 1, 1), (1, 1, 1), (1, 1, 1), 2, 1) == "mfma"
+    assert _ops.conv3d_algo(x, off, m, w, (1, 1, 1), (1, 1, 1), (1, 1, 1), 2, 1, offset_axes=6) == "invalid"
+    with pytest.raises(RuntimeError, match="offset_axes"):
+        d2c.deform_conv3d(x, off, m, w, None, 1, 1, 1, 1, 1, 2, offset_axes=6)
+
+
+@pytest.mark.parametrize("cls", ["SpatialMDConv3d", "TemporalMDConv3d"])
+def test_grouped_spatial_and_temporal_layers_against_oracle(cls, dev):
+    """groups=2 with one offset group: the layers must fall back to zeroing a copy of the offsets, and every
+    gradient must match the oracle run on the zeroed offsets (the fixed axes' offset channels get none)."""
+    torch.manual_seed(11)
+    C, dims = 128, (3, 5, 6)
+    layer = getattr(M, cls)(C, C, 3, padding=1, groups=2).to(dev)
+    layer.checkpoint_deformation = False
+    with torch.no_grad():
+        layer.deform_params.weight.normal_(0, 0.02)
+        layer.deform_params.bias.normal_(0, 0.5)
+    x = torch.randn(1, C, *dims, device=dev)
+    gout = torch.randn(1, C, *dims, device=dev)
+    axes = layer._offset_axes
+    with torch.no_grad():
+        deformation = layer.deform_params(x)
+        offsets = deformation[:, :81].clone()
+        alpha = torch.sigmoid(deformation[:, 81:])
+        for a in range(3):
+            if not (axes >> a) & 1:
+                offsets[:, a::3] = 0
+    dc = layer.deform_conv
+    f = lambda t: t.detach().float().cpu()
+    e_out = cpu.conv3d_forward(f(x), f(offsets), f(alpha), f(dc.weight), f(dc.bias), 1, 1, 1, 2, 1)
+    e = cpu.conv3d_backward(f(gout), f(x), f(offsets), f(alpha), f(dc.weight), True, 1, 1, 1, 2, 1)
+    # through the layer: the deformation is a function of x too, so compare the operator's own gradients by
+    # cutting the graph at the deformation
+    xi = x.clone().requires_grad_(True)
+    captured = {}
+    hook = layer.deform_params.register_forward_hook(lambda mod, inp, out: captured.setdefault("d", out))
+    y = layer(xi)
+    hook.remove()
+    assert_close(y, e_out, 1e-4, 1e-5, cls + " out")
+    gd, gw_, gb_ = torch.autograd.grad(y, [captured["d"], dc.weight, dc.bias], gout)
+    goff, gmask = gd[:, :81], gd[:, 81:]
+    for a in range(3):
+        if not (axes >> a) & 1:
+            assert bool((goff[:, a::3] == 0).all())
+            e[1][:, a::3] = 0
+    sg = f(alpha) * (1 - f(alpha))
+    for n, a_, e_ in (("grad_offset", goff, e[1]), ("grad_mask", gmask, e[2] * sg), ("grad_weight", gw_, e[3]),
+                      ("grad_bias", gb_, e[4])):
+        assert_close(a_, e_, 1e-4, 1e-5 * max(1.0, e_.abs().max().item()), f"{cls} {n}")
+
+
 @pytest.mark.parametrize("cls", ["SpatialMDConv3d", "TemporalMDConv3d", "SpatialDConv3d", "TemporalDConv3d"])
 @pytest.mark.parametrize("channels", [64, 6])      # matrix-core kernels (axes fixed in the kernel) / direct kernels (copy)
 def test_spatial_and_temporal_layers_with_and_without_the_kernel_path(cls, channels, dev):

@@ -64,6 +64,30 @@ def test_group_norm_from_statistics_matches_torch(shape, groups, affine, dtype, 
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_group_norm_of_values_far_from_zero(dtype, dev):
+    """Activations whose mean is 30 standard deviations from zero: the variance is the small difference of
+    sum_sq / m and mean^2.  The per-channel sums are float32 (their rounding, amplified by mean^2 / var = 900,
+    bounds the result: 1e-3 relative is asked for here, where zero-mean data meets 1e-4); they are combined and
+    the difference is taken in double, so nothing more is lost.  Expected: F.group_norm in float64."""
+    g = torch.Generator().manual_seed(37)
+    shape, groups = (2, 32, 4, 6, 8), 4
+    x = (torch.randn(shape, generator=g) + 30.0).to(dtype)
+    gy = torch.randn(shape, generator=g).to(dtype)
+    xd = x.to(dev).requires_grad_(True)
+    stats = _ops.channel_stats(xd.detach())
+    y = _ops.group_norm_from_stats(xd, stats, None, None, groups, 1e-5)
+    y.backward(gy.to(dev))
+    xr = x.double().clone().requires_grad_(True)
+    ey = F.group_norm(xr, groups, None, None, 1e-5)
+    ey.backward(gy.double())
+    if dtype == torch.float32:
+        assert_close(y, ey.detach(), 1e-3, 1e-3, "group norm forward, mean 30")
+        assert_close(xd.grad, xr.grad, 1e-3, 1e-3 * xr.grad.abs().max().item(), "grad_x, mean 30")
+    else:
+        assert rel_l2(y, ey.detach()) < 2e-2 and rel_l2(xd.grad, xr.grad) < 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", ["dma_o320", "dma_o200_ragged", "small_c64", "depthwise", "generic"])
 @pytest.mark.parametrize("relu", [None, 1.5])
 def test_convolution_returns_the_sums_of_its_output(case, relu, dtype, dev):

@@ -69,6 +69,13 @@ def test_static_workspace_forward_matches_the_workspace_entry_point(dtype, dev):
         _lib.check(lib.d2c_conv3d_forward_static(ctypes.byref(desc), _p(x), _p(off), _p(m), _p(w), _p(b), _p(out),
                                                  stream), "d2c_conv3d_forward_static")
         torch.cuda.synchronize(dev)
+        # the call itself takes no device memory: once more (everything it could set up lazily is set up now) with
+        # the free memory of the device read on both sides
+        free_before = torch.cuda.mem_get_info(dev)[0]
+        _lib.check(lib.d2c_conv3d_forward_static(ctypes.byref(desc), _p(x), _p(off), _p(m), _p(w), _p(b), _p(out),
+                                                 stream), "d2c_conv3d_forward_static (second call)")
+        torch.cuda.synchronize(dev)
+        assert torch.cuda.mem_get_info(dev)[0] == free_before, "the static-workspace call changed the free device memory"
         xh, _, _, wh, bh = host
         exp = cpu.conv3d_forward(xh.float(), off.cpu(), m.cpu(), wh.float(), bh.float(), 1, 1, 1, case[4], case[5])
         if dtype == torch.float32:
