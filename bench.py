@@ -390,6 +390,9 @@ def main():
                          "the sampled columns that the offset / mask gradient kernel writes; 2 the same with the columns "
                          "written over the grad-column rows (no buffer of their own); 0 the grad-weight kernel "
                          "samples the input again")
+    ap.add_argument("--backward-slices", type=int, default=0,
+                    help="matrix-core backward of bfloat16 problems with several offset groups: number of slices over "
+                         "the offset groups (0 or 1: one pass over all groups; the description's backward_flags)")
     ap.add_argument("--grad-input-mode", type=int, default=1, choices=[0, 1],
                     help="matrix-core backward: 1 (default) grad-column rows through device memory, offset / mask "
                          "gradient and grad_input (from sample lists) as kernels of their own; 0 everything inside "
@@ -407,7 +410,6 @@ def main():
     from d2conv3d_amd import _lib
     lib = _lib.load()  # raises if the HIP library is missing: there is no fallback
     lib.d2c_set_grad_input_mode(args.grad_input_mode)
-    lib.d2c_set_grad_weight_mode(args.grad_weight_mode)
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     if args.workload == "c2_sizemap":
@@ -437,7 +439,9 @@ def main():
     if nd == 3:
         T_, H_, W_ = dims
         desc = _lib.Conv3dDesc(N, C, C, T_, H_, W_, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, groups, G, T_, H_, W_,
-                               code, code, 0, 1.0, args.offset_axes)
+                               code, code, 0, 1.0, args.offset_axes,
+                               {1: _lib.BWD_GW_COLUMNS, 2: _lib.BWD_GW_IN_PLACE, 0: _lib.BWD_GW_RESAMPLE}[args.grad_weight_mode]
+                               | _lib.bwd_slices(args.backward_slices))
         kind = "conv3d"
         algo = _lib.ALGO_NAMES[lib.d2c_conv3d_algo(ctypes.byref(desc))]
     else:
@@ -639,6 +643,7 @@ def main():
                                else "offsets tensor [N,3*K*G,T,H,W]"),
                    "offset_axes": args.offset_axes,
                    "grad_input_mode": args.grad_input_mode, "grad_weight_mode": args.grad_weight_mode,
+                   "backward_slices": args.backward_slices,
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "taps_outside_volume": taps,

@@ -22,7 +22,7 @@ EXPORTS = (
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
-    "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_set_grad_weight_mode", "d2c_last_error", "d2c_version",
+    "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_set_grad_weight_mode", "d2c_set_backward_slices", "d2c_last_error", "d2c_version",
     "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read", "d2c_profile_kernel_name",
     "d2c_size_map_offsets_forward", "d2c_size_map_offsets_backward",
     "d2c_conv3d_sized_forward_workspace_bytes", "d2c_conv3d_sized_backward_workspace_bytes",
@@ -37,7 +37,16 @@ class Conv3dDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "N", "Cin", "Cout", "D", "H", "W", "kd", "kh", "kw", "sd", "sh", "sw",
         "pd", "ph", "pw", "dd", "dh", "dw", "groups", "offset_groups", "Do", "Ho", "Wo",
-        "dtype", "aux_dtype", "epilogue")] + [("epilogue_scale", ctypes.c_float), ("offset_axes", ctypes.c_int32)]
+        "dtype", "aux_dtype", "epilogue")] + [("epilogue_scale", ctypes.c_float), ("offset_axes", ctypes.c_int32),
+                                               ("backward_flags", ctypes.c_int32)]
+
+
+# d2c_conv3d_desc::backward_flags
+BWD_GW_DEFAULT, BWD_GW_COLUMNS, BWD_GW_IN_PLACE, BWD_GW_RESAMPLE = 0, 1, 2, 3
+
+
+def bwd_slices(n):
+    return (int(n) & 0xff) << 8
 
 
 EPILOGUE_NONE, EPILOGUE_RELU = 0, 1
@@ -111,6 +120,7 @@ def load():
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int
     lib.d2c_set_grad_input_mode.argtypes, lib.d2c_set_grad_input_mode.restype = [ctypes.c_int], None
     lib.d2c_set_grad_weight_mode.argtypes, lib.d2c_set_grad_weight_mode.restype = [ctypes.c_int], None
+    lib.d2c_set_backward_slices.argtypes, lib.d2c_set_backward_slices.restype = [ctypes.c_int], None
     psm = ctypes.POINTER(SizeMapDesc)
     lib.d2c_size_map_offsets_forward.argtypes, lib.d2c_size_map_offsets_forward.restype = [psm, vp, vp, vp], ctypes.c_int
     lib.d2c_size_map_offsets_backward.argtypes, lib.d2c_size_map_offsets_backward.restype = [psm, vp, vp, vp, vp], ctypes.c_int

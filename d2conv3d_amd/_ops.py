@@ -129,7 +129,7 @@ class _DeformConv3dFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, offset, alpha, weight, bias, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, offset_groups,
-                relu_scale=0.0, want_stats=False, offset_axes=7):
+                relu_scale=0.0, want_stats=False, offset_axes=7, backward_flags=0):
         lib = _lib.load()
         input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
         alpha = alpha.contiguous() if alpha is not None else None
@@ -140,7 +140,7 @@ class _DeformConv3dFunction(torch.autograd.Function):
         desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, sd, sh, sw, pd, ph, pw, dd, dh, dw,
                                groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype],
                                _lib.EPILOGUE_RELU if relu_scale > 0 else _lib.EPILOGUE_NONE, float(relu_scale) or 1.0,
-                               int(offset_axes))
+                               int(offset_axes), int(backward_flags))
         _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d")
         dev = input.device
         out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
@@ -188,24 +188,25 @@ class _DeformConv3dFunction(torch.autograd.Function):
                                          _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
                                          _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d backward")
-        return (gx, goff, galpha, gw, gb) + (None,) * 14
+        return (gx, goff, galpha, gw, gb) + (None,) * 15
 
 
 def deform_conv3d(input, offset, alpha, weight, bias, stride_d, stride_h, stride_w, pad_d, pad_h, pad_w,
                   dilation_d, dilation_h, dilation_w, groups, offset_groups, relu_scale=0.0, want_stats=False,
-                  offset_axes=7):
+                  offset_axes=7, backward_flags=0):
     """deform_conv3d of dconv3d.h:188-226; `alpha` and `bias` may be None.  `relu_scale` > 0 fuses
     relu_scale * relu(.) into the store of the output (see _DeformConv3dFunction).  `want_stats` also returns the
     float32 [N, Cout, 2] sums and sums of squares of the stored output per (sample, channel), added up by the
     forward kernels where they store (the statistics a GroupNorm behind the convolution needs).  `offset_axes`: mask
     of the axes (1 z, 2 y, 4 x) the offsets displace along; the others are taken as zero and their gradient
-    channels come back zero (matrix-core kernels only, see conv3d_algo)."""
+    channels come back zero (matrix-core kernels only, see conv3d_algo).  `backward_flags`: the description's field
+    of that name (_lib.BWD_GW_* | _lib.bwd_slices(n)): how the backward pass trades workspace for time."""
     _check_common(3, input, offset, alpha, weight, bias, groups, offset_groups)
     input, offset, alpha, weight, bias = _unify(input, offset, alpha, weight, bias)
     return _DeformConv3dFunction.apply(
         input, offset, alpha, weight, bias, int(stride_d), int(stride_h), int(stride_w),
         int(pad_d), int(pad_h), int(pad_w), int(dilation_d), int(dilation_h), int(dilation_w),
-        int(groups), int(offset_groups), float(relu_scale), bool(want_stats), int(offset_axes))
+        int(groups), int(offset_groups), float(relu_scale), bool(want_stats), int(offset_axes), int(backward_flags))
 
 
 class _DeformConv3dSizedFunction(torch.autograd.Function):
@@ -522,6 +523,12 @@ def set_grad_weight_mode(mode):
     "resample" (the grad-weight kernel samples the input again)."""
     _lib.load().d2c_set_grad_weight_mode(mode if isinstance(mode, int)
                                          else {"columns": 1, "in_place": 2, "resample": 0}[mode])
+
+
+def set_backward_slices(n):
+    """Test hook: number of slices over the offset groups that the matrix-core backward pass of bfloat16 problems
+    runs in (0: the library's choice, 1: one pass over all groups)."""
+    _lib.load().d2c_set_backward_slices(int(n))
 
 
 def set_grad_input_mode(mode):

@@ -20,6 +20,7 @@ std::atomic<uint64_t> g_max_intermediate{1ull << 32};  // dconv3d_gpu.cu:12
 std::atomic<int> g_algo_override{D2C_ALGO_AUTO};
 std::atomic<int> g_gx_mode{1};
 std::atomic<int> g_gw_mode{1};
+std::atomic<int> g_bwd_slices{0};
 
 struct ProfState {
     std::mutex mu;
@@ -70,6 +71,7 @@ int static_scratch(void **out)
 
 int d2c_gx_mode() { return g_gx_mode.load(); }
 int d2c_col_weight_mode() { return g_gw_mode.load(); }
+int d2c_backward_slices() { return g_bwd_slices.load(); }
 
 void d2c_set_error(const char *fmt, ...)
 {
@@ -173,12 +175,13 @@ int32_t d2c_output_size(int32_t in, int32_t k, int32_t stride, int32_t pad, int3
 }
 
 const char *d2c_last_error(void) { return g_err; }
-int d2c_version(void) { return 1; }
+int d2c_version(void) { return 2; }
 uint64_t d2c_get_max_intermediate_elements(void) { return g_max_intermediate.load(); }
 void d2c_set_max_intermediate_elements(uint64_t m) { g_max_intermediate.store(m); }
 void d2c_set_algo_override(int algo) { g_algo_override.store(algo); }
 void d2c_set_grad_input_mode(int mode) { g_gx_mode.store(mode > 0 ? mode : 0); }
 void d2c_set_grad_weight_mode(int mode) { g_gw_mode.store(mode < 0 ? 0 : (mode > 2 ? 2 : mode)); }
+void d2c_set_backward_slices(int n) { g_bwd_slices.store(n < 0 ? 0 : n); }
 
 void d2c_profile_enable(int on)
 {
@@ -272,6 +275,8 @@ int d2c_conv3d_check(const d2c_conv3d_desc *q)
                 "tensor with 2^31 or more elements is not supported");
     D2C_REQUIRE(q->offset_axes >= 0 && q->offset_axes <= 7, "offset_axes must be a mask of the axes z, y, x (0 .. 7)");
     D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || q->epilogue == D2C_EPILOGUE_RELU, "unknown epilogue %d", q->epilogue);
+    D2C_REQUIRE((q->backward_flags & ~(D2C_BWD_GW_MASK | D2C_BWD_SLICES(0xff))) == 0, "unknown bits in backward_flags %d",
+                q->backward_flags);
     D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || (q->epilogue_scale > 0.f && q->epilogue_scale < 3.0e38f),
                 "epilogue_scale must be positive and finite");
     return D2C_OK;

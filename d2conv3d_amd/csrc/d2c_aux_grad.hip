@@ -46,6 +46,8 @@ struct AuxArgs {
     void *col;           // COL: the sampled columns [chunk][tap][mpad][BKC] (what the forward pass multiplied with W),
     long mpad;           //      rows of all `ntile` position tiles (zeros past the last position); or, in place of the
                          //      grad-column rows (`col` == `gcol`, which nobody reads after this kernel then): N*P rows
+    int g_lo, g_n;       // the offset groups [g_lo, g_lo + g_n) this launch works on (a slice of the backward pass;
+                         // `gcol` and `col` then point where chunk 0 WOULD start if the buffers held all chunks)
 };
 
 // Sum over the 8 lanes of a position without LDS traffic: neighbours of a quad, the other pair of the quad, then
@@ -90,7 +92,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     // cache still holds of them is read first (0.590 -> 0.576 ms).
     const int nblk = (a.ntile + kWavesPerBlock - 1) / kWavesPerBlock, nblk_p = (nblk + 7) / 8;
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    const int share = idx % a.nshare, g = s.G - 1 - idx / (nblk_p * a.nshare);
+    const int share = idx % a.nshare, g = a.g_lo + a.g_n - 1 - idx / (nblk_p * a.nshare);
     const int blk = ((xcd + 3 * g) & 7) * nblk_p + (idx / a.nshare) % nblk_p;
     if (blk >= nblk) return;
     const int tile = blk * kWavesPerBlock + wib;
@@ -339,14 +341,17 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 // channel count is a multiple of the chunk width.
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, const SampleLists *lists, void *col, bool col_in_place, hipStream_t st)
+                        void *goff, void *gmask, const SampleLists *lists, void *col, bool col_in_place, hipStream_t st,
+                        int g_lo, int g_n)
 {
+    if (g_n <= 0) { g_lo = 0; g_n = s.G; }
     const int ntile = (s.M + kMT - 1) / kMT;
     const int nshare = s.K < kTapSplit ? s.K : kTapSplit;
     // (with the size-map source `goff` is the fp32 accumulator of the size gradient)
     AuxArgs a{s, xcl, off, mask, gcol, s.ss.on ? nullptr : goff, gmask, s.ss.on ? (float *)goff : nullptr, ntile, nshare,
-              lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}, col, col_in_place ? (long)s.M : (long)ntile * kMT};
-    dim3 grid((unsigned)(8 * (((ntile + kWavesPerBlock - 1) / kWavesPerBlock + 7) / 8) * s.G * nshare));
+              lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}, col, col_in_place ? (long)s.M : (long)ntile * kMT,
+              g_lo, g_n};
+    dim3 grid((unsigned)(8 * (((ntile + kWavesPerBlock - 1) / kWavesPerBlock + 7) / 8) * g_n * nshare));
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
     D2cProfScope prof(D2C_PROF_BWD_AUX, st, "aux_grad_kernel");
@@ -379,6 +384,6 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     return d2c_check_launch("aux_grad_kernel");
 }
 template int d2c_aux_grad_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                         void *, void *, const SampleLists *, void *, bool, hipStream_t);
+                                         void *, void *, const SampleLists *, void *, bool, hipStream_t, int, int);
 template int d2c_aux_grad_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                        void *, void *, const SampleLists *, void *, bool, hipStream_t);
+                                        void *, void *, const SampleLists *, void *, bool, hipStream_t, int, int);

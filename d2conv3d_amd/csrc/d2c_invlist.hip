@@ -67,7 +67,7 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
 // compute units with wavefronts anyway (see d2c_gx_owner_launch).
 template <typename T, bool COMPACT, int EB>
 __global__ void __launch_bounds__(256, EB == 4 ? 4 : 2)
-gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
+gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, int c_lo, int c_n)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
     const int sub = threadIdx.x & 7, ci = threadIdx.x >> 3;       // 32 cubes per workgroup: 2 x 4 x 4 of them
@@ -76,10 +76,12 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
     // Workgroups are dealt round-robin to the 8 XCDs.  An XCD takes a contiguous range of the blocks of cubes
     // (neighbours in space share bins and grad-column rows in its L2) and, block by block, the channel chunks one
     // after the other: the chunks of one offset group walk the same lists, which then come from L2.
-    const int nblk = s.N * nbz * nby * nbx, nch = s.Cin / BKC;
+    // (c_lo, c_n: the channel chunks this launch works on -- a slice of the backward pass, `gcol` then points where
+    // chunk 0 WOULD start if the buffer held all chunks)
+    const int nblk = s.N * nbz * nby * nbx, nch = c_n;
     const int xcd = blockIdx.x & 7, uidx = blockIdx.x >> 3;
     const int bq = nblk >> 3, br = nblk & 7;
-    const int cidx = uidx % nch, bi = uidx / nch;                 // channel chunk, block within the XCD's range
+    const int cidx = c_lo + uidx % nch, bi = uidx / nch;          // channel chunk, block within the XCD's range
     if (bi >= bq + (xcd < br ? 1 : 0)) return;
     int blk = xcd * bq + (xcd < br ? xcd : br) + bi;
     const int bx = blk % nbx; blk /= nbx;
@@ -183,7 +185,7 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
 // it.  One 8-lane group per (overflow entry, channel chunk of its offset group).
 template <typename T>
 __global__ void __launch_bounds__(256)
-gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
+gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, int c_lo, int c_n)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
     const int novf = min(L.counts[L.nbins], L.ovf_cap);
@@ -199,6 +201,7 @@ gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl)
         const int z0 = bin % (s.D + 1) - 1; bin /= s.D + 1;
         const int g = bin % s.G, b = bin / s.G;
         const int cidx = (g * s.cpg) / BKC + jj;
+        if (cidx < c_lo || cidx >= c_lo + c_n) continue;      // (another slice's sample)
         const uint4 row = *reinterpret_cast<const uint4 *>(gcol + (((long)cidx * s.K + e.k) * s.M + (long)b * s.P + e.p) * BKC
                                                            + sub * VEC);
         const T *re = reinterpret_cast<const T *>(&row);
@@ -472,32 +475,34 @@ int d2c_lists_fill(const TiledShape &s, const void *off, const void *mask, const
 }
 
 template <typename T>
-int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st)
+int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st,
+                        int c_lo, int c_n)
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
+    if (c_n <= 0) { c_lo = 0; c_n = s.Cin / BKC; }
     D2cProfScope prof(D2C_PROF_GX_OWNER, st, "gx_owner_cube_kernel");
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
-    dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * (s.Cin / BKC)));    // see the kernel's unit mapping
+    dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * c_n));    // see the kernel's unit mapping
     // Eight rows in flight per group of lanes where several channel chunks of an offset group walk the same lists
     // (bfloat16): the lists then come from L2 and the rows' latency is what the kernel waits for (N=2, C=256, one
     // offset group: 0.30 -> 0.23 ms; 207360 positions: 1.78 -> 1.59 ms).  With one chunk per offset group (C=512 in 8
     // groups: 0.40 -> 0.45 ms) and for float problems (0.39 -> 0.41 ms) the wavefront lost per SIMD costs more.
     const int eb = (sizeof(T) == 2 && s.cpg / BKC >= 2) ? 8 : 4;
     if (eb == 8) {
-        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
-        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
     } else {
-        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
-        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
     }
     if (int rc = d2c_check_launch("gx_owner_kernel")) return rc;
     // the overflow entries, usually none (the kernel reads their number from device memory)
-    hipLaunchKernelGGL(gx_overflow_kernel<T>, dim3(512), dim3(256), 0, st, s, (const T *)gcol, L, gxcl);
+    hipLaunchKernelGGL(gx_overflow_kernel<T>, dim3(512), dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
     return d2c_check_launch("gx_overflow_kernel");
 }
-template int d2c_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const SampleLists &, float *, hipStream_t);
-template int d2c_gx_owner_launch<float>(const TiledShape &, const void *, const SampleLists &, float *, hipStream_t);
+template int d2c_gx_owner_launch<bf16_t>(const TiledShape &, const void *, const SampleLists &, float *, hipStream_t, int, int);
+template int d2c_gx_owner_launch<float>(const TiledShape &, const void *, const SampleLists &, float *, hipStream_t, int, int);
 
 // Depthwise case: grad_input from the sample lists, the channels-last grad_out and the tap-major weights.
 template <typename T>

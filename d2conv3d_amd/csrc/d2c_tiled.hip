@@ -20,10 +20,13 @@ bool d2c_tiled_bwd_single_pass(const TiledShape &s, int dtype);
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
-                              void *gmask, float *auxacc, hipStream_t st);
+                              void *gmask, float *auxacc, hipStream_t st, int phase = 3, int g_lo = 0, int g_n = 0);
+bool d2c_bwd_sliceable(const TiledShape &s, int dtype);
+int d2c_backward_slices();
 int d2c_bwd_data_split(const TiledShape &s, int dtype);
 template <typename T>
-int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st);
+int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists &L, float *gxcl, hipStream_t st,
+                        int c_lo = 0, int c_n = 0);
 void d2c_lists_ws(const TiledShape &s, int dtype, size_t *counts, size_t *entries, size_t *ovf);
 SampleLists d2c_lists_make(const TiledShape &s, int dtype, void *counts, void *entries, void *ovf);
 int d2c_lists_clear(const SampleLists &L, hipStream_t st);
@@ -34,13 +37,14 @@ int d2c_gx_mode();
 int d2c_col_weight_mode();
 template <typename T>
 int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *gcol,
-                        void *goff, void *gmask, const SampleLists *lists, void *col, bool col_in_place, hipStream_t st);
+                        void *goff, void *gmask, const SampleLists *lists, void *col, bool col_in_place, hipStream_t st,
+                        int g_lo = 0, int g_n = 0);
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                                 const void *mask, void *goutp, float *gwacc, void *gw, const void *col, long col_rows,
-                                hipStream_t st);
+                                hipStream_t st, int phase = 7, int jp_lo = 0, int jp_n = 0);
 bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype);
-size_t d2c_bwd_col_bytes(const TiledShape &s);
+size_t d2c_bwd_col_bytes(const TiledShape &s, int nchunks = 0);
 size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype);
 template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
 template <typename T> int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st);
@@ -72,7 +76,7 @@ d2c_conv3d_desc as_3d(const d2c_conv1d_desc &q)
     r.kd = 1; r.kh = 1; r.kw = q.k; r.sd = 1; r.sh = 1; r.sw = q.s; r.pd = 0; r.ph = 0; r.pw = q.p;
     r.dd = 1; r.dh = 1; r.dw = q.d; r.groups = q.groups; r.offset_groups = q.offset_groups;
     r.Do = 1; r.Ho = 1; r.Wo = q.Lo; r.dtype = q.dtype; r.aux_dtype = q.aux_dtype;
-    r.epilogue = D2C_EPILOGUE_NONE; r.epilogue_scale = 1.f; r.offset_axes = 0;
+    r.epilogue = D2C_EPILOGUE_NONE; r.epilogue_scale = 1.f; r.offset_axes = 0; r.backward_flags = 0;
     return r;
 }
 
@@ -496,13 +500,43 @@ bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
 
 // grad_weight as a matrix product over sampled columns that the offset / mask gradient kernel writes on its way
 // (needs that kernel to run: the caller wants grad_offset or grad_mask)
+// (0 sample again, 1 columns in a buffer of their own, 2 columns over the grad-column rows: the description's
+// backward_flags, or where those say nothing the process-wide test hook)
+int gw_mode(const d2c_conv3d_desc &q)
+{
+    const int f = q.backward_flags & D2C_BWD_GW_MASK;
+    return f == D2C_BWD_GW_DEFAULT ? d2c_col_weight_mode() : (f == D2C_BWD_GW_RESAMPLE ? 0 : f);
+}
 bool use_col_weight(const d2c_conv3d_desc &q, const TiledShape &s)
 {
-    return d2c_col_weight_mode() && use_aux_kernel(q, s) && d2c_bwd_weight_from_col(s, q.dtype);
+    return gw_mode(q) && use_aux_kernel(q, s) && d2c_bwd_weight_from_col(s, q.dtype);
 }
 // ... written over the grad-column rows (mode 2): grad_input is taken from those rows first, from sample lists
 // that a pass of their own files
-bool col_in_place(const d2c_conv3d_desc &q, const TiledShape &s) { return d2c_col_weight_mode() == 2 && use_col_weight(q, s); }
+bool col_in_place(const d2c_conv3d_desc &q, const TiledShape &s) { return gw_mode(q) == 2 && use_col_weight(q, s); }
+
+// The backward pass slice by slice over the offset groups (see d2c_bwd_sliceable): `gs` groups per slice of the
+// grad-column rows (0: not sliced), `cgs` groups per block of sampled columns that one launch of the grad-weight
+// product takes (a multiple of gs that holds an even number of channel chunks).
+struct BwdSlices {
+    int gs, cgs;
+};
+BwdSlices bwd_slices(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    BwdSlices r{0, 0};
+    // the description's backward_flags, or where those say nothing the process-wide test hook; by default the pass
+    // is not sliced (one pass over all groups is the faster one: the grad_input kernel needs the parallelism of all
+    // channel chunks at once)
+    int n = (q.backward_flags >> 8) & 0xff;
+    if (n == 0) n = d2c_backward_slices();
+    if (n < 2 || gw_mode(q) == 2 || d2c_gx_mode() < 1 || s.ss.on || !d2c_bwd_sliceable(s, q.dtype) ||
+        !d2c_tiled_bwd_data_supported(s, q.dtype) || !d2c_lists_supported(s))
+        return r;
+    if (n > s.G) n = s.G;
+    r.gs = (s.G + n - 1) / n;
+    r.cgs = ((r.gs * (s.cpg / 64)) % 2 == 0) ? r.gs : 2 * r.gs;
+    return r;
+}
 
 struct BwdWs {
     size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, gsacc, sm1, col, total;
@@ -525,11 +559,13 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     if (d2c_bwd_data_split(s, q.dtype) > 1 || !d2c_tiled_bwd_single_pass(s, q.dtype))
         w.total += d2c_align_up((size_t)s.N * s.G * s.K * s.P * (s.nd + 1) * sizeof(float));
     w.gcol = w.counts = w.entries = w.ovf = 0;
+    const BwdSlices sl = bwd_slices(q, s);
     if (use_lists(q, s) || use_aux_kernel(q, s)) {
         w.gcol = w.total;
         // (+ 64 rows behind the last one: what the last tile of the grad-weight product reads when the columns took
         // the rows' place)
-        w.total = w.gcol + d2c_align_up(((size_t)(s.Cin / bkc_of(q.dtype)) * s.K * s.M + 64) * bkc_of(q.dtype) * es);
+        const size_t chunks = sl.gs ? (size_t)sl.gs * (s.cpg / bkc_of(q.dtype)) : (size_t)(s.Cin / bkc_of(q.dtype));
+        w.total = w.gcol + d2c_align_up((chunks * s.K * s.M + 64) * bkc_of(q.dtype) * es);
     }
     if (use_lists(q, s)) {
         size_t c, en, ov;
@@ -545,7 +581,8 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.sm1 = w.total;       // ... and (size - 1) per axis
     if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
     w.col = w.total;       // sampled columns for the grad-weight product
-    if (use_col_weight(q, s) && !col_in_place(q, s)) w.total += d2c_align_up(d2c_bwd_col_bytes(s));
+    if (use_col_weight(q, s) && !col_in_place(q, s))
+        w.total += d2c_align_up(d2c_bwd_col_bytes(s, sl.cgs ? sl.cgs * (s.cpg / 64) : 0));
     return w;
 }
 
@@ -603,8 +640,66 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         s.ss.on = 2;
         off = sm1;
     }
-    bool gw_from_col = false, gw_in_place = false;
-    if (gx || goff || gmask) {
+    bool gw_from_col = false, gw_in_place = false, gw_done = false;
+    const BwdSlices sl = bwd_slices(q, s);
+    if ((gx || goff || gmask) && sl.gs > 0) {
+        // Slice by slice over the offset groups: the grad-column rows of a slice are made, read by the offset / mask
+        // gradient kernel (which files the slice's samples and writes its sampled columns) and by the grad_input
+        // kernel, and the grad-weight product takes the columns of a block of slices, before the next slice
+        // overwrites the rows: the buffers hold one slice (one block), and what a kernel reads was written a moment ago.
+        constexpr int BKC = 8 * Elem<T>::VEC;
+        const size_t es = sizeof(T);
+        float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
+        const bool lists = gx != nullptr, auxk = goff || gmask;
+        gw_from_col = gw && auxk && use_col_weight(q, s);
+        SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
+        if (lists) {
+            L = d2c_lists_make(s, Elem<T>::DT, base + l.counts, base + l.entries, base + l.ovf);
+            if (int rc = auxk ? d2c_lists_clear(L, st) : d2c_lists_build(s, off, mask, L, st)) return rc;
+        }
+        if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt, nullptr, base + l.gcol,
+                                                 nullptr, nullptr, (float *)(base + l.auxacc), st, 1))
+            return rc;
+        if (gw_from_col)
+            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+                                                       (float *)(base + l.gwacc), gw, base + l.col, 0, st, 1))
+                return rc;
+        const int cpc = s.cpg / BKC;
+        const long mpad = (long)((s.M + 63) / 64) * 64;
+        for (int g0 = 0; g0 < s.G; g0 += sl.gs) {
+            const int gn = s.G - g0 < sl.gs ? s.G - g0 : sl.gs;
+            const int c_lo = g0 * cpc, blk_lo = g0 / sl.cgs * sl.cgs;
+            // (the kernels address chunk c at c * K * rows * BKC elements from the pointer they get: the pointer that
+            // puts the slice's first chunk at the start of the buffer)
+            char *gcol_v = reinterpret_cast<char *>(reinterpret_cast<uintptr_t>(base + l.gcol)
+                                                    - (uintptr_t)((size_t)c_lo * s.K * s.M * BKC * es));
+            char *col_v = reinterpret_cast<char *>(reinterpret_cast<uintptr_t>(base + l.col)
+                                                   - (uintptr_t)((size_t)blk_lo * cpc * s.K * mpad * BKC * es));
+            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt, nullptr, gcol_v,
+                                                     nullptr, nullptr, (float *)(base + l.auxacc), st, 2, g0, gn))
+                return rc;
+            if (auxk)
+                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, gcol_v, goff, gmask, lists ? &L : nullptr,
+                                                    gw_from_col ? col_v : nullptr, false, st, g0, gn))
+                    return rc;
+            if (lists)
+                if (int rc = d2c_gx_owner_launch<T>(s, gcol_v, L, gxcl, st, c_lo, gn * cpc)) return rc;
+            const int g1 = g0 + gn;
+            if (gw_from_col && (g1 == s.G || g1 % sl.cgs == 0))
+                if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+                                                           (float *)(base + l.gwacc), gw, col_v, mpad, st, 2,
+                                                           blk_lo * cpc / 2, (g1 - blk_lo) * cpc / 2))
+                    return rc;
+        }
+        if (gx)
+            if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
+        if (gw_from_col) {
+            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+                                                       (float *)(base + l.gwacc), gw, base + l.col, 0, st, 4))
+                return rc;
+            gw_done = true;
+        }
+    } else if (gx || goff || gmask) {
         if (d2c_tiled_bwd_data_supported(s, q.dtype)) {
             float *gxcl = gx ? (float *)(base + l.gxcl) : nullptr;
             const bool lists = gx && use_lists(q, s);
@@ -669,7 +764,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                 return rc;
         }
     }
-    if (gw) {
+    if (gw && !gw_done) {
         if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
             if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc),

@@ -64,6 +64,9 @@ struct BwdDataArgs {
     // gradient (a sum over the channel chunks of a group) is accumulated with atomics in fp32 scratch arrays
     // laid out like goff / gmask, which a finishing kernel converts.
     float *auxoff, *auxmask;
+    // tiled_bwd_col32_kernel: the half-steps [h_lo, h_hi) of the step sequence this launch makes (a slice of the offset
+    // groups; h_hi == 0: all of them).  `gcolbuf` then points where chunk 0 WOULD start if the buffer held all chunks.
+    int h_lo, h_hi;
 };
 
 // NKG = k-groups of the reduction over output channels held in registers.
@@ -737,7 +740,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a
         for (int q = 0; q < 8; q++) woff[q] = lbase + (unsigned)(wrow * rowB + (((q * 2 + wh) ^ wsw) << 4));
     }
 
-    const int lo = (int)((long)S2 * blockIdx.z / gridDim.z), hi = (int)((long)S2 * (blockIdx.z + 1) / gridDim.z);
+    const int hs_lo = a.h_hi ? a.h_lo : 0, hs_n = (a.h_hi ? a.h_hi : S2) - hs_lo;
+    const int lo = hs_lo + (int)((long)hs_n * blockIdx.z / gridDim.z), hi = hs_lo + (int)((long)hs_n * (blockIdx.z + 1) / gridDim.z);
     if (lo >= hi) return;
     // (past the end of the range the last half-tile is requested again, into buffers nobody reads: the same number
     // of requests in every step, which the counted waits below rely on)
@@ -1228,6 +1232,9 @@ struct BwdWeightColArgs {
                          // of the grad-column rows (the last tile then reads into the next block, or the zeroed pad
                          // behind the last one: finite values that meet the zero tail of the grad_out copy)
     int otiles, nmain, main_len, ntail, tail_len;   // as in BwdWeightArgs
+    int jp_lo, jp_n;     // the pairs of channel chunks [jp_lo, jp_lo + jp_n) of every weight group this launch works on
+                         // (a slice of the backward pass; `col` then points where chunk 0 WOULD start if the buffer
+                         // held all chunks)
 };
 
 __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeightColArgs a)
@@ -1246,8 +1253,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ntile = (s.M + MT - 1) / MT;
-    const int npair = s.nchunk / NCH;
-    const int nstep = npair * s.K;
+    const int nstep = a.jp_n * s.K;
     const int nitem = s.groups * a.otiles * nstep;
     int item, t_lo, nmy, t_step;
     if ((int)blockIdx.x < nitem * a.nmain) {
@@ -1265,7 +1271,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
     }
     if (nmy <= 0) return;
     const int st = item % nstep, otile = (item / nstep) % a.otiles, wg = item / (nstep * a.otiles);
-    const int jp = st / s.K, k = st - jp * s.K;
+    const int jp = a.jp_lo + st / s.K, k = st % s.K;
     const int o_base = otile * NT + wave * 64;
     const bool mma_wave = o_base < s.og;
 
@@ -1668,10 +1674,14 @@ int d2c_bwd_data_split(const TiledShape &s, int dtype)
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
-                              void *gmask, float *auxacc, hipStream_t st)
+                              void *gmask, float *auxacc, hipStream_t st, int phase, int g_lo, int g_n)
 {
+    // phase: 1 = the weight re-layout (and the clears), 2 = the kernel, 3 = both.  g_n > 0 (grad-column product on
+    // tiled_bwd_col32_kernel only, see d2c_bwd_sliceable): the rows of the offset groups [g_lo, g_lo + g_n) only,
+    // `gcolbuf` pointing where chunk 0 would start.
     constexpr int BKC = 8 * Elem<T>::VEC;
     const int omax = d2c_bwd_pass_channels(Elem<T>::DT);
+    const bool sliced = g_n > 0;
     int nsplit = auxacc ? d2c_bwd_data_split(s, Elem<T>::DT) : 1;
     if (gcolbuf && !gxcl && !goff && !gmask) {
         // Only the grad-column product is wanted: every (tile, step) writes its own part of the result, so the
@@ -1685,7 +1695,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const bool c32 = s.og <= omax && bwd_col32_ok(d2c_bwd_ogk(s.og, Elem<T>::DT), s.og, Elem<T>::DT);
         const int MT = c32 ? kCol32MT : 32 * (8 / (BKC / 32));
         const long items = (long)((s.M + MT - 1) / MT) * s.groups;
-        const int S = s.nchunk * s.K * (c32 ? 2 : 1), reload = c32 ? 2 : 1;
+        const int S = (sliced ? g_n * (s.cpg / BKC) : s.nchunk) * s.K * (c32 ? 2 : 1), reload = c32 ? 2 : 1;
         long best = ((items + ncu - 1) / ncu) * (S + reload);
         nsplit = 1;
         for (int k = 2; k <= 16 && k <= S; k++) {
@@ -1698,10 +1708,12 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
     if ((nsplit > 1 || s.og > omax) && (goff || gmask) && auxacc) {
         auxoff = auxacc;
         auxmask = auxacc + n_off;
-        D2cProfScope prof(D2C_PROF_PACK, st);
-        d2c_fill_zero(auxacc, (size_t)(n_off + n_mask) * sizeof(float), st);
+        if (phase & 1) {
+            D2cProfScope prof(D2C_PROF_PACK, st);
+            d2c_fill_zero(auxacc, (size_t)(n_off + n_mask) * sizeof(float), st);
+        }
     }
-    if (gxcl) {
+    if (gxcl && (phase & 1)) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(gxcl, (size_t)s.N * s.vol * s.Cin * sizeof(float), st);
     }
@@ -1711,7 +1723,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const int ogn = s.og - o0 < omax ? s.og - o0 : omax;
         const int ogk = d2c_bwd_ogk(ogn, Elem<T>::DT);
         const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
-        {
+        if (phase & 1) {
             D2cProfScope prof(D2C_PROF_PACK, st);
             constexpr int R = 128 / (int)sizeof(T);
             const size_t lds = (size_t)R * ((size_t)kPackCh * s.K * sizeof(T) + 4);
@@ -1724,13 +1736,18 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                                    (T *)wt, s, ogk, o0, ogn, total);
         }
         if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
+        if (!(phase & 2)) continue;
+        const int cpc2 = 2 * (s.cpg / BKC);
         BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0,
-                      auxoff, auxmask};
+                      auxoff, auxmask, sliced ? g_lo * cpc2 * s.K : 0, sliced ? (g_lo + g_n) * cpc2 * s.K : 0};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
         const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
         if (col_only && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
             rc = launch_bwd_col32(a, nsplit, st);
+        } else if (sliced) {
+            d2c_set_error("grad-column product: slices are made by tiled_bwd_col32_kernel only");
+            return D2C_ERR_LAUNCH;
         } else if (col_only) {
             if (nkg <= 4) rc = launch_bwd_col<T, 4>(a, nsplit, st);
             else if (nkg <= 8) rc = launch_bwd_col<T, 8>(a, nsplit, st);
@@ -1744,7 +1761,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         }
         if (rc) return rc;
     }
-    if (auxoff) {
+    if (auxoff && (phase & 2)) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         if (goff) hipLaunchKernelGGL(aux_finish_kernel, dim3(grid1d(n_off)), dim3(256), 0, st, auxoff, goff, s.adt, n_off);
         if (gmask)
@@ -1831,24 +1848,36 @@ bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype)
 {
     return dtype == D2C_BF16 && s.nd == 3 && s.nchunk % kColChunks == 0;
 }
-// bytes of the sampled columns [chunk][tap][whole 64-position tiles][64]
-size_t d2c_bwd_col_bytes(const TiledShape &s)
+// bytes of the sampled columns [chunk][tap][whole 64-position tiles][64] of `nchunks` channel chunks (0: all)
+size_t d2c_bwd_col_bytes(const TiledShape &s, int nchunks)
 {
     const long ntile = (s.M + kWDT - 1) / kWDT;
-    return (size_t)(s.Cin / 64) * s.K * ntile * kWDT * 64 * 2;
+    return (size_t)(nchunks > 0 ? nchunks : s.Cin / 64) * s.K * ntile * kWDT * 64 * 2;
+}
+
+// The backward pass of this shape can run slice by slice over its offset groups (grad-column product, offset / mask
+// gradient, grad_input and the grad-weight product of one slice after the other, with buffers for the grad-column
+// rows and the sampled columns of ONE slice): bfloat16 problems on tiled_bwd_col32_kernel with one weight group.
+bool d2c_bwd_sliceable(const TiledShape &s, int dtype)
+{
+    return dtype == D2C_BF16 && s.nd == 3 && s.groups == 1 && s.G > 1 && s.og <= d2c_bwd_pass_channels(dtype) &&
+           bwd_col32_ok(d2c_bwd_ogk(s.og, dtype), s.og, dtype) && d2c_bwd_weight_from_col(s, dtype);
 }
 
 template <typename T>
 int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                                 const void *mask, void *goutp, float *gwacc, void *gw, const void *col, long col_rows,
-                                hipStream_t st)
+                                hipStream_t st, int phase, int jp_lo, int jp_n)
 {
+    // phase: 1 = the clear of the sums and the fragment-ordered copy of grad_out, 2 = the kernel, 4 = the conversion of
+    // the sums; 7 = all.  jp_n > 0 (product over the sampled columns only): the pairs of channel chunks
+    // [jp_lo, jp_lo + jp_n) of every weight group, `col` pointing where chunk 0 would start.
     const long nw = (long)s.Cout * s.cg * s.K;
     const int steps = s.nchunk * s.K;
     const int otiles = (s.og + 511) / 512;
     const int ntp = (s.M + kWMT - 1) / kWMT;     // tiles of the packed grad_out copy
     const int ntile = (s.M + kWDT - 1) / kWDT;   // position tiles of the kernel
-    {
+    if (phase & 1) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
         // (the channels-last input is followed by a 256-byte row of zeros, written by the kernel that packed it:
@@ -1867,18 +1896,23 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     if (ncu <= 0) return D2C_ERR_LAUNCH;
     bool from_col = false;
     if constexpr (sizeof(T) == 2) from_col = col != nullptr;
-    const long items = (long)(from_col ? steps / kColChunks : steps) * otiles * s.groups;
+    if (jp_n > 0 && !from_col) {
+        d2c_set_error("grad_weight: slices are made by tiled_bwd_weight_col_kernel only");
+        return D2C_ERR_LAUNCH;
+    }
+    if (jp_n <= 0) { jp_lo = 0; jp_n = s.nchunk / kColChunks; }
+    const long items = (long)(from_col ? jp_n * s.K : steps) * otiles * s.groups;
     const GwPieces pc = gw_pieces(items, ntile, ncu, from_col ? 4 : 1);
     const int nmain = pc.nmain, main_len = pc.main_len, ntail = pc.ntail, tail_len = pc.tail_len;
-    if (from_col) {
-        BwdWeightColArgs c{s, col, goutp, gwacc, col_rows, otiles, nmain, main_len, ntail, tail_len};
+    if (from_col && (phase & 2)) {
+        BwdWeightColArgs c{s, col, goutp, gwacc, col_rows, otiles, nmain, main_len, ntail, tail_len, jp_lo, jp_n};
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st, "tiled_bwd_weight_col_kernel");
         hipLaunchKernelGGL(tiled_bwd_weight_col_kernel, dim3((unsigned)(items * (nmain + ntail))), dim3(kThreads), 0, st, c);
         if (int rc = d2c_check_launch("tiled_bwd_weight_col_kernel")) return rc;
     }
     BwdWeightDmaArgs a{{s, gout, xcl, off, mask, goutp, gwacc, otiles, nmain, main_len, ntail, tail_len},
                        (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T))};
-    if (!from_col) {
+    if (!from_col && (phase & 2)) {
         const dim3 grid((unsigned)(items * (nmain + ntail)));
         bool aux16 = false;
         if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
@@ -1913,6 +1947,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         if (!ok) return D2C_ERR_LAUNCH;   // (d2c_allow_lds has set the error text)
     }
     if (int rc = d2c_check_launch("tiled_bwd_weight_dma_kernel")) return rc;
+    if (!(phase & 4)) return D2C_OK;
     D2cProfScope prof(D2C_PROF_PACK, st);
     constexpr int BKC = 8 * Elem<T>::VEC;
     const size_t cvt_lds = (size_t)kCvtRows * ((size_t)BKC * s.K * sizeof(T) + 16);
@@ -1952,9 +1987,10 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
 #define INST(T)                                                                                                    \
     template int d2c_tiled_bwd_data_launch<T>(const TiledShape &, const void *, const void *, const void *,        \
                                               const void *, const void *, void *, float *, void *, void *, void *, \
-                                              float *, hipStream_t);                                                        \
+                                              float *, hipStream_t, int, int, int);                                         \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
-                                                const void *, void *, float *, void *, const void *, long, hipStream_t); \
+                                                const void *, void *, float *, void *, const void *, long, hipStream_t, \
+                                                int, int, int);                                                     \
     template int d2c_tiled_unpack_gx<T>(const TiledShape &, const float *, void *, hipStream_t);                   \
     template int d2c_tiled_bias_grad<T>(const TiledShape &, const void *, void *, hipStream_t);
 INST(bf16_t)

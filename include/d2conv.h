@@ -65,6 +65,19 @@ enum {
 #define D2C_EPILOGUE_NONE 0
 #define D2C_EPILOGUE_RELU 1
 
+/* d2c_conv3d_desc::backward_flags: how the matrix-core backward pass of bfloat16 problems trades workspace for time.
+ * Both d2c_conv3d_backward_workspace_bytes() and d2c_conv3d_backward() read the field from the description they
+ * are given, so the size asked for and the call agree per description.  0 = the defaults. */
+#define D2C_BWD_GW_DEFAULT   0   /* grad_weight as a matrix product over sampled columns in a buffer of their own */
+#define D2C_BWD_GW_COLUMNS   1   /* the same, said explicitly */
+#define D2C_BWD_GW_IN_PLACE  2   /* the columns written over the grad-column rows: no buffer of their own */
+#define D2C_BWD_GW_RESAMPLE  3   /* no columns at all: the grad-weight kernel samples the input again */
+#define D2C_BWD_GW_MASK      3
+/* bits 8..15: number of slices over the offset groups that the backward pass runs in (0 or 1: one pass over all
+ * groups).  Buffers of grad-column rows and sampled columns then hold one slice; several offset groups, one weight
+ * group and 128 .. 512 output channels only (other descriptions ignore the bits). */
+#define D2C_BWD_SLICES(n)    (((n) & 0xff) << 8)
+
 typedef struct d2c_conv3d_desc {
     int32_t N, Cin, Cout;
     int32_t D, H, W;
@@ -90,6 +103,8 @@ typedef struct d2c_conv3d_desc {
      * fetch them.  Served by the matrix-core kernels only: other descriptions answer D2C_ERR_UNSUPPORTED (zero the
      * channels in a copy of the tensor instead). */
     int32_t offset_axes;
+    /* D2C_BWD_GW_* | D2C_BWD_SLICES(n); 0 = defaults.  Forward calls ignore it. */
+    int32_t backward_flags;
 } d2c_conv3d_desc;
 
 typedef struct d2c_conv1d_desc {
@@ -315,18 +330,21 @@ int d2c_dwconv3d_backward(const d2c_dwconv3d_desc *desc, const void *grad_out, c
  * One setting per process, for tests only (see d2c_set_algo_override). */
 void d2c_set_grad_input_mode(int mode);
 
-/* Hook for the matrix-core backward pass of bfloat16 problems: 1 (default)
- * lets the offset / mask gradient kernel write the sampled columns, over which
- * grad_weight then runs as a plain matrix product (the reference's formulation,
- * dconv3d_gpu.cu:1037-1088, with the column buffer filled by the kernel that has
- * the corner values in registers anyway); 2 is the same with the columns written
- * over the grad-column rows (no buffer of their own: the workspace of mode 0;
- * grad_input is then taken from the rows first, from sample lists that a pass
- * of their own files, which costs part of the gain); 0 makes the grad-weight
- * kernel sample the input again, which is also what happens whenever the caller
- * wants neither grad_offset nor grad_mask.  Workspace sizes depend on the mode.
- * One setting per process (see d2c_set_algo_override). */
+/* Test hooks, not for production callers (those set d2c_conv3d_desc::backward_flags, which wins over the hooks
+ * wherever it says something): the grad-weight path of the matrix-core backward pass of bfloat16 problems for
+ * descriptions whose backward_flags leave it at the default -- 1 (the library's default) lets the offset / mask
+ * gradient kernel write the sampled columns, over which grad_weight then runs as a plain matrix product (the
+ * reference's formulation, dconv3d_gpu.cu:1037-1088, with the column buffer filled by the kernel that has the
+ * corner values in registers anyway); 2 is the same with the columns written over the grad-column rows (no buffer
+ * of their own; grad_input is then taken from the rows first, from sample lists that a pass of their own files,
+ * which costs part of the gain); 0 makes the grad-weight kernel sample the input again, which is also what happens
+ * whenever the caller wants neither grad_offset nor grad_mask.  Workspace sizes depend on the mode.  One setting
+ * per process (see d2c_set_algo_override). */
 void d2c_set_grad_weight_mode(int mode);
+
+/* ... and the number of slices over the offset groups for descriptions whose backward_flags name none (see
+ * D2C_BWD_SLICES): 0 or 1 = one pass over all groups (the library's default), n >= 2 = n slices. */
+void d2c_set_backward_slices(int n);
 
 const char *d2c_last_error(void);
 int d2c_version(void);

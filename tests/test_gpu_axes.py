@@ -78,7 +78,7 @@ def test_fixed_offset_axes_refused_where_the_backward_would_leave_the_matrix_cor
     assert _ops.conv3d_algo(x, off, m, w, (1, 1, 1), (1, 1, 1), (1, 1, 1), 2, 1) == "mfma"
     assert _ops.conv3d_algo(x, off, m, w, (1, 1, 1), (1, 1, 1), (1, 1, 1), 2, 1, offset_axes=6) == "invalid"
     with pytest.raises(RuntimeError, match="offset_axes"):
-        d2c.deform_conv3d(x, off, m, w, None, 1, 1, 1, 1, 1, 2, offset_axes=6)
+        d2c.deform_conv3d(x, off, m, w, None, 1, 1, 1, 2, 1, offset_axes=6)
 
 
 @pytest.mark.parametrize("cls", ["SpatialMDConv3d", "TemporalMDConv3d"])

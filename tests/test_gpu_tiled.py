@@ -43,6 +43,11 @@ SHAPES = {
     # four chunks per weight group, 200 output channels: half of the grad-weight product's wavefronts have no output
     # channels and only move column tiles; the last slice of output channels is ragged
     "c256_G1_o200": (2, 256, 200, (3, 6, 7), 3, 1, 1, 1, 1, 1, True, True, 1.5),
+    # several offset groups of one or two channel chunks with 128 .. 512 output channels: the bfloat16 backward
+    # pass runs slice by slice over the offset groups (test_backward_in_slices_over_the_offset_groups)
+    "c256_G4_o128": (1, 256, 128, (3, 6, 7), 3, 1, 1, 1, 1, 4, True, True, 1.5),
+    "c384_G6_o384_nomask": (2, 384, 384, (2, 5, 6), 3, 1, 1, 1, 1, 6, False, False, 1.5),
+    "c384_G3_o384": (1, 384, 384, (3, 5, 7), 3, 1, 1, 1, 1, 3, True, True, 2.0),
     # channel-separated (groups == Cin == Cout)
     "dw64": (2, 64, 64, (4, 6, 7), 3, 1, 1, 1, 64, 1, True, True, 1.5),
     "dw96_G3_nomask": (1, 96, 96, (3, 5, 9), 3, 1, 1, 1, 96, 3, False, False, 1.0),
@@ -139,6 +144,37 @@ def test_grad_weight_from_columns_matches_resampling(name, wanted, dev):
     # the two differ by the rounding of the columns to bfloat16 at most (both round them before the product)
     assert rel_l2(got["columns"], got["resample"].float().cpu()) < 1e-2
     assert rel_l2(got["in_place"], got["columns"].float().cpu()) < 1e-3
+
+
+@pytest.mark.parametrize("name", ["c256_G2_o512_tail", "c256_G4_o128", "c384_G6_o384_nomask", "c384_G3_o384"])
+@pytest.mark.parametrize("wanted", ["all", "x", "w+offset", "x+w"])
+def test_backward_in_slices_over_the_offset_groups(name, wanted, dev):
+    # The bfloat16 backward pass slice by slice over the offset groups (buffers of grad-column rows and sampled columns
+    # for one slice / one block of slices): every number of slices against the oracle, and against the pass over all
+    # groups at once.  The cases cover slices of one and two groups, blocks of sampled columns that span two slices
+    # (one chunk per group), a last slice shorter than the others, and a grad_weight that samples again (no offset /
+    # mask gradient wanted) beside sliced grad_input.
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, torch.bfloat16, seed=9)
+    eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+    need = {"all": (1, 1, 1, 1, 1), "x": (1, 0, 0, 0, 0), "w+offset": (0, 1, 0, 1, 0), "x+w": (1, 0, 0, 1, 1)}[wanted]
+    names = ("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias")
+    res = {}
+    for n in (1, 2, 3, G, 0):
+        _ops.set_backward_slices(n)
+        try:
+            ts = [t.to(dev).requires_grad_(bool(r)) if t is not None else None for t, r in zip((x, off, m, w, b), need)]
+            d2c.deform_conv3d(*ts, s, p, d, groups, G).backward(gout.to(dev))
+            res[n] = [t.grad if (t is not None and r) else None for t, r in zip(ts, need)]
+        finally:
+            _ops.set_backward_slices(0)
+        for nm, a, e in zip(names, res[n], eg):
+            if a is not None:
+                assert rel_l2(a, e) < 2e-2, (n, nm, rel_l2(a, e))
+                assert_close(a, e, 2e-2, 2e-2 * e.abs().max().item(), f"{nm} in {n} slices")
+    for n in (2, 3, G, 0):
+        for nm, a, e in zip(names, res[n], res[1]):
+            if a is not None:
+                assert rel_l2(a, e.float().cpu()) < 1e-3, (n, nm)
 
 
 @pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_tail", "dw64", "dw96_G3_nomask",
