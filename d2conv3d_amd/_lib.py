@@ -16,7 +16,7 @@ ALGO_NAMES = {ALGO_GENERIC: "generic", ALGO_MFMA: "mfma", ALGO_DEPTHWISE: "depth
 
 # every symbol that include/d2conv.h declares
 EXPORTS = (
-    "d2c_output_size", "d2c_conv3d_check", "d2c_conv3d_algo",
+    "d2c_output_size", "d2c_conv3d_check", "d2c_conv3d_algo", "d2c_conv3d_packed_supported",
     "d2c_conv3d_forward_workspace_bytes", "d2c_conv3d_backward_workspace_bytes",
     "d2c_conv3d_forward", "d2c_conv3d_backward", "d2c_conv3d_forward_static", "d2c_static_workspace_bytes",
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
@@ -38,7 +38,11 @@ class Conv3dDesc(ctypes.Structure):
         "N", "Cin", "Cout", "D", "H", "W", "kd", "kh", "kw", "sd", "sh", "sw",
         "pd", "ph", "pw", "dd", "dh", "dw", "groups", "offset_groups", "Do", "Ho", "Wo",
         "dtype", "aux_dtype", "epilogue")] + [("epilogue_scale", ctypes.c_float), ("offset_axes", ctypes.c_int32),
-                                               ("backward_flags", ctypes.c_int32)]
+                                               ("backward_flags", ctypes.c_int32), ("deform_channels", ctypes.c_int32),
+                                               ("mask_activation", ctypes.c_int32)]
+
+
+MASK_ACTIVATIONS = {"none": 0, "linear": 0, "sigmoid": 1, "relu": 2, "tanh": 3}
 
 
 # d2c_conv3d_desc::backward_flags
@@ -113,6 +117,8 @@ def load():
         f = getattr(lib, f"d2c_{name}_backward")
         f.argtypes, f.restype = [p] + [vp] * 11 + [sz, vp], ctypes.c_int
     lib.d2c_conv3d_algo.argtypes, lib.d2c_conv3d_algo.restype = [p3], ctypes.c_int
+    lib.d2c_conv3d_packed_supported.argtypes = [p3, ctypes.POINTER(SizeMapDesc)]
+    lib.d2c_conv3d_packed_supported.restype = ctypes.c_int
     lib.d2c_conv3d_forward_static.argtypes, lib.d2c_conv3d_forward_static.restype = [p3] + [vp] * 7, ctypes.c_int
     lib.d2c_static_workspace_bytes.argtypes, lib.d2c_static_workspace_bytes.restype = [], sz
     lib.d2c_conv1d_algo.argtypes, lib.d2c_conv1d_algo.restype = [p1], ctypes.c_int

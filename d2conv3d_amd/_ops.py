@@ -303,6 +303,158 @@ def deform_conv3d_sized(input, size_raw, alpha, weight, bias, mode, activation, 
                                             dilation, int(groups), float(relu_scale), bool(want_stats))
 
 
+def _ptr_at(t, channel):
+    """Device pointer of t[:, channel] of a contiguous [N, C, *spatial] tensor (first sample)."""
+    per_channel = 1
+    for d in t.shape[2:]:
+        per_channel *= d
+    return ctypes.c_void_p(t.data_ptr() + channel * per_channel * t.element_size())
+
+
+class _DeformConv3dPackedFunction(torch.autograd.Function):
+    """The operator fed by the output of the layer's deformation branch as it is (network/layers.py:107-132,
+    :233-313): `deformation` [N, lead + G*K, Do, Ho, Wo] holds the offsets (lead = 3*G*K channels) or the raw size map
+    (lead = 1 | 2 | 3 channels, `mode` given) in front of the raw modulation values.  The kernels read both parts
+    inside that tensor (description field deform_channels) and apply the modulation activation where they read a
+    mask value (mask_activation); the backward pass writes one gradient tensor of the same shape, the modulation
+    part with respect to the raw values.  No split copies and no activation kernels in either direction."""
+
+    @staticmethod
+    def forward(ctx, input, deformation, weight, bias, lead, mask_act, mode, size_activation, stride, padding,
+                dilation, groups, offset_groups, relu_scale, want_stats, offset_axes, backward_flags):
+        lib = _lib.load()
+        input, deformation, weight = input.contiguous(), deformation.contiguous(), weight.contiguous()
+        bias = bias.contiguous() if bias is not None else None
+        N, Cin, D, H, W = input.shape
+        Cout, _, kd, kh, kw = weight.shape
+        Ctot = deformation.shape[1]
+        Do, Ho, Wo = deformation.shape[2:]
+        desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, *stride, *padding, *dilation, groups, offset_groups,
+                               Do, Ho, Wo, _DT[input.dtype], _DT[deformation.dtype],
+                               _lib.EPILOGUE_RELU if relu_scale > 0 else _lib.EPILOGUE_NONE, float(relu_scale) or 1.0,
+                               int(offset_axes), int(backward_flags), Ctot, int(mask_act))
+        sdesc = None
+        if mode is not None:
+            from .grid import size_map_desc
+            sdesc = size_map_desc(deformation, mode, (kd, kh, kw), dilation, size_activation)
+        sref = ctypes.byref(sdesc) if sdesc is not None else None
+        _lib.check(lib.d2c_conv3d_check(ctypes.byref(desc)), "deform_conv3d_packed")
+        dev = input.device
+        out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
+        stats = torch.empty((N, Cout, 2), dtype=torch.float32, device=dev) if want_stats else None
+        p_off, p_mask = _ptr_at(deformation, 0), _ptr_at(deformation, lead)
+        with torch.cuda.device(dev):
+            if want_stats:
+                nb = lib.d2c_conv3d_forward_stats_workspace_bytes(ctypes.byref(desc), sref)
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_forward_stats(ctypes.byref(desc), sref, _ptr(input), p_off, p_mask, _ptr(weight),
+                                                  _ptr(bias), _ptr(out), _ptr(stats), _ptr(ws), nb, _stream(dev))
+            elif sdesc is not None:
+                nb = lib.d2c_conv3d_sized_forward_workspace_bytes(ctypes.byref(desc), sref)
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_sized_forward(ctypes.byref(desc), sref, _ptr(input), p_off, p_mask, _ptr(weight),
+                                                  _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
+            else:
+                nb = lib.d2c_conv3d_forward_workspace_bytes(ctypes.byref(desc))
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), p_off, p_mask, _ptr(weight), _ptr(bias),
+                                            _ptr(out), _ptr(ws), nb, _stream(dev))
+        _lib.check(rc, "deform_conv3d_packed forward")
+        ctx.save_for_backward(input, deformation, weight, bias, out if relu_scale > 0 else None)
+        ctx.desc, ctx.sdesc, ctx.lead = desc, sdesc, lead
+        ctx.relu_scale = float(relu_scale)
+        if want_stats:
+            ctx.mark_non_differentiable(stats)
+            return out, stats
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out, _grad_stats=None):
+        lib = _lib.load()
+        input, deformation, weight, bias, out = ctx.saved_tensors
+        desc, sdesc = ctx.desc, ctx.sdesc
+        dev = input.device
+        grad_out = grad_out.contiguous().to(input.dtype)
+        if out is not None:
+            grad_out = torch.where(out > 0, grad_out * ctx.relu_scale, torch.zeros_like(grad_out))
+        need = ctx.needs_input_grad
+        gx = torch.empty_like(input) if need[0] else None
+        gdef = torch.empty_like(deformation) if need[1] else None
+        gw = torch.empty_like(weight) if need[2] else None
+        gb = torch.empty_like(bias) if (bias is not None and need[3]) else None
+        p_off, p_mask = _ptr_at(deformation, 0), _ptr_at(deformation, ctx.lead)
+        g_off = _ptr_at(gdef, 0) if gdef is not None else ctypes.c_void_p(0)
+        g_mask = _ptr_at(gdef, ctx.lead) if gdef is not None else ctypes.c_void_p(0)
+        with torch.cuda.device(dev):
+            if sdesc is not None:
+                nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_sized_backward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(grad_out), _ptr(input),
+                                                   p_off, p_mask, _ptr(weight), _ptr(gx), g_off, g_mask, _ptr(gw),
+                                                   _ptr(gb), _ptr(ws), nb, _stream(dev))
+            else:
+                nb = lib.d2c_conv3d_backward_workspace_bytes(ctypes.byref(desc))
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_backward(ctypes.byref(desc), _ptr(grad_out), _ptr(input), p_off, p_mask,
+                                             _ptr(weight), _ptr(gx), g_off, g_mask, _ptr(gw), _ptr(gb), _ptr(ws), nb,
+                                             _stream(dev))
+        _lib.check(rc, "deform_conv3d_packed backward")
+        return (gx, gdef, gw, gb) + (None,) * 13
+
+
+def deform_conv3d_packed_supported(input, deformation, weight, lead, mask_activation, mode, size_activation, stride,
+                                   padding, dilation, groups, offset_groups, offset_axes=7):
+    """Whether the kernels take the deformation tensor as it is for these arguments (matrix-core family, both
+    directions); where not, the caller splits it and applies the activation itself."""
+    if (not input.is_cuda or input.dtype not in (torch.float32, torch.bfloat16) or deformation.device != input.device
+            or mask_activation not in _lib.MASK_ACTIVATIONS):
+        return False
+    lib = _lib.load()
+    adt = deformation.dtype if (deformation.dtype == input.dtype or
+                                (input.dtype == torch.bfloat16 and deformation.dtype == torch.float32)) else None
+    if adt is None:
+        return False
+    N, Cin, D, H, W = input.shape
+    Cout, _, kd, kh, kw = weight.shape
+    Do, Ho, Wo = deformation.shape[2:]
+    desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, *stride, *padding, *dilation, groups, offset_groups,
+                           Do, Ho, Wo, _DT[input.dtype], _DT[adt], _lib.EPILOGUE_NONE, 1.0, int(offset_axes), 0,
+                           deformation.shape[1], _lib.MASK_ACTIVATIONS[mask_activation])
+    sdesc = None
+    if mode is not None:
+        from .grid import size_map_desc
+        sdesc = size_map_desc(deformation, mode, (kd, kh, kw), dilation, size_activation)
+    with torch.cuda.device(input.device):
+        return bool(lib.d2c_conv3d_packed_supported(ctypes.byref(desc), ctypes.byref(sdesc) if sdesc is not None else None))
+
+
+def deform_conv3d_packed(input, deformation, weight, bias, lead, mask_activation, stride, padding, dilation, groups,
+                         offset_groups, mode=None, size_activation="linear", relu_scale=0.0, want_stats=False,
+                         offset_axes=7, backward_flags=0):
+    """deform_conv3d / deform_conv3d_sized on the un-split output of the deformation branch: see
+    _DeformConv3dPackedFunction.  `lead`: channels in front of the modulation values (3*G*K offsets, or the size
+    map's 1 | 2 | 3 with `mode`); `mask_activation`: "sigmoid" | "relu" | "tanh" | "linear"."""
+    K = weight.shape[2] * weight.shape[3] * weight.shape[4]
+    GK = offset_groups * K
+    if deformation.dim() != 5 or deformation.shape[1] != lead + GK:
+        raise RuntimeError(f"deform_conv3d_packed: deformation must have {lead} + {GK} channels, got {tuple(deformation.shape)}")
+    if mode is None and lead != 3 * GK:
+        raise RuntimeError(f"deform_conv3d_packed: {3 * GK} offset channels expected in front of the modulation, got {lead}")
+    stand_in = deformation.new_empty(1)
+    _check_common(3, input, stand_in.expand((deformation.shape[0], 3 * GK) + tuple(deformation.shape[2:])),
+                  stand_in.expand((deformation.shape[0], GK) + tuple(deformation.shape[2:])), weight, bias, groups,
+                  offset_groups)
+    weight = weight.to(input.dtype)
+    bias = bias.to(input.dtype) if bias is not None else None
+    if not (deformation.dtype == input.dtype or (input.dtype == torch.bfloat16 and deformation.dtype == torch.float32)):
+        deformation = deformation.to(torch.float32 if input.dtype == torch.bfloat16 else input.dtype)
+    return _DeformConv3dPackedFunction.apply(
+        input, deformation, weight, bias, int(lead), _lib.MASK_ACTIVATIONS[mask_activation], mode, size_activation,
+        tuple(int(v) for v in stride), tuple(int(v) for v in padding), tuple(int(v) for v in dilation), int(groups),
+        int(offset_groups), float(relu_scale), bool(want_stats), int(offset_axes), int(backward_flags))
+
+
 class _GroupNormFromStats(torch.autograd.Function):
     """torch.nn.functional.group_norm on the output of a convolution whose forward kernels already added up the
     per-(sample, channel) sums (d2c_conv3d_forward_stats): d2c_group_norm_forward / _backward."""

@@ -277,6 +277,10 @@ int d2c_conv3d_check(const d2c_conv3d_desc *q)
     D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || q->epilogue == D2C_EPILOGUE_RELU, "unknown epilogue %d", q->epilogue);
     D2C_REQUIRE((q->backward_flags & ~(D2C_BWD_GW_MASK | D2C_BWD_SLICES(0xff))) == 0, "unknown bits in backward_flags %d",
                 q->backward_flags);
+    D2C_REQUIRE(q->deform_channels >= 0 && (long)q->N * q->deform_channels * P < (1L << 31),
+                "deform_channels must be non-negative and the deformation tensor below 2^31 elements");
+    D2C_REQUIRE(q->mask_activation >= D2C_MASK_ACT_NONE && q->mask_activation <= D2C_MASK_ACT_TANH,
+                "unknown mask_activation %d", q->mask_activation);
     D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || (q->epilogue_scale > 0.f && q->epilogue_scale < 3.0e38f),
                 "epilogue_scale must be positive and finite");
     return D2C_OK;
@@ -307,12 +311,20 @@ int d2c_conv1d_check(const d2c_conv1d_desc *q)
 }
 
 static int choose_algo_any_axes(const d2c_conv3d_desc &q, bool quiet);
+static int sized_check(const d2c_conv3d_desc *q, const d2c_size_map_desc *z);
 
 // fixed offset axes (the Spatial / Temporal layers) are served by the matrix-core kernels only
 static int choose_algo(const d2c_conv3d_desc &q, bool quiet)
 {
     const int a = choose_algo_any_axes(q, quiet);
     const bool fixed_axis = (q.offset_axes & 7) != 0 && (q.offset_axes & 7) != 7;
+    if (a >= 0 && (q.deform_channels > 0 || q.mask_activation != D2C_MASK_ACT_NONE) &&
+        (a != D2C_ALGO_MFMA || !d2c_tiled_packed_supported(q))) {
+        if (!quiet)
+            d2c_set_error("deform_channels / mask_activation are served by the matrix-core kernels only (split the "
+                          "deformation tensor and apply the activation in front of the call instead)");
+        return -1;
+    }
     if (a >= 0 && fixed_axis && (a != D2C_ALGO_MFMA || !d2c_tiled_axes_supported(q))) {
         if (!quiet)
             d2c_set_error("offset_axes = %d is served by the matrix-core kernels only (in both directions: offset "
@@ -336,6 +348,13 @@ static int choose_algo_any_axes(const d2c_conv3d_desc &q, bool quiet)
         return a;
     }
     return tiled_ok ? d2c_tiled_algo(q) : D2C_ALGO_GENERIC;
+}
+
+int d2c_conv3d_packed_supported(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
+{
+    if (!q || (z ? sized_check(q, z) : d2c_conv3d_check(q)) != D2C_OK) return 0;
+    return choose_algo(*q, true) == D2C_ALGO_MFMA && d2c_tiled_packed_supported(*q) &&
+           (!z || d2c_tiled_sized_supported(*q, true));
 }
 
 int d2c_conv3d_algo(const d2c_conv3d_desc *q)
@@ -443,6 +462,13 @@ static int sized_check(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
         d2c_set_error("size map: float32 or bfloat16 in the element type of the mask (aux_dtype)");
         return D2C_ERR_DTYPE;
     }
+    // a size map inside the layer's deformation tensor, or a modulation activation in the sampler: only where the
+    // matrix-core kernels form the offsets themselves (the expansion in front of the other kernels reads a map of its own)
+    if ((q->deform_channels > 0 || q->mask_activation != D2C_MASK_ACT_NONE) &&
+        !(choose_algo(*q, true) == D2C_ALGO_MFMA && d2c_tiled_sized_supported(*q, true))) {
+        d2c_set_error("deform_channels / mask_activation with a size map are served by the matrix-core kernels only");
+        return D2C_ERR_UNSUPPORTED;
+    }
     return D2C_OK;
 }
 static size_t expanded_offsets_bytes(const d2c_conv3d_desc &q)
@@ -544,6 +570,7 @@ int d2c_conv3d_corner_index(const d2c_conv3d_desc *q, const void *offset, int32_
 {
     if (int rc = d2c_conv3d_check(q)) return rc;
     if (!offset || !base || !flags) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (q->deform_channels > 0) { d2c_set_error("corner index: offsets in a tensor of their own only"); return D2C_ERR_UNSUPPORTED; }
     return d2c_generic_conv3d_corners(*q, offset, base, flags, (hipStream_t)stream);
 }
 

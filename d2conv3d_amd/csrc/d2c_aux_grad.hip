@@ -119,9 +119,8 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     float craw[4] = {0.f, 0.f, 0.f, 1.f};
     auto coords_issue = [&](int k) {
         if (cvalid) {
-            const long ab = (((long)cb * s.G + g) * s.K + k) * s.P + cp;
             tap_offsets_issue<AUX16, SIZED>(s, a.off, cb, g, k, cp, craw);
-            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, ab) : 1.f;
+            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, mask_index(s, cb, g, k, cp)) : 1.f;
         }
     };
     if (k_lo < k_hi) coords_issue(k_lo);
@@ -142,7 +141,8 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
             if (cvalid) {
                 tap_offsets_finish<AUX16, SIZED>(s, k, craw);
                 const float o0 = craw[0], o1 = craw[1], o2 = craw[2];
-                al = craw[3];
+                typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+                al = (s.mact && a.mask) ? mask_act<AT>(s.mact, craw[3]) : craw[3];
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
                 const Tap3<float> t = tiled_tap3(s, bz, by, bx, o0, o1, o2);
@@ -300,7 +300,6 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                     if (m < s.M) {
                         const float al = al_r[r];
                         const int b = m / s.P, p = m - b * s.P;
-                        const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
                         if (SIZED && a.gsize) {
                             // size-map source: d(offset_a) / d(size_a) = base_a[k_a]; the taps of a position add up
                             // (fp32 atomics into [N][3][P], finished by size_grad_finish_kernel)
@@ -311,14 +310,17 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                                     atomicAdd(a.gsize + ((long)b * 3 + ax) * s.P + p,
                                               s.ss.base[ax][kq[ax]] * (al * g_acc[r][ax]));
                         } else if (a.goff && s.nd == 3) {
-                            const long ob = 3 * ab - 2 * (long)p;
+                            const long ob = offset_index(s, b, g, k, p);
                             st_aux(a.goff, ob, s.adt, (s.axes & 1) ? al * g_acc[r][0] : 0.f);
                             st_aux(a.goff, ob + s.P, s.adt, (s.axes & 2) ? al * g_acc[r][1] : 0.f);
                             st_aux(a.goff, ob + 2 * (long)s.P, s.adt, (s.axes & 4) ? al * g_acc[r][2] : 0.f);
                         } else if (a.goff) {
-                            st_aux(a.goff, ab, s.adt, al * g_acc[r][2]);
+                            st_aux(a.goff, offset_index(s, b, g, k, p), s.adt, al * g_acc[r][2]);
                         }
-                        if (a.gmask) st_aux(a.gmask, ab, s.adt, g_acc[r][3]);
+                        // (with a modulation activation in the sampler: the gradient with respect to the raw value)
+                        if (a.gmask)
+                            st_aux(a.gmask, mask_index(s, b, g, k, p), s.adt,
+                                   s.mact ? g_acc[r][3] * mask_act_grad(s.mact, al) : g_acc[r][3]);
                     }
                 }
             }

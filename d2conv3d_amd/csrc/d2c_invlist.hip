@@ -47,7 +47,7 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
         if (!t.live) continue;
         InvEntry e;
         e.p = p; e.k = k; e.hz = t.hz; e.hy = t.hy; e.hx = t.hx;
-        e.alpha = mask ? ld_aux(mask, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt) : 1.f;
+        e.alpha = mask ? mask_act_rt(s.mact, ld_aux(mask, mask_index(s, b, g, k, p), s.adt), s.adt) : 1.f;
         e.pad0 = 0; e.pad1 = 0;
         lists_insert(L, bin_of(s, b, g, t.z0, t.y0, t.x0), e);
     }

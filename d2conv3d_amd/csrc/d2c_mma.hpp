@@ -219,7 +219,45 @@ struct TiledShape {
     unsigned keep;        // corners that can have a non-zero weight: with an axis fixed, those on its near plane
     SizeSrc ss;           // offsets formed from a size map instead of read from a tensor
     FastDiv dP, dHW, dW;  // divisions by P, Ho * Wo and Wo
+    // Elements between consecutive samples of the offsets tensor (or the size map) and of the mask, and of their
+    // gradients: G * K * nd * P and G * K * P for tensors of their own; the channel count of the layer's deformation
+    // tensor times P when both pointers point into that one tensor (d2c_conv3d_desc::deform_channels).
+    long obs, mbs;
+    int mact;             // activation the sampler applies to the mask values it reads (D2C_MASK_ACT_*)
 };
+
+// The modulation activation of the self-deforming layers (network/layers.py:107-120, dconv_native/modules.py:71-84),
+// applied where a mask value is read; rounded to the storage type AT like the tensor that torch's activation
+// would have written.
+template <typename AT> D2C_DEV float mask_act(int act, float v)
+{
+    switch (act) {
+    case D2C_MASK_ACT_SIGMOID: return rnd<AT>(1.f / (1.f + expf(-v)));
+    case D2C_MASK_ACT_RELU: return fmaxf(v, 0.f);
+    case D2C_MASK_ACT_TANH: return rnd<AT>(tanhf(v));
+    default: return v;
+    }
+}
+D2C_DEV float mask_act_rt(int act, float v, int adt)
+{
+    return adt == D2C_BF16 ? mask_act<bf16_t>(act, v) : mask_act<float>(act, v);
+}
+// d(activated) / d(raw) from the activated value, as torch's backward formulas take it
+D2C_DEV float mask_act_grad(int act, float a)
+{
+    switch (act) {
+    case D2C_MASK_ACT_SIGMOID: return a * (1.f - a);
+    case D2C_MASK_ACT_RELU: return a > 0.f ? 1.f : 0.f;
+    case D2C_MASK_ACT_TANH: return 1.f - a * a;
+    default: return 1.f;
+    }
+}
+// element index of mask (b, g, k, p) / of the first offset component of (b, g, k, p)
+D2C_DEV long mask_index(const TiledShape &s, int b, int g, int k, int p) { return (long)b * s.mbs + ((long)g * s.K + k) * s.P + p; }
+D2C_DEV long offset_index(const TiledShape &s, int b, int g, int k, int p)
+{
+    return (long)b * s.obs + ((long)g * s.K + k) * (s.nd == 3 ? 3 : 1) * s.P + p;
+}
 
 // With offsets fixed along some axes only the corners on the near side of those axes can have weight: 2^(free axes) of
 // them.  Slot j of those is the corner whose bits are the bits of j spread over the free axes (corner bit 2 = z,
@@ -255,17 +293,16 @@ D2C_DEV void tap_offsets_issue(const TiledShape &s, const void *off, int b, int 
             c[0] = f[0]; c[1] = f[s.P]; c[2] = f[2 * (long)s.P];
             return;
         }
-        const int nc = mode_channels(s.ss.mode);
 #pragma unroll
         for (int ax = 0; ax < 3; ax++) {
             const int ch = axis_channel(s.ss.mode, ax);
-            c[ax] = ch < 0 ? 0.f : ld_auxT<AUX16>(off, ((long)b * nc + ch) * s.P + p);
+            c[ax] = ch < 0 ? 0.f : ld_auxT<AUX16>(off, (long)b * s.obs + (long)ch * s.P + p);
         }
         return;
     }
-    const long ab = (((long)b * s.G + g) * s.K + k) * s.P + p;
+    const long ab = offset_index(s, b, g, k, p);
     if (s.nd == 3) {
-        const long ob = 3 * ab - 2 * (long)p;   // ((b*G+g)*K+k)*3*P + p
+        const long ob = ab;
         // (all three are requested, a fixed axis is dropped by a select: no branches between the loads)
         const float v0 = ld_auxT<AUX16>(off, ob), v1 = ld_auxT<AUX16>(off, ob + s.P);
         const float v2 = ld_auxT<AUX16>(off, ob + 2 * (long)s.P);
@@ -588,12 +625,12 @@ D2C_DEV void load_offsets(const TiledShape &s, const void *off, int b, int g, in
         return;
     }
     if (s.nd == 3) {
-        const long ob = (((long)b * s.G + g) * s.K + k) * 3 * s.P + p;
+        const long ob = offset_index(s, b, g, k, p);
         o0 = (s.axes & 1) ? ld_aux(off, ob, s.adt) : 0.f;
         o1 = (s.axes & 2) ? ld_aux(off, ob + s.P, s.adt) : 0.f;
         o2 = (s.axes & 4) ? ld_aux(off, ob + 2 * (long)s.P, s.adt) : 0.f;
     } else {
         o0 = 0.f; o1 = 0.f;
-        o2 = ld_aux(off, (((long)b * s.G + g) * s.K + k) * s.P + p, s.adt);
+        o2 = ld_aux(off, offset_index(s, b, g, k, p), s.adt);
     }
 }

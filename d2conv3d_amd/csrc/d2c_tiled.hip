@@ -77,6 +77,7 @@ d2c_conv3d_desc as_3d(const d2c_conv1d_desc &q)
     r.dd = 1; r.dh = 1; r.dw = q.d; r.groups = q.groups; r.offset_groups = q.offset_groups;
     r.Do = 1; r.Ho = 1; r.Wo = q.Lo; r.dtype = q.dtype; r.aux_dtype = q.aux_dtype;
     r.epilogue = D2C_EPILOGUE_NONE; r.epilogue_scale = 1.f; r.offset_axes = 0; r.backward_flags = 0;
+    r.deform_channels = 0; r.mask_activation = D2C_MASK_ACT_NONE;
     return r;
 }
 
@@ -108,6 +109,12 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0, con
     if (!(s.axes & 2)) s.keep &= 0x33u;     // y fixed: dy = 0
     if (!(s.axes & 4)) s.keep &= 0x55u;     // x fixed: dx = 0
     s.dP = make_fastdiv(s.P); s.dHW = make_fastdiv(q.Ho * q.Wo); s.dW = make_fastdiv(q.Wo);
+    // samples of the offsets (or the size map) and of the mask: tensors of their own, or both inside the layer's
+    // deformation tensor of `deform_channels` channels
+    s.obs = q.deform_channels > 0 ? (long)q.deform_channels * s.P
+                                  : (sz ? (long)mode_channels(sz->mode) * s.P : (long)s.G * s.K * (nd == 3 ? 3 : 1) * s.P);
+    s.mbs = q.deform_channels > 0 ? (long)q.deform_channels * s.P : (long)s.G * s.K * s.P;
+    s.mact = q.mask_activation;
     const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
     s.ogp = (s.og + nt - 1) / nt * nt;
     s.geo = make_geom(q);
@@ -325,7 +332,7 @@ __global__ void __launch_bounds__(256) size_grad_finish_kernel(TiledShape s, con
 #pragma unroll
             for (int ax = 0; ax < 3; ax++)
                 if (axis_channel(s.ss.mode, ax) == c) v += acc[(n * 3 + ax) * s.P + p];
-            const long ri = (n * nc + c) * s.P + p;
+            const long ri = n * s.obs + (long)c * s.P + p;
             v *= size_act_grad(s.ss.act, ld_auxT<AUX16>(raw, ri));
             if constexpr (AUX16) reinterpret_cast<bf16_t *>(graw)[ri] = f32_to_bf16(v);
             else reinterpret_cast<float *>(graw)[ri] = v;
@@ -338,7 +345,6 @@ __global__ void __launch_bounds__(256) size_grad_finish_kernel(TiledShape s, con
 template <bool AUX16>
 __global__ void __launch_bounds__(256) size_minus_one_kernel(TiledShape s, const void *raw, float *sm1)
 {
-    const int nc = mode_channels(s.ss.mode);
     const long total = (long)s.N * s.P;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         const long n = i / s.P, p = i - n * s.P;
@@ -346,7 +352,7 @@ __global__ void __launch_bounds__(256) size_minus_one_kernel(TiledShape s, const
 #pragma unroll
         for (int ax = 0; ax < 3; ax++) {
             const int ch = axis_channel(s.ss.mode, ax);
-            c[ax] = ch < 0 ? 0.f : ld_auxT<AUX16>(raw, (n * nc + ch) * s.P + p);
+            c[ax] = ch < 0 ? 0.f : ld_auxT<AUX16>(raw, n * s.obs + (long)ch * s.P + p);
         }
         size_minus_one<AUX16>(s, c);
 #pragma unroll
@@ -842,6 +848,17 @@ bool d2c_tiled_supported(const d2c_conv3d_desc &q)
 }
 
 int d2c_tiled_algo(const d2c_conv3d_desc &q) { return is_depthwise(q) ? D2C_ALGO_DEPTHWISE : D2C_ALGO_MFMA; }
+
+// Offsets and mask read inside the layer's deformation tensor, modulation activation in the sampler
+// (d2c_conv3d_desc::deform_channels, mask_activation): matrix-core kernels whose backward pass runs the offset / mask
+// gradient kernel.
+bool d2c_tiled_packed_supported(const d2c_conv3d_desc &q)
+{
+    if (is_depthwise(q) || !mfma_channels_ok(q)) return false;
+    const size_t P = (size_t)q.Do * q.Ho * q.Wo;
+    if (q.deform_channels > 0 && (size_t)2 * q.deform_channels * P * 4 >= (1ull << 32)) return false;
+    return use_aux_kernel(q, tiled_shape(q));
+}
 
 // Offsets held at zero along some axes (offset_axes) are honoured by the tiled kernels only: every part of the
 // backward pass has to stay on them too, or the direct kernels that take over would sample with the unzeroed offsets.

@@ -5,6 +5,9 @@
 
 bool d2c_tiled_supported(const d2c_conv3d_desc &q);
 int d2c_tiled_algo(const d2c_conv3d_desc &q);  // D2C_ALGO_MFMA or D2C_ALGO_DEPTHWISE
+// whether a description that reads offsets and mask inside one deformation tensor, or applies a modulation
+// activation in the sampler, is served (in both directions)
+bool d2c_tiled_packed_supported(const d2c_conv3d_desc &q);
 // whether a description with some offset axes fixed (offset_axes != 7) stays on the tiled kernels in both directions
 bool d2c_tiled_axes_supported(const d2c_conv3d_desc &q);
 size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q, bool with_stats = false);

@@ -180,7 +180,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
             if (cvalid) {
                 float o0, o1, o2;
                 load_offsets(s, a.off, cbatch, g, k, cp, o0, o1, o2);
-                al = a.mask ? ld_aux(a.mask, (((long)cbatch * s.G + g) * s.K + k) * s.P + cp, s.adt) : 1.f;
+                al = a.mask ? mask_act_rt(s.mact, ld_aux(a.mask, mask_index(s, cbatch, g, k, cp), s.adt), s.adt) : 1.f;
                 int bz, by, bx;
                 tap_base(s.geo, k, coz, coy, cox, bz, by, bx);
                 const Tap3<float> t = tiled_tap3(s, bz, by, bx, o0, o1, o2);
@@ -975,7 +975,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
     const long cstride = s.nd == 3 ? (long)s.P * (long)sizeof(AT) : 0;
     const long off_tap = (long)(s.nd == 3 ? 3 : 1) * s.P * (long)sizeof(AT);   // bytes per (sample, group, tap)
     const long mask_tap = (long)s.P * (long)sizeof(AT);
-    const unsigned off_sample = (unsigned)(s.G * s.K) * (unsigned)off_tap, mask_sample = (unsigned)(s.G * s.K) * (unsigned)mask_tap;
+    const unsigned off_sample = (unsigned)s.obs * (unsigned)sizeof(AT), mask_sample = (unsigned)s.mbs * (unsigned)sizeof(AT);
     float craw[4] = {0.f, 0.f, 0.f, 1.f};
     int cb_ = 0, cp_ = 0;
     bool cvalid = false;
@@ -991,11 +991,11 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
         if constexpr (SIZED) {
             tap_offsets_issue<AUX16, true>(s, a.off, cb_, g, k, cp_, craw);
         } else {
-            const char *ub = reinterpret_cast<const char *>(a.off) + ((long)(b_lo * s.G + g) * s.K + k) * off_tap;
+            const char *ub = reinterpret_cast<const char *>(a.off) + (long)b_lo * s.obs * (long)sizeof(AT) + ((long)g * s.K + k) * off_tap;
             coord_offsets_issue<AUX16>(ub, cstride, (unsigned)(cb_ - b_lo) * off_sample + (unsigned)cp_ * (unsigned)sizeof(AT), craw);
         }
         if (a.mask) {
-            const char *um = reinterpret_cast<const char *>(a.mask) + ((long)(b_lo * s.G + g) * s.K + k) * mask_tap;
+            const char *um = reinterpret_cast<const char *>(a.mask) + (long)b_lo * s.mbs * (long)sizeof(AT) + ((long)g * s.K + k) * mask_tap;
             craw[3] = ld_aux_at<AUX16>(um, (unsigned)(cb_ - b_lo) * mask_sample + (unsigned)cp_ * (unsigned)sizeof(AT));
         }
     };
@@ -1010,6 +1010,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
             for (int ax = 0; ax < 3; ax++) craw[ax] = rnd<AT>(sbase[ax] * craw[ax]);
         }
         coord_offsets_select(cc, craw);
+        if (s.mact && a.mask) craw[3] = mask_act<AT>(s.mact, craw[3]);
         const CornerRow r = corner_row(cc, ((float)__mul24(oz, s.geo.sd) + tapf[0]) + craw[0],
                                        ((float)__mul24(oy, s.geo.sh) + tapf[1]) + craw[1],
                                        ((float)__mul24(ox, s.geo.sw) + tapf[2]) + craw[2], craw[3], cb_ * s.vol, cvalid);

@@ -110,7 +110,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
             const int j = st / s.K, k = st - j * s.K;
             const int g = (wg * s.cg + j * BKC) / s.cpg;
             tap_offsets_issue<AUX16, SIZED>(s, a.off, cb, g, k, cp, craw);
-            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, (((long)cb * s.G + g) * s.K + k) * s.P + cp) : 1.f;
+            craw[3] = a.mask ? ld_auxT<AUX16>(a.mask, mask_index(s, cb, g, k, cp)) : 1.f;
         }
     };
     auto coords_finish = [&](int st, int buf) {
@@ -126,8 +126,10 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
                 const Tap3<float> t = tiled_tap3(s, bz, by, bx, craw[0], craw[1], craw[2]);
                 live = t.live;
                 idx = (cb * s.vol + (t.z0 * s.H + t.y0) * s.W + t.x0) * s.Cin;   // element offset of corner 000
+                typedef typename std::conditional<AUX16, bf16_t, float>::type AT;
+                const float al = (s.mact && a.mask) ? mask_act<AT>(s.mact, craw[3]) : craw[3];
 #pragma unroll
-                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * craw[3] : 0.f;
+                for (int c = 0; c < 8; c++) w[c] = ((live >> c) & 1u) ? tap3_weight(t, c) * al : 0.f;
             }
 #pragma unroll
             for (int c = 0; c < 8; c++) s_w[buf][c][tid] = w[c];
@@ -439,8 +441,8 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         PosC c{0.f, 0.f, 0.f, 0, 0u, 0u, false, 0.f, 0.f, 0.f};
         const int m0 = w.item >= 0 ? w.tile * MT : 0;
         const int b_lo = fdiv(m0, s.dP);
-        off_item = reinterpret_cast<const char *>(a.off) + (long)b_lo * s.G * s.K * off_tap;
-        mask_item = reinterpret_cast<const char *>(a.mask) + (long)b_lo * s.G * s.K * mask_tap;
+        off_item = reinterpret_cast<const char *>(a.off) + (long)b_lo * s.obs * (long)sizeof(AT);
+        mask_item = reinterpret_cast<const char *>(a.mask) + (long)b_lo * s.mbs * (long)sizeof(AT);
         const int m = m0 + ctid;
         c.valid = w.item >= 0 && m < s.M;
         if (c.valid) {
@@ -452,8 +454,8 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
             c.fx = (float)(ox * s.geo.sw - s.geo.pw);
             c.vox0 = b * s.vol;
             // (a lane without a position keeps offset 0: its loads read the tile's first position)
-            c.aoff = (unsigned)(b - b_lo) * (unsigned)(s.G * s.K) * (unsigned)off_tap + (unsigned)p * (unsigned)sizeof(AT);
-            c.moff = (unsigned)(b - b_lo) * (unsigned)(s.G * s.K) * (unsigned)mask_tap + (unsigned)p * (unsigned)sizeof(AT);
+            c.aoff = (unsigned)(b - b_lo) * ((unsigned)s.obs * (unsigned)sizeof(AT)) + (unsigned)p * (unsigned)sizeof(AT);
+            c.moff = (unsigned)(b - b_lo) * ((unsigned)s.mbs * (unsigned)sizeof(AT)) + (unsigned)p * (unsigned)sizeof(AT);
             if (SIZED && cwave) {
                 float t[3];
                 tap_offsets_issue<AUX16, true>(s, a.off, b, 0, 0, p, t);
@@ -496,6 +498,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 craw[0] = rnd<AT>(bz * c.s0); craw[1] = rnd<AT>(by * c.s1); craw[2] = rnd<AT>(bx * c.s2);
             }
             coord_offsets_select(cc, craw);
+            if (s.mact && a.mask) craw[3] = mask_act<AT>(s.mact, craw[3]);
             const CornerRow r = corner_row(cc, (c.fz + tz) + craw[0], (c.fy + ty) + craw[1], (c.fx + tx) + craw[2],
                                            craw[3], c.vox0, c.valid);
 #pragma unroll

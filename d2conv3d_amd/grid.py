@@ -148,11 +148,14 @@ def size_map_offsets(size_raw, mode, kernel_shape=(3, 3, 3), dilation=(1, 1, 1),
 
 
 def size_map_desc(size_raw, mode, kernel_shape, dilation, activation):
-    """The d2c_size_map_desc of a raw size map [N, channels(mode), *spatial]."""
+    """The d2c_size_map_desc of a raw size map [N, channels(mode), *spatial] (or of a tensor that holds the map in its
+    leading channels: only the batch size, the spatial shape and the element type are read)."""
     from . import _lib
     desc = _lib.SizeMapDesc()
     desc.N = size_raw.shape[0]
-    desc.P = int(size_raw[0, 0].numel())
+    desc.P = 1
+    for d in size_raw.shape[2:]:
+        desc.P *= int(d)
     desc.kd, desc.kh, desc.kw = kernel_shape
     desc.mode, desc.activation = _lib.SIZE_MODES[mode.lower()], _lib.SIZE_ACTIVATIONS[activation]
     desc.dtype = _lib.D2C_BF16 if size_raw.dtype == torch.bfloat16 else _lib.D2C_F32

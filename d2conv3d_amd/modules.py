@@ -73,6 +73,8 @@ class _DConvBase(nn.Module):
         self.deform_conv = DeformConv3d(in_channels, out_channels, kernel_size, stride, padding,
                                         dilation, groups, offset_groups, bias)
         self.activation = self._activations[activation] if isinstance(activation, str) else activation
+        # (a named activation can run inside the sampler, see _packed_forward)
+        self._activation_name = {"none": "linear"}.get(activation, activation) if isinstance(activation, str) else None
         if not isinstance(deform_param_op, nn.Module):
             self._init_deform_params(activation, init)
 
@@ -104,7 +106,57 @@ class DConv3d(_DConvBase):
     pass
 
 
+def _deformation_tensor(layer, input):
+    deform_input = input if layer.norm is None else layer.norm(input)
+    if layer.checkpoint_deformation and torch.is_grad_enabled():
+        return checkpoint(layer.deform_params, deform_input, use_reentrant=False)
+    return layer.deform_params(deform_input)
+
+
+def _packed_forward(layer, input, deformation, lead, mode=None, offset_axes=7):
+    """The operator on the un-split output of the deformation branch (`lead` channels of offsets or of the raw size
+    map, then the raw modulation values): the kernels read both parts where they lie and apply the modulation
+    activation themselves; no split copies, no activation kernel, one gradient tensor coming back.  Returns None
+    where the matrix-core kernels do not serve the call (the caller then splits and activates as the reference does)."""
+    from . import _ops
+    dc = layer.deform_conv
+    name = layer._activation_name
+    if name is None or not _ops.deform_conv3d_packed_supported(input, deformation, dc.weight, lead, name, mode,
+                                                             layer.size_activation, dc.stride, dc.padding, dc.dilation,
+                                                             dc.groups, dc.offset_groups, offset_axes):
+        return None
+    from . import _lib
+    flags = {"default": _lib.BWD_GW_DEFAULT, "columns": _lib.BWD_GW_COLUMNS, "in_place": _lib.BWD_GW_IN_PLACE,
+             "resample": _lib.BWD_GW_RESAMPLE}[dc.backward_memory] | _lib.bwd_slices(dc.backward_slices)
+    out = _ops.deform_conv3d_packed(input, deformation, dc.weight, dc.bias, lead, name, dc.stride, dc.padding,
+                                    dc.dilation, dc.groups, dc.offset_groups, mode, layer.size_activation,
+                                    float(dc.output_relu_scale) if dc.output_relu_scale else 0.0, dc.keep_output_stats,
+                                    offset_axes, flags)
+    if dc.keep_output_stats:
+        out, dc.last_output_stats = out
+    return out
+
+
+def _may_fuse(layer, input):
+    return (layer.fused_deformation is True and layer._activation_name is not None and input.is_cuda
+            and input.dtype in (torch.float32, torch.bfloat16))
+
+
 class MDConv3d(_DConvBase):
+    # True: the deformation branch's output goes to the operator as it is where the kernels take it (see
+    # _packed_forward); False: split + activation in front of the operator, as the reference does
+    fused_deformation = True
+
+    def forward(self, input):
+        if not _may_fuse(self, input):
+            return super().forward(input)
+        deformation = _deformation_tensor(self, input)
+        out = _packed_forward(self, input, deformation, self.offset_channels)
+        if out is not None:
+            return out
+        offset, alpha = torch.split(deformation, [self.offset_channels, self.alpha_channels], dim=1)
+        return self.deform_conv(input, offset, self.activation(alpha))
+
     def _deform_channels(self):
         self.offset_channels = 3 * self.offset_groups * self.num_kernel_points
         self.alpha_channels = self.offset_groups * self.num_kernel_points
@@ -148,11 +200,19 @@ class _AxesMixin:
     fixed_axes_in_kernel = True
 
     def forward(self, input):
-        deform_input = input if self.norm is None else self.norm(input)
-        if self.checkpoint_deformation and torch.is_grad_enabled():
-            offsets, alpha = checkpoint(super()._get_deformation, deform_input, use_reentrant=False)
+        if isinstance(self, MDConv3d) and self.fixed_axes_in_kernel and _may_fuse(self, input):
+            deformation = _deformation_tensor(self, input)
+            out = _packed_forward(self, input, deformation, self.offset_channels, offset_axes=self._offset_axes)
+            if out is not None:
+                return out
+            offsets, alpha = torch.split(deformation, [self.offset_channels, self.alpha_channels], dim=1)
+            alpha = self.activation(alpha)
         else:
-            offsets, alpha = super()._get_deformation(deform_input)
+            deform_input = input if self.norm is None else self.norm(input)
+            if self.checkpoint_deformation and torch.is_grad_enabled():
+                offsets, alpha = checkpoint(super()._get_deformation, deform_input, use_reentrant=False)
+            else:
+                offsets, alpha = super()._get_deformation(deform_input)
         if _fixed_axes_in_kernel(self, input, offsets, alpha):
             return self.deform_conv(input, offsets, alpha, offset_axes=self._offset_axes)
         offsets = offsets.clone()
@@ -200,6 +260,21 @@ def _sized_forward(layer, input):
     autograd graph of its expansion exist.  Returns None where that does not apply (CPU tensors, float64)."""
     if layer.fused_deformation is not True or not input.is_cuda or input.dtype == torch.float64:
         return None
+    if isinstance(layer, MDConv3d) and _may_fuse(layer, input):
+        # the size map and the raw modulation values where the deformation branch wrote them
+        deformation = _deformation_tensor(layer, input)
+        out = _packed_forward(layer, input, deformation, layer._size_channels, layer._mode)
+        if out is not None:
+            return out
+        size_raw, alpha = torch.split(deformation, [layer._size_channels, layer.alpha_channels], dim=1)
+        alpha = layer.activation(alpha)
+        dc = layer.deform_conv
+        out = deform_conv3d_sized(input, size_raw, alpha, dc.weight, dc.bias, layer._mode, layer.size_activation,
+                                  dc.stride, dc.padding, dc.dilation, dc.groups, output_relu=dc.output_relu_scale,
+                                  output_stats=dc.keep_output_stats)
+        if dc.keep_output_stats:
+            out, dc.last_output_stats = out
+        return out
     deform_input = input if layer.norm is None else layer.norm(input)
     if layer.checkpoint_deformation and torch.is_grad_enabled():
         size_raw, alpha = checkpoint(layer._get_size_and_alpha, deform_input, use_reentrant=False)

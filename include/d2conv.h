@@ -65,6 +65,12 @@ enum {
 #define D2C_EPILOGUE_NONE 0
 #define D2C_EPILOGUE_RELU 1
 
+/* d2c_conv3d_desc::mask_activation */
+#define D2C_MASK_ACT_NONE    0
+#define D2C_MASK_ACT_SIGMOID 1
+#define D2C_MASK_ACT_RELU    2
+#define D2C_MASK_ACT_TANH    3
+
 /* d2c_conv3d_desc::backward_flags: how the matrix-core backward pass of bfloat16 problems trades workspace for time.
  * Both d2c_conv3d_backward_workspace_bytes() and d2c_conv3d_backward() read the field from the description they
  * are given, so the size asked for and the call agree per description.  0 = the defaults. */
@@ -105,6 +111,19 @@ typedef struct d2c_conv3d_desc {
     int32_t offset_axes;
     /* D2C_BWD_GW_* | D2C_BWD_SLICES(n); 0 = defaults.  Forward calls ignore it. */
     int32_t backward_flags;
+    /* The deformation branch of the self-deforming layers (network/layers.py:107-132, dconv_native/modules.py:71-84)
+     * writes offsets and modulation into ONE tensor [N, deform_channels, Do, Ho, Wo] and the reference splits it and
+     * applies the modulation activation before the operator sees either part.  deform_channels > 0 lets the operator
+     * read that tensor where it lies: `offset` (or the size map of the d2c_conv3d_sized_* calls) and `mask` then
+     * point at their first channels INSIDE it, consecutive samples are deform_channels * Do*Ho*Wo elements apart in
+     * both, and grad_offset / grad_mask point likewise into one gradient tensor of that shape (channels of it
+     * that belong to neither are not written).  mask_activation != D2C_MASK_ACT_NONE makes the sampler apply that
+     * function to every mask value it reads (rounded to aux_dtype, like the tensor the reference's activation
+     * writes), and grad_mask comes back with respect to the raw values.  0 / 0: tensors of their own, mask used as it is.
+     * Matrix-core kernels only (and, in the backward call, one pass over the output channels of a weight group):
+     * other descriptions answer D2C_ERR_UNSUPPORTED. */
+    int32_t deform_channels;
+    int32_t mask_activation;
 } d2c_conv3d_desc;
 
 typedef struct d2c_conv1d_desc {
@@ -121,6 +140,11 @@ int32_t d2c_output_size(int32_t in, int32_t k, int32_t stride, int32_t pad, int3
 
 int d2c_conv3d_check(const d2c_conv3d_desc *desc);
 int d2c_conv3d_algo(const d2c_conv3d_desc *desc);
+/* 1 when a description with deform_channels > 0 and / or a mask_activation is served (forward and backward; with
+ * `size_map` != NULL: through the d2c_conv3d_sized_* calls), else 0: the caller then splits the deformation tensor
+ * and applies the activation itself, as the reference does (network/layers.py:107-120). */
+struct d2c_size_map_desc;
+int d2c_conv3d_packed_supported(const d2c_conv3d_desc *desc, const struct d2c_size_map_desc *size_map);
 size_t d2c_conv3d_forward_workspace_bytes(const d2c_conv3d_desc *desc);
 size_t d2c_conv3d_backward_workspace_bytes(const d2c_conv3d_desc *desc);
 
