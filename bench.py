@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the D2Conv3D operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap|dwconv|c3_norm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+                    [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap|dwconv|c3_norm|c3_layer]
 
 One step = one forward (+ one backward with all five gradients, except for
 the forward-only workload c1) of the modulated deformable convolution through
@@ -287,6 +288,70 @@ def bench_conv_act_norm(args):
     print(json.dumps(line))
 
 
+def bench_layer(args):
+    """A whole self-deforming layer at the size of workload c3: MDConv3d(512, 512, 3, padding=1, offset_groups=8) in
+    bfloat16 -- the stock Conv3d that predicts the deformation (network/layers.py:51-60; MIOpen), then the operator --
+    forward + backward through autograd.  Timed twice on the same GPU: with the deformation tensor handed to the
+    operator as it is (the sampler reads offsets and modulation inside it and applies the sigmoid; the default), and
+    with the reference's split + sigmoid in front of the operator (network/layers.py:107-120)."""
+    import torch
+    from d2conv3d_amd import modules
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    c = WORKLOADS["c3"]
+    torch.manual_seed(c["seed"])
+    layer = modules.MDConv3d(c["C"], c["C"], 3, padding=1, offset_groups=c["G"]).to(dev)
+    with torch.no_grad():     # offsets ~ N(0, 2) like the operator workload: a branch that predicts something
+        layer.deform_params.weight.normal_(0, 2.0 / (c["C"] * 27) ** 0.5)
+    layer = layer.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(c["seed"])
+    x = torch.randn(c["N"], c["C"], *c["dims"], generator=g).to(dev, torch.bfloat16).requires_grad_(True)
+    gout = torch.randn(c["N"], c["C"], *c["dims"], generator=g).to(dev, torch.bfloat16)
+
+    def step():
+        layer.zero_grad(set_to_none=True)
+        x.grad = None
+        layer(x).backward(gout)
+
+    def timed():
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    res, outs = {}, {}
+    for fused in (False, True):
+        layer.fused_deformation = fused
+        res[fused] = timed()
+        outs[fused] = layer(x).detach().float()
+    err = float((outs[True] - outs[False]).norm() / outs[False].norm())
+    # the operator's GEMM-equivalent flops plus those of the deformation branch's convolution (864 output channels)
+    f_op, _, _ = algorithmic("c3")
+    P = c["dims"][0] * c["dims"][1] * c["dims"][2]
+    f_branch = 2.0 * c["N"] * P * (4 * c["G"] * 27) * c["C"] * 27
+    value = 3 * (f_op + f_branch) / (res[True] * 1e-3) / 1e12
+    line = {
+        "metric": "MDConv3d layer fwd+bwd effective TFLOP/s (c3_layer) on 1 GPU", "value": round(value, 3),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res[True], 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "c3_layer: MDConv3d(512, 512, 3, padding=1, offset_groups=8) on [2, 512, 8, 30, 54], bf16, "
+                               "forward + backward through autograd (allocations included), the deformation branch's "
+                               "stock Conv3d (512 -> 864 channels) included",
+                   "deformation": "read by the operator inside the branch's output tensor, sigmoid in the sampler",
+                   "split_and_sigmoid_in_front_ms_per_step": round(res[False], 4),
+                   "relative_l2_fused_vs_split": err,
+                   "algorithmic_gflop": round(3 * (f_op + f_branch) / 1e9, 2)},
+        "roofline": None,
+    }
+    print(json.dumps(line))
+
+
 def bench_dwconv(args):
     """Plain depthwise conv3d (the reference's fast-depthwise-conv3d operator; backbone shape: 256 channels,
     8x56x56, 3x3x3, stride 1, padding 1, float32), forward + backward through the C ABI with pre-allocated
@@ -380,7 +445,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv", "c3_norm"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv", "c3_norm", "c3_layer"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--offset-axes", type=int, default=7,
                     help="mask of the axes the offsets displace along (1 z, 2 y, 4 x): 6 = the Spatial layers, 1 = the "
@@ -418,6 +483,8 @@ def main():
         return bench_dwconv(args)
     if args.workload == "c3_norm":
         return bench_conv_act_norm(args)
+    if args.workload == "c3_layer":
+        return bench_layer(args)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 

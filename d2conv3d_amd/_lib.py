@@ -20,7 +20,8 @@ EXPORTS = (
     "d2c_conv3d_forward_workspace_bytes", "d2c_conv3d_backward_workspace_bytes",
     "d2c_conv3d_forward", "d2c_conv3d_backward", "d2c_conv3d_forward_static", "d2c_static_workspace_bytes",
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
-    "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index",
+    "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index", "d2c_conv3d_sample",
+    "d2c_conv3d_offset_histogram",
     "d2c_get_max_intermediate_elements", "d2c_set_max_intermediate_elements",
     "d2c_set_algo_override", "d2c_set_grad_input_mode", "d2c_set_grad_weight_mode", "d2c_set_backward_slices", "d2c_last_error", "d2c_version",
     "d2c_profile_enable", "d2c_profile_reset", "d2c_profile_read", "d2c_profile_kernel_name",
@@ -124,6 +125,9 @@ def load():
     lib.d2c_conv1d_algo.argtypes, lib.d2c_conv1d_algo.restype = [p1], ctypes.c_int
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int
+    lib.d2c_conv3d_sample.argtypes, lib.d2c_conv3d_sample.restype = [p3, i32, vp, vp, vp, vp], ctypes.c_int
+    lib.d2c_conv3d_offset_histogram.argtypes = [p3, vp, ctypes.c_float, ctypes.c_float, i32, vp, vp]
+    lib.d2c_conv3d_offset_histogram.restype = ctypes.c_int
     lib.d2c_set_grad_input_mode.argtypes, lib.d2c_set_grad_input_mode.restype = [ctypes.c_int], None
     lib.d2c_set_grad_weight_mode.argtypes, lib.d2c_set_grad_weight_mode.restype = [ctypes.c_int], None
     lib.d2c_set_backward_slices.argtypes, lib.d2c_set_backward_slices.restype = [ctypes.c_int], None

@@ -635,6 +635,62 @@ def conv3d_corner_index(input_shape, offset, kernel_size, stride=(1, 1, 1), padd
     return base, flags
 
 
+def conv3d_sample(src, offset, kernel_size, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1), offset_groups=1):
+    """`src` [N, Cs, D, H, W] read at every sampling point of an offset field [N, G*3*K, Do, Ho, Wo] with the forward
+    pass's trilinear rule (d2c_conv3d_sample): [N, G*K*Cs, Do, Ho, Wo], channel (g*K + k)*Cs + c."""
+    lib = _lib.load()
+    if not src.is_cuda or src.dtype not in _DT or offset.device != src.device:
+        raise RuntimeError("conv3d_sample: CUDA tensors of float32 / float64 / bfloat16 on one device")
+    src, offset = src.contiguous(), offset.contiguous()
+    if src.dtype == torch.bfloat16:
+        offset = offset.to(torch.bfloat16 if offset.dtype == torch.bfloat16 else torch.float32)
+    else:
+        offset = offset.to(src.dtype)
+    N, Cs, D, H, W = src.shape
+    kd, kh, kw = kernel_size
+    K = kd * kh * kw
+    Do, Ho, Wo = offset.shape[2:]
+    if offset.shape[0] != N or offset.shape[1] != offset_groups * 3 * K:
+        raise RuntimeError(f"conv3d_sample: offset must be [N, {offset_groups * 3 * K}, ...], got {tuple(offset.shape)}")
+    G = offset_groups
+    desc = _lib.Conv3dDesc(N, G, G, D, H, W, kd, kh, kw, *stride, *padding, *dilation, 1, G, Do, Ho, Wo,
+                           _DT[src.dtype], _DT[offset.dtype])
+    out = torch.empty((N, G * K * Cs, Do, Ho, Wo), dtype=src.dtype, device=src.device)
+    with torch.cuda.device(src.device):
+        rc = lib.d2c_conv3d_sample(ctypes.byref(desc), Cs, _ptr(src), _ptr(offset), _ptr(out), _stream(src.device))
+    _lib.check(rc, "conv3d_sample")
+    return out
+
+
+def conv3d_offset_histogram(offset, kernel_size, offset_groups=1, bins=64, lo=-8.0, hi=8.0):
+    """int64 [3, bins + 2]: per axis (z, y, x) the histogram of an offset field [N, G*3*K, Do, Ho, Wo] over `bins`
+    equal-width bins of [lo, hi), with the counts below lo in column 0 and at or above hi in the last column
+    (d2c_conv3d_offset_histogram)."""
+    lib = _lib.load()
+    offset = offset.contiguous()
+    if not offset.is_cuda or offset.dtype not in _DT:
+        raise RuntimeError("conv3d_offset_histogram: a CUDA tensor of float32 / float64 / bfloat16")
+    kd, kh, kw = kernel_size
+    N = offset.shape[0]
+    Do, Ho, Wo = offset.shape[2:]
+    G = offset_groups
+    if offset.shape[1] != G * 3 * kd * kh * kw:
+        raise RuntimeError(f"conv3d_offset_histogram: offset must be [N, {G * 3 * kd * kh * kw}, ...], got {tuple(offset.shape)}")
+    dt = _DT[offset.dtype]
+    # (only the offsets' own shape matters; any input volume with this output size passes the check)
+    desc = _lib.Conv3dDesc(N, G, G, Do, Ho, Wo, 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, G, Do, Ho, Wo,
+                           dt if dt != _lib.D2C_BF16 else _lib.D2C_BF16, dt)
+    desc.kd, desc.kh, desc.kw = kd, kh, kw
+    desc.pd, desc.ph, desc.pw = kd // 2, kh // 2, kw // 2
+    desc.D, desc.H, desc.W = Do + (kd - 1) - 2 * (kd // 2), Ho + (kh - 1) - 2 * (kh // 2), Wo + (kw - 1) - 2 * (kw // 2)
+    hist = torch.empty((3, bins + 2), dtype=torch.int64, device=offset.device)
+    with torch.cuda.device(offset.device):
+        rc = lib.d2c_conv3d_offset_histogram(ctypes.byref(desc), _ptr(offset), float(lo), float(hi), int(bins),
+                                             _ptr(hist), _stream(offset.device))
+    _lib.check(rc, "conv3d_offset_histogram")
+    return hist
+
+
 def conv3d_algo(input, offset, alpha, weight, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
                 groups=1, offset_groups=1, offset_axes=7):
     """Name of the kernel family ("generic", "mfma", "depthwise") these arguments are served by; "invalid" when

@@ -574,6 +574,29 @@ int d2c_conv3d_corner_index(const d2c_conv3d_desc *q, const void *offset, int32_
     return d2c_generic_conv3d_corners(*q, offset, base, flags, (hipStream_t)stream);
 }
 
+int d2c_conv3d_sample(const d2c_conv3d_desc *q, int32_t src_channels, const void *src, const void *offset,
+                      void *out, void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!src || !offset || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    D2C_REQUIRE(src_channels > 0 && (long)q->N * src_channels * q->D * q->H * q->W < (1L << 31)
+                    && (long)q->N * q->offset_groups * q->kd * q->kh * q->kw * src_channels * q->Do * q->Ho * q->Wo < (1L << 31),
+                "sample: 1 or more source channels, tensors below 2^31 elements");
+    if (q->deform_channels > 0) { d2c_set_error("sample: offsets in a tensor of their own only"); return D2C_ERR_UNSUPPORTED; }
+    return d2c_generic_conv3d_sample(*q, src_channels, src, offset, out, (hipStream_t)stream);
+}
+
+int d2c_conv3d_offset_histogram(const d2c_conv3d_desc *q, const void *offset, float lo, float hi, int32_t nbins,
+                                uint64_t *hist, void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!offset || !hist) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    D2C_REQUIRE(lo < hi, "offset histogram: lo < hi");
+    if (q->deform_channels > 0) { d2c_set_error("offset histogram: offsets in a tensor of their own only"); return D2C_ERR_UNSUPPORTED; }
+    return d2c_generic_conv3d_offset_hist(*q, offset, lo, hi, nbins, reinterpret_cast<unsigned long long *>(hist),
+                                          (hipStream_t)stream);
+}
+
 static bool use_tiled1d(const d2c_conv1d_desc &q)
 {
     return g_algo_override.load() != D2C_ALGO_GENERIC && d2c_tiled1d_supported(q);

@@ -154,6 +154,10 @@ int d2c_generic_conv3d_backward(const d2c_conv3d_desc &q, const void *gout, cons
                                 void *gb, void *ws, hipStream_t st);
 int d2c_generic_conv3d_corners(const d2c_conv3d_desc &q, const void *off, int32_t *base, uint8_t *flags,
                                hipStream_t st);
+int d2c_generic_conv3d_sample(const d2c_conv3d_desc &q, int Cs, const void *src, const void *off, void *out,
+                              hipStream_t st);
+int d2c_generic_conv3d_offset_hist(const d2c_conv3d_desc &q, const void *off, float lo, float hi, int nbins,
+                                   unsigned long long *hist, hipStream_t st);
 int d2c_generic_conv1d_forward(const d2c_conv1d_desc &q, const void *x, const void *off, const void *mask,
                                const void *w, const void *bias, void *out, hipStream_t st);
 size_t d2c_generic_conv1d_backward_ws(const d2c_conv1d_desc &q);

@@ -278,6 +278,74 @@ generic_corners3d(Shape3 s, const void *off, int32_t *base, uint8_t *flags)
     }
 }
 
+// The sampler alone: a tensor `src` [N, Cs, D, H, W] (a ground-truth mask, say) read at every sampling point of
+// the description, out[b, (g*K + k)*Cs + c, p] = trilinear(src[b, c], pos(b, g, k, p)) with the forward pass's rules
+// (dconv3d_gpu.cu:48-109: 0 outside (-1, size), corners outside the volume read as 0), no modulation, no weights.
+template <typename CT>
+__global__ void __launch_bounds__(kBlock)
+generic_sample3d(Shape3 s, int Cs, const void *src, const void *off, void *out)
+{
+    const long total = (long)s.N * s.G * s.K * s.P;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long p = idx % s.P;
+        const int k = (int)((idx / s.P) % s.K);
+        const int g = (int)((idx / (s.P * s.K)) % s.G);
+        const int b = (int)(idx / (s.P * s.K * s.G));
+        const int ox = (int)(p % s.Wo), oy = (int)((p / s.Wo) % s.Ho), oz = (int)(p / ((long)s.Wo * s.Ho));
+        CT alpha;
+        const Tap3<CT> t = load_tap<CT>(s, off, nullptr, b, g, k, p, oz, oy, ox, alpha);
+        CT a[8];
+#pragma unroll
+        for (int cc = 0; cc < 8; cc++) a[cc] = tap3_weight(t, cc);
+        for (int c = 0; c < Cs; c++) {
+            CT v[8];
+            gather8<CT>(s, src, ((long)b * Cs + c) * s.vol, t, t.live, v);
+            CT res = 0;
+#pragma unroll
+            for (int cc = 0; cc < 8; cc++) res = d2c_fma<CT>(v[cc], a[cc], res);
+            st_as<CT>(out, (((long)b * s.G + g) * s.K + k) * Cs * s.P + (long)c * s.P + p, s.dt, res);
+        }
+    }
+}
+
+// Histogram of the offsets per axis: hist[axis][0] counts values below lo, [1 .. nbins] the equal-width bins of
+// [lo, hi), [nbins + 1] values at or above hi (and NaN).  Counted in LDS per workgroup, added to `hist` (zeroed by
+// the caller of the kernel) with one atomic per non-empty counter.
+constexpr int kHistMaxBins = 1024;
+template <typename CT>
+__global__ void __launch_bounds__(kBlock)
+generic_offset_hist3d(Shape3 s, const void *off, float lo, float hi, int nbins, unsigned long long *hist)
+{
+    extern __shared__ unsigned int s_h[];           // [3][nbins + 2]
+    const int nb2 = nbins + 2;
+    for (int i = threadIdx.x; i < 3 * nb2; i += blockDim.x) s_h[i] = 0u;
+    __syncthreads();
+    const long total = (long)s.N * s.G * s.K * 3 * s.P;
+    const float scale = (float)nbins / (hi - lo);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int axis = (int)((idx / s.P) % 3);
+        const float v = (float)ld_as<CT>(off, idx, s.adt);
+        int bin;
+        if (v < lo) bin = 0;
+        else if (!(v < hi)) bin = nbins + 1;
+        else {
+            bin = 1 + (int)((v - lo) * scale);
+            if (bin > nbins) bin = nbins;            // (rounding at the upper edge)
+        }
+        atomicAdd(&s_h[axis * nb2 + bin], 1u);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 3 * nb2; i += blockDim.x)
+        if (s_h[i]) atomicAdd(&hist[i], (unsigned long long)s_h[i]);
+}
+
+__global__ void __launch_bounds__(256) zero_u64_kernel(unsigned long long *p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0ull;
+}
+
 // =========================================================== 1-D operator
 struct Shape1 {
     int N, Cin, Cout, L, K, s, p, d, G, groups, Lo, dt, adt, quirks;
@@ -486,6 +554,40 @@ int d2c_generic_conv3d_backward(const d2c_conv3d_desc &q, const void *gout, cons
         if (int rc = d2c_check_launch("generic_bias_grad")) return rc;
     }
     return D2C_OK;
+}
+
+int d2c_generic_conv3d_sample(const d2c_conv3d_desc &q, int Cs, const void *src, const void *off, void *out,
+                              hipStream_t st)
+{
+    const Shape3 s = shape_of(q);
+    const long total = (long)s.N * s.G * s.K * s.P;
+    if (q.dtype == D2C_F64)
+        hipLaunchKernelGGL(generic_sample3d<double>, dim3(grid_for(total)), dim3(kBlock), 0, st, s, Cs, src, off, out);
+    else
+        hipLaunchKernelGGL(generic_sample3d<float>, dim3(grid_for(total)), dim3(kBlock), 0, st, s, Cs, src, off, out);
+    return d2c_check_launch("generic_sample3d");
+}
+
+int d2c_generic_conv3d_offset_hist(const d2c_conv3d_desc &q, const void *off, float lo, float hi, int nbins,
+                                   unsigned long long *hist, hipStream_t st)
+{
+    if (nbins < 1 || nbins > kHistMaxBins) {
+        d2c_set_error("offset histogram: 1 .. %d bins", kHistMaxBins);
+        return D2C_ERR_SHAPE;
+    }
+    const Shape3 s = shape_of(q);
+    const int n = 3 * (nbins + 2);
+    hipLaunchKernelGGL(zero_u64_kernel, dim3((n + 255) / 256), dim3(256), 0, st, hist, n);
+    const long total = (long)s.N * s.G * s.K * 3 * s.P;
+    long g = (total + (long)kBlock * 16 - 1) / ((long)kBlock * 16);     // ~16 values per thread
+    if (g < 1) g = 1;
+    if (g > 2048) g = 2048;
+    const size_t lds = (size_t)n * sizeof(unsigned int);
+    if (q.aux_dtype == D2C_F64)
+        hipLaunchKernelGGL(generic_offset_hist3d<double>, dim3((unsigned)g), dim3(kBlock), lds, st, s, off, lo, hi, nbins, hist);
+    else
+        hipLaunchKernelGGL(generic_offset_hist3d<float>, dim3((unsigned)g), dim3(kBlock), lds, st, s, off, lo, hi, nbins, hist);
+    return d2c_check_launch("generic_offset_hist3d");
 }
 
 int d2c_generic_conv3d_corners(const d2c_conv3d_desc &q, const void *off, int32_t *base, uint8_t *flags,

@@ -168,3 +168,21 @@ def tap_statistics(input_shape, offset, kernel_size, stride=(1, 1, 1), padding=(
     full = int((f == 255).sum())
     bits = sum(((f >> c) & 1).sum() for c in range(8))
     return {"taps": n, "dead": dead / n, "partial": (n - dead - full) / n, "corners_read": int(bits) / (8.0 * n)}
+
+
+def offset_histogram(offset, kernel_size=(3, 3, 3), offset_groups=1, bins=64, value_range=(-8.0, 8.0)):
+    """Histogram of an offset field per axis (z, y, x): int64 [3, bins + 2] with the counts below / at or above
+    `value_range` in the first / last column.  With tap_statistics, the debug output that the reference's trainer
+    expects from its missing `tools.hooks.oob_tracking` hook (trainer.py:99-101)."""
+    from . import _ops
+    return _ops.conv3d_offset_histogram(offset, tuple(kernel_size), offset_groups, bins, value_range[0], value_range[1])
+
+
+def sample_at_taps(src, offset, kernel_size=(3, 3, 3), stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1),
+                   offset_groups=1):
+    """`src` [N, Cs, D, H, W] read at every sampling point of the offset field, [N, G*K*Cs, Do, Ho, Wo]: what the
+    reference's modulation loss gets from grid_sample on a zero-padded ground-truth mask (loss/region.py:97-125),
+    with the sampler's own rules."""
+    from . import _ops
+    return _ops.conv3d_sample(src, offset, tuple(kernel_size), tuple(stride), tuple(padding), tuple(dilation),
+                              offset_groups)

@@ -198,6 +198,28 @@ int d2c_conv1d_backward(const d2c_conv1d_desc *desc, const void *grad_out, const
 int d2c_conv3d_corner_index(const d2c_conv3d_desc *desc, const void *offset, int32_t *base,
                             uint8_t *flags, void *stream);
 
+/*
+ * The sampler alone, for what samples other tensors at the operator's sampling points: the reference's modulation
+ * loss reads a ground-truth mask at every deformed tap with torch's grid_sample on a zero-padded copy
+ * (loss/region.py:97-125), which is the forward pass's trilinear rule on a one-channel input.
+ *   src [N, src_channels, D, H, W] (element type `dtype`), offset as in d2c_conv3d_forward,
+ *   out [N, G*K*src_channels, Do, Ho, Wo]: out[n, (g*K + k)*src_channels + c, p] = trilinear(src[n, c], pos(n, g, k, p)),
+ * 0 for positions outside (-1, size), corners outside the volume read as 0 (dconv3d_gpu.cu:48-109); no
+ * modulation, no weights.  Only N, D, H, W, the kernel / stride / padding / dilation fields, offset_groups, Do, Ho,
+ * Wo, dtype and aux_dtype of the description are used (Cin, Cout, groups must still pass d2c_conv3d_check).
+ */
+int d2c_conv3d_sample(const d2c_conv3d_desc *desc, int32_t src_channels, const void *src, const void *offset,
+                      void *out, void *stream);
+
+/*
+ * Histogram of an offset field per axis (the debug output that the reference's trainer expects from a hook its
+ * repository does not contain, trainer.py:99-101): hist[3][nbins + 2] of uint64 in device memory, overwritten;
+ * per axis (z, y, x): [0] values below lo, [1 .. nbins] the nbins equal-width bins of [lo, hi), [nbins + 1] values
+ * at or above hi (NaN included).  1 <= nbins <= 1024.
+ */
+int d2c_conv3d_offset_histogram(const d2c_conv3d_desc *desc, const void *offset, float lo, float hi,
+                                int32_t nbins, uint64_t *hist, void *stream);
+
 /* Accepted for interface parity; the library never materialises the column
  * buffer that this limit governs in the reference (dconv3d_gpu.cu:536-553). */
 uint64_t d2c_get_max_intermediate_elements(void);
