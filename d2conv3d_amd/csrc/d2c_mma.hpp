@@ -31,26 +31,89 @@ template <> struct Elem<float> {
     static constexpr int DT = D2C_F32;
 };
 
-template <typename T> D2C_DEV void mma_kgroup(f32x16 &acc, const uint4 &a, const uint4 &b);
-template <> D2C_DEV void mma_kgroup<bf16_t>(f32x16 &acc, const uint4 &a, const uint4 &b)
-{
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
-                                                  acc, 0, 0, 0);
-}
-template <> D2C_DEV void mma_kgroup<float>(f32x16 &acc, const uint4 &a, const uint4 &b)
-{
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
-}
-
 // Two floats -> packed bfloat16 pair (round to nearest even), low half first.
 D2C_DEV uint32_t pack_bf16x2(float lo, float hi)
 {
     f32x2 v = {lo, hi};
     bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
     return __builtin_bit_cast(uint32_t, r);
+}
+
+// ---- float problems on the bfloat16 matrix instruction ---------------------------------------------------------
+// The float MFMA (v_mfma_f32_32x32x2_f32) runs at 1/16 of the bfloat16 rate.  In the FORWARD kernels a float MFMA
+// operand therefore travels as TWO bfloat16 values per element, v ~ hi + lo with hi = bf16(v) and lo = bf16(v - hi)
+// (what is left is below 2^-16 |v|), in the 16 bytes that its four floats would take:
+// (hi0, hi1) (hi2, hi3) (lo0, lo1) (lo2, lo3).  One k-group (8 channels: 4 per lane half) is then two
+// v_mfma_f32_32x32x16_bf16 whose 16-deep reductions hold all four partial products of every element,
+// (hi + lo) * (hi' + lo'), summed in float32 by the matrix core: a quarter of the matrix-pipe time of the four float
+// instructions.  The producers of the forward operands (weight re-layout, sampled tile) write this form.
+// The BACKWARD kernels keep plain floats and the float instruction: the relative error of 4e-6 that the two-term
+// operands leave in a long sum is fine for the output (values of order 1 against 1e-4 relative / 1e-5 absolute) but
+// not for gradients whose elements reach 20 .. 400 and are held to the same absolute 1e-5
+// (-DD2C_F32_SPLIT_BACKWARD builds them on split operands all the same; -DD2C_F32_NATIVE_MFMA keeps the forward
+// kernels on the float instruction).
+#ifdef D2C_F32_NATIVE_MFMA
+constexpr bool kF32SplitFwd = false;
+#else
+constexpr bool kF32SplitFwd = true;
+#endif
+#ifdef D2C_F32_SPLIT_BACKWARD
+constexpr bool kF32SplitBwd = true;
+#else
+constexpr bool kF32SplitBwd = false;
+#endif
+D2C_DEV float bf16_residual(float v, uint32_t hi_bits)
+{
+    const float h = __uint_as_float(hi_bits);
+    // (an infinite value keeps its infinity in `hi` alone)
+    return (__float_as_uint(h) & 0x7fffffffu) == 0x7f800000u ? 0.f : v - h;
+}
+D2C_DEV uint4 split_f32x4(float v0, float v1, float v2, float v3)
+{
+    const uint32_t h01 = pack_bf16x2(v0, v1), h23 = pack_bf16x2(v2, v3);
+    return make_uint4(h01, h23,
+                      pack_bf16x2(bf16_residual(v0, h01 << 16), bf16_residual(v1, h01 & 0xffff0000u)),
+                      pack_bf16x2(bf16_residual(v2, h23 << 16), bf16_residual(v3, h23 & 0xffff0000u)));
+}
+// VEC consecutive reduction elements as the 16-byte operand vector the matrix instructions take
+// (SPLIT: float elements as two bfloat16 halves)
+template <typename T, bool SPLIT> D2C_DEV uint4 operand_vec(const T *e)
+{
+    if constexpr (sizeof(T) == 2) {
+        return make_uint4(e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16), e[4] | ((uint32_t)e[5] << 16),
+                          e[6] | ((uint32_t)e[7] << 16));
+    } else if constexpr (SPLIT) {
+        return split_f32x4(e[0], e[1], e[2], e[3]);
+    } else {
+        return make_uint4(__float_as_uint(e[0]), __float_as_uint(e[1]), __float_as_uint(e[2]), __float_as_uint(e[3]));
+    }
+}
+// ... of a vector already loaded as 16 bytes of T
+template <typename T, bool SPLIT> D2C_DEV uint4 operand_vec16(const uint4 &v)
+{
+    if constexpr (sizeof(T) == 4 && SPLIT)
+        return split_f32x4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+    else return v;
+}
+
+// One k-group of the reduction: acc += A (32 rows x 16 / 8 channels) * B (those channels x 32 columns)
+template <typename T, bool SPLIT> D2C_DEV void mma_kgroup(f32x16 &acc, const uint4 &a, const uint4 &b)
+{
+    if constexpr (sizeof(T) == 2) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                      acc, 0, 0, 0);
+    } else if constexpr (SPLIT) {
+        const uint4 bh = make_uint4(b.x, b.y, b.x, b.y), bl = make_uint4(b.z, b.w, b.z, b.w);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, bh),
+                                                      acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, bl),
+                                                      acc, 0, 0, 0);
+    } else {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
+    }
 }
 
 // acc[i] += w * v[i] over one 16-byte vector of channels (fp32 accumulation).
@@ -88,10 +151,8 @@ template <> struct VecAcc<float> {
         a[2] = fmaf(w, __uint_as_float(v.z), a[2]);
         a[3] = fmaf(w, __uint_as_float(v.w), a[3]);
     }
-    D2C_DEV uint4 pack() const
-    {
-        return make_uint4(__float_as_uint(a[0]), __float_as_uint(a[1]), __float_as_uint(a[2]), __float_as_uint(a[3]));
-    }
+    // (as an operand of the forward kernels' matrix instructions, see kF32SplitFwd)
+    D2C_DEV uint4 pack() const { return operand_vec<float, kF32SplitFwd>(a); }
 };
 
 template <typename T> D2C_DEV float elem_to_f32(T v);

@@ -268,10 +268,11 @@ __global__ void __launch_bounds__(256) pack_weight_fwd_kernel(const T *w, T *wp,
         const int j = st / s.K, k = st - j * s.K;
         const int ol = obg * 32 + (lane & 31);
         const int ch = j * BKC + (2 * kg + (lane >> 5)) * VEC;
-        T *dst = wp + i * VEC;
+        alignas(16) T tmp[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; e++)
-            dst[e] = ol < s.og ? w[((long)(wg * s.og + ol) * s.cg + ch + e) * s.K + k] : (T)0;
+            tmp[e] = ol < s.og ? w[((long)(wg * s.og + ol) * s.cg + ch + e) * s.K + k] : (T)0;
+        *reinterpret_cast<uint4 *>(wp + i * VEC) = operand_vec<T, kF32SplitFwd>(tmp);
     }
 }
 
@@ -314,7 +315,7 @@ __global__ void __launch_bounds__(256) pack_weight_fwd_lds_kernel(const T *w, T 
         for (int e = 0; e < VEC; e++) tmp[e] = src[e * s.K];
         const int lane = (khi & 1) * 32 + part * R + r;
         const long vi = ((((long)wg * S + j * s.K + k) * OBT + obg) * 4 + (khi >> 1)) * 64 + lane;
-        *reinterpret_cast<uint4 *>(wp + vi * VEC) = *reinterpret_cast<const uint4 *>(tmp);
+        *reinterpret_cast<uint4 *>(wp + vi * VEC) = operand_vec<T, kF32SplitFwd>(tmp);
     }
 }
 

@@ -118,7 +118,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                 const int o = (kg * 2 + (lane >> 5)) * VEC + i;
                 e[i] = (ok && kg < nkg && o < a.ogn) ? gp[(long)o * s.P] : (T)0;
             }
-            ga[kg] = *reinterpret_cast<uint4 *>(e);
+            ga[kg] = operand_vec<T, kF32SplitBwd>(e);
         }
     }
 
@@ -238,14 +238,14 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 #pragma unroll
                 for (int kg = 0; kg < NKG; kg++) {
                     const uint4 bf = *reinterpret_cast<const uint4 *>(wa[kg & 7] + (kg >> 3) * 256);
-                    mma_kgroup<T>(acc, ga[kg], bf);
+                    mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bf);
                 }
             } else {
 #pragma unroll
                 for (int kg = 0; kg < NKG; kg++) {
                     if (kg < nkg) {
                         const uint4 bf = *reinterpret_cast<const uint4 *>(wb + (((kg * 2 + wh) ^ wsw) << 4));
-                        mma_kgroup<T>(acc, ga[kg], bf);
+                        mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bf);
                     }
                 }
             }
@@ -550,7 +550,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 const int o = (kg * 2 + (lane >> 5)) * VEC + i;
                 e[i] = (ok && kg < nkg && o < a.ogn) ? gp[(long)o * s.P] : (T)0;
             }
-            ga[kg] = *reinterpret_cast<uint4 *>(e);
+            ga[kg] = operand_vec<T, kF32SplitBwd>(e);
         }
     }
 
@@ -620,7 +620,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                     if (kg + kPF < NKG)
                         bq[(kg + kPF) % (kPF + 1)] =
                             *reinterpret_cast<const uint4 *>(wb + woff[(kg + kPF) & 7] + ((kg + kPF) >> 3) * 256);
-                    mma_kgroup<T>(acc, ga[kg], bq[kg % (kPF + 1)]);
+                    mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bq[kg % (kPF + 1)]);
                 }
             } else {
                 const int wrow = cb * 32 + (lane & 31);
@@ -630,7 +630,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 for (int kg = 0; kg < NKG; kg++) {
                     if (kg < nkg) {
                         const uint4 bf = *reinterpret_cast<const uint4 *>(wr + (((kg * 2 + wh) ^ wsw) << 4));
-                        mma_kgroup<T>(acc, ga[kg], bf);
+                        mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bf);
                     }
                 }
             }
@@ -1092,8 +1092,20 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
         } else {
             // float: stored transposed ([channel][position]), one element per store
             unsigned char *tb = s_tile + dbuf * BKC * TRS + (ivec * VEC) * TRS;
+            if constexpr (kF32SplitBwd) {
+                // (as the two bfloat16 halves of a matrix-instruction operand: the 16 bytes of four consecutive
+                // positions hold their four `hi` values, then their four `lo` values)
+                unsigned char *tg = tb + (ipos >> 2) * 16 + (ipos & 3) * 2;
 #pragma unroll
-            for (int e = 0; e < VEC; e++) *reinterpret_cast<float *>(tb + e * TRS + ipos * 4) = va.a[e];
+                for (int e = 0; e < VEC; e++) {
+                    const bf16_t hi = f32_to_bf16(va.a[e]);
+                    *reinterpret_cast<bf16_t *>(tg + e * TRS) = hi;
+                    *reinterpret_cast<bf16_t *>(tg + e * TRS + 8) = f32_to_bf16(bf16_residual(va.a[e], (uint32_t)hi << 16));
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) *reinterpret_cast<float *>(tb + e * TRS + ipos * 4) = va.a[e];
+            }
         }
     };
 
@@ -1141,7 +1153,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
 #pragma unroll
             for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], ld[kq * 2 + ob], bf[cb]);
+                for (int cb = 0; cb < CB; cb++) mma_kgroup<T, kF32SplitBwd>(acc[ob][cb], ld[kq * 2 + ob], bf[cb]);
             if (kg + 4 < NKG) {
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i, kg + 4, ob);
@@ -1364,7 +1376,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
 #pragma unroll
                     for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                        for (int cb = 0; cb < CB; cb++) mma_kgroup<T>(acc[ob][cb], ld[kg * 2 + ob], bf[cb]);
+                        for (int cb = 0; cb < CB; cb++) mma_kgroup<T, kF32SplitBwd>(acc[ob][cb], ld[kg * 2 + ob], bf[cb]);
 #pragma unroll
                     for (int ob = 0; ob < OB; ob++) ld[kg * 2 + ob] = gn[(ob * NKGP + kg) * 64];
                     // (the requests stay behind the matrix instructions of their k-group)
@@ -1420,8 +1432,10 @@ template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt, TiledShape s, int ogk, int o0,
                                                               int ogn, long total)
 {
-    constexpr int BKC = 8 * Elem<T>::VEC;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
+    // one 16-byte vector of VEC consecutive output channels (the reduction of the grad-column product) per thread
+    for (long v = (long)blockIdx.x * blockDim.x + threadIdx.x; v < total / VEC; v += (long)gridDim.x * blockDim.x) {
+        const long i = v * VEC;
         const int oo = (int)(i % ogk);
         long r = i / ogk;
         const int cc = (int)(r % BKC); r /= BKC;
@@ -1429,7 +1443,11 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
         const int wg = (int)(r / (s.K * s.nchunk));
         const int cpc = s.cpg / BKC;   // same step order as tiled_bwd_data_kernel
         const int k = (st / cpc) % s.K, j = (st / (cpc * s.K)) * cpc + st % cpc;
-        wt[i] = oo < ogn ? w[((long)(wg * s.og + o0 + oo) * s.cg + j * BKC + cc) * s.K + k] : (T)0;
+        alignas(16) T tmp[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            tmp[e] = oo + e < ogn ? w[((long)(wg * s.og + o0 + oo + e) * s.cg + j * BKC + cc) * s.K + k] : (T)0;
+        *reinterpret_cast<uint4 *>(wt + i) = operand_vec<T, kF32SplitBwd>(tmp);
     }
 }
 
@@ -1472,7 +1490,7 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_lds_kernel(const T *w, T 
         for (int e = 0; e < VEC; e++) tmp[e] = reinterpret_cast<const T *>(smem + (ov * VEC + e) * rs)[cc * s.K + k];
         const int st = ((j / cpc) * s.K + k) * cpc + j % cpc;
         const long di = (((long)wg * s.K * s.nchunk + st) * BKC + cb * kPackCh + cc) * ogk + obk * R + ov * VEC;
-        *reinterpret_cast<uint4 *>(wt + di) = *reinterpret_cast<const uint4 *>(tmp);
+        *reinterpret_cast<uint4 *>(wt + di) = operand_vec<T, kF32SplitBwd>(tmp);
     }
 }
 
@@ -1601,7 +1619,7 @@ __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp,
                 const int b = (int)(m0 / s.P), p = (int)(m0 - (long)b * s.P);
                 v = *reinterpret_cast<const uint4 *>(gout + ((long)b * s.Cout + wg * s.og + ol) * s.P + p);
             }
-            reinterpret_cast<uint4 *>(goutp)[i] = v;
+            reinterpret_cast<uint4 *>(goutp)[i] = operand_vec16<T, kF32SplitBwd>(v);
             continue;
         }
 #pragma unroll
@@ -1614,7 +1632,7 @@ __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp,
             }
             e[q] = v;
         }
-        reinterpret_cast<uint4 *>(goutp)[i] = *reinterpret_cast<const uint4 *>(e);
+        reinterpret_cast<uint4 *>(goutp)[i] = operand_vec<T, kF32SplitBwd>(e);
     }
 }
 

@@ -204,7 +204,7 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
 #pragma unroll
             for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[kg][ob], bf[pb]);
+                for (int pb = 0; pb < PB; pb++) mma_kgroup<T, kF32SplitFwd>(acc[ob][pb], af[kg][ob], bf[pb]);
             if (st + 1 < st_hi) {
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++) af[kg][ob] = wfrag(st + 1, kg, ob);
@@ -238,7 +238,52 @@ __global__ void __launch_bounds__(kThreads) tiled_fwd_kernel(FwdArgs a)
     }
 
     // --- epilogue: bias, convert, store (32 consecutive positions per row of a block)
-    if (mma_wave) {
+    if (mma_wave && a.stats && !a.outacc) {
+        // the same stores, and on the way the sum and the sum of squares of the stored values per (sample, output
+        // channel), added into the [N][Cout][2] result (zeroed by the launcher): the 32 lanes that hold the positions
+        // of a channel add up first when they lie in one sample (they nearly always do), so that one lane adds
+        T *out = reinterpret_cast<T *>(a.out);
+        const T *bias = reinterpret_cast<const T *>(a.bias);
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) {
+            const int m = m0 + wave_p * WPOS + pb * 32 + (lane & 31);
+            const bool ok = m < s.M;
+            const int b = ok ? m / s.P : -1, p = ok ? m - b * s.P : 0;
+            const int b0 = __shfl(b, lane & 32, 64);                    // sample of the half's first position
+            const unsigned long long odd = __ballot(ok && b != b0);
+            const bool uniform = ((odd >> (lane & 32)) & 0xffffffffull) == 0ull;
+#pragma unroll
+            for (int ob = 0; ob < OB; ob++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int ol = otile * NT + wave_o * 64 + ob * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    const bool live = ok && ol < s.og;                  // (ol is uniform over the half)
+                    const int o = wg * s.og + ol;
+                    float fv = 0.f;
+                    if (live) {
+                        float v = acc[ob][pb][r];
+                        if (bias) v += elem_to_f32<T>(bias[o]);
+                        const T sv = f32_to_elem<T>(d2c_epilogue(v, s.act, s.act_scale));
+                        out[((long)b * s.Cout + o) * s.P + p] = sv;
+                        fv = elem_to_f32<T>(sv);
+                    }
+                    if (ol >= s.og) continue;
+                    if (uniform) {
+                        float q0 = fv, q1 = fv * fv;
+#pragma unroll
+                        for (int d = 1; d < 32; d <<= 1) { q0 += __shfl_xor(q0, d, 64); q1 += __shfl_xor(q1, d, 64); }
+                        if ((lane & 31) == 0 && b0 >= 0) {
+                            atomicAdd(a.stats + ((long)b0 * s.Cout + o) * 2, q0);
+                            atomicAdd(a.stats + ((long)b0 * s.Cout + o) * 2 + 1, q1);
+                        }
+                    } else if (live) {
+                        atomicAdd(a.stats + ((long)b * s.Cout + o) * 2, fv);
+                        atomicAdd(a.stats + ((long)b * s.Cout + o) * 2 + 1, fv * fv);
+                    }
+                }
+            }
+        }
+    } else if (mma_wave) {
         T *out = reinterpret_cast<T *>(a.out);
         const T *bias = reinterpret_cast<const T *>(a.bias);
 #pragma unroll
@@ -650,7 +695,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
 #pragma unroll
             for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                for (int pb = 0; pb < PB; pb++) mma_kgroup<T>(acc[ob][pb], af[kg][ob], bf[pb]);
+                for (int pb = 0; pb < PB; pb++) mma_kgroup<T, kF32SplitFwd>(acc[ob][pb], af[kg][ob], bf[pb]);
 #pragma unroll
             for (int q = 0; q < DPK; q++) {
                 const int i = kg * DPK + q;
@@ -1034,9 +1079,18 @@ int d2c_fwd_split(const TiledShape &s)
 
 // Whether the forward kernels of this shape add up per-channel statistics themselves (FwdArgs::stats): the
 // DMA-gather kernel, on samples of at least one position tile (a tile then meets at most two samples).
-bool d2c_fwd_fills_stats(const TiledShape &s) { return d2c_fwd_use_dma(s.og, s.M, s.groups) && s.P >= kDMT; }
+int d2c_fwd_split(const TiledShape &s);
+// The forward kernel of this shape adds the statistics of its output up while it stores: the DMA-gather kernel
+// (per position tile, see FwdArgs::stats) and the register-gather kernel when every workgroup holds whole sums (no
+// steps shared out between workgroups).
+bool d2c_fwd_fills_stats(const TiledShape &s)
+{
+    if (d2c_fwd_use_dma(s.og, s.M, s.groups)) return s.P >= kDMT;
+    return d2c_fwd_split(s) == 1;
+}
 size_t d2c_fwd_stats_ws(const TiledShape &s)
 {
+    if (!d2c_fwd_use_dma(s.og, s.M, s.groups)) return 0;     // (the register-gather kernel adds into the result itself)
     return d2c_align_up((size_t)((s.M + kDMT - 1) / kDMT) * 2 * s.Cout * 2 * sizeof(float));
 }
 
@@ -1051,8 +1105,12 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
     // the channels-last input is followed by a row of zeros (see forward_t)
     const unsigned zrow = (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T));
     FwdArgs a{s, xcl, off, mask, wp, bias, out, nsplit > 1 ? outacc : nullptr, nsplit, zrow, 0, 0, 0, 0, 1,
-              (dma && stats) ? stats_part : nullptr};
-    if (a.stats && d2c_fwd_out_tile(s.og, s.M, s.groups) != 512) {
+              stats ? (dma ? stats_part : (nsplit == 1 ? stats : nullptr)) : nullptr};
+    if (a.stats && !dma) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(a.stats, (size_t)s.N * s.Cout * 2 * sizeof(float), st);
+    }
+    if (a.stats && dma && d2c_fwd_out_tile(s.og, s.M, s.groups) != 512) {
         // (the 256-channel tile has two wavefronts per channel, which add into their slots)
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(a.stats, d2c_fwd_stats_ws(s), st);

@@ -88,13 +88,16 @@ def test_group_norm_of_values_far_from_zero(dtype, dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", ["dma_o320", "dma_o200_ragged", "small_c64", "depthwise", "generic"])
+@pytest.mark.parametrize("case", ["dma_o320", "dma_o200_ragged", "regs_c64_many_tiles", "small_c64", "depthwise", "generic"])
 @pytest.mark.parametrize("relu", [None, 1.5])
 def test_convolution_returns_the_sums_of_its_output(case, relu, dtype, dev):
     # (N, Cin, Cout, dims, groups): the matrix-core kernel that adds the sums up where it stores (wide weight groups
     # on at least 128 position tiles of 64: whole work items and items whose steps are shared out; N = 2 makes
-    # tiles that straddle the two samples), and the families that run the separate sums kernel behind the convolution
+    # tiles that straddle the two samples), the register-gather kernel on enough position tiles that no steps are
+    # shared out (it adds into the result itself; blocks of 32 positions that straddle the samples add lane by
+    # lane), and the families that run the separate sums kernel behind the convolution
     N, Cin, Cout, dims, groups = {"dma_o320": (2, 64, 320, (5, 29, 30), 1), "dma_o200_ragged": (2, 64, 200, (7, 25, 24), 1),
+                                  "regs_c64_many_tiles": (2, 64, 64, (8, 31, 33), 1),
                                   "small_c64": (2, 64, 64, (4, 6, 7), 1), "depthwise": (2, 64, 64, (4, 6, 7), 64),
                                   "generic": (2, 6, 10, (3, 5, 6), 1)}[case]
     if case == "generic" and dtype == torch.bfloat16:
