@@ -463,6 +463,10 @@ def main():
                          "gradient and grad_input (from sample lists) as kernels of their own; 0 everything inside "
                          "the grad-column kernel, grad_input scattered with atomics (the reference's formulation; for "
                          "comparison)")
+    ap.add_argument("--prepared", choices=["off", "train", "infer"], default="off",
+                    help="3-D matrix-core workloads: keep a prepared region (d2c_conv3d_*_prepared) the way a layer would: "
+                         "'train' = the backward call reuses the input copy its forward call made (weights change every "
+                         "step); 'infer' = forward calls also reuse the re-ordered weights")
     ap.add_argument("--expanded-offsets", action="store_true",
                     help="dynamic-dilation workloads (c2_*): expand the dilation map to an offsets tensor first "
                          "and time the ordinary operator on it, instead of handing the map to the operator")
@@ -532,7 +536,20 @@ def main():
         nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
         ws = torch.empty(max(nf, nb, 256), dtype=torch.uint8, device=dev)
 
+    prep = None
+    if args.prepared != "off" and nd == 3 and not sized:
+        npre = lib.d2c_conv3d_prepared_bytes(ctypes.byref(desc))
+        if npre:
+            prep = torch.empty(npre, dtype=torch.uint8, device=dev)
+    fwd_reuse = [0]
+
     def forward():
+        if prep is not None:
+            _lib.check(lib.d2c_conv3d_forward_prepared(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(prep),
+                                                       prep.numel(), fwd_reuse[0], p(ws), nf, cur[0]), "forward")
+            if args.prepared == "infer":
+                fwd_reuse[0] = _lib.REUSE_FORWARD_WEIGHTS
+            return
         if sized:
             _lib.check(lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), p(x), p(size), p(m), p(w),
                                                     p(b), p(out), p(ws), nf, cur[0]), "forward")
@@ -540,6 +557,11 @@ def main():
         _lib.check(f_fwd(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, cur[0]), "forward")
 
     def backward():
+        if prep is not None:
+            _lib.check(lib.d2c_conv3d_backward_prepared(ctypes.byref(desc), p(gout), p(x), p(off), p(m), p(w), p(gx), p(goff),
+                                                        p(gm), p(gw), p(gb), p(prep), prep.numel(), _lib.REUSE_INPUT, p(ws),
+                                                        nb, cur[0]), "backward")
+            return
         if sized:
             _lib.check(lib.d2c_conv3d_sized_backward(ctypes.byref(desc), ctypes.byref(sdesc), p(gout), p(x), p(size),
                                                      p(m), p(w), p(gx), p(gsize), p(gm), p(gw), p(gb), p(ws), nb,
@@ -710,7 +732,7 @@ def main():
                                else "offsets tensor [N,3*K*G,T,H,W]"),
                    "offset_axes": args.offset_axes,
                    "grad_input_mode": args.grad_input_mode, "grad_weight_mode": args.grad_weight_mode,
-                   "backward_slices": args.backward_slices,
+                   "backward_slices": args.backward_slices, "prepared_region": args.prepared if prep is not None else "off",
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "taps_outside_volume": taps,

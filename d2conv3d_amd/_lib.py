@@ -19,6 +19,7 @@ EXPORTS = (
     "d2c_output_size", "d2c_conv3d_check", "d2c_conv3d_algo", "d2c_conv3d_packed_supported",
     "d2c_conv3d_forward_workspace_bytes", "d2c_conv3d_backward_workspace_bytes",
     "d2c_conv3d_forward", "d2c_conv3d_backward", "d2c_conv3d_forward_static", "d2c_static_workspace_bytes",
+    "d2c_conv3d_prepared_bytes", "d2c_conv3d_forward_prepared", "d2c_conv3d_backward_prepared",
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index", "d2c_conv3d_sample",
     "d2c_conv3d_offset_histogram",
@@ -55,6 +56,7 @@ def bwd_slices(n):
 
 
 EPILOGUE_NONE, EPILOGUE_RELU = 0, 1
+REUSE_INPUT, REUSE_FORWARD_WEIGHTS, REUSE_BACKWARD_WEIGHTS = 1, 2, 4
 
 
 SIZE_MAX_K = 16
@@ -122,6 +124,11 @@ def load():
     lib.d2c_conv3d_packed_supported.restype = ctypes.c_int
     lib.d2c_conv3d_forward_static.argtypes, lib.d2c_conv3d_forward_static.restype = [p3] + [vp] * 7, ctypes.c_int
     lib.d2c_static_workspace_bytes.argtypes, lib.d2c_static_workspace_bytes.restype = [], sz
+    lib.d2c_conv3d_prepared_bytes.argtypes, lib.d2c_conv3d_prepared_bytes.restype = [p3], sz
+    lib.d2c_conv3d_forward_prepared.argtypes = [p3] + [vp] * 6 + [vp, sz, i32, vp, sz, vp]
+    lib.d2c_conv3d_forward_prepared.restype = ctypes.c_int
+    lib.d2c_conv3d_backward_prepared.argtypes = [p3] + [vp] * 10 + [vp, sz, i32, vp, sz, vp]
+    lib.d2c_conv3d_backward_prepared.restype = ctypes.c_int
     lib.d2c_conv1d_algo.argtypes, lib.d2c_conv1d_algo.restype = [p1], ctypes.c_int
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int

@@ -122,6 +122,29 @@ def _unify(input, offset, alpha, weight, bias):
     return input, offset, alpha, weight, bias
 
 
+class PreparedRegion:
+    """What a layer keeps between calls for the matrix-core kernels (d2c_conv3d_*_prepared): the channels-last copy of
+    the last input and the weights in the kernels' operand orders, in one device buffer, with the bookkeeping that
+    says which parts still belong to the tensors of the next call.  One per layer; not shared between layers."""
+
+    def __init__(self):
+        self.buf = None
+        self.input_token = 0          # bumped by every forward call: the buffer holds the copy of that call's input
+        self.fwd_weights = None       # (data_ptr, version, shape) of the weight tensor whose forward operand is held
+        self.bwd_weights = None
+
+    def buffer(self, nbytes, dev):
+        if self.buf is None or self.buf.numel() < nbytes or self.buf.device != dev:
+            self.buf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            self.fwd_weights = self.bwd_weights = None
+            self.input_token += 1
+        return self.buf
+
+    @staticmethod
+    def key(t):
+        return (t.data_ptr(), t._version, tuple(t.shape), t.dtype)
+
+
 class _DeformConv3dFunction(torch.autograd.Function):
     """DeformConv3dFunction of dconv3d.h:70-186.  `relu_scale` > 0 (not in the reference) makes the forward
     kernels store relu_scale * max(out, 0) -- the activation that follows the convolution, fused into their last
@@ -129,7 +152,7 @@ class _DeformConv3dFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, offset, alpha, weight, bias, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, offset_groups,
-                relu_scale=0.0, want_stats=False, offset_axes=7, backward_flags=0):
+                relu_scale=0.0, want_stats=False, offset_axes=7, backward_flags=0, prepared=None):
         lib = _lib.load()
         input, offset, weight = input.contiguous(), offset.contiguous(), weight.contiguous()
         alpha = alpha.contiguous() if alpha is not None else None
@@ -149,10 +172,24 @@ class _DeformConv3dFunction(torch.autograd.Function):
             nb = (lib.d2c_conv3d_forward_stats_workspace_bytes(ctypes.byref(desc), None) if want_stats
                   else lib.d2c_conv3d_forward_workspace_bytes(ctypes.byref(desc)))
             ws = _workspace(nb, dev)
+            npre = lib.d2c_conv3d_prepared_bytes(ctypes.byref(desc)) if (prepared is not None and not want_stats) else 0
+            ctx.prepared = None
             if want_stats:
                 rc = lib.d2c_conv3d_forward_stats(ctypes.byref(desc), None, _ptr(input), _ptr(offset), _ptr(alpha),
                                                   _ptr(weight), _ptr(bias), _ptr(out), _ptr(stats), _ptr(ws), nb,
                                                   _stream(dev))
+            elif npre:
+                # the layer's prepared region: forward weights kept while the weight tensor is the same, the input's
+                # channels-last copy left there for the backward call of this forward call
+                buf = prepared.buffer(npre, dev)
+                wkey = PreparedRegion.key(weight)
+                reuse = _lib.REUSE_FORWARD_WEIGHTS if prepared.fwd_weights == wkey else 0
+                rc = lib.d2c_conv3d_forward_prepared(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha),
+                                                     _ptr(weight), _ptr(bias), _ptr(out), _ptr(buf), buf.numel(), reuse,
+                                                     _ptr(ws), nb, _stream(dev))
+                prepared.fwd_weights = wkey
+                prepared.input_token += 1
+                ctx.prepared, ctx.input_token = prepared, prepared.input_token
             else:
                 rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha), _ptr(weight),
                                             _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
@@ -181,32 +218,48 @@ class _DeformConv3dFunction(torch.autograd.Function):
         galpha = torch.empty_like(alpha) if (alpha is not None and need[2]) else None
         gw = torch.empty_like(weight) if need[3] else None
         gb = torch.empty_like(bias) if (bias is not None and need[4]) else None
+        prepared = getattr(ctx, "prepared", None)
         with torch.cuda.device(dev):
             nb = lib.d2c_conv3d_backward_workspace_bytes(ctypes.byref(desc))
             ws = _workspace(nb, dev)
-            rc = lib.d2c_conv3d_backward(ctypes.byref(desc), _ptr(grad_out), _ptr(input), _ptr(offset), _ptr(alpha),
-                                         _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
-                                         _ptr(ws), nb, _stream(dev))
+            if prepared is not None and prepared.buf is not None:
+                # (the region still holds this call's input unless another forward call has used it since)
+                wkey = PreparedRegion.key(weight)
+                reuse = (_lib.REUSE_INPUT if prepared.input_token == ctx.input_token else 0) | \
+                        (_lib.REUSE_BACKWARD_WEIGHTS if prepared.bwd_weights == wkey else 0)
+                rc = lib.d2c_conv3d_backward_prepared(ctypes.byref(desc), _ptr(grad_out), _ptr(input), _ptr(offset),
+                                                      _ptr(alpha), _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha),
+                                                      _ptr(gw), _ptr(gb), _ptr(prepared.buf), prepared.buf.numel(), reuse,
+                                                      _ptr(ws), nb, _stream(dev))
+                prepared.bwd_weights = wkey
+                if not reuse & _lib.REUSE_INPUT:
+                    prepared.input_token += 1          # (the region now holds THIS input's copy, nobody's token)
+            else:
+                rc = lib.d2c_conv3d_backward(ctypes.byref(desc), _ptr(grad_out), _ptr(input), _ptr(offset), _ptr(alpha),
+                                             _ptr(weight), _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb),
+                                             _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d backward")
-        return (gx, goff, galpha, gw, gb) + (None,) * 15
+        return (gx, goff, galpha, gw, gb) + (None,) * 16
 
 
 def deform_conv3d(input, offset, alpha, weight, bias, stride_d, stride_h, stride_w, pad_d, pad_h, pad_w,
                   dilation_d, dilation_h, dilation_w, groups, offset_groups, relu_scale=0.0, want_stats=False,
-                  offset_axes=7, backward_flags=0):
+                  offset_axes=7, backward_flags=0, prepared=None):
     """deform_conv3d of dconv3d.h:188-226; `alpha` and `bias` may be None.  `relu_scale` > 0 fuses
     relu_scale * relu(.) into the store of the output (see _DeformConv3dFunction).  `want_stats` also returns the
     float32 [N, Cout, 2] sums and sums of squares of the stored output per (sample, channel), added up by the
     forward kernels where they store (the statistics a GroupNorm behind the convolution needs).  `offset_axes`: mask
     of the axes (1 z, 2 y, 4 x) the offsets displace along; the others are taken as zero and their gradient
     channels come back zero (matrix-core kernels only, see conv3d_algo).  `backward_flags`: the description's field
-    of that name (_lib.BWD_GW_* | _lib.bwd_slices(n)): how the backward pass trades workspace for time."""
+    of that name (_lib.BWD_GW_* | _lib.bwd_slices(n)): how the backward pass trades workspace for time.  `prepared`: a
+    PreparedRegion kept by the calling layer (see DeformConv3d.reuse_prepared)."""
     _check_common(3, input, offset, alpha, weight, bias, groups, offset_groups)
     input, offset, alpha, weight, bias = _unify(input, offset, alpha, weight, bias)
     return _DeformConv3dFunction.apply(
         input, offset, alpha, weight, bias, int(stride_d), int(stride_h), int(stride_w),
         int(pad_d), int(pad_h), int(pad_w), int(dilation_d), int(dilation_h), int(dilation_w),
-        int(groups), int(offset_groups), float(relu_scale), bool(want_stats), int(offset_axes), int(backward_flags))
+        int(groups), int(offset_groups), float(relu_scale), bool(want_stats), int(offset_axes), int(backward_flags),
+        prepared)
 
 
 class _DeformConv3dSizedFunction(torch.autograd.Function):

@@ -402,6 +402,68 @@ int d2c_conv3d_forward(const d2c_conv3d_desc *q, const void *x, const void *offs
     return d2c_tiled_forward(*q, x, offset, mask, weight, bias, out, ws, st);
 }
 
+size_t d2c_conv3d_prepared_bytes(const d2c_conv3d_desc *q)
+{
+    if (d2c_conv3d_check(q) != D2C_OK) return 0;
+    return choose_algo(*q, true) == D2C_ALGO_MFMA ? d2c_tiled_prepared_bytes(*q) : 0;
+}
+
+static int check_prepared(const d2c_conv3d_desc &q, void *prepared, size_t prepared_bytes, int reuse, D2cPrepared *out)
+{
+    out->base = nullptr;
+    out->reuse = 0;
+    const size_t need = choose_algo(q, true) == D2C_ALGO_MFMA ? d2c_tiled_prepared_bytes(q) : 0;
+    if (!prepared || need == 0) return D2C_OK;      // nothing to hold: an ordinary call
+    if (prepared_bytes < need || ((uintptr_t)prepared & 255u)) {
+        d2c_set_error("prepared region of %zu bytes (256-byte aligned) required, got %zu at %p", need, prepared_bytes, prepared);
+        return D2C_ERR_WORKSPACE;
+    }
+    if (reuse & ~(D2C_REUSE_INPUT | D2C_REUSE_FORWARD_WEIGHTS | D2C_REUSE_BACKWARD_WEIGHTS)) {
+        d2c_set_error("unknown bits in reuse flags %d", reuse);
+        return D2C_ERR_SHAPE;
+    }
+    out->base = prepared;
+    out->reuse = reuse;
+    return D2C_OK;
+}
+
+int d2c_conv3d_forward_prepared(const d2c_conv3d_desc *q, const void *x, const void *offset, const void *mask,
+                                const void *weight, const void *bias, void *out, void *prepared, size_t prepared_bytes,
+                                int32_t reuse, void *ws, size_t ws_bytes, void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!x || !offset || !weight || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    const int a = choose_algo(*q, false);
+    if (a < 0) return D2C_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (a == D2C_ALGO_GENERIC) return d2c_generic_conv3d_forward(*q, x, offset, mask, weight, bias, out, st);
+    D2cPrepared prep;
+    if (int rc = check_prepared(*q, prepared, prepared_bytes, reuse, &prep)) return rc;
+    if (int rc = check_ws(d2c_tiled_forward_ws(*q), ws, ws_bytes)) return rc;
+    return d2c_tiled_forward(*q, x, offset, mask, weight, bias, out, ws, st, nullptr, nullptr, prep.base ? &prep : nullptr);
+}
+
+int d2c_conv3d_backward_prepared(const d2c_conv3d_desc *q, const void *gout, const void *x, const void *offset,
+                                 const void *mask, const void *weight, void *gx, void *goff, void *gmask, void *gw,
+                                 void *gb, void *prepared, size_t prepared_bytes, int32_t reuse, void *ws,
+                                 size_t ws_bytes, void *stream)
+{
+    if (int rc = d2c_conv3d_check(q)) return rc;
+    if (!gout || !x || !offset || !weight) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    const int a = choose_algo(*q, false);
+    if (a < 0) return D2C_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (a == D2C_ALGO_GENERIC) {
+        if (int rc = check_ws(d2c_generic_conv3d_backward_ws(*q), ws, ws_bytes)) return rc;
+        return d2c_generic_conv3d_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws, st);
+    }
+    D2cPrepared prep;
+    if (int rc = check_prepared(*q, prepared, prepared_bytes, reuse, &prep)) return rc;
+    if (int rc = check_ws(d2c_tiled_backward_ws(*q), ws, ws_bytes)) return rc;
+    return d2c_tiled_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws, st, nullptr,
+                              prep.base ? &prep : nullptr);
+}
+
 size_t d2c_static_workspace_bytes(void) { return (size_t)D2C_STATIC_WORKSPACE_BYTES; }
 
 int d2c_conv3d_forward_static(const d2c_conv3d_desc *q, const void *x, const void *offset, const void *mask,

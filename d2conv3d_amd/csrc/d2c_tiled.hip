@@ -20,7 +20,8 @@ bool d2c_tiled_bwd_single_pass(const TiledShape &s, int dtype);
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
-                              void *gmask, float *auxacc, hipStream_t st, int phase = 3, int g_lo = 0, int g_n = 0);
+                              void *gmask, float *auxacc, hipStream_t st, int phase = 3, int g_lo = 0, int g_n = 0,
+                              bool weights_packed = false);
 bool d2c_bwd_sliceable(const TiledShape &s, int dtype);
 int d2c_backward_slices();
 int d2c_bwd_data_split(const TiledShape &s, int dtype);
@@ -364,6 +365,11 @@ __global__ void __launch_bounds__(256) size_minus_one_kernel(TiledShape s, const
 struct FwdWs {
     size_t xcl, wp, outacc, total;
 };
+// Caller-held prepared region (d2c_conv3d_prepared_bytes): channels-last input + zero row | forward weights in
+// fragment order | backward weights transposed per step (single-pass reductions only)
+struct PreparedLayout {
+    size_t xcl, wp, wt, wt_bytes, total;
+};
 FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 {
     const size_t es = d2c_elem_size(q.dtype);
@@ -377,6 +383,19 @@ FwdWs fwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     if (d2c_fwd_split(s) > 1)
         w.total += d2c_align_up((size_t)((s.M + 63) / 64 * 64) * s.ogp * s.groups * sizeof(float));
     return w;
+}
+
+PreparedLayout prepared_layout(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    const size_t es = d2c_elem_size(q.dtype);
+    PreparedLayout p;
+    p.xcl = 0;
+    p.wp = d2c_align_up((size_t)s.N * s.vol * s.Cin * es + 256);
+    p.wt = p.wp + d2c_align_up((size_t)s.groups * s.nchunk * s.K * s.ogp * bkc_of(q.dtype) * es);
+    const int omax = d2c_bwd_pass_channels(q.dtype);
+    p.wt_bytes = s.og <= omax ? d2c_align_up((size_t)s.groups * s.K * s.nchunk * bkc_of(q.dtype) * d2c_bwd_ogk(s.og, q.dtype) * es) : 0;
+    p.total = p.wt + p.wt_bytes;
+    return p;
 }
 
 template <typename T>
@@ -460,7 +479,7 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 template <typename T>
 int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
               const void *bias, void *out, void *ws, hipStream_t st, int nd = 3, const d2c_size_map_desc *sz = nullptr,
-              float *stats = nullptr)
+              float *stats = nullptr, const D2cPrepared *prep = nullptr)
 {
     const TiledShape s = tiled_shape(q, nd, 0, sz);
     char *base = (char *)ws;
@@ -470,24 +489,30 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
         return d2c_depthwise_forward<T>(s, base + d.xcl, off, mask, base + d.wt, bias, out, st);
     }
     const FwdWs l = fwd_ws(q, s);
-    if (int rc = pack_input<T>(s, x, base + l.xcl, st, true)) return rc;   // with the row of zeros behind it
+    // (a caller-held prepared region takes the place of the workspace's channels-last input and packed weights; what it
+    // already holds from an earlier call is not made again)
+    const PreparedLayout pl = prepared_layout(q, s);
+    char *xcl_p = prep ? (char *)prep->base + pl.xcl : base + l.xcl;
+    char *wp_p = prep ? (char *)prep->base + pl.wp : base + l.wp;
+    if (!(prep && (prep->reuse & D2C_REUSE_INPUT)))
+        if (int rc = pack_input<T>(s, x, xcl_p, st, true)) return rc;   // with the row of zeros behind it
     const long total = (long)s.groups * s.nchunk * s.K * (s.ogp / 32) * 4 * 64;
     long g = (total + 255) / 256;
     if (g > 8192) g = 8192;
-    {
+    if (!(prep && (prep->reuse & D2C_REUSE_FORWARD_WEIGHTS))) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         const size_t lds = (size_t)kPackRows * ((size_t)bkc_of(q.dtype) * s.K * sizeof(T) + 4);
         if (lds <= 64 * 1024 && reinterpret_cast<uintptr_t>(w) % 16 == 0)
             hipLaunchKernelGGL(pack_weight_fwd_lds_kernel<T>,
                                dim3((unsigned)(s.groups * s.nchunk * (s.ogp / 32) * (32 / kPackRows))), dim3(256), lds, st,
-                               (const T *)w, (T *)(base + l.wp), s);
+                               (const T *)w, (T *)wp_p, s);
         else
             hipLaunchKernelGGL(pack_weight_fwd_kernel<T>, dim3((unsigned)g), dim3(256), 0, st, (const T *)w,
-                               (T *)(base + l.wp), s, total);
+                               (T *)wp_p, s, total);
     }
     if (int rc = d2c_check_launch("pack_weight_fwd_kernel")) return rc;
     // (the per-tile sums of the output statistics go behind everything else in the workspace)
-    return d2c_tiled_fwd_launch<T>(s, base + l.xcl, off, mask, base + l.wp, bias, out, (float *)(base + l.outacc), st,
+    return d2c_tiled_fwd_launch<T>(s, xcl_p, off, mask, wp_p, bias, out, (float *)(base + l.outacc), st,
                                    stats, stats ? (float *)(base + l.total) : nullptr);
 }
 
@@ -596,7 +621,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 template <typename T>
 int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off, const void *mask,
                const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws, hipStream_t st,
-               int nd = 3, int quirks = 0, const d2c_size_map_desc *sz = nullptr)
+               int nd = 3, int quirks = 0, const d2c_size_map_desc *sz = nullptr, const D2cPrepared *prep = nullptr)
 {
     TiledShape s = tiled_shape(q, nd, quirks, sz);
     char *base = (char *)ws;
@@ -633,7 +658,14 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         return D2C_OK;
     }
     const BwdWs l = bwd_ws(q, s);
-    if (int rc = pack_input<T>(s, x, base + l.xcl, st, true)) return rc;   // with the row of zeros behind it
+    const PreparedLayout pl = prepared_layout(q, s);
+    char *xcl_p = prep ? (char *)prep->base + pl.xcl : base + l.xcl;
+    // (the transposed weights of the region serve single-pass reductions; wider weight groups re-pack per pass)
+    const bool wt_prep = prep && pl.wt_bytes > 0;
+    char *wt_p = wt_prep ? (char *)prep->base + pl.wt : base + l.wt;
+    const bool wt_packed = wt_prep && (prep->reuse & D2C_REUSE_BACKWARD_WEIGHTS);
+    if (!(prep && (prep->reuse & D2C_REUSE_INPUT)))
+        if (int rc = pack_input<T>(s, x, xcl_p, st, true)) return rc;   // with the row of zeros behind it
     if (s.ss.on) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         long gr = ((long)s.N * s.P + 255) / 256;
@@ -664,11 +696,11 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             L = d2c_lists_make(s, Elem<T>::DT, base + l.counts, base + l.entries, base + l.ovf);
             if (int rc = auxk ? d2c_lists_clear(L, st) : d2c_lists_build(s, off, mask, L, st)) return rc;
         }
-        if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt, nullptr, base + l.gcol,
-                                                 nullptr, nullptr, (float *)(base + l.auxacc), st, 1))
+        if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, xcl_p, off, mask, w, wt_p, nullptr, base + l.gcol,
+                                                 nullptr, nullptr, (float *)(base + l.auxacc), st, 1, 0, 0, wt_packed))
             return rc;
         if (gw_from_col)
-            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, xcl_p, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc), gw, base + l.col, 0, st, 1))
                 return rc;
         const int cpc = s.cpg / BKC;
@@ -682,18 +714,18 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                                                     - (uintptr_t)((size_t)c_lo * s.K * s.M * BKC * es));
             char *col_v = reinterpret_cast<char *>(reinterpret_cast<uintptr_t>(base + l.col)
                                                    - (uintptr_t)((size_t)blk_lo * cpc * s.K * mpad * BKC * es));
-            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt, nullptr, gcol_v,
+            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, xcl_p, off, mask, w, wt_p, nullptr, gcol_v,
                                                      nullptr, nullptr, (float *)(base + l.auxacc), st, 2, g0, gn))
                 return rc;
             if (auxk)
-                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, gcol_v, goff, gmask, lists ? &L : nullptr,
+                if (int rc = d2c_aux_grad_launch<T>(s, xcl_p, off, mask, gcol_v, goff, gmask, lists ? &L : nullptr,
                                                     gw_from_col ? col_v : nullptr, false, st, g0, gn))
                     return rc;
             if (lists)
                 if (int rc = d2c_gx_owner_launch<T>(s, gcol_v, L, gxcl, st, c_lo, gn * cpc)) return rc;
             const int g1 = g0 + gn;
             if (gw_from_col && (g1 == s.G || g1 % sl.cgs == 0))
-                if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+                if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, xcl_p, off, mask, base + l.goutp,
                                                            (float *)(base + l.gwacc), gw, col_v, mpad, st, 2,
                                                            blk_lo * cpc / 2, (g1 - blk_lo) * cpc / 2))
                     return rc;
@@ -701,7 +733,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         if (gx)
             if (int rc = d2c_tiled_unpack_gx<T>(s, gxcl, gx, st)) return rc;
         if (gw_from_col) {
-            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, xcl_p, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc), gw, base + l.col, 0, st, 4))
                 return rc;
             gw_done = true;
@@ -730,10 +762,10 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                 L = d2c_lists_make(s, Elem<T>::DT, base + l.counts, base + l.entries, base + l.ovf);
                 if (int rc = (auxk && !gw_in_place) ? d2c_lists_clear(L, st) : d2c_lists_build(s, off, mask, L, st)) return rc;
             }
-            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, base + l.xcl, off, mask, w, base + l.wt,
+            if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, xcl_p, off, mask, w, wt_p,
                                                      lists ? nullptr : gxcl, (lists || auxk) ? base + l.gcol : nullptr,
                                                      auxk ? nullptr : goff, auxk ? nullptr : gmask,
-                                                     (float *)(base + l.auxacc), st))
+                                                     (float *)(base + l.auxacc), st, 3, 0, 0, wt_packed))
                 return rc;
             if (lists && gw_in_place)
                 if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, L, gxcl, st)) return rc;
@@ -743,7 +775,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                               (size_t)64 * bkc_of(q.dtype) * sizeof(T), st);
             }
             if (auxk)
-                if (int rc = d2c_aux_grad_launch<T>(s, base + l.xcl, off, mask, base + l.gcol, goff_k, gmask,
+                if (int rc = d2c_aux_grad_launch<T>(s, xcl_p, off, mask, base + l.gcol, goff_k, gmask,
                                                     (lists && !gw_in_place) ? &L : nullptr,
                                                     gw_from_col ? (gw_in_place ? base + l.gcol : base + l.col) : nullptr,
                                                     gw_in_place, st))
@@ -773,7 +805,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
     }
     if (gw && !gw_done) {
         if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
-            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, base + l.xcl, off, mask, base + l.goutp,
+            if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, xcl_p, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc),
                                                        gw, gw_from_col ? (gw_in_place ? base + l.gcol : base + l.col) : nullptr,
                                                        gw_in_place ? (long)s.M : (long)((s.M + 63) / 64) * 64, st))
@@ -893,10 +925,18 @@ bool d2c_tiled_sized_supported(const d2c_conv3d_desc &q, bool backward)
 }
 
 int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
-                      const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz, float *stats)
+                      const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz, float *stats,
+                      const D2cPrepared *prep)
 {
-    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats);
-    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats);
+    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats, prep);
+    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats, prep);
+}
+
+// Bytes of the caller-held prepared region of a description (0: the kernel family keeps nothing worth holding)
+size_t d2c_tiled_prepared_bytes(const d2c_conv3d_desc &q)
+{
+    if (is_depthwise(q) || !mfma_channels_ok(q)) return 0;
+    return prepared_layout(q, tiled_shape(q)).total;
 }
 
 // The forward kernels of this description add up per-channel statistics of the output on their way.
@@ -907,9 +947,9 @@ bool d2c_tiled_forward_fills_stats(const d2c_conv3d_desc &q)
 
 int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
                        const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
-                       void *ws, hipStream_t st, const d2c_size_map_desc *sz)
+                       void *ws, hipStream_t st, const d2c_size_map_desc *sz, const D2cPrepared *prep)
 {
     if (q.dtype == D2C_BF16)
-        return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz);
-    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz);
+        return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz, prep);
+    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz, prep);
 }

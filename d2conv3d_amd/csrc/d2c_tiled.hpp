@@ -18,12 +18,19 @@ bool d2c_tiled_sized_supported(const d2c_conv3d_desc &q, bool backward);
 // `stats` != nullptr (only where d2c_tiled_forward_fills_stats() says so): fp32 [N][Cout][2], the sum and the sum of
 // squares of the stored output per (sample, channel).
 bool d2c_tiled_forward_fills_stats(const d2c_conv3d_desc &q);
+// `prep` != nullptr: a caller-held region of d2c_tiled_prepared_bytes() bytes that takes the place of the
+// workspace's channels-last input and packed weights; the parts named in `reuse` (D2C_REUSE_*) are taken as they are.
+struct D2cPrepared {
+    void *base;
+    int reuse;
+};
+size_t d2c_tiled_prepared_bytes(const d2c_conv3d_desc &q);
 int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
                       const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz = nullptr,
-                      float *stats = nullptr);
+                      float *stats = nullptr, const D2cPrepared *prep = nullptr);
 int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
                        const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
-                       void *ws, hipStream_t st, const d2c_size_map_desc *sz = nullptr);
+                       void *ws, hipStream_t st, const d2c_size_map_desc *sz = nullptr, const D2cPrepared *prep = nullptr);
 
 // 1-D operator served by the same matrix-core kernels (1 x 1 x L volume).
 bool d2c_tiled1d_supported(const d2c_conv1d_desc &q);

@@ -1693,7 +1693,8 @@ int d2c_bwd_data_split(const TiledShape &s, int dtype)
 template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
-                              void *gmask, float *auxacc, hipStream_t st, int phase, int g_lo, int g_n)
+                              void *gmask, float *auxacc, hipStream_t st, int phase, int g_lo, int g_n,
+                              bool weights_packed)
 {
     // phase: 1 = the weight re-layout (and the clears), 2 = the kernel, 3 = both.  g_n > 0 (grad-column product on
     // tiled_bwd_col32_kernel only, see d2c_bwd_sliceable): the rows of the offset groups [g_lo, g_lo + g_n) only,
@@ -1742,7 +1743,8 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const int ogn = s.og - o0 < omax ? s.og - o0 : omax;
         const int ogk = d2c_bwd_ogk(ogn, Elem<T>::DT);
         const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
-        if (phase & 1) {
+        // (weights_packed: `wt` already holds them, from an earlier call on the same weights)
+        if ((phase & 1) && !weights_packed) {
             D2cProfScope prof(D2C_PROF_PACK, st);
             constexpr int R = 128 / (int)sizeof(T);
             const size_t lds = (size_t)R * ((size_t)kPackCh * s.K * sizeof(T) + 4);
@@ -2006,7 +2008,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
 #define INST(T)                                                                                                    \
     template int d2c_tiled_bwd_data_launch<T>(const TiledShape &, const void *, const void *, const void *,        \
                                               const void *, const void *, void *, float *, void *, void *, void *, \
-                                              float *, hipStream_t, int, int, int);                                         \
+                                              float *, hipStream_t, int, int, int, bool);                                   \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
                                                 const void *, void *, float *, void *, const void *, long, hipStream_t, \
                                                 int, int, int);                                                     \

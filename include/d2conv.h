@@ -174,6 +174,35 @@ int d2c_conv3d_backward(const d2c_conv3d_desc *desc, const void *grad_out, const
                         void *grad_x, void *grad_offset, void *grad_mask, void *grad_weight,
                         void *grad_bias, void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * The same two calls with a caller-held "prepared" region (no counterpart in the reference, whose column pipeline
+ * re-lays nothing out): the matrix-core kernels work on a channels-last copy of the input and on weights in the
+ * order their matrix instructions read them, which every call makes anew in its workspace.  A caller that keeps a
+ * region of d2c_conv3d_prepared_bytes() bytes (256-byte aligned) per layer lets the calls make them THERE and
+ * tells later calls what it still holds:
+ *   D2C_REUSE_INPUT             the region holds the copy of THIS input `x` (made by a call on the same x):
+ *                               the backward call of a training step after its forward call;
+ *   D2C_REUSE_FORWARD_WEIGHTS   ... the forward operand of THIS weight tensor: forward calls while the weights
+ *                               do not change (inference);
+ *   D2C_REUSE_BACKWARD_WEIGHTS  ... the backward operand of this weight tensor (made by a backward call).
+ * Parts not named are made by the call (and may be named in the next one).  Results are those of the plain calls
+ * (the same kernels on the same operands).  d2c_conv3d_prepared_bytes() is 0 for descriptions the other kernel families serve; the calls
+ * then ignore `prepared` and `reuse`.  The workspace is needed as before.
+ */
+#define D2C_REUSE_INPUT            1
+#define D2C_REUSE_FORWARD_WEIGHTS  2
+#define D2C_REUSE_BACKWARD_WEIGHTS 4
+size_t d2c_conv3d_prepared_bytes(const d2c_conv3d_desc *desc);
+int d2c_conv3d_forward_prepared(const d2c_conv3d_desc *desc, const void *x, const void *offset, const void *mask,
+                                const void *weight, const void *bias, void *out, void *prepared,
+                                size_t prepared_bytes, int32_t reuse, void *workspace, size_t workspace_bytes,
+                                void *stream);
+int d2c_conv3d_backward_prepared(const d2c_conv3d_desc *desc, const void *grad_out, const void *x,
+                                 const void *offset, const void *mask, const void *weight, void *grad_x,
+                                 void *grad_offset, void *grad_mask, void *grad_weight, void *grad_bias,
+                                 void *prepared, size_t prepared_bytes, int32_t reuse, void *workspace,
+                                 size_t workspace_bytes, void *stream);
+
 int d2c_conv1d_check(const d2c_conv1d_desc *desc);
 int d2c_conv1d_algo(const d2c_conv1d_desc *desc);   /* D2C_ALGO_GENERIC or D2C_ALGO_MFMA */
 size_t d2c_conv1d_forward_workspace_bytes(const d2c_conv1d_desc *desc);

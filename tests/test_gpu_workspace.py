@@ -94,3 +94,64 @@ def test_backward_flags_of_the_description_size_the_workspace_and_choose_the_pat
     finally:
         _ops.config.set_workspace_caching(True)
         _ops.config.release_workspaces()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_prepared_region_gives_the_same_results(dtype, dev):
+    """d2c_conv3d_forward_prepared / _backward_prepared through DeformConv3d.reuse_prepared: the channels-last
+    input and the re-ordered weights kept in a buffer of the layer.  Every call must return what the plain calls
+    return (the same kernels on the same operands: equal up to the order in which partial sums are added with
+    atomics, i.e. a few units in the last place): the first call (nothing held yet), a second step with unchanged weights (forward weights and,
+    in the backward call, input and backward weights reused), a step after the weights changed, two forward
+    calls before their backward calls (the second forward call takes the buffer, so the first backward call must
+    lay its input out again), and a call at another size."""
+    from d2conv3d_amd.deform_conv import DeformConv3d
+    torch.manual_seed(23)
+    C, O, G = 128, 192, 2
+    plain = DeformConv3d(C, O, 3, padding=1, offset_groups=G).to(dev, dtype)
+    kept = DeformConv3d(C, O, 3, padding=1, offset_groups=G).to(dev, dtype)
+    kept.load_state_dict(plain.state_dict())
+    kept.reuse_prepared = True
+
+    def data(dims, seed):
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(1, C, *dims, generator=g).to(dev, dtype)
+        off = (torch.randn(1, G * 81, *dims, generator=g) * 1.5).to(dev)
+        m = torch.sigmoid(torch.randn(1, G * 27, *dims, generator=g)).to(dev)
+        gout = torch.randn(1, O, *dims, generator=g).to(dev, dtype)
+        return x, off, m, gout
+
+    def step(layer, x, off, m, gout):
+        layer.zero_grad()
+        ts = [t.clone().requires_grad_(True) for t in (x, off, m)]
+        y = layer(*ts)
+        y.backward(gout)
+        return [y.detach()] + [t.grad for t in ts] + [layer.weight.grad.clone(), layer.bias.grad.clone()]
+
+    rtol = 2e-6 if dtype == torch.float32 else 8e-3      # (one unit in the last place of bfloat16 is 2^-8)
+
+    def same(a, b, what):
+        for i, (u, v) in enumerate(zip(a, b)):
+            assert_close(u, v, rtol, rtol * max(1.0, v.abs().max().item()), f"{what} [{i}]")
+
+    d1, d2 = data((4, 9, 10), 1), data((4, 9, 10), 2)
+    same(step(kept, *d1), step(plain, *d1), "first call")
+    assert kept._prepared.buf is not None and kept._prepared.buf.numel() > 0
+    same(step(kept, *d2), step(plain, *d2), "second call, weights unchanged")
+    with torch.no_grad():
+        for layer in (plain, kept):
+            layer.weight.mul_(1.5)
+    same(step(kept, *d1), step(plain, *d1), "after the weights changed")
+    # two forward calls, then their backward calls in reverse order
+    res = {}
+    for name, layer in (("kept", kept), ("plain", plain)):
+        layer.zero_grad()
+        ta = [t.clone().requires_grad_(True) for t in d1[:3]]
+        tb = [t.clone().requires_grad_(True) for t in d2[:3]]
+        ya, yb = layer(*ta), layer(*tb)
+        yb.backward(d2[3])
+        ya.backward(d1[3])
+        res[name] = [ya.detach(), yb.detach()] + [t.grad for t in ta + tb]
+    same(res["kept"], res["plain"], "two forward calls before their backward calls")
+    d3 = data((3, 12, 13), 3)
+    same(step(kept, *d3), step(plain, *d3), "another size")
