@@ -467,6 +467,9 @@ def main():
                     help="3-D matrix-core workloads: keep a prepared region (d2c_conv3d_*_prepared) the way a layer would: "
                          "'train' = the backward call reuses the input copy its forward call made (weights change every "
                          "step); 'infer' = forward calls also reuse the re-ordered weights")
+    ap.add_argument("--f32-split-backward", action="store_true",
+                    help="float32 matrix-core workloads: the backward matrix kernels on two-term bfloat16 operands too "
+                         "(D2C_BWD_F32_SPLIT; gradients with ~4e-6 relative error of their scale)")
     ap.add_argument("--expanded-offsets", action="store_true",
                     help="dynamic-dilation workloads (c2_*): expand the dilation map to an offsets tensor first "
                          "and time the ordinary operator on it, instead of handing the map to the operator")
@@ -512,7 +515,8 @@ def main():
         desc = _lib.Conv3dDesc(N, C, C, T_, H_, W_, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, groups, G, T_, H_, W_,
                                code, code, 0, 1.0, args.offset_axes,
                                {1: _lib.BWD_GW_COLUMNS, 2: _lib.BWD_GW_IN_PLACE, 0: _lib.BWD_GW_RESAMPLE}[args.grad_weight_mode]
-                               | _lib.bwd_slices(args.backward_slices))
+                               | _lib.bwd_slices(args.backward_slices)
+                               | (_lib.BWD_F32_SPLIT if args.f32_split_backward else 0))
         kind = "conv3d"
         algo = _lib.ALGO_NAMES[lib.d2c_conv3d_algo(ctypes.byref(desc))]
     else:
@@ -733,6 +737,7 @@ def main():
                    "offset_axes": args.offset_axes,
                    "grad_input_mode": args.grad_input_mode, "grad_weight_mode": args.grad_weight_mode,
                    "backward_slices": args.backward_slices, "prepared_region": args.prepared if prep is not None else "off",
+                   "f32_split_backward": bool(args.f32_split_backward),
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
                    "taps_outside_volume": taps,

@@ -49,6 +49,7 @@ MASK_ACTIVATIONS = {"none": 0, "linear": 0, "sigmoid": 1, "relu": 2, "tanh": 3}
 
 # d2c_conv3d_desc::backward_flags
 BWD_GW_DEFAULT, BWD_GW_COLUMNS, BWD_GW_IN_PLACE, BWD_GW_RESAMPLE = 0, 1, 2, 3
+BWD_F32_SPLIT = 0x10000
 
 
 def bwd_slices(n):

@@ -275,7 +275,7 @@ int d2c_conv3d_check(const d2c_conv3d_desc *q)
                 "tensor with 2^31 or more elements is not supported");
     D2C_REQUIRE(q->offset_axes >= 0 && q->offset_axes <= 7, "offset_axes must be a mask of the axes z, y, x (0 .. 7)");
     D2C_REQUIRE(q->epilogue == D2C_EPILOGUE_NONE || q->epilogue == D2C_EPILOGUE_RELU, "unknown epilogue %d", q->epilogue);
-    D2C_REQUIRE((q->backward_flags & ~(D2C_BWD_GW_MASK | D2C_BWD_SLICES(0xff))) == 0, "unknown bits in backward_flags %d",
+    D2C_REQUIRE((q->backward_flags & ~(D2C_BWD_GW_MASK | D2C_BWD_SLICES(0xff) | D2C_BWD_F32_SPLIT)) == 0, "unknown bits in backward_flags %d",
                 q->backward_flags);
     D2C_REQUIRE(q->deform_channels >= 0 && (long)q->N * q->deform_channels * P < (1L << 31),
                 "deform_channels must be non-negative and the deformation tensor below 2^31 elements");

@@ -47,20 +47,16 @@ D2C_DEV uint32_t pack_bf16x2(float lo, float hi)
 // v_mfma_f32_32x32x16_bf16 whose 16-deep reductions hold all four partial products of every element,
 // (hi + lo) * (hi' + lo'), summed in float32 by the matrix core: a quarter of the matrix-pipe time of the four float
 // instructions.  The producers of the forward operands (weight re-layout, sampled tile) write this form.
-// The BACKWARD kernels keep plain floats and the float instruction: the relative error of 4e-6 that the two-term
-// operands leave in a long sum is fine for the output (values of order 1 against 1e-4 relative / 1e-5 absolute) but
-// not for gradients whose elements reach 20 .. 400 and are held to the same absolute 1e-5
-// (-DD2C_F32_SPLIT_BACKWARD builds them on split operands all the same; -DD2C_F32_NATIVE_MFMA keeps the forward
-// kernels on the float instruction).
+// The BACKWARD kernels keep plain floats and the float instruction by default: the relative error of 4e-6 that the
+// two-term operands leave in a long sum is fine for the output (values of order 1 against 1e-4 relative / 1e-5
+// absolute) but not for gradients whose elements reach 20 .. 400 and are held to the same absolute 1e-5.  A caller
+// who prefers the speed asks for split operands there too (D2C_BWD_F32_SPLIT in the description's backward_flags:
+// TiledShape::f32split, a template parameter of the backward kernels).  -DD2C_F32_NATIVE_MFMA keeps the forward
+// kernels on the float instruction.
 #ifdef D2C_F32_NATIVE_MFMA
 constexpr bool kF32SplitFwd = false;
 #else
 constexpr bool kF32SplitFwd = true;
-#endif
-#ifdef D2C_F32_SPLIT_BACKWARD
-constexpr bool kF32SplitBwd = true;
-#else
-constexpr bool kF32SplitBwd = false;
 #endif
 D2C_DEV float bf16_residual(float v, uint32_t hi_bits)
 {
@@ -285,6 +281,7 @@ struct TiledShape {
     // tensor times P when both pointers point into that one tensor (d2c_conv3d_desc::deform_channels).
     long obs, mbs;
     int mact;             // activation the sampler applies to the mask values it reads (D2C_MASK_ACT_*)
+    int f32split;         // float problems: the backward matrix kernels take two-term bfloat16 operands too (D2C_BWD_F32_SPLIT)
 };
 
 // The modulation activation of the self-deforming layers (network/layers.py:107-120, dconv_native/modules.py:71-84),

@@ -116,6 +116,7 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0, con
                                   : (sz ? (long)mode_channels(sz->mode) * s.P : (long)s.G * s.K * (nd == 3 ? 3 : 1) * s.P);
     s.mbs = q.deform_channels > 0 ? (long)q.deform_channels * s.P : (long)s.G * s.K * s.P;
     s.mact = q.mask_activation;
+    s.f32split = (q.dtype == D2C_F32 && (q.backward_flags & D2C_BWD_F32_SPLIT)) ? 1 : 0;
     const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
     s.ogp = (s.og + nt - 1) / nt * nt;
     s.geo = make_geom(q);

@@ -70,7 +70,9 @@ struct BwdDataArgs {
 };
 
 // NKG = k-groups of the reduction over output channels held in registers.
-template <typename T, int NKG>
+// SPLIT (float problems): operands as two bfloat16 halves on the bfloat16 matrix instruction (see kF32SplitFwd in
+// d2c_mma.hpp), where the caller has asked for it (TiledShape::f32split).
+template <typename T, int NKG, bool SPLIT>
 __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 {
     constexpr int VEC = Elem<T>::VEC;
@@ -118,7 +120,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
                 const int o = (kg * 2 + (lane >> 5)) * VEC + i;
                 e[i] = (ok && kg < nkg && o < a.ogn) ? gp[(long)o * s.P] : (T)0;
             }
-            ga[kg] = operand_vec<T, kF32SplitBwd>(e);
+            ga[kg] = operand_vec<T, SPLIT>(e);
         }
     }
 
@@ -238,14 +240,14 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 #pragma unroll
                 for (int kg = 0; kg < NKG; kg++) {
                     const uint4 bf = *reinterpret_cast<const uint4 *>(wa[kg & 7] + (kg >> 3) * 256);
-                    mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bf);
+                    mma_kgroup<T, SPLIT>(acc, ga[kg], bf);
                 }
             } else {
 #pragma unroll
                 for (int kg = 0; kg < NKG; kg++) {
                     if (kg < nkg) {
                         const uint4 bf = *reinterpret_cast<const uint4 *>(wb + (((kg * 2 + wh) ^ wsw) << 4));
-                        mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bf);
+                        mma_kgroup<T, SPLIT>(acc, ga[kg], bf);
                     }
                 }
             }
@@ -505,7 +507,7 @@ D2C_DEV void mma8_bf16_t(f32x16 &acc, const uint4 *g, const unsigned *w)
 // 32 KiB, which leaves room for two 64 KiB weight tiles (512 reduced channels) in the 160 KiB of a workgroup.
 template <typename T> constexpr int col_row_stride() { return 8 * Elem<T>::VEC * 4 + (sizeof(T) == 2 ? 0 : 16); }
 
-template <typename T, int NKG, bool DB>
+template <typename T, int NKG, bool DB, bool SPLIT>
 __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
 {
     constexpr int VEC = Elem<T>::VEC;
@@ -550,7 +552,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 const int o = (kg * 2 + (lane >> 5)) * VEC + i;
                 e[i] = (ok && kg < nkg && o < a.ogn) ? gp[(long)o * s.P] : (T)0;
             }
-            ga[kg] = operand_vec<T, kF32SplitBwd>(e);
+            ga[kg] = operand_vec<T, SPLIT>(e);
         }
     }
 
@@ -620,7 +622,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                     if (kg + kPF < NKG)
                         bq[(kg + kPF) % (kPF + 1)] =
                             *reinterpret_cast<const uint4 *>(wb + woff[(kg + kPF) & 7] + ((kg + kPF) >> 3) * 256);
-                    mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bq[kg % (kPF + 1)]);
+                    mma_kgroup<T, SPLIT>(acc, ga[kg], bq[kg % (kPF + 1)]);
                 }
             } else {
                 const int wrow = cb * 32 + (lane & 31);
@@ -630,7 +632,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
                 for (int kg = 0; kg < NKG; kg++) {
                     if (kg < nkg) {
                         const uint4 bf = *reinterpret_cast<const uint4 *>(wr + (((kg * 2 + wh) ^ wsw) << 4));
-                        mma_kgroup<T, kF32SplitBwd>(acc, ga[kg], bf);
+                        mma_kgroup<T, SPLIT>(acc, ga[kg], bf);
                     }
                 }
             }
@@ -814,13 +816,20 @@ int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st)
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
     const bool db = bwd_col_lds<T>(a.ogk, true) <= 160 * 1024;
     const size_t lds = bwd_col_lds<T>(a.ogk, db);
-    const void *fn = db ? (const void *)tiled_bwd_col_kernel<T, NKG, true> : (const void *)tiled_bwd_col_kernel<T, NKG, false>;
-    if (int rc = d2c_allow_lds(fn, 160 * 1024, "tiled_bwd_col_kernel")) return rc;
     dim3 grid((a.s.M + MT - 1) / MT, a.s.groups, nsplit);
-    D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_col_kernel");
-    if (db) hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, true>), grid, dim3(kThreads), lds, st, a);
-    else hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, false>), grid, dim3(kThreads), lds, st, a);
-    return d2c_check_launch("tiled_bwd_col_kernel");
+    auto go = [&](auto split_c) -> int {
+        constexpr bool SP = decltype(split_c)::value;
+        const void *fn = db ? (const void *)tiled_bwd_col_kernel<T, NKG, true, SP> : (const void *)tiled_bwd_col_kernel<T, NKG, false, SP>;
+        if (int rc = d2c_allow_lds(fn, 160 * 1024, "tiled_bwd_col_kernel")) return rc;
+        D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_col_kernel");
+        if (db) hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, true, SP>), grid, dim3(kThreads), lds, st, a);
+        else hipLaunchKernelGGL((tiled_bwd_col_kernel<T, NKG, false, SP>), grid, dim3(kThreads), lds, st, a);
+        return d2c_check_launch("tiled_bwd_col_kernel");
+    };
+    if constexpr (sizeof(T) == 4) {
+        if (a.s.f32split) return go(std::true_type{});
+    }
+    return go(std::false_type{});
 }
 
 constexpr int kCol32MT = 256;
@@ -855,11 +864,18 @@ int launch_bwd_data(const BwdDataArgs &a, int nsplit, hipStream_t st)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
     const size_t lds = bwd_data_lds<T>(a.ogk);
-    if (int rc = d2c_allow_lds((const void *)tiled_bwd_data_kernel<T, NKG>, 160 * 1024, "tiled_bwd_data_kernel")) return rc;
     dim3 grid((a.s.M + MT - 1) / MT, a.s.groups, nsplit);
-    D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_data_kernel");
-    hipLaunchKernelGGL((tiled_bwd_data_kernel<T, NKG>), grid, dim3(kThreads), lds, st, a);
-    return d2c_check_launch("tiled_bwd_data_kernel");
+    auto go = [&](auto split_c) -> int {
+        constexpr bool SP = decltype(split_c)::value;
+        if (int rc = d2c_allow_lds((const void *)tiled_bwd_data_kernel<T, NKG, SP>, 160 * 1024, "tiled_bwd_data_kernel")) return rc;
+        D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_data_kernel");
+        hipLaunchKernelGGL((tiled_bwd_data_kernel<T, NKG, SP>), grid, dim3(kThreads), lds, st, a);
+        return d2c_check_launch("tiled_bwd_data_kernel");
+    };
+    if constexpr (sizeof(T) == 4) {
+        if (a.s.f32split) return go(std::true_type{});
+    }
+    return go(std::false_type{});
 }
 
 // ============================================================ kernel 2
@@ -893,7 +909,7 @@ struct BwdWeightDmaArgs {
 };
 
 // NC: corner rows per sampling point, 8, or 4 / 2 when offsets along one / two axes are fixed (see fwd_dma_body).
-template <typename T, bool AUX16, bool SIZED, int NC>
+template <typename T, bool AUX16, bool SIZED, int NC, bool SPLIT>
 __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(BwdWeightDmaArgs aa)
 {
     constexpr int RAWPOS = NC * 128;           // raw bytes per position
@@ -1092,7 +1108,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
         } else {
             // float: stored transposed ([channel][position]), one element per store
             unsigned char *tb = s_tile + dbuf * BKC * TRS + (ivec * VEC) * TRS;
-            if constexpr (kF32SplitBwd) {
+            if constexpr (SPLIT) {
                 // (as the two bfloat16 halves of a matrix-instruction operand: the 16 bytes of four consecutive
                 // positions hold their four `hi` values, then their four `lo` values)
                 unsigned char *tg = tb + (ipos >> 2) * 16 + (ipos & 3) * 2;
@@ -1153,7 +1169,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
 #pragma unroll
             for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                for (int cb = 0; cb < CB; cb++) mma_kgroup<T, kF32SplitBwd>(acc[ob][cb], ld[kq * 2 + ob], bf[cb]);
+                for (int cb = 0; cb < CB; cb++) mma_kgroup<T, SPLIT>(acc[ob][cb], ld[kq * 2 + ob], bf[cb]);
             if (kg + 4 < NKG) {
 #pragma unroll
                 for (int ob = 0; ob < OB; ob++) ld[kq * 2 + ob] = gfrag(i, kg + 4, ob);
@@ -1376,7 +1392,7 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
 #pragma unroll
                     for (int ob = 0; ob < OB; ob++)
 #pragma unroll
-                        for (int cb = 0; cb < CB; cb++) mma_kgroup<T, kF32SplitBwd>(acc[ob][cb], ld[kg * 2 + ob], bf[cb]);
+                        for (int cb = 0; cb < CB; cb++) mma_kgroup<T, false>(acc[ob][cb], ld[kg * 2 + ob], bf[cb]);
 #pragma unroll
                     for (int ob = 0; ob < OB; ob++) ld[kg * 2 + ob] = gn[(ob * NKGP + kg) * 64];
                     // (the requests stay behind the matrix instructions of their k-group)
@@ -1428,7 +1444,7 @@ template <typename T, int NC> constexpr size_t bwd_weight_dma_lds()
 // ============================================================ small kernels
 // W[o][c][k] -> wt[wg][step][cc][oo] for oo in [o0, o0 + ogn), padded with zeros to ogk; steps in the
 // order of the data kernel (offset group, tap, chunk of the group)
-template <typename T>
+template <typename T, bool SPLIT>
 __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt, TiledShape s, int ogk, int o0,
                                                               int ogn, long total)
 {
@@ -1447,7 +1463,7 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
 #pragma unroll
         for (int e = 0; e < VEC; e++)
             tmp[e] = oo + e < ogn ? w[((long)(wg * s.og + o0 + oo + e) * s.cg + j * BKC + cc) * s.K + k] : (T)0;
-        *reinterpret_cast<uint4 *>(wt + i) = operand_vec<T, kF32SplitBwd>(tmp);
+        *reinterpret_cast<uint4 *>(wt + i) = operand_vec<T, SPLIT>(tmp);
     }
 }
 
@@ -1455,7 +1471,7 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
 // as wide as the padding unit of ogk (128 bytes of wt) and kPackCh channels of a chunk, whose weights are
 // runs of kPackCh * K consecutive elements in W, and writes 16-byte vectors of consecutive output channels.
 constexpr int kPackCh = 8;
-template <typename T>
+template <typename T, bool SPLIT>
 __global__ void __launch_bounds__(256) pack_weight_bwd_lds_kernel(const T *w, T *wt, TiledShape s, int ogk, int o0,
                                                                   int ogn)
 {
@@ -1490,7 +1506,7 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_lds_kernel(const T *w, T 
         for (int e = 0; e < VEC; e++) tmp[e] = reinterpret_cast<const T *>(smem + (ov * VEC + e) * rs)[cc * s.K + k];
         const int st = ((j / cpc) * s.K + k) * cpc + j % cpc;
         const long di = (((long)wg * s.K * s.nchunk + st) * BKC + cb * kPackCh + cc) * ogk + obk * R + ov * VEC;
-        *reinterpret_cast<uint4 *>(wt + di) = operand_vec<T, kF32SplitBwd>(tmp);
+        *reinterpret_cast<uint4 *>(wt + di) = operand_vec<T, SPLIT>(tmp);
     }
 }
 
@@ -1597,7 +1613,7 @@ __global__ void __launch_bounds__(256) cvt_grad_weight_lds_kernel(const float *s
 //   goutp[wg][tile of kWMT positions][32-row block][k-group][lane] = 16 bytes =
 //   gout[wg*og + block*32 + lane%32][positions tile*kWMT + (2*kgroup + lane/32)*VEC + 0..VEC-1]
 // with positions numbered over the whole batch (m = b*P + p); rows past og and positions past N*P are zero.
-template <typename T>
+template <typename T, bool SPLIT>
 __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp, TiledShape s, int ntile, int OBT, long total,
                                                         bool vec)
 {
@@ -1619,7 +1635,7 @@ __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp,
                 const int b = (int)(m0 / s.P), p = (int)(m0 - (long)b * s.P);
                 v = *reinterpret_cast<const uint4 *>(gout + ((long)b * s.Cout + wg * s.og + ol) * s.P + p);
             }
-            reinterpret_cast<uint4 *>(goutp)[i] = operand_vec16<T, kF32SplitBwd>(v);
+            reinterpret_cast<uint4 *>(goutp)[i] = operand_vec16<T, SPLIT>(v);
             continue;
         }
 #pragma unroll
@@ -1632,7 +1648,7 @@ __global__ void __launch_bounds__(256) pack_gout_kernel(const T *gout, T *goutp,
             }
             e[q] = v;
         }
-        reinterpret_cast<uint4 *>(goutp)[i] = operand_vec<T, kF32SplitBwd>(e);
+        reinterpret_cast<uint4 *>(goutp)[i] = operand_vec<T, SPLIT>(e);
     }
 }
 
@@ -1747,14 +1763,17 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         if ((phase & 1) && !weights_packed) {
             D2cProfScope prof(D2C_PROF_PACK, st);
             constexpr int R = 128 / (int)sizeof(T);
+            constexpr bool SPT = sizeof(T) == 4;       // (split operands exist for float problems only)
+            const bool split = SPT && s.f32split;
+            auto k_lds = split ? &pack_weight_bwd_lds_kernel<T, SPT> : &pack_weight_bwd_lds_kernel<T, false>;
+            auto k_elem = split ? &pack_weight_bwd_kernel<T, SPT> : &pack_weight_bwd_kernel<T, false>;
             const size_t lds = (size_t)R * ((size_t)kPackCh * s.K * sizeof(T) + 4);
             if (lds <= 64 * 1024 && reinterpret_cast<uintptr_t>(w) % 16 == 0)
-                hipLaunchKernelGGL(pack_weight_bwd_lds_kernel<T>,
-                                   dim3((unsigned)(s.groups * s.nchunk * (ogk / R) * (BKC / kPackCh))), dim3(256), lds, st,
-                                   (const T *)w, (T *)wt, s, ogk, o0, ogn);
+                hipLaunchKernelGGL(k_lds, dim3((unsigned)(s.groups * s.nchunk * (ogk / R) * (BKC / kPackCh))), dim3(256), lds,
+                                   st, (const T *)w, (T *)wt, s, ogk, o0, ogn);
             else
-                hipLaunchKernelGGL(pack_weight_bwd_kernel<T>, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w,
-                                   (T *)wt, s, ogk, o0, ogn, total);
+                hipLaunchKernelGGL(k_elem, dim3(grid1d(total)), dim3(256), 0, st, (const T *)w, (T *)wt, s, ogk, o0, ogn,
+                                   total);
         }
         if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
         if (!(phase & 2)) continue;
@@ -1906,8 +1925,10 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         const int OBT = (s.og + 63) / 64 * 2;
         const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
         const bool vec = s.P % Elem<T>::VEC == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0;
-        hipLaunchKernelGGL(pack_gout_kernel<T>, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const T *)gout, (T *)goutp, s,
-                           ntp, OBT, total, vec);
+        constexpr bool SPT = sizeof(T) == 4;
+        auto k_gout = (SPT && s.f32split) ? &pack_gout_kernel<T, SPT> : &pack_gout_kernel<T, false>;
+        hipLaunchKernelGGL(k_gout, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const T *)gout, (T *)goutp, s, ntp, OBT,
+                           total, vec);
         if (int rc = d2c_check_launch("pack_gout_kernel")) return rc;
     }
     // One workgroup runs per compute unit at a time (LDS).  The pieces (see BwdWeightArgs) are the ones whose
@@ -1938,15 +1959,21 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         bool aux16 = false;
         if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st, "tiled_bwd_weight_dma_kernel");
-        auto go_nc = [&](auto aux_c, auto sized_c, auto nc_c) -> bool {
-            constexpr bool A16 = decltype(aux_c)::value, SZ = decltype(sized_c)::value;
+        auto go_sp = [&](auto aux_c, auto sized_c, auto nc_c, auto split_c) -> bool {
+            constexpr bool A16 = decltype(aux_c)::value, SZ = decltype(sized_c)::value, SP = decltype(split_c)::value;
             constexpr int NC = decltype(nc_c)::value;
             constexpr size_t lds = bwd_weight_dma_lds<T, NC>();
-            if (d2c_allow_lds((const void *)tiled_bwd_weight_dma_kernel<T, A16, SZ, NC>, 160 * 1024,
+            if (d2c_allow_lds((const void *)tiled_bwd_weight_dma_kernel<T, A16, SZ, NC, SP>, 160 * 1024,
                               "tiled_bwd_weight_dma_kernel") != D2C_OK)
                 return false;
-            hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, A16, SZ, NC>), grid, dim3(kThreads + 64), lds, st, a);
+            hipLaunchKernelGGL((tiled_bwd_weight_dma_kernel<T, A16, SZ, NC, SP>), grid, dim3(kThreads + 64), lds, st, a);
             return true;
+        };
+        auto go_nc = [&](auto aux_c, auto sized_c, auto nc_c) -> bool {
+            if constexpr (sizeof(T) == 4) {
+                if (s.f32split) return go_sp(aux_c, sized_c, nc_c, std::true_type{});
+            }
+            return go_sp(aux_c, sized_c, nc_c, std::false_type{});
         };
         const bool sized = s.ss.on != 0;
         // offsets fixed along one / two axes: 4 / 2 corner rows per sampling point (offsets-tensor source only)

@@ -83,6 +83,12 @@ enum {
  * groups).  Buffers of grad-column rows and sampled columns then hold one slice; several offset groups, one weight
  * group and 128 .. 512 output channels only (other descriptions ignore the bits). */
 #define D2C_BWD_SLICES(n)    (((n) & 0xff) << 8)
+/* float32 problems on the matrix-core kernels: let the backward matrix kernels, like the forward ones, carry every
+ * float operand as the sum of two bfloat16 values on the bfloat16 matrix instruction (a quarter of the matrix-pipe
+ * time of the float instruction).  Gradients then carry a relative error of about 4e-6 of their sums' scale
+ * instead of 1e-7 -- within 1e-4 relative, but not within 1e-5 absolute where elements reach tens or hundreds.
+ * Off by default. */
+#define D2C_BWD_F32_SPLIT    0x10000
 
 typedef struct d2c_conv3d_desc {
     int32_t N, Cin, Cout;

@@ -155,3 +155,26 @@ def test_prepared_region_gives_the_same_results(dtype, dev):
     same(res["kept"], res["plain"], "two forward calls before their backward calls")
     d3 = data((3, 12, 13), 3)
     same(step(kept, *d3), step(plain, *d3), "another size")
+
+
+@pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_o320_nomask", "c128_groups2_G1"])
+def test_float32_backward_on_split_operands(name, dev):
+    """D2C_BWD_F32_SPLIT: the backward matrix kernels of a float32 problem on two-term bfloat16 operands, like the
+    forward kernels.  Against the float64 oracle: every gradient within 2e-5 of its tensor's scale (the operands
+    keep 16 of float32's 24 significant bits: about 4e-6 relative in a long sum, against 1e-7 for plain float32),
+    and the default path on the same inputs an order of magnitude closer."""
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, torch.float32, seed=13)
+    dd = lambda t: t.double() if t is not None else None
+    eg = cpu.conv3d_backward(dd(gout), dd(x), dd(off), dd(m), dd(w), b is not None, s, p, d, groups, G)
+    errs = {}
+    for split in (True, False):
+        ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+        d2c.deform_conv3d(*ts, s, p, d, groups, G, backward_f32_split=split).backward(gout.to(dev))
+        errs[split] = []
+        for n, t, e in zip(("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias"), ts, eg):
+            if t is None:
+                continue
+            err = ((t.grad.double().cpu() - e).abs().max() / e.abs().max()).item()
+            errs[split].append(err)
+            assert err < (2e-5 if split else 2e-6), (name, n, split, err)
+    assert max(errs[True]) > max(errs[False])      # (the flag did change the arithmetic)
