@@ -712,7 +712,9 @@ def main():
         peak_l1 = 64 * 256 * 2.4  # GB/s
         npos, esz = dims[0] * dims[1] * dims[2], (2 if dt == "bf16" else 4)
         rows = N * npos * 27 * 8 * C * esz          # 8 corner values per tap and channel
-        per = {"dw_fwd_kernel": rows, "dw_bwd_kernel": rows + N * npos * 27 * C * esz,   # + the grad_out value per tap
+        # (the backward kernel stages the grad_out rows of a tile in LDS once for all its taps: they pass through the
+        #  vector-memory path once, not once per tap)
+        per = {"dw_fwd_kernel": rows, "dw_bwd_kernel": rows + N * npos * C * esz,
                "dw_gx_owner_kernel": N * npos * 27 * (32 + C * esz) + N * npos * C * 4}  # list entry + grad_out row per sample, grad_input once
         roofline_l1 = {"bound": "l1", "peak": round(peak_l1, 1), "unit": "GB/s",
                        "peak_source": "64 B/clk/CU x 256 CUs x 2.4 GHz (vector-memory path)", "kernels": {}}

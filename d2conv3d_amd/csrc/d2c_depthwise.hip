@@ -27,7 +27,7 @@ constexpr int kSlice = 64 * kCV;  // channels per workgroup
 // forward: 8 consecutive positions per wavefront (one 32-byte output segment per channel)
 constexpr int kFwdTP = 32, kFwdKB = 16;
 // backward: the taps of a batch are dealt to the wavefronts, each walks all positions of the tile
-constexpr int kBwdTP = 16, kBwdKB = 32;
+constexpr int kBwdTP = 16, kBwdKB = 16;
 
 struct DwArgs {
     TiledShape s;
@@ -65,33 +65,37 @@ D2C_DEV DwTile dw_tile(const TiledShape &s, int TP, int ny, int bid)
 }
 inline unsigned dw_grid(const TiledShape &s, int TP, int ny) { return xcd_unit_grid(s.N * ny, (s.P + TP - 1) / TP); }
 
-// View over dynamic LDS, one entry per (tap of the batch, position of the tile): the live corner
-// weights * alpha, the base voxel and live | inrange << 8; for the backward pass also the per-axis
-// fractions lz ly lx hz hy hx and alpha.
+// View over dynamic LDS, one entry per (tap of the batch, position of the tile): the base voxel and
+// live | inrange << 8, and
+//   forward:  the live corner weights * alpha, corner-major (w[corner][entry]);
+//   backward: 16 floats per entry, read as 16-byte vectors: the 8 corner weights * alpha | the per-axis fractions
+//             lz ly lx hz | hy hx, alpha, a pad.
 template <int TP, int KB> struct DwTaps {
     static constexpr int kNE = KB * TP;
     float (*w)[kNE];
+    float4 *pk;
     int *idx, *flag;
-    float (*frac)[kNE];
-    float *alpha;
 };
+constexpr int kDwEntryVecs = 4;
 template <int TP, int KB> D2C_DEV DwTaps<TP, KB> dw_taps(unsigned char *smem, bool bwd)
 {
     constexpr int kNE = KB * TP;
     DwTaps<TP, KB> t;
     float *f = reinterpret_cast<float *>(smem);
-    t.w = reinterpret_cast<float (*)[kNE]>(f); f += 8 * kNE;
+    t.w = nullptr; t.pk = nullptr;
+    if (bwd) {
+        t.pk = reinterpret_cast<float4 *>(f); f += 4 * kDwEntryVecs * kNE;
+    } else {
+        t.w = reinterpret_cast<float (*)[kNE]>(f); f += 8 * kNE;
+    }
     t.idx = reinterpret_cast<int *>(f); f += kNE;
     t.flag = reinterpret_cast<int *>(f); f += kNE;
-    t.frac = nullptr; t.alpha = nullptr;
-    if (bwd) {
-        t.frac = reinterpret_cast<float (*)[kNE]>(f); f += 6 * kNE;
-        t.alpha = f;
-    }
     return t;
 }
 constexpr size_t kDwLdsFwd = (size_t)10 * kFwdKB * kFwdTP * 4;
-constexpr size_t kDwLdsBwd = (size_t)17 * kBwdKB * kBwdTP * 4;
+// (+ the grad_out tile of the workgroup: kBwdTP rows of kSlice elements)
+constexpr size_t kDwLdsTab = (size_t)(4 * kDwEntryVecs + 2) * kBwdKB * kBwdTP * 4;
+constexpr size_t dw_lds_bwd(size_t es) { return kDwLdsTab + (size_t)kBwdTP * kSlice * es; }
 
 template <bool BWD, int TP, int KB>
 D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<TP, KB> &t, int m0, int m_end, int g, int k0, int kn)
@@ -122,12 +126,15 @@ D2C_DEV void dw_coords(const DwArgs &a, const DwTaps<TP, KB> &t, int m0, int m_e
             fr[0] = tp.lz; fr[1] = tp.ly; fr[2] = tp.lx; fr[3] = tp.hz; fr[4] = tp.hy; fr[5] = tp.hx;
         }
         const int e = kk * TP + pl;
-#pragma unroll
-        for (int c = 0; c < 8; c++) t.w[c][e] = w[c];
         if (BWD) {
+            float4 *q = t.pk + kDwEntryVecs * e;
+            q[0] = make_float4(w[0], w[1], w[2], w[3]);
+            q[1] = make_float4(w[4], w[5], w[6], w[7]);
+            q[2] = make_float4(fr[0], fr[1], fr[2], fr[3]);
+            q[3] = make_float4(fr[4], fr[5], al, 0.f);
+        } else {
 #pragma unroll
-            for (int c = 0; c < 6; c++) t.frac[c][e] = fr[c];
-            t.alpha[e] = al;
+            for (int c = 0; c < 8; c++) t.w[c][e] = w[c];
         }
         t.idx[e] = idx;
         t.flag[e] = flag;
@@ -145,6 +152,15 @@ template <typename T> D2C_DEV void ld4(const T *p, float *v)
         const uint2 t = *reinterpret_cast<const uint2 *>(p);
         v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
         v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+}
+template <typename T> D2C_DEV void st4(T *p, const float *v)
+{
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        *reinterpret_cast<uint2 *>(p) = make_uint2((__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
+                                                   (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u));
     }
 }
 static_assert(kCV == 4, "vector loads of 4 channels");
@@ -255,26 +271,6 @@ __global__ void __launch_bounds__(kDwThreads) dw_fwd_kernel(DwArgs a)
 // ----------------------------------------------------------------- backward
 // Sum of 4 per-lane values over the 64 lanes: after the exchange steps lane
 // group (lane>>4) holds the total of value (lane>>4) in all of its lanes.
-// Load of a lane's 4 channels from a wavefront-uniform row address plus the lane's byte offset.  The row
-// address is pinned to scalar registers, so that the load needs no 64-bit vector arithmetic.
-template <typename T> D2C_DEV void ld4_row(const T *row, unsigned lane_bytes, float *v)
-{
-    typedef const __attribute__((address_space(1))) char *gptr;
-    const unsigned long long a = reinterpret_cast<unsigned long long>(row);
-    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)a);
-    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(a >> 32));
-    gptr p = (gptr)(((unsigned long long)hi << 32) | lo) + lane_bytes;
-    typedef float f32x4v __attribute__((ext_vector_type(4)));
-    typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
-    if constexpr (sizeof(T) == 4) {
-        const f32x4v t = *reinterpret_cast<const __attribute__((address_space(1))) f32x4v *>(p);
-        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
-    } else {
-        const u32x2v t = *reinterpret_cast<const __attribute__((address_space(1))) u32x2v *>(p);
-        v[0] = __uint_as_float(t[0] << 16); v[1] = __uint_as_float(t[0] & 0xffff0000u);
-        v[2] = __uint_as_float(t[1] << 16); v[3] = __uint_as_float(t[1] & 0xffff0000u);
-    }
-}
 template <int CTRL> D2C_DEV float dpp_add(float v)
 {
     return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
@@ -299,7 +295,10 @@ D2C_DEV float reduce4_over_wave(float v0, float v1, float v2, float v3, int lane
     return k;   // value index = (lane >> 5) * 2 + ((lane >> 4) & 1)
 }
 
-template <typename T>
+// GXATOM: grad_input scattered with atomics from here (the mode without sample lists).
+// `xcl` is followed by one row of zeros (voxel N * vol): corners outside the volume read it, so that their dot
+// products vanish without a select and every load of a position is made unconditionally.
+template <typename T, bool GXATOM>
 __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 wavefronts per SIMD: what the LDS allows
 {
     constexpr int TP = kBwdTP, KB = kBwdKB;
@@ -312,14 +311,26 @@ __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 
     const DwTile tl = dw_tile(s, TP, s.G * nsl, blockIdx.x);
     if (!tl.ok) return;
     const int m0 = tl.m0, m_end = tl.m_end;
-    const int HW = s.H * s.W;
     const int g = tl.y / nsl, sl = tl.y - g * nsl;
     const int cl = sl * kSlice + lane * kCV;
     const bool cok = cl < s.cpg;       // lanes past the group still take part in the reductions
     const int c = g * s.cpg + (cok ? cl : 0);
-    const T *xcl = reinterpret_cast<const T *>(a.xcl);
     const T *wt = reinterpret_cast<const T *>(a.wt);
-    const T *goutcl = reinterpret_cast<const T *>(a.goutcl);
+    const T *xcl = reinterpret_cast<const T *>(a.xcl);
+    const int HW = s.H * s.W;
+    const int zrow = s.N * s.vol;
+    // grad_out of the tile's positions, this slice's channels: every tap needs it, so it is staged in LDS once
+    // (rows past the tile and channels past the offset group: zeros)
+    T *gotile = reinterpret_cast<T *>(smem + kDwLdsTab);
+    {
+        const T *goutcl = reinterpret_cast<const T *>(a.goutcl);
+        for (int r = wave; r < TP; r += kDwThreads / 64) {
+            const int m = m0 + r;
+            float v[kCV] = {0.f, 0.f, 0.f, 0.f};
+            if (cok && m < m_end) ld4<T>(goutcl + (size_t)m * s.Cout + c, v);
+            st4<T>(gotile + r * kSlice + lane * kCV, v);
+        }
+    }
     const bool want_aux = a.auxoff != nullptr || a.auxmask != nullptr;
 
     for (int k0 = 0; k0 < s.K; k0 += KB) {
@@ -328,6 +339,7 @@ __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 
         dw_coords<true, TP, KB>(a, taps, m0, m_end, g, k0, kn);
         __syncthreads();
         for (int kk = wave; kk < kn; kk += kDwThreads / 64) {
+            // (lanes past the offset group hold a zero weight: everything they add to the sums over lanes is zero)
             float wv[kCV] = {0.f, 0.f, 0.f, 0.f};
             if (cok) ld4<T>(wt + (long)(k0 + kk) * s.Cin + c, wv);
             float gwv[kCV] = {0.f, 0.f, 0.f, 0.f};
@@ -335,25 +347,24 @@ __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 
             // whole wavefront and are read out into scalar registers
             const int vflag = taps.flag[kk * TP + (lane & (TP - 1))];
             const int vidx = taps.idx[kk * TP + (lane & (TP - 1))];
-            // The rows of a position (grad_out and the 8 corners) are requested one position ahead of their use.
-            // Every request is made: a corner out of range reads voxel 0 and its dot product is dropped, a
-            // position past the tile reads the tile's last grad_out row and has no corner in range.  Lanes past
-            // the offset group read channel 0 on and hold a zero weight.
+            // The corner rows of a position are requested one position ahead of their use.  Every request is made:
+            // a corner out of range reads the row of zeros.  Lanes past the offset group read channel 0 on.
             struct Rows {
-                float x[8][kCV], go[kCV];
+                float x[8][kCV];
             };
             unsigned cbytes = (unsigned)c * (unsigned)sizeof(T);
-            asm volatile("" : "+v"(cbytes));   // kept a plain 32-bit register: the offset operand of the loads
+            asm("" : "+v"(cbytes));   // kept a plain 32-bit register: the offset operand of the loads
             auto issue = [&](Rows &r, int p) {
+                // (made opaque here, in the block of the loads: the zero-extension of the offset then stays next to
+                // them and the loads take the scalar-base + 32-bit-offset form instead of 64-bit vector additions)
+                unsigned cb = cbytes;
+                asm("" : "+v"(cb));
                 const unsigned inr = (unsigned)__builtin_amdgcn_readlane(vflag, p) >> 8;
                 const int idx = __builtin_amdgcn_readlane(vidx, p);
-                const int m = min(m0 + p, m_end - 1);
-                // row address in scalar registers + the lane's byte offset
-                ld4_row<T>(goutcl + (size_t)m * s.Cout, cbytes, r.go);
 #pragma unroll
                 for (int cc = 0; cc < 8; cc++) {
-                    const int v = ((inr >> cc) & 1u) ? idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1) : 0;
-                    ld4_row<T>(xcl + (size_t)v * s.Cin, cbytes, r.x[cc]);
+                    const int v = ((inr >> cc) & 1u) ? idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1) : zrow;
+                    ld4_row<T>(xcl + (size_t)v * s.Cin, cb, r.x[cc]);
                 }
             };
             float stash = 0.f;
@@ -361,37 +372,42 @@ __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 
             auto compute = [&](const Rows &r, int p) {
                 const int e = kk * TP + p;
                 const unsigned flag = (unsigned)__builtin_amdgcn_readlane(vflag, p);
-                const unsigned inr = flag >> 8, live = flag & 0xffu;
+                const unsigned inr = flag >> 8, live = flag & 0xffu;   // live is 0 or inr
                 if (!inr) return;
-                const int idx = __builtin_amdgcn_readlane(vidx, p);
-                float gc[kCV];
+                // the entry's 16 floats: the same address in every lane (broadcast reads)
+                const float4 q0 = taps.pk[kDwEntryVecs * e], q1 = taps.pk[kDwEntryVecs * e + 1];
+                const float wc[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};   // a_corner * alpha, 0 where not live
+                float go[kCV], gc[kCV];
+                ld4<T>(gotile + p * kSlice + lane * kCV, go);
 #pragma unroll
-                for (int j = 0; j < kCV; j++) gc[j] = wv[j] * (cok ? r.go[j] : 0.f);
+                for (int j = 0; j < kCV; j++) gc[j] = wv[j] * go[j];
                 float dot[8];
                 float sv[kCV] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int cc = 0; cc < 8; cc++) {
-                    float d = 0.f;
+                    float d = gc[0] * r.x[cc][0];
 #pragma unroll
-                    for (int j = 0; j < kCV; j++) d = fmaf(gc[j], r.x[cc][j], d);
-                    if ((live >> cc) & 1u) {
-                        const float wc = taps.w[cc][e];   // a_corner * alpha
+                    for (int j = 1; j < kCV; j++) d = fmaf(gc[j], r.x[cc][j], d);
+                    dot[cc] = d;
 #pragma unroll
-                        for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc, r.x[cc][j], sv[j]);
-                        if (a.gxcl && cok) {
+                    for (int j = 0; j < kCV; j++) sv[j] = fmaf(wc[cc], r.x[cc][j], sv[j]);
+                    if constexpr (GXATOM) {
+                        if (((live >> cc) & 1u) && cok) {
+                            const int idx = __builtin_amdgcn_readlane(vidx, p);
                             const int v = idx + ((cc >> 2) & 1) * HW + ((cc >> 1) & 1) * s.W + (cc & 1);
                             float *gp = a.gxcl + (long)v * s.Cin + c;
 #pragma unroll
-                            for (int j = 0; j < kCV; j++) atomicAdd(gp + j, wc * gc[j]);
+                            for (int j = 0; j < kCV; j++) atomicAdd(gp + j, wc[cc] * gc[j]);
                         }
                     }
-                    dot[cc] = ((inr >> cc) & 1u) ? d : 0.f;
                 }
 #pragma unroll
-                for (int j = 0; j < kCV; j++) gwv[j] = fmaf(r.go[j], sv[j], gwv[j]);   // sv already holds alpha
+                for (int j = 0; j < kCV; j++) gwv[j] = fmaf(go[j], sv[j], gwv[j]);   // sv already holds alpha
                 if (want_aux) {
-                    const float lz = taps.frac[0][e], ly = taps.frac[1][e], lx = taps.frac[2][e];
-                    const float hz = taps.frac[3][e], hy = taps.frac[4][e], hx = taps.frac[5][e];
+                    // (read here, where the rows' registers are free again)
+                    __builtin_amdgcn_sched_barrier(0);
+                    const float4 q2 = taps.pk[kDwEntryVecs * e + 2], q3 = taps.pk[kDwEntryVecs * e + 3];
+                    const float lz = q2.x, ly = q2.y, lx = q2.z, hz = q2.w, hy = q3.x, hx = q3.y;
                     // The four results are trilinear forms of the dot products; they are taken axis by axis
                     // (x, then y, then z): interpolated sums and differences.
                     float sx[4], dx[4];   // index = z * 2 + y
@@ -410,20 +426,12 @@ __global__ void __launch_bounds__(kDwThreads, 4) dw_bwd_kernel(DwArgs a)   // 4 
                     const float gz = sxy[1] - sxy[0];
                     const float gy = fmaf(hz, dy[1], lz * dy[0]);
                     const float gxx = fmaf(hz, sdx[1], lz * sdx[0]);
-                    float gm = fmaf(hz, sxy[1], lz * sxy[0]);
-                    if (live != inr) {
-                        // the modulation gradient takes the corners of the forward pass only
-                        gm = 0.f;
-#pragma unroll
-                        for (int cc = 0; cc < 8; cc++) {
-                            const float wz = (cc & 4) ? hz : lz, wy = (cc & 2) ? hy : ly, wx = (cc & 1) ? hx : lx;
-                            if ((live >> cc) & 1u) gm += (wz * wy * wx) * dot[cc];
-                        }
-                    }
+                    // the modulation gradient takes the corners of the forward pass only: all in range, or none
+                    const float gm = live ? fmaf(hz, sxy[1], lz * sxy[0]) : 0.f;
                     // sums over the 256 channels of the slice; lane (which * 16 + p) keeps result `which` of
                     // position p until all positions of the tap are done
                     const float rs = reduce4_over_wave(gz, gy, gxx, gm, lane);
-                    const float val = lane < 48 ? taps.alpha[e] * rs : rs;
+                    const float val = lane < 48 ? q3.z * rs : rs;
                     stash = (lane & (TP - 1)) == p ? val : stash;
                 }
             };
@@ -517,7 +525,8 @@ int d2c_depthwise_forward(const TiledShape &s, const void *xcl, const void *off,
     return d2c_check_launch("dw_fwd_kernel");
 }
 
-// `goutcl` is the channels-last copy of grad_out, `wt` the weights as [K][C].  `gxcl` NULL: grad_input is not wanted
+// `goutcl` is the channels-last copy of grad_out, `wt` the weights as [K][C]; `xcl` ends with a row of zeros (voxel
+// N * vol).  `gxcl` NULL: grad_input is not wanted
 // here (or comes from the sample lists afterwards); otherwise it is accumulated with atomics.  The caller has zeroed
 // `gwacc` and `auxacc`.
 template <typename T>
@@ -534,9 +543,11 @@ int d2c_depthwise_backward(const TiledShape &s, const void *goutcl, const void *
     DwArgs a{s, xcl, off, mask, wt, nullptr, nullptr, goutcl, gxcl, auxoff, auxmask, gwacc};
     const int nsl = (s.cpg + kSlice - 1) / kSlice;
     {
-        if (int rc = d2c_allow_lds((const void *)dw_bwd_kernel<T>, (int)kDwLdsBwd, "dw_bwd_kernel")) return rc;
+        auto kern = gxcl ? &dw_bwd_kernel<T, true> : &dw_bwd_kernel<T, false>;
+        const size_t lds = dw_lds_bwd(sizeof(T));
+        if (int rc = d2c_allow_lds((const void *)kern, (int)lds, "dw_bwd_kernel")) return rc;
         D2cProfScope prof(D2C_PROF_BWD_DATA, st, "dw_bwd_kernel");
-        hipLaunchKernelGGL(dw_bwd_kernel<T>, dim3(dw_grid(s, kBwdTP, s.G * nsl)), dim3(kDwThreads), kDwLdsBwd, st, a);
+        hipLaunchKernelGGL(kern, dim3(dw_grid(s, kBwdTP, s.G * nsl)), dim3(kDwThreads), lds, st, a);
     }
     if (int rc = d2c_check_launch("dw_bwd_kernel")) return rc;
     const bool want_gw = gwacc && gw;

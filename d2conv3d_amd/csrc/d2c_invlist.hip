@@ -17,6 +17,8 @@
 //      corner weights, reads each gcol row segment once and accumulates in
 //      registers; every grad_input element is written exactly once.
 #include "d2c_mma.hpp"
+#include <utility>
+
 #include "d2c_tiled.hpp"
 
 int d2c_gx_mode();
@@ -229,6 +231,11 @@ gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, int 
 // (6.6 MB for 256 fp32 channels of 8x15x27 positions) stay in its L2.
 constexpr int kOwnVox = 4, kOwnCV = 4, kOwnSlice = 64 * kOwnCV;
 
+template <class F, int... I> D2C_DEV void for_each_const(F &&f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+
 template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
 {
     if constexpr (sizeof(T) == 4) {
@@ -241,10 +248,13 @@ template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
     }
 }
 
-template <typename T>
+// WLDS: the weights of the channel slice fit LDS (compile-time, so that the wait for a weight row is a wait for LDS
+// alone and leaves the grad_out rows in flight).
+template <typename T, bool WLDS>
 __global__ void __launch_bounds__(64 * kOwnVox)
-dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, SampleLists L, float *gxcl, int w_in_lds)
+dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, SampleLists L, float *gxcl)
 {
+    constexpr bool w_in_lds = WLDS;
     // One wavefront per 2 x 2 x 2 cube of voxels (kOwnVox cubes consecutive in x per workgroup, sharing the
     // weights of the channel slice in LDS): the lists of the 27 base voxels that reach the cube are walked once
     // each and a grad_out row is read once for all the voxels of the cube it contributes to, like
@@ -272,8 +282,10 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, SampleLists L, fl
     const T *grow = goutcl + (long)b * s.P * s.Cout;
 
     const int cl = sl * kOwnSlice + t * kOwnCV;   // first channel of this lane inside the offset group
-    const int c = g * s.cpg + cl;
     const bool cok = cl < s.cpg;                  // cpg is a multiple of kOwnCV
+    // Lanes past the offset group stay in the walk (every lane holds a list entry for the others to read) on the
+    // group's first channels and store nothing.
+    const int c = g * s.cpg + (cok ? cl : 0);
     if (w_in_lds) {
         for (int i = threadIdx.x; i < s.K * kOwnSlice; i += 64 * kOwnVox) {
             const int k = i / kOwnSlice, cc = i - k * kOwnSlice;
@@ -282,69 +294,119 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, SampleLists L, fl
         }
         __syncthreads();
     }
-    if (!valid || !cok) return;
+    if (!valid) return;
     float acc[2][2][2][kOwnCV];
 #pragma unroll
     for (int i = 0; i < 8 * kOwnCV; i++) (&acc[0][0][0][0])[i] = 0.f;
+
+    // The walk is a software pipeline, because a wavefront has nobody to hide its latencies behind (the launch is
+    // one round of 3 - 4 wavefronts per SIMD): the entries of a bucket are loaded by the lanes (lane e holds entry
+    // e, two 16-byte loads for up to 64 entries) one bucket ahead and handed out with v_readlane; the grad_out rows
+    // of kGE samples are requested while the kGE before them are worked on (C=1024, 8x15x27: 0.172 / 0.136 / 0.142 /
+    // 0.158 ms with kGE = 1 / 2 / 4 / 8; a ring of three pairs: 0.139).
+    constexpr int kGE = 2;
+    unsigned cbytes = (unsigned)c * (unsigned)sizeof(T);
+    asm("" : "+v"(cbytes));
+    auto bucket = [&](int bi, uint4 &ea, uint4 &eb, int &n, int &bin) {
+        const int rz = bi / 9, ry = (bi / 3) % 3, rx = bi % 3;
+        const bool ok = z0 - 1 + rz <= s.D - 1 && y0 - 1 + ry <= s.H - 1 && rx < nxb;
+        bin = ok ? bin_of(s, b, g, z0 - 1 + rz, y0 - 1 + ry, x0 - 1 + rx) : 0;
+        n = ok ? min(L.counts[bin], L.cap) : 0;
+        const uint4 *ep = reinterpret_cast<const uint4 *>(L.entries + (long)bin * L.cap + min(t, L.cap - 1));
+        ea = ep[0]; eb = ep[1];
+    };
+    // rows of entries e0 .. e0 + kGE - 1 of the m the lanes hold (past the last one: the last one again)
+    auto rows = [&](float (*go)[kOwnCV], const uint4 &ea, int e0, int m) {
+        unsigned cb = cbytes;
+        // (keeps the loads in the scalar-base + 32-bit-offset form; not volatile: the bucket counts stay scalar loads)
+        asm("" : "+v"(cb));
 #pragma unroll
-    for (int rz = 0; rz < 3; rz++) {
-        const int zb = z0 - 1 + rz;
-        if (zb > s.D - 1) continue;
+        for (int i = 0; i < kGE; i++) {
+            const int pp = __builtin_amdgcn_readlane((int)ea.x, min(e0 + i, m - 1));
+            ld4_row<T>(grow + (size_t)pp * s.Cout, cb, go[i]);
+        }
+    };
+    uint4 ca, cb4, na = make_uint4(0, 0, 0, 0), nb = na;
+    int cn, cbin, nn = 0, nbin = 0;
+    bucket(0, ca, cb4, cn, cbin);
+    // (one copy of the code per bucket: its place in the 3 x 3 x 3 neighbourhood decides which voxels it reaches)
+    for_each_const([&](auto BI) {
+        constexpr int bi = decltype(BI)::value;
+        constexpr int rz = bi / 9, ry = (bi / 3) % 3, rx = bi % 3;
+        // The weights with which a sample reaches its 8 corners, times its modulation: every lane works them out
+        // for the entry it holds (64 entries per instruction), the walk below reads them out with v_readlane.
+        // Corner (dz, dy, dx) of a sample filed under base voxel r = (rz, ry, rx) is cube voxel a = d + r - 1.
+        float cw[8];
+        auto corner_weights = [&](const uint4 &ea, const uint4 &eb) {
+            const float hz = __uint_as_float(ea.z), hy = __uint_as_float(ea.w), hx = __uint_as_float(eb.x);
+            const float al = __uint_as_float(eb.y);
+            const float lz = 1.f - hz, ly = 1.f - hy, lx = 1.f - hx;
+            const float zy[4] = {lz * ly * al, lz * hy * al, hz * ly * al, hz * hy * al};
 #pragma unroll
-        for (int ry = 0; ry < 3; ry++) {
-            const int yb = y0 - 1 + ry;
-            if (yb > s.H - 1) continue;
-            // the (up to) three base voxels along x are adjacent bins; each has its bucket
-            const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
+            for (int q = 0; q < 4; q++) {
+                cw[2 * q] = zy[q] * lx;
+                cw[2 * q + 1] = zy[q] * hx;
+            }
+        };
+        auto work = [&](const float (*go)[kOwnCV], const uint4 &ea, int e0, int m) {
 #pragma unroll
-            for (int rx = 0; rx < 3; rx++) {
-                if (rx >= nxb) continue;
-                const int bin = bin1 + rx;
-                const int n = min(L.counts[bin], L.cap);
-                const InvEntry *entries = L.entries + (long)bin * L.cap;
-                for (int e = 0; e < n; e += 4) {
-                    InvEntry q[4];
-                    float go[4][kOwnCV];
+            for (int i = 0; i < kGE; i++) {
+                const int e = e0 + i;
+                if (e >= m) break;
+                const int k = __builtin_amdgcn_readlane((int)ea.y, e);
+                float wk[kOwnCV];
+                if (w_in_lds) ld_vec4<T>(s_w + k * kOwnSlice + t * kOwnCV, wk);
+                else ld_vec4<T>(wt + (long)k * s.Cin + c, wk);
+                float v[kOwnCV];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        q[i] = entries[min(e + i, n - 1)];
-                        ld_vec4<T>(grow + (long)q[i].p * s.Cout + c, go[i]);
-                    }
+                for (int jj = 0; jj < kOwnCV; jj++) v[jj] = wk[jj] * go[i][jj];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        float wk[kOwnCV];
-                        if (w_in_lds) ld_vec4<T>(s_w + q[i].k * kOwnSlice + t * kOwnCV, wk);
-                        else ld_vec4<T>(wt + (long)q[i].k * s.Cin + c, wk);
-                        const float al = e + i < n ? q[i].alpha : 0.f;
-                        float v[kOwnCV];
+                for (int az = 0; az < 2; az++) {
+                    constexpr int dz0 = 1 - rz;
+                    if (az + dz0 < 0 || az + dz0 > 1) continue;
 #pragma unroll
-                        for (int jj = 0; jj < kOwnCV; jj++) v[jj] = wk[jj] * go[i][jj];
-                        // x: base x0-1 reaches voxel 0 with hx; x0 reaches (1-hx, hx); x0+1 reaches voxel 1 with 1-hx
-                        const float hz = q[i].hz, hy = q[i].hy, hx = q[i].hx;
-                        const float wx0 = rx == 0 ? hx : (rx == 2 ? 0.f : 1.f - hx);
-                        const float wx1 = rx == 0 ? 0.f : (rx == 2 ? 1.f - hx : hx);
+                    for (int ay = 0; ay < 2; ay++) {
+                        constexpr int dy0 = 1 - ry;
+                        if (ay + dy0 < 0 || ay + dy0 > 1) continue;
 #pragma unroll
-                        for (int az = 0; az < 2; az++) {
-                            if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
-                            const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
+                        for (int ax = 0; ax < 2; ax++) {
+                            constexpr int dx0 = 1 - rx;
+                            if (ax + dx0 < 0 || ax + dx0 > 1) continue;
+                            const int corner = (az + dz0) * 4 + (ay + dy0) * 2 + (ax + dx0);
+                            const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cw[corner]), e));
 #pragma unroll
-                            for (int ay = 0; ay < 2; ay++) {
-                                if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
-                                const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
-                                const float wzy = wz * wy * al;
-                                const float w0 = wzy * wx0, w1 = wzy * wx1;
-#pragma unroll
-                                for (int jj = 0; jj < kOwnCV; jj++) {
-                                    if (rx != 2) acc[az][ay][0][jj] = fmaf(w0, v[jj], acc[az][ay][0][jj]);
-                                    if (rx != 0) acc[az][ay][1][jj] = fmaf(w1, v[jj], acc[az][ay][1][jj]);
-                                }
-                            }
+                            for (int jj = 0; jj < kOwnCV; jj++) acc[az][ay][ax][jj] = fmaf(w, v[jj], acc[az][ay][ax][jj]);
                         }
                     }
                 }
             }
+        };
+        float goA[kGE][kOwnCV], goB[kGE][kOwnCV];
+        if (cn > 0) {
+            int m = min(cn, 64);
+            rows(goA, ca, 0, m);
+            if (bi + 1 < 27) bucket(bi + 1, na, nb, nn, nbin);
+            for (int base = 0;;) {
+                corner_weights(ca, cb4);
+                for (int e0 = 0; e0 < m; e0 += 2 * kGE) {
+                    rows(goB, ca, e0 + kGE, m);
+                    work(goA, ca, e0, m);
+                    rows(goA, ca, e0 + 2 * kGE, m);
+                    work(goB, ca, e0 + kGE, m);
+                }
+                // buckets of more than 64 entries (large kernels): the next 64, not ahead of time
+                base += 64;
+                if (base >= cn) break;
+                m = min(cn - base, 64);
+                const uint4 *ep = reinterpret_cast<const uint4 *>(L.entries + (long)cbin * L.cap + min(base + t, L.cap - 1));
+                ca = ep[0]; cb4 = ep[1];
+                rows(goA, ca, 0, m);
+            }
+        } else if (bi + 1 < 27) {
+            bucket(bi + 1, na, nb, nn, nbin);
         }
-    }
+        ca = na; cb4 = nb; cn = nn; cbin = nbin;
+    }, std::make_integer_sequence<int, 27>{});
 #pragma unroll
     for (int az = 0; az < 2; az++)
 #pragma unroll
@@ -352,7 +414,7 @@ dw_gx_owner_kernel(TiledShape s, const T *goutcl, const T *wt, SampleLists L, fl
 #pragma unroll
             for (int ax = 0; ax < 2; ax++) {
                 const int z = z0 + az, y = y0 + ay, x = x0 + ax;
-                if (z < s.D && y < s.H && x < s.W) {
+                if (cok && z < s.D && y < s.H && x < s.W) {
                     const long vg = (long)b * s.vol + ((long)z * s.H + y) * s.W + x;
                     *reinterpret_cast<float4 *>(gxcl + vg * s.Cin + c) =
                         make_float4(acc[az][ay][ax][0], acc[az][ay][ax][1], acc[az][ay][ax][2], acc[az][ay][ax][3]);
@@ -509,16 +571,16 @@ template <typename T>
 int d2c_dw_gx_owner_launch(const TiledShape &s, const void *goutcl, const void *wt, const SampleLists &L, float *gxcl,
                            hipStream_t st)
 {
-    if (int rc = d2c_allow_lds((const void *)dw_gx_owner_kernel<T>, 160 * 1024, "dw_gx_owner_kernel")) return rc;
-    D2cProfScope prof(D2C_PROF_GX_OWNER, st, "dw_gx_owner_kernel");
     size_t lds = (size_t)s.K * kOwnSlice * sizeof(T);
-    const int w_in_lds = lds <= 144 * 1024;
+    const bool w_in_lds = lds <= 144 * 1024;
     if (!w_in_lds) lds = 0;
+    auto kern = w_in_lds ? &dw_gx_owner_kernel<T, true> : &dw_gx_owner_kernel<T, false>;
+    if (int rc = d2c_allow_lds((const void *)kern, 160 * 1024, "dw_gx_owner_kernel")) return rc;
+    D2cProfScope prof(D2C_PROF_GX_OWNER, st, "dw_gx_owner_kernel");
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const int nslice = (s.cpg + kOwnSlice - 1) / kOwnSlice;
     const unsigned nblk = xcd_unit_grid(s.N * s.G * nslice, ncz * ncy * ((ncx + kOwnVox - 1) / kOwnVox));
-    hipLaunchKernelGGL(dw_gx_owner_kernel<T>, dim3(nblk), dim3(64 * kOwnVox), lds, st, s, (const T *)goutcl,
-                       (const T *)wt, L, gxcl, w_in_lds);
+    hipLaunchKernelGGL(kern, dim3(nblk), dim3(64 * kOwnVox), lds, st, s, (const T *)goutcl, (const T *)wt, L, gxcl);
     if (int rc = d2c_check_launch("dw_gx_owner_kernel")) return rc;
     // the overflow entries, usually none (the kernel reads their number from device memory)
     hipLaunchKernelGGL(dw_gx_overflow_kernel<T>, dim3(256), dim3(256), 0, st, s, (const T *)goutcl, (const T *)wt, L, gxcl);

@@ -567,6 +567,27 @@ __host__ __device__ inline float d2c_epilogue(float v, int act, float scale)
     return (v < lo ? lo : v) * sc;
 }
 
+// Load of a lane's 4 channels from a wavefront-uniform row address plus the lane's byte offset.  The row
+// address is pinned to scalar registers, so that the load needs no 64-bit vector arithmetic.
+template <typename T> D2C_DEV void ld4_row(const T *row, unsigned lane_bytes, float *v)
+{
+    typedef const __attribute__((address_space(1))) char *gptr;
+    const unsigned long long a = reinterpret_cast<unsigned long long>(row);
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)a);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(a >> 32));
+    gptr p = (gptr)(((unsigned long long)hi << 32) | lo) + lane_bytes;
+    typedef float f32x4v __attribute__((ext_vector_type(4)));
+    typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
+    if constexpr (sizeof(T) == 4) {
+        const f32x4v t = *reinterpret_cast<const __attribute__((address_space(1))) f32x4v *>(p);
+        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+    } else {
+        const u32x2v t = *reinterpret_cast<const __attribute__((address_space(1))) u32x2v *>(p);
+        v[0] = __uint_as_float(t[0] << 16); v[1] = __uint_as_float(t[0] & 0xffff0000u);
+        v[2] = __uint_as_float(t[1] << 16); v[3] = __uint_as_float(t[1] & 0xffff0000u);
+    }
+}
+
 // ---- sample lists: every live sample (b, g, k, p) filed under its base voxel floor(z, y, x) -------------------
 struct alignas(16) InvEntry {
     int p, k;              // output position inside the sample, tap

@@ -208,6 +208,7 @@ struct DwPrepArgs {
     const void *w;
     void *wt;
     int wC, wK, nblk_w;
+    void *zrow;                // the row of zeros behind the channels-last input (wC elements)
     uint32_t *zero;
     size_t zero_words;
     int nblk_z;
@@ -240,6 +241,8 @@ template <typename T> __global__ void __launch_bounds__(256) dw_prepare_kernel(D
         T *wt = (T *)a.wt;
         const int n = a.wC * a.wK;
         for (int i = b * 256 + threadIdx.x; i < n; i += a.nblk_w * 256) wt[i] = w[(i % a.wC) * a.wK + i / a.wC];
+        if (b == 0)
+            for (int i = threadIdx.x; i < a.wC; i += 256) ((T *)a.zrow)[i] = (T)0;
         return;
     }
     b -= a.nblk_w;
@@ -434,6 +437,7 @@ int dw_prepare(const TiledShape &s, const void *x, void *xcl, const void *gout, 
     job(a.pack[0], x, xcl, s.Cin, s.vol);
     if (gout) job(a.pack[1], gout, goutcl, s.Cout, s.P);
     a.w = w; a.wt = wt; a.wC = s.Cin; a.wK = s.K;
+    a.zrow = (T *)xcl + (size_t)s.N * s.vol * s.Cin;
     a.nblk_w = std::min((s.Cin * s.K + 255) / 256, 1024);
     a.zero = (uint32_t *)zero; a.zero_words = zero_bytes / 4;
     a.nblk_z = (int)std::min<size_t>((a.zero_words + 1023) / 1024, 2048);
@@ -451,7 +455,7 @@ bool is_depthwise(const d2c_conv3d_desc &q)
     return q.groups == q.Cin && q.Cout == q.Cin && q.Cin > 1 && d2c_depthwise_supported(tiled_shape(q));
 }
 
-// depthwise workspace: channels-last input | weights [K][C] | grad_input accumulator | grad_weight accumulator |
+// depthwise workspace: channels-last input + one row of zeros | weights [K][C] | grad_input accumulator | grad_weight accumulator |
 // channels-last grad_out | sample lists (bucket counts, buckets of 32-byte entries, overflow array)
 struct DwWs {
     size_t xcl, wt, gxcl, gwacc, auxacc, goutcl, counts, entries, ovf, total_fwd, total_bwd;
@@ -461,7 +465,7 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     const size_t es = d2c_elem_size(q.dtype);
     DwWs w;
     w.xcl = 0;
-    w.wt = d2c_align_up((size_t)s.N * s.vol * s.Cin * es);
+    w.wt = d2c_align_up(((size_t)s.N * s.vol + 1) * s.Cin * es);   // input, then a row of zeros
     w.total_fwd = w.wt + d2c_align_up((size_t)s.K * s.Cin * es);
     w.gxcl = w.total_fwd;
     w.gwacc = w.gxcl + d2c_align_up((size_t)s.N * s.vol * s.Cin * sizeof(float));
