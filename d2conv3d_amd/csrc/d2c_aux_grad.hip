@@ -48,7 +48,29 @@ struct AuxArgs {
                          //      grad-column rows (`col` == `gcol`, which nobody reads after this kernel then): N*P rows
     int g_lo, g_n;       // the offset groups [g_lo, g_lo + g_n) this launch works on (a slice of the backward pass;
                          // `gcol` and `col` then point where chunk 0 WOULD start if the buffers held all chunks)
+    unsigned xbytes;     // size of `xcl` (below 4 GiB: the matrix kernels address it with 32-bit byte offsets)
 };
+
+// Gathers through buffer descriptors.  A load whose offset lies past the descriptor's size returns zeros without
+// touching memory: a corner outside the volume, or a position without any corner in range, gets the offset
+// kOutside, and neither a branch around the load nor registers cleared beforehand are needed.
+constexpr unsigned kOutside = 0xFFFFFFF0u;
+typedef unsigned u32x4_b __attribute__((ext_vector_type(4)));
+D2C_DEV __amdgpu_buffer_rsrc_t gather_rsrc(const void *p, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);   // raw buffer of dwords
+}
+// `off` when bit `bit` of `keep` is set, kOutside otherwise (kOutside has all the bits of a 16-byte aligned offset)
+D2C_DEV unsigned offset_or_outside(unsigned off, unsigned keep, int bit)
+{
+    const unsigned drop = (unsigned)((int)(~keep << (31 - bit)) >> 31);   // all ones when the bit is clear
+    return (drop & kOutside) | off;
+}
+template <int AUX> D2C_DEV uint4 ld_gather16(__amdgpu_buffer_rsrc_t r, unsigned off)
+{
+    const u32x4_b v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, AUX);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
 
 // Sum over the 8 lanes of a position without LDS traffic: neighbours of a quad, the other pair of the quad, then
 // the other quad of the 8 (row_half_mirror: lane i reads lane 7 - i of its half row; all lanes of a quad hold the
@@ -112,8 +134,9 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
     }
     // lane = (position of the round, vector) (dot-product role)
     const int rpos = lane >> 3, ivec = lane & 7;
-    const char *xb = reinterpret_cast<const char *>(a.xcl);
+    const __amdgpu_buffer_rsrc_t xres = gather_rsrc(a.xcl, a.xbytes);
     const char *gcb = reinterpret_cast<const char *>(a.gcol);
+    const unsigned grow_bytes = (unsigned)s.M * (unsigned)(BKC * sizeof(T));   // rows of one (chunk, tap): below 4 GiB
 
     // offsets and modulation of a tap are requested while the previous tap is being worked on
     float craw[4] = {0.f, 0.f, 0.f, 1.f};
@@ -192,7 +215,9 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
 #pragma unroll 1
             for (int jj = 0; jj < cpc; jj++) {
                 const int c0 = g * s.cpg + jj * BKC;
-                const long grow = ((long)(c0 / BKC) * s.K + k) * s.M;
+                // the grad-column rows of this (chunk, tap)
+                const __amdgpu_buffer_rsrc_t gres =
+                    gather_rsrc(gcb + ((long)(c0 / BKC) * s.K + k) * (long)grow_bytes, grow_bytes);
                 uint4 xv[kRounds][8], gq[kRounds];
                 // all loads of these rounds are requested before any of them is used
 #pragma unroll
@@ -207,11 +232,11 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                     for (int c = 0; c < 8; c++) {
                         const unsigned o = (unsigned)(ib + ((c >> 2) & 1) * dzc + ((c >> 1) & 1) * dyc
                                                       + ((c & 1) ? s.Cin : -qshift * s.Cin)) * (unsigned)sizeof(T);
-                        xv[r][c] = ((inr >> c) & 1u) ? *reinterpret_cast<const uint4 *>(xb + o) : make_uint4(0, 0, 0, 0);
+                        xv[r][c] = ld_gather16<0>(xres, offset_or_outside(o, inr, c));
                     }
-                    const int m = m0 + pos;
-                    // (the grad-column row: read once by this kernel)
-                    gq[r] = inr ? ld_stream16(gcb + ((grow + m) * BKC + ivec * VEC) * (long)sizeof(T)) : make_uint4(0, 0, 0, 0);
+                    // (the grad-column row: read once by this kernel, a streaming load)
+                    const unsigned go = (unsigned)((m0 + pos) * BKC + ivec * VEC) * (unsigned)sizeof(T);
+                    gq[r] = ld_gather16<2>(gres, inr ? go : kOutside);
                 }
                 if constexpr (COL) {
                     // (a streaming store: written once, read by another kernel much later; it leaves the rows that
@@ -228,13 +253,14 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                         // (the exchange first, with every lane taking part, then the choice)
                         const float al_pos = tab_of(8, pos);
                         const float alv = live ? al_pos : 0.f;
-                        const float cz[2] = {tab_of(2, pos), tab_of(5, pos)}, cy[2] = {tab_of(3, pos), tab_of(6, pos)};
+                        const float cz[2] = {tab_of(2, pos) * alv, tab_of(5, pos) * alv}, cy[2] = {tab_of(3, pos), tab_of(6, pos)};
                         const float cx[2] = {tab_of(4, pos), tab_of(7, pos)};
+                        // (the modulation goes in first: 14 products for the 8 weights instead of 24)
+                        const float czy[4] = {cz[0] * cy[0], cz[0] * cy[1], cz[1] * cy[0], cz[1] * cy[1]};
                         VecAcc<T> va;
                         va.zero();
 #pragma unroll
-                        for (int c = 0; c < 8; c++)
-                            va.fma(((cz[c >> 2] * cy[(c >> 1) & 1]) * cx[c & 1]) * alv, xv[r][c]);
+                        for (int c = 0; c < 8; c++) va.fma(czy[c >> 1] * cx[c & 1], xv[r][c]);
                         const uint4 cv = va.pack();
                         pend_v = u32x4{cv.x, cv.y, cv.z, cv.w};
                         pend_p = m0 + pos < a.mpad
@@ -352,7 +378,7 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     // (with the size-map source `goff` is the fp32 accumulator of the size gradient)
     AuxArgs a{s, xcl, off, mask, gcol, s.ss.on ? nullptr : goff, gmask, s.ss.on ? (float *)goff : nullptr, ntile, nshare,
               lists ? *lists : SampleLists{nullptr, nullptr, nullptr, 0, 0, 0}, col, col_in_place ? (long)s.M : (long)ntile * kMT,
-              g_lo, g_n};
+              g_lo, g_n, (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T))};
     dim3 grid((unsigned)(8 * (((ntile + kWavesPerBlock - 1) / kWavesPerBlock + 7) / 8) * g_n * nshare));
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;

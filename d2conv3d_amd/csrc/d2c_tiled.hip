@@ -836,6 +836,8 @@ static bool mfma_channels_ok(const d2c_conv3d_desc &q)
     // samples a position tile meets with 32-bit byte offsets from the first one
     if ((long)q.D * q.H >= (1 << 23) || q.W >= (1 << 23)) return false;
     if ((size_t)2 * q.offset_groups * q.kd * q.kh * q.kw * 3 * q.Do * q.Ho * q.Wo * 4 >= (1ull << 32)) return false;
+    // ... and the grad-column rows of one (chunk, tap), 128 bytes per position, through a buffer descriptor
+    if ((size_t)q.N * q.Do * q.Ho * q.Wo * 128 + 256 >= (1ull << 32)) return false;
     const int bkc = bkc_of(q.dtype);
     const int cg = q.Cin / q.groups, cpg = q.Cin / q.offset_groups;
     return cg % bkc == 0 && cpg % bkc == 0;
