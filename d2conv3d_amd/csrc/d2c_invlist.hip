@@ -25,6 +25,11 @@ int d2c_gx_mode();
 
 namespace {
 
+template <class F, int... I> D2C_DEV void for_each_const(F &&f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+
 D2C_DEV int xcd_swizzle(int bid, int n)
 {
     const int x = bid & 7, idx = bid >> 3;
@@ -64,11 +69,20 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
 // a in {0, 1} with weight:  r = 0: (h, -),  r = 1: (1 - h, h),  r = 2: (-, 1 - h).
 // z and y offsets are compile-time (9 unrolled visits); the 3 base voxels along x are adjacent bins, one
 // contiguous range of entries, the x offset of an entry follows from its place in the range.
-// EB: list entries (and grad-column rows) requested together by a group of lanes: 4 at registers for 4 wavefronts per
-// SIMD, or 8 at registers for 2 -- more rows in flight per lane, which pays where the problem does not fill the
-// compute units with wavefronts anyway (see d2c_gx_owner_launch).
-template <typename T, bool COMPACT, int EB>
-__global__ void __launch_bounds__(256, EB == 4 ? 4 : 2)
+//
+// The bookkeeping of an entry is done ONCE, not by all 8 lanes of its group: a batch is 8
+// entries, lane `sub` of the group loads and unpacks entry e0 + sub and works out where its grad-column row lies and
+// the (up to 8) weights with which it reaches the cube's voxels; the others read those values with ds_swizzle (a
+// broadcast inside the 8 lanes: the LDS crossbar, no LDS memory, no vector-ALU instruction).  Per entry a lane is
+// left with the row load, the conversion of its channels and the multiply-adds: about 40 % fewer vector
+// instructions than with every lane unpacking every entry, in a kernel that waits for its vector ALU as much as for
+// memory (C=512 in 8 groups, 8x30x54: 0.415 -> 0.345 ms; float, C=256: 0.406 -> 0.308 ms).
+// RB: rows of a batch requested together (8 for bfloat16, 4 for float: measured).
+template <int J> D2C_DEV int group8_bcast(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x18 | (J << 5)); }
+template <int J> D2C_DEV float group8_bcast(float v) { return __int_as_float(group8_bcast<J>(__float_as_int(v))); }
+
+template <typename T, bool COMPACT, int RB>
+__global__ void __launch_bounds__(256, 4)
 gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, int c_lo, int c_n)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
@@ -83,7 +97,7 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, in
     const int nblk = s.N * nbz * nby * nbx, nch = c_n;
     const int xcd = blockIdx.x & 7, uidx = blockIdx.x >> 3;
     const int bq = nblk >> 3, br = nblk & 7;
-    const int cidx = c_lo + uidx % nch, bi = uidx / nch;          // channel chunk, block within the XCD's range
+    const int cidx = c_lo + uidx % nch, bi = uidx / nch;
     if (bi >= bq + (xcd < br ? 1 : 0)) return;
     int blk = xcd * bq + (xcd < br ? xcd : br) + bi;
     const int bx = blk % nbx; blk /= nbx;
@@ -91,14 +105,14 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, in
     const int bz = blk % nbz;
     const int b = blk / nbz;
     const int cx = bx * 4 + (ci & 3), cy = by * 4 + ((ci >> 2) & 3), cz = bz * 2 + (ci >> 4);
-    if (cx >= ncx || cy >= ncy || cz >= ncz) return;
+    if (cx >= ncx || cy >= ncy || cz >= ncz) return;      // (whole groups of 8 lanes leave together)
     const int x0 = cx * 2, y0 = cy * 2, z0 = cz * 2;
     const int g = (cidx * BKC) / s.cpg;
     float acc[2][2][2][VEC];
 #pragma unroll
     for (int i = 0; i < 8 * VEC; i++) (&acc[0][0][0][0])[i] = 0.f;
     const T *gbase = gcol + ((long)cidx * s.K * s.M + (long)b * s.P) * BKC + sub * VEC;
-    const int nxb = x0 + 1 < s.W ? 3 : 2;          // base voxels x0-1, x0, x0+1 (the last one only if it is a voxel)
+    const int nxb = x0 + 1 < s.W ? 3 : 2;
 
 #pragma unroll
     for (int rz = 0; rz < 3; rz++) {
@@ -108,61 +122,88 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, in
         for (int ry = 0; ry < 3; ry++) {
             const int yb = y0 - 1 + ry;
             if (yb > s.H - 1) continue;
-            // the buckets of the (up to) three bins, walked as one range: [0, em1) | [em1, em2) | [em2, e1)
             const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
             const int em1 = min(L.counts[bin1], L.cap);
             const int em2 = em1 + min(L.counts[bin1 + 1], L.cap);
             const int e1 = em2 + (nxb == 3 ? min(L.counts[bin1 + 2], L.cap) : 0);
             const uint4 *eb = reinterpret_cast<const uint4 *>(L.entries) + (long)bin1 * L.cap * (COMPACT ? 1 : 2);
-            for (int e = 0; e < e1; e += EB) {
-                InvEntry en[EB];
-                uint4 row[EB];
+            // this lane's entry of a batch (past the last one: the last one again, with weight zero), requested one
+            // batch ahead
+            uint4 q0n = make_uint4(0, 0, 0, 0), q1n = q0n;
+            auto request = [&](int e0) {
+                const int ec = max(min(e0 + sub, e1 - 1), 0);
+                const int slot = ec < em1 ? ec : (ec < em2 ? ec - em1 + L.cap : ec - em2 + 2 * L.cap);
+                if constexpr (COMPACT) {
+                    q0n = eb[slot];
+                } else {
+                    q0n = eb[2 * slot]; q1n = eb[2 * slot + 1];
+                }
+            };
+            if (e1 > 0) request(0);
+            for (int e0 = 0; e0 < e1; e0 += 8) {
+                const int ei = e0 + sub, ec = min(ei, e1 - 1);
+                InvEntry en;
+                if constexpr (COMPACT) {
+                    en = unpack_entry(q0n);
+                } else {
+                    en.p = (int)q0n.x; en.k = (int)q0n.y;
+                    en.hz = __uint_as_float(q0n.z); en.hy = __uint_as_float(q0n.w);
+                    en.hx = __uint_as_float(q1n.x); en.alpha = __uint_as_float(q1n.y);
+                }
+                request(e0 + 8);
+                const int rowi = en.k * s.M + en.p;          // (N * G * K * P is below 2^31: d2c_lists_supported)
+                const float al = ei < e1 ? en.alpha : 0.f;
+                const float hz = en.hz, hy = en.hy, hx = en.hx;
+                // x: offset 0 (base x0-1) reaches voxel c=0 with hx; 1 reaches (1-hx, hx); 2 reaches c=1 with 1-hx
+                const bool r0 = ec < em1, r2 = ec >= em2;
+                const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
+                const float wx1 = r0 ? 0.f : (r2 ? 1.f - hx : hx);
+                float wq[2][2][2];
 #pragma unroll
-                for (int i = 0; i < EB; i++) {
-                    const int ei = min(e + i, e1 - 1);
-                    const int slot = ei < em1 ? ei : (ei < em2 ? ei - em1 + L.cap : ei - em2 + 2 * L.cap);
-                    if constexpr (COMPACT) {
-                        en[i] = unpack_entry(eb[slot]);
-                    } else {
-                        const uint4 q0 = eb[2 * slot], q1 = eb[2 * slot + 1];
-                        en[i].p = (int)q0.x; en[i].k = (int)q0.y;
-                        en[i].hz = __uint_as_float(q0.z); en[i].hy = __uint_as_float(q0.w);
-                        en[i].hx = __uint_as_float(q1.x); en[i].alpha = __uint_as_float(q1.y);
+                for (int az = 0; az < 2; az++) {
+                    if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
+                    const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
+#pragma unroll
+                    for (int ay = 0; ay < 2; ay++) {
+                        if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
+                        const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
+                        const float wzy = wz * wy * al;
+                        wq[az][ay][0] = wzy * wx0;
+                        wq[az][ay][1] = wzy * wx1;
                     }
                 }
+                // ---- the 8 entries of the batch, RB rows at a time
+                for_each_const([&](auto H) {
+                    constexpr int h = decltype(H)::value * RB;
+                    uint4 row[RB];
+                    for_each_const([&](auto I) {
+                        constexpr int i = decltype(I)::value;
+                        const int rj = group8_bcast<h + i>(rowi);
+                        row[i] = *reinterpret_cast<const uint4 *>(gbase + (long)rj * BKC);
+                    }, std::make_integer_sequence<int, RB>{});
+                    for_each_const([&](auto I) {
+                        constexpr int i = decltype(I)::value;
+                        const T *re = reinterpret_cast<const T *>(&row[i]);
+                        float rv[VEC];
 #pragma unroll
-                for (int i = 0; i < EB; i++)
-                    row[i] = *reinterpret_cast<const uint4 *>(gbase + ((long)en[i].k * s.M + en[i].p) * BKC);
+                        for (int j = 0; j < VEC; j++) rv[j] = elem_to_f32<T>(re[j]);
 #pragma unroll
-                for (int i = 0; i < EB; i++) {
-                    const float hz = en[i].hz, hy = en[i].hy, hx = en[i].hx;
-                    const float al = e + i < e1 ? en[i].alpha : 0.f;
-                    // x: offset 0 (base x0-1) reaches voxel c=0 with hx; 1 reaches (1-hx, hx); 2 reaches c=1 with 1-hx
-                    const bool r0 = e + i < em1, r2 = e + i >= em2;
-                    const float wx0 = r0 ? hx : (r2 ? 0.f : 1.f - hx);
-                    const float wx1 = r0 ? 0.f : (r2 ? 1.f - hx : hx);
-                    const T *re = reinterpret_cast<const T *>(&row[i]);
-                    float rv[VEC];
+                        for (int az = 0; az < 2; az++) {
+                            if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
 #pragma unroll
-                    for (int j = 0; j < VEC; j++) rv[j] = elem_to_f32<T>(re[j]);
+                            for (int ay = 0; ay < 2; ay++) {
+                                if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
+                                const float w0 = group8_bcast<h + i>(wq[az][ay][0]);
+                                const float w1 = group8_bcast<h + i>(wq[az][ay][1]);
 #pragma unroll
-                    for (int az = 0; az < 2; az++) {
-                        if ((rz == 0 && az == 1) || (rz == 2 && az == 0)) continue;
-                        const float wz = (rz == 0) ? hz : (rz == 2 ? 1.f - hz : (az ? hz : 1.f - hz));
-#pragma unroll
-                        for (int ay = 0; ay < 2; ay++) {
-                            if ((ry == 0 && ay == 1) || (ry == 2 && ay == 0)) continue;
-                            const float wy = (ry == 0) ? hy : (ry == 2 ? 1.f - hy : (ay ? hy : 1.f - hy));
-                            const float wzy = wz * wy * al;
-                            const float w0 = wzy * wx0, w1 = wzy * wx1;
-#pragma unroll
-                            for (int j = 0; j < VEC; j++) {
-                                acc[az][ay][0][j] = fmaf(w0, rv[j], acc[az][ay][0][j]);
-                                acc[az][ay][1][j] = fmaf(w1, rv[j], acc[az][ay][1][j]);
+                                for (int j = 0; j < VEC; j++) {
+                                    acc[az][ay][0][j] = fmaf(w0, rv[j], acc[az][ay][0][j]);
+                                    acc[az][ay][1][j] = fmaf(w1, rv[j], acc[az][ay][1][j]);
+                                }
                             }
                         }
-                    }
-                }
+                    }, std::make_integer_sequence<int, RB>{});
+                }, std::make_integer_sequence<int, 8 / RB>{});
             }
         }
     }
@@ -230,11 +271,6 @@ gx_overflow_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, int 
 // of one batch element at a time, so that the grad_out rows its workgroups gather
 // (6.6 MB for 256 fp32 channels of 8x15x27 positions) stay in its L2.
 constexpr int kOwnVox = 4, kOwnCV = 4, kOwnSlice = 64 * kOwnCV;
-
-template <class F, int... I> D2C_DEV void for_each_const(F &&f, std::integer_sequence<int, I...>)
-{
-    (f(std::integral_constant<int, I>{}), ...);
-}
 
 template <typename T> D2C_DEV void ld_vec4(const T *p, float *v)
 {
@@ -546,18 +582,9 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
     dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * c_n));    // see the kernel's unit mapping
-    // Eight rows in flight per group of lanes where several channel chunks of an offset group walk the same lists
-    // (bfloat16): the lists then come from L2 and the rows' latency is what the kernel waits for (N=2, C=256, one
-    // offset group: 0.30 -> 0.23 ms; 207360 positions: 1.78 -> 1.59 ms).  With one chunk per offset group (C=512 in 8
-    // groups: 0.40 -> 0.45 ms) and for float problems (0.39 -> 0.41 ms) the wavefront lost per SIMD costs more.
-    const int eb = (sizeof(T) == 2 && s.cpg / BKC >= 2) ? 8 : 4;
-    if (eb == 8) {
-        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
-        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 8>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
-    } else {
-        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
-        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, 4>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
-    }
+    constexpr int RB = sizeof(T) == 2 ? 8 : 4;
+    if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, RB>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+    else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, RB>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
     if (int rc = d2c_check_launch("gx_owner_kernel")) return rc;
     // the overflow entries, usually none (the kernel reads their number from device memory)
     hipLaunchKernelGGL(gx_overflow_kernel<T>, dim3(512), dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
