@@ -467,6 +467,10 @@ def main():
                     help="3-D matrix-core workloads: keep a prepared region (d2c_conv3d_*_prepared) the way a layer would: "
                          "'train' = the backward call reuses the input copy its forward call made (weights change every "
                          "step); 'infer' = forward calls also reuse the re-ordered weights")
+    ap.add_argument("--columns", choices=["on", "off"], default="on",
+                    help="keep the forward call's sampled columns for the backward call of the step where the "
+                         "description is served (d2c_conv3d_forward_columns / _backward_columns; the Python layer's "
+                         "default), or let the backward pass sample again")
     ap.add_argument("--f32-split-backward", action="store_true",
                     help="float32 matrix-core workloads: the backward matrix kernels on two-term bfloat16 operands too "
                          "(D2C_BWD_F32_SPLIT; gradients with ~4e-6 relative error of their scale)")
@@ -540,6 +544,17 @@ def main():
         nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
         ws = torch.empty(max(nf, nb, 256), dtype=torch.uint8, device=dev)
 
+    # The sampled columns of the forward call, kept for the backward call of the step (what the Python layer does by
+    # default where the description is served): d2c_conv3d_forward_columns / _backward_columns.
+    kept_cols = None
+    if args.columns == "on" and nd == 3 and c["backward"] and args.prepared == "off" and args.grad_weight_mode == 1 \
+            and not args.backward_slices:
+        zdesc = ctypes.byref(sdesc) if sized else None
+        ncol = lib.d2c_conv3d_columns_bytes(ctypes.byref(desc), zdesc)
+        if ncol:
+            kept_cols = torch.empty(ncol, dtype=torch.uint8, device=dev)
+            nb = lib.d2c_conv3d_backward_columns_workspace_bytes(ctypes.byref(desc), zdesc)
+
     prep = None
     if args.prepared != "off" and nd == 3 and not sized:
         npre = lib.d2c_conv3d_prepared_bytes(ctypes.byref(desc))
@@ -548,6 +563,10 @@ def main():
     fwd_reuse = [0]
 
     def forward():
+        if kept_cols is not None:
+            _lib.check(lib.d2c_conv3d_forward_columns(ctypes.byref(desc), zdesc, p(x), p(size if sized else off), p(m), p(w),
+                                                      p(b), p(out), p(kept_cols), kept_cols.numel(), p(ws), nf, cur[0]), "forward")
+            return
         if prep is not None:
             _lib.check(lib.d2c_conv3d_forward_prepared(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(prep),
                                                        prep.numel(), fwd_reuse[0], p(ws), nf, cur[0]), "forward")
@@ -561,6 +580,12 @@ def main():
         _lib.check(f_fwd(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, cur[0]), "forward")
 
     def backward():
+        if kept_cols is not None:
+            _lib.check(lib.d2c_conv3d_backward_columns(ctypes.byref(desc), zdesc, p(gout), p(x), p(size if sized else off),
+                                                       p(m), p(w), p(kept_cols), kept_cols.numel(), p(gx),
+                                                       p(gsize if sized else goff), p(gm), p(gw), p(gb), p(ws), nb,
+                                                       cur[0]), "backward")
+            return
         if prep is not None:
             _lib.check(lib.d2c_conv3d_backward_prepared(ctypes.byref(desc), p(gout), p(x), p(off), p(m), p(w), p(gx), p(goff),
                                                         p(gm), p(gw), p(gb), p(prep), prep.numel(), _lib.REUSE_INPUT, p(ws),
@@ -694,7 +719,9 @@ def main():
         per = {}
         for kname, r in role.items():
             if r == "bwd_aux":
-                cols = rows if (dt == "bf16" and nd == 3 and args.grad_weight_mode >= 1 and (C // groups) % 128 == 0) else 0
+                # (the sampled columns it writes -- unless the forward call kept them)
+                cols = rows if (dt == "bf16" and nd == 3 and args.grad_weight_mode >= 1 and (C // groups) % 128 == 0
+                                and kept_cols is None) else 0
                 aux = N * P * K * G * (nd + 1) * es
                 per[kname] = rows + cols + N * P * C * es + 2 * aux + N * P * K * G * (16 if dt == "bf16" else 32)
             elif r == "gx_owner":
@@ -739,6 +766,7 @@ def main():
                    "offset_axes": args.offset_axes,
                    "grad_input_mode": args.grad_input_mode, "grad_weight_mode": args.grad_weight_mode,
                    "backward_slices": args.backward_slices, "prepared_region": args.prepared if prep is not None else "off",
+                   "columns_kept_for_backward_mbytes": round(kept_cols.numel() / 1e6, 1) if kept_cols is not None else 0,
                    "f32_split_backward": bool(args.f32_split_backward),
                    "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
                    "graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,

@@ -20,6 +20,8 @@ EXPORTS = (
     "d2c_conv3d_forward_workspace_bytes", "d2c_conv3d_backward_workspace_bytes",
     "d2c_conv3d_forward", "d2c_conv3d_backward", "d2c_conv3d_forward_static", "d2c_static_workspace_bytes",
     "d2c_conv3d_prepared_bytes", "d2c_conv3d_forward_prepared", "d2c_conv3d_backward_prepared",
+    "d2c_conv3d_columns_bytes", "d2c_conv3d_forward_columns", "d2c_conv3d_backward_columns_workspace_bytes",
+    "d2c_conv3d_backward_columns",
     "d2c_conv1d_check", "d2c_conv1d_algo", "d2c_conv1d_forward_workspace_bytes", "d2c_conv1d_backward_workspace_bytes",
     "d2c_conv1d_forward", "d2c_conv1d_backward", "d2c_conv3d_corner_index", "d2c_conv3d_sample",
     "d2c_conv3d_offset_histogram",
@@ -130,6 +132,14 @@ def load():
     lib.d2c_conv3d_forward_prepared.restype = ctypes.c_int
     lib.d2c_conv3d_backward_prepared.argtypes = [p3] + [vp] * 10 + [vp, sz, i32, vp, sz, vp]
     lib.d2c_conv3d_backward_prepared.restype = ctypes.c_int
+    # (the second argument: a pointer to a size-map description, or None)
+    lib.d2c_conv3d_columns_bytes.argtypes, lib.d2c_conv3d_columns_bytes.restype = [p3, vp], sz
+    lib.d2c_conv3d_backward_columns_workspace_bytes.argtypes = [p3, vp]
+    lib.d2c_conv3d_backward_columns_workspace_bytes.restype = sz
+    lib.d2c_conv3d_forward_columns.argtypes = [p3, vp] + [vp] * 6 + [vp, sz, vp, sz, vp]
+    lib.d2c_conv3d_forward_columns.restype = ctypes.c_int
+    lib.d2c_conv3d_backward_columns.argtypes = [p3, vp] + [vp] * 5 + [vp, sz] + [vp] * 5 + [vp, sz, vp]
+    lib.d2c_conv3d_backward_columns.restype = ctypes.c_int
     lib.d2c_conv1d_algo.argtypes, lib.d2c_conv1d_algo.restype = [p1], ctypes.c_int
     lib.d2c_conv3d_corner_index.argtypes = [p3, vp, vp, vp, vp]
     lib.d2c_conv3d_corner_index.restype = ctypes.c_int

@@ -145,6 +145,27 @@ class PreparedRegion:
         return (t.data_ptr(), t._version, tuple(t.shape), t.dtype)
 
 
+# The sampled columns of a forward call kept for its backward call (d2c_conv3d_forward_columns): taps x the size of
+# the input, held from the forward to the backward pass of a step, in exchange for the backward pass's second
+# sampling pass.  On where the description is served, grad_weight is wanted and the buffer stays under the limit.
+_KEEP_COLUMNS = {"on": True, "max_bytes": 4 << 30}
+
+
+def _set_keep_columns(on=True, max_bytes=None):
+    _KEEP_COLUMNS["on"] = bool(on)
+    if max_bytes is not None:
+        _KEEP_COLUMNS["max_bytes"] = int(max_bytes)
+
+
+def _columns_for(lib, desc, sdesc, weight_grad_wanted, dev):
+    if not (_KEEP_COLUMNS["on"] and weight_grad_wanted):
+        return None
+    n = lib.d2c_conv3d_columns_bytes(ctypes.byref(desc), ctypes.byref(sdesc) if sdesc is not None else None)
+    if n == 0 or n > _KEEP_COLUMNS["max_bytes"]:
+        return None
+    return torch.empty(n, dtype=torch.uint8, device=dev)
+
+
 class _DeformConv3dFunction(torch.autograd.Function):
     """DeformConv3dFunction of dconv3d.h:70-186.  `relu_scale` > 0 (not in the reference) makes the forward
     kernels store relu_scale * max(out, 0) -- the activation that follows the convolution, fused into their last
@@ -174,6 +195,7 @@ class _DeformConv3dFunction(torch.autograd.Function):
             ws = _workspace(nb, dev)
             npre = lib.d2c_conv3d_prepared_bytes(ctypes.byref(desc)) if (prepared is not None and not want_stats) else 0
             ctx.prepared = None
+            columns = None
             if want_stats:
                 rc = lib.d2c_conv3d_forward_stats(ctypes.byref(desc), None, _ptr(input), _ptr(offset), _ptr(alpha),
                                                   _ptr(weight), _ptr(bias), _ptr(out), _ptr(stats), _ptr(ws), nb,
@@ -191,10 +213,16 @@ class _DeformConv3dFunction(torch.autograd.Function):
                 prepared.input_token += 1
                 ctx.prepared, ctx.input_token = prepared, prepared.input_token
             else:
-                rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha), _ptr(weight),
-                                            _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
+                columns = _columns_for(lib, desc, None, ctx.needs_input_grad[3], dev)
+                if columns is not None:
+                    rc = lib.d2c_conv3d_forward_columns(ctypes.byref(desc), None, _ptr(input), _ptr(offset), _ptr(alpha),
+                                                        _ptr(weight), _ptr(bias), _ptr(out), _ptr(columns),
+                                                        columns.numel(), _ptr(ws), nb, _stream(dev))
+                else:
+                    rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), _ptr(offset), _ptr(alpha),
+                                                _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d forward")
-        ctx.save_for_backward(input, offset, alpha, weight, bias, out if relu_scale > 0 else None)
+        ctx.save_for_backward(input, offset, alpha, weight, bias, out if relu_scale > 0 else None, columns)
         ctx.desc = desc
         ctx.relu_scale = float(relu_scale)
         if want_stats:
@@ -206,7 +234,7 @@ class _DeformConv3dFunction(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, grad_out, _grad_stats=None):
         lib = _lib.load()
-        input, offset, alpha, weight, bias, out = ctx.saved_tensors
+        input, offset, alpha, weight, bias, out, columns = ctx.saved_tensors
         desc = ctx.desc
         dev = input.device
         grad_out = grad_out.contiguous().to(input.dtype)
@@ -220,9 +248,16 @@ class _DeformConv3dFunction(torch.autograd.Function):
         gb = torch.empty_like(bias) if (bias is not None and need[4]) else None
         prepared = getattr(ctx, "prepared", None)
         with torch.cuda.device(dev):
-            nb = lib.d2c_conv3d_backward_workspace_bytes(ctypes.byref(desc))
+            nb = (lib.d2c_conv3d_backward_columns_workspace_bytes(ctypes.byref(desc), None) if columns is not None
+                  else lib.d2c_conv3d_backward_workspace_bytes(ctypes.byref(desc)))
             ws = _workspace(nb, dev)
-            if prepared is not None and prepared.buf is not None:
+            if columns is not None:
+                # (the columns the forward call of this step kept: no second sampling pass)
+                rc = lib.d2c_conv3d_backward_columns(ctypes.byref(desc), None, _ptr(grad_out), _ptr(input), _ptr(offset),
+                                                     _ptr(alpha), _ptr(weight), _ptr(columns), columns.numel(),
+                                                     _ptr(gx), _ptr(goff), _ptr(galpha), _ptr(gw), _ptr(gb), _ptr(ws),
+                                                     nb, _stream(dev))
+            elif prepared is not None and prepared.buf is not None:
                 # (the region still holds this call's input unless another forward call has used it since)
                 wkey = PreparedRegion.key(weight)
                 reuse = (_lib.REUSE_INPUT if prepared.input_token == ctx.input_token else 0) | \
@@ -291,16 +326,23 @@ class _DeformConv3dSizedFunction(torch.autograd.Function):
             nb = (lib.d2c_conv3d_forward_stats_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc)) if want_stats
                   else lib.d2c_conv3d_sized_forward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc)))
             ws = _workspace(nb, dev)
+            columns = None
             if want_stats:
                 rc = lib.d2c_conv3d_forward_stats(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input), _ptr(size_raw),
                                                   _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out), _ptr(stats),
                                                   _ptr(ws), nb, _stream(dev))
             else:
-                rc = lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input), _ptr(size_raw),
-                                                  _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), nb,
-                                                  _stream(dev))
+                columns = _columns_for(lib, desc, sdesc, ctx.needs_input_grad[3], dev)
+                if columns is not None:
+                    rc = lib.d2c_conv3d_forward_columns(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input),
+                                                        _ptr(size_raw), _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out),
+                                                        _ptr(columns), columns.numel(), _ptr(ws), nb, _stream(dev))
+                else:
+                    rc = lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(input),
+                                                      _ptr(size_raw), _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(out),
+                                                      _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d_sized forward")
-        ctx.save_for_backward(input, size_raw, alpha, weight, bias, out if relu_scale > 0 else None)
+        ctx.save_for_backward(input, size_raw, alpha, weight, bias, out if relu_scale > 0 else None, columns)
         ctx.desc, ctx.sdesc = desc, sdesc
         ctx.relu_scale = float(relu_scale)
         if want_stats:
@@ -312,7 +354,7 @@ class _DeformConv3dSizedFunction(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, grad_out, _grad_stats=None):
         lib = _lib.load()
-        input, size_raw, alpha, weight, bias, out = ctx.saved_tensors
+        input, size_raw, alpha, weight, bias, out, columns = ctx.saved_tensors
         desc, sdesc = ctx.desc, ctx.sdesc
         dev = input.device
         grad_out = grad_out.contiguous().to(input.dtype)
@@ -325,11 +367,19 @@ class _DeformConv3dSizedFunction(torch.autograd.Function):
         gw = torch.empty_like(weight) if need[3] else None
         gb = torch.empty_like(bias) if (bias is not None and need[4]) else None
         with torch.cuda.device(dev):
-            nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
-            ws = _workspace(nb, dev)
-            rc = lib.d2c_conv3d_sized_backward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(grad_out), _ptr(input),
-                                               _ptr(size_raw), _ptr(alpha), _ptr(weight), _ptr(gx), _ptr(gsize),
-                                               _ptr(galpha), _ptr(gw), _ptr(gb), _ptr(ws), nb, _stream(dev))
+            if columns is not None:
+                nb = lib.d2c_conv3d_backward_columns_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_backward_columns(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(grad_out), _ptr(input),
+                                                     _ptr(size_raw), _ptr(alpha), _ptr(weight), _ptr(columns),
+                                                     columns.numel(), _ptr(gx), _ptr(gsize), _ptr(galpha), _ptr(gw),
+                                                     _ptr(gb), _ptr(ws), nb, _stream(dev))
+            else:
+                nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_sized_backward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(grad_out), _ptr(input),
+                                                   _ptr(size_raw), _ptr(alpha), _ptr(weight), _ptr(gx), _ptr(gsize),
+                                                   _ptr(galpha), _ptr(gw), _ptr(gb), _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d_sized backward")
         return (gx, gsize, galpha, gw, gb) + (None,) * 8
 
@@ -661,6 +711,9 @@ config = types.SimpleNamespace(
     release_workspaces=_release_workspaces,
     set_workspace_caching=_set_workspace_caching,
     cached_workspace_bytes=_workspace_bytes_cached,
+    # not in the reference: whether forward calls keep their sampled columns for the backward call (and up to what size)
+    set_keep_columns=_set_keep_columns,
+    keep_columns=lambda: dict(_KEEP_COLUMNS),
 )
 
 

@@ -627,6 +627,63 @@ int d2c_conv3d_forward_stats(const d2c_conv3d_desc *q, const d2c_size_map_desc *
     return d2c_channel_stats(&g, out, chan_stats, stream);
 }
 
+// ---- the sampled columns of a forward call, kept for the backward call of the same step
+static bool columns_served(const d2c_conv3d_desc &q, const d2c_size_map_desc *z)
+{
+    return choose_algo(q, true) == D2C_ALGO_MFMA && (!z || (sized_fused(q, false) && sized_fused(q, true))) &&
+           d2c_tiled_columns_bytes(q, z) > 0;
+}
+
+size_t d2c_conv3d_columns_bytes(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
+{
+    if ((z ? sized_check(q, z) : d2c_conv3d_check(q)) != D2C_OK) return 0;
+    return columns_served(*q, z) ? d2c_tiled_columns_bytes(*q, z) : 0;
+}
+
+static int check_columns(const d2c_conv3d_desc &q, const d2c_size_map_desc *z, const void *columns, size_t columns_bytes)
+{
+    const size_t need = columns_served(q, z) ? d2c_tiled_columns_bytes(q, z) : 0;
+    if (need == 0) {
+        d2c_set_error("this description keeps no columns (d2c_conv3d_columns_bytes is 0): use the plain calls");
+        return D2C_ERR_UNSUPPORTED;
+    }
+    if (!columns || columns_bytes < need || ((uintptr_t)columns & 255u)) {
+        d2c_set_error("column buffer of %zu bytes (256-byte aligned) required, got %zu at %p", need, columns_bytes, columns);
+        return D2C_ERR_WORKSPACE;
+    }
+    return D2C_OK;
+}
+
+int d2c_conv3d_forward_columns(const d2c_conv3d_desc *q, const d2c_size_map_desc *z, const void *x, const void *offset,
+                               const void *mask, const void *weight, const void *bias, void *out, void *columns,
+                               size_t columns_bytes, void *ws, size_t ws_bytes, void *stream)
+{
+    if (int rc = z ? sized_check(q, z) : d2c_conv3d_check(q)) return rc;
+    if (!x || !offset || !weight || !out) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (int rc = check_columns(*q, z, columns, columns_bytes)) return rc;
+    if (int rc = check_ws(d2c_tiled_forward_ws(*q), ws, ws_bytes)) return rc;
+    return d2c_tiled_forward(*q, x, offset, mask, weight, bias, out, ws, (hipStream_t)stream, z, nullptr, nullptr, columns);
+}
+
+size_t d2c_conv3d_backward_columns_workspace_bytes(const d2c_conv3d_desc *q, const d2c_size_map_desc *z)
+{
+    if ((z ? sized_check(q, z) : d2c_conv3d_check(q)) != D2C_OK || !columns_served(*q, z)) return 0;
+    return d2c_tiled_backward_ws(*q, z, true);
+}
+
+int d2c_conv3d_backward_columns(const d2c_conv3d_desc *q, const d2c_size_map_desc *z, const void *gout, const void *x,
+                                const void *offset, const void *mask, const void *weight, const void *columns,
+                                size_t columns_bytes, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws,
+                                size_t ws_bytes, void *stream)
+{
+    if (int rc = z ? sized_check(q, z) : d2c_conv3d_check(q)) return rc;
+    if (!gout || !x || !offset || !weight) { d2c_set_error("null tensor pointer"); return D2C_ERR_SHAPE; }
+    if (int rc = check_columns(*q, z, columns, columns_bytes)) return rc;
+    if (int rc = check_ws(d2c_tiled_backward_ws(*q, z, true), ws, ws_bytes)) return rc;
+    return d2c_tiled_backward(*q, gout, x, offset, mask, weight, gx, goff, gmask, gw, gb, ws, (hipStream_t)stream, z,
+                              nullptr, columns);
+}
+
 int d2c_conv3d_corner_index(const d2c_conv3d_desc *q, const void *offset, int32_t *base, uint8_t *flags,
                             void *stream)
 {

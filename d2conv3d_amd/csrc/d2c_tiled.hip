@@ -7,7 +7,10 @@
 int d2c_fwd_out_tile(int og, int M, int groups);
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
-                         const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part);
+                         const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part,
+                         void *col = nullptr);
+bool d2c_fwd_writes_columns(const TiledShape &s, int dtype);
+long d2c_columns_rows(const TiledShape &s);
 bool d2c_fwd_fills_stats(const TiledShape &s);
 size_t d2c_fwd_stats_ws(const TiledShape &s);
 int d2c_fwd_split(const TiledShape &s);
@@ -484,7 +487,7 @@ DwWs dw_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 template <typename T>
 int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
               const void *bias, void *out, void *ws, hipStream_t st, int nd = 3, const d2c_size_map_desc *sz = nullptr,
-              float *stats = nullptr, const D2cPrepared *prep = nullptr)
+              float *stats = nullptr, const D2cPrepared *prep = nullptr, void *columns = nullptr)
 {
     const TiledShape s = tiled_shape(q, nd, 0, sz);
     char *base = (char *)ws;
@@ -518,7 +521,7 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
     if (int rc = d2c_check_launch("pack_weight_fwd_kernel")) return rc;
     // (the per-tile sums of the output statistics go behind everything else in the workspace)
     return d2c_tiled_fwd_launch<T>(s, xcl_p, off, mask, wp_p, bias, out, (float *)(base + l.outacc), st,
-                                   stats, stats ? (float *)(base + l.total) : nullptr);
+                                   stats, stats ? (float *)(base + l.total) : nullptr, columns);
 }
 
 // grad_input by sample lists (see d2c_invlist.hip) needs the whole reduction over output
@@ -578,7 +581,8 @@ BwdSlices bwd_slices(const d2c_conv3d_desc &q, const TiledShape &s)
 struct BwdWs {
     size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, gsacc, sm1, col, total;
 };
-BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
+// `saved_columns`: the caller brings the sampled columns of the forward call (no column region, no slices)
+BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s, bool saved_columns = false)
 {
     const size_t es = d2c_elem_size(q.dtype);
     BwdWs w;
@@ -596,7 +600,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     if (d2c_bwd_data_split(s, q.dtype) > 1 || !d2c_tiled_bwd_single_pass(s, q.dtype))
         w.total += d2c_align_up((size_t)s.N * s.G * s.K * s.P * (s.nd + 1) * sizeof(float));
     w.gcol = w.counts = w.entries = w.ovf = 0;
-    const BwdSlices sl = bwd_slices(q, s);
+    const BwdSlices sl = saved_columns ? BwdSlices{0, 0} : bwd_slices(q, s);
     if (use_lists(q, s) || use_aux_kernel(q, s)) {
         w.gcol = w.total;
         // (+ 64 rows behind the last one: what the last tile of the grad-weight product reads when the columns took
@@ -618,7 +622,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
     w.sm1 = w.total;       // ... and (size - 1) per axis
     if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
     w.col = w.total;       // sampled columns for the grad-weight product
-    if (use_col_weight(q, s) && !col_in_place(q, s))
+    if (!saved_columns && use_col_weight(q, s) && !col_in_place(q, s))
         w.total += d2c_align_up(d2c_bwd_col_bytes(s, sl.cgs ? sl.cgs * (s.cpg / 64) : 0));
     return w;
 }
@@ -626,7 +630,8 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s)
 template <typename T>
 int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off, const void *mask,
                const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb, void *ws, hipStream_t st,
-               int nd = 3, int quirks = 0, const d2c_size_map_desc *sz = nullptr, const D2cPrepared *prep = nullptr)
+               int nd = 3, int quirks = 0, const d2c_size_map_desc *sz = nullptr, const D2cPrepared *prep = nullptr,
+               const void *columns = nullptr)
 {
     TiledShape s = tiled_shape(q, nd, quirks, sz);
     char *base = (char *)ws;
@@ -662,7 +667,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         }
         return D2C_OK;
     }
-    const BwdWs l = bwd_ws(q, s);
+    const BwdWs l = bwd_ws(q, s, columns != nullptr);
     const PreparedLayout pl = prepared_layout(q, s);
     char *xcl_p = prep ? (char *)prep->base + pl.xcl : base + l.xcl;
     // (the transposed weights of the region serve single-pass reductions; wider weight groups re-pack per pass)
@@ -685,7 +690,9 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         off = sm1;
     }
     bool gw_from_col = false, gw_in_place = false, gw_done = false;
-    const BwdSlices sl = bwd_slices(q, s);
+    // (`columns`: the sampled columns the forward call kept -- the offset / mask gradient kernel then writes none, the
+    // grad-weight product takes these, and the settings that save workspace by other means do not apply)
+    const BwdSlices sl = columns ? BwdSlices{0, 0} : bwd_slices(q, s);
     if ((gx || goff || gmask) && sl.gs > 0) {
         // Slice by slice over the offset groups: the grad-column rows of a slice are made, read by the offset / mask
         // gradient kernel (which files the slice's samples and writes its sampled columns) and by the grad_input
@@ -758,10 +765,10 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                 D2cProfScope prof(D2C_PROF_PACK, st);
                 d2c_fill_zero(goff_k, (size_t)s.N * 3 * s.P * sizeof(float), st);
             }
-            gw_from_col = gw && auxk && use_col_weight(q, s);
+            gw_from_col = gw && (columns ? d2c_bwd_weight_from_col(s, q.dtype) : (auxk && use_col_weight(q, s)));
             // (the sampled columns over the grad-column rows: grad_input has to be done with the rows before the
             // offset / mask gradient kernel runs, so the samples are filed by a pass of their own)
-            gw_in_place = gw_from_col && col_in_place(q, s);
+            gw_in_place = gw_from_col && !columns && col_in_place(q, s);
             SampleLists L{nullptr, nullptr, nullptr, 0, 0, 0};
             if (lists) {
                 L = d2c_lists_make(s, Elem<T>::DT, base + l.counts, base + l.entries, base + l.ovf);
@@ -782,7 +789,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             if (auxk)
                 if (int rc = d2c_aux_grad_launch<T>(s, xcl_p, off, mask, base + l.gcol, goff_k, gmask,
                                                     (lists && !gw_in_place) ? &L : nullptr,
-                                                    gw_from_col ? (gw_in_place ? base + l.gcol : base + l.col) : nullptr,
+                                                    (gw_from_col && !columns) ? (gw_in_place ? base + l.gcol : base + l.col) : nullptr,
                                                     gw_in_place, st))
                     return rc;
             if (s.ss.on && goff) {
@@ -809,10 +816,11 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         }
     }
     if (gw && !gw_done) {
+        if (columns && d2c_bwd_weight_from_col(s, q.dtype)) gw_from_col = true;   // (also when nothing else was wanted)
         if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
             if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, xcl_p, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc),
-                                                       gw, gw_from_col ? (gw_in_place ? base + l.gcol : base + l.col) : nullptr,
+                                                       gw, gw_from_col ? (columns ? (char *)columns : (gw_in_place ? base + l.gcol : base + l.col)) : nullptr,
                                                        gw_in_place ? (long)s.M : (long)((s.M + 63) / 64) * 64, st))
                 return rc;
         } else {
@@ -916,10 +924,24 @@ size_t d2c_tiled_forward_ws(const d2c_conv3d_desc &q, bool with_stats)
     return fwd_ws(q, s).total + (with_stats && d2c_fwd_fills_stats(s) ? d2c_fwd_stats_ws(s) : 0);
 }
 
-size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q, const d2c_size_map_desc *sz)
+size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q, const d2c_size_map_desc *sz, bool saved_columns)
 {
     const TiledShape s = tiled_shape(q, 3, 0, sz);
-    return is_depthwise(q) ? dw_ws(q, s).total_bwd : bwd_ws(q, s).total;
+    return is_depthwise(q) ? dw_ws(q, s).total_bwd : bwd_ws(q, s, saved_columns).total;
+}
+
+// Bytes of the sampled columns that a forward call can keep for the backward call of the same step:
+// [chunk][tap][rows][64] bfloat16, rows = position tiles x 64.  0 where the forward kernel does not write them or
+// the backward pass cannot multiply over them.
+size_t d2c_tiled_columns_bytes(const d2c_conv3d_desc &q, const d2c_size_map_desc *sz)
+{
+    if (is_depthwise(q) || !mfma_channels_ok(q)) return 0;
+    if (sz && !d2c_tiled_sized_supported(q, true)) return 0;
+    const TiledShape s = tiled_shape(q, 3, 0, sz);
+    if (!d2c_fwd_writes_columns(s, q.dtype) || !d2c_bwd_weight_from_col(s, q.dtype) || !use_aux_kernel(q, s)) return 0;
+    const long rows = d2c_columns_rows(s), chunks = s.Cin / bkc_of(q.dtype);
+    if (chunks * s.K * rows >= (1L << 31)) return 0;      // (the kernel counts rows in 32 bits)
+    return (size_t)chunks * s.K * rows * bkc_of(q.dtype) * d2c_elem_size(q.dtype);
 }
 
 // The matrix-core kernels can form the offsets from a size map themselves; the backward pass then needs the
@@ -933,10 +955,10 @@ bool d2c_tiled_sized_supported(const d2c_conv3d_desc &q, bool backward)
 
 int d2c_tiled_forward(const d2c_conv3d_desc &q, const void *x, const void *off, const void *mask, const void *w,
                       const void *bias, void *out, void *ws, hipStream_t st, const d2c_size_map_desc *sz, float *stats,
-                      const D2cPrepared *prep)
+                      const D2cPrepared *prep, void *columns)
 {
-    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats, prep);
-    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats, prep);
+    if (q.dtype == D2C_BF16) return forward_t<bf16_t>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats, prep, columns);
+    return forward_t<float>(q, x, off, mask, w, bias, out, ws, st, 3, sz, stats, prep, columns);
 }
 
 // Bytes of the caller-held prepared region of a description (0: the kernel family keeps nothing worth holding)
@@ -954,9 +976,10 @@ bool d2c_tiled_forward_fills_stats(const d2c_conv3d_desc &q)
 
 int d2c_tiled_backward(const d2c_conv3d_desc &q, const void *gout, const void *x, const void *off,
                        const void *mask, const void *w, void *gx, void *goff, void *gmask, void *gw, void *gb,
-                       void *ws, hipStream_t st, const d2c_size_map_desc *sz, const D2cPrepared *prep)
+                       void *ws, hipStream_t st, const d2c_size_map_desc *sz, const D2cPrepared *prep,
+                       const void *columns)
 {
     if (q.dtype == D2C_BF16)
-        return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz, prep);
-    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz, prep);
+        return backward_t<bf16_t>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz, prep, columns);
+    return backward_t<float>(q, gout, x, off, mask, w, gx, goff, gmask, gw, gb, ws, st, 3, 0, sz, prep, columns);
 }

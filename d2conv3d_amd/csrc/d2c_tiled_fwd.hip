@@ -50,6 +50,11 @@ struct FwdArgs {
     // one); every entry has exactly one writer (no atomics: they would all land on the same few cache lines), and
     // stats_reduce_kernel adds the tiles of a sample up.  Filled by the DMA-gather kernel and its finishing kernel.
     float *stats;
+    // The sampled, modulated columns kept for the backward pass (or NULL): what the matrix step multiplies with the
+    // weights, [chunk][tap][col_rows][BKC] in the element type, col_rows = position tiles x 64 (zeros past the last
+    // position) -- the layout tiled_bwd_weight_col_kernel reads.  Written by the DMA-gather kernel (bfloat16).
+    void *col;
+    long col_rows;
 };
 
 // Tiles that are neighbours in space go to the same XCD (workgroups are dealt
@@ -394,7 +399,7 @@ D2C_DEV bool seg_advance(SegWalk &w, const int4 *s_seg, int nseg, const TiledSha
 // which the compiler makes every LDS store wait for all DMA transfers in flight, whatever region they fill.)
 // NC: corner rows fetched and interpolated per sampling point: 8, or 4 / 2 when offsets along one / two axes are fixed
 // (TiledShape::axes; the corners on the far side of a fixed axis have weight zero and no slot at all).
-template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED, int NC>
+template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED, int NC, bool COLS>
 D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, unsigned char *__restrict__ s_tile,
                           float *__restrict__ s_w, int2 *__restrict__ s_if,
                           int *__restrict__ s_meta, int4 *__restrict__ s_seg)
@@ -555,6 +560,10 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         if (cwave && ctid == 0) {
             s_meta[buf * 4] = w.wg * s.cg + w.j * BKC;
             s_meta[buf * 4 + 1] = (w.wg * S + w.j * s.K + w.k) * OBT + w.otile * (NT / 32);
+            // COLS: the row of the column buffer where this step's tile goes (the first output tile writes it)
+            if constexpr (COLS)
+                s_meta[buf * 4 + 2] = w.otile == 0 ? (int)((((long)(w.wg * s.nchunk + w.j)) * s.K + w.k) * a.col_rows) + w.tile * MT
+                                                   : -1;
         }
     };
     // a table that fetches rows of zeros: steps past the end of a sequence shorter than the pipeline
@@ -563,7 +572,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
 #pragma unroll
             for (int q = 0; q < 8; q++) s_w[(buf * 8 + q) * MT + ctid] = 0.f;
             s_if[buf * MT + ctid] = make_int2(0, 0);
-            if (ctid == 0) { s_meta[buf * 4] = 0; s_meta[buf * 4 + 1] = 0; }
+            if (ctid == 0) { s_meta[buf * 4] = 0; s_meta[buf * 4 + 1] = 0; s_meta[buf * 4 + 2] = -1; }
         }
     };
 
@@ -650,10 +659,32 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         }
         return va;
     };
+    // COLS: the tile of a step also goes to the column buffer, one 16-byte streaming store per thread.  It is kept
+    // for one step and issued right behind the wait at the top of the next iteration (col_flush), so that it has a
+    // whole step to complete before that wait comes round again (the wait counts stores as well as loads).
+    typedef unsigned u32x4_c __attribute__((ext_vector_type(4)));
+    u32x4_c col_v = {0u, 0u, 0u, 0u};
+    int col_row = -1;                                  // (wavefront-uniform)
+    auto col_keep = [&](const uint4 &v, int tbuf) {
+        if constexpr (COLS) {
+            col_v = u32x4_c{v.x, v.y, v.z, v.w};
+            col_row = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4 + 2]);
+        }
+    };
+    auto col_flush = [&]() {
+        if constexpr (COLS) {
+            // (a thread's 16 bytes of its tile: position tid / 8, vector tid % 8 of a 128-byte row)
+            if (col_row >= 0)
+                __builtin_nontemporal_store(col_v, reinterpret_cast<u32x4_c *>(reinterpret_cast<char *>(a.col)
+                                                       + (long)col_row * (BKC * (long)sizeof(T)) + tid * 16));
+        }
+    };
     auto interp_store = [&](int rbuf, int tbuf, int dbuf) {
         if (!worker) return;
         VecAcc<T> va = interp_rows(rbuf, tbuf, [](int) {});
-        *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = va.pack();
+        const uint4 v = va.pack();
+        *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = v;
+        col_keep(v, tbuf);
     };
 
     // --- MMA role
@@ -711,7 +742,9 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
 #pragma unroll
             for (int f = c * (8 / NC); f < (c + 1) * (8 / NC); f++) af[f / OB][f % OB] = wfrag(wstep, f / OB, f % OB);
         });
-        *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = va.pack();
+        const uint4 v = va.pack();
+        *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = v;
+        col_keep(v, tbuf);
     };
     // end of a segment: whole items get bias, conversion and store; pieces of an item add into its fp32 tile
     auto flush_acc = [&](const SegWalk &w) {
@@ -855,6 +888,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 // during the last interpolation) and the rows of step it+1 (requested during the last matrix step)
                 __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
                 mma_dma_step(it & 1, it & 1, (it + 2) % 3);
+                col_flush();                            // (the tile of this step, interpolated in the last iteration)
                 // (past the end of the sequence the interpolation works on stale rows into the tile nobody reads)
                 interp_wload_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
             }
@@ -878,7 +912,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     }
 }
 
-template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED, int NC>
+template <typename T, bool AUX16, int WAVES_O, int WAVES_P, bool SIZED, int NC, bool COLS = false>
 __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
 {
     constexpr int MT = kDMT;
@@ -890,7 +924,7 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_fwd_dma_kernel(FwdArgs a)
     __shared__ int2 s_if[3 * MT];                                     // [3][MT] (offset of corner 000, live corners)
     __shared__ int s_meta[3 * 4];                                     // [3][first channel, weight-fragment row]
     __shared__ int4 s_seg[2 * kMaxSeg];                               // [kMaxSeg][2]
-    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P, SIZED, NC>(a, s_raw, s_tile, s_w, s_if, s_meta, s_seg);
+    fwd_dma_body<T, AUX16, WAVES_O, WAVES_P, SIZED, NC, COLS>(a, s_raw, s_tile, s_w, s_if, s_meta, s_seg);
 }
 
 // out = fp32 tile + bias for the items whose steps were shared out (see FwdArgs).  One block = 32 output
@@ -995,7 +1029,17 @@ int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
         D2cProfScope prof(D2C_PROF_FWD, st, "tiled_fwd_dma_kernel");
         // offsets fixed along one / two axes (the layers that deform in space or in time only): 4 / 2 corner rows
         const int nfree = a.s.nd == 3 ? __builtin_popcount(a.s.axes & 7) : 3;
-        if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+        bool done = false;
+        if constexpr (sizeof(T) == 2) {
+            // (the variants that also write the columns: bfloat16, all three offset axes)
+            if (a.col && nfree == 3) {
+                if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+                else hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 8, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+                done = true;
+            }
+        }
+        if (done) {
+        } else if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         else if (nfree == 2) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 4>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         else if (nfree == 1) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 2>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         else hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 8>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
@@ -1094,10 +1138,19 @@ size_t d2c_fwd_stats_ws(const TiledShape &s)
     return d2c_align_up((size_t)((s.M + kDMT - 1) / kDMT) * 2 * s.Cout * 2 * sizeof(float));
 }
 
+// Whether the forward kernel of this shape can write the sampled columns for the backward pass (FwdArgs::col): the
+// DMA-gather kernel on bfloat16 problems with offsets along all three axes.
+bool d2c_fwd_writes_columns(const TiledShape &s, int dtype)
+{
+    return dtype == D2C_BF16 && s.nd == 3 && (s.axes & 7) == 7 && d2c_fwd_use_dma(s.og, s.M, s.groups);
+}
+long d2c_columns_rows(const TiledShape &s) { return (long)((s.M + kDMT - 1) / kDMT) * kDMT; }
 // `stats` / `stats_part`: the [N][Cout][2] result and the per-tile scratch of d2c_fwd_stats_ws() bytes, or NULL.
+// `col`: where the sampled columns go (d2c_fwd_writes_columns), or NULL.
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
-                         const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part)
+                         const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part,
+                         void *col)
 {
     const bool dma = d2c_fwd_use_dma(s.og, s.M, s.groups);
     const int nsplit = (outacc && !dma) ? d2c_fwd_split(s) : 1;
@@ -1105,7 +1158,11 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
     // the channels-last input is followed by a row of zeros (see forward_t)
     const unsigned zrow = (unsigned)((size_t)s.N * s.vol * s.Cin * sizeof(T));
     FwdArgs a{s, xcl, off, mask, wp, bias, out, nsplit > 1 ? outacc : nullptr, nsplit, zrow, 0, 0, 0, 0, 1,
-              stats ? (dma ? stats_part : (nsplit == 1 ? stats : nullptr)) : nullptr};
+              stats ? (dma ? stats_part : (nsplit == 1 ? stats : nullptr)) : nullptr, nullptr, 0};
+    if (col && d2c_fwd_writes_columns(s, (int)Elem<T>::DT)) {
+        a.col = col;
+        a.col_rows = d2c_columns_rows(s);
+    }
     if (a.stats && !dma) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(a.stats, (size_t)s.N * s.Cout * 2 * sizeof(float), st);
@@ -1155,6 +1212,6 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
     return d2c_check_launch("fwd_finish_kernel");
 }
 template int d2c_tiled_fwd_launch<bf16_t>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                          const void *, void *, float *, hipStream_t, float *, float *);
+                                          const void *, void *, float *, hipStream_t, float *, float *, void *);
 template int d2c_tiled_fwd_launch<float>(const TiledShape &, const void *, const void *, const void *, const void *,
-                                         const void *, void *, float *, hipStream_t, float *, float *);
+                                         const void *, void *, float *, hipStream_t, float *, float *, void *);
