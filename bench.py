@@ -661,6 +661,24 @@ def main():
         torch.cuda.synchronize()
         t_f += ev[0].elapsed_time(ev[1]) / nprof
         t_b += ev[1].elapsed_time(ev[2]) / nprof
+    # With the columns kept, the forward kernel also writes them (work of the backward pass moved into it): its
+    # duration in a plain forward call is measured as well, so that its GEMM rate can be read both ways.
+    plain_fwd_ms = None
+    if kept_cols is not None:
+        lib.d2c_profile_reset()
+        lib.d2c_profile_enable(1)
+        for _ in range(nprof):
+            if sized:
+                _lib.check(lib.d2c_conv3d_sized_forward(ctypes.byref(desc), ctypes.byref(sdesc), p(x), p(size), p(m), p(w),
+                                                        p(b), p(out), p(ws), nf, cur[0]), "forward")
+            else:
+                _lib.check(f_fwd(ctypes.byref(desc), p(x), p(off), p(m), p(w), p(b), p(out), p(ws), nf, cur[0]), "forward")
+        torch.cuda.synchronize()
+        lib.d2c_profile_enable(0)
+        tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
+        lib.d2c_profile_read(_lib.PROF_FWD, ctypes.byref(tot), ctypes.byref(cnt))
+        if cnt.value:
+            plain_fwd_ms = tot.value / nprof
     lib.d2c_profile_reset()
     lib.d2c_profile_enable(1)
     for _ in range(nprof):
@@ -698,6 +716,13 @@ def main():
                     "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dt], 4), "traffic": traffic,
                     "traffic_source": traffic_source, "algorithmic_gflop_per_launch": round(f_fwd_flops / 1e9, 2),
                     "whole_step_frac": round(value / PEAK_TFLOPS[dt], 4), "kernel_ms": kms}
+        if plain_fwd_ms and role[dom] == "fwd":
+            ach0 = f_fwd_flops / (plain_fwd_ms * 1e-3) / 1e12
+            roofline["note"] = ("this launch also writes the sampled columns that the backward call of the step "
+                                "multiplies over (config.columns_kept_for_backward_mbytes); `in_a_plain_forward_call` "
+                                "is the same kernel without that store")
+            roofline["in_a_plain_forward_call"] = {"kernel_ms": round(plain_fwd_ms, 4), "achieved": round(ach0, 2),
+                                                   "frac": round(ach0 / PEAK_TFLOPS[dt], 4)}
     elif main_k:
         # bandwidth-bound workloads: the longest kernel against every tensor of its direction once
         dom = max(main_k, key=main_k.get)
