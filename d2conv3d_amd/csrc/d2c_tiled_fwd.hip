@@ -660,8 +660,11 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         return va;
     };
     // COLS: the tile of a step also goes to the column buffer, one 16-byte streaming store per thread.  It is kept
-    // for one step and issued right behind the wait at the top of the next iteration (col_flush), so that it has a
-    // whole step to complete before that wait comes round again (the wait counts stores as well as loads).
+    // for one step and issued in the matrix step of the next iteration, behind that step's last row request
+    // (col_flush): it then has most of a step to complete before the wait at the top of the iteration comes round
+    // again (that wait counts stores as well as loads), and meets the vector-memory path when the row requests are
+    // out (N=2, C=512, 8x30x54: kernel +10 % with the store right behind the wait, +6 % in front of the
+    // interpolation, +4 % here; as a plain instead of a streaming store +26 %).
     typedef unsigned u32x4_c __attribute__((ext_vector_type(4)));
     u32x4_c col_v = {0u, 0u, 0u, 0u};
     int col_row = -1;                                  // (wavefront-uniform)
@@ -733,6 +736,8 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 if (i >= MT / 8 / PPI) break;
                 dma_request(i, vif.x, vif.y, c0, rbuf);
             }
+            // (the kept columns of this step's tile: behind the last row requests, while matrix instructions remain)
+            if (kg == (MT / 8 / PPI + DPK - 1) / DPK) col_flush();
         }
     };
     // interpolation of one step; the weight fragments of that step are fetched on the way
@@ -888,7 +893,6 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
                 // during the last interpolation) and the rows of step it+1 (requested during the last matrix step)
                 __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
                 mma_dma_step(it & 1, it & 1, (it + 2) % 3);
-                col_flush();                            // (the tile of this step, interpolated in the last iteration)
                 // (past the end of the sequence the interpolation works on stale rows into the tile nobody reads)
                 interp_wload_store((it + 1) & 1, (it + 1) % 3, (it + 1) & 1);
             }
