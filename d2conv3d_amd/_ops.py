@@ -446,8 +446,18 @@ class _DeformConv3dPackedFunction(torch.autograd.Function):
         out = torch.empty((N, Cout, Do, Ho, Wo), dtype=input.dtype, device=dev)
         stats = torch.empty((N, Cout, 2), dtype=torch.float32, device=dev) if want_stats else None
         p_off, p_mask = _ptr_at(deformation, 0), _ptr_at(deformation, lead)
+        columns = None
         with torch.cuda.device(dev):
-            if want_stats:
+            if not want_stats:
+                columns = _columns_for(lib, desc, sdesc, ctx.needs_input_grad[2], dev)
+            if columns is not None:
+                nb = (lib.d2c_conv3d_sized_forward_workspace_bytes(ctypes.byref(desc), sref) if sdesc is not None
+                      else lib.d2c_conv3d_forward_workspace_bytes(ctypes.byref(desc)))
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_forward_columns(ctypes.byref(desc), sref, _ptr(input), p_off, p_mask, _ptr(weight),
+                                                    _ptr(bias), _ptr(out), _ptr(columns), columns.numel(), _ptr(ws), nb,
+                                                    _stream(dev))
+            elif want_stats:
                 nb = lib.d2c_conv3d_forward_stats_workspace_bytes(ctypes.byref(desc), sref)
                 ws = _workspace(nb, dev)
                 rc = lib.d2c_conv3d_forward_stats(ctypes.byref(desc), sref, _ptr(input), p_off, p_mask, _ptr(weight),
@@ -463,7 +473,7 @@ class _DeformConv3dPackedFunction(torch.autograd.Function):
                 rc = lib.d2c_conv3d_forward(ctypes.byref(desc), _ptr(input), p_off, p_mask, _ptr(weight), _ptr(bias),
                                             _ptr(out), _ptr(ws), nb, _stream(dev))
         _lib.check(rc, "deform_conv3d_packed forward")
-        ctx.save_for_backward(input, deformation, weight, bias, out if relu_scale > 0 else None)
+        ctx.save_for_backward(input, deformation, weight, bias, out if relu_scale > 0 else None, columns)
         ctx.desc, ctx.sdesc, ctx.lead = desc, sdesc, lead
         ctx.relu_scale = float(relu_scale)
         if want_stats:
@@ -475,7 +485,7 @@ class _DeformConv3dPackedFunction(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, grad_out, _grad_stats=None):
         lib = _lib.load()
-        input, deformation, weight, bias, out = ctx.saved_tensors
+        input, deformation, weight, bias, out, columns = ctx.saved_tensors
         desc, sdesc = ctx.desc, ctx.sdesc
         dev = input.device
         grad_out = grad_out.contiguous().to(input.dtype)
@@ -490,7 +500,14 @@ class _DeformConv3dPackedFunction(torch.autograd.Function):
         g_off = _ptr_at(gdef, 0) if gdef is not None else ctypes.c_void_p(0)
         g_mask = _ptr_at(gdef, ctx.lead) if gdef is not None else ctypes.c_void_p(0)
         with torch.cuda.device(dev):
-            if sdesc is not None:
+            if columns is not None:
+                sref = ctypes.byref(sdesc) if sdesc is not None else None
+                nb = lib.d2c_conv3d_backward_columns_workspace_bytes(ctypes.byref(desc), sref)
+                ws = _workspace(nb, dev)
+                rc = lib.d2c_conv3d_backward_columns(ctypes.byref(desc), sref, _ptr(grad_out), _ptr(input), p_off, p_mask,
+                                                     _ptr(weight), _ptr(columns), columns.numel(), _ptr(gx), g_off, g_mask,
+                                                     _ptr(gw), _ptr(gb), _ptr(ws), nb, _stream(dev))
+            elif sdesc is not None:
                 nb = lib.d2c_conv3d_sized_backward_workspace_bytes(ctypes.byref(desc), ctypes.byref(sdesc))
                 ws = _workspace(nb, dev)
                 rc = lib.d2c_conv3d_sized_backward(ctypes.byref(desc), ctypes.byref(sdesc), _ptr(grad_out), _ptr(input),

@@ -153,3 +153,27 @@ def test_column_buffer_checks(dev):
     assert call(f32, p(cols), ncol) == 5 and "keeps no columns" in _lib.last_error()
     assert call(desc, p(cols), ncol) == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("cls", ["MDConv3d", "XYZSizeConditionedMDConv3d"])
+def test_layers_keep_columns_with_the_deformation_tensor_read_in_place(cls, dev, keep_columns_restored):
+    """The self-deforming layers hand the operator their deformation branch's output as it is (offsets and raw
+    modulation in one tensor, activation in the sampler): the same step with and without kept columns."""
+    from d2conv3d_amd import modules as M
+    torch.manual_seed(29)
+    layer = getattr(M, cls)(128, 192, 3, padding=1).to(dev)
+    with torch.no_grad():
+        layer.deform_params.weight.normal_(0, 0.02)
+        layer.deform_params.bias.normal_(0, 0.5)
+    layer = layer.to(torch.bfloat16)
+    x = torch.randn(1, 128, 9, 32, 32, device=dev).bfloat16()
+    gout = torch.randn(1, 192, 9, 32, 32, device=dev).bfloat16()
+    res = []
+    for keep in (True, False):
+        _ops.config.set_keep_columns(keep)
+        layer.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        layer(xi).backward(gout)
+        res.append([xi.grad] + [p.grad.clone() for p in layer.parameters()])
+    for i, (a, p) in enumerate(zip(*res)):
+        assert rel_l2(a, p) < 5e-3, (cls, i, rel_l2(a, p))
