@@ -163,7 +163,10 @@ def _columns_for(lib, desc, sdesc, weight_grad_wanted, dev):
     n = lib.d2c_conv3d_columns_bytes(ctypes.byref(desc), ctypes.byref(sdesc) if sdesc is not None else None)
     if n == 0 or n > _KEEP_COLUMNS["max_bytes"]:
         return None
-    return torch.empty(n, dtype=torch.uint8, device=dev)
+    try:
+        return torch.empty(n, dtype=torch.uint8, device=dev)
+    except torch.cuda.OutOfMemoryError:
+        return None      # (no room to keep them: the backward pass samples again)
 
 
 class _DeformConv3dFunction(torch.autograd.Function):

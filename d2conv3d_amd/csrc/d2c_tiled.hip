@@ -119,7 +119,9 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0, con
                                   : (sz ? (long)mode_channels(sz->mode) * s.P : (long)s.G * s.K * (nd == 3 ? 3 : 1) * s.P);
     s.mbs = q.deform_channels > 0 ? (long)q.deform_channels * s.P : (long)s.G * s.K * s.P;
     s.mact = q.mask_activation;
-    s.f32split = (q.dtype == D2C_F32 && (q.backward_flags & D2C_BWD_F32_SPLIT)) ? 1 : 0;
+    // float problems: 1 = every backward matrix kernel on two-term bfloat16 operands (asked for in the description),
+    // 2 = the grad-column product alone, like the forward kernels (the default: every tolerance gate stays green)
+    s.f32split = q.dtype != D2C_F32 ? 0 : ((q.backward_flags & D2C_BWD_F32_SPLIT) ? 1 : (kF32SplitFwd ? 2 : 0));
     const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
     s.ogp = (s.og + nt - 1) / nt * nt;
     s.geo = make_geom(q);

@@ -811,7 +811,7 @@ template <typename T> size_t bwd_col_lds(int ogk, bool db)
 }
 
 template <typename T, int NKG>
-int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st)
+int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st, bool split)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
     const bool db = bwd_col_lds<T>(a.ogk, true) <= 160 * 1024;
@@ -827,7 +827,7 @@ int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st)
         return d2c_check_launch("tiled_bwd_col_kernel");
     };
     if constexpr (sizeof(T) == 4) {
-        if (a.s.f32split) return go(std::true_type{});
+        if (split) return go(std::true_type{});
     }
     return go(std::false_type{});
 }
@@ -860,7 +860,7 @@ template <typename T> size_t bwd_data_lds(int ogk)
 }
 
 template <typename T, int NKG>
-int launch_bwd_data(const BwdDataArgs &a, int nsplit, hipStream_t st)
+int launch_bwd_data(const BwdDataArgs &a, int nsplit, hipStream_t st, bool split)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
     const size_t lds = bwd_data_lds<T>(a.ogk);
@@ -873,7 +873,7 @@ int launch_bwd_data(const BwdDataArgs &a, int nsplit, hipStream_t st)
         return d2c_check_launch("tiled_bwd_data_kernel");
     };
     if constexpr (sizeof(T) == 4) {
-        if (a.s.f32split) return go(std::true_type{});
+        if (split) return go(std::true_type{});
     }
     return go(std::false_type{});
 }
@@ -1759,12 +1759,16 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const int ogn = s.og - o0 < omax ? s.og - o0 : omax;
         const int ogk = d2c_bwd_ogk(ogn, Elem<T>::DT);
         const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
+        // two-term bfloat16 operands for this pass (float problems): wherever the description asks for them, and for
+        // the grad-column product on its own by default (f32split == 2)
+        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
+        const bool split_pass = sizeof(T) == 4 && (s.f32split == 1 || (s.f32split == 2 && col_only));
         // (weights_packed: `wt` already holds them, from an earlier call on the same weights)
         if ((phase & 1) && !weights_packed) {
             D2cProfScope prof(D2C_PROF_PACK, st);
             constexpr int R = 128 / (int)sizeof(T);
             constexpr bool SPT = sizeof(T) == 4;       // (split operands exist for float problems only)
-            const bool split = SPT && s.f32split;
+            const bool split = SPT && split_pass;
             auto k_lds = split ? &pack_weight_bwd_lds_kernel<T, SPT> : &pack_weight_bwd_lds_kernel<T, false>;
             auto k_elem = split ? &pack_weight_bwd_kernel<T, SPT> : &pack_weight_bwd_kernel<T, false>;
             const size_t lds = (size_t)R * ((size_t)kPackCh * s.K * sizeof(T) + 4);
@@ -1782,22 +1786,21 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                       auxoff, auxmask, sliced ? g_lo * cpc2 * s.K : 0, sliced ? (g_lo + g_n) * cpc2 * s.K : 0};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
-        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
         if (col_only && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
             rc = launch_bwd_col32(a, nsplit, st);
         } else if (sliced) {
             d2c_set_error("grad-column product: slices are made by tiled_bwd_col32_kernel only");
             return D2C_ERR_LAUNCH;
         } else if (col_only) {
-            if (nkg <= 4) rc = launch_bwd_col<T, 4>(a, nsplit, st);
-            else if (nkg <= 8) rc = launch_bwd_col<T, 8>(a, nsplit, st);
-            else if (nkg <= 16) rc = launch_bwd_col<T, 16>(a, nsplit, st);
-            else rc = launch_bwd_col<T, 32>(a, nsplit, st);
+            if (nkg <= 4) rc = launch_bwd_col<T, 4>(a, nsplit, st, split_pass);
+            else if (nkg <= 8) rc = launch_bwd_col<T, 8>(a, nsplit, st, split_pass);
+            else if (nkg <= 16) rc = launch_bwd_col<T, 16>(a, nsplit, st, split_pass);
+            else rc = launch_bwd_col<T, 32>(a, nsplit, st, split_pass);
         } else {
-            if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, nsplit, st);
-            else if (nkg <= 8) rc = launch_bwd_data<T, 8>(a, nsplit, st);
-            else if (nkg <= 16) rc = launch_bwd_data<T, 16>(a, nsplit, st);
-            else rc = launch_bwd_data<T, 32>(a, nsplit, st);
+            if (nkg <= 4) rc = launch_bwd_data<T, 4>(a, nsplit, st, split_pass);
+            else if (nkg <= 8) rc = launch_bwd_data<T, 8>(a, nsplit, st, split_pass);
+            else if (nkg <= 16) rc = launch_bwd_data<T, 16>(a, nsplit, st, split_pass);
+            else rc = launch_bwd_data<T, 32>(a, nsplit, st, split_pass);
         }
         if (rc) return rc;
     }
@@ -1926,7 +1929,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
         const bool vec = s.P % Elem<T>::VEC == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0;
         constexpr bool SPT = sizeof(T) == 4;
-        auto k_gout = (SPT && s.f32split) ? &pack_gout_kernel<T, SPT> : &pack_gout_kernel<T, false>;
+        auto k_gout = (SPT && s.f32split == 1) ? &pack_gout_kernel<T, SPT> : &pack_gout_kernel<T, false>;
         hipLaunchKernelGGL(k_gout, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const T *)gout, (T *)goutp, s, ntp, OBT,
                            total, vec);
         if (int rc = d2c_check_launch("pack_gout_kernel")) return rc;
@@ -1971,7 +1974,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         };
         auto go_nc = [&](auto aux_c, auto sized_c, auto nc_c) -> bool {
             if constexpr (sizeof(T) == 4) {
-                if (s.f32split) return go_sp(aux_c, sized_c, nc_c, std::true_type{});
+                if (s.f32split == 1) return go_sp(aux_c, sized_c, nc_c, std::true_type{});
             }
             return go_sp(aux_c, sized_c, nc_c, std::false_type{});
         };

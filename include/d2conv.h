@@ -83,10 +83,12 @@ enum {
  * groups).  Buffers of grad-column rows and sampled columns then hold one slice; several offset groups, one weight
  * group and 128 .. 512 output channels only (other descriptions ignore the bits). */
 #define D2C_BWD_SLICES(n)    (((n) & 0xff) << 8)
-/* float32 problems on the matrix-core kernels: let the backward matrix kernels, like the forward ones, carry every
- * float operand as the sum of two bfloat16 values on the bfloat16 matrix instruction (a quarter of the matrix-pipe
- * time of the float instruction).  Gradients then carry a relative error of about 4e-6 of their sums' scale
- * instead of 1e-7 -- within 1e-4 relative, but not within 1e-5 absolute where elements reach tens or hundreds.
+/* float32 problems on the matrix-core kernels: the forward kernels and the grad-column product of the backward pass
+ * (from which grad_input, grad_offset and grad_mask follow) carry every float operand as the sum of two bfloat16
+ * values on the bfloat16 matrix instruction (a quarter of the matrix-pipe time of the float instruction; results
+ * within about 4e-6 of their sums' scale instead of 1e-7, inside 1e-4 relative / 1e-5 absolute at every size
+ * measured).  With this bit ALL backward matrix kernels do so -- also the grad-weight product, whose elements
+ * (sums over all positions, tens to hundreds in size) then miss 1e-5 absolute -- and the 1-D and fallback kernels.
  * Off by default. */
 #define D2C_BWD_F32_SPLIT    0x10000
 

@@ -159,10 +159,11 @@ def test_prepared_region_gives_the_same_results(dtype, dev):
 
 @pytest.mark.parametrize("name", ["c128_G2_o96", "c64_stride_dil", "c64_o320_nomask", "c128_groups2_G1"])
 def test_float32_backward_on_split_operands(name, dev):
-    """D2C_BWD_F32_SPLIT: the backward matrix kernels of a float32 problem on two-term bfloat16 operands, like the
+    """D2C_BWD_F32_SPLIT: every backward matrix kernel of a float32 problem on two-term bfloat16 operands, like the
     forward kernels.  Against the float64 oracle: every gradient within 2e-5 of its tensor's scale (the operands
-    keep 16 of float32's 24 significant bits: about 4e-6 relative in a long sum, against 1e-7 for plain float32),
-    and the default path on the same inputs an order of magnitude closer."""
+    keep 16 of float32's 24 significant bits: about 4e-6 relative in a long sum, against 1e-7 for plain float32).
+    By default only the grad-column product takes such operands (grad_input, grad_offset and grad_mask then sit at
+    the same 4e-6), and grad_weight / grad_bias, on float32 instructions, an order of magnitude closer."""
     (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, torch.float32, seed=13)
     dd = lambda t: t.double() if t is not None else None
     eg = cpu.conv3d_backward(dd(gout), dd(x), dd(off), dd(m), dd(w), b is not None, s, p, d, groups, G)
@@ -176,5 +177,5 @@ def test_float32_backward_on_split_operands(name, dev):
                 continue
             err = ((t.grad.double().cpu() - e).abs().max() / e.abs().max()).item()
             errs[split].append(err)
-            assert err < (2e-5 if split else 2e-6), (name, n, split, err)
-    assert max(errs[True]) > max(errs[False])      # (the flag did change the arithmetic)
+            assert err < (2e-5 if (split or n in ("grad_input", "grad_offset", "grad_mask")) else 2e-6), (name, n, split, err)
+    assert errs[True][-2 if b is not None else -1] > errs[False][-2 if b is not None else -1]   # (grad_weight: the flag did change the arithmetic)
