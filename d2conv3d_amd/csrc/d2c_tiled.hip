@@ -48,6 +48,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
                                 const void *mask, void *goutp, float *gwacc, void *gw, const void *col, long col_rows,
                                 hipStream_t st, int phase = 7, int jp_lo = 0, int jp_n = 0);
 bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype);
+bool d2c_bwd_weight_from_kept_col(const TiledShape &s, int dtype);
 size_t d2c_bwd_col_bytes(const TiledShape &s, int nchunks = 0);
 size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype);
 template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
@@ -767,7 +768,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
                 D2cProfScope prof(D2C_PROF_PACK, st);
                 d2c_fill_zero(goff_k, (size_t)s.N * 3 * s.P * sizeof(float), st);
             }
-            gw_from_col = gw && (columns ? d2c_bwd_weight_from_col(s, q.dtype) : (auxk && use_col_weight(q, s)));
+            gw_from_col = gw && (columns ? d2c_bwd_weight_from_kept_col(s, q.dtype) : (auxk && use_col_weight(q, s)));
             // (the sampled columns over the grad-column rows: grad_input has to be done with the rows before the
             // offset / mask gradient kernel runs, so the samples are filed by a pass of their own)
             gw_in_place = gw_from_col && !columns && col_in_place(q, s);
@@ -818,7 +819,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
         }
     }
     if (gw && !gw_done) {
-        if (columns && d2c_bwd_weight_from_col(s, q.dtype)) gw_from_col = true;   // (also when nothing else was wanted)
+        if (columns && d2c_bwd_weight_from_kept_col(s, q.dtype)) gw_from_col = true;   // (also when nothing else was wanted)
         if (d2c_tiled_bwd_weight_supported(s, q.dtype)) {
             if (int rc = d2c_tiled_bwd_weight_launch<T>(s, gout, xcl_p, off, mask, base + l.goutp,
                                                        (float *)(base + l.gwacc),
@@ -933,14 +934,14 @@ size_t d2c_tiled_backward_ws(const d2c_conv3d_desc &q, const d2c_size_map_desc *
 }
 
 // Bytes of the sampled columns that a forward call can keep for the backward call of the same step:
-// [chunk][tap][rows][64] bfloat16, rows = position tiles x 64.  0 where the forward kernel does not write them or
+// [chunk][tap][rows][64 bfloat16 / 32 float], rows = position tiles x 64.  0 where the forward kernel does not write them or
 // the backward pass cannot multiply over them.
 size_t d2c_tiled_columns_bytes(const d2c_conv3d_desc &q, const d2c_size_map_desc *sz)
 {
     if (is_depthwise(q) || !mfma_channels_ok(q)) return 0;
     if (sz && !d2c_tiled_sized_supported(q, true)) return 0;
     const TiledShape s = tiled_shape(q, 3, 0, sz);
-    if (!d2c_fwd_writes_columns(s, q.dtype) || !d2c_bwd_weight_from_col(s, q.dtype) || !use_aux_kernel(q, s)) return 0;
+    if (!d2c_fwd_writes_columns(s, q.dtype) || !d2c_bwd_weight_from_kept_col(s, q.dtype) || !use_aux_kernel(q, s)) return 0;
     const long rows = d2c_columns_rows(s), chunks = s.Cin / bkc_of(q.dtype);
     if (chunks * s.K * rows >= (1L << 31)) return 0;      // (the kernel counts rows in 32 bits)
     return (size_t)chunks * s.K * rows * bkc_of(q.dtype) * d2c_elem_size(q.dtype);

@@ -1240,21 +1240,23 @@ __global__ void __launch_bounds__(kThreads + 64) tiled_bwd_weight_dma_kernel(Bwd
 }
 
 // ============================================================ kernel 2b
-// grad_weight as a plain matrix product over the sampled columns that the offset / mask gradient kernel left in
-// device memory (aux_grad_kernel<.., COL>; bfloat16 problems):
+// grad_weight as a plain matrix product over sampled columns held in device memory -- the ones the offset / mask
+// gradient kernel left there (aux_grad_kernel<.., COL>; bfloat16 problems), or the ones the forward call of the same
+// step kept (tiled_fwd_dma_kernel<.., COLS>; bfloat16 and float):
 //     gW[o, (chunk, tap, c)] += sum_pos gout[o, pos] * col[chunk][tap][pos][c]
-// One workgroup = one tap and kColChunks channel chunks (128 columns), all output channels of the weight group (8
+// One workgroup = one tap and kColChunks channel chunks (128 / 64 columns), all output channels of the weight group (8
 // wavefronts x 64 rows), looping over its piece of the 64-position tiles.  No sampling here: the input is not read
 // again, there is no coordinate wavefront and no interpolation.  The column tiles (2 x 8 KiB per step) go through
-// registers into a double-buffered LDS tile (one 16-byte load and one LDS store per lane and tile, requested a step
-// ahead), the grad_out fragments come straight from the fragment-ordered copy, a step ahead as well.  All loads are
-// ordinary ones, so the compiler counts its waits; the barrier waits for LDS operations only.  Twice the columns per
-// grad_out fragment of tiled_bwd_weight_dma_kernel: half the fragment traffic per product.
+// registers into a double-buffered LDS tile (one 16-byte load per lane and tile, requested a step ahead, and one
+// LDS store -- float: four, the tile is kept [channel][position] as the float matrix instruction wants it), the
+// grad_out fragments come straight from the fragment-ordered copy, ahead as well.  All loads are ordinary ones, so
+// the compiler counts its waits; the barrier waits for LDS operations only.  Twice the columns per grad_out fragment
+// of tiled_bwd_weight_dma_kernel: half the fragment traffic per product.
 constexpr int kColChunks = 2;
 
 struct BwdWeightColArgs {
     TiledShape s;
-    const void *col;     // [chunk][tap][mpad][64]
+    const void *col;     // [chunk][tap][mpad][BKC]
     const void *goutp;   // grad_out in MFMA fragment order, see pack_gout_kernel
     float *gwacc;        // as in BwdWeightArgs
     long mpad;           // rows per (chunk, tap) of `col`: whole 64-position tiles, or N*P when the columns took the place
@@ -1266,17 +1268,24 @@ struct BwdWeightColArgs {
                          // held all chunks)
 };
 
+template <typename T>
 __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeightColArgs a)
 {
-    typedef bf16_t T;
-    constexpr int MT = kWDT, VEC = 8, BKC = 64, NCH = kColChunks, CB = NCH * (BKC / 32), OB = 2, NT = 64 * 8;
-    // tile row stride ([position][channel]): 64 bytes more than a row, so that the 64-byte segments of four consecutive
-    // rows, which 32 lanes of a transposing read fetch together, fall into different quarters of the 64 banks
-    constexpr int TRS = MT * (int)sizeof(T) + 64;
+    constexpr bool F32 = sizeof(T) == 4;
+    constexpr int MT = kWDT, VEC = Elem<T>::VEC, BKC = 8 * VEC, NCH = kColChunks, CPB = BKC / 32, CB = NCH * CPB, OB = 2,
+                  NT = 64 * 8;
+    // bfloat16: tile rows are positions ([position][channel]), 64 bytes more than a row apart, so that the 64-byte
+    // segments of four consecutive rows, which 32 lanes of a transposing read fetch together, fall into different
+    // quarters of the 64 banks.  float: tile rows are channels ([channel][position]), an odd number of 16-byte units apart
+    constexpr int TRS = F32 ? MT * 4 + 16 : MT * 2 + 64;
+    constexpr int TROWS = F32 ? BKC : MT;      // rows of one tile
     constexpr int NKG = MT / (2 * VEC);        // k-groups per iteration
     constexpr int NKGP = kWMT / (2 * VEC);     // k-groups per tile of the packed grad_out copy
+    // tiles of grad_out fragments in flight (float: 16 fragments per tile and 64 matrix instructions per fragment
+    // pair, one tile ahead is a long time)
+    constexpr int LA = F32 ? 1 : 2;
     static_assert(MT * 8 == kThreads, "one (position, vector) item per thread and column tile");
-    __shared__ __align__(16) unsigned char s_tile[2 * NCH * MT * TRS];
+    __shared__ __align__(16) unsigned char s_tile[2 * NCH * TROWS * TRS];
 
     const TiledShape &s = a.s;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1325,7 +1334,18 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
     // a tile to arrive from device memory
     uint4 crO0, crO1, crE0, crE1;
     auto col_row0 = [&](int i) { return (long)(t_lo + min(i, nmy - 1) * t_step) * MT * (BKC / VEC); };
-    unsigned char *const st_p = s_tile + ipos * TRS + ivec * 16;
+    // this thread's vector of tile `t` (buffer * NCH + chunk of the step) into LDS
+    unsigned char *const st_p = F32 ? s_tile + (ivec * VEC) * TRS + ipos * 4 : s_tile + ipos * TRS + ivec * 16;
+    auto put = [&](int t, const uint4 &v) {
+        if constexpr (F32) {
+            *reinterpret_cast<unsigned *>(st_p + (t * TROWS + 0) * TRS) = v.x;
+            *reinterpret_cast<unsigned *>(st_p + (t * TROWS + 1) * TRS) = v.y;
+            *reinterpret_cast<unsigned *>(st_p + (t * TROWS + 2) * TRS) = v.z;
+            *reinterpret_cast<unsigned *>(st_p + (t * TROWS + 3) * TRS) = v.w;
+        } else {
+            *reinterpret_cast<uint4 *>(st_p + t * TROWS * TRS) = v;
+        }
+    };
 
     // --- gW block += gout[o, pos] * tile[pos, c]; gout fragments straight from the packed copy
     const int OBT = (s.og + 63) / 64 * 2;
@@ -1338,13 +1358,15 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
         const int kgp = (int)(t64 % (kWMT / MT)) * NKG;
         return gp4 + ((tp * OBT) * NKGP + kgp) * 64;
     };
-    // the fragments of two tiles in flight (even / odd iterations); a slot is refilled, for the tile after next, as
-    // soon as the matrix cores have taken it: two whole steps for a fragment to arrive
-    uint4 ldA[2 * NKG], ldB[2 * NKG];
+    // the fragments of LA tiles in flight (two: even / odd iterations); a slot is refilled, for the tile LA steps on,
+    // as soon as the matrix cores have taken it
+    uint4 ldA[2 * NKG], ldB[LA == 2 ? 2 * NKG : 1];
     typedef short v4s __attribute__((ext_vector_type(4)));
     const int l16 = lane & 15, g16 = lane >> 4;
-    // this lane's part of the transposing reads: position (g16 >> 1) * 8 + (l16 >> 2), channel (g16 & 1) * 16 + (l16 & 3) * 4
-    const unsigned char *const rd_p = s_tile + ((g16 >> 1) * 8 + (l16 >> 2)) * TRS + ((g16 & 1) * 16 + (l16 & 3) * 4) * 2;
+    // this lane's part of the operand reads.  bfloat16, transposing: position (g16 >> 1) * 8 + (l16 >> 2), channel
+    // (g16 & 1) * 16 + (l16 & 3) * 4; float: channel lane % 32, positions 4 * (lane / 32) ..
+    const unsigned char *const rd_p = F32 ? s_tile + (lane & 31) * TRS + (lane >> 5) * 16
+                                          : s_tile + ((g16 >> 1) * 8 + (l16 >> 2)) * TRS + ((g16 & 1) * 16 + (l16 & 3) * 4) * 2;
 
     {
         const uint4 *g0 = gfrag_p(0), *g1 = gfrag_p(1);
@@ -1352,17 +1374,19 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
         for (int kg = 0; kg < NKG; kg++)
 #pragma unroll
             for (int ob = 0; ob < OB; ob++) ldA[kg * 2 + ob] = g0[(ob * NKGP + kg) * 64];
+        if constexpr (LA == 2) {
 #pragma unroll
-        for (int kg = 0; kg < NKG; kg++)
+            for (int kg = 0; kg < NKG; kg++)
 #pragma unroll
-            for (int ob = 0; ob < OB; ob++) ldB[kg * 2 + ob] = g1[(ob * NKGP + kg) * 64];
+                for (int ob = 0; ob < OB; ob++) ldB[kg * 2 + ob] = g1[(ob * NKGP + kg) * 64];
+        }
         const long r0 = col_row0(0), r1 = col_row0(1), r2 = col_row0(2);
         crE0 = ld_stream16(colp0 + r0);
         crE1 = ld_stream16(colp1 + r0);
         crO0 = ld_stream16(colp0 + r1);
         crO1 = ld_stream16(colp1 + r1);
-        *reinterpret_cast<uint4 *>(st_p) = crE0;
-        *reinterpret_cast<uint4 *>(st_p + MT * TRS) = crE1;
+        put(0, crE0);
+        put(1, crE1);
         crE0 = ld_stream16(colp0 + r2);
         crE1 = ld_stream16(colp1 + r2);
     }
@@ -1374,20 +1398,26 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
         auto step = [&](int it, uint4(&ld)[2 * NKG], uint4 &cr0, uint4 &cr1) {
             const int dbuf = it & 1;
             if constexpr (MMA) {
-                const uint4 *gn = gfrag_p(it + 2);
+                const uint4 *gn = gfrag_p(it + LA);
 #pragma unroll
                 for (int kg = 0; kg < NKG; kg++) {
                     uint4 bf[CB];
-                    // ds_read_b64_tr_b16, as in tiled_bwd_weight_dma_kernel: two loads make the 8 positions of an
-                    // operand vector
+                    if constexpr (F32) {
 #pragma unroll
-                    for (int cb = 0; cb < CB; cb++) {
-                        const unsigned char *ap = rd_p + ((dbuf * NCH + (cb >> 1)) * MT + kg * 16) * TRS + (cb & 1) * 64;
-                        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)ap);
-                        const v4s hi =
-                            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(ap + 4 * TRS));
-                        const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
-                        bf[cb] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+                        for (int cb = 0; cb < CB; cb++)
+                            bf[cb] = *reinterpret_cast<const uint4 *>(rd_p + ((dbuf * NCH + cb) * TROWS) * TRS + kg * 32);
+                    } else {
+                        // ds_read_b64_tr_b16, as in tiled_bwd_weight_dma_kernel: two loads make the 8 positions of an
+                        // operand vector
+#pragma unroll
+                        for (int cb = 0; cb < CB; cb++) {
+                            const unsigned char *ap = rd_p + ((dbuf * NCH + (cb >> 1)) * MT + kg * 16) * TRS + (cb & 1) * 64;
+                            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)ap);
+                            const v4s hi =
+                                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(ap + 4 * TRS));
+                            const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+                            bf[cb] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+                        }
                     }
 #pragma unroll
                     for (int ob = 0; ob < OB; ob++)
@@ -1400,8 +1430,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
                 }
             }
             // (the other buffer was last read in the iteration before, which every wavefront has left)
-            *reinterpret_cast<uint4 *>(st_p + ((dbuf ^ 1) * NCH * MT) * TRS) = cr0;
-            *reinterpret_cast<uint4 *>(st_p + ((dbuf ^ 1) * NCH + 1) * MT * TRS) = cr1;
+            put((dbuf ^ 1) * NCH, cr0);
+            put((dbuf ^ 1) * NCH + 1, cr1);
             const long r3 = col_row0(it + 3);
             cr0 = ld_stream16(colp0 + r3);
             cr1 = ld_stream16(colp1 + r3);
@@ -1409,9 +1439,16 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
         };
         // pairs of steps, then the odd one out: no branch inside the loop (see above)
         int it = 0;
-        for (; it + 1 < nmy; it += 2) {
-            step(it, ldA, crO0, crO1);
-            step(it + 1, ldB, crE0, crE1);
+        if constexpr (LA == 2) {
+            for (; it + 1 < nmy; it += 2) {
+                step(it, ldA, crO0, crO1);
+                step(it + 1, ldB, crE0, crE1);
+            }
+        } else {
+            for (; it + 1 < nmy; it += 2) {
+                step(it, ldA, crO0, crO1);
+                step(it + 1, ldA, crE0, crE1);
+            }
         }
         if (it < nmy) step(it, ldA, crO0, crO1);
     };
@@ -1423,12 +1460,12 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
         for (int ob = 0; ob < OB; ob++)
 #pragma unroll
             for (int cb = 0; cb < CB; cb++) {
-                const int stw = (jp * NCH + (cb >> 1)) * s.K + k;
+                const int stw = (jp * NCH + cb / CPB) * s.K + k;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int ol = o_base + ob * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                     if (ol < s.og)
-                        atomicAdd(a.gwacc + (((long)wg * s.nchunk * s.K + stw) * s.og + ol) * BKC + (cb & 1) * 32 + (lane & 31),
+                        atomicAdd(a.gwacc + (((long)wg * s.nchunk * s.K + stw) * s.og + ol) * BKC + (cb % CPB) * 32 + (lane & 31),
                                   acc[ob][cb][r]);
                 }
             }
@@ -1891,6 +1928,11 @@ bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype)
 {
     return dtype == D2C_BF16 && s.nd == 3 && s.nchunk % kColChunks == 0;
 }
+// ... from the columns that the forward call kept (d2c_fwd_writes_columns): float problems as well
+bool d2c_bwd_weight_from_kept_col(const TiledShape &s, int dtype)
+{
+    return (dtype == D2C_BF16 || dtype == D2C_F32) && s.nd == 3 && s.nchunk % kColChunks == 0;
+}
 // bytes of the sampled columns [chunk][tap][whole 64-position tiles][64] of `nchunks` channel chunks (0: all)
 size_t d2c_bwd_col_bytes(const TiledShape &s, int nchunks)
 {
@@ -1920,6 +1962,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     const int otiles = (s.og + 511) / 512;
     const int ntp = (s.M + kWMT - 1) / kWMT;     // tiles of the packed grad_out copy
     const int ntile = (s.M + kWDT - 1) / kWDT;   // position tiles of the kernel
+    const bool from_col = col != nullptr;
     if (phase & 1) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
@@ -1929,7 +1972,8 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
         const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
         const bool vec = s.P % Elem<T>::VEC == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0;
         constexpr bool SPT = sizeof(T) == 4;
-        auto k_gout = (SPT && s.f32split == 1) ? &pack_gout_kernel<T, SPT> : &pack_gout_kernel<T, false>;
+        // (the product over kept columns runs on the float instruction whatever the flags say)
+        auto k_gout = (SPT && s.f32split == 1 && !from_col) ? &pack_gout_kernel<T, SPT> : &pack_gout_kernel<T, false>;
         hipLaunchKernelGGL(k_gout, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const T *)gout, (T *)goutp, s, ntp, OBT,
                            total, vec);
         if (int rc = d2c_check_launch("pack_gout_kernel")) return rc;
@@ -1939,8 +1983,10 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     // first.
     const int ncu = d2c_num_cus();
     if (ncu <= 0) return D2C_ERR_LAUNCH;
-    bool from_col = false;
-    if constexpr (sizeof(T) == 2) from_col = col != nullptr;
+    if (from_col && !d2c_bwd_weight_from_kept_col(s, (int)Elem<T>::DT)) {
+        d2c_set_error("grad_weight: tiled_bwd_weight_col_kernel does not take this shape");
+        return D2C_ERR_LAUNCH;
+    }
     if (jp_n > 0 && !from_col) {
         d2c_set_error("grad_weight: slices are made by tiled_bwd_weight_col_kernel only");
         return D2C_ERR_LAUNCH;
@@ -1952,7 +1998,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     if (from_col && (phase & 2)) {
         BwdWeightColArgs c{s, col, goutp, gwacc, col_rows, otiles, nmain, main_len, ntail, tail_len, jp_lo, jp_n};
         D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st, "tiled_bwd_weight_col_kernel");
-        hipLaunchKernelGGL(tiled_bwd_weight_col_kernel, dim3((unsigned)(items * (nmain + ntail))), dim3(kThreads), 0, st, c);
+        hipLaunchKernelGGL(tiled_bwd_weight_col_kernel<T>, dim3((unsigned)(items * (nmain + ntail))), dim3(kThreads), 0, st, c);
         if (int rc = d2c_check_launch("tiled_bwd_weight_col_kernel")) return rc;
     }
     BwdWeightDmaArgs a{{s, gout, xcl, off, mask, goutp, gwacc, otiles, nmain, main_len, ntail, tail_len},

@@ -52,7 +52,7 @@ struct FwdArgs {
     float *stats;
     // The sampled, modulated columns kept for the backward pass (or NULL): what the matrix step multiplies with the
     // weights, [chunk][tap][col_rows][BKC] in the element type, col_rows = position tiles x 64 (zeros past the last
-    // position) -- the layout tiled_bwd_weight_col_kernel reads.  Written by the DMA-gather kernel (bfloat16).
+    // position) -- the layout tiled_bwd_weight_col_kernel reads.  Written by the DMA-gather kernel.
     void *col;
     long col_rows;
 };
@@ -668,9 +668,13 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
     typedef unsigned u32x4_c __attribute__((ext_vector_type(4)));
     u32x4_c col_v = {0u, 0u, 0u, 0u};
     int col_row = -1;                                  // (wavefront-uniform)
-    auto col_keep = [&](const uint4 &v, int tbuf) {
+    // (float: the interpolated values themselves, not the two-term operand form the matrix step reads)
+    auto col_keep = [&](const VecAcc<T> &va, const uint4 &v, int tbuf) {
         if constexpr (COLS) {
-            col_v = u32x4_c{v.x, v.y, v.z, v.w};
+            if constexpr (sizeof(T) == 4)
+                col_v = u32x4_c{__float_as_uint(va.a[0]), __float_as_uint(va.a[1]), __float_as_uint(va.a[2]),
+                                __float_as_uint(va.a[3])};
+            else col_v = u32x4_c{v.x, v.y, v.z, v.w};
             col_row = __builtin_amdgcn_readfirstlane(s_meta[tbuf * 4 + 2]);
         }
     };
@@ -687,7 +691,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         VecAcc<T> va = interp_rows(rbuf, tbuf, [](int) {});
         const uint4 v = va.pack();
         *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = v;
-        col_keep(v, tbuf);
+        col_keep(va, v, tbuf);
     };
 
     // --- MMA role
@@ -749,7 +753,7 @@ D2C_DEV void fwd_dma_body(const FwdArgs &a, unsigned char *__restrict__ s_raw, u
         });
         const uint4 v = va.pack();
         *reinterpret_cast<uint4 *>(s_tile + (dbuf * MT + ipos) * kRS + ivec * 16) = v;
-        col_keep(v, tbuf);
+        col_keep(va, v, tbuf);
     };
     // end of a segment: whole items get bias, conversion and store; pieces of an item add into its fp32 tile
     auto flush_acc = [&](const SegWalk &w) {
@@ -1033,16 +1037,10 @@ int launch_fwd_dma(FwdArgs a, float *outacc, hipStream_t st)
         D2cProfScope prof(D2C_PROF_FWD, st, "tiled_fwd_dma_kernel");
         // offsets fixed along one / two axes (the layers that deform in space or in time only): 4 / 2 corner rows
         const int nfree = a.s.nd == 3 ? __builtin_popcount(a.s.axes & 7) : 3;
-        bool done = false;
-        if constexpr (sizeof(T) == 2) {
-            // (the variants that also write the columns: bfloat16, all three offset axes)
-            if (a.col && nfree == 3) {
-                if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
-                else hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 8, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
-                done = true;
-            }
-        }
-        if (done) {
+        // (the variants that also write the columns: all three offset axes)
+        if (a.col && nfree == 3) {
+            if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
+            else hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 8, true>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         } else if (sized) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, true, 8>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         else if (nfree == 2) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 4>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
         else if (nfree == 1) hipLaunchKernelGGL((tiled_fwd_dma_kernel<T, AUX16, WO, WP, false, 2>), dim3(nwg), dim3(kThreads + 64), 0, st, a);
@@ -1143,10 +1141,10 @@ size_t d2c_fwd_stats_ws(const TiledShape &s)
 }
 
 // Whether the forward kernel of this shape can write the sampled columns for the backward pass (FwdArgs::col): the
-// DMA-gather kernel on bfloat16 problems with offsets along all three axes.
+// DMA-gather kernel on problems with offsets along all three axes.
 bool d2c_fwd_writes_columns(const TiledShape &s, int dtype)
 {
-    return dtype == D2C_BF16 && s.nd == 3 && (s.axes & 7) == 7 && d2c_fwd_use_dma(s.og, s.M, s.groups);
+    return (dtype == D2C_BF16 || dtype == D2C_F32) && s.nd == 3 && (s.axes & 7) == 7 && d2c_fwd_use_dma(s.og, s.M, s.groups);
 }
 long d2c_columns_rows(const TiledShape &s) { return (long)((s.M + kDMT - 1) / kDMT) * kDMT; }
 // `stats` / `stats_part`: the [N][Cout][2] result and the per-tile scratch of d2c_fwd_stats_ws() bytes, or NULL.

@@ -93,6 +93,38 @@ def test_kept_columns_against_oracle_and_plain_calls(name, dev, keep_columns_res
         assert rel_l2(a, p) < (4e-3 if n == "grad_weight" else 1e-3), (name, n, rel_l2(a, p))
 
 
+@pytest.mark.parametrize("name", ["c128_o192_G2", "c256_groups2_o640_nomask"])
+def test_kept_columns_float32(name, dev, keep_columns_restored):
+    """float32: the forward kernel keeps the interpolated values themselves (not the two-term operands its matrix
+    step reads) and the grad-weight product runs on the float32 matrix instruction: against the float64 oracle
+    grad_weight stays within 3e-6 of the tensor's scale, as on the path that samples again."""
+    N, Cin, Cout, dims, groups, G, bias, mask, sig = SHAPES[name]
+    (x, off, m, w, b), gout, _ = make(name, seed=2)
+    x, w, gout = x.float(), w.float(), gout.float()
+    b = b.float() if b is not None else None
+    dd = lambda t: t.double() if t is not None else None
+    e_out = cpu.conv3d_forward(dd(x), dd(off), dd(m), dd(w), dd(b), 1, 1, 1, groups, G)
+    eg = cpu.conv3d_backward(dd(gout), dd(x), dd(off), dd(m), dd(w), b is not None, 1, 1, 1, groups, G)
+    expected = [e_out] + list(eg)
+    _ops.config.set_keep_columns(True)
+    kept = step((x, off, m, w, b), gout, groups, G, dev)
+    _ops.config.set_keep_columns(False)
+    plain = step((x, off, m, w, b), gout, groups, G, dev)
+    names = ("out", "grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias")
+    for n, a, p, e in zip(names, kept, plain, expected):
+        if a is None:
+            assert p is None
+            continue
+        d = (a.double().cpu() - e).abs() / e.abs().max()
+        if n == "grad_offset":
+            # (a sampling coordinate within float32 rounding of a whole number lands on the other side of it than in
+            # float64, where the derivative jumps: a few entries in a million, the same ones on both paths)
+            assert (d > 2e-5).sum().item() <= 1e-5 * d.numel(), (name, n, (d > 2e-5).sum().item())
+        else:
+            assert d.max().item() < (3e-6 if n in ("grad_weight", "grad_bias") else 2e-5), (name, n, d.max().item())
+        assert rel_l2(a, p) < 2e-6, (name, n, rel_l2(a, p))
+
+
 def test_kept_columns_when_only_the_weights_want_a_gradient(dev, keep_columns_restored):
     (x, off, m, w, b), gout, (groups, G) = make("c128_o192_G2", seed=1)
     f = lambda t: t.float() if t is not None else None
@@ -133,9 +165,11 @@ def test_column_buffer_checks(dev):
     lib = _lib.load()
     (x, off, m, w, b), gout, (groups, G) = make("c128_o192_G2")
     dims = SHAPES["c128_o192_G2"][3]
-    # descriptions that keep no columns: float32, and problems on the small-tile forward kernel
+    # float32: [chunk of 32 channels][tap][rows][32] floats
     f32 = desc_of(x, w, dims, groups, G, dtype=_lib.D2C_F32)
-    assert lib.d2c_conv3d_columns_bytes(ctypes.byref(f32), None) == 0
+    rows = (dims[0] * dims[1] * dims[2] + 63) // 64 * 64
+    assert lib.d2c_conv3d_columns_bytes(ctypes.byref(f32), None) == x.shape[1] // 32 * 27 * rows * 32 * 4
+    # descriptions that keep no columns: problems on the small-tile forward kernel
     small = desc_of(x, w, (3, 6, 9), groups, G)
     assert lib.d2c_conv3d_columns_bytes(ctypes.byref(small), None) == 0
     desc = desc_of(x, w, dims, groups, G)
@@ -150,7 +184,7 @@ def test_column_buffer_checks(dev):
                                                           p(ts[4]), p(out), c, n, p(ws), nws, None)
     assert call(desc, p(cols), ncol - 1) == 3 and "column buffer" in _lib.last_error()
     assert call(desc, None, ncol) == 3
-    assert call(f32, p(cols), ncol) == 5 and "keeps no columns" in _lib.last_error()
+    assert call(small, p(cols), ncol) == 5 and "keeps no columns" in _lib.last_error()
     assert call(desc, p(cols), ncol) == 0
     torch.cuda.synchronize()
 
