@@ -190,10 +190,13 @@ int d2c_conv3d_backward(const d2c_conv3d_desc *desc, const void *grad_out, const
  * taps x the size of the input, in the element type): the forward kernel writes there what it multiplies with the
  * weights anyway, and d2c_conv3d_backward_columns, given that buffer UNCHANGED together with the same tensors, runs
  * its grad-weight product over it instead of sampling again (N=2, C=512, 8x30x54, bfloat16: 2.46 -> 2.39 ms per step
- * for 717 MB held between the two calls, and 0.72 GB less backward workspace).  Results are those of the plain calls
- * up to the order of floating-point sums.  `size_map` as in d2c_conv3d_forward_stats: NULL, or the description of
+ * for 717 MB held between the two calls, and 0.72 GB less backward workspace; N=2, C=256, 8x30x54, float32: 2.77 ->
+ * 2.48 ms for 717 MB).  Results are those of the plain calls up to the order of floating-point sums; float32
+ * columns are the interpolated floats themselves and their product runs on the float32 matrix instruction,
+ * whatever D2C_BWD_F32_SPLIT says.  `size_map` as in d2c_conv3d_forward_stats: NULL, or the description of
  * the size map that `offset` then is.  d2c_conv3d_columns_bytes() is 0 where this is not served (anything but
- * bfloat16 problems on the large-tile matrix-core kernels with offsets along all three axes); the two calls then
+ * bfloat16 and float32 problems on the large-tile matrix-core kernels with offsets along all three axes and an even
+ * number of 64- / 32-channel chunks per weight group); the two calls then
  * fail with D2C_ERR_UNSUPPORTED and the caller uses the plain ones.  The memory-saving bits of
  * d2c_conv3d_desc::backward_flags are ignored by d2c_conv3d_backward_columns.
  */
