@@ -1472,6 +1472,237 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col_kernel(BwdWeigh
     }
 }
 
+// ============================================================ kernel 2c
+// The same product for float problems on the bfloat16 matrix instruction, with float32's accuracy: every float is
+// taken apart into THREE bfloat16 terms, v = h + m + l exactly (8 + 8 + 8 significant bits), and of the nine partial
+// products of a pair the six largest are summed,
+//     h h' + m h'   |   h m' + m m'   |   l h' + h l'
+// three v_mfma_f32_32x32x16_bf16 per 8 positions (each 16-deep reduction holds two partial products of 8 pairs)
+// against four v_mfma_f32_32x32x2_f32 of twice their length: 3/8 of the matrix-pipe time.  What is dropped
+// (m l' + l m' + l l') is below 2^-25 of a product, under float32's own rounding.  The first instruction carries the
+// leading term and adds into one accumulator, the two others (terms of at most 2^-8 of it) into a second one, and
+// the two are added at the end: the large sum is rounded once per 8 positions instead of four times.
+//
+// One workgroup = one tap and four channel chunks (128 columns), 256 output channels (8 wavefronts x 32 rows),
+// looping over its piece of the 64-position tiles like tiled_bwd_weight_col_kernel.  The float columns are taken
+// apart where they are stored to LDS -- three planes [position][32 channels] of bfloat16 per chunk, read with the
+// transposing LDS load -- and grad_out comes from a fragment-ordered copy that holds the three terms (pack_gout3_kernel).
+constexpr int kCol3Chunks = 4;
+constexpr int kCol3Rows = 256;     // output channels per workgroup
+constexpr size_t kCol3Lds = (size_t)2 * kCol3Chunks * 3 * kWDT * 64;
+
+// v -> (h, m, l), bfloat16 bits
+D2C_DEV void split3(float v, uint32_t &h, uint32_t &m, uint32_t &l)
+{
+    h = f32_to_bf16(v);
+    const float r1 = bf16_residual(v, h << 16);
+    m = f32_to_bf16(r1);
+    l = f32_to_bf16(r1 - __uint_as_float(m << 16));
+}
+
+// grad_out [N][Cout][P] -> fragments of the three terms, indexed like pack_gout_kernel's (float: 16 k-groups of 8
+// positions per tile of kWMT): lh[i] = (l0 l1)(l2 l3)(h0 h1)(h2 h3) of the lane's four positions, md[i] = (m0 m1)(m2 m3);
+// `md` follows the `total` 16-byte entries of `lh`
+__global__ void __launch_bounds__(256) pack_gout3_kernel(const float *gout, uint4 *lh, TiledShape s, int ntile, int OBT,
+                                                         long total)
+{
+    constexpr int VEC = 4, NKGT = kWMT / (2 * VEC);
+    uint2 *md = reinterpret_cast<uint2 *>(lh + total);
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int lane = (int)(i & 63);
+        long r = i >> 6;
+        const int kg = (int)(r % NKGT); r /= NKGT;
+        const int ob = (int)(r % OBT); r /= OBT;
+        const int tile = (int)(r % ntile);
+        const int wg = (int)(r / ntile);
+        const int ol = ob * 32 + (lane & 31);
+        const long m0 = (long)tile * kWMT + (2 * kg + (lane >> 5)) * VEC;
+        uint32_t h[VEC], m[VEC], l[VEC];
+#pragma unroll
+        for (int q = 0; q < VEC; q++) {
+            const long mm = m0 + q;
+            float v = 0.f;
+            if (ol < s.og && mm < s.M) {
+                const int b = (int)(mm / s.P), pp = (int)(mm - (long)b * s.P);
+                v = gout[((long)b * s.Cout + wg * s.og + ol) * s.P + pp];
+            }
+            split3(v, h[q], m[q], l[q]);
+        }
+        lh[i] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        md[i] = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
+    }
+}
+
+struct BwdWeightCol3Args {
+    TiledShape s;
+    const void *col;     // [chunk][tap][mpad][32] float
+    const uint4 *lh;     // grad_out fragments, see pack_gout3_kernel
+    const uint2 *md;
+    float *gwacc;        // as in BwdWeightArgs
+    long mpad;           // rows per (chunk, tap) of `col`: whole 64-position tiles
+    int otiles, nmain, main_len, ntail, tail_len;   // as in BwdWeightArgs (output tiles of kCol3Rows channels)
+};
+
+__global__ void __launch_bounds__(kThreads) tiled_bwd_weight_col3_kernel(BwdWeightCol3Args a)
+{
+    constexpr int MT = kWDT, NCH = kCol3Chunks, CB = NCH, NT = kCol3Rows;
+    constexpr int NKG = MT / 8;                // k-groups (8 positions) per tile
+    constexpr int NKGP = kWMT / 8;             // ... per tile of the packed grad_out copy
+    constexpr int PLANE = MT * 64;             // bytes of one term of one chunk: [position][32 channels] bfloat16
+    constexpr int LAK = 4;                     // k-groups of grad_out fragments in flight
+    static_assert(MT * 8 == kThreads, "one (position, vector) item per thread and column tile");
+    extern __shared__ __align__(16) unsigned char s_tile[];   // [2 buffers][NCH][3 terms][PLANE]
+
+    const TiledShape &s = a.s;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ntile = (s.M + MT - 1) / MT;
+    const int nstep = (s.nchunk / NCH) * s.K;
+    const int nitem = s.groups * a.otiles * nstep;
+    int item, t_lo, nmy, t_step;
+    if ((int)blockIdx.x < nitem * a.nmain) {
+        item = blockIdx.x % nitem;
+        t_lo = blockIdx.x / nitem;
+        t_step = a.nmain;
+        const int nt = min(ntile, a.nmain * a.main_len);
+        nmy = nt > t_lo ? (nt - t_lo + t_step - 1) / t_step : 0;
+    } else {
+        const int id = blockIdx.x - nitem * a.nmain;
+        item = id % nitem;
+        t_lo = a.nmain * a.main_len + id / nitem;
+        t_step = a.ntail;
+        nmy = ntile > t_lo ? (ntile - t_lo + t_step - 1) / t_step : 0;
+    }
+    if (nmy <= 0) return;
+    const int st = item % nstep, otile = (item / nstep) % a.otiles, wg = item / (nstep * a.otiles);
+    const int jq = st / s.K, k = st % s.K;
+    const int o_base = otile * NT + wave * 32;
+    const bool mma_wave = o_base < s.og;
+
+    f32x16 big[CB], small[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) big[cb][r] = small[cb][r] = 0.f;
+
+    // --- column tiles: thread = (position, 16-byte vector of 4 channels) of each of the four tiles of a step
+    const int ipos = tid >> 3, ivec = tid & 7;
+    const long chunk0 = (long)wg * s.nchunk + jq * NCH;
+    const long cstride = (long)s.K * a.mpad * 8;      // 16-byte vectors from one chunk to the next
+    const uint4 *const colp = reinterpret_cast<const uint4 *>(a.col) + ((chunk0 * s.K + k) * a.mpad + ipos) * 8 + ivec;
+    // (past the end of the piece the last tile is requested again: the same loads in every iteration)
+    auto col_row0 = [&](int i) { return (long)(t_lo + min(i, nmy - 1) * t_step) * MT * 8; };
+    uint4 cr[NCH];       // the tile after the one on the matrix cores, requested a whole step before it is stored
+    unsigned char *const st_p = s_tile + ipos * 64 + ivec * 8;
+    auto put = [&](int buf, int c, const uint4 &v) {
+        uint32_t h[4], m[4], l[4];
+        split3(__uint_as_float(v.x), h[0], m[0], l[0]);
+        split3(__uint_as_float(v.y), h[1], m[1], l[1]);
+        split3(__uint_as_float(v.z), h[2], m[2], l[2]);
+        split3(__uint_as_float(v.w), h[3], m[3], l[3]);
+        unsigned char *d = st_p + ((buf * NCH + c) * 3) * PLANE;
+        *reinterpret_cast<uint2 *>(d) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        *reinterpret_cast<uint2 *>(d + PLANE) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
+        *reinterpret_cast<uint2 *>(d + 2 * PLANE) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
+    };
+
+    // --- grad_out fragments of this wavefront's 32 rows
+    const int OBT = (s.og + 63) / 64 * 2;
+    const int ntp = (s.M + kWMT - 1) / kWMT;
+    const long f0 = (((long)wg * ntp * OBT + (mma_wave ? o_base >> 5 : 0)) * NKGP) * 64 + lane;
+    auto frag_at = [&](int i, int kg) {       // index of k-group kg of tile i of this piece
+        const long t64 = t_lo + (long)min(i, nmy - 1) * t_step;
+        const long tp = t64 / (kWMT / MT);
+        const int kgp = (int)(t64 % (kWMT / MT)) * NKG + kg;
+        return f0 + ((tp * OBT) * NKGP + kgp) * 64;
+    };
+    uint4 alh[LAK];
+    uint2 amd[LAK];
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    const int l16 = lane & 15, g16 = lane >> 4;
+    // this lane's part of the transposing reads (ds_read_b64_tr_b16: within 16 lanes, lane l element j comes from lane
+    // 4j + l/4, element l%4): it reads 4 channels of position 4 * (g16 >> 1) + (l16 >> 2) of a k-group and receives
+    // channel (g16 & 1) * 16 + l16 at the four positions 4 * (g16 >> 1) ..
+    const unsigned char *const rd_p = s_tile + (4 * (g16 >> 1) + (l16 >> 2)) * 64 + ((g16 & 1) * 16 + (l16 & 3) * 4) * 2;
+    auto tr = [&](const unsigned char *p) {
+        return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)p));
+    };
+
+    {
+#pragma unroll
+        for (int q = 0; q < LAK; q++) {
+            const long f = frag_at(0, q);
+            alh[q] = a.lh[f];
+            amd[q] = a.md[f];
+        }
+        const long r0 = col_row0(0), r1 = col_row0(1);
+#pragma unroll
+        for (int c = 0; c < NCH; c++) cr[c] = ld_stream16(colp + c * cstride + r0);
+#pragma unroll
+        for (int c = 0; c < NCH; c++) {
+            put(0, c, cr[c]);
+            cr[c] = ld_stream16(colp + c * cstride + r1);
+        }
+    }
+    lds_only_barrier();
+    auto run = [&](auto mma_c) {
+        constexpr bool MMA = decltype(mma_c)::value;
+        for (int it = 0; it < nmy; it++) {
+            const int dbuf = it & 1;
+            if constexpr (MMA) {
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    const int q = kg % LAK;
+                    const uint4 a_lh = alh[q];
+                    const uint4 a_hm = make_uint4(alh[q].z, alh[q].w, amd[q].x, amd[q].y);
+#pragma unroll
+                    for (int cb = 0; cb < CB; cb++) {
+                        const unsigned char *bp = rd_p + ((dbuf * NCH + cb) * 3) * PLANE + kg * 8 * 64;
+                        const uint2 bh = tr(bp), bm = tr(bp + PLANE), bl = tr(bp + 2 * PLANE);
+                        const uint4 b_hh = make_uint4(bh.x, bh.y, bh.x, bh.y), b_mm = make_uint4(bm.x, bm.y, bm.x, bm.y);
+                        const uint4 b_hl = make_uint4(bh.x, bh.y, bl.x, bl.y);
+                        big[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a_hm),
+                                                                          __builtin_bit_cast(bf16x8_t, b_hh), big[cb], 0, 0, 0);
+                        small[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a_hm),
+                                                                            __builtin_bit_cast(bf16x8_t, b_mm), small[cb], 0, 0, 0);
+                        small[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a_lh),
+                                                                            __builtin_bit_cast(bf16x8_t, b_hl), small[cb], 0, 0, 0);
+                    }
+                    // the slot is refilled with the fragment LAK k-groups on (of the next tile, past this one's last)
+                    const long f = kg + LAK < NKG ? frag_at(it, kg + LAK) : frag_at(it + 1, kg + LAK - NKG);
+                    alh[q] = a.lh[f];
+                    amd[q] = a.md[f];
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            // (the other buffer was last read in the iteration before, which every wavefront has left)
+            const long r2 = col_row0(it + 2);
+#pragma unroll
+            for (int c = 0; c < NCH; c++) {
+                put(dbuf ^ 1, c, cr[c]);
+                cr[c] = ld_stream16(colp + c * cstride + r2);
+            }
+            lds_only_barrier();
+        }
+    };
+    if (mma_wave) run(std::true_type{});
+    else run(std::false_type{});
+
+    if (mma_wave) {
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            const int stw = (jq * NCH + cb) * s.K + k;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int ol = o_base + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (ol < s.og)
+                    atomicAdd(a.gwacc + (((long)wg * s.nchunk * s.K + stw) * s.og + ol) * 32 + (lane & 31),
+                              big[cb][r] + small[cb][r]);
+            }
+        }
+    }
+}
+
 template <typename T, int NC> constexpr size_t bwd_weight_dma_lds()
 {
     constexpr int BKC = 8 * Elem<T>::VEC;
@@ -1856,7 +2087,8 @@ size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype)
 {
     const int vec = dtype == D2C_BF16 ? 8 : 4;
     const long ntile = (s.M + kWMT - 1) / kWMT, OBT = (s.og + 63) / 64 * 2;
-    return (size_t)s.groups * ntile * OBT * (kWMT / (2 * vec)) * 64 * 16;
+    // (float: 24 bytes per entry where the copy holds three bfloat16 terms, see pack_gout3_kernel)
+    return (size_t)s.groups * ntile * OBT * (kWMT / (2 * vec)) * 64 * (dtype == D2C_BF16 ? 16 : 24);
 }
 
 // How the position tiles of the grad-weight items are cut into workgroups (see BwdWeightArgs), found by simulating
@@ -1928,6 +2160,8 @@ bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype)
 {
     return dtype == D2C_BF16 && s.nd == 3 && s.nchunk % kColChunks == 0;
 }
+// float problems over kept columns on three-term bfloat16 operands: weight groups of whole sets of kCol3Chunks chunks
+bool d2c_bwd_weight_col3(const TiledShape &s) { return s.nd == 3 && s.nchunk % kCol3Chunks == 0; }
 // ... from the columns that the forward call kept (d2c_fwd_writes_columns): float problems as well
 bool d2c_bwd_weight_from_kept_col(const TiledShape &s, int dtype)
 {
@@ -1963,13 +2197,22 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     const int ntp = (s.M + kWMT - 1) / kWMT;     // tiles of the packed grad_out copy
     const int ntile = (s.M + kWDT - 1) / kWDT;   // position tiles of the kernel
     const bool from_col = col != nullptr;
-    if (phase & 1) {
+    // float problems over kept columns: the product on three-term bfloat16 operands (tiled_bwd_weight_col3_kernel)
+    bool col3 = false;
+    if constexpr (sizeof(T) == 4) col3 = from_col && d2c_bwd_weight_col3(s);
+    const int OBT = (s.og + 63) / 64 * 2;
+    const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
+    if ((phase & 1) && col3) {
+        D2cProfScope prof(D2C_PROF_PACK, st);
+        d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
+        hipLaunchKernelGGL(pack_gout3_kernel, dim3(grid1d(total, 16384)), dim3(256), 0, st, (const float *)gout,
+                           (uint4 *)goutp, s, ntp, OBT, total);
+        if (int rc = d2c_check_launch("pack_gout3_kernel")) return rc;
+    } else if (phase & 1) {
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(gwacc, (size_t)nw * sizeof(float), st);
         // (the channels-last input is followed by a 256-byte row of zeros, written by the kernel that packed it:
         // what dead corners read)
-        const int OBT = (s.og + 63) / 64 * 2;
-        const long total = (long)s.groups * ntp * OBT * (kWMT / (2 * Elem<T>::VEC)) * 64;
         const bool vec = s.P % Elem<T>::VEC == 0 && reinterpret_cast<uintptr_t>(gout) % 16 == 0;
         constexpr bool SPT = sizeof(T) == 4;
         // (the product over kept columns runs on the float instruction whatever the flags say)
@@ -1990,6 +2233,26 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
     if (jp_n > 0 && !from_col) {
         d2c_set_error("grad_weight: slices are made by tiled_bwd_weight_col_kernel only");
         return D2C_ERR_LAUNCH;
+    }
+    if (col3) {
+        if (jp_n > 0) {
+            d2c_set_error("grad_weight: tiled_bwd_weight_col3_kernel takes no slices");
+            return D2C_ERR_LAUNCH;
+        }
+        if (phase & 2) {
+            const int otiles3 = (s.og + kCol3Rows - 1) / kCol3Rows;
+            const long items3 = (long)(s.nchunk / kCol3Chunks) * s.K * otiles3 * s.groups;
+            const GwPieces pc = gw_pieces(items3, ntile, ncu, 4);
+            BwdWeightCol3Args c{s, col, (const uint4 *)goutp, reinterpret_cast<const uint2 *>((const uint4 *)goutp + total),
+                                gwacc, col_rows, otiles3, pc.nmain, pc.main_len, pc.ntail, pc.tail_len};
+            if (int rc = d2c_allow_lds((const void *)tiled_bwd_weight_col3_kernel, (int)kCol3Lds, "tiled_bwd_weight_col3_kernel"))
+                return rc;
+            D2cProfScope prof(D2C_PROF_BWD_WEIGHT, st, "tiled_bwd_weight_col3_kernel");
+            hipLaunchKernelGGL(tiled_bwd_weight_col3_kernel, dim3((unsigned)(items3 * (pc.nmain + pc.ntail))), dim3(kThreads),
+                               kCol3Lds, st, c);
+            if (int rc = d2c_check_launch("tiled_bwd_weight_col3_kernel")) return rc;
+        }
+        phase &= ~2;
     }
     if (jp_n <= 0) { jp_lo = 0; jp_n = s.nchunk / kColChunks; }
     const long items = (long)(from_col ? jp_n * s.K : steps) * otiles * s.groups;
