@@ -716,6 +716,21 @@ def main():
                     "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dt], 4), "traffic": traffic,
                     "traffic_source": traffic_source, "algorithmic_gflop_per_launch": round(f_fwd_flops / 1e9, 2),
                     "whole_step_frac": round(value / PEAK_TFLOPS[dt], 4), "kernel_ms": kms}
+        # float32 workloads: most matrix kernels run on the bfloat16 instruction with every float operand taken apart
+        # into two or three bfloat16 terms, so `frac` (against the float32 instruction's peak) can pass 1; the
+        # instructions executed are the partial products
+        if dt == "f32":
+            terms = {"tiled_fwd_dma_kernel": 4, "tiled_fwd_kernel": 4, "tiled_bwd_weight_col3_kernel": 6,
+                     "tiled_bwd_col_kernel": 4}
+            if args.f32_split_backward:
+                terms.update({"tiled_bwd_weight_dma_kernel": 4, "tiled_bwd_data_kernel": 4})
+            if dom in terms:
+                ex = terms[dom] * ach
+                roofline["on_bf16_instructions"] = {
+                    "partial_products_per_product": terms[dom], "executed_tflops": round(ex, 1),
+                    "frac_of_bf16_peak": round(ex / PEAK_TFLOPS["bf16"], 4),
+                    "note": "float operands as sums of bfloat16 terms on v_mfma_f32_32x32x16_bf16; `peak` above is "
+                            "the float32 instruction's"}
         if plain_fwd_ms and role[dom] == "fwd":
             ach0 = f_fwd_flops / (plain_fwd_ms * 1e-3) / 1e12
             roofline["note"] = ("this launch also writes the sampled columns that the backward call of the step "

@@ -191,9 +191,9 @@ int d2c_conv3d_backward(const d2c_conv3d_desc *desc, const void *grad_out, const
  * weights anyway, and d2c_conv3d_backward_columns, given that buffer UNCHANGED together with the same tensors, runs
  * its grad-weight product over it instead of sampling again (N=2, C=512, 8x30x54, bfloat16: 2.46 -> 2.39 ms per step
  * for 717 MB held between the two calls, and 0.72 GB less backward workspace; N=2, C=256, 8x30x54, float32: 2.77 ->
- * 2.48 ms for 717 MB).  Results are those of the plain calls up to the order of floating-point sums; float32
- * columns are the interpolated floats themselves and their product runs on the float32 matrix instruction,
- * whatever D2C_BWD_F32_SPLIT says.  `size_map` as in d2c_conv3d_forward_stats: NULL, or the description of
+ * 2.25 ms for 717 MB).  Results are those of the plain calls up to the order of floating-point sums; float32
+ * columns are the interpolated floats themselves and their product keeps float32's accuracy (three bfloat16 terms
+ * per float on the bfloat16 matrix instruction, or the float32 instruction), whatever D2C_BWD_F32_SPLIT says.  `size_map` as in d2c_conv3d_forward_stats: NULL, or the description of
  * the size map that `offset` then is.  d2c_conv3d_columns_bytes() is 0 where this is not served (anything but
  * bfloat16 and float32 problems on the large-tile matrix-core kernels with offsets along all three axes and an even
  * number of 64- / 32-channel chunks per weight group); the two calls then
