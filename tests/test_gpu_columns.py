@@ -98,7 +98,7 @@ def test_kept_columns_against_oracle_and_plain_calls(name, dev, keep_columns_res
         assert rel_l2(a, p) < (4e-3 if n == "grad_weight" else 1e-3), (name, n, rel_l2(a, p))
 
 
-@pytest.mark.parametrize("name", ["c128_o192_G2", "c256_groups2_o640_nomask", "c192_o256_G2"])
+@pytest.mark.parametrize("name", ["c128_o192_G2", "c256_o512_G4_ragged", "c256_groups2_o640_nomask", "c192_o256_G2"])
 def test_kept_columns_float32(name, dev, keep_columns_restored):
     """float32: the forward kernel keeps the interpolated values themselves (not the two-term operands its matrix
     step reads) and the grad-weight product runs over them with float32's accuracy -- on three-term bfloat16
@@ -127,8 +127,13 @@ def test_kept_columns_float32(name, dev, keep_columns_restored):
             # (a sampling coordinate within float32 rounding of a whole number lands on the other side of it than in
             # float64, where the derivative jumps: a few entries in a million, the same ones on both paths)
             assert (d > 2e-5).sum().item() <= 1e-5 * d.numel(), (name, n, (d > 2e-5).sum().item())
+        elif n in ("grad_weight", "grad_bias"):
+            # (3e-6 of the tensor's scale, or what the path that samples again leaves: weight groups wider than one
+            # pass of the backward kernels keep no columns, both steps then are the plain one)
+            dp = ((p.double().cpu() - e).abs() / e.abs().max()).max().item()
+            assert d.max().item() < max(3e-6, 1.2 * dp), (name, n, d.max().item(), dp)
         else:
-            assert d.max().item() < (3e-6 if n in ("grad_weight", "grad_bias") else 2e-5), (name, n, d.max().item())
+            assert d.max().item() < 2e-5, (name, n, d.max().item())
         assert rel_l2(a, p) < 2e-6, (name, n, rel_l2(a, p))
 
 
@@ -196,8 +201,9 @@ def test_column_buffer_checks(dev):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("cls", ["MDConv3d", "XYZSizeConditionedMDConv3d"])
-def test_layers_keep_columns_with_the_deformation_tensor_read_in_place(cls, dev, keep_columns_restored):
+def test_layers_keep_columns_with_the_deformation_tensor_read_in_place(cls, dtype, dev, keep_columns_restored):
     """The self-deforming layers hand the operator their deformation branch's output as it is (offsets and raw
     modulation in one tensor, activation in the sampler): the same step with and without kept columns."""
     from d2conv3d_amd import modules as M
@@ -206,9 +212,9 @@ def test_layers_keep_columns_with_the_deformation_tensor_read_in_place(cls, dev,
     with torch.no_grad():
         layer.deform_params.weight.normal_(0, 0.02)
         layer.deform_params.bias.normal_(0, 0.5)
-    layer = layer.to(torch.bfloat16)
-    x = torch.randn(1, 128, 9, 32, 32, device=dev).bfloat16()
-    gout = torch.randn(1, 192, 9, 32, 32, device=dev).bfloat16()
+    layer = layer.to(dtype)
+    x = torch.randn(1, 128, 9, 32, 32, device=dev).to(dtype)
+    gout = torch.randn(1, 192, 9, 32, 32, device=dev).to(dtype)
     res = []
     for keep in (True, False):
         _ops.config.set_keep_columns(keep)
@@ -217,4 +223,4 @@ def test_layers_keep_columns_with_the_deformation_tensor_read_in_place(cls, dev,
         layer(xi).backward(gout)
         res.append([xi.grad] + [p.grad.clone() for p in layer.parameters()])
     for i, (a, p) in enumerate(zip(*res)):
-        assert rel_l2(a, p) < 5e-3, (cls, i, rel_l2(a, p))
+        assert rel_l2(a, p) < (5e-3 if dtype == torch.bfloat16 else 5e-6), (cls, i, rel_l2(a, p))
