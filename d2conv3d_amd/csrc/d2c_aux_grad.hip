@@ -261,8 +261,14 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) aux_grad_kernel(AuxArgs a
                         va.zero();
 #pragma unroll
                         for (int c = 0; c < 8; c++) va.fma(czy[c >> 1] * cx[c & 1], xv[r][c]);
-                        const uint4 cv = va.pack();
-                        pend_v = u32x4{cv.x, cv.y, cv.z, cv.w};
+                        // (float: the interpolated values themselves, not the two-term operand form of pack())
+                        if constexpr (sizeof(T) == 4) {
+                            pend_v = u32x4{__float_as_uint(va.a[0]), __float_as_uint(va.a[1]), __float_as_uint(va.a[2]),
+                                           __float_as_uint(va.a[3])};
+                        } else {
+                            const uint4 cv = va.pack();
+                            pend_v = u32x4{cv.x, cv.y, cv.z, cv.w};
+                        }
                         pend_p = m0 + pos < a.mpad
                                      ? reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(a.col)
                                            + ((((long)(c0 / BKC) * s.K + k) * a.mpad + m0 + pos) * BKC + ivec * VEC) * (long)sizeof(T))
@@ -384,30 +390,25 @@ int d2c_aux_grad_launch(const TiledShape &s, const void *xcl, const void *off, c
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;
     D2cProfScope prof(D2C_PROF_BWD_AUX, st, "aux_grad_kernel");
     const dim3 blk(64 * kWavesPerBlock);
-    if constexpr (sizeof(T) == 2) {
-        // (the sampled columns are written for bfloat16 problems in three dimensions only, see d2c_bwd_weight_from_col)
-        if (col && s.nd == 3) {
-            if (aux16) {
-                if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, true, true, true>), grid, blk, 0, st, a);
-                else hipLaunchKernelGGL((aux_grad_kernel<T, true, false, true>), grid, blk, 0, st, a);
-            } else {
-                if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, false, true, true>), grid, blk, 0, st, a);
-                else hipLaunchKernelGGL((aux_grad_kernel<T, false, false, true>), grid, blk, 0, st, a);
-            }
-            return d2c_check_launch("aux_grad_kernel");
-        }
-        if (aux16) {
-            if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, true, true, false>), grid, blk, 0, st, a);
-            else hipLaunchKernelGGL((aux_grad_kernel<T, true, false, false>), grid, blk, 0, st, a);
-        }
-    }
-    if (col && (sizeof(T) != 2 || s.nd != 3)) {
-        d2c_set_error("aux_grad_kernel: sampled columns are written for bfloat16 problems in three dimensions only");
+    if (col && s.nd != 3) {
+        d2c_set_error("aux_grad_kernel: sampled columns are written for problems in three dimensions only");
         return D2C_ERR_LAUNCH;
     }
+    // (the sampled columns: problems in three dimensions, see d2c_bwd_weight_from_col)
+    auto go = [&](auto aux_c, auto sized_c) {
+        constexpr bool A16 = decltype(aux_c)::value, SZ = decltype(sized_c)::value;
+        if (col) hipLaunchKernelGGL((aux_grad_kernel<T, A16, SZ, true>), grid, blk, 0, st, a);
+        else hipLaunchKernelGGL((aux_grad_kernel<T, A16, SZ, false>), grid, blk, 0, st, a);
+    };
+    if constexpr (sizeof(T) == 2) {
+        if (aux16) {
+            if (s.ss.on) go(std::true_type{}, std::true_type{});
+            else go(std::true_type{}, std::false_type{});
+        }
+    }
     if (!aux16) {
-        if (s.ss.on) hipLaunchKernelGGL((aux_grad_kernel<T, false, true, false>), grid, blk, 0, st, a);
-        else hipLaunchKernelGGL((aux_grad_kernel<T, false, false, false>), grid, blk, 0, st, a);
+        if (s.ss.on) go(std::false_type{}, std::true_type{});
+        else go(std::false_type{}, std::false_type{});
     }
     return d2c_check_launch("aux_grad_kernel");
 }

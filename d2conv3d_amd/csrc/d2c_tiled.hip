@@ -49,7 +49,7 @@ int d2c_tiled_bwd_weight_launch(const TiledShape &s, const void *gout, const voi
                                 hipStream_t st, int phase = 7, int jp_lo = 0, int jp_n = 0);
 bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype);
 bool d2c_bwd_weight_from_kept_col(const TiledShape &s, int dtype);
-size_t d2c_bwd_col_bytes(const TiledShape &s, int nchunks = 0);
+size_t d2c_bwd_col_bytes(const TiledShape &s, int dtype, int nchunks = 0);
 size_t d2c_bwd_goutp_bytes(const TiledShape &s, int dtype);
 template <typename T> int d2c_tiled_unpack_gx(const TiledShape &s, const float *gxcl, void *gx, hipStream_t st);
 template <typename T> int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStream_t st);
@@ -552,11 +552,16 @@ int gw_mode(const d2c_conv3d_desc &q)
 }
 bool use_col_weight(const d2c_conv3d_desc &q, const TiledShape &s)
 {
+    if (q.dtype != D2C_BF16 && gw_mode(q) != 1) return false;
     return gw_mode(q) && use_aux_kernel(q, s) && d2c_bwd_weight_from_col(s, q.dtype);
 }
 // ... written over the grad-column rows (mode 2): grad_input is taken from those rows first, from sample lists
 // that a pass of their own files
-bool col_in_place(const d2c_conv3d_desc &q, const TiledShape &s) { return gw_mode(q) == 2 && use_col_weight(q, s); }
+// (bfloat16 only: float problems asked for it sample again, as they always did)
+bool col_in_place(const d2c_conv3d_desc &q, const TiledShape &s)
+{
+    return gw_mode(q) == 2 && q.dtype == D2C_BF16 && use_col_weight(q, s);
+}
 
 // The backward pass slice by slice over the offset groups (see d2c_bwd_sliceable): `gs` groups per slice of the
 // grad-column rows (0: not sliced), `cgs` groups per block of sampled columns that one launch of the grad-weight
@@ -626,7 +631,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s, bool saved_columns =
     if (s.ss.on) w.total += d2c_align_up((size_t)s.N * 3 * s.P * sizeof(float));
     w.col = w.total;       // sampled columns for the grad-weight product
     if (!saved_columns && use_col_weight(q, s) && !col_in_place(q, s))
-        w.total += d2c_align_up(d2c_bwd_col_bytes(s, sl.cgs ? sl.cgs * (s.cpg / 64) : 0));
+        w.total += d2c_align_up(d2c_bwd_col_bytes(s, q.dtype, sl.cgs ? sl.cgs * (s.cpg / 64) : 0));
     return w;
 }
 

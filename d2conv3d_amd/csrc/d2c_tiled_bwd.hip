@@ -2154,24 +2154,23 @@ static GwPieces gw_pieces(long items, int ntile, int ncu, int max_main = 1)
     return r;
 }
 
-// grad_weight from the sampled columns (tiled_bwd_weight_col_kernel): bfloat16 problems in three dimensions whose
-// weight groups hold whole sets of kColChunks channel chunks.
+// grad_weight from the sampled columns (tiled_bwd_weight_col_kernel, tiled_bwd_weight_col3_kernel): problems in three
+// dimensions whose weight groups hold whole sets of kColChunks channel chunks.
 bool d2c_bwd_weight_from_col(const TiledShape &s, int dtype)
-{
-    return dtype == D2C_BF16 && s.nd == 3 && s.nchunk % kColChunks == 0;
-}
-// float problems over kept columns on three-term bfloat16 operands: weight groups of whole sets of kCol3Chunks chunks
-bool d2c_bwd_weight_col3(const TiledShape &s) { return s.nd == 3 && s.nchunk % kCol3Chunks == 0; }
-// ... from the columns that the forward call kept (d2c_fwd_writes_columns): float problems as well
-bool d2c_bwd_weight_from_kept_col(const TiledShape &s, int dtype)
 {
     return (dtype == D2C_BF16 || dtype == D2C_F32) && s.nd == 3 && s.nchunk % kColChunks == 0;
 }
-// bytes of the sampled columns [chunk][tap][whole 64-position tiles][64] of `nchunks` channel chunks (0: all)
-size_t d2c_bwd_col_bytes(const TiledShape &s, int nchunks)
+// float problems over kept columns on three-term bfloat16 operands: weight groups of whole sets of kCol3Chunks chunks
+bool d2c_bwd_weight_col3(const TiledShape &s) { return s.nd == 3 && s.nchunk % kCol3Chunks == 0; }
+// ... from the columns that the forward call kept (d2c_fwd_writes_columns): the same shapes
+bool d2c_bwd_weight_from_kept_col(const TiledShape &s, int dtype) { return d2c_bwd_weight_from_col(s, dtype); }
+// bytes of the sampled columns [chunk][tap][whole 64-position tiles][64 bfloat16 / 32 float] of `nchunks` channel
+// chunks (0: all)
+size_t d2c_bwd_col_bytes(const TiledShape &s, int dtype, int nchunks)
 {
     const long ntile = (s.M + kWDT - 1) / kWDT;
-    return (size_t)(nchunks > 0 ? nchunks : s.Cin / 64) * s.K * ntile * kWDT * 64 * 2;
+    const int bkc = dtype == D2C_BF16 ? 64 : 32;
+    return (size_t)(nchunks > 0 ? nchunks : s.Cin / bkc) * s.K * ntile * kWDT * 128;
 }
 
 // The backward pass of this shape can run slice by slice over its offset groups (grad-column product, offset / mask

@@ -146,6 +146,33 @@ def test_grad_weight_from_columns_matches_resampling(name, wanted, dev):
     assert rel_l2(got["in_place"], got["columns"].float().cpu()) < 1e-3
 
 
+@pytest.mark.parametrize("name", ["c64_g1", "c128_G2_o96", "c256_groups2_G4_o384", "c256_G1_o200"])
+def test_float32_grad_weight_from_columns_matches_resampling(name, dev):
+    # float32 grad_weight on the plain calls (the forward call's columns not kept): as a matrix product over the float
+    # columns that the offset / mask gradient kernel writes -- on three-term bfloat16 operands where the weight groups
+    # hold sets of four 32-channel chunks, on the float32 matrix instruction otherwise -- or by sampling again; both
+    # against the float64 oracle, to 3e-6 of the tensor's scale
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, torch.float32, seed=6)
+    dd = lambda t: t.double() if t is not None else None
+    eg = cpu.conv3d_backward(dd(gout), dd(x), dd(off), dd(m), dd(w), b is not None, s, p, d, groups, G)
+    before = _ops.config.keep_columns()
+    _ops.config.set_keep_columns(False)
+    got = {}
+    try:
+        for mode in ("columns", "resample"):
+            _ops.set_grad_weight_mode(mode)
+            ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+            d2c.deform_conv3d(*ts, s, p, d, groups, G).backward(gout.to(dev))
+            got[mode] = ts[3].grad
+            err = ((got[mode].double().cpu() - eg[3]).abs().max() / eg[3].abs().max()).item()
+            assert err < 3e-6, (name, mode, err)
+            assert rel_l2(ts[0].grad, eg[0]) < 1e-5, (name, mode, rel_l2(ts[0].grad, eg[0]))
+    finally:
+        _ops.set_grad_weight_mode("columns")
+        _ops.config.set_keep_columns(before["on"], before["max_bytes"])
+    assert rel_l2(got["columns"], got["resample"].cpu()) < 2e-6
+
+
 @pytest.mark.parametrize("name", ["c256_G2_o512_tail", "c256_G4_o128", "c384_G6_o384_nomask", "c384_G3_o384"])
 @pytest.mark.parametrize("wanted", ["all", "x", "w+offset", "x+w"])
 def test_backward_in_slices_over_the_offset_groups(name, wanted, dev):

@@ -168,10 +168,11 @@ def test_float32_backward_on_split_operands(name, dev):
     dd = lambda t: t.double() if t is not None else None
     eg = cpu.conv3d_backward(dd(gout), dd(x), dd(off), dd(m), dd(w), b is not None, s, p, d, groups, G)
     errs = {}
-    # (without the forward call's columns: where those are kept, grad_weight is a product over them on the float32
-    # instruction whatever the flag says)
+    # (with grad_weight from the kernel that samples again: over sampled columns, the forward call's or the backward
+    # pass's own, the product keeps float32's accuracy whatever the flag says)
     before = _ops.config.keep_columns()
     _ops.config.set_keep_columns(False)
+    _ops.set_grad_weight_mode("resample")
     try:
         for split in (True, False):
             ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
@@ -184,5 +185,6 @@ def test_float32_backward_on_split_operands(name, dev):
                 errs[split].append(err)
                 assert err < (2e-5 if (split or n in ("grad_input", "grad_offset", "grad_mask")) else 2e-6), (name, n, split, err)
     finally:
+        _ops.set_grad_weight_mode("columns")
         _ops.config.set_keep_columns(before["on"], before["max_bytes"])
     assert errs[True][-2 if b is not None else -1] > errs[False][-2 if b is not None else -1]   # (grad_weight: the flag did change the arithmetic)
