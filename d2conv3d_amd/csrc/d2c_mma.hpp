@@ -47,12 +47,16 @@ D2C_DEV uint32_t pack_bf16x2(float lo, float hi)
 // v_mfma_f32_32x32x16_bf16 whose 16-deep reductions hold all four partial products of every element,
 // (hi + lo) * (hi' + lo'), summed in float32 by the matrix core: a quarter of the matrix-pipe time of the four float
 // instructions.  The producers of the forward operands (weight re-layout, sampled tile) write this form.
-// The BACKWARD kernels keep plain floats and the float instruction by default: the relative error of 4e-6 that the
-// two-term operands leave in a long sum is fine for the output (values of order 1 against 1e-4 relative / 1e-5
-// absolute) but not for gradients whose elements reach 20 .. 400 and are held to the same absolute 1e-5.  A caller
-// who prefers the speed asks for split operands there too (D2C_BWD_F32_SPLIT in the description's backward_flags:
-// TiledShape::f32split, a template parameter of the backward kernels).  -DD2C_F32_NATIVE_MFMA keeps the forward
-// kernels on the float instruction.
+// In the BACKWARD pass the grad-column product takes two-term operands as well (TiledShape::f32split == 2, the
+// default); the grad-weight kernel that samples again and the 1-D / fallback data kernel keep plain floats and the
+// float instruction: the relative error of 4e-6 that two-term operands leave in a long sum is fine for the output
+// and for grad_input (values of order 1 against 1e-4 relative / 1e-5 absolute) but not for gradients whose elements
+// reach 20 .. 400 and are held to the same absolute 1e-5.  A caller who prefers the speed asks for split operands
+// there too (D2C_BWD_F32_SPLIT in the description's backward_flags: f32split == 1, a template parameter of the
+// backward kernels).  The grad-weight product over sampled columns is neither: it takes every float apart into THREE
+// bfloat16 terms, which represent it exactly, and keeps float32's accuracy on the bfloat16 instruction
+// (tiled_bwd_weight_col3_kernel in d2c_tiled_bwd.hip).  -DD2C_F32_NATIVE_MFMA keeps the forward kernels and the
+// grad-column product on the float instruction.
 #ifdef D2C_F32_NATIVE_MFMA
 constexpr bool kF32SplitFwd = false;
 #else

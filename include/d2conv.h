@@ -71,12 +71,13 @@ enum {
 #define D2C_MASK_ACT_RELU    2
 #define D2C_MASK_ACT_TANH    3
 
-/* d2c_conv3d_desc::backward_flags: how the matrix-core backward pass of bfloat16 problems trades workspace for time.
+/* d2c_conv3d_desc::backward_flags: how the matrix-core backward pass trades workspace for time.
  * Both d2c_conv3d_backward_workspace_bytes() and d2c_conv3d_backward() read the field from the description they
  * are given, so the size asked for and the call agree per description.  0 = the defaults. */
 #define D2C_BWD_GW_DEFAULT   0   /* grad_weight as a matrix product over sampled columns in a buffer of their own */
 #define D2C_BWD_GW_COLUMNS   1   /* the same, said explicitly */
-#define D2C_BWD_GW_IN_PLACE  2   /* the columns written over the grad-column rows: no buffer of their own */
+#define D2C_BWD_GW_IN_PLACE  2   /* the columns written over the grad-column rows: no buffer of their own
+                                  * (bfloat16; float32 problems then sample again) */
 #define D2C_BWD_GW_RESAMPLE  3   /* no columns at all: the grad-weight kernel samples the input again */
 #define D2C_BWD_GW_MASK      3
 /* bits 8..15: number of slices over the offset groups that the backward pass runs in (0 or 1: one pass over all
@@ -87,9 +88,11 @@ enum {
  * (from which grad_input, grad_offset and grad_mask follow) carry every float operand as the sum of two bfloat16
  * values on the bfloat16 matrix instruction (a quarter of the matrix-pipe time of the float instruction; results
  * within about 4e-6 of their sums' scale instead of 1e-7, inside 1e-4 relative / 1e-5 absolute at every size
- * measured).  With this bit ALL backward matrix kernels do so -- also the grad-weight product, whose elements
- * (sums over all positions, tens to hundreds in size) then miss 1e-5 absolute -- and the 1-D and fallback kernels.
- * Off by default. */
+ * measured).  With this bit ALL backward matrix kernels do so -- also the grad-weight kernel that samples again
+ * (D2C_BWD_GW_RESAMPLE, 1-D problems, calls that want neither grad_offset nor grad_mask), whose elements (sums over
+ * all positions, tens to hundreds in size) then miss 1e-5 absolute -- and the 1-D and fallback kernels.  The
+ * grad-weight product over sampled columns is not touched by it: that one takes every float apart into three
+ * bfloat16 terms, which keeps float32's accuracy.  Off by default. */
 #define D2C_BWD_F32_SPLIT    0x10000
 
 typedef struct d2c_conv3d_desc {
@@ -446,7 +449,7 @@ int d2c_dwconv3d_backward(const d2c_dwconv3d_desc *desc, const void *grad_out, c
 void d2c_set_grad_input_mode(int mode);
 
 /* Test hooks, not for production callers (those set d2c_conv3d_desc::backward_flags, which wins over the hooks
- * wherever it says something): the grad-weight path of the matrix-core backward pass of bfloat16 problems for
+ * wherever it says something): the grad-weight path of the matrix-core backward pass for
  * descriptions whose backward_flags leave it at the default -- 1 (the library's default) lets the offset / mask
  * gradient kernel write the sampled columns, over which grad_weight then runs as a plain matrix product (the
  * reference's formulation, dconv3d_gpu.cu:1037-1088, with the column buffer filled by the kernel that has the
