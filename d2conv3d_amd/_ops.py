@@ -851,10 +851,10 @@ def set_algo_override(name):
 
 
 def set_grad_weight_mode(mode):
-    """Test hook for bfloat16 problems on the matrix-core kernels: "columns" (default; grad_weight as a matrix
-    product over the sampled columns that the offset / mask gradient kernel writes), "in_place" (the same, the
-    columns written over the grad-column rows: no buffer of their own, grad_input taken from the rows first) or
-    "resample" (the grad-weight kernel samples the input again)."""
+    """Test hook for the matrix-core kernels: "columns" (default; grad_weight as a matrix product over the sampled
+    columns that the offset / mask gradient kernel writes), "in_place" (bfloat16: the same, the columns written over
+    the grad-column rows: no buffer of their own, grad_input taken from the rows first; float32 problems sample
+    again) or "resample" (the grad-weight kernel samples the input again)."""
     _lib.load().d2c_set_grad_weight_mode(mode if isinstance(mode, int)
                                          else {"columns": 1, "in_place": 2, "resample": 0}[mode])
 
