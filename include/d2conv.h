@@ -465,6 +465,9 @@ void d2c_set_grad_weight_mode(int mode);
 void d2c_set_backward_slices(int n);
 
 const char *d2c_last_error(void);
+/* Version of this interface.  2: d2c_conv3d_desc ends in backward_flags, deform_channels and mask_activation, and the
+ * _prepared, _columns, _sized, _stats, sample / histogram entry points exist.  A binding checks it before it fills a
+ * description. */
 int d2c_version(void);
 
 #ifdef __cplusplus
