@@ -1946,6 +1946,28 @@ inline unsigned grid1d(long n, int cap = 8192)
 // Output channels of a pass rounded up so that a row of the transposed weight tile is a multiple of 128 bytes.
 int d2c_bwd_ogk(int og, int dtype) { const int rw = dtype == D2C_BF16 ? 64 : 32; return (og + rw - 1) / rw * rw; }
 
+// dst += src over the grad-column rows (16-byte vectors; bfloat16: the sum formed in float, rounded once): how the
+// passes of the grad-column product over the output channels of a wide weight group add up
+template <typename T>
+__global__ void __launch_bounds__(256) gcol_add_kernel(uint4 *dst, const uint4 *src, long n16)
+{
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (long)gridDim.x * blockDim.x) {
+        const uint4 a = dst[i], b = ld_stream16(src + i);
+        if constexpr (sizeof(T) == 2) {
+            VecAcc<bf16_t> va;
+            va.zero();
+            va.fma(1.f, a);
+            va.fma(1.f, b);
+            dst[i] = va.pack();
+        } else {
+            dst[i] = make_uint4(__float_as_uint(__uint_as_float(a.x) + __uint_as_float(b.x)),
+                                __float_as_uint(__uint_as_float(a.y) + __uint_as_float(b.y)),
+                                __float_as_uint(__uint_as_float(a.z) + __uint_as_float(b.z)),
+                                __float_as_uint(__uint_as_float(a.w) + __uint_as_float(b.w)));
+        }
+    }
+}
+
 // Output channels one pass of the data kernel reduces over: 32 k-groups of the
 // stationary operand fit the register file (512 bf16 / 256 float channels).
 int d2c_bwd_pass_channels(int dtype) { return 32 * (dtype == D2C_BF16 ? 16 : 8); }
@@ -1978,8 +2000,11 @@ template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
                               void *gmask, float *auxacc, hipStream_t st, int phase, int g_lo, int g_n,
-                              bool weights_packed)
+                              bool weights_packed, void *gcol2)
 {
+    // gcol2: a second buffer the size of `gcolbuf`, or NULL.  With it, weight groups wider than one pass get their
+    // grad-column rows from the product-only kernels too: the first pass writes `gcolbuf`, every later one `gcol2`,
+    // which gcol_add_kernel adds to the rows.
     // phase: 1 = the weight re-layout (and the clears), 2 = the kernel, 3 = both.  g_n > 0 (grad-column product on
     // tiled_bwd_col32_kernel only, see d2c_bwd_sliceable): the rows of the offset groups [g_lo, g_lo + g_n) only,
     // `gcolbuf` pointing where chunk 0 would start.
@@ -1996,7 +2021,8 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         if (ncu <= 0) return D2C_ERR_LAUNCH;
         // (the 256-position kernel of bfloat16 problems walks half-steps; reloading its stationary operand costs
         // about two of them)
-        const bool c32 = s.og <= omax && bwd_col32_ok(d2c_bwd_ogk(s.og, Elem<T>::DT), s.og, Elem<T>::DT);
+        const int og1 = s.og < omax ? s.og : omax;     // (the first pass; sized for it)
+        const bool c32 = (s.og <= omax || gcol2) && bwd_col32_ok(d2c_bwd_ogk(og1, Elem<T>::DT), og1, Elem<T>::DT);
         const int MT = c32 ? kCol32MT : 32 * (8 / (BKC / 32));
         const long items = (long)((s.M + MT - 1) / MT) * s.groups;
         const int S = (sliced ? g_n * (s.cpg / BKC) : s.nchunk) * s.K * (c32 ? 2 : 1), reload = c32 ? 2 : 1;
@@ -2029,7 +2055,8 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
         // two-term bfloat16 operands for this pass (float problems): wherever the description asks for them, and for
         // the grad-column product on its own by default (f32split == 2)
-        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && s.og <= omax && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
+        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && (s.og <= omax || gcol2) &&
+                              bwd_col_lds<T>(ogk, false) <= 160 * 1024;
         const bool split_pass = sizeof(T) == 4 && (s.f32split == 1 || (s.f32split == 2 && col_only));
         // (weights_packed: `wt` already holds them, from an earlier call on the same weights)
         if ((phase & 1) && !weights_packed) {
@@ -2050,7 +2077,8 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
         if (!(phase & 2)) continue;
         const int cpc2 = 2 * (s.cpg / BKC);
-        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0,
+        const bool later_rows = col_only && o0 > 0;    // (a later pass of the product-only kernels: rows to be added)
+        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, later_rows ? gcol2 : gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0,
                       auxoff, auxmask, sliced ? g_lo * cpc2 * s.K : 0, sliced ? (g_lo + g_n) * cpc2 * s.K : 0};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
@@ -2071,6 +2099,13 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
             else rc = launch_bwd_data<T, 32>(a, nsplit, st, split_pass);
         }
         if (rc) return rc;
+        if (later_rows) {
+            D2cProfScope prof(D2C_PROF_PACK, st);
+            const long n16 = (long)(s.Cin / BKC) * s.K * s.M * BKC * (long)sizeof(T) / 16;
+            hipLaunchKernelGGL(gcol_add_kernel<T>, dim3(grid1d(n16, 16384)), dim3(256), 0, st, (uint4 *)gcolbuf,
+                               (const uint4 *)gcol2, n16);
+            if (int rc2 = d2c_check_launch("gcol_add_kernel")) return rc2;
+        }
     }
     if (auxoff && (phase & 2)) {
         D2cProfScope prof(D2C_PROF_PACK, st);
@@ -2346,7 +2381,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
 #define INST(T)                                                                                                    \
     template int d2c_tiled_bwd_data_launch<T>(const TiledShape &, const void *, const void *, const void *,        \
                                               const void *, const void *, void *, float *, void *, void *, void *, \
-                                              float *, hipStream_t, int, int, int, bool);                                   \
+                                              float *, hipStream_t, int, int, int, bool, void *);                                   \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
                                                 const void *, void *, float *, void *, const void *, long, hipStream_t, \
                                                 int, int, int);                                                     \

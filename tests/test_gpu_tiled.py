@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import d2conv3d_amd as d2c
-from d2conv3d_amd import _ops
+from d2conv3d_amd import _lib, _ops
 from oracle import cpu
 from _util import assert_close, rel_l2
 
@@ -171,6 +171,40 @@ def test_float32_grad_weight_from_columns_matches_resampling(name, dev):
         _ops.set_grad_weight_mode("columns")
         _ops.config.set_keep_columns(before["on"], before["max_bytes"])
     assert rel_l2(got["columns"], got["resample"].cpu()) < 2e-6
+
+
+@pytest.mark.parametrize("name,dtype", [("c64_o600", torch.bfloat16), ("c64_o1100_big", torch.bfloat16),
+                                        ("c64_o320_nomask", torch.float32), ("c64_o600", torch.float32)])
+def test_wide_weight_groups_stay_on_the_list_based_backward(name, dtype, dev):
+    # Weight groups wider than one pass of the grad-column product (512 bfloat16 / 256 float32 output channels): the
+    # passes' rows are added up and the backward pass stays on the product-only kernel, the offset / mask gradient
+    # kernel and the owner kernel (the fused kernel with its atomic scatter per pass is an order of magnitude slower
+    # at layer sizes).  Which kernels ran is read from the library's own instrumentation; the values against the oracle.
+    import ctypes
+    lib = _lib.load()
+    (x, off, m, w, b), gout, (s, p, d, groups, G) = make(name, dtype, seed=21)
+    eg = cpu.conv3d_backward(f32(gout), f32(x), off, m, f32(w), b is not None, s, p, d, groups, G)
+    ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+    out = d2c.deform_conv3d(*ts, s, p, d, groups, G)
+    lib.d2c_profile_reset()
+    lib.d2c_profile_enable(1)
+    try:
+        out.backward(gout.to(dev))
+        torch.cuda.synchronize()
+    finally:
+        lib.d2c_profile_enable(0)
+    ran = {}
+    for kid in (_lib.PROF_BWD_DATA, _lib.PROF_GX_OWNER, _lib.PROF_BWD_AUX):
+        tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
+        lib.d2c_profile_read(kid, ctypes.byref(tot), ctypes.byref(cnt))
+        ran[kid] = (cnt.value, lib.d2c_profile_kernel_name(kid).decode())
+    lib.d2c_profile_reset()
+    assert ran[_lib.PROF_BWD_DATA][0] >= 2 and ran[_lib.PROF_BWD_DATA][1] in ("tiled_bwd_col32_kernel", "tiled_bwd_col_kernel"), ran
+    assert ran[_lib.PROF_GX_OWNER][0] >= 1 and ran[_lib.PROF_BWD_AUX][0] >= 1, ran
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-5
+    for n, t, e in zip(("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias"), ts, eg):
+        if t is not None:
+            assert rel_l2(t.grad, e) < tol, (name, n, rel_l2(t.grad, e))
 
 
 @pytest.mark.parametrize("name", ["c256_G2_o512_tail", "c256_G4_o128", "c384_G6_o384_nomask", "c384_G3_o384"])
