@@ -40,6 +40,10 @@ WORKLOADS = {
                     seed=1002, backward=True, bound="mfma"),
     "c3": dict(nd=3, N=2, C=512, dims=(8, 30, 54), groups=1, G=8, dt="bf16", off=("normal", 2.0), seed=1003,
                backward=True, bound="mfma"),
+    # the headline shape in float32 (the reference's default precision): weight groups of 512 output channels, two
+    # passes of the float32 grad-column product
+    "c3_f32": dict(nd=3, N=2, C=512, dims=(8, 30, 54), groups=1, G=8, dt="f32", off=("normal", 2.0), seed=1003,
+                   backward=True, bound="mfma"),
     "c4": dict(nd=3, N=2, C=1024, dims=(8, 15, 27), groups=1024, G=1, dt="f32", off=("normal", 1.5), seed=1004,
                backward=True, bound="hbm"),
     "c5a": dict(nd=1, N=4, C=512, dims=(64,), groups=1, G=1, dt="f32", off=("normal", 1.5), seed=1005,
@@ -50,7 +54,7 @@ WORKLOADS = {
 PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 PEAK_GBS = 8000.0
 # largest sample the CPU leg runs (the oracle does ~0.09 TFLOP/s on 16 cores): N and leading dim cut down to this
-CPU_CROP = {"c3": (1, (8, 30, 54)), "c5b": (1, (8, 60, 108))}
+CPU_CROP = {"c3": (1, (8, 30, 54)), "c3_f32": (1, (8, 30, 54)), "c5b": (1, (8, 60, 108))}
 
 
 def make_inputs(name, torch, crop=None, want_size=False):

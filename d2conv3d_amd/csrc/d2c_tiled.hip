@@ -24,7 +24,7 @@ template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
                               void *gmask, float *auxacc, hipStream_t st, int phase = 3, int g_lo = 0, int g_n = 0,
-                              bool weights_packed = false, void *gcol2 = nullptr);
+                              bool weights_packed = false);
 bool d2c_bwd_sliceable(const TiledShape &s, int dtype);
 int d2c_backward_slices();
 int d2c_bwd_data_split(const TiledShape &s, int dtype);
@@ -535,8 +535,8 @@ bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 // grad_offset / grad_mask by the kernel of d2c_aux_grad.hip (from the grad-column rows).  (Weight groups wider than
-// one pass of the grad-column product get whole rows too: the passes over their output channels are added up in a
-// second row buffer, see d2c_tiled_bwd_data_launch.
+// one pass of the grad-column product get whole rows too: the later passes over their output channels add to the
+// rows, see d2c_tiled_bwd_data_launch.
 // That needs the product-only kernels, i.e. grad_input from sample lists: where grad_input is scattered with
 // atomics by the fused kernel, wide weight groups keep the fused kernel's passes.)
 bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
@@ -591,7 +591,7 @@ BwdSlices bwd_slices(const d2c_conv3d_desc &q, const TiledShape &s)
 }
 
 struct BwdWs {
-    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, gcol2, counts, entries, ovf, gsacc, sm1, col, total;
+    size_t xcl, wt, gxcl, gwacc, goutp, auxacc, gcol, counts, entries, ovf, gsacc, sm1, col, total;
 };
 // `saved_columns`: the caller brings the sampled columns of the forward call (no column region, no slices)
 BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s, bool saved_columns = false)
@@ -611,7 +611,7 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s, bool saved_columns =
     w.total = w.auxacc;
     if (d2c_bwd_data_split(s, q.dtype) > 1 || !d2c_tiled_bwd_single_pass(s, q.dtype))
         w.total += d2c_align_up((size_t)s.N * s.G * s.K * s.P * (s.nd + 1) * sizeof(float));
-    w.gcol = w.gcol2 = w.counts = w.entries = w.ovf = 0;
+    w.gcol = w.counts = w.entries = w.ovf = 0;
     const BwdSlices sl = saved_columns ? BwdSlices{0, 0} : bwd_slices(q, s);
     if (use_lists(q, s) || use_aux_kernel(q, s)) {
         w.gcol = w.total;
@@ -619,9 +619,6 @@ BwdWs bwd_ws(const d2c_conv3d_desc &q, const TiledShape &s, bool saved_columns =
         // the rows' place)
         const size_t chunks = sl.gs ? (size_t)sl.gs * (s.cpg / bkc_of(q.dtype)) : (size_t)(s.Cin / bkc_of(q.dtype));
         w.total = w.gcol + d2c_align_up((chunks * s.K * s.M + 64) * bkc_of(q.dtype) * es);
-        // ... and the rows of the later passes over the output channels of a weight group wider than one pass
-        w.gcol2 = w.total;
-        if (!d2c_tiled_bwd_single_pass(s, q.dtype)) w.total += d2c_align_up(chunks * s.K * s.M * bkc_of(q.dtype) * es);
     }
     if (use_lists(q, s)) {
         size_t c, en, ov;
@@ -792,8 +789,7 @@ int backward_t(const d2c_conv3d_desc &q, const void *gout, const void *x, const 
             if (int rc = d2c_tiled_bwd_data_launch<T>(s, gout, xcl_p, off, mask, w, wt_p,
                                                      lists ? nullptr : gxcl, (lists || auxk) ? base + l.gcol : nullptr,
                                                      auxk ? nullptr : goff, auxk ? nullptr : gmask,
-                                                     (float *)(base + l.auxacc), st, 3, 0, 0, wt_packed,
-                                                     d2c_tiled_bwd_single_pass(s, q.dtype) ? nullptr : base + l.gcol2))
+                                                     (float *)(base + l.auxacc), st, 3, 0, 0, wt_packed))
                 return rc;
             if (lists && gw_in_place)
                 if (int rc = d2c_gx_owner_launch<T>(s, base + l.gcol, L, gxcl, st)) return rc;

@@ -645,7 +645,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
             *reinterpret_cast<float *>(s_gcol + pl * GRS + ch * 4) = acc[r];
         }
         lds_only_barrier();
-        // rows out to memory, 16 bytes per thread
+        // rows out to memory, 16 bytes per thread.  A later pass over the output channels of a wide weight group
+        // (a.add_aux) adds to the rows the passes before it left: the sum formed in float, bfloat16 rounded once more
         T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
 #pragma unroll
         for (int i = 0; i < ITEMS; i++) {
@@ -654,14 +655,20 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
             const int m = m0 + pos;
             if (m < s.M) {
                 const float *gp = reinterpret_cast<const float *>(s_gcol + pos * GRS + vec * VEC * 4);
+                uint4 *dst = reinterpret_cast<uint4 *>(gb + (long)m * BKC + vec * VEC);
+                VecAcc<T> va;
+#pragma unroll
+                for (int e = 0; e < VEC; e++) va.a[e] = gp[e];
+                if (a.add_aux) va.fma(1.f, *dst);
                 uint4 o;
                 if constexpr (sizeof(T) == 2) {
-                    o = make_uint4(pack_bf16x2(gp[0], gp[1]), pack_bf16x2(gp[2], gp[3]), pack_bf16x2(gp[4], gp[5]),
-                                   pack_bf16x2(gp[6], gp[7]));
+                    o = make_uint4(pack_bf16x2(va.a[0], va.a[1]), pack_bf16x2(va.a[2], va.a[3]),
+                                   pack_bf16x2(va.a[4], va.a[5]), pack_bf16x2(va.a[6], va.a[7]));
                 } else {
-                    o = *reinterpret_cast<const uint4 *>(gp);
+                    o = make_uint4(__float_as_uint(va.a[0]), __float_as_uint(va.a[1]), __float_as_uint(va.a[2]),
+                                   __float_as_uint(va.a[3]));
                 }
-                *reinterpret_cast<uint4 *>(gb + (long)m * BKC + vec * VEC) = o;
+                *dst = o;
             }
         }
     }
@@ -1946,28 +1953,6 @@ inline unsigned grid1d(long n, int cap = 8192)
 // Output channels of a pass rounded up so that a row of the transposed weight tile is a multiple of 128 bytes.
 int d2c_bwd_ogk(int og, int dtype) { const int rw = dtype == D2C_BF16 ? 64 : 32; return (og + rw - 1) / rw * rw; }
 
-// dst += src over the grad-column rows (16-byte vectors; bfloat16: the sum formed in float, rounded once): how the
-// passes of the grad-column product over the output channels of a wide weight group add up
-template <typename T>
-__global__ void __launch_bounds__(256) gcol_add_kernel(uint4 *dst, const uint4 *src, long n16)
-{
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (long)gridDim.x * blockDim.x) {
-        const uint4 a = dst[i], b = ld_stream16(src + i);
-        if constexpr (sizeof(T) == 2) {
-            VecAcc<bf16_t> va;
-            va.zero();
-            va.fma(1.f, a);
-            va.fma(1.f, b);
-            dst[i] = va.pack();
-        } else {
-            dst[i] = make_uint4(__float_as_uint(__uint_as_float(a.x) + __uint_as_float(b.x)),
-                                __float_as_uint(__uint_as_float(a.y) + __uint_as_float(b.y)),
-                                __float_as_uint(__uint_as_float(a.z) + __uint_as_float(b.z)),
-                                __float_as_uint(__uint_as_float(a.w) + __uint_as_float(b.w)));
-        }
-    }
-}
-
 // Output channels one pass of the data kernel reduces over: 32 k-groups of the
 // stationary operand fit the register file (512 bf16 / 256 float channels).
 int d2c_bwd_pass_channels(int dtype) { return 32 * (dtype == D2C_BF16 ? 16 : 8); }
@@ -2000,11 +1985,10 @@ template <typename T>
 int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void *xcl, const void *off,
                               const void *mask, const void *w, void *wt, float *gxcl, void *gcolbuf, void *goff,
                               void *gmask, float *auxacc, hipStream_t st, int phase, int g_lo, int g_n,
-                              bool weights_packed, void *gcol2)
+                              bool weights_packed)
 {
-    // gcol2: a second buffer the size of `gcolbuf`, or NULL.  With it, weight groups wider than one pass get their
-    // grad-column rows from the product-only kernels too: the first pass writes `gcolbuf`, every later one `gcol2`,
-    // which gcol_add_kernel adds to the rows.
+    // Weight groups wider than one pass get their grad-column rows from the product-only kernels too: the first pass
+    // writes the rows, every later one (on tiled_bwd_col_kernel, which can) adds to them.
     // phase: 1 = the weight re-layout (and the clears), 2 = the kernel, 3 = both.  g_n > 0 (grad-column product on
     // tiled_bwd_col32_kernel only, see d2c_bwd_sliceable): the rows of the offset groups [g_lo, g_lo + g_n) only,
     // `gcolbuf` pointing where chunk 0 would start.
@@ -2022,7 +2006,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         // (the 256-position kernel of bfloat16 problems walks half-steps; reloading its stationary operand costs
         // about two of them)
         const int og1 = s.og < omax ? s.og : omax;     // (the first pass; sized for it)
-        const bool c32 = (s.og <= omax || gcol2) && bwd_col32_ok(d2c_bwd_ogk(og1, Elem<T>::DT), og1, Elem<T>::DT);
+        const bool c32 = bwd_col32_ok(d2c_bwd_ogk(og1, Elem<T>::DT), og1, Elem<T>::DT);
         const int MT = c32 ? kCol32MT : 32 * (8 / (BKC / 32));
         const long items = (long)((s.M + MT - 1) / MT) * s.groups;
         const int S = (sliced ? g_n * (s.cpg / BKC) : s.nchunk) * s.K * (c32 ? 2 : 1), reload = c32 ? 2 : 1;
@@ -2055,8 +2039,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
         // two-term bfloat16 operands for this pass (float problems): wherever the description asks for them, and for
         // the grad-column product on its own by default (f32split == 2)
-        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && (s.og <= omax || gcol2) &&
-                              bwd_col_lds<T>(ogk, false) <= 160 * 1024;
+        const bool col_only = gcolbuf && !gxcl && !goff && !gmask && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
         const bool split_pass = sizeof(T) == 4 && (s.f32split == 1 || (s.f32split == 2 && col_only));
         // (weights_packed: `wt` already holds them, from an earlier call on the same weights)
         if ((phase & 1) && !weights_packed) {
@@ -2077,12 +2060,11 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         if (int rc = d2c_check_launch("pack_weight_bwd_kernel")) return rc;
         if (!(phase & 2)) continue;
         const int cpc2 = 2 * (s.cpg / BKC);
-        const bool later_rows = col_only && o0 > 0;    // (a later pass of the product-only kernels: rows to be added)
-        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, later_rows ? gcol2 : gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0,
+        BwdDataArgs a{s, gout, xcl, off, mask, wt, gxcl, gcolbuf, goff, gmask, ogk, o0, ogn, o0 > 0 ? 1 : 0,
                       auxoff, auxmask, sliced ? g_lo * cpc2 * s.K : 0, sliced ? (g_lo + g_n) * cpc2 * s.K : 0};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
-        if (col_only && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
+        if (col_only && o0 == 0 && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
             rc = launch_bwd_col32(a, nsplit, st);
         } else if (sliced) {
             d2c_set_error("grad-column product: slices are made by tiled_bwd_col32_kernel only");
@@ -2099,13 +2081,6 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
             else rc = launch_bwd_data<T, 32>(a, nsplit, st, split_pass);
         }
         if (rc) return rc;
-        if (later_rows) {
-            D2cProfScope prof(D2C_PROF_PACK, st);
-            const long n16 = (long)(s.Cin / BKC) * s.K * s.M * BKC * (long)sizeof(T) / 16;
-            hipLaunchKernelGGL(gcol_add_kernel<T>, dim3(grid1d(n16, 16384)), dim3(256), 0, st, (uint4 *)gcolbuf,
-                               (const uint4 *)gcol2, n16);
-            if (int rc2 = d2c_check_launch("gcol_add_kernel")) return rc2;
-        }
     }
     if (auxoff && (phase & 2)) {
         D2cProfScope prof(D2C_PROF_PACK, st);
@@ -2381,7 +2356,7 @@ int d2c_tiled_bias_grad(const TiledShape &s, const void *gout, void *gb, hipStre
 #define INST(T)                                                                                                    \
     template int d2c_tiled_bwd_data_launch<T>(const TiledShape &, const void *, const void *, const void *,        \
                                               const void *, const void *, void *, float *, void *, void *, void *, \
-                                              float *, hipStream_t, int, int, int, bool, void *);                                   \
+                                              float *, hipStream_t, int, int, int, bool);                                   \
     template int d2c_tiled_bwd_weight_launch<T>(const TiledShape &, const void *, const void *, const void *,      \
                                                 const void *, void *, float *, void *, const void *, long, hipStream_t, \
                                                 int, int, int);                                                     \
