@@ -131,7 +131,7 @@ typedef struct d2c_conv3d_desc {
      * that belong to neither are not written).  mask_activation != D2C_MASK_ACT_NONE makes the sampler apply that
      * function to every mask value it reads (rounded to aux_dtype, like the tensor the reference's activation
      * writes), and grad_mask comes back with respect to the raw values.  0 / 0: tensors of their own, mask used as it is.
-     * Matrix-core kernels only (and, in the backward call, one pass over the output channels of a weight group):
+     * Matrix-core kernels only (and, in the backward call, offset groups that lie inside one weight group):
      * other descriptions answer D2C_ERR_UNSUPPORTED. */
     int32_t deform_channels;
     int32_t mask_activation;
