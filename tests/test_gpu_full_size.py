@@ -68,7 +68,7 @@ def literal_gate_excess(actual, exact):
     return ((a - e).abs() / (1e-5 + 1e-4 * e.abs())).max().item()
 
 
-@pytest.mark.parametrize("name", ["c1", "c5a", "c4", "c2_f32", "c2_bf16", "c3"])
+@pytest.mark.parametrize("name", ["c1", "c5a", "c4", "c2_f32", "c2_bf16", "c3", "c3_f32"])
 def test_full_size_against_oracle(name, dev):
     c, x, off, m, w, b, gout = _tensors(name)
     f = lambda t: t.float()
