@@ -818,16 +818,22 @@ def conv3d_offset_histogram(offset, kernel_size, offset_groups=1, bins=64, lo=-8
 
 
 def conv3d_algo(input, offset, alpha, weight, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
-                groups=1, offset_groups=1, offset_axes=7):
+                groups=1, offset_groups=1, offset_axes=7, as_dtype=None):
     """Name of the kernel family ("generic", "mfma", "depthwise") these arguments are served by; "invalid" when
-    none takes them (a partial `offset_axes` on a shape the matrix-core kernels do not serve in both directions)."""
+    none takes them (a partial `offset_axes` on a shape the matrix-core kernels do not serve in both directions).
+    `as_dtype`: answer for tensors of this element type instead of the ones given (no tensor is converted)."""
     lib = _lib.load()
-    input, offset, alpha, weight, _ = _unify(input, offset, alpha, weight, None)
+    dt = input.dtype if as_dtype is None else as_dtype
+    if dt not in _DT:
+        raise RuntimeError(f"deform_conv: unsupported input dtype {dt}")
+    adt = dt
+    if dt == torch.bfloat16 and not (offset.dtype == torch.bfloat16 and (alpha is None or alpha.dtype == torch.bfloat16)):
+        adt = torch.float32
     N, Cin, D, H, W = input.shape
     Cout, _, kd, kh, kw = weight.shape
     Do, Ho, Wo = offset.shape[2:]
     desc = _lib.Conv3dDesc(N, Cin, Cout, D, H, W, kd, kh, kw, *stride, *padding, *dilation,
-                           groups, offset_groups, Do, Ho, Wo, _DT[input.dtype], _DT[offset.dtype],
+                           groups, offset_groups, Do, Ho, Wo, _DT[dt], _DT[adt],
                            _lib.EPILOGUE_NONE, 1.0, int(offset_axes))
     return _lib.ALGO_NAMES.get(lib.d2c_conv3d_algo(ctypes.byref(desc)), "invalid")
 
