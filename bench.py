@@ -2,7 +2,8 @@
 """Benchmark of the D2Conv3D operator path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload c3|c1|c2_f32|c2_bf16|c4|c5a|c5b|c2_sizemap|dwconv|c3_norm|c3_layer]
+                    [--workload c3|c1|c2_f32|c2_bf16|c3_f32|c4|c5a|c5b|c2_sizemap|dwconv|c3_norm|c3_layer]
+                    [--shape N,Cin,Cout,T,H,W,kd,kh,kw,G,dtype[,groups]]
 
 One step = one forward (+ one backward with all five gradients, except for
 the forward-only workload c1) of the modulated deformable convolution through
@@ -356,6 +357,60 @@ def bench_layer(args):
     print(json.dumps(line))
 
 
+def bench_shape(args):
+    """`--shape N,Cin,Cout,T,H,W,kd,kh,kw,G,dtype[,groups]`: modulated deformable conv3d of any size (stride 1,
+    "same" padding, offsets ~N(0,1.5), sigmoid mask, bias) through d2conv3d_amd.deform_conv3d, forward and backward timed
+    apart with HIP events.  For the layer shapes of the reference's own networks, e.g. the refinement blocks of
+    network/segmentation/encoder_decoder.py:112-131 (`--shape 1,1024,256,8,30,54,3,3,3,1,bf16`) or its global-convolution
+    bridge (network/modules/bridging.py:14-22: `--shape 1,2048,256,8,30,54,1,7,1,1,bf16`)."""
+    import torch
+    import d2conv3d_amd as d2c
+    from d2conv3d_amd import _ops
+    f = args.shape.split(",")
+    N, Cin, Cout, T, H, W, kd, kh, kw, G = (int(v) for v in f[:10])
+    dtype = {"bf16": torch.bfloat16, "f32": torch.float32}[f[10]]
+    groups = int(f[11]) if len(f) > 11 else 1
+    dev = torch.device("cuda:0")
+    dims, ks, pad, K = (T, H, W), (kd, kh, kw), (kd // 2, kh // 2, kw // 2), kd * kh * kw
+    g = torch.Generator().manual_seed(4242)
+    bound = 1.0 / (Cin // groups * K) ** 0.5
+    x = torch.randn(N, Cin, *dims, generator=g).to(dtype).to(dev).requires_grad_(True)
+    w = ((torch.rand(Cout, Cin // groups, *ks, generator=g) * 2 - 1) * bound).to(dtype).to(dev).requires_grad_(True)
+    b = ((torch.rand(Cout, generator=g) * 2 - 1) * bound).to(dtype).to(dev).requires_grad_(True)
+    off = (torch.randn(N, 3 * K * G, *dims, generator=g) * 1.5).to(dev).requires_grad_(True)
+    m = torch.sigmoid(torch.randn(N, K * G, *dims, generator=g)).to(dev).requires_grad_(True)
+    gout = torch.randn(N, Cout, *dims, generator=g).to(dtype).to(dev)
+    algo = _ops.conv3d_algo(x, off, m, w, (1, 1, 1), pad, (1, 1, 1), groups, G)
+    if algo == "generic" and dtype == torch.bfloat16 and \
+            _ops.conv3d_algo(x, off, m, w, (1, 1, 1), pad, (1, 1, 1), groups, G, as_dtype=torch.float32) == "mfma":
+        algo = "mfma, in float32 and rounded (channel counts the bfloat16 kernels cannot chunk)"
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    t_f = t_b = 0.0
+    for it in range(args.warmup + args.steps):
+        for t in (x, w, b, off, m):
+            t.grad = None
+        ev[0].record()
+        out = d2c.deform_conv3d(x, off, m, w, b, 1, pad, 1, groups, G)
+        ev[1].record()
+        out.backward(gout)
+        ev[2].record()
+        torch.cuda.synchronize()
+        if it >= args.warmup:
+            t_f += ev[0].elapsed_time(ev[1]) / args.steps
+            t_b += ev[1].elapsed_time(ev[2]) / args.steps
+    flop = 2.0 * N * T * H * W * Cout * (Cin // groups) * K
+    print(json.dumps({
+        "metric": "modulated deformable conv3d fwd+bwd effective TFLOP/s (--shape) on 1 GPU",
+        "value": round(3 * flop / ((t_f + t_b) * 1e-3) / 1e12, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(t_f + t_b, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": f[10], "data": "synthetic",
+        "config": {"workload": f"--shape {args.shape}: N={N}, {Cin}->{Cout} channels, {T}x{H}x{W}, kernel {kd}x{kh}x{kw}, "
+                               f"{G} offset group(s), {groups} weight group(s), through d2conv3d_amd.deform_conv3d",
+                   "kernel_family": algo, "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
+                   "forward_tflops": round(flop / (t_f * 1e-3) / 1e12, 1),
+                   "backward_tflops": round(2 * flop / (t_b * 1e-3) / 1e12, 1)}}))
+
+
 def bench_dwconv(args):
     """Plain depthwise conv3d (the reference's fast-depthwise-conv3d operator; backbone shape: 256 channels,
     8x56x56, 3x3x3, stride 1, padding 1, float32), forward + backward through the C ABI with pre-allocated
@@ -450,6 +505,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2_sizemap", "dwconv", "c3_norm", "c3_layer"])
+    ap.add_argument("--shape", default=None,
+                    help="instead of a named workload: N,Cin,Cout,T,H,W,kd,kh,kw,G,dtype[,groups] (dtype bf16 | f32), "
+                         "timed through the Python layer (see bench_shape)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--offset-axes", type=int, default=7,
                     help="mask of the axes the offsets displace along (1 z, 2 y, 4 x): 6 = the Spatial layers, 1 = the "
@@ -492,6 +550,8 @@ def main():
     lib.d2c_set_grad_input_mode(args.grad_input_mode)
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    if args.shape:
+        return bench_shape(args)
     if args.workload == "c2_sizemap":
         return bench_size_map(args)
     if args.workload == "dwconv":
