@@ -78,3 +78,41 @@ def test_unchunked_bfloat16_with_the_size_map_in_the_operator(dev):
     assert res[0][0].dtype == torch.bfloat16 and res[0][1].dtype == torch.bfloat16
     for i, (a, e) in enumerate(zip(*res)):
         assert rel_l2(a, e) < 4e-3, (i, rel_l2(a, e))
+
+
+@pytest.mark.parametrize("dtype,cin", [(torch.float32, 48), (torch.bfloat16, 40), (torch.float32, 80)])
+def test_channel_counts_off_the_chunking_are_padded_with_zero_channels(dtype, cin, dev):
+    """One weight group, one offset group, a channel count that is no multiple of the chunk but fills at least half
+    of its last one: input and weight get zero channels up to the next chunk and the matrix-core kernels run; results
+    and gradients (of the original shapes) against the oracle."""
+    N, Cout, dims = 1, 40, (3, 8, 9)
+    g = torch.Generator().manual_seed(8300 + cin)
+    x = torch.randn(N, cin, *dims, generator=g).to(dtype)
+    w = ((torch.rand(Cout, cin, 3, 3, 3, generator=g) * 2 - 1) / (cin * 27) ** 0.5).to(dtype)
+    b = ((torch.rand(Cout, generator=g) * 2 - 1) * 0.1).to(dtype)
+    off = torch.randn(N, 81, *dims, generator=g) * 1.5
+    m = torch.sigmoid(torch.randn(N, 27, *dims, generator=g))
+    gout = torch.randn(N, Cout, *dims, generator=g).to(dtype)
+    f = lambda t: t.float()
+    e_out = cpu.conv3d_forward(f(x), off, m, f(w), f(b), 1, 1, 1, 1, 1)
+    eg = cpu.conv3d_backward(f(gout), f(x), off, m, f(w), True, 1, 1, 1, 1, 1)
+    ts = [t.to(dev).requires_grad_(True) for t in (x, off, m, w, b)]
+    lib = _lib.load()
+    lib.d2c_profile_reset()
+    lib.d2c_profile_enable(1)
+    try:
+        out = d2c.deform_conv3d(*ts, 1, 1, 1, 1, 1)
+        out.backward(gout.to(dev))
+        torch.cuda.synchronize()
+    finally:
+        lib.d2c_profile_enable(0)
+    tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
+    lib.d2c_profile_read(_lib.PROF_FWD, ctypes.byref(tot), ctypes.byref(cnt))
+    kernel = lib.d2c_profile_kernel_name(_lib.PROF_FWD).decode()
+    lib.d2c_profile_reset()
+    assert cnt.value >= 1 and kernel.startswith("tiled_fwd"), (cnt.value, kernel)
+    assert out.dtype == dtype and ts[0].grad.shape == x.shape and ts[3].grad.shape == w.shape
+    tol = 1e-2 if dtype == torch.bfloat16 else 2e-5
+    assert rel_l2(out, e_out) < tol
+    for n, t, e in zip(("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias"), ts, eg):
+        assert rel_l2(t.grad, e) < tol, (dtype, cin, n, rel_l2(t.grad, e))
