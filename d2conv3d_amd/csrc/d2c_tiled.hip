@@ -531,7 +531,8 @@ int forward_t(const d2c_conv3d_desc &q, const void *x, const void *off, const vo
 // channels of a weight group (in one pass of the product-only kernels, or in several whose rows are added up).
 bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
 {
-    return d2c_gx_mode() >= 1 && d2c_lists_supported(s) && d2c_tiled_bwd_data_supported(s, q.dtype);
+    return d2c_gx_mode() >= 1 && d2c_lists_supported(s) && d2c_tiled_bwd_data_supported(s, q.dtype) &&
+           (s.nd == 3 || d2c_tiled_bwd_single_pass(s, q.dtype));
 }
 
 // grad_offset / grad_mask by the kernel of d2c_aux_grad.hip (from the grad-column rows).  (Weight groups wider than
@@ -542,7 +543,9 @@ bool use_lists(const d2c_conv3d_desc &q, const TiledShape &s)
 bool use_aux_kernel(const d2c_conv3d_desc &q, const TiledShape &s)
 {
     if (!d2c_tiled_bwd_data_supported(s, q.dtype)) return false;
-    return d2c_tiled_bwd_single_pass(s, q.dtype) || (d2c_gx_mode() >= 1 && d2c_lists_supported(s));
+    // (1-D problems with wide weight groups keep the fused kernel: their float32 gradients are held to the literal
+    // gate, which the two-term operands of the product-only kernel miss there)
+    return d2c_tiled_bwd_single_pass(s, q.dtype) || (s.nd == 3 && d2c_gx_mode() >= 1 && d2c_lists_supported(s));
 }
 
 // grad_weight as a matrix product over sampled columns that the offset / mask gradient kernel writes on its way
