@@ -204,3 +204,43 @@ def test_full_size_linearity_and_adjoints(name, dev):
     assert abs(lhs - via_w) < atol, (lhs, via_w)
     e_gb = go.double().sum(dim=[0] + list(range(2, go.dim())))
     assert rel_l2(gb, e_gb) < (1e-2 if c["dt"] == "bf16" else 1e-5)
+
+
+# Layer shapes of the reference's own networks on an 8-frame 480x854 clip at stride 16 (refinement block of
+# network/segmentation/encoder_decoder.py:129, global-convolution bridge of network/modules/bridging.py:14-22, a
+# deformable convolution without modulation, network/layers.py:103-105): (Cin, Cout, kernel, modulation, dtype)
+NETWORK_LAYERS = {
+    "refine_1024_256_bf16": (1024, 256, (3, 3, 3), True, torch.bfloat16),
+    "bridge_2048_256_1x7x1_bf16": (2048, 256, (1, 7, 1), True, torch.bfloat16),
+    "dconv_256_256_f32": (256, 256, (3, 3, 3), False, torch.float32),
+}
+
+
+@pytest.mark.parametrize("name", list(NETWORK_LAYERS))
+def test_network_layer_shapes_against_oracle(name, dev):
+    cin, cout, ks, modulated, dtype = NETWORK_LAYERS[name]
+    dims, K = (8, 30, 54), ks[0] * ks[1] * ks[2]
+    pad = tuple(k // 2 for k in ks)
+    g = torch.Generator().manual_seed(9000 + cin)
+    bound = 1.0 / (cin * K) ** 0.5
+    x = torch.randn(1, cin, *dims, generator=g).to(dtype)
+    w = ((torch.rand(cout, cin, *ks, generator=g) * 2 - 1) * bound).to(dtype)
+    b = ((torch.rand(cout, generator=g) * 2 - 1) * bound).to(dtype)
+    off = torch.randn(1, 3 * K, *dims, generator=g) * 1.5
+    m = torch.sigmoid(torch.randn(1, K, *dims, generator=g)) if modulated else None
+    gout = torch.randn(1, cout, *dims, generator=g).to(dtype)
+    f = lambda t: t.float() if t is not None else None
+    e_out = cpu.conv3d_forward(f(x), off, m, f(w), f(b), 1, pad, 1, 1, 1)
+    eg = cpu.conv3d_backward(f(gout), f(x), off, m, f(w), True, 1, pad, 1, 1, 1)
+    ts = [t.to(dev).requires_grad_(True) if t is not None else None for t in (x, off, m, w, b)]
+    out = d2c.deform_conv3d(*ts, 1, pad, 1, 1, 1)
+    out.backward(gout.to(dev))
+    pairs = [("out", out.detach(), e_out)] + [(n, t.grad, e) for n, t, e in zip(
+        ("grad_input", "grad_offset", "grad_mask", "grad_weight", "grad_bias"), ts, eg) if t is not None]
+    for n, a, e in pairs:
+        if dtype == torch.bfloat16:
+            assert rel_l2(a, e) < 2e-2, (name, n, rel_l2(a, e))
+            assert_close(a, e, 2e-2, 2e-2 * e.abs().max().item(), f"{name} {n}")
+        else:
+            # float32 against the float32 oracle: 1e-4 relative / 1e-5 absolute scaled by the tensor's magnitude
+            assert_close(a, e, 1e-4, 1e-5 * max(1.0, e.abs().max().item()), f"{name} {n}")
