@@ -295,7 +295,7 @@ def bench_conv_act_norm(args):
 
 def bench_layer(args):
     """A whole self-deforming layer at the size of workload c3: MDConv3d(512, 512, 3, padding=1, offset_groups=8) in
-    bfloat16 -- the stock Conv3d that predicts the deformation (network/layers.py:51-60; MIOpen), then the operator --
+    bfloat16 -- the Conv3d that predicts the deformation (network/layers.py:51-60), then the operator --
     forward + backward through autograd.  Timed twice on the same GPU: with the deformation tensor handed to the
     operator as it is (the sampler reads offsets and modulation inside it and applies the sigmoid; the default), and
     with the reference's split + sigmoid in front of the operator (network/layers.py:107-120)."""
@@ -336,6 +336,13 @@ def bench_layer(args):
         res[fused] = timed()
         outs[fused] = layer(x).detach().float()
     err = float((outs[True] - outs[False]).norm() / outs[False].norm())
+    # ... and with the branch's convolution on the vendor library (what the reference runs) instead of on the operator
+    # at zero offsets (modules._branch_conv, the default)
+    layer.branch_on_operator = False
+    stock_branch_ms = timed()
+    stock_out = layer(x).detach().float()
+    layer.branch_on_operator = True
+    err_branch = float((outs[True] - stock_out).norm() / stock_out.norm())
     # the operator's GEMM-equivalent flops plus those of the deformation branch's convolution (864 output channels)
     f_op, _, _ = algorithmic("c3")
     P = c["dims"][0] * c["dims"][1] * c["dims"][2]
@@ -351,6 +358,9 @@ def bench_layer(args):
                    "deformation": "read by the operator inside the branch's output tensor, sigmoid in the sampler",
                    "split_and_sigmoid_in_front_ms_per_step": round(res[False], 4),
                    "relative_l2_fused_vs_split": err,
+                   "branch": "the layer's Conv3d 512 -> 864 evaluated by the operator at zero offsets",
+                   "branch_on_the_vendor_library_ms_per_step": round(stock_branch_ms, 4),
+                   "relative_l2_branch_on_operator_vs_vendor": err_branch,
                    "algorithmic_gflop": round(3 * (f_op + f_branch) / 1e9, 2)},
         "roofline": None,
     }

@@ -156,3 +156,51 @@ def test_tap_statistics_match_the_oracle(dev):
     assert st["partial"] == int(((ef != 0) & (ef != 255)).sum()) / n
     assert st["corners_read"] == sum(int(((ef >> c) & 1).sum()) for c in range(8)) / (8.0 * n)
     assert 0.05 < st["dead"] < 0.6 and st["partial"] > 0.05     # the case does leave the volume
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("cls", ["MDConv3d", "DConv3d", "XYZSizeConditionedMDConv3d"])
+def test_branch_convolution_on_the_operator(cls, dtype, dev):
+    """The deformation branch's nn.Conv3d evaluated by the operator at zero offsets (modules._branch_conv: the default
+    for bfloat16, "all" for float32 too) against the stock call, both held to a float64 run of the same layer (direct
+    kernels): in bfloat16 the operator's branch is no further from it than the stock one (both carry the 5 - 10 % that
+    bfloat16 offsets leave in the gradients that pass through them); in float32 the output agrees to 1e-4 and the
+    gradients through the offsets to 1e-2 (sampling points that change their voxel, see _branch_conv)."""
+    from d2conv3d_amd import modules as M
+    torch.manual_seed(31)
+    layer = getattr(M, cls)(128, 64, 3, padding=1).to(dev)
+    with torch.no_grad():
+        layer.deform_params.weight.normal_(0, 0.02)
+        layer.deform_params.bias.normal_(0, 0.3)
+    l64 = getattr(M, cls)(128, 64, 3, padding=1).to(dev).double()
+    layer = layer.to(dtype)
+    with torch.no_grad():
+        for p64, p in zip(l64.parameters(), layer.parameters()):
+            p64.copy_(p.double())
+    x = torch.randn(1, 128, 5, 12, 13, device=dev).to(dtype)
+    gout = torch.randn(1, 64, 5, 12, 13, device=dev).to(dtype)
+
+    def step(lay, cast):
+        lay.zero_grad()
+        xi = cast(x).clone().requires_grad_(True)
+        out = lay(xi)
+        out.backward(cast(gout))
+        return [out.detach().double(), xi.grad.double()] + [p.grad.double().clone() for p in lay.parameters()]
+
+    exact = step(l64, lambda t: t.double())
+    res = {}
+    for on in ("all", False):
+        layer.branch_on_operator = on
+        res[on] = step(layer, lambda t: t)
+    err = lambda a, e: ((a - e).norm() / e.norm().clamp_min(1e-30)).item()
+    for i, e in enumerate(exact):
+        on_op, stock = err(res["all"][i], e), err(res[False][i], e)
+        if dtype == torch.bfloat16:
+            assert on_op < max(1.5 * stock, 2e-2), (cls, i, on_op, stock)
+        else:
+            assert on_op < (1e-4 if i == 0 else 1e-2), (cls, i, on_op, stock)
+    # the default: on for bfloat16 only
+    layer.branch_on_operator = True
+    out = step(layer, lambda t: t)[0]
+    same, other = ("all", False) if dtype == torch.bfloat16 else (False, "all")
+    assert err(out, res[same][0]) < 0.2 * err(out, res[other][0]), (err(out, res[same][0]), err(out, res[other][0]))
