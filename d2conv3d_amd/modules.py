@@ -46,6 +46,11 @@ def _zero_offsets(device, n, channels, dims):
     return t
 
 
+def release_zero_offsets():
+    """Frees the zero tensors that _branch_conv keeps per feature-map shape (81 x positions floats each)."""
+    _ZERO_OFFSETS.clear()
+
+
 def _branch_conv(layer, x):
     """The deformation branch of a layer: its stock convolution `deform_params` (network/layers.py:66-68).  Where that
     is a plain nn.Conv3d whose shape the matrix-core kernels serve, it is evaluated by the deformable operator at
