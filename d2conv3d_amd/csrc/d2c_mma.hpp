@@ -547,11 +547,15 @@ D2C_DEV CornerRow corner_row(const CoordConst &cc, float z, float y, float x, fl
     const float fz = floorf(zs), fy = floorf(ys), fx = floorf(xs);
     const float hz = zs - fz, hy = ys - fy, hx = xs - fx;
     const float lz = (fz + 1.f) - zs, ly = (fy + 1.f) - ys, lx = (fx + 1.f) - xs;
-    const bool z0 = in & (fz >= 0.f), z1 = in & (fz < cc.Dm1);
-    const bool y0 = in & (fy >= 0.f), y1 = in & (fy < cc.Hm1);
-    const bool x0 = in & (fx >= 0.f), x1 = in & (fx < cc.Wm1);
+    // (a corner is fetched where it lies inside the volume AND has a weight: a sampling point that sits on a voxel
+    // plane -- zero offsets, i.e. an ordinary convolution, or whole-voxel offsets -- gives the corners on the far side
+    // of the plane weight zero, and a modulation of exactly zero, common behind a ReLU, all eight; such corners read
+    // the row of zeros like those outside the volume.  For finite inputs the sum is the same.)
+    const bool z0 = in & (fz >= 0.f), z1 = in & (fz < cc.Dm1) & (hz > 0.f);
+    const bool y0 = in & (fy >= 0.f), y1 = in & (fy < cc.Hm1) & (hy > 0.f);
+    const bool x0 = in & (fx >= 0.f), x1 = in & (fx < cc.Wm1) & (hx > 0.f);
     r.live = ((z0 ? 0x0Fu : 0u) | (z1 ? 0xF0u : 0u)) & ((y0 ? 0x33u : 0u) | (y1 ? 0xCCu : 0u))
-             & ((x0 ? 0x55u : 0u) | (x1 ? 0xAAu : 0u)) & cc.keep;
+             & ((x0 ? 0x55u : 0u) | (x1 ? 0xAAu : 0u)) & cc.keep & (ms != 0.f ? 0xFFu : 0u);
     const float az[2] = {z0 ? lz : 0.f, z1 ? hz : 0.f};
     const float ay[2] = {y0 ? ly : 0.f, y1 ? hy : 0.f};
     const float ax[2] = {x0 ? lx : 0.f, x1 ? hx : 0.f};
