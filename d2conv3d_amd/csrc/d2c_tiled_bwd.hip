@@ -684,7 +684,9 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col_kernel(BwdDataArgs a)
 // stored from the registers: the lane's weight row is chosen such that its 16 accumulator registers are two runs
 // of 8 consecutive channels (see mma8_bf16_t).
 constexpr int kColRing = 4, kColAhead = 3;
-template <int NB>   // blocks of 8 k-groups: ogk = 128 NB
+// ADD (the later passes over a weight group wider than 512 channels): the rows that the passes before it left are
+// added, the sum formed in float and rounded to bfloat16 once more.
+template <int NB, bool ADD>   // blocks of 8 k-groups: ogk = 128 NB
 __global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a)
 {
     typedef bf16_t T;
@@ -760,15 +762,35 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a
         for (int q = 0; q < R; q++) dma_piece(min(lo + d, hi - 1), d, q);
 
     const int cpc2 = 2 * (s.cpg / BKC);        // half-steps per (offset group, tap)
-    for (int h2 = lo, it = 0; h2 < hi; h2++, it++) {
-        // step order: offset group (outer), tap, chunk of the group, half (inner)
+    // where this lane's 2 x 8 channels of half-step h2 go (step order: offset group (outer), tap, chunk of the group,
+    // half (inner))
+    const int m_lane = m0 + wave * 32 + (lane & 31);
+    auto row_of = [&](int h2) -> T * {
         const int jj2 = h2 % cpc2, k = (h2 / cpc2) % s.K, gi = h2 / (cpc2 * s.K);
         const int j = gi * (cpc2 >> 1) + (jj2 >> 1), half = jj2 & 1;
+        const int c0 = wg * s.cg + j * BKC;
+        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
+        return gb + (long)m_lane * BKC + half * HC + 8 * (lane >> 5);
+    };
+    for (int h2 = lo, it = 0; h2 < hi; h2++, it++) {
         // Half-tile `it` has landed when no more of this wavefront's operations are in flight than it has issued
         // since: the requests of the kColAhead - 1 half-tiles behind it, and the 2 stores of each step since then
-        // (only counted when every wavefront of the workgroup stores in every step).
-        wait_vm_at_most((kColAhead - 1) * R + ((full_tile && it >= kColAhead) ? 2 * kColAhead : 0));
+        // (only counted when every wavefront of the workgroup stores in every step); ADD: also the 2 loads at the
+        // top of the kColAhead - 1 steps since.
+        wait_vm_at_most((kColAhead - 1) * R +
+                        ((full_tile && it >= kColAhead) ? 2 * kColAhead + (ADD ? 2 * (kColAhead - 1) : 0) : 0));
         lds_only_barrier();
+        // (ADD: the rows as the passes before left them, wanted at the end of the step.  Requesting them up to four
+        // steps ahead made the pass slower: the counter above completes in order, so a row that is late holds up
+        // the weight tiles requested after it.)
+        T *row = row_of(h2);
+        uint4 pv0 = make_uint4(0, 0, 0, 0), pv1 = pv0;
+        if constexpr (ADD) {
+            if (m_lane < s.M) {
+                pv0 = *reinterpret_cast<const uint4 *>(row);
+                pv1 = *reinterpret_cast<const uint4 *>(row + 16);
+            }
+        }
 
         f32x16 acc;
 #pragma unroll
@@ -795,11 +817,15 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a
 #pragma unroll
         for (int q = 0; q < 8; q++) woff[q] += adv;
 
-        const int c0 = wg * s.cg + j * BKC;
-        T *gb = reinterpret_cast<T *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
-        const int m = m0 + wave * 32 + (lane & 31);
-        if (m < s.M) {
-            T *row = gb + (long)m * BKC + half * HC + 8 * (lane >> 5);
+        if (m_lane < s.M) {
+            if constexpr (ADD) {
+                const unsigned pw[8] = {pv0.x, pv0.y, pv0.z, pv0.w, pv1.x, pv1.y, pv1.z, pv1.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    acc[2 * e] += __uint_as_float(pw[e] << 16);
+                    acc[2 * e + 1] += __uint_as_float(pw[e] & 0xffff0000u);
+                }
+            }
             *reinterpret_cast<uint4 *>(row) =
                 make_uint4(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
                            pack_bf16x2(acc[6], acc[7]));
@@ -845,19 +871,23 @@ int launch_bwd_col32(const BwdDataArgs &a, int nsplit, hipStream_t st)
 {
     const size_t lds = (size_t)kColRing * 32 * a.ogk * 2;
     const dim3 grid((a.s.M + kCol32MT - 1) / kCol32MT, a.s.groups, nsplit);
-    auto go = [&](auto nb_c) -> int {
+    auto go = [&](auto nb_c, auto add_c) -> int {
         constexpr int NB = decltype(nb_c)::value;
-        if (int rc = d2c_allow_lds((const void *)tiled_bwd_col32_kernel<NB>, 160 * 1024, "tiled_bwd_col32_kernel")) return rc;
+        constexpr bool ADD = decltype(add_c)::value;
+        if (int rc = d2c_allow_lds((const void *)tiled_bwd_col32_kernel<NB, ADD>, 160 * 1024, "tiled_bwd_col32_kernel")) return rc;
         D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_col32_kernel");
-        hipLaunchKernelGGL((tiled_bwd_col32_kernel<NB>), grid, dim3(kThreads), lds, st, a);
+        hipLaunchKernelGGL((tiled_bwd_col32_kernel<NB, ADD>), grid, dim3(kThreads), lds, st, a);
         return d2c_check_launch("tiled_bwd_col32_kernel");
     };
-    switch (a.ogk / 128) {
-    case 1: return go(std::integral_constant<int, 1>{});
-    case 2: return go(std::integral_constant<int, 2>{});
-    case 3: return go(std::integral_constant<int, 3>{});
-    default: return go(std::integral_constant<int, 4>{});
-    }
+    auto pick = [&](auto add_c) -> int {
+        switch (a.ogk / 128) {
+        case 1: return go(std::integral_constant<int, 1>{}, add_c);
+        case 2: return go(std::integral_constant<int, 2>{}, add_c);
+        case 3: return go(std::integral_constant<int, 3>{}, add_c);
+        default: return go(std::integral_constant<int, 4>{}, add_c);
+        }
+    };
+    return a.add_aux ? pick(std::true_type{}) : pick(std::false_type{});
 }
 
 template <typename T> size_t bwd_data_lds(int ogk)
@@ -1988,7 +2018,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                               bool weights_packed)
 {
     // Weight groups wider than one pass get their grad-column rows from the product-only kernels too: the first pass
-    // writes the rows, every later one (on tiled_bwd_col_kernel, which can) adds to them.
+    // writes the rows, every later one adds to them.
     // phase: 1 = the weight re-layout (and the clears), 2 = the kernel, 3 = both.  g_n > 0 (grad-column product on
     // tiled_bwd_col32_kernel only, see d2c_bwd_sliceable): the rows of the offset groups [g_lo, g_lo + g_n) only,
     // `gcolbuf` pointing where chunk 0 would start.
@@ -2035,7 +2065,11 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
     // quantity downstream of the grad-column product is linear in it, so the passes add up.
     for (int o0 = 0; o0 < s.og; o0 += omax) {
         const int ogn = s.og - o0 < omax ? s.og - o0 : omax;
-        const int ogk = d2c_bwd_ogk(ogn, Elem<T>::DT);
+        int ogk = d2c_bwd_ogk(ogn, Elem<T>::DT);
+        // (a later pass of the grad-column product on its own: padded to what tiled_bwd_col32_kernel takes, which
+        // the buffer of the first pass has room for)
+        const bool only_col = gcolbuf && !gxcl && !goff && !gmask;
+        if (only_col && o0 > 0 && bwd_col32_ok((ogk + 127) / 128 * 128, ogn, Elem<T>::DT)) ogk = (ogk + 127) / 128 * 128;
         const long total = (long)s.groups * s.K * s.nchunk * BKC * ogk;
         // two-term bfloat16 operands for this pass (float problems): wherever the description asks for them, and for
         // the grad-column product on its own by default (f32split == 2)
@@ -2064,7 +2098,7 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
                       auxoff, auxmask, sliced ? g_lo * cpc2 * s.K : 0, sliced ? (g_lo + g_n) * cpc2 * s.K : 0};
         const int nkg = ogk / (2 * Elem<T>::VEC);
         int rc;
-        if (col_only && o0 == 0 && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
+        if (col_only && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
             rc = launch_bwd_col32(a, nsplit, st);
         } else if (sliced) {
             d2c_set_error("grad-column product: slices are made by tiled_bwd_col32_kernel only");

@@ -32,6 +32,9 @@ SHAPES = {
     "c64_o320_big": (1, 64, 320, (7, 35, 34), 3, 1, 1, 1, 1, 1, True, True, 1.5),       # N*P = 8330: ragged
     "c128_groups2_o640_big": (1, 128, 640, (4, 32, 33), 3, 1, 1, 1, 2, 2, True, True, 2.0),
     "c64_o200_big": (1, 64, 200, (7, 35, 34), 3, 1, 1, 1, 1, 1, True, True, 1.5),       # 256-wide output tile
+    # narrow weight groups with more than 160 position tiles: the same kernel, most of its output tile empty
+    "c64_o96_many_tiles": (1, 64, 96, (9, 34, 35), 3, 1, 1, 1, 1, 1, True, True, 1.5),  # N*P = 10710: ragged
+    "c128_groups2_o48_many_tiles": (1, 128, 48, (8, 32, 21), 3, 1, 1, 1, 2, 2, True, False, 1.0),   # 84 tiles x 2 groups
     # the same kernel's schedule: three output tiles per position tile (399 work items on 256 compute units: one
     # whole round, the rest cut into step ranges), two weight groups with few position tiles (all items cut)
     "c64_o1100_big": (1, 64, 1100, (7, 35, 35), 3, 1, 1, 1, 1, 1, True, True, 1.5),
