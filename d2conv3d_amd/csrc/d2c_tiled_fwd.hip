@@ -1092,16 +1092,18 @@ int launch_fwd_cfg(const FwdArgs &a, int nt, hipStream_t st)
 
 }  // namespace
 
-// Problems with enough position tiles run the DMA-gather kernel (64-position tiles, 512 or 256 output channels per
-// workgroup); everything else the register-gather kernel (128-position tiles). Narrow weight groups leave most of the
-// DMA kernel's output tile empty, but it is bound by its sampling, not by its matrix work: with enough tiles to fill
-// the chip without cutting their steps it is 1.3 - 2.2 x faster there too (1024 -> 108 channels on 8x30x54: 1.44 ->
-// 0.65 ms), and at the 128 tiles of 64 -> 64 channels on 8x32x32 it is 25 % slower.
-bool d2c_fwd_use_dma(int og, int M, int groups)
-{
-    const long tiles = (long)((M + kDMT - 1) / kDMT) * groups;
-    return tiles >= (og > 128 ? 128 : 160);
-}
+// Which of the two forward kernels a shape runs on: the DMA-gather kernel (64-position tiles, 512 or 256 output channels
+// per workgroup, persistent, the steps of its last round of work items shared out) or the register-gather kernel
+// (128-position tiles).  Weight groups wider than 128 output channels take the DMA kernel from 4 position tiles on:
+// with few tiles it cuts their steps into as many pieces as there are compute units (512 -> 512 channels on 8x15x27,
+// 51 tiles: 0.74 -> 0.22 ms; 1024 -> 1024 on 4x8x14, 7 tiles: 0.46 -> 0.21 ms; with one or two tiles it is 10 - 30 %
+// slower).  Narrow weight groups leave most of its output tile empty, but it is bound by its sampling, not by its
+// matrix work: with enough tiles to fill the chip without cutting their steps it is 1.3 - 2.2 x faster there too
+// (1024 -> 108 channels on 8x30x54: 1.44 -> 0.65 ms), and at the 128 tiles of 64 -> 64 channels on 8x32x32 it is 25 %
+// slower.
+constexpr int kDmaTilesWide = 4, kDmaTilesNarrow = 160, kColsTiles = 48;
+static long dma_tiles(int M, int groups) { return (long)((M + kDMT - 1) / kDMT) * groups; }
+bool d2c_fwd_use_dma(int og, int M, int groups) { return dma_tiles(M, groups) >= (og > 128 ? kDmaTilesWide : kDmaTilesNarrow); }
 
 int d2c_fwd_pos_tile(int og, int M, int groups) { return d2c_fwd_use_dma(og, M, groups) ? kDMT : kMT; }
 
@@ -1148,10 +1150,13 @@ size_t d2c_fwd_stats_ws(const TiledShape &s)
 }
 
 // Whether the forward kernel of this shape can write the sampled columns for the backward pass (FwdArgs::col): the
-// DMA-gather kernel on problems with offsets along all three axes.
+// DMA-gather kernel on problems with offsets along all three axes and at least kColsTiles position tiles (below that
+// the backward kernels that read the columns lose to the ones that sample again: 256 -> 256 channels on 4x15x27, 26
+// tiles: 0.25 -> 0.30 ms).
 bool d2c_fwd_writes_columns(const TiledShape &s, int dtype)
 {
-    return (dtype == D2C_BF16 || dtype == D2C_F32) && s.nd == 3 && (s.axes & 7) == 7 && d2c_fwd_use_dma(s.og, s.M, s.groups);
+    return (dtype == D2C_BF16 || dtype == D2C_F32) && s.nd == 3 && (s.axes & 7) == 7 &&
+           d2c_fwd_use_dma(s.og, s.M, s.groups) && dma_tiles(s.M, s.groups) >= kColsTiles;
 }
 long d2c_columns_rows(const TiledShape &s) { return (long)((s.M + kDMT - 1) / kDMT) * kDMT; }
 // `stats` / `stats_part`: the [N][Cout][2] result and the per-tile scratch of d2c_fwd_stats_ws() bytes, or NULL.

@@ -198,8 +198,9 @@ int d2c_conv3d_backward(const d2c_conv3d_desc *desc, const void *grad_out, const
  * columns are the interpolated floats themselves and their product keeps float32's accuracy (three bfloat16 terms
  * per float on the bfloat16 matrix instruction, or the float32 instruction), whatever D2C_BWD_F32_SPLIT says.  `size_map` as in d2c_conv3d_forward_stats: NULL, or the description of
  * the size map that `offset` then is.  d2c_conv3d_columns_bytes() is 0 where this is not served (anything but
- * bfloat16 and float32 problems on the large-tile matrix-core kernels with offsets along all three axes and an even
- * number of 64- / 32-channel chunks per weight group); the two calls then
+ * bfloat16 and float32 problems on the matrix-core kernels with at least 48 tiles of 64 output positions (times
+ * weight groups), offsets along all three axes and an even number of 64- / 32-channel chunks per weight group); the
+ * two calls then
  * fail with D2C_ERR_UNSUPPORTED and the caller uses the plain ones.  The memory-saving bits of
  * d2c_conv3d_desc::backward_flags are ignored by d2c_conv3d_backward_columns.
  */
