@@ -4,7 +4,7 @@
 #include "d2c_tiled.hpp"
 #include "d2c_mma.hpp"
 
-int d2c_fwd_out_tile(int og, int M, int groups);
+int d2c_fwd_out_tile(const TiledShape &s);
 template <typename T>
 int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, const void *mask, const void *wp,
                          const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part,
@@ -123,7 +123,7 @@ TiledShape tiled_shape(const d2c_conv3d_desc &q, int nd = 3, int quirks = 0, con
     // float problems: 1 = every backward matrix kernel on two-term bfloat16 operands (asked for in the description),
     // 2 = the grad-column product alone, like the forward kernels (the default: every tolerance gate stays green)
     s.f32split = q.dtype != D2C_F32 ? 0 : ((q.backward_flags & D2C_BWD_F32_SPLIT) ? 1 : (kF32SplitFwd ? 2 : 0));
-    const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
+    const int nt = d2c_fwd_out_tile(s);
     s.ogp = (s.og + nt - 1) / nt * nt;
     s.geo = make_geom(q);
     return s;

@@ -1094,27 +1094,34 @@ int launch_fwd_cfg(const FwdArgs &a, int nt, hipStream_t st)
 
 // Which of the two forward kernels a shape runs on: the DMA-gather kernel (64-position tiles, 512 or 256 output channels
 // per workgroup, persistent, the steps of its last round of work items shared out) or the register-gather kernel
-// (128-position tiles).  Weight groups wider than 128 output channels take the DMA kernel from 4 position tiles on:
-// with few tiles it cuts their steps into as many pieces as there are compute units (512 -> 512 channels on 8x15x27,
-// 51 tiles: 0.74 -> 0.22 ms; 1024 -> 1024 on 4x8x14, 7 tiles: 0.46 -> 0.21 ms; with one or two tiles it is 10 - 30 %
-// slower).  Narrow weight groups leave most of its output tile empty, but it is bound by its sampling, not by its
-// matrix work: with enough tiles to fill the chip without cutting their steps it is 1.3 - 2.2 x faster there too
-// (1024 -> 108 channels on 8x30x54: 1.44 -> 0.65 ms), and at the 128 tiles of 64 -> 64 channels on 8x32x32 it is 25 %
-// slower.
-constexpr int kDmaTilesWide = 4, kDmaTilesNarrow = 160, kColsTiles = 48;
-static long dma_tiles(int M, int groups) { return (long)((M + kDMT - 1) / kDMT) * groups; }
-bool d2c_fwd_use_dma(int og, int M, int groups) { return dma_tiles(M, groups) >= (og > 128 ? kDmaTilesWide : kDmaTilesNarrow); }
+// (128-position tiles).  Weight groups wider than 128 output channels take the DMA kernel when they fill the chip
+// with whole tiles (128 and more) or have at least 1024 steps in all: with few tiles it cuts their steps into as
+// many pieces as there are compute units (512 -> 512 channels on 8x15x27, 51 tiles: 0.74 -> 0.22 ms; 1024 -> 1024
+// on 4x8x14, 7 tiles of 432 steps: 0.46 -> 0.21 ms), which pays from about a thousand steps on (4 tiles of 48 steps,
+// 512 channels on 4 rows of 64 positions: 13 % slower; 2 tiles of 216 steps: 30 % slower).  Narrow weight groups leave
+// most of its output tile empty, but it is bound by its sampling, not by its matrix work: with enough tiles to fill
+// the chip without cutting their steps it is 1.3 - 2.2 x faster there too (1024 -> 108 channels on 8x30x54: 1.44 ->
+// 0.65 ms), and at the 128 tiles of 64 -> 64 channels on 8x32x32 it is 25 % slower.
+constexpr int kDmaTilesNarrow = 160, kDmaTilesWide = 128, kDmaStepsWide = 1024, kColsTiles = 48;
+static long dma_tiles(const TiledShape &s) { return (long)((s.M + kDMT - 1) / kDMT) * s.groups; }
+bool d2c_fwd_use_dma(const TiledShape &s)
+{
+    const long tiles = dma_tiles(s);
+    if (s.og <= 128) return tiles >= kDmaTilesNarrow;
+    return tiles >= kDmaTilesWide || tiles * s.nchunk * s.K >= kDmaStepsWide;
+}
 
-int d2c_fwd_pos_tile(int og, int M, int groups) { return d2c_fwd_use_dma(og, M, groups) ? kDMT : kMT; }
+int d2c_fwd_pos_tile(const TiledShape &s) { return d2c_fwd_use_dma(s) ? kDMT : kMT; }
 
 // Output channels per workgroup: as wide as the weight group needs (the sampled
 // tile is then produced once), but narrower when there are too few position
 // tiles to occupy the chip.
-int d2c_fwd_out_tile(int og, int M, int groups)
+int d2c_fwd_out_tile(const TiledShape &s)
 {
-    if (d2c_fwd_use_dma(og, M, groups)) return og > 256 ? 512 : 256;
+    const int og = s.og;
+    if (d2c_fwd_use_dma(s)) return og > 256 ? 512 : 256;
     int nt = og > 256 ? 512 : (og > 128 ? 256 : (og > 64 ? 128 : 64));
-    const int ntile = (M + kMT - 1) / kMT;
+    const int ntile = (s.M + kMT - 1) / kMT;
     while (nt > 64 && ntile * ((og + nt - 1) / nt) < 128) nt >>= 1;
     return nt;
 }
@@ -1123,8 +1130,8 @@ int d2c_fwd_out_tile(int og, int M, int groups)
 int d2c_fwd_split(const TiledShape &s)
 {
     // the DMA-gather kernel shares out the steps of its last round of work items, whatever their number
-    if (d2c_fwd_use_dma(s.og, s.M, s.groups)) return 2;
-    const int mt = d2c_fwd_pos_tile(s.og, s.M, s.groups), nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
+    if (d2c_fwd_use_dma(s)) return 2;
+    const int mt = d2c_fwd_pos_tile(s), nt = d2c_fwd_out_tile(s);
     const long wgs = (long)((s.M + mt - 1) / mt) * (s.ogp / nt) * s.groups;
     if (wgs >= 128) return 1;
     const int S = s.nchunk * s.K;
@@ -1140,12 +1147,12 @@ int d2c_fwd_split(const TiledShape &s);
 // steps shared out between workgroups).
 bool d2c_fwd_fills_stats(const TiledShape &s)
 {
-    if (d2c_fwd_use_dma(s.og, s.M, s.groups)) return s.P >= kDMT;
+    if (d2c_fwd_use_dma(s)) return s.P >= kDMT;
     return d2c_fwd_split(s) == 1;
 }
 size_t d2c_fwd_stats_ws(const TiledShape &s)
 {
-    if (!d2c_fwd_use_dma(s.og, s.M, s.groups)) return 0;     // (the register-gather kernel adds into the result itself)
+    if (!d2c_fwd_use_dma(s)) return 0;     // (the register-gather kernel adds into the result itself)
     return d2c_align_up((size_t)((s.M + kDMT - 1) / kDMT) * 2 * s.Cout * 2 * sizeof(float));
 }
 
@@ -1156,7 +1163,7 @@ size_t d2c_fwd_stats_ws(const TiledShape &s)
 bool d2c_fwd_writes_columns(const TiledShape &s, int dtype)
 {
     return (dtype == D2C_BF16 || dtype == D2C_F32) && s.nd == 3 && (s.axes & 7) == 7 &&
-           d2c_fwd_use_dma(s.og, s.M, s.groups) && dma_tiles(s.M, s.groups) >= kColsTiles;
+           d2c_fwd_use_dma(s) && dma_tiles(s) >= kColsTiles;
 }
 long d2c_columns_rows(const TiledShape &s) { return (long)((s.M + kDMT - 1) / kDMT) * kDMT; }
 // `stats` / `stats_part`: the [N][Cout][2] result and the per-tile scratch of d2c_fwd_stats_ws() bytes, or NULL.
@@ -1166,7 +1173,7 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
                          const void *bias, void *out, float *outacc, hipStream_t st, float *stats, float *stats_part,
                          void *col)
 {
-    const bool dma = d2c_fwd_use_dma(s.og, s.M, s.groups);
+    const bool dma = d2c_fwd_use_dma(s);
     const int nsplit = (outacc && !dma) ? d2c_fwd_split(s) : 1;
     const long n = (long)s.N * s.Cout * s.P;
     // the channels-last input is followed by a row of zeros (see forward_t)
@@ -1181,7 +1188,7 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(a.stats, (size_t)s.N * s.Cout * 2 * sizeof(float), st);
     }
-    if (a.stats && dma && d2c_fwd_out_tile(s.og, s.M, s.groups) != 512) {
+    if (a.stats && dma && d2c_fwd_out_tile(s) != 512) {
         // (the 256-channel tile has two wavefronts per channel, which add into their slots)
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(a.stats, d2c_fwd_stats_ws(s), st);
@@ -1190,7 +1197,7 @@ int d2c_tiled_fwd_launch(const TiledShape &s, const void *xcl, const void *off, 
         D2cProfScope prof(D2C_PROF_PACK, st);
         d2c_fill_zero(outacc, (size_t)n * sizeof(float), st);
     }
-    const int nt = d2c_fwd_out_tile(s.og, s.M, s.groups);
+    const int nt = d2c_fwd_out_tile(s);
     int rc = 0;
     bool aux16 = false;
     if constexpr (sizeof(T) == 2) aux16 = s.adt == D2C_BF16;

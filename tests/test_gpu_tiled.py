@@ -32,9 +32,10 @@ SHAPES = {
     "c64_o320_big": (1, 64, 320, (7, 35, 34), 3, 1, 1, 1, 1, 1, True, True, 1.5),       # N*P = 8330: ragged
     "c128_groups2_o640_big": (1, 128, 640, (4, 32, 33), 3, 1, 1, 1, 2, 2, True, True, 2.0),
     "c64_o200_big": (1, 64, 200, (7, 35, 34), 3, 1, 1, 1, 1, 1, True, True, 1.5),       # 256-wide output tile
-    # wide weight groups with a handful of position tiles: the same kernel, every work item cut into step ranges
-    "c64_o320_few_tiles": (1, 64, 320, (4, 9, 12), 3, 1, 1, 1, 1, 1, True, True, 1.5),   # N*P = 432: 7 tiles
-    "c128_groups2_o512_few_tiles": (2, 128, 512, (3, 8, 9), 3, 1, 1, 1, 2, 2, True, True, 1.0),
+    # wide weight groups with a handful of position tiles but more than a thousand steps in all: the same kernel, every
+    # work item cut into step ranges
+    "c256_o320_few_tiles": (1, 256, 320, (4, 12, 16), 3, 1, 1, 1, 1, 1, True, True, 1.5),   # N*P = 768: 12 tiles
+    "c512_groups2_o512_few_tiles": (2, 512, 512, (3, 8, 9), 3, 1, 1, 1, 2, 2, True, True, 1.0),   # 7 tiles x 2 groups
     # narrow weight groups with more than 160 position tiles: the same kernel, most of its output tile empty
     "c64_o96_many_tiles": (1, 64, 96, (9, 34, 35), 3, 1, 1, 1, 1, 1, True, True, 1.5),  # N*P = 10710: ragged
     "c128_groups2_o48_many_tiles": (1, 128, 48, (8, 32, 21), 3, 1, 1, 1, 2, 2, True, False, 1.0),   # 84 tiles x 2 groups
