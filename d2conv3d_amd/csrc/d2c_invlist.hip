@@ -78,17 +78,20 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
 // instructions than with every lane unpacking every entry, in a kernel that waits for its vector ALU as much as for
 // memory (C=512 in 8 groups, 8x30x54: 0.415 -> 0.345 ms; float, C=256: 0.406 -> 0.308 ms).
 // RB: rows of a batch requested together (8 for bfloat16, 4 for float: measured).
+// SMALL: workgroups of 8 cubes (1 x 2 x 4, one wavefront) instead of 32 (2 x 4 x 4): problems that make fewer than a
+// few hundred of the large workgroups spread over all compute units that way.
 template <int J> D2C_DEV int group8_bcast(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x18 | (J << 5)); }
 template <int J> D2C_DEV float group8_bcast(float v) { return __int_as_float(group8_bcast<J>(__float_as_int(v))); }
 
-template <typename T, bool COMPACT, int RB>
-__global__ void __launch_bounds__(256, 4)
+template <typename T, bool COMPACT, int RB, bool SMALL>
+__global__ void __launch_bounds__(SMALL ? 64 : 256, SMALL ? 16 : 4)
 gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, int c_lo, int c_n)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
-    const int sub = threadIdx.x & 7, ci = threadIdx.x >> 3;       // 32 cubes per workgroup: 2 x 4 x 4 of them
+    constexpr int BY = SMALL ? 2 : 4, BZ = SMALL ? 1 : 2;          // cubes per workgroup: BZ x BY x 4
+    const int sub = threadIdx.x & 7, ci = threadIdx.x >> 3;
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
-    const int nbx = (ncx + 3) / 4, nby = (ncy + 3) / 4, nbz = (ncz + 1) / 2;
+    const int nbx = (ncx + 3) / 4, nby = (ncy + BY - 1) / BY, nbz = (ncz + BZ - 1) / BZ;
     // Workgroups are dealt round-robin to the 8 XCDs.  An XCD takes a contiguous range of the blocks of cubes
     // (neighbours in space share bins and grad-column rows in its L2) and, block by block, the channel chunks one
     // after the other: the chunks of one offset group walk the same lists, which then come from L2.
@@ -104,7 +107,7 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, in
     const int by = blk % nby; blk /= nby;
     const int bz = blk % nbz;
     const int b = blk / nbz;
-    const int cx = bx * 4 + (ci & 3), cy = by * 4 + ((ci >> 2) & 3), cz = bz * 2 + (ci >> 4);
+    const int cx = bx * 4 + (ci & 3), cy = by * BY + ((ci >> 2) & (BY - 1)), cz = bz * BZ + (ci >> 2) / BY;
     if (cx >= ncx || cy >= ncy || cz >= ncz) return;      // (whole groups of 8 lanes leave together)
     const int x0 = cx * 2, y0 = cy * 2, z0 = cz * 2;
     const int g = (cidx * BKC) / s.cpg;
@@ -581,10 +584,19 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists
     D2cProfScope prof(D2C_PROF_GX_OWNER, st, "gx_owner_cube_kernel");
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
-    dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * c_n));    // see the kernel's unit mapping
     constexpr int RB = sizeof(T) == 2 ? 8 : 4;
-    if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, RB>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
-    else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, RB>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+    // (fewer than two of the large workgroups per compute unit: one-wavefront workgroups, 3 - 5 % faster backward
+    // pass at 512 channels on 8x15x27 and 128 channels on 8x30x54)
+    if (8 * ((nblk + 7) / 8) * c_n < 512) {
+        const long nblk8 = (long)s.N * ncz * ((ncy + 1) / 2) * ((ncx + 3) / 4);
+        dim3 grid((unsigned)(8 * ((nblk8 + 7) / 8) * c_n));
+        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, RB, true>), grid, dim3(64), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, RB, true>), grid, dim3(64), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+    } else {
+        dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * c_n));    // see the kernel's unit mapping
+        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, RB, false>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, RB, false>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+    }
     if (int rc = d2c_check_launch("gx_owner_kernel")) return rc;
     // the overflow entries, usually none (the kernel reads their number from device memory)
     hipLaunchKernelGGL(gx_overflow_kernel<T>, dim3(512), dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
