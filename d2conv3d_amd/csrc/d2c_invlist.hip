@@ -78,18 +78,22 @@ lists_pass_kernel(TiledShape s, const void *off, const void *mask, SampleLists L
 // instructions than with every lane unpacking every entry, in a kernel that waits for its vector ALU as much as for
 // memory (C=512 in 8 groups, 8x30x54: 0.415 -> 0.345 ms; float, C=256: 0.406 -> 0.308 ms).
 // RB: rows of a batch requested together (8 for bfloat16, 4 for float: measured).
-// SMALL: workgroups of 8 cubes (1 x 2 x 4, one wavefront) instead of 32 (2 x 4 x 4): problems that make fewer than a
-// few hundred of the large workgroups spread over all compute units that way.
+// SMALL (problems that make fewer than a few hundred of the large workgroups): a workgroup is 8 cubes (1 x 2 x 4)
+// and nine wavefronts, one per (z, y) offset of the base voxels; each walks the three x bins of its offset for the 8
+// cubes, the nine add their sums in LDS (ds_add_f32), and the workgroup stores the block.  The walk over the 27 base
+// voxels of a cube is a chain of dependent loads (list entries, then rows), a ninth as long this way, on nine times
+// the wavefronts.
 template <int J> D2C_DEV int group8_bcast(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x18 | (J << 5)); }
 template <int J> D2C_DEV float group8_bcast(float v) { return __int_as_float(group8_bcast<J>(__float_as_int(v))); }
 
 template <typename T, bool COMPACT, int RB, bool SMALL>
-__global__ void __launch_bounds__(SMALL ? 64 : 256, SMALL ? 16 : 4)
+__global__ void __launch_bounds__(SMALL ? 576 : 256, SMALL ? 1 : 4)
 gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, int c_lo, int c_n)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC;
     constexpr int BY = SMALL ? 2 : 4, BZ = SMALL ? 1 : 2;          // cubes per workgroup: BZ x BY x 4
-    const int sub = threadIdx.x & 7, ci = threadIdx.x >> 3;
+    const int sub = threadIdx.x & 7, ci = SMALL ? (threadIdx.x & 63) >> 3 : threadIdx.x >> 3;
+    const int part = SMALL ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;      // (z, y) offset of this wavefront
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const int nbx = (ncx + 3) / 4, nby = (ncy + BY - 1) / BY, nbz = (ncz + BZ - 1) / BZ;
     // Workgroups are dealt round-robin to the 8 XCDs.  An XCD takes a contiguous range of the blocks of cubes
@@ -108,7 +112,13 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, in
     const int bz = blk % nbz;
     const int b = blk / nbz;
     const int cx = bx * 4 + (ci & 3), cy = by * BY + ((ci >> 2) & (BY - 1)), cz = bz * BZ + (ci >> 2) / BY;
-    if (cx >= ncx || cy >= ncy || cz >= ncz) return;      // (whole groups of 8 lanes leave together)
+    const bool inside = cx < ncx && cy < ncy && cz < ncz;
+    if (!SMALL && !inside) return;                        // (whole groups of 8 lanes leave together)
+    __shared__ float s_sum[SMALL ? 8 * 8 * BKC : 1];      // [cube][voxel of the cube][channel]
+    if constexpr (SMALL) {
+        for (int i = threadIdx.x; i < 8 * 8 * BKC; i += 576) s_sum[i] = 0.f;
+        __syncthreads();
+    }
     const int x0 = cx * 2, y0 = cy * 2, z0 = cz * 2;
     const int g = (cidx * BKC) / s.cpg;
     float acc[2][2][2][VEC];
@@ -121,10 +131,12 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, in
     for (int rz = 0; rz < 3; rz++) {
         const int zb = z0 - 1 + rz;
         if (zb > s.D - 1) continue;
+        if (SMALL && (rz != part % 3 || !inside)) continue;
 #pragma unroll
         for (int ry = 0; ry < 3; ry++) {
             const int yb = y0 - 1 + ry;
             if (yb > s.H - 1) continue;
+            if (SMALL && ry != part / 3) continue;
             const int bin1 = bin_of(s, b, g, zb, yb, x0 - 1);
             const int em1 = min(L.counts[bin1], L.cap);
             const int em2 = em1 + min(L.counts[bin1 + 1], L.cap);
@@ -209,6 +221,34 @@ gx_owner_cube_kernel(TiledShape s, const T *gcol, SampleLists L, float *gxcl, in
                 }, std::make_integer_sequence<int, 8 / RB>{});
             }
         }
+    }
+    if constexpr (SMALL) {
+        const int prz = part % 3, pry = part / 3;
+        if (inside) {
+#pragma unroll
+            for (int az = 0; az < 2; az++) {
+                if ((prz == 0 && az == 1) || (prz == 2 && az == 0)) continue;      // (voxels this offset does not reach)
+#pragma unroll
+                for (int ay = 0; ay < 2; ay++) {
+                    if ((pry == 0 && ay == 1) || (pry == 2 && ay == 0)) continue;
+#pragma unroll
+                    for (int ax = 0; ax < 2; ax++)
+#pragma unroll
+                        for (int i = 0; i < VEC; i++)
+                            atomicAdd(&s_sum[(ci * 8 + az * 4 + ay * 2 + ax) * BKC + sub * VEC + i], acc[az][ay][ax][i]);
+                }
+            }
+        }
+        __syncthreads();
+        for (int q = threadIdx.x; q < 8 * 8 * BKC / 4; q += 576) {
+            const int c4 = q % (BKC / 4), v = (q / (BKC / 4)) & 7, cube = q / (8 * BKC / 4);
+            const int z = (bz * BZ) * 2 + (v >> 2), y = (by * BY + (cube >> 2)) * 2 + ((v >> 1) & 1),
+                      x = (bx * 4 + (cube & 3)) * 2 + (v & 1);
+            if (z < s.D && y < s.H && x < s.W)
+                *reinterpret_cast<float4 *>(gxcl + ((long)b * s.vol + ((long)z * s.H + y) * s.W + x) * s.Cin + cidx * BKC + c4 * 4) =
+                    *reinterpret_cast<const float4 *>(&s_sum[q * 4]);
+        }
+        return;
     }
 #pragma unroll
     for (int az = 0; az < 2; az++)
@@ -585,13 +625,13 @@ int d2c_gx_owner_launch(const TiledShape &s, const void *gcol, const SampleLists
     const int ncx = (s.W + 1) / 2, ncy = (s.H + 1) / 2, ncz = (s.D + 1) / 2;
     const long nblk = (long)s.N * ((ncz + 1) / 2) * ((ncy + 3) / 4) * ((ncx + 3) / 4);
     constexpr int RB = sizeof(T) == 2 ? 8 : 4;
-    // (fewer than two of the large workgroups per compute unit: one-wavefront workgroups, 3 - 5 % faster backward
-    // pass at 512 channels on 8x15x27 and 128 channels on 8x30x54)
-    if (8 * ((nblk + 7) / 8) * c_n < 512) {
+    // (512 channels on 8x15x27, 128 large workgroups: backward pass 0.41 -> 0.36 ms; 128 channels on 8x30x54, 112:
+    // 0.31 -> 0.27; from 224 workgroups on -- 256 channels on 8x30x54 -- the large workgroups are faster)
+    if (8 * ((nblk + 7) / 8) * c_n < 160) {
         const long nblk8 = (long)s.N * ncz * ((ncy + 1) / 2) * ((ncx + 3) / 4);
         dim3 grid((unsigned)(8 * ((nblk8 + 7) / 8) * c_n));
-        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, RB, true>), grid, dim3(64), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
-        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, RB, true>), grid, dim3(64), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+        if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, RB, true>), grid, dim3(576), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
+        else hipLaunchKernelGGL((gx_owner_cube_kernel<T, false, RB, true>), grid, dim3(576), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
     } else {
         dim3 grid((unsigned)(8 * ((nblk + 7) / 8) * c_n));    // see the kernel's unit mapping
         if (L.compact) hipLaunchKernelGGL((gx_owner_cube_kernel<T, true, RB, false>), grid, dim3(256), 0, st, s, (const T *)gcol, L, gxcl, c_lo, c_n);
