@@ -286,7 +286,7 @@ struct TiledShape {
     long obs, mbs;
     int mact;             // activation the sampler applies to the mask values it reads (D2C_MASK_ACT_*)
     int f32split;         // float problems: 1 = all backward matrix kernels take two-term bfloat16 operands
-                          // (D2C_BWD_F32_SPLIT), 2 = the grad-column product alone (tiled_bwd_col_kernel), 0 = none
+                          // (D2C_BWD_F32_SPLIT), 2 = the grad-column product alone (tiled_bwd_col32f_kernel / tiled_bwd_col_kernel), 0 = none
 };
 
 // The modulation activation of the self-deforming layers (network/layers.py:107-120, dconv_native/modules.py:71-84),

@@ -427,28 +427,22 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_data_kernel(BwdDataArgs a)
 // no multiple of 128 channels; the others take tiled_bwd_col32_kernel further down.
 D2C_DEV void lds_only_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// at most `n` vector-memory operations of this wavefront still in flight
+// at most `n` vector-memory operations of this wavefront still in flight (the counter has six bits: its low four in
+// bits 3:0 of the operand, the other two in bits 15:14; counts above 31 wait as for 31)
 D2C_DEV void wait_vm_at_most(int n)
 {
-    switch (n) {
-    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
-    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
-    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
-    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
-    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
-    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
-    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
-    case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
-    case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
-    case 9: __builtin_amdgcn_s_waitcnt(0x0F79); break;
-    case 10: __builtin_amdgcn_s_waitcnt(0x0F7A); break;
-    case 11: __builtin_amdgcn_s_waitcnt(0x0F7B); break;
-    case 12: __builtin_amdgcn_s_waitcnt(0x0F7C); break;
-    case 13: __builtin_amdgcn_s_waitcnt(0x0F7D); break;
-    case 14: __builtin_amdgcn_s_waitcnt(0x0F7E); break;
-    case 15: __builtin_amdgcn_s_waitcnt(0x0F7F); break;
-    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+#define D2C_WAIT_VM_CASE(k) case k: __builtin_amdgcn_s_waitcnt(0x0F70 | ((k) & 15) | (((k) >> 4) << 14)); break;
+    switch (n < 0 ? 0 : (n > 31 ? 31 : n)) {
+        D2C_WAIT_VM_CASE(0) D2C_WAIT_VM_CASE(1) D2C_WAIT_VM_CASE(2) D2C_WAIT_VM_CASE(3)
+        D2C_WAIT_VM_CASE(4) D2C_WAIT_VM_CASE(5) D2C_WAIT_VM_CASE(6) D2C_WAIT_VM_CASE(7)
+        D2C_WAIT_VM_CASE(8) D2C_WAIT_VM_CASE(9) D2C_WAIT_VM_CASE(10) D2C_WAIT_VM_CASE(11)
+        D2C_WAIT_VM_CASE(12) D2C_WAIT_VM_CASE(13) D2C_WAIT_VM_CASE(14) D2C_WAIT_VM_CASE(15)
+        D2C_WAIT_VM_CASE(16) D2C_WAIT_VM_CASE(17) D2C_WAIT_VM_CASE(18) D2C_WAIT_VM_CASE(19)
+        D2C_WAIT_VM_CASE(20) D2C_WAIT_VM_CASE(21) D2C_WAIT_VM_CASE(22) D2C_WAIT_VM_CASE(23)
+        D2C_WAIT_VM_CASE(24) D2C_WAIT_VM_CASE(25) D2C_WAIT_VM_CASE(26) D2C_WAIT_VM_CASE(27)
+        D2C_WAIT_VM_CASE(28) D2C_WAIT_VM_CASE(29) D2C_WAIT_VM_CASE(30) D2C_WAIT_VM_CASE(31)
     }
+#undef D2C_WAIT_VM_CASE
 }
 
 // (XOR over 8 piece positions.  Spreading the pieces over 16 positions, the 64 banks of this LDS, took the
@@ -837,6 +831,153 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a
     wait_vm_at_most(0);     // (transfers into this workgroup's LDS must not outlive it)
 }
 
+// The same kernel for float problems on two-term bfloat16 operands (TiledShape::f32split).  A step = the 32 channels
+// of one chunk and tap; its weight tile in LDS is [32 channels][high halves of the 128 NBP reduced channels | their
+// low halves] in bfloat16 (pack_weight_bwd_planes_kernel), as large as the bfloat16 kernel's for twice the
+// channels; the stationary grad_out rows are kept as a high and a low half too, and the product is
+// high x high + low(weight) x high + high(weight) x low, three blocks of matrix instructions per 128 channels instead
+// of one (the product of the two low halves is below float's own rounding).  The rows leave as floats, two runs of 8
+// consecutive channels per lane.  ADD as above.
+template <int NBP, bool ADD>   // reduced channels: 128 NBP
+__global__ void __launch_bounds__(kThreads) tiled_bwd_col32f_kernel(BwdDataArgs a)
+{
+    constexpr int BKC = 32, MT = 256, NKG = 8 * NBP, NW = kThreads / 64;
+    constexpr int R = 2 * NBP;               // requests per wavefront and tile (32 rows x 512 NBP bytes / 16 / 64 / 8)
+    constexpr int ST = 4, LD = ADD ? 4 : 0;  // 16-byte stores / loads of rows per step
+    static_assert(kColAhead < kColRing && kColRing == 4, "a buffer is refilled a step after its last reader at the earliest");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const TiledShape &s = a.s;
+    constexpr int rowB = 2 * 128 * NBP * 2, tileB = BKC * rowB, rp = rowB / 16;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tile = xcd_swizzle(blockIdx.x, gridDim.x);
+    const int wg = blockIdx.y;
+    const int m0 = tile * MT;
+    const int S = s.nchunk * s.K;
+    const bool full_tile = m0 + MT <= s.M;
+
+    // ---- stationary operand: gout[pos, o] of this wavefront's 32 positions, high and low halves
+    uint4 gh[NKG], gm[NKG];
+    {
+        const int m = m0 + wave * 32 + (lane & 31);
+        const bool ok = m < s.M;
+        const int b = ok ? m / s.P : 0, p = ok ? m - b * s.P : 0;
+        const float *gp = reinterpret_cast<const float *>(a.gout) + ((long)b * s.Cout + wg * s.og + a.o0) * s.P + p;
+#pragma unroll
+        for (int kg = 0; kg < NKG; kg++) {
+            float e[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int o = (kg * 2 + (lane >> 5)) * 8 + i;
+                e[i] = (ok && o < a.ogn) ? gp[(long)o * s.P] : 0.f;
+            }
+            uint32_t h[4], l[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                h[i] = pack_bf16x2(e[2 * i], e[2 * i + 1]);
+                l[i] = pack_bf16x2(bf16_residual(e[2 * i], h[i] << 16), bf16_residual(e[2 * i + 1], h[i] & 0xffff0000u));
+            }
+            gh[kg] = make_uint4(h[0], h[1], h[2], h[3]);
+            gm[kg] = make_uint4(l[0], l[1], l[2], l[3]);
+        }
+    }
+
+    int psrc[R];
+#pragma unroll
+    for (int q = 0; q < R; q++) {
+        const int pos = (wave + q * NW) * 64 + lane;
+        const int row = pos / rp, pc = pos - row * rp;
+        psrc[q] = row * rp + (pc ^ swizzle_of_row(row));
+    }
+    auto dma_piece = [&](int st, int buf, int q) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.wt) + ((long)wg * S + st) * BKC * rp;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + psrc[q]),
+                                         (__attribute__((address_space(3))) void *)(smem + buf * tileB + (wave + q * NW) * 1024),
+                                         16, 0, 0);
+    };
+    unsigned woff[8];
+    {
+        const int ml = lane & 31, i = ml >> 3, hq = (ml >> 2) & 1, j = ml & 3;
+        const int wrow = i < 2 ? 8 * hq + 4 * i + j : 16 + 8 * hq + 4 * (i - 2) + j;
+        const int wsw = swizzle_of_row(wrow), wh = lane >> 5;
+        const unsigned lbase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
+#pragma unroll
+        for (int q = 0; q < 8; q++) woff[q] = lbase + (unsigned)(wrow * rowB + (((q * 2 + wh) ^ wsw) << 4));
+    }
+
+    const int lo = (int)((long)S * blockIdx.z / gridDim.z), hi = (int)((long)S * (blockIdx.z + 1) / gridDim.z);
+    if (lo >= hi) return;
+#pragma unroll
+    for (int d = 0; d < kColAhead; d++)
+#pragma unroll
+        for (int q = 0; q < R; q++) dma_piece(min(lo + d, hi - 1), d, q);
+
+    const int cpc = s.cpg / BKC;               // steps per (offset group, tap)
+    const int m_lane = m0 + wave * 32 + (lane & 31);
+    // where this lane's 2 x 8 channels of a step go (step order: offset group (outer), tap, chunk of the group)
+    auto row_of = [&](int st) -> float * {
+        const int jj = st % cpc, k = (st / cpc) % s.K, gi = st / (cpc * s.K);
+        const int c0 = wg * s.cg + (gi * cpc + jj) * BKC;
+        float *gb = reinterpret_cast<float *>(a.gcolbuf) + ((long)(c0 / BKC) * s.K + k) * s.M * BKC;
+        return gb + (long)m_lane * BKC + 8 * (lane >> 5);
+    };
+    for (int st = lo, it = 0; st < hi; st++, it++) {
+        // (the counted wait of tiled_bwd_col32_kernel: the requests of the kColAhead - 1 tiles behind this one, and
+        // the stores and loads of rows since its own requests)
+        wait_vm_at_most((kColAhead - 1) * R +
+                        ((full_tile && it >= kColAhead) ? ST * kColAhead + LD * (kColAhead - 1) : 0));
+        lds_only_barrier();
+        float *row = row_of(st);
+        float4 pv[4] = {};
+        if constexpr (ADD) {
+            if (m_lane < s.M) {
+                pv[0] = *reinterpret_cast<const float4 *>(row);
+                pv[1] = *reinterpret_cast<const float4 *>(row + 4);
+                pv[2] = *reinterpret_cast<const float4 *>(row + 16);
+                pv[3] = *reinterpret_cast<const float4 *>(row + 20);
+            }
+        }
+
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.f;
+        const int nx = min(st + kColAhead, hi - 1), nbuf = (it + kColAhead) & (kColRing - 1);
+        asm volatile("s_nop 4" ::: "memory");
+        // high x high, then the weights' low halves x high, then high x the rows' low halves
+        mma8_bf16_t<0>(acc, gh, woff);
+        dma_piece(nx, nbuf, 0);
+        if constexpr (NBP == 2) {
+            mma8_bf16_t<256>(acc, gh + 8, woff);
+            dma_piece(nx, nbuf, 1);
+        }
+        mma8_bf16_t<256 * NBP>(acc, gh, woff);
+        dma_piece(nx, nbuf, NBP);
+        if constexpr (NBP == 2) {
+            mma8_bf16_t<768>(acc, gh + 8, woff);
+            dma_piece(nx, nbuf, 3);
+        }
+        mma8_bf16_t<0>(acc, gm, woff);
+        if constexpr (NBP == 2) mma8_bf16_t<256>(acc, gm + 8, woff);
+        asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc)::"memory");
+        const unsigned adv = ((it + 1) & (kColRing - 1)) ? (unsigned)tileB : (unsigned)(-(kColRing - 1) * tileB);
+#pragma unroll
+        for (int q = 0; q < 8; q++) woff[q] += adv;
+
+        if (m_lane < s.M) {
+            if constexpr (ADD) {
+                const float pw[16] = {pv[0].x, pv[0].y, pv[0].z, pv[0].w, pv[1].x, pv[1].y, pv[1].z, pv[1].w,
+                                      pv[2].x, pv[2].y, pv[2].z, pv[2].w, pv[3].x, pv[3].y, pv[3].z, pv[3].w};
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[e] += pw[e];
+            }
+            *reinterpret_cast<float4 *>(row) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            *reinterpret_cast<float4 *>(row + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+            *reinterpret_cast<float4 *>(row + 16) = make_float4(acc[8], acc[9], acc[10], acc[11]);
+            *reinterpret_cast<float4 *>(row + 20) = make_float4(acc[12], acc[13], acc[14], acc[15]);
+        }
+    }
+    wait_vm_at_most(0);     // (transfers into this workgroup's LDS must not outlive it)
+}
+
 template <typename T> size_t bwd_col_lds(int ogk, bool db)
 {
     constexpr int VEC = Elem<T>::VEC, BKC = 8 * VEC, CB = BKC / 32, MT = 32 * (8 / CB);
@@ -866,6 +1007,28 @@ int launch_bwd_col(const BwdDataArgs &a, int nsplit, hipStream_t st, bool split)
 }
 
 constexpr int kCol32MT = 256;
+// float problems on two-term operands: passes of 97 .. 128 or 225 .. 256 reduced channels (the two bfloat16 planes of
+// 128 / 256 channels then fill exactly the buffer that holds the pass's float weights)
+bool bwd_col32f_ok(int ogn, int dtype, bool split)
+{
+    return dtype == D2C_F32 && split && ((ogn > 96 && ogn <= 128) || (ogn > 224 && ogn <= 256));
+}
+int launch_bwd_col32f(const BwdDataArgs &a, int nsplit, hipStream_t st)
+{
+    const int nbp = a.ogn > 128 ? 2 : 1;
+    const size_t lds = (size_t)kColRing * 32 * (2 * 128 * nbp * 2);
+    const dim3 grid((a.s.M + kCol32MT - 1) / kCol32MT, a.s.groups, nsplit);
+    auto go = [&](auto nb_c, auto add_c) -> int {
+        constexpr int NBP = decltype(nb_c)::value;
+        constexpr bool ADD = decltype(add_c)::value;
+        if (int rc = d2c_allow_lds((const void *)tiled_bwd_col32f_kernel<NBP, ADD>, 160 * 1024, "tiled_bwd_col32f_kernel")) return rc;
+        D2cProfScope prof(D2C_PROF_BWD_DATA, st, "tiled_bwd_col32f_kernel");
+        hipLaunchKernelGGL((tiled_bwd_col32f_kernel<NBP, ADD>), grid, dim3(kThreads), lds, st, a);
+        return d2c_check_launch("tiled_bwd_col32f_kernel");
+    };
+    if (nbp == 2) return a.add_aux ? go(std::integral_constant<int, 2>{}, std::true_type{}) : go(std::integral_constant<int, 2>{}, std::false_type{});
+    return a.add_aux ? go(std::integral_constant<int, 1>{}, std::true_type{}) : go(std::integral_constant<int, 1>{}, std::false_type{});
+}
 bool bwd_col32_ok(int ogk, int ogn, int dtype) { return dtype == D2C_BF16 && ogk % 128 == 0 && ogk <= 512 && ogn > 0; }
 int launch_bwd_col32(const BwdDataArgs &a, int nsplit, hipStream_t st)
 {
@@ -1772,6 +1935,38 @@ __global__ void __launch_bounds__(256) pack_weight_bwd_kernel(const T *w, T *wt,
     }
 }
 
+// W[o][c][k] (float) -> wt[wg][step][cc][high halves of 128 nbp output channels | their low halves] in bfloat16, for
+// tiled_bwd_col32f_kernel; channels past ogn are zeros; steps in the order of the data kernel.  One thread = 8
+// consecutive output channels of one plane.
+__global__ void __launch_bounds__(256) pack_weight_bwd_planes_kernel(const float *w, bf16_t *wt, TiledShape s, int nbp,
+                                                                     int o0, int ogn, long total)
+{
+    constexpr int BKC = 32;
+    const int pw = 128 * nbp;            // plane width
+    for (long v = (long)blockIdx.x * blockDim.x + threadIdx.x; v < total / 8; v += (long)gridDim.x * blockDim.x) {
+        const long i = v * 8;
+        const int op = (int)(i % (2 * pw)), plane = op / pw, oo = op - plane * pw;
+        long r = i / (2 * pw);
+        const int cc = (int)(r % BKC); r /= BKC;
+        const int st = (int)(r % (s.K * s.nchunk));
+        const int wg = (int)(r / (s.K * s.nchunk));
+        const int cpc = s.cpg / BKC;
+        const int k = (st / cpc) % s.K, j = (st / (cpc * s.K)) * cpc + st % cpc;
+        float e[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++)
+            e[q] = oo + q < ogn ? w[((long)(wg * s.og + o0 + oo + q) * s.cg + j * BKC + cc) * s.K + k] : 0.f;
+        uint32_t out[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t h = pack_bf16x2(e[2 * q], e[2 * q + 1]);
+            out[q] = plane == 0 ? h
+                                : pack_bf16x2(bf16_residual(e[2 * q], h << 16), bf16_residual(e[2 * q + 1], h & 0xffff0000u));
+        }
+        *reinterpret_cast<uint4 *>(wt + i) = make_uint4(out[0], out[1], out[2], out[3]);
+    }
+}
+
 // The same re-layout through LDS (needs a 16-byte aligned W): a workgroup takes a block of output channels
 // as wide as the padding unit of ogk (128 bytes of wt) and kPackCh channels of a chunk, whose weights are
 // runs of kPackCh * K consecutive elements in W, and writes 16-byte vectors of consecutive output channels.
@@ -2037,9 +2232,10 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         // about two of them)
         const int og1 = s.og < omax ? s.og : omax;     // (the first pass; sized for it)
         const bool c32 = bwd_col32_ok(d2c_bwd_ogk(og1, Elem<T>::DT), og1, Elem<T>::DT);
+        const bool c32f = bwd_col32f_ok(og1, Elem<T>::DT, s.f32split != 0);
         const int MT = c32 ? kCol32MT : 32 * (8 / (BKC / 32));
         const long items = (long)((s.M + MT - 1) / MT) * s.groups;
-        const int S = (sliced ? g_n * (s.cpg / BKC) : s.nchunk) * s.K * (c32 ? 2 : 1), reload = c32 ? 2 : 1;
+        const int S = (sliced ? g_n * (s.cpg / BKC) : s.nchunk) * s.K * (c32 ? 2 : 1), reload = c32 || c32f ? 2 : 1;
         long best = ((items + ncu - 1) / ncu) * (S + reload);
         nsplit = 1;
         for (int k = 2; k <= 16 && k <= S; k++) {
@@ -2076,7 +2272,16 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         const bool col_only = gcolbuf && !gxcl && !goff && !gmask && bwd_col_lds<T>(ogk, false) <= 160 * 1024;
         const bool split_pass = sizeof(T) == 4 && (s.f32split == 1 || (s.f32split == 2 && col_only));
         // (weights_packed: `wt` already holds them, from an earlier call on the same weights)
-        if ((phase & 1) && !weights_packed) {
+        const bool planes = col_only && bwd_col32f_ok(ogn, Elem<T>::DT, split_pass);
+        if ((phase & 1) && !weights_packed && planes) {
+            if constexpr (sizeof(T) == 4) {
+                D2cProfScope prof(D2C_PROF_PACK, st);
+                const int nbp = ogn > 128 ? 2 : 1;
+                const long tot = (long)s.groups * s.K * s.nchunk * BKC * 2 * 128 * nbp;
+                hipLaunchKernelGGL(pack_weight_bwd_planes_kernel, dim3(grid1d(tot / 8)), dim3(256), 0, st, (const float *)w,
+                                   (bf16_t *)wt, s, nbp, o0, ogn, tot);
+            }
+        } else if ((phase & 1) && !weights_packed) {
             D2cProfScope prof(D2C_PROF_PACK, st);
             constexpr int R = 128 / (int)sizeof(T);
             constexpr bool SPT = sizeof(T) == 4;       // (split operands exist for float problems only)
@@ -2100,6 +2305,8 @@ int d2c_tiled_bwd_data_launch(const TiledShape &s, const void *gout, const void 
         int rc;
         if (col_only && bwd_col32_ok(ogk, ogn, Elem<T>::DT)) {
             rc = launch_bwd_col32(a, nsplit, st);
+        } else if (planes) {
+            rc = launch_bwd_col32f(a, nsplit, st);
         } else if (sliced) {
             d2c_set_error("grad-column product: slices are made by tiled_bwd_col32_kernel only");
             return D2C_ERR_LAUNCH;
