@@ -836,7 +836,8 @@ __global__ void __launch_bounds__(kThreads) tiled_bwd_col32_kernel(BwdDataArgs a
 // low halves] in bfloat16 (pack_weight_bwd_planes_kernel), as large as the bfloat16 kernel's for twice the
 // channels; the stationary grad_out rows are kept as a high and a low half too, and the product is
 // high x high + low(weight) x high + high(weight) x low, three blocks of matrix instructions per 128 channels instead
-// of one (the product of the two low halves is below float's own rounding).  The rows leave as floats, two runs of 8
+// of one (the product of the two low halves, at most 2^-18 of the term, is of the size of the error that the
+// rounding of the low halves leaves in the other two and is left out).  The rows leave as floats, two runs of 8
 // consecutive channels per lane.  ADD as above.
 template <int NBP, bool ADD>   // reduced channels: 128 NBP
 __global__ void __launch_bounds__(kThreads) tiled_bwd_col32f_kernel(BwdDataArgs a)
