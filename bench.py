@@ -795,7 +795,7 @@ def main():
         # instructions executed are the partial products
         if dt == "f32":
             terms = {"tiled_fwd_dma_kernel": 4, "tiled_fwd_kernel": 4, "tiled_bwd_weight_col3_kernel": 6,
-                     "tiled_bwd_col_kernel": 4}
+                     "tiled_bwd_col_kernel": 4, "tiled_bwd_col32f_kernel": 3}
             if args.f32_split_backward:
                 terms.update({"tiled_bwd_weight_dma_kernel": 4, "tiled_bwd_data_kernel": 4})
             if dom in terms:
